@@ -1,0 +1,166 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention forward hot path on one MI355X.
+
+Headline workload (config.workload): long-context prefill, B=8 H=16 L=2048 d=64, causal mask,
+q/k/v = 0.5*N(0,1), fp32 -- the configuration the metric's MFMA target is quoted on.  One step is one
+fused attention call over that batch with the inputs already resident in HBM.  The decode workload
+(B=16 H=16 d=64, 4096-row cache, 64 append+attend steps) is reported beside it in "decode".
+
+Prints ONE JSON line.  `value` is algorithmic TFLOP/s (4*d flops per unblocked query-key pair) over the
+wall time of the K timed steps; roofline.achieved uses the HIP-event time of the same K launches.
+cpu_baseline times the CPU oracle (a restatement of the reference's generic CPU engine) on a bounded
+sample of the same workload, single-threaded like the reference's engine.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+
+def prefill(ctx, lib, steps, warmup):
+    B, H, L, d = 8, 16, 2048, 64
+    rng = np.random.Generator(np.random.PCG64(1004))
+    q, k, v = (rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5) for _ in range(3))
+    dq, dk, dv = ctx.to_device(q), ctx.to_device(k), ctx.to_device(v)
+    out = ctx.empty((B, H, L, d))
+    desc = ctx.mask_desc(lib.MASK_CAUSAL)
+    flops = 4.0 * d * B * H * (L * (L + 1) // 2)
+    for _ in range(warmup):
+        ctx.sdpa_fwd(dq, dk, dv, out, B, H, L, L, d, d, 0.125, desc, 0)
+    ctx.sync()
+    t0 = time.perf_counter()
+    ctx.timer_begin()
+    for _ in range(steps):
+        ctx.sdpa_fwd(dq, dk, dv, out, B, H, L, L, d, d, 0.125, desc, 0)
+    ev_ms = ctx.timer_end()
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    o = out.numpy()
+    if not (np.isfinite(o).all() and np.allclose(o[:, :, 0], v[:, :, 0], atol=1e-6)):
+        raise RuntimeError("prefill output failed its sanity check")
+    for b in (dq, dk, dv, out):
+        b.release()
+    return {"flops": flops, "wall_s": wall, "event_ms_per_launch": ev_ms / steps,
+            "shape": {"B": B, "H": H, "L": L, "d": d}, "inputs": (q, k, v)}
+
+
+def decode(ctx, lib, repeats):
+    B, H, d, T0, steps = 16, 16, 64, 4096, 64
+    Tcap = T0 + steps
+    rng = np.random.Generator(np.random.PCG64(1005))
+    kc = ctx.to_device(rng.standard_normal((B, H, Tcap, d), dtype=np.float32))
+    vc = ctx.to_device(rng.standard_normal((B, H, Tcap, d), dtype=np.float32))
+    qs = ctx.to_device(rng.standard_normal((steps, B, H, 1, d), dtype=np.float32))
+    kn = ctx.to_device(rng.standard_normal((steps, B, H, 1, d), dtype=np.float32))
+    vn = ctx.to_device(rng.standard_normal((steps, B, H, 1, d), dtype=np.float32))
+    out = ctx.empty((steps, B, H, 1, d))
+    sb = B * H * d * 4
+
+    def run():
+        for t in range(steps):
+            ctx.sdpa_decode_step(qs.offset(t * sb), kc, vc, kn.offset(t * sb), vn.offset(t * sb), out.offset(t * sb),
+                                 B, H, T0 + t, Tcap, d, 0.125)
+    run()
+    ctx.sync()
+    per_step_us = []
+    for _ in range(repeats):
+        ctx.timer_begin()
+        run()
+        per_step_us.append(ctx.timer_end() * 1e3 / steps)
+    o = out.numpy()
+    if not np.isfinite(o).all():
+        raise RuntimeError("decode output failed its sanity check")
+    for b in (kc, vc, qs, kn, vn, out):
+        b.release()
+    us = float(np.median(per_step_us))
+    # algorithmic bytes per step: K and V rows 0..T-1 read once, q read, out written, the new k/v row written
+    Tavg = T0 + (steps + 1) / 2.0
+    bytes_step = 2 * B * H * Tavg * d * 4 + 2 * B * H * d * 4 + 2 * B * H * d * 4
+    return {"us_per_step": us, "us_per_step_min": float(np.min(per_step_us)), "tokens_per_s": B / (us * 1e-6),
+            "bytes_per_step": bytes_step, "gbs": bytes_step / (us * 1e-6) / 1e9,
+            "shape": {"B": B, "H": H, "d": d, "T0": T0, "steps": steps}}
+
+
+def cpu_baseline_prefill(q, k, v, pairs):
+    from oracle import binding as orc
+    L, d = q.shape[2], q.shape[3]
+    i, j = np.indices((L, L))
+    mask = (j > i).astype(np.float32)
+    orc.lib()
+    t0 = time.perf_counter()
+    for p in range(pairs):
+        b, h = divmod(p, q.shape[1])
+        orc.sdpa(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mask)
+    dt = time.perf_counter() - t0
+    flops = 4.0 * d * pairs * (L * (L + 1) // 2)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "%d of %d (batch, head) slices of the headline workload (L=%d, d=%d, dense causal mask), "
+                      "%.1f s of single-thread CPU time; host has %d cores" % (pairs, q.shape[0] * q.shape[1], L, d, dt,
+                                                                             os.cpu_count() or 0)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--cpu-pairs", type=int, default=6, help="(batch, head) slices timed on the CPU oracle; 0 disables")
+    ap.add_argument("--decode-repeats", type=int, default=5)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (every attention problem fits one MI355X); --gpus %d is not "
+              "supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    from dl4s_amd import lib
+    ctx = lib.Context(0)
+    info = ctx.device_info()
+    pre = prefill(ctx, lib, args.steps, args.warmup)
+    dec = decode(ctx, lib, args.decode_repeats) if args.decode_repeats > 0 else None
+    ctx.close()
+
+    tflops = pre["flops"] * args.steps / pre["wall_s"] / 1e12
+    ach = pre["flops"] / (pre["event_ms_per_launch"] * 1e-3) / 1e12
+    line = {
+        "metric": "attention fwd TFLOP/s (fp32)",
+        "value": tflops,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": pre["wall_s"] / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "long-context prefill B=8 H=16 L=2048 d=64 causal, q/k/v=0.5*N(0,1) (BASELINE config 4)",
+                   "flops_per_step": pre["flops"], "device": info["name"], "cu_count": info["cu_count"]},
+        "roofline": {"bound": "mfma", "achieved": ach, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": ach / MFMA_FP32_PEAK_TFLOPS, "traffic": None, "kernel": "sdpa_prefill_f32_d64",
+                     "ms_per_launch": pre["event_ms_per_launch"]},
+    }
+    if dec:
+        line["decode"] = {"workload": "incremental decode B=16 H=16 d=64, KV cache 4096 rows + 64 append+attend steps "
+                                      "(BASELINE config 5)",
+                          "us_per_step": dec["us_per_step"], "tokens_per_s": dec["tokens_per_s"],
+                          "roofline": {"bound": "hbm", "achieved": dec["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                       "frac": dec["gbs"] / HBM_PEAK_GBS, "traffic": None,
+                                       "kernel": "sdpa_decode_splitk_f32", "bytes_per_step": dec["bytes_per_step"]}}
+    if args.cpu_pairs > 0:
+        q, k, v = pre["inputs"]
+        line["cpu_baseline"] = cpu_baseline_prefill(q, k, v, args.cpu_pairs)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,66 @@
+// Shared internals of libdl4s_hip.so: the context object, error reporting and launch helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/dl4s_hip.h"
+
+struct dl4s_hip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    int cu_count = 0;
+    int clock_khz = 0;
+    char name[256] = {0};
+    std::mutex mu;
+    // pooled allocator: live blocks (base -> rounded size) and free lists per rounded size
+    std::map<uintptr_t, size_t> live;
+    std::unordered_map<size_t, std::vector<void *>> pool;
+    size_t bytes_in_use = 0, bytes_pooled = 0;
+    // scratch owned by the library for split-K partial results (grown on demand, never shrunk)
+    void *scratch = nullptr;
+    size_t scratch_bytes = 0;
+    // one ticket per (batch, head) for the split-K merge; all zero whenever no kernel is running
+    unsigned int *tickets = nullptr;
+    static constexpr int kMaxTickets = 65536;
+};
+
+namespace dl4s {
+
+int set_error(int code, const char *fmt, ...);
+int hip_error(hipError_t e, const char *what);
+// Grows ctx->scratch to at least `bytes`; returns 0 or a status.
+int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes);
+
+#define DL4S_CHECK_CTX(ctx)                                                        \
+    do {                                                                           \
+        if (!(ctx)) return dl4s::set_error(DL4S_HIP_EINVALID_ARG, "%s: ctx is NULL", __func__); \
+        hipError_t e__ = hipSetDevice((ctx)->device);                              \
+        if (e__ != hipSuccess) return dl4s::hip_error(e__, "hipSetDevice");        \
+    } while (0)
+
+#define DL4S_HIP_TRY(expr)                                               \
+    do {                                                                 \
+        hipError_t e__ = (expr);                                         \
+        if (e__ != hipSuccess) return dl4s::hip_error(e__, #expr);       \
+    } while (0)
+
+#define DL4S_REQUIRE(cond, code, ...)                                    \
+    do {                                                                 \
+        if (!(cond)) return dl4s::set_error((code), __VA_ARGS__);        \
+    } while (0)
+
+inline int launch_status(const char *kernel) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_error(e, kernel);
+    return DL4S_HIP_OK;
+}
+
+}  // namespace dl4s

@@ -1,0 +1,242 @@
+// Context, pooled allocator, copies and the stream timer of libdl4s_hip.so.
+#include "common.h"
+
+#include <cstring>
+
+namespace dl4s {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_error(hipError_t e, const char *what) {
+    snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+    (void)hipGetLastError();  // clear the sticky flag so that the next call reports its own failure
+    return e == hipErrorOutOfMemory ? DL4S_HIP_EOOM : DL4S_HIP_EHIP;
+}
+
+// Allocation sizes are rounded so that freed blocks are reusable: 512 B granules up to 1 MiB,
+// 2 MiB granules above.
+static size_t round_size(size_t bytes) {
+    if (bytes == 0) bytes = 1;
+    const size_t small = 512, large = size_t(2) << 20;
+    if (bytes <= (size_t(1) << 20)) return (bytes + small - 1) / small * small;
+    return (bytes + large - 1) / large * large;
+}
+
+int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes) {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    if (bytes <= ctx->scratch_bytes) return DL4S_HIP_OK;
+    // the old block may still be read by enqueued kernels: wait before releasing it
+    if (ctx->scratch) {
+        DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        DL4S_HIP_TRY(hipFree(ctx->scratch));
+        ctx->scratch = nullptr;
+        ctx->scratch_bytes = 0;
+    }
+    size_t want = round_size(bytes);
+    DL4S_HIP_TRY(hipMalloc(&ctx->scratch, want));
+    ctx->scratch_bytes = want;
+    return DL4S_HIP_OK;
+}
+
+}  // namespace dl4s
+
+using namespace dl4s;
+
+extern "C" {
+
+const char *dl4s_hip_last_error(void) { return g_err; }
+
+int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx) {
+    DL4S_REQUIRE(out_ctx, DL4S_HIP_EINVALID_ARG, "dl4s_hip_create: out_ctx is NULL");
+    *out_ctx = nullptr;
+    int n = 0;
+    DL4S_HIP_TRY(hipGetDeviceCount(&n));
+    DL4S_REQUIRE(device_ordinal >= 0 && device_ordinal < n, DL4S_HIP_EINVALID_ARG,
+                 "dl4s_hip_create: device %d not in [0,%d)", device_ordinal, n);
+    DL4S_HIP_TRY(hipSetDevice(device_ordinal));
+    hipDeviceProp_t prop;
+    DL4S_HIP_TRY(hipGetDeviceProperties(&prop, device_ordinal));
+    DL4S_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0, DL4S_HIP_EUNSUPPORTED,
+                 "dl4s_hip_create: device %d is %s; this library holds gfx950 code only", device_ordinal,
+                 prop.gcnArchName);
+    dl4s_hip_ctx *c = new (std::nothrow) dl4s_hip_ctx();
+    DL4S_REQUIRE(c, DL4S_HIP_EOOM, "dl4s_hip_create: host allocation failed");
+    c->device = device_ordinal;
+    c->cu_count = prop.multiProcessorCount;
+    c->clock_khz = prop.clockRate;
+    snprintf(c->name, sizeof(c->name), "%s (%s)", prop.name, prop.gcnArchName);
+    hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev_begin);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev_end);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&c->tickets), dl4s_hip_ctx::kMaxTickets * sizeof(unsigned int));
+    if (e == hipSuccess) e = hipMemsetAsync(c->tickets, 0, dl4s_hip_ctx::kMaxTickets * sizeof(unsigned int), c->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    if (e != hipSuccess) {
+        if (c->tickets) (void)hipFree(c->tickets);
+        if (c->ev_end) (void)hipEventDestroy(c->ev_end);
+        if (c->ev_begin) (void)hipEventDestroy(c->ev_begin);
+        if (c->stream) (void)hipStreamDestroy(c->stream);
+        delete c;
+        return hip_error(e, "dl4s_hip_create");
+    }
+    *out_ctx = c;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_destroy(dl4s_hip_ctx *ctx) {
+    DL4S_CHECK_CTX(ctx);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (auto &kv : ctx->pool)
+        for (void *p : kv.second) (void)hipFree(p);
+    for (auto &kv : ctx->live) (void)hipFree(reinterpret_cast<void *>(kv.first));
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->tickets) (void)hipFree(ctx->tickets);
+    (void)hipEventDestroy(ctx->ev_begin);
+    (void)hipEventDestroy(ctx->ev_end);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_sync(dl4s_hip_ctx *ctx) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_device_info(dl4s_hip_ctx *ctx, int *out_cu_count, int *out_clock_khz, char *name_buf, size_t name_len) {
+    DL4S_CHECK_CTX(ctx);
+    if (out_cu_count) *out_cu_count = ctx->cu_count;
+    if (out_clock_khz) *out_clock_khz = ctx->clock_khz;
+    if (name_buf && name_len) snprintf(name_buf, name_len, "%s", ctx->name);
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_timer_begin(dl4s_hip_ctx *ctx) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_HIP_TRY(hipEventRecord(ctx->ev_begin, ctx->stream));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(out_ms, DL4S_HIP_EINVALID_ARG, "dl4s_hip_timer_end: out_ms is NULL");
+    DL4S_HIP_TRY(hipEventRecord(ctx->ev_end, ctx->stream));
+    DL4S_HIP_TRY(hipEventSynchronize(ctx->ev_end));
+    DL4S_HIP_TRY(hipEventElapsedTime(out_ms, ctx->ev_begin, ctx->ev_end));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_alloc(dl4s_hip_ctx *ctx, size_t bytes, void **out_ptr) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(out_ptr, DL4S_HIP_EINVALID_ARG, "dl4s_hip_alloc: out_ptr is NULL");
+    *out_ptr = nullptr;
+    size_t sz = round_size(bytes);
+    std::lock_guard<std::mutex> g(ctx->mu);
+    void *p = nullptr;
+    auto it = ctx->pool.find(sz);
+    if (it != ctx->pool.end() && !it->second.empty()) {
+        p = it->second.back();
+        it->second.pop_back();
+        ctx->bytes_pooled -= sz;
+    } else {
+        hipError_t e = hipMalloc(&p, sz);
+        if (e == hipErrorOutOfMemory) {
+            // give the pooled blocks back to the driver and try once more
+            (void)hipGetLastError();
+            (void)hipStreamSynchronize(ctx->stream);
+            for (auto &kv : ctx->pool) {
+                for (void *q : kv.second) (void)hipFree(q);
+                kv.second.clear();
+            }
+            ctx->bytes_pooled = 0;
+            e = hipMalloc(&p, sz);
+        }
+        if (e != hipSuccess) return hip_error(e, "dl4s_hip_alloc(hipMalloc)");
+    }
+    ctx->live[reinterpret_cast<uintptr_t>(p)] = sz;
+    ctx->bytes_in_use += sz;
+    *out_ptr = p;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_free(dl4s_hip_ctx *ctx, void *ptr) {
+    DL4S_CHECK_CTX(ctx);
+    if (!ptr) return DL4S_HIP_OK;
+    std::lock_guard<std::mutex> g(ctx->mu);
+    auto it = ctx->live.find(reinterpret_cast<uintptr_t>(ptr));
+    DL4S_REQUIRE(it != ctx->live.end(), DL4S_HIP_EINVALID_ARG,
+                 "dl4s_hip_free: %p is not the base of a live allocation (double free or offset view)", ptr);
+    size_t sz = it->second;
+    ctx->live.erase(it);
+    ctx->bytes_in_use -= sz;
+    ctx->pool[sz].push_back(ptr);
+    ctx->bytes_pooled += sz;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_get_size(dl4s_hip_ctx *ctx, const void *ptr, size_t *out_bytes) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(ptr && out_bytes, DL4S_HIP_EINVALID_ARG, "dl4s_hip_get_size: NULL argument");
+    std::lock_guard<std::mutex> g(ctx->mu);
+    uintptr_t a = reinterpret_cast<uintptr_t>(ptr);
+    auto it = ctx->live.upper_bound(a);
+    DL4S_REQUIRE(it != ctx->live.begin(), DL4S_HIP_EINVALID_ARG, "dl4s_hip_get_size: %p is not inside a live allocation", ptr);
+    --it;
+    DL4S_REQUIRE(a < it->first + it->second, DL4S_HIP_EINVALID_ARG, "dl4s_hip_get_size: %p is not inside a live allocation", ptr);
+    *out_bytes = it->first + it->second - a;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_mem_stats(dl4s_hip_ctx *ctx, size_t *out_bytes_in_use, size_t *out_bytes_pooled) {
+    DL4S_CHECK_CTX(ctx);
+    std::lock_guard<std::mutex> g(ctx->mu);
+    if (out_bytes_in_use) *out_bytes_in_use = ctx->bytes_in_use;
+    if (out_bytes_pooled) *out_bytes_pooled = ctx->bytes_pooled;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_assign_h2d(dl4s_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    DL4S_CHECK_CTX(ctx);
+    if (bytes == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(dst_dev && src_host, DL4S_HIP_EINVALID_ARG, "dl4s_hip_assign_h2d: NULL pointer");
+    // pageable source: the async copy stages the data before returning only for small sizes, so wait
+    DL4S_HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_assign_d2d(dl4s_hip_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes) {
+    DL4S_CHECK_CTX(ctx);
+    if (bytes == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(dst_dev && src_dev, DL4S_HIP_EINVALID_ARG, "dl4s_hip_assign_d2d: NULL pointer");
+    DL4S_HIP_TRY(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_assign_d2h(dl4s_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    DL4S_CHECK_CTX(ctx);
+    if (bytes == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(dst_host && src_dev, DL4S_HIP_EINVALID_ARG, "dl4s_hip_assign_d2h: NULL pointer");
+    DL4S_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_get_value_f32(dl4s_hip_ctx *ctx, const float *src_dev, float *out_value) {
+    return dl4s_hip_assign_d2h(ctx, out_value, src_dev, sizeof(float));
+}
+
+int dl4s_hip_set_pointee_f32(dl4s_hip_ctx *ctx, float *dst_dev, float value) {
+    return dl4s_hip_assign_h2d(ctx, dst_dev, &value, sizeof(float));
+}
+
+}  // extern "C"

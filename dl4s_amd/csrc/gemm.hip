@@ -1,0 +1,167 @@
+// fp32 GEMM on v_mfma_f32_32x32x2_f32 for gfx950:  C = alpha * op(A) . op(B) + beta * C, row-major,
+// optional strided batch.  A workgroup (4 wavefronts, 2x2) computes a 128x128 tile of C; each
+// wavefront holds a 64x64 sub-tile as 2x2 MFMA accumulators.  K is walked in steps of 16 through
+// LDS tiles stored k-major ([k][m] and [k][n]) so that the MFMA operand reads (lane l wants row
+// l % 32 at k = l / 32) are consecutive 32-bit words, and the next K step is prefetched into
+// registers while the current one is multiplied.  Transposes are handled by the loader only: the
+// operand is addressed through (row stride, column stride), and the thread-to-element mapping is
+// chosen so that the unit-stride direction runs along the lanes.
+#include "common.h"
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int GBM = 128, GBN = 128, GBK = 16;
+constexpr int GLS = GBM + 4;  // LDS row stride in floats
+
+struct GemmArgs {
+    const float *A, *B;
+    float *C;
+    int M, N, K;
+    long long a_rs, a_cs;  // element strides of op(A)[m][k]
+    long long b_rs, b_cs;  // element strides of op(B)[k][n]
+    long long a_bs, b_bs, c_bs;  // batch strides
+    float alpha, beta;
+    int tiles_n;
+};
+
+__global__ __launch_bounds__(256, 2) void gemm_f32_mfma(GemmArgs g) {
+    __shared__ float As[2][GBK][GLS];
+    __shared__ float Bs[2][GBK][GLS];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int half = lane >> 5, ln = lane & 31;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tile_m = blockIdx.x / g.tiles_n, tile_n = blockIdx.x % g.tiles_n;
+    const int m0 = tile_m * GBM, n0 = tile_n * GBN;
+    const float *A = g.A + (long long)blockIdx.z * g.a_bs;
+    const float *B = g.B + (long long)blockIdx.z * g.b_bs;
+    float *C = g.C + (long long)blockIdx.z * g.c_bs;
+
+    // loader mappings: unit stride along k -> 16 lanes walk k; otherwise 128 threads walk m (or n)
+    const bool a_kfast = (g.a_cs == 1);
+    const bool b_kfast = (g.b_rs == 1);
+    float ast[8], bst[8];
+    auto load = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int kk, mm;
+            if (a_kfast) { kk = tid & 15; mm = (tid >> 4) + 16 * i; } else { mm = tid & 127; kk = (tid >> 7) + 2 * i; }
+            const int gm = m0 + mm, gk = kt * GBK + kk;
+            ast[i] = (gm < g.M && gk < g.K) ? A[gm * g.a_rs + gk * g.a_cs] : 0.f;
+            int kb, nn;
+            if (b_kfast) { kb = tid & 15; nn = (tid >> 4) + 16 * i; } else { nn = tid & 127; kb = (tid >> 7) + 2 * i; }
+            const int gn = n0 + nn, gkb = kt * GBK + kb;
+            bst[i] = (gn < g.N && gkb < g.K) ? B[gkb * g.b_rs + gn * g.b_cs] : 0.f;
+        }
+    };
+    auto store = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int kk, mm;
+            if (a_kfast) { kk = tid & 15; mm = (tid >> 4) + 16 * i; } else { mm = tid & 127; kk = (tid >> 7) + 2 * i; }
+            As[buf][kk][mm] = ast[i];
+            int kb, nn;
+            if (b_kfast) { kb = tid & 15; nn = (tid >> 4) + 16 * i; } else { nn = tid & 127; kb = (tid >> 7) + 2 * i; }
+            Bs[buf][kb][nn] = bst[i];
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int ktiles = (g.K + GBK - 1) / GBK;
+    if (ktiles > 0) { load(0); store(0); }
+    __syncthreads();
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int buf = kt & 1;
+        const bool more = kt + 1 < ktiles;
+        if (more) load(kt + 1);
+#pragma unroll
+        for (int ks = 0; ks < GBK / 2; ++ks) {
+            const int kk = 2 * ks + half;
+            const float a0 = As[buf][kk][wm * 64 + ln];
+            const float a1 = As[buf][kk][wm * 64 + 32 + ln];
+            const float b0 = Bs[buf][kk][wn * 64 + ln];
+            const float b1 = Bs[buf][kk][wn * 64 + 32 + ln];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        if (more) store(buf ^ 1);
+        __syncthreads();
+    }
+
+    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*half + r%4, column ln
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int gn = n0 + wn * 64 + j * 32 + ln;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int gm = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (gm < g.M && gn < g.N) {
+                    float *cp = C + (long long)gm * g.N + gn;
+                    float val = g.alpha * acc[i][j][r];
+                    if (g.beta != 0.f) val = val + g.beta * (*cp);
+                    *cp = val;
+                }
+            }
+        }
+}
+
+int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int64_t lbs, const float *rhs, int64_t rr,
+                int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb) {
+    DL4S_REQUIRE(lr >= 0 && lc >= 0 && rr >= 0 && rc >= 0 && batch >= 0, DL4S_HIP_EINVALID_ARG, "gemm: negative extent");
+    const int64_t M = ta ? lc : lr, K = ta ? lr : lc;
+    const int64_t K2 = tb ? rc : rr, N = tb ? rr : rc;
+    DL4S_REQUIRE(K == K2, DL4S_HIP_ESHAPE, "gemm: inner dimensions differ (%lld vs %lld)", (long long)K, (long long)K2);
+    if (M * N * batch == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(result && (K == 0 || (lhs && rhs)), DL4S_HIP_EINVALID_ARG, "gemm: NULL pointer");
+    DL4S_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch <= 65535, DL4S_HIP_EUNSUPPORTED,
+                 "gemm: extent too large");
+    GemmArgs g{};
+    g.A = lhs; g.B = rhs; g.C = result;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.a_rs = ta ? 1 : lc; g.a_cs = ta ? lc : 1;
+    g.b_rs = tb ? 1 : rc; g.b_cs = tb ? rc : 1;
+    g.a_bs = lbs; g.b_bs = rbs; g.c_bs = cbs;
+    g.alpha = alpha; g.beta = beta;
+    const long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
+    g.tiles_n = (int)tn;
+    DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
+    hipLaunchKernelGGL(gemm_f32_mfma, dim3((unsigned)(tm * tn), 1, (unsigned)batch), dim3(256), 0, ctx->stream, g);
+    return dl4s::launch_status("gemm_f32_mfma");
+}
+
+}  // namespace
+
+extern "C" {
+
+int dl4s_hip_gemm_f32(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols, const float *rhs,
+                      int64_t rhs_rows, int64_t rhs_cols, float *result, float alpha, float beta, int transpose_first,
+                      int transpose_second) {
+    DL4S_CHECK_CTX(ctx);
+    return gemm_launch(ctx, lhs, lhs_rows, lhs_cols, 0, rhs, rhs_rows, rhs_cols, 0, result, 0, 1, alpha, beta,
+                       transpose_first, transpose_second);
+}
+
+int dl4s_hip_gemm_batched_f32(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols, int64_t lhs_stride,
+                              const float *rhs, int64_t rhs_rows, int64_t rhs_cols, int64_t rhs_stride, float *result,
+                              int64_t result_stride, int64_t batch, float alpha, float beta, int transpose_first,
+                              int transpose_second) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(lhs_stride >= 0 && rhs_stride >= 0 && result_stride >= 0, DL4S_HIP_EINVALID_ARG, "gemm: negative batch stride");
+    return gemm_launch(ctx, lhs, lhs_rows, lhs_cols, lhs_stride, rhs, rhs_rows, rhs_cols, rhs_stride, result, result_stride,
+                       batch, alpha, beta, transpose_first, transpose_second);
+}
+
+}  // extern "C"

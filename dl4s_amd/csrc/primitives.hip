@@ -1,0 +1,466 @@
+// Engine primitives the attention layers call around the fused kernels: same-shape and broadcast
+// binaries, unary maps, reductions, permuteAxes, band, stack, LayerNorm and bias+GELU.  All are
+// HBM-bound streaming kernels: one pass, coalesced, grid-stride.
+#include "common.h"
+
+namespace {
+
+constexpr int TPB = 256;
+
+inline unsigned grid_for(long long n, int per_thread = 4) {
+    long long b = (n + (long long)TPB * per_thread - 1) / ((long long)TPB * per_thread);
+    if (b < 1) b = 1;
+    if (b > 65536) b = 65536;
+    return (unsigned)b;
+}
+
+enum { U_NEG, U_EXP, U_SQRT, U_RELU, U_TANH };
+
+template <int OP>
+__global__ void unary_f32(const float *__restrict__ x, float *__restrict__ y, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        float v = x[i], r;
+        if (OP == U_NEG) r = -v;
+        else if (OP == U_EXP) r = expf(v);
+        else if (OP == U_SQRT) r = sqrtf(v);
+        else if (OP == U_RELU) r = v > 0.f ? v : 0.f;
+        else r = tanhf(v);
+        y[i] = r;
+    }
+}
+
+template <int OP>
+__global__ void binary_f32(const float *a, const float *b, float *y, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        float r;
+        if (OP == DL4S_OP_ADD) r = __fadd_rn(a[i], b[i]);
+        else if (OP == DL4S_OP_SUB) r = __fsub_rn(a[i], b[i]);
+        else if (OP == DL4S_OP_MUL) r = __fmul_rn(a[i], b[i]);
+        else r = __fdiv_rn(a[i], b[i]);
+        y[i] = r;
+    }
+}
+
+__global__ void fill_f32(float v, float *y, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) y[i] = v;
+}
+
+struct Bcast {
+    int dim;
+    long long oshape[DL4S_HIP_MAX_DIM];
+    long long ls[DL4S_HIP_MAX_DIM], rs[DL4S_HIP_MAX_DIM];  // element strides, 0 on broadcast axes
+};
+
+// mode: 0 element by element, 1 lhs is a scalar per slice, 2 rhs is a scalar per slice (Engine/CPU/CPUEngine.swift:117-176)
+template <int OP>
+__global__ void broadcast_f32(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ y, Bcast bc,
+                              int mode, long long n) {
+    for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (long long)gridDim.x * blockDim.x) {
+        long long rem = e, li = 0, ri = 0;
+#pragma unroll 1
+        for (int i = bc.dim - 1; i >= 0; --i) {
+            const long long idx = rem % bc.oshape[i];
+            rem /= bc.oshape[i];
+            li += idx * bc.ls[i];
+            ri += idx * bc.rs[i];
+        }
+        const float x = a[li], z = b[ri];
+        float r;
+        if (OP == DL4S_OP_ADD) r = __fadd_rn(x, z);
+        else if (OP == DL4S_OP_MUL) r = __fmul_rn(x, z);
+        else if (OP == DL4S_OP_SUB) {
+            if (mode == 2) r = __fadd_rn(x, -z);             // x + (-s)
+            else if (mode == 1) r = -__fadd_rn(z, -x);       // -(x + (-s))
+            else r = __fsub_rn(x, z);
+        } else {
+            if (mode == 2) r = __fmul_rn(x, __fdiv_rn(1.0f, z));  // x * (1/s)
+            else r = __fdiv_rn(x, z);
+        }
+        y[e] = r;
+    }
+}
+
+// ---- reductions: one workgroup per output element, strided gather of the reduced elements
+struct Reduce {
+    int kdim, rdim;
+    long long kshape[DL4S_HIP_MAX_DIM], kstride[DL4S_HIP_MAX_DIM];  // kept axes: extents and source strides
+    long long rshape[DL4S_HIP_MAX_DIM], rstride[DL4S_HIP_MAX_DIM];  // reduced axes
+    long long rcount;
+};
+
+template <bool IS_MAX>
+__global__ __launch_bounds__(TPB) void reduce_f32(const float *__restrict__ x, float *__restrict__ y, Reduce rd) {
+    __shared__ float sm[TPB / 64];
+    long long o = blockIdx.x, base = 0;
+    for (int i = rd.kdim - 1; i >= 0; --i) {
+        base += (o % rd.kshape[i]) * rd.kstride[i];
+        o /= rd.kshape[i];
+    }
+    float acc = IS_MAX ? -INFINITY : 0.f;
+    for (long long j = threadIdx.x; j < rd.rcount; j += TPB) {
+        long long rem = j, off = base;
+        for (int i = rd.rdim - 1; i >= 0; --i) {
+            off += (rem % rd.rshape[i]) * rd.rstride[i];
+            rem /= rd.rshape[i];
+        }
+        const float v = x[off];
+        if (IS_MAX) acc = fmaxf(acc, v);   // NaN never selected, like the reference's "v > max" scan
+        else acc += v;
+    }
+    for (int s = 32; s > 0; s >>= 1) {
+        const float t = __shfl_xor(acc, s, 64);
+        acc = IS_MAX ? fmaxf(acc, t) : acc + t;
+    }
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float r = sm[0];
+        for (int w = 1; w < TPB / 64; ++w) r = IS_MAX ? fmaxf(r, sm[w]) : r + sm[w];
+        y[blockIdx.x] = r;
+    }
+}
+
+struct Permute {
+    int dim;
+    long long sshape[DL4S_HIP_MAX_DIM];
+    long long dstride[DL4S_HIP_MAX_DIM];  // destination stride for source axis i
+};
+
+__global__ void permute_f32(const float *__restrict__ x, float *__restrict__ y, Permute p, long long n) {
+    for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (long long)gridDim.x * blockDim.x) {
+        long long rem = e, d = 0;
+#pragma unroll 1
+        for (int i = p.dim - 1; i >= 0; --i) {
+            d += (rem % p.sshape[i]) * p.dstride[i];
+            rem /= p.sshape[i];
+        }
+        y[d] = x[e];
+    }
+}
+
+__global__ void band_f32(const float *__restrict__ x, float *__restrict__ y, long long rows, long long cols, long long below,
+                         long long above) {
+    const long long n = rows * cols;
+    for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (long long)gridDim.x * blockDim.x) {
+        const long long i = e / cols, j = e % cols;
+        long long start = i - below; if (start < 0) start = 0; if (start > cols) start = cols;
+        long long end = i + above + 1; if (end > cols) end = cols; if (end < start) end = start;
+        if (j >= start && j < end) y[e] = x[e];
+    }
+}
+
+// ---- LayerNorm over rows*D elements per batch item (NN/Layer/LayerNorm.swift:62-77)
+__device__ __forceinline__ void block_sum2(float &a, float &b, float *sm) {
+    for (int s = 32; s > 0; s >>= 1) { a += __shfl_xor(a, s, 64); b += __shfl_xor(b, s, 64); }
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) { sm[2 * w] = a; sm[2 * w + 1] = b; }
+    __syncthreads();
+    a = 0.f; b = 0.f;
+    for (int i = 0; i < TPB / 64; ++i) { a += sm[2 * i]; b += sm[2 * i + 1]; }
+}
+
+__global__ __launch_bounds__(TPB) void ln_partial_f32(const float *__restrict__ x, const float *__restrict__ res,
+                                                       float *__restrict__ part, long long n, int nblk) {
+    __shared__ float sm[2 * TPB / 64];
+    const long long b = blockIdx.y;
+    const float *xp = x + b * n;
+    const float *rp = res ? res + b * n : nullptr;
+    float s = 0.f, ss = 0.f;
+    for (long long i = (long long)blockIdx.x * TPB + threadIdx.x; i < n; i += (long long)nblk * TPB) {
+        float v = xp[i];
+        if (rp) v = __fadd_rn(v, rp[i]);
+        s += v;
+        ss += __fmul_rn(v, v);
+    }
+    block_sum2(s, ss, sm);
+    if (threadIdx.x == 0) { part[(b * nblk + blockIdx.x) * 2] = s; part[(b * nblk + blockIdx.x) * 2 + 1] = ss; }
+}
+
+__global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x, const float *__restrict__ res,
+                                                     const float *__restrict__ scale, const float *__restrict__ shift,
+                                                     float *__restrict__ y, const float *__restrict__ part, long long n,
+                                                     long long D, int nblk) {
+    const long long b = blockIdx.y;
+    float s = 0.f, ss = 0.f;
+    for (int i = 0; i < nblk; ++i) { s += part[(b * nblk + i) * 2]; ss += part[(b * nblk + i) * 2 + 1]; }
+    const float rN = __fdiv_rn(1.0f, (float)n);
+    const float mean = __fmul_rn(s, rN);
+    const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
+    const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrtf(var), 1e-5f));
+    const float *xp = x + b * n;
+    const float *rp = res ? res + b * n : nullptr;
+    float *yp = y + b * n;
+    for (long long i = (long long)blockIdx.x * TPB + threadIdx.x; i < n; i += (long long)gridDim.x * TPB) {
+        float v = xp[i];
+        if (rp) v = __fadd_rn(v, rp[i]);
+        const float c = __fadd_rn(v, -mean);
+        const float nrm = __fmul_rn(c, rden);
+        const long long d = i % D;
+        yp[i] = __fadd_rn(__fmul_rn(nrm, scale[d]), shift[d]);
+    }
+}
+
+// one workgroup per batch item, for short rows (per-token LayerNorm of the feed-forward block)
+__global__ __launch_bounds__(TPB) void ln_small_f32(const float *__restrict__ x, const float *__restrict__ res,
+                                                     const float *__restrict__ scale, const float *__restrict__ shift,
+                                                     float *__restrict__ y, long long n, long long D) {
+    __shared__ float sm[2 * TPB / 64];
+    const long long b = blockIdx.x;
+    const float *xp = x + b * n;
+    const float *rp = res ? res + b * n : nullptr;
+    float s = 0.f, ss = 0.f;
+    for (long long i = threadIdx.x; i < n; i += TPB) {
+        float v = xp[i];
+        if (rp) v = __fadd_rn(v, rp[i]);
+        s += v;
+        ss += __fmul_rn(v, v);
+    }
+    block_sum2(s, ss, sm);
+    const float rN = __fdiv_rn(1.0f, (float)n);
+    const float mean = __fmul_rn(s, rN);
+    const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
+    const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrtf(var), 1e-5f));
+    float *yp = y + b * n;
+    for (long long i = threadIdx.x; i < n; i += TPB) {
+        float v = xp[i];
+        if (rp) v = __fadd_rn(v, rp[i]);
+        const float nrm = __fmul_rn(__fadd_rn(v, -mean), rden);
+        const long long d = i % D;
+        yp[i] = __fadd_rn(__fmul_rn(nrm, scale[d]), shift[d]);
+    }
+}
+
+__global__ void bias_gelu_f32(const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ y, long long n,
+                              long long D) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        float v = x[i];
+        if (bias) v = __fadd_rn(v, bias[i % D]);
+        const float a = __fmul_rn(v, 1.702f);
+        const float t = tanhf(__fmul_rn(a, 0.5f));
+        const float sg = __fadd_rn(__fmul_rn(0.5f, t), 0.5f);
+        y[i] = __fmul_rn(v, sg);
+    }
+}
+
+template <int OP>
+int launch_unary(dl4s_hip_ctx *ctx, const float *x, float *y, int64_t n, const char *name) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(n >= 0, DL4S_HIP_EINVALID_ARG, "%s: negative count", name);
+    if (n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(x && y, DL4S_HIP_EINVALID_ARG, "%s: NULL pointer", name);
+    hipLaunchKernelGGL(unary_f32<OP>, dim3(grid_for(n)), dim3(TPB), 0, ctx->stream, x, y, (long long)n);
+    return dl4s::launch_status(name);
+}
+
+template <int OP>
+int launch_binary(dl4s_hip_ctx *ctx, const float *a, const float *b, float *y, int64_t n, const char *name) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(n >= 0, DL4S_HIP_EINVALID_ARG, "%s: negative count", name);
+    if (n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(a && b && y, DL4S_HIP_EINVALID_ARG, "%s: NULL pointer", name);
+    hipLaunchKernelGGL(binary_f32<OP>, dim3(grid_for(n)), dim3(TPB), 0, ctx->stream, a, b, y, (long long)n);
+    return dl4s::launch_status(name);
+}
+
+}  // namespace
+
+extern "C" {
+
+int dl4s_hip_fill_f32(dl4s_hip_ctx *ctx, float value, float *result, int64_t count) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(count >= 0, DL4S_HIP_EINVALID_ARG, "fill: negative count");
+    if (count == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(result, DL4S_HIP_EINVALID_ARG, "fill: NULL pointer");
+    hipLaunchKernelGGL(fill_f32, dim3(grid_for(count)), dim3(TPB), 0, ctx->stream, value, result, (long long)count);
+    return dl4s::launch_status("fill");
+}
+
+int dl4s_hip_vadd_f32(dl4s_hip_ctx *c, const float *l, const float *r, float *y, int64_t n) { return launch_binary<DL4S_OP_ADD>(c, l, r, y, n, "vAdd"); }
+int dl4s_hip_vsub_f32(dl4s_hip_ctx *c, const float *l, const float *r, float *y, int64_t n) { return launch_binary<DL4S_OP_SUB>(c, l, r, y, n, "vSub"); }
+int dl4s_hip_vmul_f32(dl4s_hip_ctx *c, const float *l, const float *r, float *y, int64_t n) { return launch_binary<DL4S_OP_MUL>(c, l, r, y, n, "vMul"); }
+int dl4s_hip_vdiv_f32(dl4s_hip_ctx *c, const float *l, const float *r, float *y, int64_t n) { return launch_binary<DL4S_OP_DIV>(c, l, r, y, n, "vDiv"); }
+int dl4s_hip_vneg_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_NEG>(c, x, y, n, "vNeg"); }
+int dl4s_hip_exp_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_EXP>(c, x, y, n, "exp"); }
+int dl4s_hip_sqrt_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_SQRT>(c, x, y, n, "sqrt"); }
+int dl4s_hip_relu_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_RELU>(c, x, y, n, "relu"); }
+int dl4s_hip_tanh_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_TANH>(c, x, y, n, "tanh"); }
+
+int dl4s_hip_broadcast_f32(dl4s_hip_ctx *ctx, int op, const float *lhs, const int64_t *lhs_shape, int lhs_dim,
+                           const float *rhs, const int64_t *rhs_shape, int rhs_dim, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(op >= DL4S_OP_ADD && op <= DL4S_OP_DIV, DL4S_HIP_EINVALID_ARG, "broadcast: unknown op %d", op);
+    DL4S_REQUIRE(lhs_dim >= 0 && rhs_dim >= 0 && lhs_dim <= DL4S_HIP_MAX_DIM && rhs_dim <= DL4S_HIP_MAX_DIM,
+                 DL4S_HIP_EINVALID_ARG, "broadcast: rank outside [0,%d]", DL4S_HIP_MAX_DIM);
+    DL4S_REQUIRE((lhs_dim == 0 || lhs_shape) && (rhs_dim == 0 || rhs_shape), DL4S_HIP_EINVALID_ARG, "broadcast: NULL shape");
+    const int dim = lhs_dim > rhs_dim ? lhs_dim : rhs_dim;
+    long long ls[DL4S_HIP_MAX_DIM], rs[DL4S_HIP_MAX_DIM];
+    Bcast bc{};
+    bc.dim = dim;
+    long long n = 1;
+    for (int i = 0; i < dim; ++i) {
+        ls[i] = i < dim - lhs_dim ? 1 : lhs_shape[i - (dim - lhs_dim)];
+        rs[i] = i < dim - rhs_dim ? 1 : rhs_shape[i - (dim - rhs_dim)];
+        DL4S_REQUIRE(ls[i] >= 0 && rs[i] >= 0, DL4S_HIP_EINVALID_ARG, "broadcast: negative extent");
+        DL4S_REQUIRE(ls[i] == rs[i] || ls[i] == 1 || rs[i] == 1, DL4S_HIP_ESHAPE,
+                     "broadcast: axis %d has sizes %lld and %lld", i, ls[i], rs[i]);
+        bc.oshape[i] = ls[i] > rs[i] ? ls[i] : rs[i];
+        if (ls[i] == 0 || rs[i] == 0) bc.oshape[i] = 0;
+        n *= bc.oshape[i];
+    }
+    if (n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(lhs && rhs && result, DL4S_HIP_EINVALID_ARG, "broadcast: NULL pointer");
+    long long lstride = 1, rstride = 1;
+    for (int i = dim - 1; i >= 0; --i) {
+        bc.ls[i] = ls[i] == 1 ? 0 : lstride;
+        bc.rs[i] = rs[i] == 1 ? 0 : rstride;
+        lstride *= ls[i];
+        rstride *= rs[i];
+    }
+    // mode selection of Engine/CPU/CPUEngine.swift:117-176
+    long long sc = 1;
+    for (int i = dim - 1; i >= 0 && ls[i] == rs[i]; --i) sc *= ls[i];
+    int mode = 0;
+    if (sc <= 1)
+        for (int i = dim - 1; i >= 0; --i) {
+            if (ls[i] > rs[i]) { mode = 2; break; }
+            if (rs[i] > ls[i]) { mode = 1; break; }
+        }
+    const dim3 g(grid_for(n, 2)), b(TPB);
+    switch (op) {
+        case DL4S_OP_ADD: hipLaunchKernelGGL(broadcast_f32<DL4S_OP_ADD>, g, b, 0, ctx->stream, lhs, rhs, result, bc, mode, n); break;
+        case DL4S_OP_SUB: hipLaunchKernelGGL(broadcast_f32<DL4S_OP_SUB>, g, b, 0, ctx->stream, lhs, rhs, result, bc, mode, n); break;
+        case DL4S_OP_MUL: hipLaunchKernelGGL(broadcast_f32<DL4S_OP_MUL>, g, b, 0, ctx->stream, lhs, rhs, result, bc, mode, n); break;
+        default: hipLaunchKernelGGL(broadcast_f32<DL4S_OP_DIV>, g, b, 0, ctx->stream, lhs, rhs, result, bc, mode, n); break;
+    }
+    return dl4s::launch_status("broadcast");
+}
+
+static int reduce_common(dl4s_hip_ctx *ctx, bool is_max, const float *values, const int64_t *shape, int dim,
+                         const int32_t *axes, int naxes, float *result) {
+    DL4S_REQUIRE(dim >= 0 && dim <= DL4S_HIP_MAX_DIM, DL4S_HIP_EINVALID_ARG, "reduce: rank outside [0,%d]", DL4S_HIP_MAX_DIM);
+    DL4S_REQUIRE(naxes >= 0 && naxes <= dim && (dim == 0 || shape) && (naxes == 0 || axes), DL4S_HIP_EINVALID_ARG,
+                 "reduce: bad axes");
+    bool red[DL4S_HIP_MAX_DIM] = {false};
+    for (int i = 0; i < naxes; ++i) {
+        DL4S_REQUIRE(axes[i] >= 0 && axes[i] < dim && !red[axes[i]], DL4S_HIP_EINVALID_ARG, "reduce: axis %d invalid or repeated", axes[i]);
+        red[axes[i]] = true;
+    }
+    Reduce rd{};
+    long long stride[DL4S_HIP_MAX_DIM], s = 1, nout = 1;
+    for (int i = dim - 1; i >= 0; --i) {
+        DL4S_REQUIRE(shape[i] >= 0, DL4S_HIP_EINVALID_ARG, "reduce: negative extent");
+        stride[i] = s;
+        s *= shape[i];
+    }
+    rd.rcount = 1;
+    for (int i = 0; i < dim; ++i) {
+        if (red[i]) { rd.rshape[rd.rdim] = shape[i]; rd.rstride[rd.rdim] = stride[i]; rd.rcount *= shape[i]; ++rd.rdim; }
+        else { rd.kshape[rd.kdim] = shape[i]; rd.kstride[rd.kdim] = stride[i]; nout *= shape[i]; ++rd.kdim; }
+    }
+    if (nout == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(values && result, DL4S_HIP_EINVALID_ARG, "reduce: NULL pointer");
+    DL4S_REQUIRE(nout < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "reduce: too many output elements");
+    if (is_max) hipLaunchKernelGGL(reduce_f32<true>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, values, result, rd);
+    else hipLaunchKernelGGL(reduce_f32<false>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, values, result, rd);
+    return dl4s::launch_status("reduce");
+}
+
+int dl4s_hip_reduce_sum_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim, const int32_t *axes,
+                            int naxes, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    return reduce_common(ctx, false, values, shape, dim, axes, naxes, result);
+}
+
+int dl4s_hip_reduce_max_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim, int axis, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    int32_t ax = axis;
+    return reduce_common(ctx, true, values, shape, dim, &ax, 1, result);
+}
+
+int dl4s_hip_permute_axes_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim,
+                              const int32_t *arrangement, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(dim >= 0 && dim <= DL4S_HIP_MAX_DIM && (dim == 0 || (shape && arrangement)), DL4S_HIP_EINVALID_ARG,
+                 "permuteAxes: bad rank or NULL shape");
+    Permute p{};
+    p.dim = dim;
+    long long dshape[DL4S_HIP_MAX_DIM], dstr[DL4S_HIP_MAX_DIM], n = 1;
+    bool seen[DL4S_HIP_MAX_DIM] = {false};
+    for (int i = 0; i < dim; ++i) {
+        const int a = arrangement[i];
+        DL4S_REQUIRE(a >= 0 && a < dim && !seen[a], DL4S_HIP_EINVALID_ARG, "permuteAxes: arrangement is not a permutation");
+        DL4S_REQUIRE(shape[i] >= 0, DL4S_HIP_EINVALID_ARG, "permuteAxes: negative extent");
+        seen[a] = true;
+        dshape[a] = shape[i];
+        p.sshape[i] = shape[i];
+        n *= shape[i];
+    }
+    if (n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(values && result, DL4S_HIP_EINVALID_ARG, "permuteAxes: NULL pointer");
+    long long s = 1;
+    for (int i = dim - 1; i >= 0; --i) { dstr[i] = s; s *= dshape[i]; }
+    for (int i = 0; i < dim; ++i) p.dstride[i] = dstr[arrangement[i]];
+    hipLaunchKernelGGL(permute_f32, dim3(grid_for(n, 2)), dim3(TPB), 0, ctx->stream, values, result, p, n);
+    return dl4s::launch_status("permuteAxes");
+}
+
+int dl4s_hip_band_f32(dl4s_hip_ctx *ctx, const float *buffer, float *result, int64_t rows, int64_t cols, int has_below,
+                      int64_t below, int has_above, int64_t above) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(rows >= 0 && cols >= 0, DL4S_HIP_EINVALID_ARG, "band: negative extent");
+    if (rows * cols == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(buffer && result, DL4S_HIP_EINVALID_ARG, "band: NULL pointer");
+    const long long mx = rows > cols ? rows : cols;
+    hipLaunchKernelGGL(band_f32, dim3(grid_for(rows * cols, 2)), dim3(TPB), 0, ctx->stream, buffer, result, (long long)rows,
+                       (long long)cols, has_below ? (long long)below : mx, has_above ? (long long)above : mx);
+    return dl4s::launch_status("band");
+}
+
+int dl4s_hip_stack_f32(dl4s_hip_ctx *ctx, const float *const *buffers, int64_t n, int64_t count, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(n >= 0 && count >= 0, DL4S_HIP_EINVALID_ARG, "stack: negative extent");
+    if (n * count == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(buffers && result, DL4S_HIP_EINVALID_ARG, "stack: NULL pointer");
+    for (int64_t i = 0; i < n; ++i) {
+        DL4S_REQUIRE(buffers[i], DL4S_HIP_EINVALID_ARG, "stack: buffer %lld is NULL", (long long)i);
+        DL4S_HIP_TRY(hipMemcpyAsync(result + i * count, buffers[i], (size_t)count * sizeof(float), hipMemcpyDeviceToDevice, ctx->stream));
+    }
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *residual, const float *scale, const float *shift,
+                           float *result, int64_t B, int64_t rows, int64_t D) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(B >= 0 && rows >= 0 && D >= 0, DL4S_HIP_EINVALID_ARG, "layernorm: negative extent");
+    const long long n = rows * D;
+    if (B * n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(x && scale && shift && result, DL4S_HIP_EINVALID_ARG, "layernorm: NULL pointer");
+    DL4S_REQUIRE(B < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "layernorm: batch too large");
+    if (n <= 16384) {
+        hipLaunchKernelGGL(ln_small_f32, dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+        return dl4s::launch_status("layernorm");
+    }
+    DL4S_REQUIRE(B <= 65535, DL4S_HIP_EUNSUPPORTED, "layernorm: batch above 65535 with long rows");
+    long long want = n / (TPB * 8);
+    int nblk = (int)(want < 1 ? 1 : (want > 256 ? 256 : want));
+    int rc = dl4s::ensure_scratch(ctx, (size_t)B * nblk * 2 * sizeof(float));
+    if (rc) return rc;
+    float *part = reinterpret_cast<float *>(ctx->scratch);
+    hipLaunchKernelGGL(ln_partial_f32, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, part, n, nblk);
+    hipLaunchKernelGGL(ln_apply_f32, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, part, n,
+                       (long long)D, nblk);
+    return dl4s::launch_status("layernorm");
+}
+
+int dl4s_hip_bias_gelu_f32(dl4s_hip_ctx *ctx, const float *x, const float *bias, float *result, int64_t rows, int64_t D) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(rows >= 0 && D >= 0, DL4S_HIP_EINVALID_ARG, "bias_gelu: negative extent");
+    const long long n = rows * D;
+    if (n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(x && result, DL4S_HIP_EINVALID_ARG, "bias_gelu: NULL pointer");
+    hipLaunchKernelGGL(bias_gelu_f32, dim3(grid_for(n)), dim3(TPB), 0, ctx->stream, x, bias, result, n, (long long)D);
+    return dl4s::launch_status("bias_gelu");
+}
+
+}  // extern "C"

@@ -1,0 +1,407 @@
+// Fused attention forward for gfx950: out = softmax((q * rT) . k^T - mask * 1e9) . v
+//
+// sdpa_prefill_f32_d64 is the hot kernel (head dim 64).  One workgroup = 4 wavefronts = 128
+// queries of one (batch, head); each wavefront owns 32 queries and walks the keys in LDS tiles of
+// 64.  Both contractions run on v_mfma_f32_32x32x2_f32 and are set up TRANSPOSED so that the
+// probabilities never leave the registers they were computed in:
+//
+//   S^T[key, query] = K[key, :] . Q[query, :]      A operand = K (from LDS), B operand = Q (registers)
+//   O^T[d,   query] = V[key, d]^T . P^T[key, query] A operand = V (from LDS), B operand = P (the S^T
+//                                                   accumulator registers, used as they are)
+//
+// In the 32x32 accumulator layout lane l holds column (l % 32) = one query and 16 rows = 16 keys,
+// which is exactly the B-operand layout of the second contraction (k = l / 32, n = l % 32) once
+// the key order inside a tile is permuted consistently for V.  The row maximum and row sum are
+// therefore 16 in-lane operations plus one exchange with lane l ^ 32.
+//
+// The scale is applied to Q once (q * rT), as the reference does before its first matrix product
+// (NN/Models/Transformer/ScaledDotProductAttention.swift:53); the mask is applied in registers as
+// s - m * 1e9 (ibid. :55-57) before the running maximum; normalisation by the row sum is deferred
+// to the end.  Keys beyond Lk contribute nothing; queries beyond Lq are computed and not stored.
+#include "common.h"
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int HD = 64;       // head dim of the MFMA kernel
+constexpr int BM = 128;      // queries per workgroup
+constexpr int BN = 64;       // keys per LDS tile
+constexpr int LSTR = 68;     // LDS row stride in floats: 64 + 4 keeps 128-bit reads of 8 rows on distinct banks
+constexpr int TILE_FLOATS = BN * LSTR;
+constexpr float LOG2E = 1.44269504088896340736f;
+
+struct MaskArgs {
+    int kind;
+    const float *dense;
+    long long sb, sh, sq, sk;  // element strides of the dense mask, 0 on broadcast axes
+    const int *lengths;
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__restrict__ q,
+                                                                const float *__restrict__ k,
+                                                                const float *__restrict__ v,
+                                                                float *__restrict__ out, int H, int Lq,
+                                                                int Lk, float rT, MaskArgs mask, int strict,
+                                                                int nqb, int total_blocks) {
+    extern __shared__ __align__(16) float lds[];
+    float *Ks = lds;                     // [2][BN][LSTR]
+    float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
+
+    // Workgroups are handed to the 8 XCDs round-robin by index: give every XCD one contiguous run of
+    // the (batch*head)-major work order so that the workgroups sharing a K/V pair share an L2.
+    const int chunk = (total_blocks + 7) / 8;
+    const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
+    if (w >= total_blocks) return;
+    const int bh = w / nqb;
+    const int qb = nqb - 1 - (w % nqb);  // longest causal rows first
+    const int b = bh / H;
+    const int hh = bh % H;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int half = lane >> 5;
+    const int ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int q0 = qb * BM + wave * 32;  // first query of this wavefront
+    const int qi = q0 + ln;
+    const int qic = qi < Lq ? qi : Lq - 1;
+
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+
+    // Keys this workgroup / wavefront has to visit.  Skipping is exact when every row keeps at least one
+    // unblocked key (true unless len == 0) and K, V are finite at blocked keys.
+    int kend = Lk, wkend = Lk;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) {
+            kend = min(kend, qb * BM + BM);
+            wkend = min(wkend, q0 + 32);
+        }
+        if (LENS) {
+            kend = min(kend, len);
+            wkend = min(wkend, len);
+        }
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    // Q fragment: lane holds Q[qi][half*32 + s] * rT for s = 0..31 (one rounding, like the reference)
+    float qr[32];
+    {
+        const float *qp = q + ((long long)bh * Lq + qic) * HD + half * 32;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+            qr[4 * j + 0] = t.x * rT;
+            qr[4 * j + 1] = t.y * rT;
+            qr[4 * j + 2] = t.z * rT;
+            qr[4 * j + 3] = t.w * rT;
+        }
+    }
+
+    // global -> LDS staging: thread covers rows (i*16 + tid/16), 4 floats at column (tid%16)*4
+    const int ld_row = tid >> 4;
+    const int ld_col = (tid & 15) * 4;
+    const float *kbase = k + (long long)bh * Lk * HD + ld_col;
+    const float *vbase = v + (long long)bh * Lk * HD + ld_col;
+    f32x4 kst[4], vst[4];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int row = t * BN + i * 16 + ld_row;
+            row = row < Lk ? row : Lk - 1;
+            kst[i] = *reinterpret_cast<const f32x4 *>(kbase + (long long)row * HD);
+            vst[i] = *reinterpret_cast<const f32x4 *>(vbase + (long long)row * HD);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int off = buf * TILE_FLOATS + (i * 16 + ld_row) * LSTR + ld_col;
+            *reinterpret_cast<f32x4 *>(Ks + off) = kst[i];
+            *reinterpret_cast<f32x4 *>(Vs + off) = vst[i];
+        }
+    };
+
+    f32x16 o0, o1;  // O^T rows d = 2*m + {0,1}
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { o0[i] = 0.f; o1[i] = 0.f; }
+    float m_run = -INFINITY;
+    float l_run = 0.f;
+
+    if (ntiles > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+
+    const int k_lds = ln * LSTR + half * 32;        // K fragment base: row ln, columns half*32..
+    const int v_lds = (4 * half) * LSTR + 2 * ln;   // V fragment base: row 4*half (+ const), columns 2*ln, 2*ln+1
+
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        const bool more = (t + 1 < ntiles);
+        if (more) load_tile(t + 1);
+        const int k0 = t * BN;
+
+        if (k0 < wkend) {
+            // ---- S^T = K . Q^T for two 32-key sub-tiles
+            f32x16 s0, s1;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+            const float *Kb = Ks + buf * TILE_FLOATS + k_lds;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
+                f32x4 a1 = *reinterpret_cast<const f32x4 *>(Kb + 32 * LSTR + 4 * j);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.x, qr[4 * j + 0], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.y, qr[4 * j + 1], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, qr[4 * j + 2], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.z, qr[4 * j + 2], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.w, qr[4 * j + 3], s1, 0, 0, 0);
+            }
+
+            // ---- mask, in registers.  Accumulator register r of sub-tile u is key k0 + 32u + 8(r/4) + 4*half + r%4.
+            const bool need_mask = DENSE || (CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len)) || (k0 + BN > Lk);
+            if (need_mask) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int kg = k0 + 32 * u + 8 * (r >> 2) + 4 * half + (r & 3);
+                        float s = u == 0 ? s0[r] : s1[r];
+                        if (DENSE) {
+                            const int kc = kg < Lk ? kg : Lk - 1;
+                            const float mval = mask.dense[b * mask.sb + hh * mask.sh + qic * mask.sq + kc * mask.sk];
+                            s = __fsub_rn(s, __fmul_rn(mval, 1e9f));
+                        } else {
+                            bool blocked = false;
+                            if (CAUSAL) blocked = blocked || (kg > qi);
+                            if (LENS) blocked = blocked || (kg >= len);
+                            if (blocked) s = __fsub_rn(s, 1e9f);
+                        }
+                        if (kg >= Lk) s = -INFINITY;
+                        if (u == 0) s0[r] = s; else s1[r] = s;
+                    }
+                }
+            }
+
+            // ---- online softmax: lane (query ln) sees 32 of the 64 keys, lane ^ 32 the other 32
+            float tmax = fmaxf(s0[0], s1[0]);
+#pragma unroll
+            for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, fmaxf(s0[r], s1[r]));
+            tmax = fmaxf(tmax, xor32(tmax));
+            const float m_new = fmaxf(m_run, tmax);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a row of -inf so far: weights 0, not NaN
+            const float alpha = fast_exp2((m_run - m_use) * LOG2E);
+            m_run = m_new;
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                s0[r] = fast_exp2((s0[r] - m_use) * LOG2E);
+                s1[r] = fast_exp2((s1[r] - m_use) * LOG2E);
+                psum += s0[r] + s1[r];
+            }
+            l_run = l_run * alpha + psum;
+            if (__any(alpha != 1.0f)) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { o0[i] *= alpha; o1[i] *= alpha; }
+            }
+
+            // ---- O^T += V^T . P^T
+            const float *Vb = Vs + buf * TILE_FLOATS + v_lds;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = 8 * (r >> 2) + (r & 3);  // + 4*half, folded into v_lds
+                f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + key * LSTR);
+                o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s0[r], o0, 0, 0, 0);
+                o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s0[r], o1, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = 32 + 8 * (r >> 2) + (r & 3);
+                f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + key * LSTR);
+                o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s1[r], o0, 0, 0, 0);
+                o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s1[r], o1, 0, 0, 0);
+            }
+        }
+
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and store.  Register r of o0/o1 is d = 2*(8(r/4) + 4*half + r%4) + {0,1}.
+    const float l_tot = l_run + xor32(l_run);
+    const float inv = 1.0f / l_tot;
+    if (qi < Lq) {
+        float *op = out + ((long long)bh * Lq + qi) * HD + 8 * half;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            f32x4 a, c;
+            a.x = o0[4 * g + 0] * inv; a.y = o1[4 * g + 0] * inv;
+            a.z = o0[4 * g + 1] * inv; a.w = o1[4 * g + 1] * inv;
+            c.x = o0[4 * g + 2] * inv; c.y = o1[4 * g + 2] * inv;
+            c.z = o0[4 * g + 3] * inv; c.w = o1[4 * g + 3] * inv;
+            *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
+            *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
+        }
+    }
+}
+
+// Plain fused kernel for head dims other than 64 (up to 256): one wavefront per query row, two passes over
+// the keys like the reference's softmax (max, then exp / sum), keys handled 64 at a time through LDS.
+constexpr int GEN_MAXD = 256;
+__global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__ q, const float *__restrict__ k,
+                                                        const float *__restrict__ v, float *__restrict__ out, int H,
+                                                        int Lq, int Lk, int dk, int dv, float rT, MaskArgs mask) {
+    __shared__ float qs[GEN_MAXD];
+    __shared__ float ps[64];
+    const int row = blockIdx.x;  // over B*H*Lq
+    const int qi = row % Lq;
+    const int bh = row / Lq;
+    const int b = bh / H, hh = bh % H;
+    const int lane = threadIdx.x;
+    for (int c = lane; c < dk; c += 64) qs[c] = q[(long long)row * dk + c] * rT;
+    __syncthreads();
+    const float *kp = k + (long long)bh * Lk * dk;
+    const float *vp = v + (long long)bh * Lk * dv;
+    int len = Lk;
+    if (mask.kind == DL4S_MASK_KEY_LENGTHS || mask.kind == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS) len = mask.lengths[b];
+    auto score = [&](int j) {
+        float s = 0.f;
+        for (int c = 0; c < dk; ++c) s = __fadd_rn(s, __fmul_rn(qs[c], kp[(long long)j * dk + c]));
+        switch (mask.kind) {
+            case DL4S_MASK_DENSE_F32: {
+                float mval = mask.dense[b * mask.sb + hh * mask.sh + qi * mask.sq + j * mask.sk];
+                s = __fsub_rn(s, __fmul_rn(mval, 1e9f));
+                break;
+            }
+            case DL4S_MASK_CAUSAL: if (j > qi) s = __fsub_rn(s, 1e9f); break;
+            case DL4S_MASK_KEY_LENGTHS: if (j >= len) s = __fsub_rn(s, 1e9f); break;
+            case DL4S_MASK_CAUSAL_OR_KEY_LENGTHS: if (j > qi || j >= len) s = __fsub_rn(s, 1e9f); break;
+            default: break;
+        }
+        return s;
+    };
+    float mx = -INFINITY;
+    for (int j = lane; j < Lk; j += 64) mx = fmaxf(mx, score(j));
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float acc[GEN_MAXD / 64];
+    for (int i = 0; i < GEN_MAXD / 64; ++i) acc[i] = 0.f;
+    float sum = 0.f;
+    for (int j0 = 0; j0 < Lk; j0 += 64) {
+        const int j = j0 + lane;
+        float p = 0.f;
+        if (j < Lk) p = expf(score(j) - mx);   // -inf - -inf = NaN for an all -inf row, like the reference
+        sum += p;
+        ps[lane] = p;
+        __syncthreads();
+        const int n = min(64, Lk - j0);
+        for (int i = 0; i < GEN_MAXD / 64; ++i) {
+            const int c = lane + 64 * i;
+            if (c < dv)
+                for (int jj = 0; jj < n; ++jj) acc[i] += ps[jj] * vp[(long long)(j0 + jj) * dv + c];
+        }
+        __syncthreads();
+    }
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    const float inv = 1.0f / sum;
+    for (int i = 0; i < GEN_MAXD / 64; ++i) {
+        const int c = lane + 64 * i;
+        if (c < dv) out[(long long)row * dv + c] = acc[i] * inv;
+    }
+}
+
+template <int KIND>
+int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq,
+               int Lk, float rT, const MaskArgs &m, int strict) {
+    const int nqb = (Lq + BM - 1) / BM;
+    const long long total = (long long)nqb * B * H;
+    DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
+    const int chunk = (int)((total + 7) / 8);
+    const size_t lds_bytes = 4 * TILE_FLOATS * sizeof(float);
+    static bool attr_set[8] = {false};
+    if (!attr_set[KIND]) {
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_prefill_f32_d64<KIND>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        attr_set[KIND] = true;
+    }
+    hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
+                       Lq, Lk, rT, m, strict, nqb, (int)total);
+    return dl4s::launch_status("sdpa_prefill_f32_d64");
+}
+
+}  // namespace
+
+extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
+                                     int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
+                                     float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(B >= 0 && H >= 0 && Lq >= 0 && Lk >= 0 && dk >= 0 && dv >= 0, DL4S_HIP_EINVALID_ARG,
+                 "sdpa: negative extent");
+    if (B * H * Lq * dv == 0) return DL4S_HIP_OK;  // nothing to write
+    DL4S_REQUIRE(q && k && v && out, DL4S_HIP_EINVALID_ARG, "sdpa: NULL tensor pointer");
+    DL4S_REQUIRE(Lk > 0, DL4S_HIP_ESHAPE, "sdpa: keyCount is 0 (softmax over an empty axis)");
+    DL4S_REQUIRE(dk > 0, DL4S_HIP_ESHAPE, "sdpa: keyDim is 0");
+    DL4S_REQUIRE(B * H * (Lq > Lk ? Lq : Lk) * (dk > dv ? dk : dv) < (1ll << 40) && Lq < (1ll << 30) && Lk < (1ll << 30),
+                 DL4S_HIP_EUNSUPPORTED, "sdpa: extents too large");
+    MaskArgs m{};
+    m.kind = mask ? mask->kind : DL4S_MASK_NONE;
+    switch (m.kind) {
+        case DL4S_MASK_NONE: break;
+        case DL4S_MASK_DENSE_F32: {
+            DL4S_REQUIRE(mask->dense, DL4S_HIP_EINVALID_ARG, "sdpa: dense mask pointer is NULL");
+            const int64_t full[4] = {B, H, Lq, Lk};
+            long long stride = 1, st[4];
+            for (int i = 3; i >= 0; --i) {
+                DL4S_REQUIRE(mask->shape[i] == 1 || mask->shape[i] == full[i], DL4S_HIP_ESHAPE,
+                             "sdpa: mask axis %d has size %lld, expected 1 or %lld", i, (long long)mask->shape[i],
+                             (long long)full[i]);
+                st[i] = mask->shape[i] == 1 ? 0 : stride;
+                stride *= mask->shape[i];
+            }
+            m.dense = mask->dense;
+            m.sb = st[0]; m.sh = st[1]; m.sq = st[2]; m.sk = st[3];
+            break;
+        }
+        case DL4S_MASK_KEY_LENGTHS:
+        case DL4S_MASK_CAUSAL_OR_KEY_LENGTHS:
+            DL4S_REQUIRE(mask->lengths, DL4S_HIP_EINVALID_ARG, "sdpa: lengths pointer is NULL");
+            m.lengths = mask->lengths;
+            break;
+        case DL4S_MASK_CAUSAL: break;
+        default: return dl4s::set_error(DL4S_HIP_EINVALID_ARG, "sdpa: unknown mask kind %d", m.kind);
+    }
+    const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
+    if (dk == HD && dv == HD) {
+        switch (m.kind) {
+            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
+            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
+            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
+            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
+            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
+        }
+    }
+    DL4S_REQUIRE(dk <= GEN_MAXD && dv <= GEN_MAXD && dv > 0, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa: head dims (%lld, %lld) above %d are not implemented", (long long)dk, (long long)dv, GEN_MAXD);
+    const long long rows = B * H * Lq;
+    DL4S_REQUIRE(rows < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "sdpa: too many rows for the plain kernel");
+    hipLaunchKernelGGL(sdpa_generic_f32, dim3((unsigned)rows), dim3(64), 0, ctx->stream, q, k, v, out, (int)H, (int)Lq,
+                       (int)Lk, (int)dk, (int)dv, inv_temperature, m);
+    return dl4s::launch_status("sdpa_generic_f32");
+}

@@ -1,0 +1,194 @@
+/*
+ * dl4s_hip.h -- C ABI of libdl4s_hip.so: an MI355X (gfx950) backend for the attention
+ * forward path of DL4S (ScaledDotProductAttention / MultiHeadAttention and the engine
+ * primitives those layers call), fp32, one GPU.
+ *
+ * The library owns the device context, one HIP stream, a pooled allocator and every kernel
+ * launch.  Handles are raw device pointers; an offset view is plain pointer arithmetic and is
+ * never passed to dl4s_hip_free.  Every function is callable from any thread, returns 0 on
+ * success or a negative dl4s_hip_status, never aborts and never throws across the ABI; the
+ * message for the last failure on the calling thread is dl4s_hip_last_error().
+ *
+ * Compute entry points only ENQUEUE work on the context's stream.  Results are visible to a
+ * following dl4s_hip_assign_d2h / dl4s_hip_get_value (which wait for the stream) or after
+ * dl4s_hip_sync.  Host pointers handed to dl4s_hip_assign_h2d may be reused as soon as the
+ * call returns.
+ *
+ * Citations are to the reference sources, relative to Sources/DL4S/.
+ */
+#ifndef DL4S_HIP_H
+#define DL4S_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dl4s_hip_ctx dl4s_hip_ctx;
+
+typedef enum dl4s_hip_status {
+    DL4S_HIP_OK = 0,
+    DL4S_HIP_EINVALID_ARG = -1, /* null pointer, negative size, unknown enum value */
+    DL4S_HIP_ESHAPE = -2,       /* operand shapes do not fit each other (the reference traps with precondition) */
+    DL4S_HIP_EOOM = -3,         /* device allocation failed */
+    DL4S_HIP_EHIP = -4,         /* a HIP runtime call failed; the message holds hipGetErrorString */
+    DL4S_HIP_EUNSUPPORTED = -5  /* valid request outside what this backend implements */
+} dl4s_hip_status;
+
+#define DL4S_HIP_MAX_DIM 8
+
+/* ------------------------------------------------------------------ context / device */
+/* Engine/Engine.swift:30-35 (DeviceType): one context stands for the `HIP` device type. */
+int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx);
+int dl4s_hip_destroy(dl4s_hip_ctx *ctx);
+const char *dl4s_hip_last_error(void);
+int dl4s_hip_sync(dl4s_hip_ctx *ctx);
+/* Number of compute units and device name (for roofline reports). */
+int dl4s_hip_device_info(dl4s_hip_ctx *ctx, int *out_cu_count, int *out_clock_khz, char *name_buf, size_t name_len);
+/* Stream-ordered timer on the context's stream (HIP events): begin, enqueue work, end.
+ * dl4s_hip_timer_end waits for the stop event and returns the elapsed milliseconds. */
+int dl4s_hip_timer_begin(dl4s_hip_ctx *ctx);
+int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms);
+
+/* ------------------------------------------------------- MemoryOperatorsType subset */
+/* Engine/Engine.swift:49,55 allocateBuffer.  Memory is NOT zeroed (the reference's is not either,
+ * Engine/CPU/CPU.swift:71-96).  bytes == 0 yields a valid unique pointer. */
+int dl4s_hip_alloc(dl4s_hip_ctx *ctx, size_t bytes, void **out_ptr);
+/* Engine/Engine.swift:59,63 free.  Stream-ordered: the block returns to the pool and may be
+ * handed out again at once, because every consumer runs on the one stream
+ * (Tensor/Tensor.swift:38-42 frees from deinit right after the last use was enqueued). */
+int dl4s_hip_free(dl4s_hip_ctx *ctx, void *ptr);
+/* Engine/Engine.swift:70 assign(from: UnsafeBufferPointer, to: Buffer) -- host to device. */
+int dl4s_hip_assign_h2d(dl4s_hip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+/* Engine/Engine.swift:77 assign(from: Buffer, to: Buffer) -- device to device. */
+int dl4s_hip_assign_d2d(dl4s_hip_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
+/* Engine/Engine.swift:84 assign(from: Buffer, to: UnsafeMutableBufferPointer) -- device to host; waits. */
+int dl4s_hip_assign_d2h(dl4s_hip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+/* Engine/Engine.swift:88 getValue / :132 setPointee, for Float. */
+int dl4s_hip_get_value_f32(dl4s_hip_ctx *ctx, const float *src_dev, float *out_value);
+int dl4s_hip_set_pointee_f32(dl4s_hip_ctx *ctx, float *dst_dev, float value);
+/* Engine/Engine.swift:92 getSize: bytes from ptr to the end of its allocation (works for offset views). */
+int dl4s_hip_get_size(dl4s_hip_ctx *ctx, const void *ptr, size_t *out_bytes);
+/* Bytes currently handed out / held by the pool (leak checks; Engine/CPU/CPU.swift:38-44 traces the same). */
+int dl4s_hip_mem_stats(dl4s_hip_ctx *ctx, size_t *out_bytes_in_use, size_t *out_bytes_pooled);
+
+/* ------------------------------------------------------------ fused attention entry */
+/* Mask descriptor.  The reference takes a dense float tensor (1 = blocked, 0 = keep, any value is
+ * a scaled penalty) broadcastable to [B,H,Lq,Lk] and computes  scores - mask * 1e9
+ * (NN/Models/Transformer/ScaledDotProductAttention.swift:55-57).  DENSE_F32 is that tensor;
+ * the structured kinds describe the masks TransformerUtil.swift:29-50 builds without
+ * materialising them and give bit-identical results to DENSE_F32 on the same logical mask. */
+typedef enum dl4s_mask_kind {
+    DL4S_MASK_NONE = 0,
+    DL4S_MASK_DENSE_F32 = 1,             /* dense: device ptr + shape[4], a 1 in shape = broadcast axis */
+    DL4S_MASK_CAUSAL = 2,                /* blocked where key j > query i (bandMatrix(below:-1, above:nil)) */
+    DL4S_MASK_KEY_LENGTHS = 3,           /* blocked where key j >= lengths[b] (makeEncoderMasks) */
+    DL4S_MASK_CAUSAL_OR_KEY_LENGTHS = 4  /* union of the two (makeDecoderMasks) */
+} dl4s_mask_kind;
+
+typedef struct dl4s_mask_desc {
+    int32_t kind;            /* dl4s_mask_kind */
+    const float *dense;      /* DENSE_F32: device pointer, row-major, shape below */
+    int64_t shape[4];        /* DENSE_F32: right-aligned to [B,H,Lq,Lk]; each entry is 1 or the full size */
+    const int32_t *lengths;  /* KEY_LENGTHS kinds: device pointer to B valid lengths */
+} dl4s_mask_desc;
+
+/* flags for dl4s_hip_sdpa_fwd_f32 */
+#define DL4S_SDPA_STRICT 1u /* visit every key tile even where a structured mask blocks all of it.  Without it
+                               fully blocked tiles are skipped, which is exact as long as K and V hold finite
+                               values at blocked positions (the reference computes 0 * v there, so a NaN/Inf in
+                               V or K at a blocked key reaches the output only in strict mode). */
+
+/* out = softmax((q * inv_temperature) . k^T - mask * 1e9, axis = keys) . v
+ * NN/Models/Transformer/ScaledDotProductAttention.swift:43-64.  q [B,H,Lq,dk], k [B,H,Lk,dk],
+ * v [B,H,Lk,dv], out [B,H,Lq,dv], all row-major contiguous device fp32.  inv_temperature is the
+ * fp32 reciprocal the reference forms once (Engine/CPU/CPUEngine.swift:635).  mask may be NULL
+ * (= DL4S_MASK_NONE).  dk = dv = 64 runs the fused MFMA kernel; other sizes up to 256 run a
+ * plain fused kernel. */
+int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
+                          int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
+                          float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
+
+/* One decode step: the same attention with Lq = 1 over the first T rows of a key/value cache laid
+ * out [B,H,Tcap,d] (d = 64).  q, out [B,H,1,d].  The reference has no cache (greedy decoding re-runs
+ * the prefix, NN/Models/Transformer/Transformer.swift:118-137); the result equals its
+ * ScaledDotProductAttention on the gathered [B,H,T,d] tensors, no mask. */
+int dl4s_hip_sdpa_decode_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache,
+                             float *out, int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d,
+                             float inv_temperature);
+/* Writes k_new, v_new [B,H,1,d] into row `pos` of the caches [B,H,Tcap,d]
+ * (replaces the concatenation a cache-less caller would do with Engine.stack). */
+int dl4s_hip_kv_append_f32(dl4s_hip_ctx *ctx, float *kcache, float *vcache, const float *k_new,
+                           const float *v_new, int64_t B, int64_t H, int64_t pos, int64_t Tcap, int64_t d);
+/* Append at row `pos`, then attend over rows 0..pos (T = pos + 1) in one call. */
+int dl4s_hip_sdpa_decode_step_f32(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcache,
+                                  const float *k_new, const float *v_new, float *out, int64_t B, int64_t H,
+                                  int64_t pos, int64_t Tcap, int64_t d, float inv_temperature);
+
+/* ------------------------------------------------------------------ EngineType subset */
+/* The primitives the layers on the path call (Engine/Engine.swift:143-581); fp32 only.
+ * `result` may alias an input wherever the reference allows it (same-shape elementwise ops). */
+int dl4s_hip_fill_f32(dl4s_hip_ctx *ctx, float value, float *result, int64_t count);                     /* :153 */
+int dl4s_hip_vadd_f32(dl4s_hip_ctx *ctx, const float *lhs, const float *rhs, float *result, int64_t count); /* :161 */
+int dl4s_hip_vneg_f32(dl4s_hip_ctx *ctx, const float *val, float *result, int64_t count);                /* :168 */
+int dl4s_hip_vsub_f32(dl4s_hip_ctx *ctx, const float *lhs, const float *rhs, float *result, int64_t count); /* :176 */
+int dl4s_hip_vmul_f32(dl4s_hip_ctx *ctx, const float *lhs, const float *rhs, float *result, int64_t count); /* :184 */
+int dl4s_hip_vdiv_f32(dl4s_hip_ctx *ctx, const float *lhs, const float *rhs, float *result, int64_t count); /* :192 */
+/* :225 gemm: row-major result[M,N] = alpha * op(lhs) . op(rhs) + beta * result; shapes are the STORED
+ * shapes of lhs and rhs.  beta != 0 really accumulates (cblas semantics of the MKL/Accelerate builds,
+ * Engine/CPU/Numeric/CPUFloat.swift:268-279). */
+int dl4s_hip_gemm_f32(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols,
+                      const float *rhs, int64_t rhs_rows, int64_t rhs_cols, float *result,
+                      float alpha, float beta, int transpose_first, int transpose_second);
+/* Strided-batched form of the same gemm: `batch` problems, element strides between consecutive
+ * operands (0 = shared).  One launch replaces the per-slice loop + stack of
+ * Tensor/Operators/Matrix.swift:106-116. */
+int dl4s_hip_gemm_batched_f32(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols,
+                              int64_t lhs_stride, const float *rhs, int64_t rhs_rows, int64_t rhs_cols,
+                              int64_t rhs_stride, float *result, int64_t result_stride, int64_t batch,
+                              float alpha, float beta, int transpose_first, int transpose_second);
+/* :233 band: copies columns max(0,i-below) .. min(cols,i+above+1)-1 of each row i; other elements of
+ * result are left untouched (the caller zero-fills first, Tensor/Operators/UtilOps.swift:117-121).
+ * has_below / has_above == 0 stand for nil. */
+int dl4s_hip_band_f32(dl4s_hip_ctx *ctx, const float *buffer, float *result, int64_t rows, int64_t cols,
+                      int has_below, int64_t below, int has_above, int64_t above);
+/* :242-263 broadcastAdd/Sub/Mul/Div.  Shapes right-aligned, size-1 axes broadcast.  Sub and Div use
+ * the reference's scalar forms where it does (x + (-s), x * (1/s); Engine/CPU/CPUEngine.swift:601-637). */
+typedef enum dl4s_binary_op { DL4S_OP_ADD = 0, DL4S_OP_SUB = 1, DL4S_OP_MUL = 2, DL4S_OP_DIV = 3 } dl4s_binary_op;
+int dl4s_hip_broadcast_f32(dl4s_hip_ctx *ctx, int op, const float *lhs, const int64_t *lhs_shape, int lhs_dim,
+                           const float *rhs, const int64_t *rhs_shape, int rhs_dim, float *result);
+/* :302 reduceSum(axes:) and :280 reduceMax(axis:, context: nil). */
+int dl4s_hip_reduce_sum_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim,
+                            const int32_t *axes, int naxes, float *result);
+int dl4s_hip_reduce_max_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim,
+                            int axis, float *result);
+/* :363 exp, :375 sqrt, :381 relu, :423 tanh */
+int dl4s_hip_exp_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+int dl4s_hip_sqrt_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+int dl4s_hip_relu_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+int dl4s_hip_tanh_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+/* :478 permuteAxes: source axis i becomes destination axis arrangement[i]
+ * (Engine/CPU/CPUEngine.swift:897-935). */
+int dl4s_hip_permute_axes_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim,
+                              const int32_t *arrangement, float *result);
+/* :536 stack along axis 0 of `n` equally shaped buffers of `count` elements each
+ * (Tensor/Operators/Stack.swift:79-98 as used by broadcastMatrixMultiplied). */
+int dl4s_hip_stack_f32(dl4s_hip_ctx *ctx, const float *const *buffers, int64_t n, int64_t count, float *result);
+
+/* ------------------------------------------------ fused layer tails (next to the path) */
+/* NN/Layer/LayerNorm.swift:62-77 on x [B, rows, D] -> result, statistics over rows*D jointly per b:
+ * mean = sum/N, var = sum(x^2)/N - mean^2, y = (x - mean) * (1 / (sqrt(var) + 1e-5)) * scale + shift.
+ * If residual != NULL the input is x + residual (MultiHeadAttention.swift:123-124). */
+int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *residual, const float *scale,
+                           const float *shift, float *result, int64_t B, int64_t rows, int64_t D);
+/* Tensor/Operators/Unary.swift:245-247: x * (0.5 * tanh(0.5 * (1.702 * x)) + 0.5), optional bias[D] added first
+ * (Dense bias, NN/Layer/Dense.swift:64-68). */
+int dl4s_hip_bias_gelu_f32(dl4s_hip_ctx *ctx, const float *x, const float *bias, float *result, int64_t rows,
+                           int64_t D);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DL4S_HIP_H */

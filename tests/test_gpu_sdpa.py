@@ -1,0 +1,323 @@
+"""Parity of the fused HIP attention kernels (through the C ABI) against the CPU oracle.
+
+Gate: |gpu - oracle| <= 1e-4 + 1e-4 * |oracle| element-wise (fp32), NaN/Inf at exactly the same
+positions, structured masks bit-identical to the dense mask they describe, mask == nil bit-identical
+to an all-zero mask.
+"""
+import numpy as np
+import pytest
+
+from helpers import assert_parity, causal_mask, lengths_mask
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from dl4s_amd import lib
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temperature=None):
+    from dl4s_amd import lib
+    B, H, Lq, dk = q.shape
+    Lk, dv = v.shape[2], v.shape[3]
+    T = np.float32(np.sqrt(np.float32(dk))) if temperature is None else np.float32(temperature)
+    rT = float(np.float32(1.0) / T)
+    bufs = [ctx.to_device(q), ctx.to_device(k), ctx.to_device(v), ctx.empty((B, H, Lq, dv))]
+    desc = None
+    if kind is None:
+        kind = lib.MASK_NONE if mask is None else lib.MASK_DENSE
+    if kind == lib.MASK_DENSE:
+        md = ctx.to_device(mask)
+        bufs.append(md)
+        desc = ctx.mask_desc(lib.MASK_DENSE, dense=md)
+    elif kind in (lib.MASK_KEY_LENGTHS, lib.MASK_CAUSAL_OR_KEY_LENGTHS):
+        ld = ctx.to_device(np.asarray(lens, np.int32), dtype=np.int32)
+        bufs.append(ld)
+        desc = ctx.mask_desc(kind, lengths=ld)
+    elif kind == lib.MASK_CAUSAL:
+        desc = ctx.mask_desc(lib.MASK_CAUSAL)
+    ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], bufs[3], B, H, Lq, Lk, dk, dv, rT, desc, lib.SDPA_STRICT if strict else 0)
+    out = bufs[3].numpy()
+    for b in bufs:
+        b.release()
+    return out
+
+
+def rand(rng, *shape, scale=1.0):
+    return (rng.standard_normal(shape) * scale).astype(np.float32)
+
+
+# ------------------------------------------------------------------ small shapes, every mask kind
+SHAPES = [  # B, H, Lq, Lk, d
+    (1, 2, 5, 7, 4),        # the golden-fixture shape: plain kernel
+    (2, 3, 9, 11, 8),
+    (1, 2, 5, 7, 64),       # MFMA kernel, ragged single tile
+    (2, 3, 130, 70, 64),    # ragged: Lq and Lk cross tile edges
+    (1, 2, 128, 128, 64),
+    (2, 2, 200, 333, 64),
+    (1, 1, 1, 1, 64),       # single query, single key
+    (1, 1, 300, 1, 64),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("mk", ["none", "dense_qk", "dense_full", "dense_b11k", "causal", "lens", "causal_lens", "half"])
+def test_sdpa_matches_oracle(ctx, orc, shape, mk):
+    from dl4s_amd import lib
+    B, H, Lq, Lk, d = shape
+    rng = np.random.default_rng(hash((shape, mk)) % (2 ** 32))
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    lens = rng.integers(0, Lk + 1, size=B)
+    lens[0] = max(1, Lk // 2)
+    kind, mask, lens_arg = None, None, None
+    if mk == "dense_qk":
+        mask = (rng.random((Lq, Lk)) < 0.4).astype(np.float32)
+    elif mk == "dense_full":
+        mask = (rng.random((B, H, Lq, Lk)) < 0.4).astype(np.float32)
+    elif mk == "dense_b11k":
+        mask = lengths_mask(lens, Lk)
+    elif mk == "half":
+        mask = (causal_mask(Lq, Lk) * np.float32(0.5)).reshape(1, 1, Lq, Lk)   # non-binary: a -5e8 penalty
+    elif mk == "causal":
+        kind, mask = lib.MASK_CAUSAL, causal_mask(Lq, Lk)
+    elif mk == "lens":
+        kind, mask, lens_arg = lib.MASK_KEY_LENGTHS, lengths_mask(lens, Lk), lens
+    elif mk == "causal_lens":
+        kind, lens_arg = lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lk)[None, None])
+    ref = orc.sdpa(q, k, v, mask)
+    got = run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg)
+    assert_parity(got, ref, "sdpa %s %s" % (shape, mk))
+    if kind is not None:
+        # structured descriptor == the dense mask it stands for, bit for bit (strict visits the same tiles)
+        dense = run_sdpa(ctx, q, k, v, mask)
+        strict = run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=True)
+        assert np.array_equal(strict, dense)
+        assert_parity(got, dense, "skip vs dense")
+
+
+def test_nil_mask_equals_zero_mask_bitwise(ctx):
+    rng = np.random.default_rng(3)
+    for d in (8, 64):
+        q, k, v = rand(rng, 2, 2, 70, d), rand(rng, 2, 2, 90, d), rand(rng, 2, 2, 90, d)
+        a = run_sdpa(ctx, q, k, v, None)
+        b = run_sdpa(ctx, q, k, v, np.zeros((70, 90), np.float32))
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("d", [8, 64])
+def test_blocked_keys_have_exactly_zero_weight_and_blocked_rows_are_uniform(ctx, orc, d):
+    rng = np.random.default_rng(5)
+    B, H, Lq, Lk = 1, 2, 70, 100
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    mask = np.zeros((Lq, Lk), np.float32)
+    mask[:, 61:] = 1
+    mask[33, :] = 1                      # fully blocked row
+    base = run_sdpa(ctx, q, k, v, mask)
+    k2, v2 = k.copy(), v.copy()
+    k2[:, :, 61:] = 7.0                  # finite changes at blocked keys must not move a single bit
+    v2[:, :, 61:] = -321.0
+    other = run_sdpa(ctx, q, k2, v2, mask)
+    rows = [r for r in range(Lq) if r != 33]
+    assert np.array_equal(base[:, :, rows], other[:, :, rows])
+    ref = orc.sdpa(q, k, v, mask)
+    assert_parity(base, ref, "blocked")
+    assert np.allclose(base[:, :, 33], v.mean(axis=2), atol=1e-5)       # uniform 1/Lk, never NaN
+    assert not np.isnan(base).any()
+
+
+@pytest.mark.parametrize("d", [8, 64])
+def test_nan_inf_placement_matches_oracle(ctx, orc, d):
+    rng = np.random.default_rng(9)
+    B, H, Lq, Lk = 1, 1, 40, 150
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    q[0, 0, 3, 0] = np.nan               # NaN scores in row 3     -> row NaN
+    q[0, 0, 5, :] = 0
+    q[0, 0, 5, 1] = np.inf               # +/-Inf scores in row 5  -> row NaN
+    k[0, 0, 140, :] = 0
+    k[0, 0, 140, 2] = 3e38               # huge finite key: q.k overflows for some rows only
+    mask = np.zeros((Lq, Lk), np.float32)
+    mask[7, :] = np.inf                  # every score of row 7 is -Inf -> row NaN
+    mask[9, 100:] = np.inf               # -Inf on a suffix (whole later tiles) -> weights 0 there, row finite
+    mask[11, :70] = np.inf               # -Inf on the leading tile -> still finite
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa(q, k, v, mask)
+    got = run_sdpa(ctx, q, k, v, mask)
+    assert np.isnan(ref[0, 0, 3]).all() and np.isnan(ref[0, 0, 5]).all() and np.isnan(ref[0, 0, 7]).all()
+    assert not np.isnan(ref[0, 0, 9]).any() and not np.isnan(ref[0, 0, 11]).any()
+    assert_parity(got, ref, "nan/inf d=%d" % d)
+
+
+def test_nan_in_v_at_blocked_key_reaches_output_only_in_strict_mode(ctx, orc):
+    from dl4s_amd import lib
+    rng = np.random.default_rng(10)
+    B, H, L, d = 1, 1, 256, 64
+    q, k, v = rand(rng, B, H, L, d), rand(rng, B, H, L, d), rand(rng, B, H, L, d)
+    v[0, 0, 255, 5] = np.nan             # last key: blocked for every query but the last
+    mask = causal_mask(L, L)
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa(q, k, v, mask)    # 0 * NaN = NaN in column 5 of every row
+    assert np.isnan(ref[0, 0, :, 5]).all()
+    strict = run_sdpa(ctx, q, k, v, mask, kind=lib.MASK_CAUSAL, strict=True)
+    assert_parity(strict, ref, "strict NaN")
+    dense = run_sdpa(ctx, q, k, v, mask)
+    assert_parity(dense, ref, "dense NaN")
+    fast = run_sdpa(ctx, q, k, v, mask, kind=lib.MASK_CAUSAL)
+    assert not np.isnan(fast[0, 0, :128]).any()     # documented: skipped tiles do not propagate it
+
+
+def test_temperature_is_a_reciprocal_multiply_on_q(ctx, orc):
+    rng = np.random.default_rng(12)
+    q, k, v = rand(rng, 1, 2, 50, 64), rand(rng, 1, 2, 60, 64), rand(rng, 1, 2, 60, 64)
+    got = run_sdpa(ctx, q, k, v, None, temperature=3.0)
+    assert_parity(got, orc.sdpa(q, k, v, None, temperature=3.0), "T=3")
+
+
+def test_error_paths(ctx):
+    from dl4s_amd import lib
+    q = ctx.empty((1, 1, 4, 64))
+    with pytest.raises(lib.Dl4sHipError) as e:
+        ctx.sdpa_fwd(q, q, q, q, 1, 1, 4, 0, 64, 64, 0.125)          # empty key axis
+    assert e.value.code == -2
+    bad = ctx.empty((3, 5))
+    with pytest.raises(lib.Dl4sHipError) as e:
+        ctx.sdpa_fwd(q, q, q, q, 1, 1, 4, 4, 64, 64, 0.125, ctx.mask_desc(lib.MASK_DENSE, dense=bad))
+    assert e.value.code == -2
+    with pytest.raises(lib.Dl4sHipError) as e:
+        ctx.sdpa_fwd(q, q, q, q, 1, 1, 4, 4, 512, 512, 0.125)
+    assert e.value.code == -5
+    ctx.sdpa_fwd(q, q, q, q, 0, 1, 4, 4, 64, 64, 0.125)              # empty batch is a no-op
+    q.release()
+    bad.release()
+
+
+# ------------------------------------------------------------------ the BASELINE configurations
+def test_config1_sdpa_b1_h8_l128_d64(ctx, orc):
+    rng = np.random.Generator(np.random.PCG64(1001))
+    q, k, v = (rng.standard_normal((1, 8, 128, 64), dtype=np.float32) for _ in range(3))
+    ref = orc.sdpa(q, k, v, None)
+    got = run_sdpa(ctx, q, k, v, None)
+    err = assert_parity(got, ref, "config 1")
+    assert err < 1e-5
+
+
+def test_config4_long_causal_prefill_sampled_against_oracle(ctx, orc):
+    """B8 H16 L2048 d64 causal, inputs 0.5*N(0,1).  The oracle is evaluated on sampled (batch, head)
+    pairs and query rows (rows are independent), the full output is checked through invariants."""
+    from dl4s_amd import lib
+    B, H, L, d = 8, 16, 2048, 64
+    rng = np.random.Generator(np.random.PCG64(1004))
+    q, k, v = (rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5) for _ in range(3))
+    got = run_sdpa(ctx, q, k, v, kind=lib.MASK_CAUSAL)
+    assert np.isfinite(got).all()
+    # row 0 attends to key 0 only
+    assert np.allclose(got[:, :, 0], v[:, :, 0], atol=1e-6)
+    # every output is a convex combination of the visible V rows
+    vmax = np.maximum.accumulate(v, axis=2)
+    vmin = np.minimum.accumulate(v, axis=2)
+    assert (got <= vmax + 1e-5).all() and (got >= vmin - 1e-5).all()
+    srng = np.random.default_rng(4)
+    rows = np.unique(np.concatenate([[0, 1, 31, 32, 63, 64, 127, 128, 2047], srng.integers(0, L, 40)]))
+    cm = causal_mask(L, L)[rows]
+    for (b, h) in [(0, 0), (3, 7), (7, 15)]:
+        ref = orc.sdpa(q[b:b + 1, h:h + 1, rows], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], cm)
+        assert_parity(got[b:b + 1, h:h + 1, rows], ref, "config 4 (b=%d,h=%d)" % (b, h))
+
+
+def test_config3_shape_padding_mask_sampled(ctx, orc):
+    """SDPA core of the encoder block: B8 H16 L1024 d64, key-length mask U[512,1024]."""
+    from dl4s_amd import lib
+    B, H, L, d = 8, 16, 1024, 64
+    rng = np.random.Generator(np.random.PCG64(1003))
+    q, k, v = (rng.standard_normal((B, H, L, d), dtype=np.float32) for _ in range(3))
+    lens = rng.integers(512, 1025, size=B)
+    got = run_sdpa(ctx, q, k, v, kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    rows = np.array([0, 5, 511, 512, 777, 1023])
+    for (b, h) in [(0, 0), (5, 9)]:
+        m = np.broadcast_to(lengths_mask(lens, L)[b:b + 1], (1, 1, len(rows), L)).copy()
+        ref = orc.sdpa(q[b:b + 1, h:h + 1, rows], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], m)
+        assert_parity(got[b:b + 1, h:h + 1, rows], ref, "config 3 core (b=%d,h=%d)" % (b, h))
+
+
+# ------------------------------------------------------------------ decode
+def run_decode(ctx, q, kc, vc, T):
+    B, H, Tcap, d = kc.shape
+    bufs = [ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc), ctx.empty((B, H, 1, d))]
+    ctx.sdpa_decode(bufs[0], bufs[1], bufs[2], bufs[3], B, H, T, Tcap, d, 0.125)
+    out = bufs[3].numpy()
+    for b in bufs:
+        b.release()
+    return out
+
+
+@pytest.mark.parametrize("B,H,T,Tcap", [(1, 1, 1, 1), (2, 3, 9, 12), (2, 2, 256, 256), (1, 4, 257, 300), (3, 2, 1000, 1024),
+                                        (2, 2, 4097, 4160)])
+def test_decode_matches_oracle(ctx, orc, B, H, T, Tcap):
+    rng = np.random.default_rng(T)
+    q, kc, vc = rand(rng, B, H, 1, 64), rand(rng, B, H, Tcap, 64), rand(rng, B, H, Tcap, 64)
+    kc[:, :, T:] = np.nan           # rows beyond T must never be read into the result
+    vc[:, :, T:] = np.nan
+    ref = orc.sdpa_decode(q, kc, vc, T)
+    got = run_decode(ctx, q, kc, vc, T)
+    assert_parity(got, ref, "decode T=%d" % T)
+    # and it is the same function as the prefill kernel with one query
+    pre = run_sdpa(ctx, q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T]))
+    assert_parity(got, pre, "decode vs prefill")
+
+
+def test_decode_nan_inf(ctx, orc):
+    rng = np.random.default_rng(77)
+    B, H, T = 2, 2, 600
+    q, kc, vc = rand(rng, B, H, 1, 64), rand(rng, B, H, T, 64), rand(rng, B, H, T, 64)
+    kc[0, 0, 300, 0] = np.nan       # (0,0): NaN score -> NaN output
+    q[1, 1, 0, :] = 0
+    q[1, 1, 0, 3] = np.inf          # (1,1): +/-Inf scores -> NaN output
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa_decode(q, kc, vc, T)
+    got = run_decode(ctx, q, kc, vc, T)
+    assert np.isnan(ref[0, 0]).all() and np.isnan(ref[1, 1]).all() and not np.isnan(ref[0, 1]).any()
+    assert_parity(got, ref, "decode nan/inf")
+
+
+def test_config5_incremental_decode_append_then_attend(ctx, orc):
+    """B16 H16 d64, cache of 4096 rows, 64 steps: step t appends row 4096+t and attends over 4097+t rows.
+    Checked against the oracle at the first, a middle and the last step on sampled (b, h), and through
+    the append invariant (the cache equals the concatenation) at the end."""
+    B, H, d, T0, steps = 16, 16, 64, 4096, 64
+    Tcap = T0 + steps
+    rng = np.random.Generator(np.random.PCG64(1005))
+    qs = rng.standard_normal((steps, B, H, 1, d), dtype=np.float32)
+    kc = np.zeros((B, H, Tcap, d), np.float32)
+    vc = np.zeros((B, H, Tcap, d), np.float32)
+    kc[:, :, :T0] = rng.standard_normal((B, H, T0, d), dtype=np.float32)
+    vc[:, :, :T0] = rng.standard_normal((B, H, T0, d), dtype=np.float32)
+    kn = rng.standard_normal((steps, B, H, 1, d), dtype=np.float32)
+    vn = rng.standard_normal((steps, B, H, 1, d), dtype=np.float32)
+    dk_, dv_ = ctx.to_device(kc), ctx.to_device(vc)
+    dq, dkn, dvn = ctx.to_device(qs), ctx.to_device(kn), ctx.to_device(vn)
+    dout = ctx.empty((steps, B, H, 1, d))
+    step_bytes = B * H * d * 4
+    for t in range(steps):
+        if t % 2 == 0:   # fused append+attend
+            ctx.sdpa_decode_step(dq.offset(t * step_bytes), dk_, dv_, dkn.offset(t * step_bytes), dvn.offset(t * step_bytes),
+                                 dout.offset(t * step_bytes), B, H, T0 + t, Tcap, d, 0.125)
+        else:            # separate append, then attend
+            ctx.kv_append(dk_, dv_, dkn.offset(t * step_bytes), dvn.offset(t * step_bytes), B, H, T0 + t, Tcap, d)
+            ctx.sdpa_decode(dq.offset(t * step_bytes), dk_, dv_, dout.offset(t * step_bytes), B, H, T0 + t + 1, Tcap, d, 0.125)
+    out = dout.numpy()
+    kfin, vfin = dk_.numpy(), dv_.numpy()
+    for t in range(steps):
+        kc[:, :, T0 + t] = kn[t, :, :, 0]
+        vc[:, :, T0 + t] = vn[t, :, :, 0]
+    assert np.array_equal(kfin, kc) and np.array_equal(vfin, vc)
+    assert np.isfinite(out).all()
+    for t in (0, 1, 31, 62, 63):
+        for (b, h) in [(0, 0), (9, 4), (15, 15)]:
+            ref = orc.sdpa_decode(qs[t, b:b + 1, h:h + 1], kc[b:b + 1, h:h + 1], vc[b:b + 1, h:h + 1], T0 + t + 1)
+            assert_parity(out[t, b:b + 1, h:h + 1], ref, "config 5 step %d (b=%d,h=%d)" % (t, b, h))
+    for buf in (dk_, dv_, dq, dkn, dvn, dout):
+        buf.release()
