@@ -27,9 +27,6 @@ struct dl4s_hip_ctx {
     // scratch owned by the library for split-K partial results (grown on demand, never shrunk)
     void *scratch = nullptr;
     size_t scratch_bytes = 0;
-    // one ticket per (batch, head) for the split-K merge; all zero whenever no kernel is running
-    unsigned int *tickets = nullptr;
-    static constexpr int kMaxTickets = 65536;
 };
 
 namespace dl4s {

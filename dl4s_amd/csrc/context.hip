@@ -76,11 +76,7 @@ int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx) {
     hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_begin);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_end);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void **>(&c->tickets), dl4s_hip_ctx::kMaxTickets * sizeof(unsigned int));
-    if (e == hipSuccess) e = hipMemsetAsync(c->tickets, 0, dl4s_hip_ctx::kMaxTickets * sizeof(unsigned int), c->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
     if (e != hipSuccess) {
-        if (c->tickets) (void)hipFree(c->tickets);
         if (c->ev_end) (void)hipEventDestroy(c->ev_end);
         if (c->ev_begin) (void)hipEventDestroy(c->ev_begin);
         if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -98,7 +94,6 @@ int dl4s_hip_destroy(dl4s_hip_ctx *ctx) {
         for (void *p : kv.second) (void)hipFree(p);
     for (auto &kv : ctx->live) (void)hipFree(reinterpret_cast<void *>(kv.first));
     if (ctx->scratch) (void)hipFree(ctx->scratch);
-    if (ctx->tickets) (void)hipFree(ctx->tickets);
     (void)hipEventDestroy(ctx->ev_begin);
     (void)hipEventDestroy(ctx->ev_end);
     (void)hipStreamDestroy(ctx->stream);

@@ -1,12 +1,18 @@
 // Single-query attention over a key/value cache (one decode step), split over the keys.
 //
-// The cache is [B,H,Tcap,64] fp32.  A workgroup (4 wavefronts) owns one (batch, head) and one chunk
-// of CHUNK keys; each wavefront streams 64 keys: a 16-lane group reads one 256-byte key row with one
-// 128-bit load per lane, so every load instruction of a wavefront covers four whole rows and all the
-// K loads and V loads of the wavefront are in flight together.  The dot product is reduced inside
-// the 16-lane group with DPP adds.  Each workgroup leaves (max, sum, 64 partial outputs) in a scratch
-// buffer; the last workgroup of a (batch, head) to finish (agent-scope ticket) merges the partials
-// with the usual softmax rescaling and writes the output, so that one launch serves a whole step.
+// The cache is [B,H,Tcap,64] fp32.  A 16-lane group reads one 256-byte key (or value) row with one
+// 128-bit load per lane, so every load instruction of a wavefront covers four whole rows (1 KiB,
+// contiguous), and a wavefront keeps the 8 K loads and 8 V loads of a 32-key block in flight together.
+// The dot product is reduced inside the 16-lane group with DPP adds.  With 16 wavefronts resident per CU
+// that is ample memory-level parallelism to keep HBM busy.
+//
+// Work split: grid = (nsplit, B*H).  When B*H alone fills the GPU (the decode benchmark: 256 pairs on 256
+// CUs) nsplit is 1, a 16-wavefront workgroup streams the whole cache row range of its pair and writes the
+// output itself: ONE launch per step.  Otherwise the key range is split, every workgroup leaves
+// (max, sum, 64 partial outputs) in a scratch record and a small second kernel merges the records of each
+// pair with the usual softmax rescaling.  (A single-launch merge by the last workgroup to finish needs
+// agent-scope release/acquire fences, i.e. an L2 write-back and invalidate per workgroup on gfx950, and ran
+// an order of magnitude slower than the two launches.)
 #include "common.h"
 
 namespace {
@@ -14,9 +20,7 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int HD = 64;
-constexpr int WAVES = 4;
-constexpr int KEYS_PER_WAVE = 64;
-constexpr int CHUNK = WAVES * KEYS_PER_WAVE;  // keys per workgroup
+constexpr int KB = 32;                        // keys per wavefront iteration
 constexpr int PSTR = 68;                      // floats per partial record: o[0..63], m, l, pad
 constexpr float LOG2E = 1.44269504088896340736f;
 
@@ -35,16 +39,18 @@ __device__ __forceinline__ float row16_sum(float x) {
     return x;
 }
 
-template <bool APPEND>
-__global__ __launch_bounds__(256) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
-                                                               float *vcache, const float *__restrict__ k_new,
-                                                               const float *__restrict__ v_new,
-                                                               float *__restrict__ out, float *part,
-                                                               unsigned int *tickets, int T, int Tcap, int pos,
-                                                               float rT, int nsplit) {
-    __shared__ float sm_o[WAVES][HD];
-    __shared__ float sm_m[WAVES], sm_l[WAVES];
-    __shared__ int sm_last;
+// NW wavefronts per workgroup; the wavefronts of a workgroup take 32-key blocks of the workgroup's key range
+// [split*chunk, split*chunk + chunk) round-robin.  Inside a wavefront each 16-lane group keeps its own running
+// (max, sum, 4 output columns per lane), so the loop has no cross-lane traffic beyond the 16-lane dot-product
+// reduction; groups, wavefronts and (through the scratch records) workgroups are merged once at the end.
+template <bool APPEND, int NW>
+__global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
+                                                                   float *vcache, const float *__restrict__ k_new,
+                                                                   const float *__restrict__ v_new,
+                                                                   float *__restrict__ out, float *part, int T, int Tcap,
+                                                                   int pos, float rT, int nsplit, int chunk) {
+    __shared__ float sm_o[NW][HD];
+    __shared__ float sm_m[NW], sm_l[NW];
     const int split = blockIdx.x;
     const int bh = blockIdx.y;
     const int tid = threadIdx.x;
@@ -54,75 +60,95 @@ __global__ __launch_bounds__(256) void sdpa_decode_splitk_f32(const float *__res
     f32x4 qv = *reinterpret_cast<const f32x4 *>(q + (long long)bh * HD + 4 * c);
     qv.x *= rT; qv.y *= rT; qv.z *= rT; qv.w *= rT;
 
-    const int kbeg = split * CHUNK + wave * KEYS_PER_WAVE + g;
     const long long base = (long long)bh * Tcap * HD + 4 * c;
-    f32x4 kk[16], vv[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int key = kbeg + 4 * i;
-        const int kc = key < T ? key : T - 1;
-        if (APPEND && kc == pos) {
-            kk[i] = *reinterpret_cast<const f32x4 *>(k_new + (long long)bh * HD + 4 * c);
-            if (key == pos) *reinterpret_cast<f32x4 *>(kcache + base + (long long)pos * HD) = kk[i];
-        } else {
-            kk[i] = *reinterpret_cast<const f32x4 *>(kcache + base + (long long)kc * HD);
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int key = kbeg + 4 * i;
-        const int kc = key < T ? key : T - 1;
-        if (APPEND && kc == pos) {
-            vv[i] = *reinterpret_cast<const f32x4 *>(v_new + (long long)bh * HD + 4 * c);
-            if (key == pos) *reinterpret_cast<f32x4 *>(vcache + base + (long long)pos * HD) = vv[i];
-        } else {
-            vv[i] = *reinterpret_cast<const f32x4 *>(vcache + base + (long long)kc * HD);
+    const int c0 = split * chunk;
+    const int c1 = min(T, c0 + chunk);
+    // Row `pos` is the row being appended in this step: it is read from k_new / v_new (the cache does not
+    // hold it yet) by selecting the ADDRESS per lane, so that all loads stay unconditional; one 16-lane
+    // group of the workgroup whose range holds the row writes it into the cache from its own copy.
+    const float *kn_row = nullptr, *vn_row = nullptr;
+    if (APPEND) {
+        kn_row = k_new + (long long)bh * HD + 4 * c;
+        vn_row = v_new + (long long)bh * HD + 4 * c;
+        if (pos >= c0 && pos < c1 && wave == 0 && g == 0) {
+            *reinterpret_cast<f32x4 *>(kcache + base + (long long)pos * HD) = *reinterpret_cast<const f32x4 *>(kn_row);
+            *reinterpret_cast<f32x4 *>(vcache + base + (long long)pos * HD) = *reinterpret_cast<const f32x4 *>(vn_row);
         }
     }
 
-    float s[16];
-    float mw = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        float d = qv.x * kk[i].x;
-        d += qv.y * kk[i].y;
-        d += qv.z * kk[i].z;
-        d += qv.w * kk[i].w;
-        d = row16_sum(d);
-        if (kbeg + 4 * i >= T) d = -INFINITY;
-        s[i] = d;
-        mw = fmaxf(mw, d);
-    }
-    mw = fmaxf(mw, __shfl_xor(mw, 16, 64));
-    mw = fmaxf(mw, __shfl_xor(mw, 32, 64));
-    const float m_use = (mw == -INFINITY) ? 0.f : mw;
-    float l = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int kb = c0 + wave * KB; kb < c1; kb += NW * KB) {
+        f32x4 kk[KB / 4], vv[KB / 4];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const float p = fast_exp2((s[i] - m_use) * LOG2E);
-        l += p;
-        acc.x += p * vv[i].x; acc.y += p * vv[i].y; acc.z += p * vv[i].z; acc.w += p * vv[i].w;
+        for (int i = 0; i < KB / 4; ++i) {
+            const int key = kb + 4 * i + g;
+            const int kc = key < T ? key : T - 1;
+            const float *kp = kcache + base + (long long)kc * HD;
+            if (APPEND) kp = (kc == pos) ? kn_row : kp;
+            kk[i] = *reinterpret_cast<const f32x4 *>(kp);
+        }
+#pragma unroll
+        for (int i = 0; i < KB / 4; ++i) {
+            const int key = kb + 4 * i + g;
+            const int kc = key < T ? key : T - 1;
+            const float *vp = vcache + base + (long long)kc * HD;
+            if (APPEND) vp = (kc == pos) ? vn_row : vp;
+            vv[i] = *reinterpret_cast<const f32x4 *>(vp);
+        }
+        float s[KB / 4];
+        float bm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < KB / 4; ++i) {
+            float d = qv.x * kk[i].x;
+            d += qv.y * kk[i].y;
+            d += qv.z * kk[i].z;
+            d += qv.w * kk[i].w;
+            d = row16_sum(d);
+            if (kb + 4 * i + g >= c1) d = -INFINITY;
+            s[i] = d;
+            bm = fmaxf(bm, d);
+        }
+        const float m_new = fmaxf(m_run, bm);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2((m_run - m_use) * LOG2E);
+        m_run = m_new;
+        l_run *= alpha;
+        acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
+#pragma unroll
+        for (int i = 0; i < KB / 4; ++i) {
+            const float p = fast_exp2((s[i] - m_use) * LOG2E);
+            l_run += p;
+            acc.x += p * vv[i].x; acc.y += p * vv[i].y; acc.z += p * vv[i].z; acc.w += p * vv[i].w;
+        }
+    }
+    // merge the four 16-lane groups of the wavefront
+    float mw = fmaxf(m_run, __shfl_xor(m_run, 16, 64));
+    mw = fmaxf(mw, __shfl_xor(mw, 32, 64));
+    {
+        const float mu = (mw == -INFINITY) ? 0.f : mw;
+        const float f = fast_exp2((m_run - mu) * LOG2E);
+        l_run *= f;
+        acc.x *= f; acc.y *= f; acc.z *= f; acc.w *= f;
     }
 #pragma unroll
     for (int o = 16; o <= 32; o <<= 1) {
-        l += __shfl_xor(l, o, 64);
+        l_run += __shfl_xor(l_run, o, 64);
         acc.x += __shfl_xor(acc.x, o, 64); acc.y += __shfl_xor(acc.y, o, 64);
         acc.z += __shfl_xor(acc.z, o, 64); acc.w += __shfl_xor(acc.w, o, 64);
     }
     if (g == 0) *reinterpret_cast<f32x4 *>(&sm_o[wave][4 * c]) = acc;
-    if (lane == 0) { sm_m[wave] = mw; sm_l[wave] = l; }
+    if (lane == 0) { sm_m[wave] = mw; sm_l[wave] = l_run; }
     __syncthreads();
 
-    float *rec = part + ((long long)bh * nsplit + split) * PSTR;
     if (tid < HD) {
         float M = sm_m[0];
 #pragma unroll
-        for (int w = 1; w < WAVES; ++w) M = fmaxf(M, sm_m[w]);
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, sm_m[w]);
         const float Mu = (M == -INFINITY) ? 0.f : M;
         float L = 0.f, O = 0.f;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) {
+        for (int w = 0; w < NW; ++w) {
             const float f = fast_exp2((sm_m[w] - Mu) * LOG2E);
             L += sm_l[w] * f;
             O += sm_o[w][tid] * f;
@@ -130,37 +156,28 @@ __global__ __launch_bounds__(256) void sdpa_decode_splitk_f32(const float *__res
         if (nsplit == 1) {
             out[(long long)bh * HD + tid] = O * (1.0f / L);
         } else {
+            float *rec = part + ((long long)bh * nsplit + split) * PSTR;
             rec[tid] = O;
             if (tid == 0) { rec[HD] = M; rec[HD + 1] = L; }
         }
     }
-    if (nsplit == 1) return;
+}
 
-    // Ticket: the workgroup that takes the last one merges all partial records of this (batch, head).
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        unsigned int t = __hip_atomic_fetch_add(&tickets[bh], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        sm_last = (t == (unsigned int)(nsplit - 1));
+// Merges the partial records of one (batch, head): one wavefront, lane = output column.
+__global__ __launch_bounds__(64) void sdpa_decode_merge_f32(const float *__restrict__ part, float *__restrict__ out,
+                                                             int nsplit) {
+    const int bh = blockIdx.x, tid = threadIdx.x;
+    const float *recs = part + (long long)bh * nsplit * PSTR;
+    float M = -INFINITY;
+    for (int sidx = 0; sidx < nsplit; ++sidx) M = fmaxf(M, recs[sidx * PSTR + HD]);
+    const float Mu = (M == -INFINITY) ? 0.f : M;
+    float L = 0.f, O = 0.f;
+    for (int sidx = 0; sidx < nsplit; ++sidx) {
+        const float f = fast_exp2((recs[sidx * PSTR + HD] - Mu) * LOG2E);
+        L += recs[sidx * PSTR + HD + 1] * f;
+        O += recs[sidx * PSTR + tid] * f;
     }
-    __syncthreads();
-    if (!sm_last) return;
-    __threadfence();
-    if (tid < HD) {
-        const float *recs = part + (long long)bh * nsplit * PSTR;
-        float M = -INFINITY;
-        for (int sidx = 0; sidx < nsplit; ++sidx)
-            M = fmaxf(M, __builtin_nontemporal_load(recs + sidx * PSTR + HD));
-        const float Mu = (M == -INFINITY) ? 0.f : M;
-        float L = 0.f, O = 0.f;
-        for (int sidx = 0; sidx < nsplit; ++sidx) {
-            const float f = fast_exp2((__builtin_nontemporal_load(recs + sidx * PSTR + HD) - Mu) * LOG2E);
-            L += __builtin_nontemporal_load(recs + sidx * PSTR + HD + 1) * f;
-            O += __builtin_nontemporal_load(recs + sidx * PSTR + tid) * f;
-        }
-        out[(long long)bh * HD + tid] = O * (1.0f / L);
-    }
-    if (tid == 0) __hip_atomic_store(&tickets[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    out[(long long)bh * HD + tid] = O * (1.0f / L);
 }
 
 __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restrict__ k_new,
@@ -184,22 +201,34 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     DL4S_REQUIRE(T >= 1 && T <= Tcap, DL4S_HIP_ESHAPE, "sdpa_decode: T=%lld must be in [1, Tcap=%lld]", (long long)T,
                  (long long)Tcap);
     DL4S_REQUIRE(BH <= 65535 && Tcap < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa_decode: B*H=%lld above 65535", (long long)BH);
-    const int nsplit = (int)((T + CHUNK - 1) / CHUNK);
-    // partial records live in the context's scratch block; size it for the whole cache capacity so that
-    // the following steps of the same sequence do not grow it again
-    const int cap_split = (int)((Tcap + CHUNK - 1) / CHUNK);
-    int rc = dl4s::ensure_scratch(ctx, (size_t)BH * cap_split * PSTR * sizeof(float));
-    if (rc) return rc;
-    float *part = reinterpret_cast<float *>(ctx->scratch);
-    unsigned int *tickets = ctx->tickets;  // BH <= 65535 entries, zero between launches
+    // Aim at 16 resident wavefronts on every CU.  Long caches use 16-wavefront workgroups; the key range is split
+    // over several workgroups only when batch*heads alone does not fill the GPU.
+    const int nw = T >= 2048 ? 16 : 4;
+    const long long want_wg = ((long long)ctx->cu_count * 16 + nw - 1) / nw;
+    long long max_split = (T + (long long)nw * KB - 1) / ((long long)nw * KB);
+    long long ns = (want_wg + BH - 1) / BH;
+    if (ns > max_split) ns = max_split;
+    if (ns < 1) ns = 1;
+    int chunk = (int)((T + ns - 1) / ns);
+    chunk = (chunk + KB - 1) / KB * KB;
+    const int nsplit = (int)((T + chunk - 1) / chunk);
+    float *part = nullptr;
+    if (nsplit > 1) {
+        int rc = dl4s::ensure_scratch(ctx, (size_t)BH * nsplit * PSTR * sizeof(float));
+        if (rc) return rc;
+        part = reinterpret_cast<float *>(ctx->scratch);
+    }
     dim3 grid(nsplit, (unsigned)BH);
-    if (append)
-        hipLaunchKernelGGL(sdpa_decode_splitk_f32<true>, grid, dim3(256), 0, ctx->stream, q, kcache, vcache, k_new, v_new,
-                           out, part, tickets, (int)T, (int)Tcap, (int)pos, rT, nsplit);
-    else
-        hipLaunchKernelGGL(sdpa_decode_splitk_f32<false>, grid, dim3(256), 0, ctx->stream, q, kcache, vcache, k_new, v_new,
-                           out, part, tickets, (int)T, (int)Tcap, -1, rT, nsplit);
-    return dl4s::launch_status("sdpa_decode_splitk_f32");
+#define DL4S_DECODE_LAUNCH(AP, NW_)                                                                                    \
+    hipLaunchKernelGGL((sdpa_decode_splitk_f32<AP, NW_>), grid, dim3(NW_ * 64), 0, ctx->stream, q, kcache, vcache, k_new,  \
+                       v_new, out, part, (int)T, (int)Tcap, (int)(AP ? pos : -1), rT, nsplit, chunk)
+    if (append) { if (nw == 16) DL4S_DECODE_LAUNCH(true, 16); else DL4S_DECODE_LAUNCH(true, 4); }
+    else { if (nw == 16) DL4S_DECODE_LAUNCH(false, 16); else DL4S_DECODE_LAUNCH(false, 4); }
+#undef DL4S_DECODE_LAUNCH
+    int st = dl4s::launch_status("sdpa_decode_splitk_f32");
+    if (st || nsplit == 1) return st;
+    hipLaunchKernelGGL(sdpa_decode_merge_f32, dim3((unsigned)BH), dim3(64), 0, ctx->stream, part, out, nsplit);
+    return dl4s::launch_status("sdpa_decode_merge_f32");
 }
 
 }  // namespace
