@@ -115,6 +115,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-pairs", type=int, default=6, help="(batch, head) slices timed on the CPU oracle; 0 disables")
     ap.add_argument("--decode-repeats", type=int, default=5)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one streaming kernel (negate, 1 GiB read + 1 GiB written) so that a counter run of "
+                         "this command can scale FETCH_SIZE / WRITE_SIZE by a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (every attention problem fits one MI355X); --gpus %d is not "
@@ -126,6 +129,14 @@ def main():
     info = ctx.device_info()
     pre = prefill(ctx, lib, args.steps, args.warmup)
     dec = decode(ctx, lib, args.decode_repeats) if args.decode_repeats > 0 else None
+    if args.copy_calibration:
+        n = 1 << 28
+        x, y = ctx.empty((n,)), ctx.empty((n,))
+        ctx.fill(1.0, x, n)
+        ctx.vneg(x, y, n)
+        ctx.sync()
+        x.release()
+        y.release()
     ctx.close()
 
     tflops = pre["flops"] * args.steps / pre["wall_s"] / 1e12
