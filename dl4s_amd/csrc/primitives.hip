@@ -16,13 +16,18 @@ inline unsigned grid_for(long long n, int per_thread = 4) {
 
 enum { U_NEG, U_EXP, U_SQRT, U_RELU, U_TANH };
 
+// IEEE-exact fp32 square root (the device sqrtf is 1 ulp): the correctly rounded fp64 root rounds to the
+// correctly rounded fp32 root because 53 >= 2*24 + 2.
+__device__ __forceinline__ float sqrt_rn(float v) { return (float)sqrt((double)v); }
+
+
 template <int OP>
 __global__ void unary_f32(const float *__restrict__ x, float *__restrict__ y, long long n) {
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
         float v = x[i], r;
         if (OP == U_NEG) r = -v;
         else if (OP == U_EXP) r = expf(v);
-        else if (OP == U_SQRT) r = sqrtf(v);
+        else if (OP == U_SQRT) r = sqrt_rn(v);
         else if (OP == U_RELU) r = v > 0.f ? v : 0.f;
         else r = tanhf(v);
         y[i] = r;
@@ -187,7 +192,7 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     const float rN = __fdiv_rn(1.0f, (float)n);
     const float mean = __fmul_rn(s, rN);
     const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
-    const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrtf(var), 1e-5f));
+    const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
     const float *xp = x + b * n;
     const float *rp = res ? res + b * n : nullptr;
     float *yp = y + b * n;
@@ -220,7 +225,7 @@ __global__ __launch_bounds__(TPB) void ln_small_f32(const float *__restrict__ x,
     const float rN = __fdiv_rn(1.0f, (float)n);
     const float mean = __fmul_rn(s, rN);
     const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
-    const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrtf(var), 1e-5f));
+    const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
     float *yp = y + b * n;
     for (long long i = threadIdx.x; i < n; i += TPB) {
         float v = xp[i];

@@ -1,0 +1,237 @@
+"""Parity of the engine primitives (C ABI) against the CPU oracle: element-wise results bit-exact where the
+arithmetic is a single IEEE operation, 1e-4 tolerance where summation order or libm differ."""
+import numpy as np
+import pytest
+
+from helpers import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from dl4s_amd import lib
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+RNG = np.random.default_rng(21)
+
+
+def rnd(*shape):
+    return RNG.standard_normal(shape).astype(np.float32)
+
+
+def test_memory_roundtrip_views_and_stats(ctx):
+    from dl4s_amd import lib
+    import ctypes as C
+    a = rnd(1000)
+    d = ctx.to_device(a)
+    assert np.array_equal(d.numpy(), a)
+    # an offset view is pointer arithmetic; getSize reports what is left of the allocation
+    sz = C.c_size_t()
+    lib._check(ctx.lib.dl4s_hip_get_size(ctx.handle, C.c_void_p(d.offset(400)), C.byref(sz)))
+    assert sz.value >= 3600
+    v = C.c_float()
+    lib._check(ctx.lib.dl4s_hip_get_value_f32(ctx.handle, C.c_void_p(d.offset(4 * 17)), C.byref(v)))
+    assert v.value == a[17]
+    lib._check(ctx.lib.dl4s_hip_set_pointee_f32(ctx.handle, C.c_void_p(d.offset(4 * 17)), C.c_float(2.5)))
+    assert d.numpy()[17] == 2.5
+    e = ctx.empty((1000,))
+    lib._check(ctx.lib.dl4s_hip_assign_d2d(ctx.handle, C.c_void_p(e.ptr), C.c_void_p(d.ptr), C.c_size_t(4000)))
+    assert e.numpy()[17] == 2.5
+    used0, _ = ctx.mem_stats()
+    d.release()
+    e.release()
+    used1, pooled = ctx.mem_stats()
+    assert used1 < used0 and pooled > 0
+    # freeing an offset view or freeing twice is an error, not a crash
+    f = ctx.empty((16,))
+    p = f.ptr
+    assert ctx.lib.dl4s_hip_free(ctx.handle, C.c_void_p(f.offset(8))) == -1
+    f.release()
+    assert ctx.lib.dl4s_hip_free(ctx.handle, C.c_void_p(p)) == -1
+    assert b"double free" in ctx.lib.dl4s_hip_last_error()
+    assert ctx.lib.dl4s_hip_free(ctx.handle, None) == 0      # NULL is a no-op
+
+
+def test_elementwise_bit_exact(ctx, orc):
+    n = 100003
+    a, b = rnd(n), np.abs(rnd(n)) + np.float32(0.5)      # b > 0: it is also the sqrt argument
+    da, db, dy = ctx.to_device(a), ctx.to_device(b), ctx.empty((n,))
+    for fn, ref in [(ctx.vadd, a + b), (ctx.vsub, a - b), (ctx.vmul, a * b), (ctx.vdiv, a / b)]:
+        fn(da, db, dy, n)
+        assert np.array_equal(dy.numpy(), ref)
+    ctx.vneg(da, dy, n)
+    assert np.array_equal(dy.numpy(), -a)
+    ctx.relu(da, dy, n)
+    assert np.array_equal(dy.numpy(), orc.relu(a))
+    ctx.sqrt(db, dy, n)
+    assert np.array_equal(dy.numpy(), orc.sqrt(b))
+    ctx.exp(da, dy, n)
+    assert_parity(dy.numpy(), orc.exp(a), "exp")
+    ctx.tanh(da, dy, n)
+    assert_parity(dy.numpy(), orc.tanh(a), "tanh")
+    ctx.fill(1.5, dy, n)
+    assert (dy.numpy() == 1.5).all()
+    ctx.vadd(da, db, da, n)            # result may alias an input
+    assert np.array_equal(da.numpy(), a + b)
+    for x in (da, db, dy):
+        x.release()
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 7, 6), (128, 128, 16), (130, 70, 33), (257, 129, 100), (64, 512, 512)])
+def test_gemm(ctx, orc, ta, tb, M, N, K):
+    A = rnd(K, M) if ta else rnd(M, K)
+    B = rnd(N, K) if tb else rnd(K, N)
+    dA, dB, dC = ctx.to_device(A), ctx.to_device(B), ctx.empty((M, N))
+    ctx.gemm(dA, A.shape, dB, B.shape, dC, 1.0, 0.0, ta, tb)
+    ref = orc.gemm(A, B, ta, tb)
+    assert_parity(dC.numpy(), ref, "gemm %s" % ((M, N, K, ta, tb),))
+    # alpha, and beta = 0 must ignore whatever C held (NaN included)
+    ctx.fill(float("nan"), dC, M * N)
+    ctx.gemm(dA, A.shape, dB, B.shape, dC, 2.0, 0.0, ta, tb)
+    assert_parity(dC.numpy(), orc.gemm(A, B, ta, tb, alpha=2.0), "gemm alpha")
+    for x in (dA, dB, dC):
+        x.release()
+
+
+def test_gemm_known_answers_and_beta(ctx):
+    # Tests/DL4STests/VecTests.swift:127-156
+    c = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
+    dc, r33, r22 = ctx.to_device(c), ctx.empty((3, 3)), ctx.empty((2, 2))
+    ctx.gemm(dc, c.shape, dc, c.shape, r33, 1.0, 0.0, True, False)
+    assert r33.numpy().tolist() == [[17, 22, 27], [22, 29, 36], [27, 36, 45]]
+    ctx.gemm(dc, c.shape, dc, c.shape, r22, 1.0, 0.0, False, True)
+    assert r22.numpy().tolist() == [[14, 32], [32, 77]]
+    ctx.gemm(dc, c.shape, dc, c.shape, r22, 1.0, 1.0, False, True)      # beta accumulates (cblas semantics)
+    assert r22.numpy().tolist() == [[28, 64], [64, 154]]
+    for x in (dc, r33, r22):
+        x.release()
+
+
+def test_gemm_shape_error(ctx):
+    from dl4s_amd import lib
+    a = ctx.empty((4, 4))
+    with pytest.raises(lib.Dl4sHipError) as e:
+        ctx.gemm(a, (2, 3), a, (2, 3), a)
+    assert e.value.code == -2
+    a.release()
+
+
+def test_gemm_batched_equals_loop_and_stack(ctx, orc):
+    B, M, N, K = 5, 70, 40, 64
+    A, W = rnd(B, M, K), rnd(K, N)
+    dA, dW, dC = ctx.to_device(A), ctx.to_device(W), ctx.empty((B, M, N))
+    ctx.gemm_batched(dA, (M, K), M * K, dW, (K, N), 0, dC, M * N, B)
+    assert_parity(dC.numpy(), orc.bmm(A, W), "batched gemm")
+    # the reference's form: one gemm per slice into its own buffer, then stack
+    parts = [ctx.empty((M, N)) for _ in range(B)]
+    for b in range(B):
+        ctx.gemm(dA.offset(b * M * K * 4), (M, K), dW, (K, N), parts[b])
+    dS = ctx.empty((B, M, N))
+    ctx.stack(parts, M * N, dS)
+    assert np.array_equal(dS.numpy(), dC.numpy())
+    for x in [dA, dW, dC, dS] + parts:
+        x.release()
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+@pytest.mark.parametrize("sa,sb", [((2, 3, 4), (4,)), ((2, 3, 4), (3, 1)), ((2, 3, 4), ()), ((), (2, 3)), ((2, 1, 4), (1, 3, 1)),
+                                   ((2, 3, 4, 5), (2, 1, 1, 5)), ((3, 4), (3, 4)), ((2, 2, 33, 33), (33, 33)), ((40, 1), (1, 50)),
+                                   ((2, 3, 7, 9), (2, 3, 7, 1))])
+def test_broadcast_bit_exact(ctx, orc, op, sa, sb):
+    from dl4s_amd import lib
+    a, b = rnd(*sa), rnd(*sb) + np.float32(2.5)
+    ref = orc.broadcast(op, a, b)
+    da, db, dy = ctx.to_device(a), ctx.to_device(b), ctx.empty(ref.shape)
+    ctx.broadcast({"add": lib.OP_ADD, "sub": lib.OP_SUB, "mul": lib.OP_MUL, "div": lib.OP_DIV}[op], da, sa, db, sb, dy)
+    assert np.array_equal(dy.numpy(), ref)          # includes x*(1/s) and x+(-s) roundings of the scalar forms
+    for x in (da, db, dy):
+        x.release()
+
+
+def test_broadcast_shape_error(ctx):
+    from dl4s_amd import lib
+    a = ctx.empty((12,))
+    with pytest.raises(lib.Dl4sHipError) as e:
+        ctx.broadcast(lib.OP_ADD, a, (3, 4), a, (2, 4), a)
+    assert e.value.code == -2
+    a.release()
+
+
+@pytest.mark.parametrize("shape,axes", [((3, 4, 5), [2]), ((3, 4, 5), [1, 2]), ((3, 4, 5), [0]), ((2, 3, 4, 50), [3]),
+                                        ((2, 300, 70), [1, 2]), ((6,), [0]), ((4, 5), [0, 1])])
+def test_reduce_sum(ctx, orc, shape, axes):
+    x = rnd(*shape)
+    ref = orc.reduce_sum(x, axes)
+    dx, dy = ctx.to_device(x), ctx.empty(ref.shape if ref.shape else (1,))
+    ctx.reduce_sum(dx, shape, axes, dy)
+    assert_parity(dy.numpy().reshape(ref.shape), ref, "reduceSum")
+    dx.release()
+    dy.release()
+
+
+@pytest.mark.parametrize("shape,axis", [((3, 4, 5), 2), ((3, 4, 5), 1), ((3, 4, 5), 0), ((2, 2, 9, 1000), 3)])
+def test_reduce_max_exact_and_nan_skipping(ctx, orc, shape, axis):
+    x = rnd(*shape)
+    x.flat[3] = np.nan
+    ref = orc.reduce_max(x, axis)
+    dx, dy = ctx.to_device(x), ctx.empty(ref.shape)
+    ctx.reduce_max(dx, shape, axis, dy)
+    assert np.array_equal(dy.numpy(), ref)
+    dx.release()
+    dy.release()
+
+
+@pytest.mark.parametrize("shape,arr", [((2, 3, 4, 5), (0, 2, 1, 3)), ((2, 3, 4, 5), (1, 2, 3, 0)), ((2, 3, 4, 5), (3, 0, 1, 2)),
+                                       ((7, 9), (1, 0)), ((4, 16, 8, 64), (0, 2, 1, 3))])
+def test_permute_axes_scatter_convention(ctx, orc, shape, arr):
+    x = rnd(*shape)
+    ref = orc.permute(x, arr)
+    dx, dy = ctx.to_device(x), ctx.empty(ref.shape)
+    ctx.permute_axes(dx, shape, arr, dy)
+    assert np.array_equal(dy.numpy(), ref)
+    dx.release()
+    dy.release()
+
+
+def test_band_and_decoder_mask_recipe(ctx, orc):
+    from dl4s_amd import lib
+    L = 37
+    ones = np.ones((L, L), np.float32)
+    dx, dy = ctx.to_device(ones), ctx.empty((L, L))
+    for below, above in [(-1, None), (0, 0), (None, 0), (2, 3), (None, None)]:
+        ctx.fill(0.0, dy, L * L)                   # bandMatrix zero-fills first (UtilOps.swift:117-121)
+        ctx.band(dx, dy, L, L, below, above)
+        assert np.array_equal(dy.numpy(), orc.band(ones, below, above)), (below, above)
+    dx.release()
+    dy.release()
+
+
+@pytest.mark.parametrize("B,rows,D", [(3, 7, 16), (5, 1, 1024), (4, 512, 512), (2, 1, 33)])
+def test_layernorm(ctx, orc, B, rows, D):
+    x, res = rnd(B, rows, D) * 2 + np.float32(0.3), rnd(B, rows, D)
+    scale, shift = rnd(D), rnd(D)
+    dx, dr, ds, dh, dy = ctx.to_device(x), ctx.to_device(res), ctx.to_device(scale), ctx.to_device(shift), ctx.empty((B, rows, D))
+    ctx.layernorm(dx, None, ds, dh, dy, B, rows, D)
+    assert_parity(dy.numpy(), orc.layernorm(x, scale, shift), "layernorm")
+    ctx.layernorm(dx, dr, ds, dh, dy, B, rows, D)
+    assert_parity(dy.numpy(), orc.layernorm(x + res, scale, shift), "layernorm+residual")
+    for t in (dx, dr, ds, dh, dy):
+        t.release()
+
+
+def test_bias_gelu(ctx, orc):
+    rows, D = 50, 129
+    x, bias = rnd(rows, D) * 3, rnd(D)
+    dx, db, dy = ctx.to_device(x), ctx.to_device(bias), ctx.empty((rows, D))
+    ctx.bias_gelu(dx, db, dy, rows, D)
+    assert_parity(dy.numpy(), orc.gelu(x + bias), "bias+gelu")
+    ctx.bias_gelu(dx, None, dy, rows, D)
+    assert_parity(dy.numpy(), orc.gelu(x), "gelu")
+    for t in (dx, db, dy):
+        t.release()
