@@ -10,6 +10,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdl4s_hip.so")
+HOST_LIB = os.path.join(HERE, "libdl4s_host.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -46,7 +47,18 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed")
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(cmd)
+    build_host(verbose)
     return LIB
+
+
+def build_host(verbose=False):
+    """The C++ host layer (no device code): g++ against the C ABI, linked to libdl4s_hip.so next to it."""
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", HOST_LIB,
+           os.path.join(HERE, "host", "dl4s_host_capi.cpp"), "-L" + HERE, "-ldl4s_hip", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return HOST_LIB
 
 
 if __name__ == "__main__":

@@ -1,0 +1,673 @@
+// Host-side mirror of the DL4S interfaces on the attention forward path, written against the C ABI of
+// libdl4s_hip.so.  The reference is Swift; this is the C++ rendering of the same surface with the same
+// names, argument meaning and error behaviour:
+//
+//   DeviceType / MemoryOperatorsType / EngineType   Engine/Engine.swift:30-35, :39-139, :143-581
+//   Buffer / ShapedBuffer                           Engine/Buffer.swift:30-107
+//   Tensor / TensorHandle                           Tensor/Tensor.swift:29-176
+//   tensor operators                                Tensor/Operators/{Binary,Unary,Reduce,Matrix,Shape,Stack,Subscript,UtilOps}.swift
+//   LayerNorm, Dense, Dropout                       NN/Layer/{LayerNorm,Dense,Dropout}.swift
+//   ScaledDotProductAttention, MultiHeadAttention, PointwiseFeedForward, TransformerEncoderBlock,
+//   TransformerDecoderBlock, makeEncoderMasks, makeDecoderMasks   NN/Models/Transformer/*.swift
+//
+// Contract violations that the reference traps on (precondition / fatalError) throw dl4s::Trap here.
+//
+// Two execution modes, selected by HIP::fused():
+//   false  every tensor operator issues exactly the engine calls the reference issues (per-slice gemm loop +
+//          stack, materialised score tensors, softmax and LayerNorm as primitive sequences);
+//   true   the layers take the backend's fused entry points where it has them: one fused attention launch in
+//          ScaledDotProductAttention, one strided-batched gemm per broadcastMatrixMultiplied, fused
+//          residual + LayerNorm, fused bias + GELU.
+#pragma once
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <memory>
+#include <numeric>
+#include <optional>
+#include <random>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/dl4s_hip.h"
+
+namespace dl4s {
+
+struct Trap : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+inline void precondition(bool ok, const char *msg) {
+    if (!ok) throw Trap(msg);
+}
+
+using Shape = std::vector<int64_t>;
+
+inline int64_t count_of(const Shape &s) {
+    int64_t n = 1;
+    for (int64_t v : s) n *= v;
+    return n;
+}
+
+// Util.swift:40-45
+inline Shape shapeForBroadcastedOperands(const Shape &lhs, const Shape &rhs) {
+    const size_t dim = std::max(lhs.size(), rhs.size());
+    Shape out(dim);
+    for (size_t i = 0; i < dim; ++i) {
+        const int64_t l = i < dim - lhs.size() ? 1 : lhs[i - (dim - lhs.size())];
+        const int64_t r = i < dim - rhs.size() ? 1 : rhs[i - (dim - rhs.size())];
+        out[i] = std::max(l, r);
+    }
+    return out;
+}
+
+// ------------------------------------------------------------------------- Buffer.swift
+struct Buffer {
+    float *memory = nullptr;  // RawBuffer of the HIP device: a device pointer (offset views are pointer arithmetic)
+};
+
+struct ShapedBuffer {
+    Buffer values;
+    Shape shape;
+    int dim() const { return (int)shape.size(); }
+    int64_t count() const { return count_of(shape); }
+    ShapedBuffer reshaped(Shape s) const { return ShapedBuffer{values, std::move(s)}; }
+};
+
+// ------------------------------------------------------------------------- the HIP device
+struct HIP {
+    static dl4s_hip_ctx *&context() {
+        static dl4s_hip_ctx *ctx = nullptr;
+        return ctx;
+    }
+    static bool &fused() {
+        static bool f = true;
+        return f;
+    }
+    static void check(int rc) {
+        if (rc != DL4S_HIP_OK) throw Trap(std::string("dl4s_hip: ") + dl4s_hip_last_error());
+    }
+
+    // MemoryOperatorsType (Engine/Engine.swift:39-139), the subset the path uses
+    struct Memory {
+        static Buffer allocateBuffer(int64_t capacity) {
+            void *p = nullptr;
+            check(dl4s_hip_alloc(context(), (size_t)capacity * sizeof(float), &p));
+            return Buffer{static_cast<float *>(p)};
+        }
+        static ShapedBuffer allocateBuffer(const Shape &shape) { return ShapedBuffer{allocateBuffer(count_of(shape)), shape}; }
+        static void free(Buffer b) { check(dl4s_hip_free(context(), b.memory)); }
+        static void assign(const float *host, Buffer dst, int64_t count) {
+            check(dl4s_hip_assign_h2d(context(), dst.memory, host, (size_t)count * sizeof(float)));
+        }
+        static void assign(Buffer src, Buffer dst, int64_t count) {
+            check(dl4s_hip_assign_d2d(context(), dst.memory, src.memory, (size_t)count * sizeof(float)));
+        }
+        static void assign(Buffer src, float *host, int64_t count) {
+            check(dl4s_hip_assign_d2h(context(), host, src.memory, (size_t)count * sizeof(float)));
+        }
+        static float getValue(Buffer src) {
+            float v;
+            check(dl4s_hip_get_value_f32(context(), src.memory, &v));
+            return v;
+        }
+        static int64_t getSize(Buffer b) {
+            size_t bytes;
+            check(dl4s_hip_get_size(context(), b.memory, &bytes));
+            return (int64_t)(bytes / sizeof(float));
+        }
+        static Buffer advance(Buffer b, int64_t by) { return Buffer{b.memory + by}; }
+    };
+
+    // EngineType (Engine/Engine.swift:143-581), the subset the path uses
+    struct Engine {
+        static void fill(float value, Buffer result, int64_t count) { check(dl4s_hip_fill_f32(context(), value, result.memory, count)); }
+        static void vAdd(Buffer l, Buffer r, Buffer res, int64_t n) { check(dl4s_hip_vadd_f32(context(), l.memory, r.memory, res.memory, n)); }
+        static void vNeg(Buffer v, Buffer res, int64_t n) { check(dl4s_hip_vneg_f32(context(), v.memory, res.memory, n)); }
+        static void vSub(Buffer l, Buffer r, Buffer res, int64_t n) { check(dl4s_hip_vsub_f32(context(), l.memory, r.memory, res.memory, n)); }
+        static void vMul(Buffer l, Buffer r, Buffer res, int64_t n) { check(dl4s_hip_vmul_f32(context(), l.memory, r.memory, res.memory, n)); }
+        static void vDiv(Buffer l, Buffer r, Buffer res, int64_t n) { check(dl4s_hip_vdiv_f32(context(), l.memory, r.memory, res.memory, n)); }
+        static void gemm(const ShapedBuffer &lhs, const ShapedBuffer &rhs, const ShapedBuffer &result, float alpha, float beta,
+                         bool transposeFirst, bool transposeSecond) {
+            check(dl4s_hip_gemm_f32(context(), lhs.values.memory, lhs.shape[0], lhs.shape[1], rhs.values.memory, rhs.shape[0],
+                                    rhs.shape[1], result.values.memory, alpha, beta, transposeFirst, transposeSecond));
+        }
+        static void band(const ShapedBuffer &buffer, const ShapedBuffer &result, std::optional<int64_t> below,
+                         std::optional<int64_t> above) {
+            precondition(buffer.shape == result.shape, "Shape of result must be equal to shape of buffer.");
+            precondition(buffer.dim() == 2, "Band can only be computed on tensor of dimensionality 2.");
+            check(dl4s_hip_band_f32(context(), buffer.values.memory, result.values.memory, buffer.shape[0], buffer.shape[1],
+                                    below.has_value(), below.value_or(0), above.has_value(), above.value_or(0)));
+        }
+        static void broadcast(int op, const ShapedBuffer &l, const ShapedBuffer &r, const ShapedBuffer &res) {
+            check(dl4s_hip_broadcast_f32(context(), op, l.values.memory, l.shape.data(), l.dim(), r.values.memory, r.shape.data(),
+                                         r.dim(), res.values.memory));
+        }
+        static void broadcastAdd(const ShapedBuffer &l, const ShapedBuffer &r, const ShapedBuffer &res) { broadcast(DL4S_OP_ADD, l, r, res); }
+        static void broadcastSub(const ShapedBuffer &l, const ShapedBuffer &r, const ShapedBuffer &res) { broadcast(DL4S_OP_SUB, l, r, res); }
+        static void broadcastMul(const ShapedBuffer &l, const ShapedBuffer &r, const ShapedBuffer &res) { broadcast(DL4S_OP_MUL, l, r, res); }
+        static void broadcastDiv(const ShapedBuffer &l, const ShapedBuffer &r, const ShapedBuffer &res) { broadcast(DL4S_OP_DIV, l, r, res); }
+        static void reduceSum(const ShapedBuffer &values, const ShapedBuffer &result, const std::vector<int> &axes) {
+            std::vector<int32_t> ax(axes.begin(), axes.end());
+            check(dl4s_hip_reduce_sum_f32(context(), values.values.memory, values.shape.data(), values.dim(), ax.data(), (int)ax.size(),
+                                          result.values.memory));
+        }
+        static void reduceMax(const ShapedBuffer &values, const ShapedBuffer &result, int axis) {
+            check(dl4s_hip_reduce_max_f32(context(), values.values.memory, values.shape.data(), values.dim(), axis, result.values.memory));
+        }
+        static void exp(const ShapedBuffer &v, const ShapedBuffer &r) { check(dl4s_hip_exp_f32(context(), v.values.memory, r.values.memory, v.count())); }
+        static void tanh(const ShapedBuffer &v, const ShapedBuffer &r) { check(dl4s_hip_tanh_f32(context(), v.values.memory, r.values.memory, v.count())); }
+        static void sqrt(const ShapedBuffer &v, const ShapedBuffer &r) { check(dl4s_hip_sqrt_f32(context(), v.values.memory, r.values.memory, v.count())); }
+        static void relu(const ShapedBuffer &v, const ShapedBuffer &r) { check(dl4s_hip_relu_f32(context(), v.values.memory, r.values.memory, v.count())); }
+        static void permuteAxes(const ShapedBuffer &values, const ShapedBuffer &result, const std::vector<int> &arangement) {
+            std::vector<int32_t> ar(arangement.begin(), arangement.end());
+            check(dl4s_hip_permute_axes_f32(context(), values.values.memory, values.shape.data(), values.dim(), ar.data(),
+                                            result.values.memory));
+        }
+        static void stack(const std::vector<ShapedBuffer> &buffers, const ShapedBuffer &result, int axis) {
+            precondition(axis == 0, "stack: only axis 0 is available for HIP");
+            std::vector<const float *> ptrs;
+            for (auto &b : buffers) {
+                precondition(b.shape == buffers[0].shape, "stack: buffers must have equal shapes");
+                ptrs.push_back(b.values.memory);
+            }
+            check(dl4s_hip_stack_f32(context(), ptrs.data(), (int64_t)ptrs.size(), buffers.empty() ? 0 : buffers[0].count(),
+                                     result.values.memory));
+        }
+        // Fused entry points of this backend (no counterpart in EngineType).
+        static void fusedAttention(const ShapedBuffer &q, const ShapedBuffer &k, const ShapedBuffer &v, const ShapedBuffer *mask,
+                                   const ShapedBuffer &result, float temperature) {
+            dl4s_mask_desc md{};
+            if (mask) {
+                precondition(mask->dim() <= 4, "mask must be broadcastable to [batchSize, heads, queryCount, keyCount]");
+                md.kind = DL4S_MASK_DENSE_F32;
+                md.dense = mask->values.memory;
+                for (int i = 0; i < 4; ++i) md.shape[i] = 1;
+                for (int i = 0; i < mask->dim(); ++i) md.shape[4 - mask->dim() + i] = mask->shape[i];
+            }
+            check(dl4s_hip_sdpa_fwd_f32(context(), q.values.memory, k.values.memory, v.values.memory, result.values.memory,
+                                        q.shape[0], q.shape[1], q.shape[2], k.shape[2], q.shape[3], v.shape[3],
+                                        1.0f / temperature, mask ? &md : nullptr, DL4S_SDPA_STRICT));
+        }
+        static void gemmBatched(const ShapedBuffer &lhs, int64_t lstride, const ShapedBuffer &rhs, int64_t rstride,
+                                const ShapedBuffer &result, int64_t batch, bool tA, bool tB) {
+            const int ld = lhs.dim(), rd = rhs.dim(), od = result.dim();
+            check(dl4s_hip_gemm_batched_f32(context(), lhs.values.memory, lhs.shape[ld - 2], lhs.shape[ld - 1], lstride,
+                                            rhs.values.memory, rhs.shape[rd - 2], rhs.shape[rd - 1], rstride, result.values.memory,
+                                            result.shape[od - 2] * result.shape[od - 1], batch, 1.0f, 0.0f, tA, tB));
+        }
+        static void layerNorm(const ShapedBuffer &x, const ShapedBuffer *residual, const ShapedBuffer &scale,
+                              const ShapedBuffer &shift, const ShapedBuffer &result) {
+            const int64_t B = x.shape[0], D = scale.count();
+            check(dl4s_hip_layernorm_f32(context(), x.values.memory, residual ? residual->values.memory : nullptr, scale.values.memory,
+                                         shift.values.memory, result.values.memory, B, x.count() / (B * D), D));
+        }
+        static void biasGelu(const ShapedBuffer &x, const ShapedBuffer &bias, const ShapedBuffer &result) {
+            const int64_t D = bias.count();
+            check(dl4s_hip_bias_gelu_f32(context(), x.values.memory, bias.values.memory, result.values.memory, x.count() / D, D));
+        }
+    };
+};
+
+using Device = HIP;
+
+// ------------------------------------------------------------------------- Tensor.swift
+// Owns a buffer; a handle with a parent is a view into the parent's allocation and frees nothing
+// (Tensor/Tensor.swift:29-43).
+struct TensorHandle {
+    ShapedBuffer values;
+    std::shared_ptr<TensorHandle> parent;
+    TensorHandle(ShapedBuffer v, std::shared_ptr<TensorHandle> p) : values(std::move(v)), parent(std::move(p)) {}
+    TensorHandle(const TensorHandle &) = delete;
+    ~TensorHandle() {
+        if (!parent) dl4s_hip_free(Device::context(), values.values.memory);
+    }
+};
+
+class Tensor {
+   public:
+    std::shared_ptr<TensorHandle> handle;
+    Shape shape;
+
+    Tensor() = default;
+    // Tensor(using:context:) -- takes ownership of a freshly allocated buffer
+    explicit Tensor(ShapedBuffer buffer) : handle(std::make_shared<TensorHandle>(buffer, nullptr)), shape(buffer.shape) {}
+    Tensor(std::shared_ptr<TensorHandle> h, Shape s) : handle(std::move(h)), shape(std::move(s)) {}
+    // Tensor([Float], shape:)  (Tensor/Tensor.swift:143-153)
+    Tensor(const float *host, const Shape &s) : Tensor(Device::Memory::allocateBuffer(s)) {
+        Device::Memory::assign(host, handle->values.values, count());
+    }
+    Tensor(const std::vector<float> &host, const Shape &s) : Tensor(host.data(), s) {
+        precondition((int64_t)host.size() == count_of(s), "element count does not match shape");
+    }
+    // Tensor(scalar): shape []  (Tensor/TensorExt.swift:88-90)
+    explicit Tensor(float scalar) : Tensor(&scalar, Shape{}) {}
+    // Tensor(repeating:shape:)
+    static Tensor repeating(float value, const Shape &s) {
+        Tensor t(Device::Memory::allocateBuffer(s));
+        Device::Engine::fill(value, t.buffer(), t.count());
+        return t;
+    }
+
+    int dim() const { return (int)shape.size(); }
+    int64_t count() const { return count_of(shape); }
+    Buffer buffer() const { return handle->values.values; }
+    ShapedBuffer values() const { return ShapedBuffer{handle->values.values, shape}; }
+    // elements (Tensor/TensorExt.swift:275-281)
+    std::vector<float> elements() const {
+        std::vector<float> out((size_t)count());
+        Device::Memory::assign(buffer(), out.data(), count());
+        return out;
+    }
+    float item() const { return Device::Memory::getValue(buffer()); }
+
+    // view(as:) -- shares the handle; one extent may be -1 (Tensor/Operators/Shape.swift:40-67)
+    Tensor view(Shape s) const {
+        int64_t known = 1;
+        int unknown = -1;
+        for (size_t i = 0; i < s.size(); ++i) {
+            if (s[i] == -1) {
+                precondition(unknown < 0, "The size of at most one dimension can be unknown (-1).");
+                unknown = (int)i;
+            } else known *= s[i];
+        }
+        if (unknown >= 0) s[unknown] = known == 0 ? 0 : count() / known;
+        precondition(count_of(s) == count(), "Number of elements in result must be equal to number of elements in source");
+        return Tensor(handle, s);
+    }
+    Tensor unsqueezed(int at) const {
+        Shape s = shape;
+        s.insert(s.begin() + at, 1);
+        return view(s);
+    }
+    // subscript with a prefix index: a zero-copy view kept alive through `parent`
+    // (Tensor/Operators/Subscript.swift:42-67, Engine/CPU/CPU.swift:137-158)
+    Tensor operator[](const std::vector<int64_t> &index) const {
+        precondition((int)index.size() <= dim(), "index has more entries than the tensor has axes");
+        int64_t offset = 0, stride = count();
+        for (size_t i = 0; i < index.size(); ++i) {
+            precondition(index[i] >= 0 && index[i] < shape[i], "index out of bounds");
+            stride /= shape[i];
+            offset += index[i] * stride;
+        }
+        Shape rest(shape.begin() + index.size(), shape.end());
+        auto h = std::make_shared<TensorHandle>(ShapedBuffer{Device::Memory::advance(buffer(), offset), rest}, handle);
+        return Tensor(h, rest);
+    }
+
+    // ---- binary operators (Tensor/Operators/Binary.swift:44-52, :104-112, :161-169, :235-243)
+   private:
+    template <class Same, class Bc>
+    static Tensor binary(const Tensor &l, const Tensor &r, Same same, Bc bc) {
+        Tensor res(Device::Memory::allocateBuffer(shapeForBroadcastedOperands(l.shape, r.shape)));
+        if (l.shape == r.shape) same(l.buffer(), r.buffer(), res.buffer(), l.count());
+        else bc(l.values(), r.values(), res.values());
+        return res;
+    }
+
+   public:
+    friend Tensor operator+(const Tensor &l, const Tensor &r) { return binary(l, r, Device::Engine::vAdd, Device::Engine::broadcastAdd); }
+    friend Tensor operator-(const Tensor &l, const Tensor &r) { return binary(l, r, Device::Engine::vSub, Device::Engine::broadcastSub); }
+    friend Tensor operator*(const Tensor &l, const Tensor &r) { return binary(l, r, Device::Engine::vMul, Device::Engine::broadcastMul); }
+    friend Tensor operator/(const Tensor &l, const Tensor &r) { return binary(l, r, Device::Engine::vDiv, Device::Engine::broadcastDiv); }
+    Tensor operator-() const {
+        Tensor res(Device::Memory::allocateBuffer(shape));
+        Device::Engine::vNeg(buffer(), res.buffer(), count());
+        return res;
+    }
+
+    // ---- unary (Tensor/Operators/Unary.swift)
+   private:
+    template <class F>
+    Tensor unary(F f) const {
+        Tensor res(Device::Memory::allocateBuffer(shape));
+        f(values(), res.values());
+        return res;
+    }
+
+   public:
+    Tensor exp() const { return unary(Device::Engine::exp); }          // :33-36
+    Tensor tanh() const { return unary(Device::Engine::tanh); }        // :79-82
+    Tensor sqrt() const { return unary(Device::Engine::sqrt); }
+    Tensor rectifiedLinear() const { return unary(Device::Engine::relu); }
+    Tensor sigmoid() const { return Tensor(0.5f) * (*this * Tensor(0.5f)).tanh() + Tensor(0.5f); }        // :184-186
+    Tensor gaussianErrorLinear() const { return *this * (*this * Tensor(1.702f)).sigmoid(); }             // :245-247
+    Tensor softmax(int axis = 1) const {                                                                   // :190-194
+        Tensor normalizer = reduceMax({axis}).unsqueezed(axis);
+        Tensor exponentiated = (*this - normalizer).exp();
+        return exponentiated / exponentiated.reduceSum({axis}).unsqueezed(axis);
+    }
+
+    // ---- reductions (Tensor/Operators/Reduce.swift:35-46, :87-110, :216-256)
+    Shape reducedShape(const std::vector<int> &axes) const {
+        Shape s;
+        for (int i = 0; i < dim(); ++i)
+            if (std::find(axes.begin(), axes.end(), i) == axes.end()) s.push_back(shape[i]);
+        return s;
+    }
+    Tensor reduceSum(const std::vector<int> &axes) const {
+        if (axes.empty()) return *this;
+        Tensor res(Device::Memory::allocateBuffer(reducedShape(axes)));
+        Device::Engine::reduceSum(values(), res.values(), axes);
+        return res;
+    }
+    Tensor reduceMean(const std::vector<int> &axes) const {
+        int64_t n = 1;
+        for (int a : axes) n *= shape[a];
+        return reduceSum(axes) / Tensor((float)n);
+    }
+    Tensor variance(const std::vector<int> &axes) const {
+        Tensor m = reduceMean(axes);
+        return (*this * *this).reduceMean(axes) - m * m;
+    }
+    Tensor reduceMax(const std::vector<int> &axes) const {
+        precondition(axes.size() == 1, "reduceMax along several axes is not available for HIP");
+        Tensor res(Device::Memory::allocateBuffer(reducedShape(axes)));
+        Device::Engine::reduceMax(values(), res.values(), axes[0]);
+        return res;
+    }
+
+    // ---- shape (Tensor/Operators/Shape.swift:121-155): source axis i goes to destination axis axes[i]
+    Tensor permuted(const std::vector<int> &axes) const {
+        precondition((int)axes.size() == dim(), "Axis arangement must have dimensionality of source tensor");
+        Shape dst(dim());
+        for (int i = 0; i < dim(); ++i) {
+            precondition(axes[i] >= 0 && axes[i] < dim(), "Axis arangement must be a permutation");
+            dst[axes[i]] = shape[i];
+        }
+        Tensor res(Device::Memory::allocateBuffer(dst));
+        Device::Engine::permuteAxes(values(), res.values(), axes);
+        return res;
+    }
+    // Tensor(stacking:) along axis 0 (Tensor/Operators/Stack.swift:79-122)
+    static Tensor stacking(const std::vector<Tensor> &tensors) {
+        precondition(!tensors.empty(), "cannot stack zero tensors");
+        Shape s = tensors[0].shape;
+        precondition(!s.empty(), "cannot stack scalars");
+        std::vector<ShapedBuffer> bufs;
+        int64_t rows = 0;
+        for (auto &t : tensors) {
+            precondition(Shape(t.shape.begin() + 1, t.shape.end()) == Shape(s.begin() + 1, s.end()),
+                         "All vectors must have same shape except along the stacking axis");
+            rows += t.shape[0];
+            bufs.push_back(t.values());
+        }
+        s[0] = rows;
+        Tensor res(Device::Memory::allocateBuffer(s));
+        bool equal = true;
+        for (auto &t : tensors) equal = equal && t.shape == tensors[0].shape;
+        if (equal) Device::Engine::stack(bufs, res.values(), 0);
+        else {
+            int64_t off = 0;
+            for (auto &t : tensors) {
+                Device::Memory::assign(t.buffer(), Device::Memory::advance(res.buffer(), off), t.count());
+                off += t.count();
+            }
+        }
+        return res;
+    }
+    // bandMatrix (Tensor/Operators/UtilOps.swift:117-132)
+    Tensor bandMatrix(std::optional<int64_t> belowDiagonal, std::optional<int64_t> aboveDiagonal) const {
+        Tensor res(Device::Memory::allocateBuffer(shape));
+        Device::Engine::fill(0.f, res.buffer(), res.count());
+        Device::Engine::band(values(), res.values(), belowDiagonal, aboveDiagonal);
+        return res;
+    }
+
+    // ---- matrix products (Tensor/Operators/Matrix.swift:35-68, :79-135)
+   private:
+    Tensor _matMul(const Tensor &other, bool transposeSelf, bool transposeOther) const {
+        precondition(dim() == 2 && other.dim() == 2, "_matMul operands must be two dimensional");
+        precondition(shape[transposeSelf ? 0 : 1] == other.shape[transposeOther ? 1 : 0], "Matrix multiplication operands must have matching shapes.");
+        Tensor res(Device::Memory::allocateBuffer(Shape{shape[transposeSelf ? 1 : 0], other.shape[transposeOther ? 0 : 1]}));
+        Device::Engine::gemm(values(), other.values(), res.values(), 1.f, 0.f, transposeSelf, transposeOther);
+        return res;
+    }
+
+   public:
+    Tensor matrixMultiplied(const Tensor &other, bool transposeSelf = false, bool transposeOther = false) const {
+        precondition(dim() >= 1 && dim() <= 2 && other.dim() >= 1 && other.dim() <= 2,
+                     "Matrix multiplication operands must both be one or two dimensional.");
+        precondition(!(dim() == 2 && other.dim() == 2) || shape[transposeSelf ? 0 : 1] == other.shape[transposeOther ? 1 : 0],
+                     "Matrix multiplication operands must have matching shapes.");
+        Tensor l = dim() == 1 ? view({1, -1}) : *this;
+        Tensor r = other.dim() == 1 ? other.view({-1, 1}) : other;
+        Shape resultViewShape;
+        if (dim() == 1 && other.dim() == 1) resultViewShape = {};
+        else if (dim() == 1) resultViewShape = {other.shape[transposeOther ? 0 : 1]};
+        else if (other.dim() == 1) resultViewShape = {shape[transposeSelf ? 1 : 0]};
+        else resultViewShape = {shape[transposeSelf ? 1 : 0], other.shape[transposeOther ? 0 : 1]};
+        return l._matMul(r, transposeSelf && dim() == 2, transposeOther && other.dim() == 2).view(resultViewShape);
+    }
+    Tensor broadcastMatrixMultiplied(const Tensor &other, bool transposeSelf = false, bool transposeOther = false) const {
+        precondition(dim() >= 2 && other.dim() >= 2, "Operands must both be at least 2-dimensional.");
+        precondition(shape[dim() - 2 + (transposeSelf ? 0 : 1)] == other.shape[other.dim() - 2 + (transposeOther ? 1 : 0)],
+                     "Matmul operands must have matching shapes");
+        const int d = std::max(dim(), other.dim());
+        Shape ls(d - dim(), 1), rs(d - other.dim(), 1);
+        ls.insert(ls.end(), shape.begin(), shape.end());
+        rs.insert(rs.end(), other.shape.begin(), other.shape.end());
+        Tensor lhs = view(ls), rhs = other.view(rs);
+        const Shape lb(ls.begin(), ls.end() - 2), rb(rs.begin(), rs.end() - 2);
+        const Shape bshape = shapeForBroadcastedOperands(lb, rb);
+        Shape mm = {ls[d - 2 + (transposeSelf ? 1 : 0)], rs[d - 2 + (transposeOther ? 0 : 1)]};
+        Shape full = bshape;
+        full.insert(full.end(), mm.begin(), mm.end());
+        const int64_t nb = count_of(bshape);
+
+        if (Device::fused()) {
+            // one strided-batched launch when each operand is either fully batched or fully shared
+            const bool lfull = lb == bshape, rfull = rb == bshape;
+            const bool lone = count_of(lb) == 1, rone = count_of(rb) == 1;
+            if ((lfull || lone) && (rfull || rone)) {
+                Tensor res(Device::Memory::allocateBuffer(full));
+                Device::Engine::gemmBatched(lhs.values(), lfull ? ls[d - 2] * ls[d - 1] : 0, rhs.values(), rfull ? rs[d - 2] * rs[d - 1] : 0,
+                                            res.values(), nb, transposeSelf, transposeOther);
+                return res;
+            }
+        }
+        // the reference's loop: one gemm per broadcast index into its own buffer, then stack, then view
+        std::vector<Tensor> results;
+        std::vector<int64_t> idx(bshape.size()), li(bshape.size()), ri(bshape.size());
+        for (int64_t n = 0; n < nb; ++n) {
+            int64_t rem = n;
+            for (int i = (int)bshape.size() - 1; i >= 0; --i) {
+                idx[i] = rem % bshape[i];
+                rem /= bshape[i];
+                li[i] = std::min(idx[i], ls[i] - 1);
+                ri[i] = std::min(idx[i], rs[i] - 1);
+            }
+            results.push_back(lhs[li]._matMul(rhs[ri], transposeSelf, transposeOther));
+        }
+        return stacking(results).view(full);
+    }
+};
+
+inline Tensor operator*(const Tensor &l, float r) { return l * Tensor(r); }
+inline Tensor operator*(float l, const Tensor &r) { return Tensor(l) * r; }
+inline Tensor operator+(const Tensor &l, float r) { return l + Tensor(r); }
+inline Tensor operator-(float l, const Tensor &r) { return Tensor(l) - r; }
+inline Tensor operator/(const Tensor &l, float r) { return l / Tensor(r); }
+inline Tensor sqrt(const Tensor &t) { return t.sqrt(); }
+inline Tensor relu(const Tensor &t) { return t.rectifiedLinear(); }
+inline Tensor softmax(const Tensor &t, int axis) { return t.softmax(axis); }
+
+// ------------------------------------------------------------------------- layers
+// NN/Layer/LayerNorm.swift:29-78
+struct LayerNorm {
+    Tensor shift, scale;
+    explicit LayerNorm(const Shape &inputSize) : shift(Tensor::repeating(0.f, inputSize)), scale(Tensor::repeating(1.f, inputSize)) {}
+    Tensor operator()(const Tensor &x) const { return normalize(x, nullptr); }
+    // residual != nullptr: LayerNorm(x + residual) in one pass (fused mode only)
+    Tensor normalize(const Tensor &x, const Tensor *residual) const {
+        if (Device::fused() && scale.dim() == 1 && x.dim() >= 2 && x.shape.back() == scale.shape[0]) {
+            Tensor res(Device::Memory::allocateBuffer(x.shape));
+            ShapedBuffer rb;
+            if (residual) rb = residual->values();
+            Device::Engine::layerNorm(x.values(), residual ? &rb : nullptr, scale.values(), shift.values(), res.values());
+            return res;
+        }
+        const Tensor in = residual ? x + *residual : x;
+        std::vector<int> axes;
+        for (int i = 1; i < in.dim(); ++i) axes.push_back(i);
+        Shape ms(in.dim(), 1);
+        ms[0] = in.shape[0];
+        Tensor mean = in.reduceMean(axes).view(ms);
+        Tensor variance = in.variance(axes).view(ms);
+        Tensor normalized = (in - mean) / (sqrt(variance) + 1e-5f);
+        return normalized * scale + shift;
+    }
+};
+
+// NN/Layer/Dropout.swift:29-56: multiplies by a Bernoulli(1 - rate) mask drawn on the host; identity when inactive
+struct Dropout {
+    float rate;
+    bool isActive = true;
+    explicit Dropout(float r) : rate(r) {}
+    Tensor operator()(const Tensor &x) const {
+        if (!isActive) return x;
+        static std::mt19937_64 rng(0);
+        std::bernoulli_distribution keep(1.0 - rate);
+        std::vector<float> m((size_t)x.count());
+        for (auto &v : m) v = keep(rng) ? 1.f : 0.f;
+        return x * Tensor(m, x.shape);
+    }
+};
+
+// NN/Layer/Dense.swift:29-69
+struct Dense {
+    Tensor weights, bias;
+    Dense(int64_t inputSize, int64_t outputSize)
+        : weights(Tensor::repeating(0.f, {inputSize, outputSize})), bias(Tensor::repeating(0.f, {outputSize})) {}
+    Tensor operator()(const Tensor &inputs) const { return inputs.matrixMultiplied(weights) + bias; }
+};
+
+// NN/Models/Transformer/ScaledDotProductAttention.swift:29-65
+struct ScaledDotProductAttention {
+    float temperature;
+    explicit ScaledDotProductAttention(float t) : temperature(t) {}
+    Tensor operator()(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask) const {
+        precondition(k.dim() == 4, "k must have 4 dimensions");
+        if (Device::fused()) {
+            precondition(q.dim() == 4 && v.dim() == 4 && q.shape[0] == k.shape[0] && q.shape[1] == k.shape[1] &&
+                             v.shape[0] == k.shape[0] && v.shape[1] == k.shape[1] && q.shape[3] == k.shape[3] && k.shape[2] == v.shape[2],
+                         "Matmul operands must have matching shapes");
+            Tensor out(Device::Memory::allocateBuffer(Shape{q.shape[0], q.shape[1], q.shape[2], v.shape[3]}));
+            ShapedBuffer mb;
+            if (mask) mb = mask->values();
+            Device::Engine::fusedAttention(q.values(), k.values(), v.values(), mask ? &mb : nullptr, out.values(), temperature);
+            return out;
+        }
+        Tensor attn = (q / Tensor(temperature)).broadcastMatrixMultiplied(k, false, true);
+        if (mask) attn = attn - *mask * 1e9f;
+        attn = softmax(attn, 3);
+        return attn.broadcastMatrixMultiplied(v);
+    }
+};
+
+// NN/Models/Transformer/MultiHeadAttention.swift:29-128
+struct MultiHeadAttention {
+    int64_t heads, keyDim, valueDim, hiddenDim;
+    ScaledDotProductAttention attn;
+    Tensor qDense, kDense, vDense, fc;
+    LayerNorm norm;
+    Dropout dropout;
+    MultiHeadAttention(int64_t heads_, int64_t hiddenDim_, int64_t keyDim_, int64_t valueDim_, float dropoutRate = 0.1f)
+        : heads(heads_), keyDim(keyDim_), valueDim(valueDim_), hiddenDim(hiddenDim_), attn(std::sqrt((float)keyDim_)),
+          qDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})), kDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})),
+          vDense(Tensor::repeating(0.f, {hiddenDim_, valueDim_ * heads_})), fc(Tensor::repeating(0.f, {valueDim_ * heads_, hiddenDim_})),
+          norm(Shape{hiddenDim_}), dropout(dropoutRate) {}
+    Tensor operator()(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask) const {
+        const int64_t batchSize = q.shape[0], queryCount = q.shape[1], keyCount = k.shape[1], valueCount = v.shape[1];
+        const Tensor &res = q;
+        Tensor q_prep = q.broadcastMatrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
+        Tensor k_prep = k.broadcastMatrixMultiplied(kDense).view({batchSize, keyCount, heads, keyDim});
+        Tensor v_prep = v.broadcastMatrixMultiplied(vDense).view({batchSize, valueCount, heads, valueDim});
+        Tensor q_trans = q_prep.permuted({0, 2, 1, 3});
+        Tensor k_trans = k_prep.permuted({0, 2, 1, 3});
+        Tensor v_trans = v_prep.permuted({0, 2, 1, 3});
+        Tensor q_attn = attn(q_trans, k_trans, v_trans, mask);
+        Tensor out = q_attn.permuted({0, 2, 1, 3}).view({batchSize, queryCount, -1}).broadcastMatrixMultiplied(fc);
+        Tensor out_drop = dropout(out);
+        if (Device::fused()) return norm.normalize(out_drop, &res);
+        Tensor q_res = out_drop + res;
+        return norm(q_res);
+    }
+};
+
+// NN/Models/Transformer/PointwiseFeedForward.swift:32-83
+struct PointwiseFeedForward {
+    Dense dense1, dense2;
+    LayerNorm norm;
+    Dropout dropout;
+    PointwiseFeedForward(int64_t size, int64_t hiddenSize, float dropoutRate)
+        : dense1(size, hiddenSize), dense2(hiddenSize, size), norm(Shape{size}), dropout(dropoutRate) {}
+    Tensor operator()(const Tensor &inputs) const {
+        const int64_t batchSize = inputs.shape[0], seqlen = inputs.shape[1], size = inputs.shape[2];
+        Tensor denseInputs = inputs.view({batchSize * seqlen, size});
+        if (Device::fused()) {
+            Tensor h = denseInputs.matrixMultiplied(dense1.weights);
+            Device::Engine::biasGelu(h.values(), dense1.bias.values(), h.values());
+            Tensor tmp4 = dropout(dense2(h));
+            return norm.normalize(tmp4, &denseInputs).view({batchSize, seqlen, size});
+        }
+        Tensor tmp1 = dense1(denseInputs);
+        Tensor tmp2 = tmp1.gaussianErrorLinear();
+        Tensor tmp3 = dense2(tmp2);
+        Tensor tmp4 = dropout(tmp3);
+        Tensor n = norm(tmp4 + denseInputs);
+        return n.view({batchSize, seqlen, size});
+    }
+};
+
+// NN/Models/Transformer/TransformerEncoderBlock.swift:29-66
+struct TransformerEncoderBlock {
+    MultiHeadAttention selfAttention;
+    PointwiseFeedForward pointwiseFeedForward;
+    TransformerEncoderBlock(int64_t hiddenDim, int64_t forwardDim, int64_t heads, int64_t keyDim, int64_t valueDim, float dropoutRate)
+        : selfAttention(heads, hiddenDim, keyDim, valueDim, dropoutRate), pointwiseFeedForward(hiddenDim, forwardDim, dropoutRate) {}
+    Tensor operator()(const Tensor &inputs, const Tensor &mask) const {
+        Tensor attn = selfAttention(inputs, inputs, inputs, &mask);
+        return pointwiseFeedForward(attn);
+    }
+};
+
+// NN/Models/Transformer/TransformerDecoderBlock.swift:29-69
+struct TransformerDecoderBlock {
+    MultiHeadAttention selfAttention, encoderAttention;
+    PointwiseFeedForward pointwiseFeedForward;
+    TransformerDecoderBlock(int64_t hiddenDim, int64_t forwardDim, int64_t heads, int64_t keyDim, int64_t valueDim, float dropoutRate)
+        : selfAttention(heads, hiddenDim, keyDim, valueDim, dropoutRate), encoderAttention(heads, hiddenDim, keyDim, valueDim, dropoutRate),
+          pointwiseFeedForward(hiddenDim, forwardDim, dropoutRate) {}
+    Tensor operator()(const Tensor &decoderInput, const Tensor &encoderOutput, const Tensor &encoderMask, const Tensor &decoderMask) const {
+        Tensor decAttn = selfAttention(decoderInput, decoderInput, decoderInput, &decoderMask);
+        Tensor encAttn = encoderAttention(decAttn, encoderOutput, encoderOutput, &encoderMask);
+        return pointwiseFeedForward(encAttn);
+    }
+};
+
+// NN/Models/Transformer/TransformerUtil.swift:29-36
+inline Tensor makeEncoderMasks(const std::vector<int64_t> &sequenceLengths) {
+    const int64_t maxInLen = sequenceLengths.empty() ? 0 : *std::max_element(sequenceLengths.begin(), sequenceLengths.end());
+    const int64_t batchSize = (int64_t)sequenceLengths.size();
+    std::vector<float> m((size_t)(batchSize * maxInLen));
+    for (int64_t b = 0; b < batchSize; ++b)
+        for (int64_t j = 0; j < maxInLen; ++j) m[b * maxInLen + j] = j < sequenceLengths[b] ? 0.f : 1.f;
+    return Tensor(m, {batchSize, maxInLen}).view({batchSize, 1, 1, maxInLen});
+}
+
+// NN/Models/Transformer/TransformerUtil.swift:38-50
+inline Tensor makeDecoderMasks(const std::vector<int64_t> &sequenceLengths) {
+    const int64_t batchSize = (int64_t)sequenceLengths.size();
+    const int64_t maxLen = sequenceLengths.empty() ? 0 : *std::max_element(sequenceLengths.begin(), sequenceLengths.end());
+    std::vector<float> m((size_t)(batchSize * maxLen));
+    for (int64_t b = 0; b < batchSize; ++b)
+        for (int64_t j = 0; j < maxLen; ++j) m[b * maxLen + j] = j < sequenceLengths[b] ? 0.f : 1.f;
+    Tensor decoderSeqMask(m, {batchSize, maxLen});
+    Tensor decoderCausalMask = Tensor::repeating(1.f, {maxLen, maxLen}).bandMatrix(-1, std::nullopt);
+    return 1.f - relu(1.f - decoderSeqMask.view({batchSize, 1, 1, maxLen}) - decoderCausalMask);
+}
+
+}  // namespace dl4s

@@ -1,0 +1,168 @@
+// C entry points over the C++ host layer (see include/dl4s_host.h).
+#include "../../include/dl4s_host.h"
+
+#include <cstdio>
+#include <cstring>
+#include <functional>
+
+#include "dl4s_host.hpp"
+
+using namespace dl4s;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int guarded(dl4s_hip_ctx *ctx, int fused, const std::function<void()> &body) {
+    if (!ctx) {
+        snprintf(g_err, sizeof(g_err), "ctx is NULL");
+        return -1;
+    }
+    HIP::context() = ctx;
+    HIP::fused() = fused != 0;
+    try {
+        body();
+        return 0;
+    } catch (const std::exception &e) {
+        snprintf(g_err, sizeof(g_err), "%s", e.what());
+        return -1;
+    }
+}
+
+std::optional<Tensor> mask_tensor(const float *mask, const int64_t *mshape, int mdim) {
+    if (!mask) return std::nullopt;
+    Shape s(mshape, mshape + mdim);
+    return Tensor(mask, s);
+}
+
+void load(MultiHeadAttention &m, const dl4s_host_mha_params *p) {
+    m.qDense = Tensor(p->qDense, m.qDense.shape);
+    m.kDense = Tensor(p->kDense, m.kDense.shape);
+    m.vDense = Tensor(p->vDense, m.vDense.shape);
+    m.fc = Tensor(p->fc, m.fc.shape);
+    m.norm.scale = Tensor(p->norm_scale, m.norm.scale.shape);
+    m.norm.shift = Tensor(p->norm_shift, m.norm.shift.shape);
+    m.dropout.isActive = false;
+}
+
+void load(PointwiseFeedForward &f, const dl4s_host_ffn_params *p) {
+    f.dense1.weights = Tensor(p->w1, f.dense1.weights.shape);
+    f.dense1.bias = Tensor(p->b1, f.dense1.bias.shape);
+    f.dense2.weights = Tensor(p->w2, f.dense2.weights.shape);
+    f.dense2.bias = Tensor(p->b2, f.dense2.bias.shape);
+    f.norm.scale = Tensor(p->norm_scale, f.norm.scale.shape);
+    f.norm.shift = Tensor(p->norm_shift, f.norm.shift.shape);
+    f.dropout.isActive = false;
+}
+
+// runs fn `iters` times between the stream timer's begin/end and returns the last result
+Tensor timed(dl4s_hip_ctx *ctx, int iters, float *out_ms, const std::function<Tensor()> &fn) {
+    if (iters < 1) iters = 1;
+    Tensor r;
+    if (out_ms) {
+        r = fn();  // warm-up: allocations come from the pool afterwards
+        HIP::check(dl4s_hip_sync(ctx));
+        HIP::check(dl4s_hip_timer_begin(ctx));
+    }
+    for (int i = 0; i < iters; ++i) r = fn();
+    if (out_ms) {
+        float ms = 0.f;
+        HIP::check(dl4s_hip_timer_end(ctx, &ms));
+        *out_ms = ms / iters;
+    }
+    return r;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *dl4s_host_last_error(void) { return g_err; }
+
+int dl4s_host_sdpa(dl4s_hip_ctx *ctx, int fused, const float *q, const float *k, const float *v, const float *mask,
+                   const int64_t *mshape, int mdim, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
+                   float temperature, float *out, int iters, float *out_ms) {
+    return guarded(ctx, fused, [&] {
+        Tensor tq(q, {B, H, Lq, dk}), tk(k, {B, H, Lk, dk}), tv(v, {B, H, Lk, dv});
+        auto m = mask_tensor(mask, mshape, mdim);
+        ScaledDotProductAttention layer(temperature);
+        Tensor r = timed(ctx, iters, out_ms, [&] { return layer(tq, tk, tv, m ? &*m : nullptr); });
+        HIP::Memory::assign(r.buffer(), out, r.count());
+    });
+}
+
+int dl4s_host_mha(dl4s_hip_ctx *ctx, int fused, const float *q, const float *k, const float *v, const float *mask,
+                  const int64_t *mshape, int mdim, int64_t B, int64_t Lq, int64_t Lk, int64_t D, int64_t H, int64_t dk,
+                  int64_t dv, const dl4s_host_mha_params *p, float *out, int iters, float *out_ms) {
+    return guarded(ctx, fused, [&] {
+        Tensor tq(q, {B, Lq, D});
+        // q, k and v may be the same host array (self-attention): share the tensor like the caller would
+        Tensor tk = (k == q) ? tq : Tensor(k, {B, Lk, D});
+        Tensor tv = (v == q) ? tq : (v == k ? tk : Tensor(v, {B, Lk, D}));
+        auto m = mask_tensor(mask, mshape, mdim);
+        MultiHeadAttention layer(H, D, dk, dv);
+        load(layer, p);
+        Tensor r = timed(ctx, iters, out_ms, [&] { return layer(tq, tk, tv, m ? &*m : nullptr); });
+        HIP::Memory::assign(r.buffer(), out, r.count());
+    });
+}
+
+int dl4s_host_encoder_block(dl4s_hip_ctx *ctx, int fused, const float *x, const float *mask, const int64_t *mshape, int mdim,
+                            int64_t B, int64_t L, int64_t D, int64_t H, int64_t dk, int64_t dv, int64_t F,
+                            const dl4s_host_mha_params *attn, const dl4s_host_ffn_params *ffn, float *out, int iters,
+                            float *out_ms) {
+    return guarded(ctx, fused, [&] {
+        precondition(mask != nullptr, "TransformerEncoderBlock takes a mask");
+        Tensor tx(x, {B, L, D});
+        Tensor m(mask, Shape(mshape, mshape + mdim));
+        TransformerEncoderBlock block(D, F, H, dk, dv, 0.1f);
+        load(block.selfAttention, attn);
+        load(block.pointwiseFeedForward, ffn);
+        Tensor r = timed(ctx, iters, out_ms, [&] { return block(tx, m); });
+        HIP::Memory::assign(r.buffer(), out, r.count());
+    });
+}
+
+int dl4s_host_decoder_block(dl4s_hip_ctx *ctx, int fused, const float *dec, const float *enc, const float *enc_mask,
+                            const int64_t *emshape, int emdim, const float *dec_mask, const int64_t *dmshape, int dmdim,
+                            int64_t B, int64_t Ld, int64_t Le, int64_t D, int64_t H, int64_t dk, int64_t dv, int64_t F,
+                            const dl4s_host_mha_params *self_attn, const dl4s_host_mha_params *enc_attn,
+                            const dl4s_host_ffn_params *ffn, float *out, int iters, float *out_ms) {
+    return guarded(ctx, fused, [&] {
+        precondition(enc_mask && dec_mask, "TransformerDecoderBlock takes both masks");
+        Tensor td(dec, {B, Ld, D}), te(enc, {B, Le, D});
+        Tensor em(enc_mask, Shape(emshape, emshape + emdim)), dm(dec_mask, Shape(dmshape, dmshape + dmdim));
+        TransformerDecoderBlock block(D, F, H, dk, dv, 0.1f);
+        load(block.selfAttention, self_attn);
+        load(block.encoderAttention, enc_attn);
+        load(block.pointwiseFeedForward, ffn);
+        Tensor r = timed(ctx, iters, out_ms, [&] { return block(td, te, em, dm); });
+        HIP::Memory::assign(r.buffer(), out, r.count());
+    });
+}
+
+int dl4s_host_make_encoder_masks(dl4s_hip_ctx *ctx, const int64_t *lengths, int64_t B, float *out, int64_t *out_len) {
+    return guarded(ctx, 0, [&] {
+        std::vector<int64_t> lens(lengths, lengths + B);
+        int64_t L = 0;
+        for (auto l : lens) L = std::max(L, l);
+        if (out_len) *out_len = L;
+        if (!out) return;
+        Tensor m = makeEncoderMasks(lens);
+        HIP::Memory::assign(m.buffer(), out, m.count());
+    });
+}
+
+int dl4s_host_make_decoder_masks(dl4s_hip_ctx *ctx, const int64_t *lengths, int64_t B, float *out, int64_t *out_len) {
+    return guarded(ctx, 0, [&] {
+        std::vector<int64_t> lens(lengths, lengths + B);
+        int64_t L = 0;
+        for (auto l : lens) L = std::max(L, l);
+        if (out_len) *out_len = L;
+        if (!out) return;
+        Tensor m = makeDecoderMasks(lens);
+        HIP::Memory::assign(m.buffer(), out, m.count());
+    });
+}
+
+}  // extern "C"

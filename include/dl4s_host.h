@@ -1,0 +1,61 @@
+/*
+ * dl4s_host.h -- C entry points of libdl4s_host.so, the C++ host layer that mirrors DL4S's Tensor and
+ * layer interfaces (dl4s_amd/host/dl4s_host.hpp) on top of libdl4s_hip.so.  They exist so that a test
+ * or benchmark harness in any language can drive whole layers: every function uploads its host inputs,
+ * runs the layer `iters` times on the GPU (timed with the context's stream timer when out_ms != NULL),
+ * downloads the last result and returns 0, or -1 with the text in dl4s_host_last_error().
+ *
+ * `fused` selects the execution mode of the host layer: 0 issues exactly the engine primitive calls the
+ * reference's tensor operators issue; 1 lets the layers use the backend's fused entry points.
+ * A mask pointer may be NULL (no mask); mshape/mdim describe the mask tensor handed to the layer
+ * (float, 1 = blocked), which must be broadcastable to [B,H,Lq,Lk].
+ */
+#ifndef DL4S_HOST_H
+#define DL4S_HOST_H
+
+#include "dl4s_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct dl4s_host_mha_params {
+    const float *qDense, *kDense, *vDense, *fc; /* [D,H*dk], [D,H*dk], [D,H*dv], [H*dv,D] */
+    const float *norm_scale, *norm_shift;       /* [D] */
+} dl4s_host_mha_params;
+
+typedef struct dl4s_host_ffn_params {
+    const float *w1, *b1, *w2, *b2;       /* [D,F], [F], [F,D], [D] */
+    const float *norm_scale, *norm_shift; /* [D] */
+} dl4s_host_ffn_params;
+
+const char *dl4s_host_last_error(void);
+
+/* ScaledDotProductAttention(temperature)((q, k, v, mask)) -- NN/Models/Transformer/ScaledDotProductAttention.swift:43 */
+int dl4s_host_sdpa(dl4s_hip_ctx *ctx, int fused, const float *q, const float *k, const float *v, const float *mask,
+                   const int64_t *mshape, int mdim, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
+                   float temperature, float *out, int iters, float *out_ms);
+/* MultiHeadAttention(heads, hiddenDim, keyDim, valueDim)((q, k, v, mask)), dropout inactive -- MultiHeadAttention.swift:97 */
+int dl4s_host_mha(dl4s_hip_ctx *ctx, int fused, const float *q, const float *k, const float *v, const float *mask,
+                  const int64_t *mshape, int mdim, int64_t B, int64_t Lq, int64_t Lk, int64_t D, int64_t H, int64_t dk,
+                  int64_t dv, const dl4s_host_mha_params *p, float *out, int iters, float *out_ms);
+/* TransformerEncoderBlock((inputs, mask)) -- TransformerEncoderBlock.swift:58 */
+int dl4s_host_encoder_block(dl4s_hip_ctx *ctx, int fused, const float *x, const float *mask, const int64_t *mshape, int mdim,
+                            int64_t B, int64_t L, int64_t D, int64_t H, int64_t dk, int64_t dv, int64_t F,
+                            const dl4s_host_mha_params *attn, const dl4s_host_ffn_params *ffn, float *out, int iters,
+                            float *out_ms);
+/* TransformerDecoderBlock((decoderInput, encoderOutput, encoderMask, decoderMask)) -- TransformerDecoderBlock.swift:61 */
+int dl4s_host_decoder_block(dl4s_hip_ctx *ctx, int fused, const float *dec, const float *enc, const float *enc_mask,
+                            const int64_t *emshape, int emdim, const float *dec_mask, const int64_t *dmshape, int dmdim,
+                            int64_t B, int64_t Ld, int64_t Le, int64_t D, int64_t H, int64_t dk, int64_t dv, int64_t F,
+                            const dl4s_host_mha_params *self_attn, const dl4s_host_mha_params *enc_attn,
+                            const dl4s_host_ffn_params *ffn, float *out, int iters, float *out_ms);
+/* makeEncoderMasks / makeDecoderMasks -- TransformerUtil.swift:29-50.  out may be NULL to query *out_len only;
+ * encoder mask is [B,1,1,maxLen], decoder mask [B,1,maxLen,maxLen]. */
+int dl4s_host_make_encoder_masks(dl4s_hip_ctx *ctx, const int64_t *lengths, int64_t B, float *out, int64_t *out_len);
+int dl4s_host_make_decoder_masks(dl4s_hip_ctx *ctx, const int64_t *lengths, int64_t B, float *out, int64_t *out_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,74 @@
+"""Independent fp64 model of the layers on the path (numpy + scipy, BLAS matmuls).  TEST INFRASTRUCTURE.
+
+It shares no code with the C oracle: tests pin the oracle against it on small shapes, and use it as the
+referee at sizes where the single-threaded oracle would take minutes."""
+import numpy as np
+import scipy.special
+
+
+def f64(a):
+    return np.asarray(a, np.float64)
+
+
+def sdpa64(q, k, v, mask=None, temperature=None):
+    q, k, v = f64(q), f64(k), f64(v)
+    T = np.sqrt(q.shape[-1]) if temperature is None else temperature
+    s = np.matmul(q, np.swapaxes(k, -1, -2)) / T
+    if mask is not None:
+        s = s - f64(mask) * 1e9
+    return np.matmul(scipy.special.softmax(s, axis=-1), v)
+
+
+def layernorm64(x, scale, shift):
+    """NN/Layer/LayerNorm.swift:62-77: statistics over all non-batch axes, eps outside the square root."""
+    x = f64(x)
+    axes = tuple(range(1, x.ndim))
+    mean = x.mean(axis=axes, keepdims=True)
+    std = np.sqrt((x * x).mean(axis=axes, keepdims=True) - mean ** 2)
+    return (x - mean) / (std + 1e-5) * f64(scale) + f64(shift)
+
+
+def mha64(q, k, v, mask, p, H, dk, dv):
+    B, Lq, D = q.shape
+    Lk = k.shape[1]
+    qp = (f64(q) @ f64(p["Wq"])).reshape(B, Lq, H, dk).transpose(0, 2, 1, 3)
+    kp = (f64(k) @ f64(p["Wk"])).reshape(B, Lk, H, dk).transpose(0, 2, 1, 3)
+    vp = (f64(v) @ f64(p["Wv"])).reshape(B, Lk, H, dv).transpose(0, 2, 1, 3)
+    a = sdpa64(qp, kp, vp, mask, np.sqrt(dk))
+    o = a.transpose(0, 2, 1, 3).reshape(B, Lq, H * dv) @ f64(p["Wo"]) + f64(q)
+    return layernorm64(o, p["ln_scale"], p["ln_shift"])
+
+
+def ffn64(x, p):
+    shape = np.shape(x)
+    x2 = f64(x).reshape(-1, shape[-1])
+    h = x2 @ f64(p["W1"]) + f64(p["b1"])
+    g = h * scipy.special.expit(1.702 * h)
+    o = g @ f64(p["W2"]) + f64(p["b2"]) + x2
+    return layernorm64(o, p["ln_scale"], p["ln_shift"]).reshape(shape)
+
+
+def encoder_block64(x, mask, attn, ffn, H, dk, dv):
+    return ffn64(mha64(x, x, x, mask, attn, H, dk, dv), ffn)
+
+
+def decoder_block64(dec, enc, dec_mask, enc_mask, self_p, cross_p, ffn, H, dk, dv):
+    a = mha64(dec, dec, dec, dec_mask, self_p, H, dk, dv)
+    c = mha64(a, enc, enc, enc_mask, cross_p, H, dk, dv)
+    return ffn64(c, ffn)
+
+
+def xavier_uniform(rng, fan_in, fan_out):
+    a = np.sqrt(6.0 / (fan_in + fan_out))
+    return rng.uniform(-a, a, (fan_in, fan_out)).astype(np.float32)
+
+
+def make_params(rng, D, H, dk, dv, F, trivial_affine=False):
+    """Xavier-uniform weights; LayerNorm scale/shift and biases are 1/0 (the reference's init) when trivial_affine."""
+    def aff(n, centre):
+        return np.full(n, centre, np.float32) if trivial_affine else (centre + 0.1 * rng.standard_normal(n)).astype(np.float32)
+    mha = dict(Wq=xavier_uniform(rng, D, H * dk), Wk=xavier_uniform(rng, D, H * dk), Wv=xavier_uniform(rng, D, H * dv),
+               Wo=xavier_uniform(rng, H * dv, D), ln_scale=aff(D, 1.0), ln_shift=aff(D, 0.0))
+    ffn = dict(W1=xavier_uniform(rng, D, F), b1=aff(F, 0.0), W2=xavier_uniform(rng, F, D), b2=aff(D, 0.0),
+               ln_scale=aff(D, 1.0), ln_shift=aff(D, 0.0))
+    return mha, ffn

@@ -336,31 +336,7 @@ def test_mha_core_vs_torch_multi_head_attention_forward(orc):
     assert np.allclose(attn, want, rtol=1e-5, atol=5e-6)
 
 
-def _mha64(q, k, v, mask, p, H, dk, dv):
-    f = lambda a: np.asarray(a, np.float64)
-    B, Lq, D = q.shape
-    Lk = k.shape[1]
-    qp = (f(q) @ f(p["Wq"])).reshape(B, Lq, H, dk).transpose(0, 2, 1, 3)
-    kp = (f(k) @ f(p["Wk"])).reshape(B, Lk, H, dk).transpose(0, 2, 1, 3)
-    vp = (f(v) @ f(p["Wv"])).reshape(B, Lk, H, dv).transpose(0, 2, 1, 3)
-    s = np.einsum("bhqd,bhkd->bhqk", qp, kp) / np.sqrt(dk)
-    if mask is not None:
-        s = s - f(mask) * 1e9
-    a = scipy.special.softmax(s, axis=-1)
-    o = np.einsum("bhqk,bhkd->bhqd", a, vp).transpose(0, 2, 1, 3).reshape(B, Lq, H * dv) @ f(p["Wo"]) + f(q)
-    mean = o.mean(axis=(1, 2), keepdims=True)
-    std = np.sqrt((o * o).mean(axis=(1, 2), keepdims=True) - mean ** 2)
-    return (o - mean) / (std + 1e-5) * f(p["ln_scale"]) + f(p["ln_shift"])
-
-
-def _ffn64(x, p):
-    f = lambda a: np.asarray(a, np.float64)
-    h = f(x) @ f(p["W1"]) + f(p["b1"])
-    g = h * scipy.special.expit(1.702 * h)
-    o = g @ f(p["W2"]) + f(p["b2"]) + f(x)
-    mean = o.mean(axis=-1, keepdims=True)
-    std = np.sqrt((o * o).mean(axis=-1, keepdims=True) - mean ** 2)
-    return (o - mean) / (std + 1e-5) * f(p["ln_scale"]) + f(p["ln_shift"])
+from oracle.fp64_model import ffn64 as _ffn64, mha64 as _mha64  # noqa: E402
 
 
 def test_mha_ffn_blocks_vs_independent_fp64_model(orc):
@@ -392,3 +368,17 @@ def test_mha_residual_is_the_unprojected_query(orc):
     kv = rng.standard_normal((B, 3, D)).astype(np.float32)
     got = orc.mha(q, kv, kv, None, mha, H, dk, dk)
     assert np.array_equal(got, orc.layernorm(q, mha["ln_scale"], mha["ln_shift"]))
+
+
+from oracle import fp64_model as m64  # noqa: E402
+
+
+def test_oracle_agrees_with_fp64_model_on_one_config3_token_block(orc):
+    """Ties the referee used above to the oracle at the config-3 widths (D 1024, F 4096) on a short sequence."""
+    B, L, D, H, dk, F = 1, 48, 1024, 16, 64, 4096
+    rng = np.random.default_rng(33)
+    x = rng.standard_normal((B, L, D)).astype(np.float32)
+    attn, ffn = m64.make_params(rng, D, H, dk, dk, F, trivial_affine=True)
+    mask = (np.arange(L)[None, None, None, :] >= 30).astype(np.float32)
+    assert np.allclose(orc.encoder_block(x, mask, attn, ffn, H, dk, dk), m64.encoder_block64(x, mask, attn, ffn, H, dk, dk),
+                       rtol=1e-4, atol=1e-4)
