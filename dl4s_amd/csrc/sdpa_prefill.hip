@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
                                                                 const float *__restrict__ v,
                                                                 float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict,
-                                                                int nqb, int total_blocks) {
+                                                                int nqb, int total_blocks, int pair) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                     // [2][BN][LSTR]
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
@@ -60,8 +60,12 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
     const int chunk = (total_blocks + 7) / 8;
     const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
     if (w >= total_blocks) return;
-    const int bh = w / nqb;
-    const int qb = nqb - 1 - (w % nqb);  // longest causal rows first
+    // A unit of work is one block of 128 queries, or -- with causal masks on large problems -- the pair of
+    // blocks (nqb-1-p, p), whose key ranges add up to the same length for every p: all workgroups then do
+    // equal work and the launch has no long-row tail.
+    const int nunits = pair ? (nqb + 1) / 2 : nqb;
+    const int bh = w / nunits;
+    const int unit = w % nunits;
     const int b = bh / H;
     const int hh = bh % H;
 
@@ -75,6 +79,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
     constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
 
+    const int npass = (pair && unit != nqb - 1 - unit) ? 2 : 1;
+    for (int pass = 0; pass < npass; ++pass) {
+    const int qb = pair ? (pass == 0 ? nqb - 1 - unit : unit) : nqb - 1 - unit;  // longest rows first
     const int q0 = qb * BM + wave * 32;  // first query of this wavefront
     const int qi = q0 + ln;
     const int qic = qi < Lq ? qi : Lq - 1;
@@ -223,19 +230,17 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
                 for (int i = 0; i < 16; ++i) { o0[i] *= alpha; o1[i] *= alpha; }
             }
 
-            // ---- O^T += V^T . P^T
+            // ---- O^T += V^T . P^T.  Row = key (+ 4*half, folded into v_lds), columns 2*ln, 2*ln+1.
             const float *Vb = Vs + buf * TILE_FLOATS + v_lds;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int key = 8 * (r >> 2) + (r & 3);  // + 4*half, folded into v_lds
-                f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + key * LSTR);
+                const f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + (8 * (r >> 2) + (r & 3)) * LSTR);
                 o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s0[r], o0, 0, 0, 0);
                 o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s0[r], o1, 0, 0, 0);
             }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int key = 32 + 8 * (r >> 2) + (r & 3);
-                f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + key * LSTR);
+                const f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + (32 + 8 * (r >> 2) + (r & 3)) * LSTR);
                 o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s1[r], o0, 0, 0, 0);
                 o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s1[r], o1, 0, 0, 0);
             }
@@ -261,6 +266,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
             *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
         }
     }
+    }  // pass
 }
 
 // Plain fused kernel for head dims other than 64 (up to 256): one wavefront per query row, two passes over
@@ -331,7 +337,10 @@ template <int KIND>
 int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq,
                int Lk, float rT, const MaskArgs &m, int strict) {
     const int nqb = (Lq + BM - 1) / BM;
-    const long long total = (long long)nqb * B * H;
+    constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    // pair long and short causal query blocks when there is enough work to fill the GPU twice over anyway
+    const int pair = (causal_kind && !strict && nqb >= 2 && (long long)nqb * B * H >= 8ll * ctx->cu_count) ? 1 : 0;
+    const long long total = (long long)(pair ? (nqb + 1) / 2 : nqb) * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int chunk = (int)((total + 7) / 8);
     const size_t lds_bytes = 4 * TILE_FLOATS * sizeof(float);
@@ -342,7 +351,7 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         attr_set[KIND] = true;
     }
     hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
-                       Lq, Lk, rT, m, strict, nqb, (int)total);
+                       Lq, Lk, rT, m, strict, nqb, (int)total, pair);
     return dl4s::launch_status("sdpa_prefill_f32_d64");
 }
 

@@ -228,6 +228,23 @@ def test_config4_long_causal_prefill_sampled_against_oracle(ctx, orc):
         assert_parity(got[b:b + 1, h:h + 1, rows], ref, "config 4 (b=%d,h=%d)" % (b, h))
 
 
+def test_paired_causal_blocks_with_an_odd_block_count(ctx, orc):
+    """Large causal launches pair long and short 128-query blocks in one workgroup; 9 blocks leave the middle
+    one unpaired.  B16 H16 L1152 d64, checked on sampled rows of every block."""
+    from dl4s_amd import lib
+    B, H, L, d = 16, 16, 1152, 64
+    rng = np.random.default_rng(1152)
+    q, k, v = (rng.standard_normal((B, H, L, d), dtype=np.float32) for _ in range(3))
+    got = run_sdpa(ctx, q, k, v, kind=lib.MASK_CAUSAL)
+    strict = run_sdpa(ctx, q, k, v, kind=lib.MASK_CAUSAL, strict=True)     # unpaired, visits every tile
+    assert_parity(got, strict, "paired vs strict")
+    rows = np.concatenate([np.arange(0, L, 128), np.arange(127, L, 128), [500, 640, 1151]])
+    cm = causal_mask(L, L)[rows]
+    for (b, h) in [(0, 0), (15, 15)]:
+        ref = orc.sdpa(q[b:b + 1, h:h + 1, rows], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], cm)
+        assert_parity(got[b:b + 1, h:h + 1, rows], ref, "paired (b=%d,h=%d)" % (b, h))
+
+
 def test_config3_shape_padding_mask_sampled(ctx, orc):
     """SDPA core of the encoder block: B8 H16 L1024 d64, key-length mask U[512,1024]."""
     from dl4s_amd import lib
