@@ -90,6 +90,88 @@ def decode(ctx, lib, repeats):
             "shape": {"B": B, "H": H, "d": d, "T0": T0, "steps": steps}}
 
 
+def other_configs(ctx, lib, cpu):
+    """Configs 1-3 of the baseline: us/call, TFLOP/s on the algorithmic flops, fraction of the fp32 MFMA peak; the
+    CPU oracle beside each (whole call for configs 1 and 2, one batch item of config 3), single thread."""
+    from dl4s_amd import host_lib
+    from oracle import fp64_model as m64
+    res = {}
+    # config 1: SDPA B1 H8 L128 d64, no mask
+    rng = np.random.Generator(np.random.PCG64(1001))
+    q, k, v = (rng.standard_normal((1, 8, 128, 64), dtype=np.float32) for _ in range(3))
+    dq, dk, dv, out = ctx.to_device(q), ctx.to_device(k), ctx.to_device(v), ctx.empty((1, 8, 128, 64))
+    for _ in range(5):
+        ctx.sdpa_fwd(dq, dk, dv, out, 1, 8, 128, 128, 64, 64, 0.125, None, 0)
+    ctx.sync()
+    ctx.timer_begin()
+    for _ in range(200):
+        ctx.sdpa_fwd(dq, dk, dv, out, 1, 8, 128, 128, 64, 64, 0.125, None, 0)
+    us = ctx.timer_end() * 1e3 / 200
+    fl = 4.0 * 64 * 8 * 128 * 128
+    res["config1_sdpa_B1_H8_L128_d64"] = {"us_per_call": us, "tflops": fl / us / 1e6, "frac_mfma_peak": fl / us / 1e6 / MFMA_FP32_PEAK_TFLOPS,
+                                          "flops": fl, "note": "launch-latency bound (33.6 MFLOP)"}
+    for b in (dq, dk, dv, out):
+        b.release()
+    if cpu:
+        from oracle import binding as orc
+        t0 = time.perf_counter()
+        orc.sdpa(q, k, v, None)
+        dt = time.perf_counter() - t0
+        res["config1_sdpa_B1_H8_L128_d64"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
+    # config 2: MHA layer B4 L512 D512 H8 causal (dense mask tensor, as the layer receives it)
+    B, L, D, H, dk_ = 4, 512, 512, 8, 64
+    rng = np.random.Generator(np.random.PCG64(1002))
+    x = rng.standard_normal((B, L, D), dtype=np.float32)
+    attn, _ = m64.make_params(rng, D, H, dk_, dk_, 8, trivial_affine=True)
+    i, j = np.indices((L, L))
+    mask = (j > i).astype(np.float32)
+    fl = 4.0 * 64 * B * H * (L * (L + 1) // 2) + 4 * 2.0 * B * L * D * D
+    for mode, fused in (("fused", True), ("primitive", False)):
+        _, ms = host_lib.mha(ctx, x, x, x, mask, attn, H, dk_, dk_, fused=fused, iters=20)
+        res["config2_mha_B4_L512_D512_H8_causal_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
+                                                            "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
+    if cpu:
+        t0 = time.perf_counter()
+        orc.mha(x, x, x, mask, attn, H, dk_, dk_)
+        dt = time.perf_counter() - t0
+        res["config2_mha_B4_L512_D512_H8_causal_fused"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
+    # config 3: encoder block B8 L1024 D1024 H16 F4096, key-length mask
+    B, L, D, H, F = 8, 1024, 1024, 16, 4096
+    rng = np.random.Generator(np.random.PCG64(1003))
+    x = rng.standard_normal((B, L, D), dtype=np.float32)
+    attn, ffn = m64.make_params(rng, D, H, 64, 64, F, trivial_affine=True)
+    lens = rng.integers(512, 1025, size=B)
+    mask = (np.arange(L)[None, None, None, :] >= lens[:, None, None, None]).astype(np.float32)
+    fl = 4.0 * 64 * H * L * float(lens.sum()) + 4 * 2.0 * B * L * D * D + 2 * 2.0 * B * L * D * F
+    _, ms = host_lib.encoder_block(ctx, x, mask, attn, ffn, H, 64, 64, fused=True, iters=5)
+    res["config3_encoder_block_B8_L1024_D1024_H16_F4096_fused"] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
+                                                                   "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
+    if cpu:
+        t0 = time.perf_counter()
+        orc.encoder_block(x[:1, :256], mask[:1, :, :, :256], attn, ffn, H, 64, 64)
+        dt = time.perf_counter() - t0
+        fl1 = 4.0 * 64 * H * 256 * min(int(lens[0]), 256) + 4 * 2.0 * 256 * D * D + 2 * 2.0 * 256 * D * F
+        res["config3_encoder_block_B8_L1024_D1024_H16_F4096_fused"]["cpu_baseline"] = {
+            "tflops": fl1 / dt / 1e12, "cores": 1, "kind": "port",
+            "sample": "one batch item cut to 256 tokens (%.1f s); extrapolated whole call %.0f s" % (dt, dt * fl / fl1)}
+    return res
+
+
+def cpu_baseline_decode(steps_sample=1):
+    """One decode step (B16 H16 d64, T=4097) on the CPU oracle, single thread."""
+    from oracle import binding as orc
+    B, H, d, T = 16, 16, 64, 4097
+    rng = np.random.Generator(np.random.PCG64(1005))
+    kc = rng.standard_normal((B, H, T, d), dtype=np.float32)
+    vc = rng.standard_normal((B, H, T, d), dtype=np.float32)
+    q = rng.standard_normal((B, H, 1, d), dtype=np.float32)
+    t0 = time.perf_counter()
+    for _ in range(steps_sample):
+        orc.sdpa_decode(q, kc, vc, T)
+    dt = (time.perf_counter() - t0) / steps_sample
+    return {"us_per_step": dt * 1e6, "tokens_per_s": B / dt, "cores": 1, "kind": "port", "sample": "%d whole step(s) at T=4097" % steps_sample}
+
+
 def cpu_baseline_prefill(q, k, v, pairs):
     from oracle import binding as orc
     L, d = q.shape[2], q.shape[3]
@@ -113,8 +195,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--cpu-pairs", type=int, default=6, help="(batch, head) slices timed on the CPU oracle; 0 disables")
+    ap.add_argument("--cpu-pairs", type=int, default=24, help="(batch, head) slices timed on the CPU oracle; 0 disables")
     ap.add_argument("--decode-repeats", type=int, default=5)
+    ap.add_argument("--no-other-configs", dest="other_configs", action="store_false",
+                    help="skip configs 1-3 (SDPA, MHA layer, encoder block) that are reported beside the headline")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one streaming kernel (negate, 1 GiB read + 1 GiB written) so that a counter run of "
                          "this command can scale FETCH_SIZE / WRITE_SIZE by a kernel of known traffic")
@@ -137,6 +221,7 @@ def main():
         ctx.sync()
         x.release()
         y.release()
+    others = other_configs(ctx, lib, args.cpu_pairs > 0) if args.other_configs else None
     ctx.close()
 
     tflops = pre["flops"] * args.steps / pre["wall_s"] / 1e12
@@ -170,6 +255,10 @@ def main():
     if args.cpu_pairs > 0:
         q, k, v = pre["inputs"]
         line["cpu_baseline"] = cpu_baseline_prefill(q, k, v, args.cpu_pairs)
+        if dec:
+            line["decode"]["cpu_baseline"] = cpu_baseline_decode()
+    if others is not None:
+        line["other_configs"] = others
     print(json.dumps(line))
 
 
