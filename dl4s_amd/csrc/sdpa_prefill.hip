@@ -28,7 +28,7 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int HD = 64;       // head dim of the MFMA kernel
 constexpr int BM = 128;      // queries per workgroup
-constexpr int BN = 64;       // keys per LDS tile
+constexpr int BN = 32;       // keys per LDS tile
 constexpr int LSTR = 68;     // LDS row stride in floats: 64 + 4 keeps 128-bit reads of 8 rows on distinct banks
 constexpr int TILE_FLOATS = BN * LSTR;
 constexpr float LOG2E = 1.44269504088896340736f;
@@ -45,12 +45,12 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
 
 template <int KIND>
-__global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__restrict__ q,
+__global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__restrict__ q,
                                                                 const float *__restrict__ k,
                                                                 const float *__restrict__ v,
                                                                 float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict,
-                                                                int nqb, int total_blocks, int pair) {
+                                                                int nqb, int total_blocks, int lpt) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                     // [2][BN][LSTR]
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
@@ -60,12 +60,18 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
     const int chunk = (total_blocks + 7) / 8;
     const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
     if (w >= total_blocks) return;
-    // A unit of work is one block of 128 queries, or -- with causal masks on large problems -- the pair of
-    // blocks (nqb-1-p, p), whose key ranges add up to the same length for every p: all workgroups then do
-    // equal work and the launch has no long-row tail.
-    const int nunits = pair ? (nqb + 1) / 2 : nqb;
-    const int bh = w / nunits;
-    const int unit = w % nunits;
+    // Work order.  By default (batch*head)-major, so that the workgroups resident on an XCD share few K/V pairs.
+    // With causal masks on large problems (`lpt`) the blocks of each XCD's run are instead handed out longest
+    // first -- the latest query block of every pair, then the one before, ... -- so that the launch ends with the
+    // cheapest blocks and has no long-row tail.
+    int bh = w / nqb;
+    int unit = w % nqb;
+    if (lpt) {
+        const int bh_per_x = total_blocks / nqb / 8;   // the host guarantees divisibility
+        const int wl = blockIdx.x / 8;
+        unit = wl / bh_per_x;
+        bh = (blockIdx.x % 8) * bh_per_x + wl % bh_per_x;
+    }
     const int b = bh / H;
     const int hh = bh % H;
 
@@ -79,9 +85,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
     constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
 
-    const int npass = (pair && unit != nqb - 1 - unit) ? 2 : 1;
-    for (int pass = 0; pass < npass; ++pass) {
-    const int qb = pair ? (pass == 0 ? nqb - 1 - unit : unit) : nqb - 1 - unit;  // longest rows first
+    const int qb = nqb - 1 - unit;  // longest rows first
     const int q0 = qb * BM + wave * 32;  // first query of this wavefront
     const int qi = q0 + ln;
     const int qic = qi < Lq ? qi : Lq - 1;
@@ -123,10 +127,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
     const int ld_col = (tid & 15) * 4;
     const float *kbase = k + (long long)bh * Lk * HD + ld_col;
     const float *vbase = v + (long long)bh * Lk * HD + ld_col;
-    f32x4 kst[4], vst[4];
+    f32x4 kst[2], vst[2];
     auto load_tile = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 2; ++i) {
             int row = t * BN + i * 16 + ld_row;
             row = row < Lk ? row : Lk - 1;
             kst[i] = *reinterpret_cast<const f32x4 *>(kbase + (long long)row * HD);
@@ -135,7 +139,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 2; ++i) {
             int off = buf * TILE_FLOATS + (i * 16 + ld_row) * LSTR + ld_col;
             *reinterpret_cast<f32x4 *>(Ks + off) = kst[i];
             *reinterpret_cast<f32x4 *>(Vs + off) = vst[i];
@@ -164,54 +168,48 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
         const int k0 = t * BN;
 
         if (k0 < wkend) {
-            // ---- S^T = K . Q^T for two 32-key sub-tiles
-            f32x16 s0, s1;
+            // ---- S^T = K . Q^T for one 32-key tile
+            f32x16 s0, s1;   // two accumulation chains over the head dimension, added afterwards
 #pragma unroll
             for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
             const float *Kb = Ks + buf * TILE_FLOATS + k_lds;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
-                f32x4 a1 = *reinterpret_cast<const f32x4 *>(Kb + 32 * LSTR + 4 * j);
                 s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.x, qr[4 * j + 0], s1, 0, 0, 0);
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.y, qr[4 * j + 1], s1, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s1, 0, 0, 0);
                 s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, qr[4 * j + 2], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.z, qr[4 * j + 2], s1, 0, 0, 0);
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.w, qr[4 * j + 3], s1, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s1, 0, 0, 0);
             }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s0[i] += s1[i];
 
-            // ---- mask, in registers.  Accumulator register r of sub-tile u is key k0 + 32u + 8(r/4) + 4*half + r%4.
+            // ---- mask, in registers.  Accumulator register r is key k0 + 8(r/4) + 4*half + r%4.
             const bool need_mask = DENSE || (CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len)) || (k0 + BN > Lk);
             if (need_mask) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int kg = k0 + 32 * u + 8 * (r >> 2) + 4 * half + (r & 3);
-                        float s = u == 0 ? s0[r] : s1[r];
-                        if (DENSE) {
-                            const int kc = kg < Lk ? kg : Lk - 1;
-                            const float mval = mask.dense[b * mask.sb + hh * mask.sh + qic * mask.sq + kc * mask.sk];
-                            s = __fsub_rn(s, __fmul_rn(mval, 1e9f));
-                        } else {
-                            bool blocked = false;
-                            if (CAUSAL) blocked = blocked || (kg > qi);
-                            if (LENS) blocked = blocked || (kg >= len);
-                            if (blocked) s = __fsub_rn(s, 1e9f);
-                        }
-                        if (kg >= Lk) s = -INFINITY;
-                        if (u == 0) s0[r] = s; else s1[r] = s;
+                for (int r = 0; r < 16; ++r) {
+                    const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    float s = s0[r];
+                    if (DENSE) {
+                        const int kc = kg < Lk ? kg : Lk - 1;
+                        const float mval = mask.dense[b * mask.sb + hh * mask.sh + qic * mask.sq + kc * mask.sk];
+                        s = __fsub_rn(s, __fmul_rn(mval, 1e9f));
+                    } else {
+                        bool blocked = false;
+                        if (CAUSAL) blocked = blocked || (kg > qi);
+                        if (LENS) blocked = blocked || (kg >= len);
+                        if (blocked) s = __fsub_rn(s, 1e9f);
                     }
+                    if (kg >= Lk) s = -INFINITY;
+                    s0[r] = s;
                 }
             }
 
-            // ---- online softmax: lane (query ln) sees 32 of the 64 keys, lane ^ 32 the other 32
-            float tmax = fmaxf(s0[0], s1[0]);
+            // ---- online softmax: lane (query ln) sees 16 of the 32 keys, lane ^ 32 the other 16
+            float tmax = s0[0];
 #pragma unroll
-            for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, fmaxf(s0[r], s1[r]));
+            for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, s0[r]);
             tmax = fmaxf(tmax, xor32(tmax));
             const float m_new = fmaxf(m_run, tmax);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a row of -inf so far: weights 0, not NaN
@@ -221,8 +219,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 s0[r] = fast_exp2((s0[r] - m_use) * LOG2E);
-                s1[r] = fast_exp2((s1[r] - m_use) * LOG2E);
-                psum += s0[r] + s1[r];
+                psum += s0[r];
             }
             l_run = l_run * alpha + psum;
             if (__any(alpha != 1.0f)) {
@@ -237,12 +234,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
                 const f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + (8 * (r >> 2) + (r & 3)) * LSTR);
                 o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s0[r], o0, 0, 0, 0);
                 o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s0[r], o1, 0, 0, 0);
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + (32 + 8 * (r >> 2) + (r & 3)) * LSTR);
-                o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s1[r], o0, 0, 0, 0);
-                o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s1[r], o1, 0, 0, 0);
             }
         }
 
@@ -266,7 +257,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d64(const float *__re
             *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
         }
     }
-    }  // pass
 }
 
 // Plain fused kernel for head dims other than 64 (up to 256): one wavefront per query row, two passes over
@@ -338,9 +328,9 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                int Lk, float rT, const MaskArgs &m, int strict) {
     const int nqb = (Lq + BM - 1) / BM;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
-    // pair long and short causal query blocks when there is enough work to fill the GPU twice over anyway
-    const int pair = (causal_kind && !strict && nqb >= 2 && (long long)nqb * B * H >= 8ll * ctx->cu_count) ? 1 : 0;
-    const long long total = (long long)(pair ? (nqb + 1) / 2 : nqb) * B * H;
+    // longest-first order for causal masks when there is enough work to fill the GPU several times over
+    const int lpt = (causal_kind && !strict && nqb >= 2 && (B * H) % 8 == 0 && (long long)nqb * B * H >= 8ll * ctx->cu_count) ? 1 : 0;
+    const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int chunk = (int)((total + 7) / 8);
     const size_t lds_bytes = 4 * TILE_FLOATS * sizeof(float);
@@ -351,7 +341,7 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         attr_set[KIND] = true;
     }
     hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
-                       Lq, Lk, rT, m, strict, nqb, (int)total, pair);
+                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt);
     return dl4s::launch_status("sdpa_prefill_f32_d64");
 }
 
