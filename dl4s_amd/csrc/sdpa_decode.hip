@@ -78,7 +78,15 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
 
     float m_run = -INFINITY, l_run = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int kb = c0 + wave * KB; kb < c1; kb += NW * KB) {
+    // The wavefronts take the 32-key blocks of [c0, c1) round-robin, starting at a block that depends on the
+    // (batch, head) pair: all workgroups run in lockstep, and without the rotation they would all be at the same
+    // offset of their cache rows at the same time, which for some row strides (Tcap) lands on few HBM channels.
+    const int nblk = (c1 - c0 + KB - 1) / KB;
+    const int rot = nblk > 0 ? (int)(((unsigned)bh * 37u) % (unsigned)nblk) : 0;
+    for (int bi = wave; bi < nblk; bi += NW) {
+        int bb = bi + rot;
+        if (bb >= nblk) bb -= nblk;
+        const int kb = c0 + bb * KB;
         f32x4 kk[KB / 4], vv[KB / 4];
 #pragma unroll
         for (int i = 0; i < KB / 4; ++i) {
