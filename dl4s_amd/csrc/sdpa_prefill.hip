@@ -61,16 +61,21 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
     if (w >= total_blocks) return;
     // Work order.  By default (batch*head)-major, so that the workgroups resident on an XCD share few K/V pairs.
-    // With causal masks on large problems (`lpt`) the blocks of each XCD's run are instead handed out longest
-    // first -- the latest query block of every pair, then the one before, ... -- so that the launch ends with the
-    // cheapest blocks and has no long-row tail.
+    // With causal masks on large problems (`lpt` > 0) the blocks of each XCD's run are instead handed out longest
+    // first -- the latest query block of every pair of a group, then the one before, ... -- so that the launch ends
+    // with the cheapest blocks and has no long-row tail.
     int bh = w / nqb;
     int unit = w % nqb;
     if (lpt) {
+        // lpt = number of (batch, head) pairs per group: within an XCD's run the pairs are taken group by group, and
+        // inside a group longest blocks first
         const int bh_per_x = total_blocks / nqb / 8;   // the host guarantees divisibility
         const int wl = blockIdx.x / 8;
-        unit = wl / bh_per_x;
-        bh = (blockIdx.x % 8) * bh_per_x + wl % bh_per_x;
+        const int per_group = lpt * nqb;
+        const int grp = wl / per_group, r = wl % per_group;
+        const int gsize = min(lpt, bh_per_x - grp * lpt);
+        unit = r / gsize;
+        bh = (blockIdx.x % 8) * bh_per_x + grp * lpt + r % gsize;
     }
     const int b = bh / H;
     const int hh = bh % H;
@@ -329,7 +334,10 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
     const int nqb = (Lq + BM - 1) / BM;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     // longest-first order for causal masks when there is enough work to fill the GPU several times over
-    const int lpt = (causal_kind && !strict && nqb >= 2 && (B * H) % 8 == 0 && (long long)nqb * B * H >= 8ll * ctx->cu_count) ? 1 : 0;
+    // group = all pairs of the XCD: measured on B8 H16 L2048 causal, groups of 16 / 8 / 4 / 1 pairs give 120 / 111 / 107 / 87
+    // TFLOP/s and 754 / 391 / 263 / 248 MiB of L2 fills (the floor is 192 MiB): the kernel is MFMA-bound, the fills stay far
+    // below what the memory side delivers, so balance wins over L2 reuse
+    const int lpt = (causal_kind && !strict && nqb >= 2 && (B * H) % 8 == 0 && (long long)nqb * B * H >= 8ll * ctx->cu_count) ? B * H / 8 : 0;
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int chunk = (int)((total + 7) / 8);
