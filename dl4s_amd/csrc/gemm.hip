@@ -126,50 +126,63 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_mfma(GemmArgs g) {
 constexpr int ALS = GBK + 4;   // A LDS row stride (floats)
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// MI x NI = MFMA tiles per wavefront (2x2: 128x128 workgroup tile for large products, 1x1: 64x64 so that small
+// products still put a workgroup on every CU).
+template <int MI, int NI>
 __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
-    __shared__ __align__(16) float As[2][GBM][ALS];
-    __shared__ __align__(16) float Bs[2][GBK][GLS];
+    constexpr int TM = 64 * MI, TN = 64 * NI;       // workgroup tile
+    constexpr int BLS = TN + 4;                      // B LDS row stride (floats)
+    __shared__ __align__(16) float As[2][TM][ALS];
+    __shared__ __align__(16) float Bs[2][GBK][BLS];
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int half = lane >> 5, ln = lane & 31;
     const int wm = wave >> 1, wn = wave & 1;
     const int tile_m = blockIdx.x / g.tiles_n, tile_n = blockIdx.x % g.tiles_n;
-    const int m0 = tile_m * GBM, n0 = tile_n * GBN;
+    const int m0 = tile_m * TM, n0 = tile_n * TN;
     const float *A = g.A + (long long)blockIdx.z * g.a_bs;
     const float *B = g.B + (long long)blockIdx.z * g.b_bs;
     float *C = g.C + (long long)blockIdx.z * g.c_bs;
 
-    // loaders: A tile 128 x 16 = 512 float4, thread -> rows (tid/4) and (tid/4 + 64), k quad tid%4;
-    //          B tile 16 x 128 = 512 float4, thread -> rows (tid/32) and (tid/32 + 8), n quad tid%32
+    // loaders: A tile TM x 16 = TM*4 float4: thread -> rows (tid/4 + 64*i), k quad tid%4;
+    //          B tile 16 x TN = 4*TN float4: thread -> row (tid / (TN/4) + (1024/TN)*i), n quad tid % (TN/4)
+    constexpr int BQ = TN / 4, BROWS = 256 / BQ;     // float4 per B row, B rows covered per pass
     const int a_row = tid >> 2, a_kq = (tid & 3) * 4;
-    const int b_row = tid >> 5, b_nq = (tid & 31) * 4;
-    const float *ap0 = A + (long long)min(m0 + a_row, g.M - 1) * g.a_rs + a_kq;
-    const float *ap1 = A + (long long)min(m0 + a_row + 64, g.M - 1) * g.a_rs + a_kq;
-    const bool a_ok0 = m0 + a_row < g.M, a_ok1 = m0 + a_row + 64 < g.M;
+    const int b_row = tid / BQ, b_nq = (tid % BQ) * 4;
+    const float *ap[MI];
+    bool a_ok[MI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+        a_ok[i] = m0 + a_row + 64 * i < g.M;
+        ap[i] = A + (long long)min(m0 + a_row + 64 * i, g.M - 1) * g.a_rs + a_kq;
+    }
     const bool b_ok = n0 + b_nq < g.N;
     const float *bp = B + (b_ok ? n0 + b_nq : 0);
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    f32x4 ast[2], bst[2];
+    f32x4 ast[MI], bst[NI];
     auto load = [&](int kt) {
         const int k0 = kt * GBK;
         const bool kok = k0 + a_kq < g.K;
-        ast[0] = (a_ok0 && kok) ? *reinterpret_cast<const f32x4 *>(ap0 + k0) : zero;
-        ast[1] = (a_ok1 && kok) ? *reinterpret_cast<const f32x4 *>(ap1 + k0) : zero;
-        bst[0] = (b_ok && k0 + b_row < g.K) ? *reinterpret_cast<const f32x4 *>(bp + (long long)(k0 + b_row) * g.b_rs) : zero;
-        bst[1] = (b_ok && k0 + b_row + 8 < g.K) ? *reinterpret_cast<const f32x4 *>(bp + (long long)(k0 + b_row + 8) * g.b_rs) : zero;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) ast[i] = (a_ok[i] && kok) ? *reinterpret_cast<const f32x4 *>(ap[i] + k0) : zero;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int kr = k0 + b_row + BROWS * i;
+            bst[i] = (b_ok && kr < g.K) ? *reinterpret_cast<const f32x4 *>(bp + (long long)kr * g.b_rs) : zero;
+        }
     };
     auto store = [&](int buf) {
-        *reinterpret_cast<f32x4 *>(&As[buf][a_row][a_kq]) = ast[0];
-        *reinterpret_cast<f32x4 *>(&As[buf][a_row + 64][a_kq]) = ast[1];
-        *reinterpret_cast<f32x4 *>(&Bs[buf][b_row][b_nq]) = bst[0];
-        *reinterpret_cast<f32x4 *>(&Bs[buf][b_row + 8][b_nq]) = bst[1];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) *reinterpret_cast<f32x4 *>(&As[buf][a_row + 64 * i][a_kq]) = ast[i];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) *reinterpret_cast<f32x4 *>(&Bs[buf][b_row + BROWS * i][b_nq]) = bst[i];
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[MI][NI];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NI; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -181,36 +194,36 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
         const int buf = kt & 1;
         const bool more = kt + 1 < ktiles;
         if (more) load(kt + 1);
-        // A fragments of this K tile: row (wm*64 + i*32 + ln), k = 8*half .. 8*half+7
-        f32x4 af[2][2];
+        // A fragments of this K tile: row (wm*32*MI + i*32 + ln), k = 8*half .. 8*half+7
+        f32x4 af[MI][2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            af[i][0] = *reinterpret_cast<const f32x4 *>(&As[buf][wm * 64 + i * 32 + ln][8 * half]);
-            af[i][1] = *reinterpret_cast<const f32x4 *>(&As[buf][wm * 64 + i * 32 + ln][8 * half + 4]);
+        for (int i = 0; i < MI; ++i) {
+            af[i][0] = *reinterpret_cast<const f32x4 *>(&As[buf][wm * 32 * MI + i * 32 + ln][8 * half]);
+            af[i][1] = *reinterpret_cast<const f32x4 *>(&As[buf][wm * 32 * MI + i * 32 + ln][8 * half + 4]);
         }
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) {
-            const float b0 = Bs[buf][8 * half + s8][wn * 64 + ln];
-            const float b1 = Bs[buf][8 * half + s8][wn * 64 + 32 + ln];
-            const float a0 = af[0][s8 >> 2][s8 & 3];
-            const float a1 = af[1][s8 >> 2][s8 & 3];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            float bv[NI];
+#pragma unroll
+            for (int j = 0; j < NI; ++j) bv[j] = Bs[buf][8 * half + s8][wn * 32 * NI + j * 32 + ln];
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s8 >> 2][s8 & 3], bv[j], acc[i][j], 0, 0, 0);
         }
         if (more) store(buf ^ 1);
         __syncthreads();
     }
 
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int gn = n0 + wn * 64 + j * 32 + ln;
+        for (int j = 0; j < NI; ++j) {
+            const int gn = n0 + wn * 32 * NI + j * 32 + ln;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int gm = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const int gm = m0 + wm * 32 * MI + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
                 if (gm < g.M && gn < g.N) {
                     float *cp = C + (long long)gm * g.N + gn;
                     float val = g.alpha * acc[i][j][r];
@@ -238,14 +251,19 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.b_rs = tb ? 1 : rc; g.b_cs = tb ? rc : 1;
     g.a_bs = lbs; g.b_bs = rbs; g.c_bs = cbs;
     g.alpha = alpha; g.beta = beta;
-    const long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
-    g.tiles_n = (int)tn;
-    DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
     const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     const bool fast = !ta && !tb && K % 4 == 0 && N % 4 == 0 && K > 0 && aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 &&
                       rbs % 4 == 0;
-    if (fast) hipLaunchKernelGGL(gemm_f32_mfma_nn, dim3((unsigned)(tm * tn), 1, (unsigned)batch), dim3(256), 0, ctx->stream, g);
-    else hipLaunchKernelGGL(gemm_f32_mfma, dim3((unsigned)(tm * tn), 1, (unsigned)batch), dim3(256), 0, ctx->stream, g);
+    long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
+    // small products: 64x64 tiles, so that there are at least about two workgroups per CU
+    const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;
+    if (small) { tm = (M + 63) / 64; tn = (N + 63) / 64; }
+    g.tiles_n = (int)tn;
+    DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
+    const dim3 grid((unsigned)(tm * tn), 1, (unsigned)batch);
+    if (small) hipLaunchKernelGGL((gemm_f32_mfma_nn<1, 1>), grid, dim3(256), 0, ctx->stream, g);
+    else if (fast) hipLaunchKernelGGL((gemm_f32_mfma_nn<2, 2>), grid, dim3(256), 0, ctx->stream, g);
+    else hipLaunchKernelGGL(gemm_f32_mfma, grid, dim3(256), 0, ctx->stream, g);
     return dl4s::launch_status("gemm_f32_mfma");
 }
 
