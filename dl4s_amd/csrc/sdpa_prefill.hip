@@ -113,17 +113,19 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     }
     const int ntiles = (kend + BN - 1) / BN;
 
-    // Q fragment: lane holds Q[qi][half*32 + s] * rT for s = 0..31 (one rounding, like the reference)
+    // Q fragment: lane holds Q[qi][half*32 + s] * rT (one rounding, like the reference's q / temperature) times log2(e):
+    // the scores then come out of the MFMAs in the base-2 exponent domain and the weights are exp2(s - max), one
+    // subtraction per score and -- as in the reference -- the subtraction before anything can overflow.
     float qr[32];
     {
         const float *qp = q + ((long long)bh * Lq + qic) * HD + half * 32;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
-            qr[4 * j + 0] = t.x * rT;
-            qr[4 * j + 1] = t.y * rT;
-            qr[4 * j + 2] = t.z * rT;
-            qr[4 * j + 3] = t.w * rT;
+            qr[4 * j + 0] = (t.x * rT) * LOG2E;
+            qr[4 * j + 1] = (t.y * rT) * LOG2E;
+            qr[4 * j + 2] = (t.z * rT) * LOG2E;
+            qr[4 * j + 3] = (t.w * rT) * LOG2E;
         }
     }
 
@@ -154,7 +156,8 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     f32x16 o0, o1;  // O^T rows d = 2*m + {0,1}
 #pragma unroll
     for (int i = 0; i < 16; ++i) { o0[i] = 0.f; o1[i] = 0.f; }
-    float m_run = -INFINITY;
+    float m_run = -INFINITY;   // reference maximum of the row, base-2 exponent domain (see the softmax step)
+    float m_use = 0.f;         // m_run, or 0 while m_run is -inf
     float l_run = 0.f;
 
     if (ntiles > 0) {
@@ -174,20 +177,22 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
 
         if (k0 < wkend) {
             // ---- S^T = K . Q^T for one 32-key tile
-            f32x16 s0, s1;   // two accumulation chains over the head dimension, added afterwards
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+            // (one dependent accumulation chain keeps the matrix pipe full; the first MFMA takes a literal zero)
+            f32x16 s0;
             const float *Kb = Ks + buf * TILE_FLOATS + k_lds;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s1, 0, 0, 0);
+                const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
+                if (j == 0) {
+                    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[0], zero, 0, 0, 0);
+                } else {
+                    s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
+                }
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s0, 0, 0, 0);
                 s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, qr[4 * j + 2], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s0, 0, 0, 0);
             }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s0[i] += s1[i];
 
             // ---- mask, in registers.  Accumulator register r is key k0 + 8(r/4) + 4*half + r%4.
             const bool need_mask = DENSE || (CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len)) || (k0 + BN > Lk);
@@ -199,38 +204,47 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
                     if (DENSE) {
                         const int kc = kg < Lk ? kg : Lk - 1;
                         const float mval = mask.dense[b * mask.sb + hh * mask.sh + qic * mask.sq + kc * mask.sk];
-                        s = __fsub_rn(s, __fmul_rn(mval, 1e9f));
+                        s = __fsub_rn(s, __fmul_rn(__fmul_rn(mval, 1e9f), LOG2E));
                     } else {
                         bool blocked = false;
                         if (CAUSAL) blocked = blocked || (kg > qi);
                         if (LENS) blocked = blocked || (kg >= len);
-                        if (blocked) s = __fsub_rn(s, 1e9f);
+                        if (blocked) s = __fsub_rn(s, __fmul_rn(1e9f, LOG2E));
                     }
                     if (kg >= Lk) s = -INFINITY;
                     s0[r] = s;
                 }
             }
 
-            // ---- online softmax: lane (query ln) sees 16 of the 32 keys, lane ^ 32 the other 16
-            float tmax = s0[0];
+            // ---- online softmax: lane (query ln) sees 16 of the 32 keys, lane ^ 32 the other 16.
+            // Vector-ALU instructions do not overlap the matrix pipe on a SIMD (measured: their cycles add to the MFMA
+            // cycles), so the reduction is kept to about four instructions per score: max3, one fma + exp2, one add.
+            // The reference maximum m_run only moves -- and the accumulators are only rescaled -- when a tile's maximum
+            // would give a weight above 2^8; any per-row factor 2^(max - m_run) left in the weights cancels in the
+            // final division by the row sum.
+            float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
 #pragma unroll
-            for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, s0[r]);
+            for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
+            tmax = fmaxf(tmax, s0[15]);
             tmax = fmaxf(tmax, xor32(tmax));
-            const float m_new = fmaxf(m_run, tmax);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;   // a row of -inf so far: weights 0, not NaN
-            const float alpha = fast_exp2((m_run - m_use) * LOG2E);
-            m_run = m_new;
-            float psum = 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                s0[r] = fast_exp2((s0[r] - m_use) * LOG2E);
-                psum += s0[r];
-            }
-            l_run = l_run * alpha + psum;
-            if (__any(alpha != 1.0f)) {
+            const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+            if (__any(upd)) {
+                const float m_new = fmaxf(m_run, tmax);
+                // lanes whose maximum did not move keep factor 1 (also when it is still -inf: -inf - -inf would be NaN)
+                const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
+                m_run = m_new;
+                m_use = (m_new == -INFINITY) ? 0.f : m_new;      // a row of -inf so far: weights 0, not NaN
+                l_run *= alpha;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) { o0[i] *= alpha; o1[i] *= alpha; }
             }
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                s0[r] = fast_exp2(s0[r] - m_use);
+                psum += s0[r];
+            }
+            l_run += psum;
 
             // ---- O^T += V^T . P^T.  Row = key (+ 4*half, folded into v_lds), columns 2*ln, 2*ln+1.
             const float *Vb = Vs + buf * TILE_FLOATS + v_lds;
