@@ -24,6 +24,13 @@ sys.path.insert(0, ROOT)
 
 MFMA_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
+# Memory traffic per launch of the two timed kernels on these exact workloads, in bytes: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (two separate runs of this script; KiB per dispatch), scaled by what the same counters read for a 1 GiB
+# streaming kernel (--copy-calibration: x2.00 and x1.00).  The runs and their figures are summarised in
+# profiles/bench_prefill_config4_decode_config5.md; they are constants here because a counter run cannot be part of
+# the timed process.
+PREFILL_TRAFFIC_BYTES = (403886 * 2.00 + 65536 * 1.00) * 1024      # L2 fills (K/V re-reads included) + writes
+DECODE_TRAFFIC_BYTES = (264356 * 2.00 + 192 * 1.00) * 1024
 PREHEAT_S = 0.25
 
 
@@ -252,7 +259,8 @@ def main():
         "config": {"workload": "long-context prefill B=8 H=16 L=2048 d=64 causal, q/k/v=0.5*N(0,1) (BASELINE config 4)",
                    "flops_per_step": pre["flops"], "device": info["name"], "cu_count": info["cu_count"]},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": ach / MFMA_FP32_PEAK_TFLOPS, "traffic": None, "kernel": "sdpa_prefill_f32_d64",
+                     "frac": ach / MFMA_FP32_PEAK_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
+                     "traffic_unit": "bytes per launch (L2 fills + writes, rocprofv3 --pmc)", "kernel": "sdpa_prefill_f32_d64",
                      "ms_per_launch": pre["event_ms_per_launch"]},
     }
     if dec:
@@ -260,7 +268,7 @@ def main():
                                       "(BASELINE config 5)",
                           "us_per_step": dec["us_per_step"], "tokens_per_s": dec["tokens_per_s"],
                           "roofline": {"bound": "hbm", "achieved": dec["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                       "frac": dec["gbs"] / HBM_PEAK_GBS, "traffic": None,
+                                       "frac": dec["gbs"] / HBM_PEAK_GBS, "traffic": DECODE_TRAFFIC_BYTES,
                                        "kernel": "sdpa_decode_splitk_f32", "bytes_per_step": dec["bytes_per_step"]}}
     if args.cpu_pairs > 0:
         q, k, v = pre["inputs"]
