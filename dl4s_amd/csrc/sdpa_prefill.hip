@@ -2,7 +2,7 @@
 //
 // sdpa_prefill_f32_d64 is the hot kernel (head dim 64).  One workgroup = 4 wavefronts = 128
 // queries of one (batch, head); each wavefront owns 32 queries and walks the keys in LDS tiles of
-// 64.  Both contractions run on v_mfma_f32_32x32x2_f32 and are set up TRANSPOSED so that the
+// 32.  Both contractions run on v_mfma_f32_32x32x2_f32 and are set up TRANSPOSED so that the
 // probabilities never leave the registers they were computed in:
 //
 //   S^T[key, query] = K[key, :] . Q[query, :]      A operand = K (from LDS), B operand = Q (registers)
@@ -25,6 +25,7 @@ namespace {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int HD = 64;       // head dim of the MFMA kernel
 constexpr int BM = 128;      // queries per workgroup
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
                                                                 const float *__restrict__ v,
                                                                 float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict,
-                                                                int nqb, int total_blocks, int lpt) {
+                                                                int nqb, int total_blocks, int lpt, int token_major) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                     // [2][BN][LSTR]
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
@@ -98,6 +99,12 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     int len = Lk;
     if (LENS) len = mask.lengths[b];
 
+    // Tensor layout: [B,H,L,64] (row stride 64) or, token-major, [B,L,H,64] (row stride H*64): the projections of
+    // MultiHeadAttention come out token-major, so reading them in place saves the four permuteAxes copies.
+    const int rs = token_major ? H * HD : HD;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+
     // Keys this workgroup / wavefront has to visit.  Skipping is exact when every row keeps at least one
     // unblocked key (true unless len == 0) and K, V are finite at blocked keys.
     int kend = Lk, wkend = Lk;
@@ -118,7 +125,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     // subtraction per score and -- as in the reference -- the subtraction before anything can overflow.
     float qr[32];
     {
-        const float *qp = q + ((long long)bh * Lq + qic) * HD + half * 32;
+        const float *qp = q + q_base + (long long)qic * rs + half * 32;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
@@ -129,20 +136,24 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
         }
     }
 
-    // global -> LDS staging: thread covers rows (i*16 + tid/16), 4 floats at column (tid%16)*4
+    // global -> LDS staging: thread covers rows (i*16 + tid/16), 4 floats at column (tid%16)*4.  K and V are read with
+    // buffer loads: the per-thread byte offset is fixed, the tile offset is a scalar, and rows at or beyond Lk fall
+    // outside the descriptor's range and read as zeros (their scores are then set to -inf by the key bound below).
     const int ld_row = tid >> 4;
     const int ld_col = (tid & 15) * 4;
-    const float *kbase = k + (long long)bh * Lk * HD + ld_col;
-    const float *vbase = v + (long long)bh * Lk * HD + ld_col;
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + HD) * 4);   // extent of this pair's rows; the host keeps it below 2^31
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
+    const int ld_off0 = (ld_row * rs + ld_col) * 4;
+    const int ld_off1 = ld_off0 + 16 * rs * 4;
+    const int tile_bytes = BN * rs * 4;
     f32x4 kst[2], vst[2];
     auto load_tile = [&](int t) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            int row = t * BN + i * 16 + ld_row;
-            row = row < Lk ? row : Lk - 1;
-            kst[i] = *reinterpret_cast<const f32x4 *>(kbase + (long long)row * HD);
-            vst[i] = *reinterpret_cast<const f32x4 *>(vbase + (long long)row * HD);
-        }
+        const int so = t * tile_bytes;
+        kst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, ld_off0, so, 0));
+        vst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, ld_off0, so, 0));
+        kst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, ld_off1, so, 0));
+        vst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, ld_off1, so, 0));
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
@@ -264,7 +275,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     const float l_tot = l_run + xor32(l_run);
     const float inv = 1.0f / l_tot;
     if (qi < Lq) {
-        float *op = out + ((long long)bh * Lq + qi) * HD + 8 * half;
+        float *op = out + q_base + (long long)qi * rs + 8 * half;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             f32x4 a, c;
@@ -344,7 +355,7 @@ __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__
 
 template <int KIND>
 int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq,
-               int Lk, float rT, const MaskArgs &m, int strict) {
+               int Lk, float rT, const MaskArgs &m, int strict, int token_major) {
     const int nqb = (Lq + BM - 1) / BM;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     // longest-first order for causal masks when there is enough work to fill the GPU several times over
@@ -363,7 +374,7 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         attr_set[KIND] = true;
     }
     hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
-                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt);
+                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major);
     return dl4s::launch_status("sdpa_prefill_f32_d64");
 }
 
@@ -409,15 +420,22 @@ extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
         default: return dl4s::set_error(DL4S_HIP_EINVALID_ARG, "sdpa: unknown mask kind %d", m.kind);
     }
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
+    const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
+    DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR)) == 0, DL4S_HIP_EINVALID_ARG,
+                 "sdpa: unknown flag bits 0x%x", flags);
     if (dk == HD && dv == HD) {
+        // the MFMA kernel addresses one (batch, head) pair's K/V rows through a 32-bit byte offset
+        DL4S_REQUIRE(Lk * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
+                     "sdpa: the K/V rows of one (batch, head) pair span more than 2 GiB");
         switch (m.kind) {
-            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
-            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
-            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
-            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
-            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict);
+            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
+            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
+            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
+            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
+            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
         }
     }
+    DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs head dims of 64");
     DL4S_REQUIRE(dk <= GEN_MAXD && dv <= GEN_MAXD && dv > 0, DL4S_HIP_EUNSUPPORTED,
                  "sdpa: head dims (%lld, %lld) above %d are not implemented", (long long)dk, (long long)dv, GEN_MAXD);
     const long long rows = B * H * Lq;

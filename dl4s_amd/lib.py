@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libdl4s_hip.so")
 
 MASK_NONE, MASK_DENSE, MASK_CAUSAL, MASK_KEY_LENGTHS, MASK_CAUSAL_OR_KEY_LENGTHS = range(5)
 SDPA_STRICT = 1
+SDPA_TOKEN_MAJOR = 2
 OP_ADD, OP_SUB, OP_MUL, OP_DIV = range(4)
 
 _vp = C.c_void_p

@@ -100,6 +100,10 @@ typedef struct dl4s_mask_desc {
                                fully blocked tiles are skipped, which is exact as long as K and V hold finite
                                values at blocked positions (the reference computes 0 * v there, so a NaN/Inf in
                                V or K at a blocked key reaches the output only in strict mode). */
+#define DL4S_SDPA_TOKEN_MAJOR 2u /* q, out are [B,Lq,H,64] and k, v are [B,Lk,H,64] (the layout the projections of
+                                    MultiHeadAttention produce, NN/Models/Transformer/MultiHeadAttention.swift:105-107
+                                    before its permutes :109-111, and the layout its output permute :117 produces), so a
+                                    caller can drop the four permuteAxes copies.  Head dims of 64 only. */
 
 /* out = softmax((q * inv_temperature) . k^T - mask * 1e9, axis = keys) . v
  * NN/Models/Transformer/ScaledDotProductAttention.swift:43-64.  q [B,H,Lq,dk], k [B,H,Lk,dk],

@@ -20,12 +20,14 @@ def ctx():
     c.close()
 
 
-def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temperature=None):
+def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temperature=None, token_major=False):
     from dl4s_amd import lib
     B, H, Lq, dk = q.shape
     Lk, dv = v.shape[2], v.shape[3]
     T = np.float32(np.sqrt(np.float32(dk))) if temperature is None else np.float32(temperature)
     rT = float(np.float32(1.0) / T)
+    if token_major:     # hand the kernel [B,L,H,d] tensors and give the caller back [B,H,L,d]
+        q, k, v = (np.ascontiguousarray(x.transpose(0, 2, 1, 3)) for x in (q, k, v))
     bufs = [ctx.to_device(q), ctx.to_device(k), ctx.to_device(v), ctx.empty((B, H, Lq, dv))]
     desc = None
     if kind is None:
@@ -40,8 +42,11 @@ def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temper
         desc = ctx.mask_desc(kind, lengths=ld)
     elif kind == lib.MASK_CAUSAL:
         desc = ctx.mask_desc(lib.MASK_CAUSAL)
-    ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], bufs[3], B, H, Lq, Lk, dk, dv, rT, desc, lib.SDPA_STRICT if strict else 0)
+    flags = (lib.SDPA_STRICT if strict else 0) | (lib.SDPA_TOKEN_MAJOR if token_major else 0)
+    ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], bufs[3], B, H, Lq, Lk, dk, dv, rT, desc, flags)
     out = bufs[3].numpy()
+    if token_major:
+        out = np.ascontiguousarray(out.reshape(B, Lq, H, dv).transpose(0, 2, 1, 3))
     for b in bufs:
         b.release()
     return out
@@ -338,3 +343,31 @@ def test_config5_incremental_decode_append_then_attend(ctx, orc):
             assert_parity(out[t, b:b + 1, h:h + 1], ref, "config 5 step %d (b=%d,h=%d)" % (t, b, h))
     for buf in (dk_, dv_, dq, dkn, dvn, dout):
         buf.release()
+
+
+@pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 70), (1, 2, 5, 7), (2, 4, 256, 256), (1, 5, 33, 161)])
+def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk):
+    """[B,L,H,64] operands (what the projections of MultiHeadAttention produce before its permutes,
+    NN/Models/Transformer/MultiHeadAttention.swift:105-117) give the same bits as the permuted [B,H,L,64] ones."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(B * 1000 + Lq)
+    q, k, v = rand(rng, B, H, Lq, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lk, 64)
+    lens = rng.integers(1, Lk + 1, size=B)
+    dense = (rng.random((B, 1, Lq, Lk)) < 0.3).astype(np.float32)
+    cases = [dict(), dict(mask=dense), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)]
+    if Lq == Lk:
+        cases += [dict(kind=lib.MASK_CAUSAL), dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens), dict(kind=lib.MASK_CAUSAL, strict=True)]
+    for kw in cases:
+        a = run_sdpa(ctx, q, k, v, **kw)
+        b = run_sdpa(ctx, q, k, v, token_major=True, **kw)
+        assert np.array_equal(a, b), kw.keys()
+
+
+def test_token_major_rejected_for_other_head_dims_and_unknown_flags(ctx):
+    from dl4s_amd import lib
+    q = ctx.empty((1, 2, 4, 8))
+    with pytest.raises(lib.Dl4sHipError):
+        ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, 8, 8, 0.5, None, lib.SDPA_TOKEN_MAJOR)
+    with pytest.raises(lib.Dl4sHipError):
+        ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, 8, 8, 0.5, None, 64)
+    q.release()
