@@ -24,7 +24,24 @@ struct GemmArgs {
     long long a_bs, b_bs, c_bs;  // batch strides
     float alpha, beta;
     int tiles_n;
+    // epilogue of the fused Dense forms: C = act(alpha * A.B + bias[n]) + residual[m][n]
+    const float *bias, *residual;
+    int act;   // 0 none, 1 gaussianErrorLinear
 };
+
+// x * (0.5 * tanh(0.5 * (1.702 * x)) + 0.5), every operation rounded, as Tensor/Operators/Unary.swift:184-186, :245-247
+__device__ __forceinline__ float gelu_sigmoid(float v) {
+    const float a = __fmul_rn(v, 1.702f);
+    const float t = tanhf(__fmul_rn(a, 0.5f));
+    return __fmul_rn(v, __fadd_rn(__fmul_rn(0.5f, t), 0.5f));
+}
+
+__device__ __forceinline__ float epilogue(const GemmArgs &g, float val, long long gm, int gn) {
+    if (g.bias) val = __fadd_rn(val, g.bias[gn]);
+    if (g.act == 1) val = gelu_sigmoid(val);
+    if (g.residual) val = __fadd_rn(val, g.residual[gm * g.N + gn]);
+    return val;
+}
 
 __global__ __launch_bounds__(256, 2) void gemm_f32_mfma(GemmArgs g) {
     __shared__ float As[2][GBK][GLS];
@@ -112,7 +129,7 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_mfma(GemmArgs g) {
                     float *cp = C + (long long)gm * g.N + gn;
                     float val = g.alpha * acc[i][j][r];
                     if (g.beta != 0.f) val = val + g.beta * (*cp);
-                    *cp = val;
+                    *cp = epilogue(g, val, gm, gn);
                 }
             }
         }
@@ -128,7 +145,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // MI x NI = MFMA tiles per wavefront (2x2: 128x128 workgroup tile for large products, 1x1: 64x64 so that small
 // products still put a workgroup on every CU).
-template <int MI, int NI>
+template <int MI, int NI, bool EPI>
 __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
     constexpr int TM = 64 * MI, TN = 64 * NI;       // workgroup tile
     constexpr int BLS = TN + 4;                      // B LDS row stride (floats)
@@ -228,14 +245,15 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
                     float *cp = C + (long long)gm * g.N + gn;
                     float val = g.alpha * acc[i][j][r];
                     if (g.beta != 0.f) val = val + g.beta * (*cp);
-                    *cp = val;
+                    *cp = EPI ? epilogue(g, val, gm, gn) : val;
                 }
             }
         }
 }
 
 int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int64_t lbs, const float *rhs, int64_t rr,
-                int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb) {
+                int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb,
+                const float *bias = nullptr, const float *residual = nullptr, int act = 0) {
     DL4S_REQUIRE(lr >= 0 && lc >= 0 && rr >= 0 && rc >= 0 && batch >= 0, DL4S_HIP_EINVALID_ARG, "gemm: negative extent");
     const int64_t M = ta ? lc : lr, K = ta ? lr : lc;
     const int64_t K2 = tb ? rc : rr, N = tb ? rr : rc;
@@ -251,6 +269,8 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.b_rs = tb ? 1 : rc; g.b_cs = tb ? rc : 1;
     g.a_bs = lbs; g.b_bs = rbs; g.c_bs = cbs;
     g.alpha = alpha; g.beta = beta;
+    g.bias = bias; g.residual = residual; g.act = act;
+    const bool epi = bias || residual || act;
     const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     const bool fast = !ta && !tb && K % 4 == 0 && N % 4 == 0 && K > 0 && aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 &&
                       rbs % 4 == 0;
@@ -261,8 +281,10 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.tiles_n = (int)tn;
     DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
     const dim3 grid((unsigned)(tm * tn), 1, (unsigned)batch);
-    if (small) hipLaunchKernelGGL((gemm_f32_mfma_nn<1, 1>), grid, dim3(256), 0, ctx->stream, g);
-    else if (fast) hipLaunchKernelGGL((gemm_f32_mfma_nn<2, 2>), grid, dim3(256), 0, ctx->stream, g);
+    if (small && epi) hipLaunchKernelGGL((gemm_f32_mfma_nn<1, 1, true>), grid, dim3(256), 0, ctx->stream, g);
+    else if (small) hipLaunchKernelGGL((gemm_f32_mfma_nn<1, 1, false>), grid, dim3(256), 0, ctx->stream, g);
+    else if (fast && epi) hipLaunchKernelGGL((gemm_f32_mfma_nn<2, 2, true>), grid, dim3(256), 0, ctx->stream, g);
+    else if (fast) hipLaunchKernelGGL((gemm_f32_mfma_nn<2, 2, false>), grid, dim3(256), 0, ctx->stream, g);
     else hipLaunchKernelGGL(gemm_f32_mfma, grid, dim3(256), 0, ctx->stream, g);
     return dl4s::launch_status("gemm_f32_mfma");
 }
@@ -287,6 +309,15 @@ int dl4s_hip_gemm_batched_f32(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_r
     DL4S_REQUIRE(lhs_stride >= 0 && rhs_stride >= 0 && result_stride >= 0, DL4S_HIP_EINVALID_ARG, "gemm: negative batch stride");
     return gemm_launch(ctx, lhs, lhs_rows, lhs_cols, lhs_stride, rhs, rhs_rows, rhs_cols, rhs_stride, result, result_stride,
                        batch, alpha, beta, transpose_first, transpose_second);
+}
+
+int dl4s_hip_dense_fused_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t in_features, const float *weights,
+                             int64_t out_features, const float *bias, int activation, const float *residual, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(activation == DL4S_ACT_NONE || activation == DL4S_ACT_GELU, DL4S_HIP_EINVALID_ARG,
+                 "dense: unknown activation %d", activation);
+    return gemm_launch(ctx, x, rows, in_features, 0, weights, in_features, out_features, 0, result, 0, 1, 1.0f, 0.0f, 0, 0, bias,
+                       residual, activation);
 }
 
 }  // extern "C"

@@ -177,8 +177,9 @@ struct HIP {
                                      result.values.memory));
         }
         // Fused entry points of this backend (no counterpart in EngineType).
+        // tokenMajor: q, result are [B,Lq,H,d] and k, v [B,Lk,H,d] (the projections before their permutes)
         static void fusedAttention(const ShapedBuffer &q, const ShapedBuffer &k, const ShapedBuffer &v, const ShapedBuffer *mask,
-                                   const ShapedBuffer &result, float temperature) {
+                                   const ShapedBuffer &result, float temperature, bool tokenMajor = false) {
             dl4s_mask_desc md{};
             if (mask) {
                 precondition(mask->dim() <= 4, "mask must be broadcastable to [batchSize, heads, queryCount, keyCount]");
@@ -187,9 +188,19 @@ struct HIP {
                 for (int i = 0; i < 4; ++i) md.shape[i] = 1;
                 for (int i = 0; i < mask->dim(); ++i) md.shape[4 - mask->dim() + i] = mask->shape[i];
             }
+            const int h = tokenMajor ? 2 : 1, l = tokenMajor ? 1 : 2;
             check(dl4s_hip_sdpa_fwd_f32(context(), q.values.memory, k.values.memory, v.values.memory, result.values.memory,
-                                        q.shape[0], q.shape[1], q.shape[2], k.shape[2], q.shape[3], v.shape[3],
-                                        1.0f / temperature, mask ? &md : nullptr, DL4S_SDPA_STRICT));
+                                        q.shape[0], q.shape[h], q.shape[l], k.shape[l], q.shape[3], v.shape[3],
+                                        1.0f / temperature, mask ? &md : nullptr,
+                                        DL4S_SDPA_STRICT | (tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u)));
+        }
+        // result = act(x . weights + bias) + residual  (bias, residual optional)
+        static void denseFused(const ShapedBuffer &x, const ShapedBuffer &weights, const ShapedBuffer *bias, int activation,
+                               const ShapedBuffer *residual, const ShapedBuffer &result) {
+            precondition(x.count() % weights.shape[0] == 0, "Matmul operands must have matching shapes");
+            check(dl4s_hip_dense_fused_f32(context(), x.values.memory, x.count() / weights.shape[0], weights.shape[0],
+                                           weights.values.memory, weights.shape[1], bias ? bias->values.memory : nullptr, activation,
+                                           residual ? residual->values.memory : nullptr, result.values.memory));
         }
         static void gemmBatched(const ShapedBuffer &lhs, int64_t lstride, const ShapedBuffer &rhs, int64_t rstride,
                                 const ShapedBuffer &result, int64_t batch, bool tA, bool tB) {
@@ -542,6 +553,17 @@ struct Dense {
     Dense(int64_t inputSize, int64_t outputSize)
         : weights(Tensor::repeating(0.f, {inputSize, outputSize})), bias(Tensor::repeating(0.f, {outputSize})) {}
     Tensor operator()(const Tensor &inputs) const { return inputs.matrixMultiplied(weights) + bias; }
+    // fused mode: act(inputs . weights + bias) + residual as one product with an epilogue; inputs [..., inputSize]
+    Tensor fused(const Tensor &inputs, int activation, const Tensor *residual) const {
+        Shape os(inputs.shape.begin(), inputs.shape.end() - 1);
+        os.push_back(weights.shape[1]);
+        Tensor out(Device::Memory::allocateBuffer(os));
+        const ShapedBuffer bb = bias.values();
+        ShapedBuffer rb;
+        if (residual) rb = residual->values();
+        Device::Engine::denseFused(inputs.values(), weights.values(), &bb, activation, residual ? &rb : nullptr, out.values());
+        return out;
+    }
 };
 
 // NN/Models/Transformer/ScaledDotProductAttention.swift:29-65
@@ -582,6 +604,27 @@ struct MultiHeadAttention {
     Tensor operator()(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask) const {
         const int64_t batchSize = q.shape[0], queryCount = q.shape[1], keyCount = k.shape[1], valueCount = v.shape[1];
         const Tensor &res = q;
+        if (Device::fused() && keyDim == 64 && valueDim == 64) {
+            // the projections are read where they lie ([B,L,H,64]) and the attention output is written as
+            // [B,Lq,H,64] = [B,Lq,H*64]: no permuteAxes; the residual rides in the epilogue of the fc product
+            precondition(q.dim() == 3 && k.dim() == 3 && v.dim() == 3 && keyCount == valueCount, "Matmul operands must have matching shapes");
+            Tensor qp = q.view({batchSize * queryCount, hiddenDim}).matrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
+            Tensor kp = k.view({batchSize * keyCount, hiddenDim}).matrixMultiplied(kDense).view({batchSize, keyCount, heads, keyDim});
+            Tensor vp = v.view({batchSize * valueCount, hiddenDim}).matrixMultiplied(vDense).view({batchSize, valueCount, heads, valueDim});
+            Tensor a(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, heads, valueDim}));
+            ShapedBuffer mb;
+            if (mask) mb = mask->values();
+            Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true);
+            Tensor a2 = a.view({batchSize * queryCount, heads * valueDim});
+            if (!dropout.isActive) {
+                Tensor sum(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, hiddenDim}));
+                const ShapedBuffer rb = res.values();
+                Device::Engine::denseFused(a2.values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, sum.values());
+                return norm.normalize(sum, nullptr);
+            }
+            Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
+            return norm.normalize(out_drop, &res);
+        }
         Tensor q_prep = q.broadcastMatrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
         Tensor k_prep = k.broadcastMatrixMultiplied(kDense).view({batchSize, keyCount, heads, keyDim});
         Tensor v_prep = v.broadcastMatrixMultiplied(vDense).view({batchSize, valueCount, heads, valueDim});
@@ -608,9 +651,9 @@ struct PointwiseFeedForward {
         const int64_t batchSize = inputs.shape[0], seqlen = inputs.shape[1], size = inputs.shape[2];
         Tensor denseInputs = inputs.view({batchSize * seqlen, size});
         if (Device::fused()) {
-            Tensor h = denseInputs.matrixMultiplied(dense1.weights);
-            Device::Engine::biasGelu(h.values(), dense1.bias.values(), h.values());
-            Tensor tmp4 = dropout(dense2(h));
+            Tensor h = dense1.fused(denseInputs, DL4S_ACT_GELU, nullptr);
+            if (!dropout.isActive) return norm.normalize(dense2.fused(h, DL4S_ACT_NONE, &denseInputs), nullptr).view({batchSize, seqlen, size});
+            Tensor tmp4 = dropout(dense2.fused(h, DL4S_ACT_NONE, nullptr));
             return norm.normalize(tmp4, &denseInputs).view({batchSize, seqlen, size});
         }
         Tensor tmp1 = dense1(denseInputs);

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libdl4s_hip.so")
 MASK_NONE, MASK_DENSE, MASK_CAUSAL, MASK_KEY_LENGTHS, MASK_CAUSAL_OR_KEY_LENGTHS = range(5)
 SDPA_STRICT = 1
 SDPA_TOKEN_MAJOR = 2
+ACT_NONE, ACT_GELU = 0, 1
 OP_ADD, OP_SUB, OP_MUL, OP_DIV = range(4)
 
 _vp = C.c_void_p
@@ -219,6 +220,11 @@ class Context:
     def layernorm(self, x, residual, scale, shift, y, B, rows, D):
         _check(self.lib.dl4s_hip_layernorm_f32(self.handle, _vp(_ptr(x)), _vp(_ptr(residual)) if residual is not None else None,
                                                _vp(_ptr(scale)), _vp(_ptr(shift)), _vp(_ptr(y)), _i64(B), _i64(rows), _i64(D)))
+
+    def dense_fused(self, x, rows, in_features, weights, out_features, bias, activation, residual, y):
+        _check(self.lib.dl4s_hip_dense_fused_f32(self.handle, _vp(_ptr(x)), _i64(rows), _i64(in_features), _vp(_ptr(weights)),
+                                                 _i64(out_features), _vp(_ptr(bias)) if bias is not None else None, int(activation),
+                                                 _vp(_ptr(residual)) if residual is not None else None, _vp(_ptr(y))))
 
     def bias_gelu(self, x, bias, y, rows, D):
         _check(self.lib.dl4s_hip_bias_gelu_f32(self.handle, _vp(_ptr(x)), _vp(_ptr(bias)) if bias is not None else None,

@@ -191,6 +191,18 @@ int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *resid
  * (Dense bias, NN/Layer/Dense.swift:64-68). */
 int dl4s_hip_bias_gelu_f32(dl4s_hip_ctx *ctx, const float *x, const float *bias, float *result, int64_t rows,
                            int64_t D);
+/* The Dense layer with its neighbours folded into the product's epilogue:
+ *   result = act(x . weights + bias) + residual
+ * x [rows, in], weights [in, out], bias [out] or NULL, residual [rows, out] or NULL, result [rows, out].
+ * Dense: NN/Layer/Dense.swift:64-68 (matrixMultiplied, then + bias); activation DL4S_ACT_GELU is
+ * gaussianErrorLinear (Tensor/Operators/Unary.swift:245-247) as PointwiseFeedForward applies it to dense1
+ * (NN/Models/Transformer/PointwiseFeedForward.swift:75-76); the residual is the `+ denseInputs` of
+ * PointwiseFeedForward.swift:79 and the `+ res` of MultiHeadAttention.swift:122 (fc has no bias).  Every step is
+ * rounded to fp32 like the separate engine calls, in the same order.  result may alias residual. */
+#define DL4S_ACT_NONE 0
+#define DL4S_ACT_GELU 1
+int dl4s_hip_dense_fused_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t in_features, const float *weights,
+                             int64_t out_features, const float *bias, int activation, const float *residual, float *result);
 
 #ifdef __cplusplus
 }

@@ -235,3 +235,48 @@ def test_bias_gelu(ctx, orc):
     assert_parity(dy.numpy(), orc.gelu(x), "gelu")
     for t in (dx, db, dy):
         t.release()
+
+
+@pytest.mark.parametrize("M,K,N", [(130, 64, 72), (256, 128, 256), (64, 512, 1024), (7, 5, 3), (300, 100, 260)])
+@pytest.mark.parametrize("act", [0, 1])
+@pytest.mark.parametrize("with_bias,with_res", [(True, False), (False, True), (True, True)])
+def test_dense_fused_equals_separate_engine_calls(ctx, orc, M, K, N, act, with_bias, with_res):
+    """act(x.W + b) + r as one product with an epilogue: the same bits as gemm, then bias (+ GELU), then vAdd, and within
+    tolerance of the oracle's Dense / gaussianErrorLinear / residual sequence."""
+    from dl4s_amd import lib
+    x, W, b, r = rnd(M, K), rnd(K, N) * np.float32(0.2), rnd(N), rnd(M, N)
+    dx, dW, db, dr = ctx.to_device(x), ctx.to_device(W), ctx.to_device(b), ctx.to_device(r)
+    fused, sep = ctx.empty((M, N)), ctx.empty((M, N))
+    ctx.dense_fused(dx, M, K, dW, N, db if with_bias else None, act, dr if with_res else None, fused)
+    ctx.gemm(dx, (M, K), dW, (K, N), sep)
+    if act:
+        ctx.bias_gelu(sep, db if with_bias else None, sep, M, N)
+    elif with_bias:
+        ctx.broadcast(lib.OP_ADD, sep, (M, N), db, (N,), sep)
+    if with_res:
+        ctx.vadd(sep, dr, sep, M * N)
+    assert np.array_equal(fused.numpy(), sep.numpy())
+    ref = orc.gemm(x, W, False, False)
+    if with_bias:
+        ref = ref + b
+    if act:
+        ref = orc.gelu(ref)
+    if with_res:
+        ref = ref + r
+    assert_parity(fused.numpy(), ref, "dense fused")
+    # the result may alias the residual
+    if with_res:
+        ctx.dense_fused(dx, M, K, dW, N, db if with_bias else None, act, dr, dr)
+        assert np.array_equal(dr.numpy(), fused.numpy())
+    for t in (dx, dW, db, dr, fused, sep):
+        t.release()
+
+
+def test_dense_fused_errors(ctx):
+    from dl4s_amd import lib
+    a = ctx.empty((4, 4))
+    with pytest.raises(lib.Dl4sHipError):
+        ctx.dense_fused(a, 4, 4, a, 4, None, 7, None, a)
+    with pytest.raises(lib.Dl4sHipError):
+        ctx.dense_fused(a, -1, 4, a, 4, None, 0, None, a)
+    a.release()
