@@ -39,7 +39,38 @@ struct MaskArgs {
     const float *dense;
     long long sb, sh, sq, sk;  // element strides of the dense mask, 0 on broadcast axes
     const int *lengths;
+    // dense masks, optional: one class per 32-query x 32-key tile (0 = all zeros, 1 = all ones, 2 = anything else),
+    // laid out [slab][q tile][k tile] with slab / tile strides 0 on the mask's broadcast axes
+    const unsigned char *cls;
+    int cls_sb, cls_sh, cls_sq, cls_sk;
 };
+
+// Classifies the 32 x 32 tiles of a dense mask so that the attention kernel only reads mask values where a tile is
+// neither all zeros nor all ones.  One wavefront per tile; elements outside [Lq, Lk] count as matching.
+__global__ __launch_bounds__(256) void sdpa_mask_classify(MaskArgs m, int MB, int MH, int nqt, int nkt, int Lq, int Lk,
+                                                          long long total, unsigned char *cls) {
+    const long long tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tile >= total) return;
+    const int lane = threadIdx.x & 63;
+    const int kt = (int)(tile % nkt);
+    const int qt = (int)((tile / nkt) % nqt);
+    const int hm = (int)((tile / nkt / nqt) % MH);
+    const int bm = (int)(tile / nkt / nqt / MH);
+    const int col = kt * 32 + (lane & 31);
+    const int nrow = m.sq ? 32 : 1, ncol_ok = (m.sk ? col < Lk : (lane & 31) == 0);
+    bool all0 = true, all1 = true;
+    const float *base = m.dense + bm * m.sb + hm * m.sh;
+    for (int r = lane >> 5; r < nrow; r += 2) {
+        const int row = qt * 32 + r;
+        if (ncol_ok && (!m.sq || row < Lq)) {
+            const float x = base[row * m.sq + col * m.sk];
+            all0 = all0 && (x == 0.0f);
+            all1 = all1 && (x == 1.0f);
+        }
+    }
+    const int z = __all(all0), o = __all(all1);
+    if (lane == 0) cls[tile] = z ? 0 : (o ? 1 : 2);
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -62,21 +93,32 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
     if (w >= total_blocks) return;
     // Work order.  By default (batch*head)-major, so that the workgroups resident on an XCD share few K/V pairs.
-    // With causal masks on large problems (`lpt` > 0) the blocks of each XCD's run are instead handed out longest
-    // first -- the latest query block of every pair of a group, then the one before, ... -- so that the launch ends
-    // with the cheapest blocks and has no long-row tail.
+    // With causal masks (`lpt`) the items of each XCD's run are instead handed out longest first -- the latest query
+    // block of every pair in the run, then the one before, ... -- so that the hardware dispatcher does
+    // longest-processing-time scheduling and the launch ends on the cheapest blocks.
     int bh = w / nqb;
-    int unit = w % nqb;
+    int unit = w % nqb;   // 0 = the last (longest) query block of the pair
     if (lpt) {
-        // lpt = number of (batch, head) pairs per group: within an XCD's run the pairs are taken group by group, and
-        // inside a group longest blocks first
-        const int bh_per_x = total_blocks / nqb / 8;   // the host guarantees divisibility
+        // The run is w in [a, a + n).  Item `wl` of the run in (unit ascending, w ascending) order: every unit occurs c
+        // times, the `rem` units of the cyclic interval starting at s once more.
+        const int a = (blockIdx.x % 8) * chunk;
+        const int n = min(chunk, total_blocks - a);
         const int wl = blockIdx.x / 8;
-        const int per_group = lpt * nqb;
-        const int grp = wl / per_group, r = wl % per_group;
-        const int gsize = min(lpt, bh_per_x - grp * lpt);
-        unit = r / gsize;
-        bh = (blockIdx.x % 8) * bh_per_x + grp * lpt + r % gsize;
+        const int c = n / nqb, rem = n % nqb, s = a % nqb;
+        const int wrap = s + rem - nqb;   // > 0: the interval wraps around to units [0, wrap)
+        auto before = [&](int U) {        // items with unit < U
+            const int extra = wrap > 0 ? min(U, wrap) + max(0, U - s) : min(max(U - s, 0), rem);
+            return c * U + extra;
+        };
+        int lo = 0, hi = nqb - 1;         // largest U with before(U) <= wl
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (before(mid) <= wl) lo = mid; else hi = mid - 1;
+        }
+        unit = lo;
+        const int j = wl - before(lo);
+        const int w2 = a + (lo - s + nqb) % nqb + j * nqb;
+        bh = w2 / nqb;
     }
     const int b = bh / H;
     const int hh = bh % H;
@@ -180,11 +222,16 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     const int k_lds = ln * LSTR + half * 32;        // K fragment base: row ln, columns half*32..
     const int v_lds = (4 * half) * LSTR + 2 * ln;   // V fragment base: row 4*half (+ const), columns 2*ln, 2*ln+1
 
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;   // wavefronts past Lq store nothing
+
     for (int t = 0; t < ntiles; ++t) {
         const int buf = t & 1;
         const bool more = (t + 1 < ntiles);
         if (more) load_tile(t + 1);
         const int k0 = t * BN;
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk];
 
         if (k0 < wkend) {
             // ---- S^T = K . Q^T for one 32-key tile
@@ -206,24 +253,34 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
             }
 
             // ---- mask, in registers.  Accumulator register r is key k0 + 8(r/4) + 4*half + r%4.
-            const bool need_mask = DENSE || (CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len)) || (k0 + BN > Lk);
-            if (need_mask) {
+            if (DENSE) {
+                if (cls == 1) {           // every element of the tile is 1: the penalty is a constant
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+                } else if (cls == 2) {    // mixed tile: read the mask values (class 0 = all zeros needs nothing)
+                    const float *mrow = mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        const int kc = kg < Lk ? kg : Lk - 1;
+                        s0[r] = __fsub_rn(s0[r], __fmul_rn(__fmul_rn(mrow[kc * mask.sk], 1e9f), LOG2E));
+                    }
+                }
+            } else if ((CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len))) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    float s = s0[r];
-                    if (DENSE) {
-                        const int kc = kg < Lk ? kg : Lk - 1;
-                        const float mval = mask.dense[b * mask.sb + hh * mask.sh + qic * mask.sq + kc * mask.sk];
-                        s = __fsub_rn(s, __fmul_rn(__fmul_rn(mval, 1e9f), LOG2E));
-                    } else {
-                        bool blocked = false;
-                        if (CAUSAL) blocked = blocked || (kg > qi);
-                        if (LENS) blocked = blocked || (kg >= len);
-                        if (blocked) s = __fsub_rn(s, __fmul_rn(1e9f, LOG2E));
-                    }
-                    if (kg >= Lk) s = -INFINITY;
-                    s0[r] = s;
+                    bool blocked = false;
+                    if (CAUSAL) blocked = blocked || (kg > qi);
+                    if (LENS) blocked = blocked || (kg >= len);
+                    if (blocked) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+                }
+            }
+            if (k0 + BN > Lk) {           // keys past the end of the tensor take no part
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    if (kg >= Lk) s0[r] = -INFINITY;
                 }
             }
 
@@ -358,11 +415,11 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                int Lk, float rT, const MaskArgs &m, int strict, int token_major) {
     const int nqb = (Lq + BM - 1) / BM;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
-    // longest-first order for causal masks when there is enough work to fill the GPU several times over
-    // group = all pairs of the XCD: measured on B8 H16 L2048 causal, groups of 16 / 8 / 4 / 1 pairs give 120 / 111 / 107 / 87
-    // TFLOP/s and 754 / 391 / 263 / 248 MiB of L2 fills (the floor is 192 MiB): the kernel is MFMA-bound, the fills stay far
-    // below what the memory side delivers, so balance wins over L2 reuse
-    const int lpt = (causal_kind && !strict && nqb >= 2 && (B * H) % 8 == 0 && (long long)nqb * B * H >= 8ll * ctx->cu_count) ? B * H / 8 : 0;
+    // longest-first order for causal masks.  Measured on B8 H16 L2048 causal with the order applied to groups of
+    // 16 (= the whole run) / 8 / 4 / 1 pairs: 120 / 111 / 107 / 87 TFLOP/s and 754 / 391 / 263 / 248 MiB of L2 fills
+    // (the floor is 192 MiB): the kernel is MFMA-bound, the fills stay far below what the memory side delivers, so
+    // balance wins over L2 reuse.
+    const int lpt = (causal_kind && !strict && nqb >= 2) ? 1 : 0;
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int chunk = (int)((total + 7) / 8);
@@ -418,6 +475,25 @@ extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
             break;
         case DL4S_MASK_CAUSAL: break;
         default: return dl4s::set_error(DL4S_HIP_EINVALID_ARG, "sdpa: unknown mask kind %d", m.kind);
+    }
+    if (m.kind == DL4S_MASK_DENSE_F32 && dk == HD && dv == HD) {
+        const int64_t MB = m.sb ? B : 1, MH = m.sh ? H : 1;
+        const int64_t nqt = m.sq ? (Lq + 31) / 32 : 1, nkt = m.sk ? (Lk + 31) / 32 : 1;
+        const long long total = MB * MH * nqt * nkt;
+        if (total < (1ll << 31)) {
+            const int rc = dl4s::ensure_scratch(ctx, (size_t)total);
+            if (rc != DL4S_HIP_OK) return rc;
+            unsigned char *cls = static_cast<unsigned char *>(ctx->scratch);
+            hipLaunchKernelGGL(sdpa_mask_classify, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, ctx->stream, m, (int)MB,
+                               (int)MH, (int)nqt, (int)nkt, (int)Lq, (int)Lk, total, cls);
+            const int st = dl4s::launch_status("sdpa_mask_classify");
+            if (st != DL4S_HIP_OK) return st;
+            m.cls = cls;
+            m.cls_sk = m.sk ? 1 : 0;
+            m.cls_sq = m.sq ? (int)nkt : 0;
+            m.cls_sh = m.sh ? (int)(nqt * nkt) : 0;
+            m.cls_sb = m.sb ? (int)(MH * nqt * nkt) : 0;
+        }
     }
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;

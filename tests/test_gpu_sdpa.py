@@ -371,3 +371,34 @@ def test_token_major_rejected_for_other_head_dims_and_unknown_flags(ctx):
     with pytest.raises(lib.Dl4sHipError):
         ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, 8, 8, 0.5, None, 64)
     q.release()
+
+
+@pytest.mark.parametrize("mshape", ["full", "b1qk", "qk", "b11k", "k", "bh1k", "1hq1"])
+def test_dense_mask_with_uniform_and_mixed_tiles(ctx, orc, mshape):
+    """Dense masks whose 32 x 32 tiles are all zeros, all ones or mixed (the kernel reads mask values only in mixed
+    tiles), on every broadcast shape the reference accepts."""
+    B, H, Lq, Lk = 2, 3, 150, 200
+    rng = np.random.default_rng(len(mshape) * 17 + 3)
+    q, k, v = rand(rng, B, H, Lq, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lk, 64)
+    shape = {"full": (B, H, Lq, Lk), "b1qk": (B, 1, Lq, Lk), "qk": (Lq, Lk), "b11k": (B, 1, 1, Lk), "k": (Lk,),
+             "bh1k": (B, H, 1, Lk), "1hq1": (1, H, Lq, 1)}[mshape]
+    full = np.broadcast_to(np.zeros(shape, np.float32), shape).copy()
+    # block structure: tiles of 32 set to 0, 1, random 0/1, or a non-binary value
+    m4 = full.reshape((1,) * (4 - full.ndim) + full.shape)
+    for qi in range(0, m4.shape[2], 32):
+        for ki in range(0, m4.shape[3], 32):
+            for bb in range(m4.shape[0]):
+                for hh in range(m4.shape[1]):
+                    c = rng.integers(0, 4)
+                    blk = m4[bb, hh, qi:qi + 32, ki:ki + 32]
+                    if c == 1:
+                        blk[...] = 1.0
+                    elif c == 2:
+                        blk[...] = (rng.random(blk.shape) < 0.5)
+                    elif c == 3:
+                        blk[...] = 0.5
+    got = run_sdpa(ctx, q, k, v, full)
+    ref = orc.sdpa(q, k, v, full, np.float32(8.0))
+    assert_parity(got, ref, "dense mask tiles " + mshape)
+    got_tm = run_sdpa(ctx, q, k, v, full, token_major=True)
+    assert np.array_equal(got, got_tm)
