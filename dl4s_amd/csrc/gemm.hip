@@ -162,31 +162,40 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
     float *C = g.C + (long long)blockIdx.z * g.c_bs;
 
     // loaders: A tile TM x 16 = TM*4 float4: thread -> rows (tid/4 + 64*i), k quad tid%4;
-    //          B tile 16 x TN = 4*TN float4: thread -> row (tid / (TN/4) + (1024/TN)*i), n quad tid % (TN/4)
+    //          B tile 16 x TN = 4*TN float4: thread -> row (tid / (TN/4) + (1024/TN)*i), n quad tid % (TN/4).
+    // Both through buffer loads with the whole byte offset in the (range-checked) vector operand: rows of A past M,
+    // rows of B past K and -- through an offset beyond any descriptor -- columns of B past N read as zeros, so a K step
+    // costs one add per load and no predication.
     constexpr int BQ = TN / 4, BROWS = 256 / BQ;     // float4 per B row, B rows covered per pass
+    constexpr unsigned OUTSIDE = 0x80000000u;        // the host keeps every descriptor below 2^31 bytes
     const int a_row = tid >> 2, a_kq = (tid & 3) * 4;
     const int b_row = tid / BQ, b_nq = (tid % BQ) * 4;
-    const float *ap[MI];
-    bool a_ok[MI];
+    const long long a_rem = ((long long)(g.M - m0 - 1) * g.a_rs + g.K) * 4;
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(A + (long long)m0 * g.a_rs), 0, (int)(a_rem < 0x7fffffffll ? a_rem : 0x7fffffffll), 0x00020000);
+    const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(B + n0), 0, (int)((((long long)g.K - 1) * g.b_rs + (g.N - n0)) * 4), 0x00020000);
+    unsigned a_off[MI], b_off[NI];
 #pragma unroll
-    for (int i = 0; i < MI; ++i) {
-        a_ok[i] = m0 + a_row + 64 * i < g.M;
-        ap[i] = A + (long long)min(m0 + a_row + 64 * i, g.M - 1) * g.a_rs + a_kq;
-    }
-    const bool b_ok = n0 + b_nq < g.N;
-    const float *bp = B + (b_ok ? n0 + b_nq : 0);
-    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < MI; ++i)
+        a_off[i] = (m0 + a_row + 64 * i < g.M) ? (unsigned)((a_row + 64 * i) * (int)g.a_rs + a_kq) * 4u : OUTSIDE;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+        b_off[i] = (n0 + b_nq < g.N) ? (unsigned)((b_row + BROWS * i) * (int)g.b_rs + b_nq) * 4u : OUTSIDE;
+    const bool ragged_k = (g.K % GBK) != 0;
+    const unsigned b_step = (unsigned)GBK * (unsigned)g.b_rs * 4u;
     f32x4 ast[MI], bst[NI];
     auto load = [&](int kt) {
         const int k0 = kt * GBK;
-        const bool kok = k0 + a_kq < g.K;
+        // the last K step of a ragged K: quads at or past K lie inside the next row of A, so they are sent outside
+        const bool a_past = ragged_k && (k0 + a_kq >= g.K);
 #pragma unroll
-        for (int i = 0; i < MI; ++i) ast[i] = (a_ok[i] && kok) ? *reinterpret_cast<const f32x4 *>(ap[i] + k0) : zero;
+        for (int i = 0; i < MI; ++i)
+            ast[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                   arsrc, (int)(a_past ? OUTSIDE : a_off[i] + (unsigned)k0 * 4u), 0, 0));
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int kr = k0 + b_row + BROWS * i;
-            bst[i] = (b_ok && kr < g.K) ? *reinterpret_cast<const f32x4 *>(bp + (long long)kr * g.b_rs) : zero;
-        }
+        for (int i = 0; i < NI; ++i)
+            bst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(brsrc, (int)(b_off[i] + kt * b_step), 0, 0));
     };
     auto store = [&](int buf) {
 #pragma unroll
@@ -272,8 +281,9 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.bias = bias; g.residual = residual; g.act = act;
     const bool epi = bias || residual || act;
     const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    // the fast kernels address A within a tile's rows and B as a whole through 32-bit byte offsets below 2^31
     const bool fast = !ta && !tb && K % 4 == 0 && N % 4 == 0 && K > 0 && aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 &&
-                      rbs % 4 == 0;
+                      rbs % 4 == 0 && K < (1ll << 21) && K * N * 4 < (1ll << 31);
     long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
     // small products: 64x64 tiles, so that there are at least about two workgroups per CU
     const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;

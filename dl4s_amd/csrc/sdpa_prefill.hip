@@ -179,23 +179,24 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     }
 
     // global -> LDS staging: thread covers rows (i*16 + tid/16), 4 floats at column (tid%16)*4.  K and V are read with
-    // buffer loads: the per-thread byte offset is fixed, the tile offset is a scalar, and rows at or beyond Lk fall
-    // outside the descriptor's range and read as zeros (their scores are then set to -inf by the key bound below).
+    // buffer loads whose whole byte offset is in the vector operand (the only part the hardware range-checks): rows at
+    // or beyond Lk fall outside the descriptor's range and read as zeros (their scores are then set to -inf by the key
+    // bound below), so the loop needs neither address arithmetic beyond one add nor clamps.
     const int ld_row = tid >> 4;
     const int ld_col = (tid & 15) * 4;
     const int kv_bytes = (int)(((long long)(Lk - 1) * rs + HD) * 4);   // extent of this pair's rows; the host keeps it below 2^31
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
-    const int ld_off0 = (ld_row * rs + ld_col) * 4;
-    const int ld_off1 = ld_off0 + 16 * rs * 4;
-    const int tile_bytes = BN * rs * 4;
+    const unsigned ld_off0 = (unsigned)(ld_row * rs + ld_col) * 4u;   // unsigned: the last tile may step past 2^31
+    const unsigned ld_off1 = ld_off0 + 16u * rs * 4u;
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
     f32x4 kst[2], vst[2];
     auto load_tile = [&](int t) {
-        const int so = t * tile_bytes;
-        kst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, ld_off0, so, 0));
-        vst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, ld_off0, so, 0));
-        kst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, ld_off1, so, 0));
-        vst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, ld_off1, so, 0));
+        const int o0 = (int)(ld_off0 + t * tile_bytes), o1 = (int)(ld_off1 + t * tile_bytes);
+        kst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o0, 0, 0));
+        vst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o0, 0, 0));
+        kst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o1, 0, 0));
+        vst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o1, 0, 0));
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
