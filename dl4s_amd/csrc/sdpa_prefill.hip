@@ -76,6 +76,104 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
 
+// One 32-key tile for one wavefront (32 queries): S^T = K.Q^T, mask, online softmax update, O^T += V^T.P^T.
+// Kb / Vb point at the lane's K and V fragment bases of the tile in LDS; mrow is the lane's row of a dense mask
+// (element stride msk along keys), cls the tile's mask class.
+template <int KIND>
+__device__ __forceinline__ void attend_tile(const float *Kb, const float *Vb, const float (&qr)[32], f32x16 &o0, f32x16 &o1,
+                                            float &m_run, float &m_use, float &l_run, const int k0, const int q0, const int qi,
+                                            const int half, const int Lk, const int len, const float *mrow, const long long msk,
+                                            const int cls) {
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+    // ---- S^T = K . Q^T for one 32-key tile
+    // (one dependent accumulation chain keeps the matrix pipe full; the first MFMA takes a literal zero)
+    f32x16 s0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
+        if (j == 0) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[0], zero, 0, 0, 0);
+        } else {
+            s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
+        }
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s0, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, qr[4 * j + 2], s0, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s0, 0, 0, 0);
+    }
+
+    // ---- mask, in registers.  Accumulator register r is key k0 + 8(r/4) + 4*half + r%4.
+    if (DENSE) {
+        if (cls == 1) {           // every element of the tile is 1: the penalty is a constant
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+        } else if (cls == 2) {    // mixed tile: read the mask values (class 0 = all zeros needs nothing)
+        #pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const int kc = kg < Lk ? kg : Lk - 1;
+                s0[r] = __fsub_rn(s0[r], __fmul_rn(__fmul_rn(mrow[kc * msk], 1e9f), LOG2E));
+            }
+        }
+    } else if ((CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len))) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+            bool blocked = false;
+            if (CAUSAL) blocked = blocked || (kg > qi);
+            if (LENS) blocked = blocked || (kg >= len);
+            if (blocked) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+        }
+    }
+    if (k0 + BN > Lk) {           // keys past the end of the tensor take no part
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (kg >= Lk) s0[r] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax: lane (query ln) sees 16 of the 32 keys, lane ^ 32 the other 16.
+    // Vector-ALU instructions do not overlap the matrix pipe on a SIMD (measured: their cycles add to the MFMA
+    // cycles), so the reduction is kept to about four instructions per score: max3, one fma + exp2, one add.
+    // The reference maximum m_run only moves -- and the accumulators are only rescaled -- when a tile's maximum
+    // would give a weight above 2^8; any per-row factor 2^(max - m_run) left in the weights cancels in the
+    // final division by the row sum.
+    float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
+#pragma unroll
+    for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
+    tmax = fmaxf(tmax, s0[15]);
+    tmax = fmaxf(tmax, xor32(tmax));
+    const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+    if (__any(upd)) {
+        const float m_new = fmaxf(m_run, tmax);
+        // lanes whose maximum did not move keep factor 1 (also when it is still -inf: -inf - -inf would be NaN)
+        const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
+        m_run = m_new;
+        m_use = (m_new == -INFINITY) ? 0.f : m_new;      // a row of -inf so far: weights 0, not NaN
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { o0[i] *= alpha; o1[i] *= alpha; }
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        s0[r] = fast_exp2(s0[r] - m_use);
+        psum += s0[r];
+    }
+    l_run += psum;
+
+    // ---- O^T += V^T . P^T.  Row = key (+ 4*half, folded into v_lds), columns 2*ln, 2*ln+1.
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + (8 * (r >> 2) + (r & 3)) * LSTR);
+        o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s0[r], o0, 0, 0, 0);
+        o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s0[r], o1, 0, 0, 0);
+    }
+}
+
 template <int KIND>
 __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__restrict__ q,
                                                                 const float *__restrict__ k,
@@ -223,6 +321,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     const int k_lds = ln * LSTR + half * 32;        // K fragment base: row ln, columns half*32..
     const int v_lds = (4 * half) * LSTR + 2 * ln;   // V fragment base: row 4*half (+ const), columns 2*ln, 2*ln+1
 
+    const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;   // wavefronts past Lq store nothing
 
@@ -235,94 +334,8 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk];
 
         if (k0 < wkend) {
-            // ---- S^T = K . Q^T for one 32-key tile
-            // (one dependent accumulation chain keeps the matrix pipe full; the first MFMA takes a literal zero)
-            f32x16 s0;
-            const float *Kb = Ks + buf * TILE_FLOATS + k_lds;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
-                if (j == 0) {
-                    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                    s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[0], zero, 0, 0, 0);
-                } else {
-                    s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
-                }
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s0, 0, 0, 0);
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, qr[4 * j + 2], s0, 0, 0, 0);
-                s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s0, 0, 0, 0);
-            }
-
-            // ---- mask, in registers.  Accumulator register r is key k0 + 8(r/4) + 4*half + r%4.
-            if (DENSE) {
-                if (cls == 1) {           // every element of the tile is 1: the penalty is a constant
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
-                } else if (cls == 2) {    // mixed tile: read the mask values (class 0 = all zeros needs nothing)
-                    const float *mrow = mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                        const int kc = kg < Lk ? kg : Lk - 1;
-                        s0[r] = __fsub_rn(s0[r], __fmul_rn(__fmul_rn(mrow[kc * mask.sk], 1e9f), LOG2E));
-                    }
-                }
-            } else if ((CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len))) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    bool blocked = false;
-                    if (CAUSAL) blocked = blocked || (kg > qi);
-                    if (LENS) blocked = blocked || (kg >= len);
-                    if (blocked) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
-                }
-            }
-            if (k0 + BN > Lk) {           // keys past the end of the tensor take no part
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    if (kg >= Lk) s0[r] = -INFINITY;
-                }
-            }
-
-            // ---- online softmax: lane (query ln) sees 16 of the 32 keys, lane ^ 32 the other 16.
-            // Vector-ALU instructions do not overlap the matrix pipe on a SIMD (measured: their cycles add to the MFMA
-            // cycles), so the reduction is kept to about four instructions per score: max3, one fma + exp2, one add.
-            // The reference maximum m_run only moves -- and the accumulators are only rescaled -- when a tile's maximum
-            // would give a weight above 2^8; any per-row factor 2^(max - m_run) left in the weights cancels in the
-            // final division by the row sum.
-            float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
-#pragma unroll
-            for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
-            tmax = fmaxf(tmax, s0[15]);
-            tmax = fmaxf(tmax, xor32(tmax));
-            const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
-            if (__any(upd)) {
-                const float m_new = fmaxf(m_run, tmax);
-                // lanes whose maximum did not move keep factor 1 (also when it is still -inf: -inf - -inf would be NaN)
-                const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
-                m_run = m_new;
-                m_use = (m_new == -INFINITY) ? 0.f : m_new;      // a row of -inf so far: weights 0, not NaN
-                l_run *= alpha;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) { o0[i] *= alpha; o1[i] *= alpha; }
-            }
-            float psum = 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                s0[r] = fast_exp2(s0[r] - m_use);
-                psum += s0[r];
-            }
-            l_run += psum;
-
-            // ---- O^T += V^T . P^T.  Row = key (+ 4*half, folded into v_lds), columns 2*ln, 2*ln+1.
-            const float *Vb = Vs + buf * TILE_FLOATS + v_lds;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const f32x2 vv = *reinterpret_cast<const f32x2 *>(Vb + (8 * (r >> 2) + (r & 3)) * LSTR);
-                o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.x, s0[r], o0, 0, 0, 0);
-                o1 = __builtin_amdgcn_mfma_f32_32x32x2f32(vv.y, s0[r], o1, 0, 0, 0);
-            }
+            attend_tile<KIND>(Ks + buf * TILE_FLOATS + k_lds, Vs + buf * TILE_FLOATS + v_lds, qr, o0, o1, m_run, m_use, l_run, k0, q0,
+                              qi, half, Lk, len, mrow, mask.sk, cls);
         }
 
         if (more) store_tile(buf ^ 1);
@@ -343,6 +356,175 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
             c.z = o0[4 * g + 3] * inv; c.w = o1[4 * g + 3] * inv;
             *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
             *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
+        }
+    }
+}
+
+// Variant for launches with too few wavefronts to fill the GPU (fewer 32-query wavefronts than about two per SIMD):
+// one workgroup = 32 queries of one (batch, head), and its 4 wavefronts share the keys, wavefront w taking the 32-key
+// tiles w, w + 4, w + 8, ... through a wavefront-private LDS tile (no workgroup barrier in the loop).  At the end the
+// four partial results (reference maximum, row sum, O^T) are merged through LDS and wavefront 0 stores the rows.
+// Same tile arithmetic as the kernel above; the summation order over keys differs, so results agree with it within
+// rounding, not bit for bit.  Which of the two kernels runs depends on the extents only, never on the mask.
+constexpr int SPLIT_WAVES = 4;
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
+                                                                      const float *__restrict__ v, float *__restrict__ out,
+                                                                      int H, int Lq, int Lk, float rT, MaskArgs mask,
+                                                                      int strict, int nqb, int total_blocks, int token_major) {
+    extern __shared__ __align__(16) float lds[];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int half = lane >> 5;
+    const int ln = lane & 31;
+    float *Ks = lds + wave * 2 * TILE_FLOATS;   // this wavefront's K tile, then its V tile
+    float *Vs = Ks + TILE_FLOATS;
+
+    const int chunk = (total_blocks + 7) / 8;   // one contiguous run of the (batch*head)-major order per XCD
+    const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
+    if (w >= total_blocks) return;
+    const int bh = w / nqb;
+    const int qb = nqb - 1 - w % nqb;
+    const int b = bh / H;
+    const int hh = bh % H;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int q0 = qb * 32;
+    const int qi = q0 + ln;
+    const int qic = qi < Lq ? qi : Lq - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * HD : HD;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+
+    int kend = Lk;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) kend = min(kend, q0 + 32);
+        if (LENS) kend = min(kend, len);
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    float qr[32];
+    {
+        const float *qp = q + q_base + (long long)qic * rs + half * 32;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+            qr[4 * j + 0] = (t.x * rT) * LOG2E;
+            qr[4 * j + 1] = (t.y * rT) * LOG2E;
+            qr[4 * j + 2] = (t.z * rT) * LOG2E;
+            qr[4 * j + 3] = (t.w * rT) * LOG2E;
+        }
+    }
+
+    // the wavefront stages its own tiles: lane covers rows (i*4 + lane/16), 4 floats at column (lane%16)*4
+    const int ld_row = lane >> 4;
+    const int ld_col = (lane & 15) * 4;
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + HD) * 4);
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
+    const unsigned ld_off = (unsigned)(ld_row * rs + ld_col) * 4u;
+    const unsigned row4_bytes = 4u * rs * 4u;
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[8], vst[8];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int o = (int)(ld_off + t * tile_bytes + i * row4_bytes);
+            kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o, 0, 0));
+            vst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o, 0, 0));
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int off = (i * 4 + ld_row) * LSTR + ld_col;
+            *reinterpret_cast<f32x4 *>(Ks + off) = kst[i];
+            *reinterpret_cast<f32x4 *>(Vs + off) = vst[i];
+        }
+    };
+
+    f32x16 o0, o1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { o0[i] = 0.f; o1[i] = 0.f; }
+    float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
+
+    const int k_lds = ln * LSTR + half * 32;
+    const int v_lds = (4 * half) * LSTR + 2 * ln;
+    const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
+
+    // LDS operations of one wavefront execute in order, so the tile can be overwritten right after the reads of the
+    // previous one were issued: no barrier, the prefetch of the next tile sits in registers meanwhile.
+    if (wave < ntiles) {
+        load_tile(wave);
+        store_tile();
+    }
+    for (int t = wave; t < ntiles; t += SPLIT_WAVES) {
+        const bool more = (t + SPLIT_WAVES < ntiles);
+        if (more) load_tile(t + SPLIT_WAVES);
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk];
+        attend_tile<KIND>(Ks + k_lds, Vs + v_lds, qr, o0, o1, m_run, m_use, l_run, t * BN, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+        if (more) store_tile();
+    }
+
+    // ---- merge the four partial results.  Wavefront w > 0 leaves (m_run, row sum, O^T) in its own LDS region (the tiles
+    // are dead by now); wavefront 0 folds them in.  A partial result with m_run = -inf has seen no finite score: its
+    // sums are zeros (or NaN, which must survive), so it is added with factor 1.
+    float l_tot = l_run + xor32(l_run);
+    __syncthreads();   // every wavefront is done with its tile region
+    float *mine = lds + wave * 2 * TILE_FLOATS;   // [34][64]: rows 0..31 = o0/o1 registers, row 32 = m_run, row 33 = l_tot
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            mine[(2 * r) * 64 + lane] = o0[r];
+            mine[(2 * r + 1) * 64 + lane] = o1[r];
+        }
+        mine[32 * 64 + lane] = m_run;
+        mine[33 * 64 + lane] = l_tot;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float m_all = m_run;
+#pragma unroll
+        for (int x = 1; x < SPLIT_WAVES; ++x) m_all = fmaxf(m_all, lds[x * 2 * TILE_FLOATS + 32 * 64 + lane]);
+        const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
+        const float f0 = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - m_ref);
+        l_tot *= f0;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { o0[r] *= f0; o1[r] *= f0; }
+#pragma unroll
+        for (int x = 1; x < SPLIT_WAVES; ++x) {
+            const float *other = lds + x * 2 * TILE_FLOATS;
+            const float mx = other[32 * 64 + lane];
+            const float fx = (mx == -INFINITY) ? 1.0f : fast_exp2(mx - m_ref);
+            l_tot += other[33 * 64 + lane] * fx;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                o0[r] += other[(2 * r) * 64 + lane] * fx;
+                o1[r] += other[(2 * r + 1) * 64 + lane] * fx;
+            }
+        }
+        const float inv = 1.0f / l_tot;
+        if (qi < Lq) {
+            float *op = out + q_base + (long long)qi * rs + 8 * half;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4 a, c;
+                a.x = o0[4 * g + 0] * inv; a.y = o1[4 * g + 0] * inv;
+                a.z = o0[4 * g + 1] * inv; a.w = o1[4 * g + 1] * inv;
+                c.x = o0[4 * g + 2] * inv; c.y = o1[4 * g + 2] * inv;
+                c.z = o0[4 * g + 3] * inv; c.w = o1[4 * g + 3] * inv;
+                *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
+                *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
+            }
         }
     }
 }
@@ -413,7 +595,25 @@ __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__
 
 template <int KIND>
 int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq,
-               int Lk, float rT, const MaskArgs &m, int strict, int token_major) {
+               int Lk, float rT, const MaskArgs &m, int strict, int token_major, int no_split) {
+    // Too few 32-query wavefronts to give every SIMD about two: split the keys of each query block over 4 wavefronts.
+    // The choice depends on the extents only, so every mask kind of one problem runs the same kernel.
+    const long long waves = (long long)B * H * ((Lq + 31) / 32);
+    if (!no_split && waves < 8ll * ctx->cu_count && Lk >= 2 * BN) {
+        const int nqb32 = (Lq + 31) / 32;
+        const long long total32 = (long long)nqb32 * B * H;
+        DL4S_REQUIRE(total32 < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total32);
+        const size_t lds_split = (size_t)SPLIT_WAVES * 2 * TILE_FLOATS * sizeof(float);
+        static bool split_attr_set[8] = {false};
+        if (!split_attr_set[KIND]) {
+            DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_prefill_split_f32_d64<KIND>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_split));
+            split_attr_set[KIND] = true;
+        }
+        hipLaunchKernelGGL(sdpa_prefill_split_f32_d64<KIND>, dim3((unsigned)((total32 + 7) / 8 * 8)), dim3(256), lds_split,
+                           ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major);
+        return dl4s::launch_status("sdpa_prefill_split_f32_d64");
+    }
     const int nqb = (Lq + BM - 1) / BM;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     // longest-first order for causal masks.  Measured on B8 H16 L2048 causal with the order applied to groups of
@@ -498,18 +698,19 @@ extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     }
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
-    DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR)) == 0, DL4S_HIP_EINVALID_ARG,
+    const int no_split = (flags & DL4S_SDPA_NO_KEY_SPLIT) ? 1 : 0;
+    DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR | DL4S_SDPA_NO_KEY_SPLIT)) == 0, DL4S_HIP_EINVALID_ARG,
                  "sdpa: unknown flag bits 0x%x", flags);
     if (dk == HD && dv == HD) {
         // the MFMA kernel addresses one (batch, head) pair's K/V rows through a 32-bit byte offset
         DL4S_REQUIRE(Lk * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
                      "sdpa: the K/V rows of one (batch, head) pair span more than 2 GiB");
         switch (m.kind) {
-            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
-            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
-            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
-            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
-            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major);
+            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
+            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
+            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
+            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
+            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
         }
     }
     DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs head dims of 64");

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libdl4s_hip.so")
 MASK_NONE, MASK_DENSE, MASK_CAUSAL, MASK_KEY_LENGTHS, MASK_CAUSAL_OR_KEY_LENGTHS = range(5)
 SDPA_STRICT = 1
 SDPA_TOKEN_MAJOR = 2
+SDPA_NO_KEY_SPLIT = 4
 ACT_NONE, ACT_GELU = 0, 1
 OP_ADD, OP_SUB, OP_MUL, OP_DIV = range(4)
 

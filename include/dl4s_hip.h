@@ -104,6 +104,11 @@ typedef struct dl4s_mask_desc {
                                     MultiHeadAttention produce, NN/Models/Transformer/MultiHeadAttention.swift:105-107
                                     before its permutes :109-111, and the layout its output permute :117 produces), so a
                                     caller can drop the four permuteAxes copies.  Head dims of 64 only. */
+#define DL4S_SDPA_NO_KEY_SPLIT 4u /* small launches (fewer 32-query blocks than about two per SIMD) normally split each
+                                     block's keys over the 4 wavefronts of a workgroup and merge the partial softmax
+                                     results; this flag keeps the one-wavefront-per-block kernel.  The two agree within
+                                     rounding (different summation order over keys), each well inside the parity
+                                     tolerance. */
 
 /* out = softmax((q * inv_temperature) . k^T - mask * 1e9, axis = keys) . v
  * NN/Models/Transformer/ScaledDotProductAttention.swift:43-64.  q [B,H,Lq,dk], k [B,H,Lk,dk],

@@ -20,7 +20,7 @@ def ctx():
     c.close()
 
 
-def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temperature=None, token_major=False):
+def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temperature=None, token_major=False, no_split=None):
     from dl4s_amd import lib
     B, H, Lq, dk = q.shape
     Lk, dv = v.shape[2], v.shape[3]
@@ -42,7 +42,9 @@ def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temper
         desc = ctx.mask_desc(kind, lengths=ld)
     elif kind == lib.MASK_CAUSAL:
         desc = ctx.mask_desc(lib.MASK_CAUSAL)
-    flags = (lib.SDPA_STRICT if strict else 0) | (lib.SDPA_TOKEN_MAJOR if token_major else 0)
+    if no_split is None:
+        no_split = NO_SPLIT_DEFAULT[0]
+    flags = (lib.SDPA_STRICT if strict else 0) | (lib.SDPA_TOKEN_MAJOR if token_major else 0) | (lib.SDPA_NO_KEY_SPLIT if no_split else 0)
     ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], bufs[3], B, H, Lq, Lk, dk, dv, rT, desc, flags)
     out = bufs[3].numpy()
     if token_major:
@@ -50,6 +52,17 @@ def run_sdpa(ctx, q, k, v, mask=None, kind=None, lens=None, strict=False, temper
     for b in bufs:
         b.release()
     return out
+
+
+# Small launches run the key-split kernel unless DL4S_SDPA_NO_KEY_SPLIT is set; the module's tests run once per variant.
+NO_SPLIT_DEFAULT = [False]
+
+
+@pytest.fixture(autouse=True, params=["key_split_auto", "no_key_split"])
+def kernel_variant(request):
+    NO_SPLIT_DEFAULT[0] = request.param == "no_key_split"
+    yield
+    NO_SPLIT_DEFAULT[0] = False
 
 
 def rand(rng, *shape, scale=1.0):
