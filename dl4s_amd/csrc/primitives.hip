@@ -14,7 +14,7 @@ inline unsigned grid_for(long long n, int per_thread = 4) {
     return (unsigned)b;
 }
 
-enum { U_NEG, U_EXP, U_SQRT, U_RELU, U_TANH };
+enum { U_NEG, U_EXP, U_SQRT, U_RELU, U_TANH, U_LOG, U_SIN, U_COS };
 
 // IEEE-exact fp32 square root (the device sqrtf is 1 ulp): the correctly rounded fp64 root rounds to the
 // correctly rounded fp32 root because 53 >= 2*24 + 2.
@@ -29,6 +29,9 @@ __global__ void unary_f32(const float *__restrict__ x, float *__restrict__ y, lo
         else if (OP == U_EXP) r = expf(v);
         else if (OP == U_SQRT) r = sqrt_rn(v);
         else if (OP == U_RELU) r = v > 0.f ? v : 0.f;
+        else if (OP == U_LOG) r = logf(v);
+        else if (OP == U_SIN) r = sinf(v);
+        else if (OP == U_COS) r = cosf(v);
         else r = tanhf(v);
         y[i] = r;
     }
@@ -267,6 +270,80 @@ int launch_binary(dl4s_hip_ctx *ctx, const float *a, const float *b, float *y, i
     hipLaunchKernelGGL(binary_f32<OP>, dim3(grid_for(n)), dim3(TPB), 0, ctx->stream, a, b, y, (long long)n);
     return dl4s::launch_status(name);
 }
+// First index of the largest value, scanning like `if v > maxV` from (-inf, index 0): NaN is never selected, ties keep
+// the earliest index (Engine/CPU/Numeric/CPUFloat.swift:294-318, generic branch).  One workgroup; out = {value, index}.
+__global__ __launch_bounds__(1024) void argmax_f32(const float *__restrict__ x, long long n, float *out_value, long long *out_index) {
+    __shared__ float sv[1024];
+    __shared__ long long si[1024];
+    float bv = -INFINITY;
+    long long bi = 0;
+    for (long long i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = x[i];
+        if (v > bv) { bv = v; bi = i; }     // ascending i per thread: the first of equal values stays
+    }
+    sv[threadIdx.x] = bv;
+    si[threadIdx.x] = bi;
+    __syncthreads();
+    for (int o = blockDim.x / 2; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) {
+            const float v = sv[threadIdx.x + o];
+            const long long i = si[threadIdx.x + o];
+            // a candidate wins on a larger value, or on an equal value found earlier -- but never from the initial
+            // state (-inf, 0) of a thread that selected nothing
+            if (v > sv[threadIdx.x] || (v == sv[threadIdx.x] && v != -INFINITY && i < si[threadIdx.x])) {
+                sv[threadIdx.x] = v;
+                si[threadIdx.x] = i;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) { *out_value = sv[0]; *out_index = si[0]; }
+}
+
+// Embedding lookup with the scale and positional term of Transformer.prepareInputs folded in:
+// out[t][:] = (token[t] == ignore ? 0 : table[token[t]][:]) * scale + positions[t % L][:]
+__global__ void embed_positions_f32(const float *__restrict__ table, const int *__restrict__ tokens, const float *__restrict__ pos,
+                                    float *__restrict__ out, long long ntok, long long L, long long D, int ignore, float scale,
+                                    int has_scale) {
+    const long long n = ntok * D;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        const long long t = i / D, c = i % D;
+        const int tok = tokens[t];
+        float v = tok == ignore ? 0.0f : table[(long long)tok * D + c];
+        if (has_scale) v = __fmul_rn(v, scale);
+        if (pos) v = __fadd_rn(v, pos[(t % L) * D + c]);
+        out[i] = v;
+    }
+}
+
+// logSoftmax over the last axis, one workgroup per row: x - max, exp, sum, log, subtract
+// (Tensor/Operators/Unary.swift:198-204).  The row sum is taken in index order by one thread per 256-element
+// stripe and then across stripes, within the parity tolerance of the reference's sequential sum.
+__global__ __launch_bounds__(256) void log_softmax_f32(const float *__restrict__ x, float *__restrict__ y, long long n) {
+    __shared__ float red[256];
+    const float *xr = x + (long long)blockIdx.x * n;
+    float *yr = y + (long long)blockIdx.x * n;
+    float mx = -INFINITY;
+    for (long long i = threadIdx.x; i < n; i += 256) { const float v = xr[i]; if (v > mx) mx = v; }
+    red[threadIdx.x] = mx;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) red[threadIdx.x] = red[threadIdx.x + o] > red[threadIdx.x] ? red[threadIdx.x + o] : red[threadIdx.x];
+        __syncthreads();
+    }
+    mx = red[0];
+    __syncthreads();
+    float sum = 0.f;
+    for (long long i = threadIdx.x; i < n; i += 256) sum += expf(__fadd_rn(xr[i], -mx));
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    const float lse = logf(red[0]);
+    for (long long i = threadIdx.x; i < n; i += 256) yr[i] = __fsub_rn(__fadd_rn(xr[i], -mx), lse);
+}
 
 }  // namespace
 
@@ -290,6 +367,9 @@ int dl4s_hip_exp_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { ret
 int dl4s_hip_sqrt_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_SQRT>(c, x, y, n, "sqrt"); }
 int dl4s_hip_relu_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_RELU>(c, x, y, n, "relu"); }
 int dl4s_hip_tanh_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_TANH>(c, x, y, n, "tanh"); }
+int dl4s_hip_log_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_LOG>(c, x, y, n, "log"); }
+int dl4s_hip_sin_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_SIN>(c, x, y, n, "sin"); }
+int dl4s_hip_cos_f32(dl4s_hip_ctx *c, const float *x, float *y, int64_t n) { return launch_unary<U_COS>(c, x, y, n, "cos"); }
 
 int dl4s_hip_broadcast_f32(dl4s_hip_ctx *ctx, int op, const float *lhs, const int64_t *lhs_shape, int lhs_dim,
                            const float *rhs, const int64_t *rhs_shape, int rhs_dim, float *result) {
@@ -432,6 +512,74 @@ int dl4s_hip_stack_f32(dl4s_hip_ctx *ctx, const float *const *buffers, int64_t n
         DL4S_HIP_TRY(hipMemcpyAsync(result + i * count, buffers[i], (size_t)count * sizeof(float), hipMemcpyDeviceToDevice, ctx->stream));
     }
     return DL4S_HIP_OK;
+}
+
+int dl4s_hip_stack_axis_f32(dl4s_hip_ctx *ctx, const float *const *buffers, const int64_t *chunks, int64_t n, int64_t outer,
+                            float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(n >= 0 && outer >= 0, DL4S_HIP_EINVALID_ARG, "stack: negative extent");
+    if (n == 0 || outer == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(buffers && chunks && result, DL4S_HIP_EINVALID_ARG, "stack: NULL pointer");
+    int64_t total = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        DL4S_REQUIRE(chunks[i] >= 0, DL4S_HIP_EINVALID_ARG, "stack: negative extent");
+        total += chunks[i];
+    }
+    int64_t at = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        if (chunks[i] == 0) continue;
+        DL4S_REQUIRE(buffers[i], DL4S_HIP_EINVALID_ARG, "stack: buffer %lld is NULL", (long long)i);
+        DL4S_HIP_TRY(hipMemcpy2DAsync(result + at, (size_t)total * sizeof(float), buffers[i], (size_t)chunks[i] * sizeof(float),
+                                      (size_t)chunks[i] * sizeof(float), (size_t)outer, hipMemcpyDeviceToDevice, ctx->stream));
+        at += chunks[i];
+    }
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_argmax_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, int64_t *out_index, float *out_value) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(count >= 0 && out_index && out_value, DL4S_HIP_EINVALID_ARG, "argmax: bad arguments");
+    *out_index = 0;
+    *out_value = -INFINITY;            // the reference's result for an empty buffer
+    if (count == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(values, DL4S_HIP_EINVALID_ARG, "argmax: NULL pointer");
+    int rc = dl4s::ensure_scratch(ctx, 16);
+    if (rc) return rc;
+    float *dv = reinterpret_cast<float *>(ctx->scratch);
+    long long *di = reinterpret_cast<long long *>(reinterpret_cast<char *>(ctx->scratch) + 8);
+    hipLaunchKernelGGL(argmax_f32, dim3(1), dim3(1024), 0, ctx->stream, values, (long long)count, dv, di);
+    rc = dl4s::launch_status("argmax");
+    if (rc) return rc;
+    struct { float v; float pad; long long i; } host;
+    DL4S_HIP_TRY(hipMemcpyAsync(&host, ctx->scratch, 16, hipMemcpyDeviceToHost, ctx->stream));
+    DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    *out_index = host.i;
+    *out_value = host.v;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_embed_positions_f32(dl4s_hip_ctx *ctx, const float *table, int64_t vocab, int64_t D, const int32_t *tokens,
+                                 int64_t batch, int64_t L, int32_t ignore_index, const float *scale, const float *positions,
+                                 float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(vocab >= 0 && D >= 0 && batch >= 0 && L >= 0, DL4S_HIP_EINVALID_ARG, "embedding: negative extent");
+    const long long n = batch * L * D;
+    if (n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(table && tokens && result, DL4S_HIP_EINVALID_ARG, "embedding: NULL pointer");
+    // token values are not checked on the device: the caller (like the reference's subscript) must keep them in range
+    hipLaunchKernelGGL(embed_positions_f32, dim3(grid_for(n)), dim3(TPB), 0, ctx->stream, table, tokens, positions, result,
+                       (long long)(batch * L), (long long)L, (long long)D, (int)ignore_index, scale ? *scale : 1.0f, scale ? 1 : 0);
+    return dl4s::launch_status("embedding");
+}
+
+int dl4s_hip_log_softmax_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t n, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(rows >= 0 && n >= 0, DL4S_HIP_EINVALID_ARG, "logSoftmax: negative extent");
+    if (rows * n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(x && result, DL4S_HIP_EINVALID_ARG, "logSoftmax: NULL pointer");
+    DL4S_REQUIRE(rows < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "logSoftmax: too many rows");
+    hipLaunchKernelGGL(log_softmax_f32, dim3((unsigned)rows), dim3(256), 0, ctx->stream, x, result, (long long)n);
+    return dl4s::launch_status("logSoftmax");
 }
 
 int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *residual, const float *scale, const float *shift,

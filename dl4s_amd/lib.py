@@ -180,6 +180,28 @@ class Context:
     def sqrt(self, x, y, n): self._un("dl4s_hip_sqrt_f32", x, y, n)
     def relu(self, x, y, n): self._un("dl4s_hip_relu_f32", x, y, n)
     def tanh(self, x, y, n): self._un("dl4s_hip_tanh_f32", x, y, n)
+    def log(self, x, y, n): self._un("dl4s_hip_log_f32", x, y, n)
+    def sin(self, x, y, n): self._un("dl4s_hip_sin_f32", x, y, n)
+    def cos(self, x, y, n): self._un("dl4s_hip_cos_f32", x, y, n)
+
+    def argmax(self, x, count):
+        idx, val = C.c_int64(), C.c_float()
+        _check(self.lib.dl4s_hip_argmax_f32(self.handle, _vp(_ptr(x)), _i64(count), C.byref(idx), C.byref(val)))
+        return idx.value, val.value
+
+    def stack_axis(self, buffers, chunks, outer, y):
+        arr = (_vp * max(1, len(buffers)))(*[_ptr(b) for b in buffers])
+        ch = (C.c_int64 * max(1, len(chunks)))(*chunks)
+        _check(self.lib.dl4s_hip_stack_axis_f32(self.handle, arr, ch, _i64(len(buffers)), _i64(outer), _vp(_ptr(y))))
+
+    def embed_positions(self, table, vocab, D, tokens, batch, L, ignore_index, scale, positions, y):
+        sc = C.byref(C.c_float(scale)) if scale is not None else None
+        _check(self.lib.dl4s_hip_embed_positions_f32(self.handle, _vp(_ptr(table)), _i64(vocab), _i64(D), _vp(_ptr(tokens)),
+                                                     _i64(batch), _i64(L), C.c_int32(ignore_index), sc,
+                                                     _vp(_ptr(positions)) if positions is not None else None, _vp(_ptr(y))))
+
+    def log_softmax(self, x, rows, n, y):
+        _check(self.lib.dl4s_hip_log_softmax_f32(self.handle, _vp(_ptr(x)), _i64(rows), _i64(n), _vp(_ptr(y))))
 
     def gemm(self, lhs, lshape, rhs, rshape, result, alpha=1.0, beta=0.0, ta=False, tb=False):
         _check(self.lib.dl4s_hip_gemm_f32(self.handle, _vp(_ptr(lhs)), _i64(lshape[0]), _i64(lshape[1]), _vp(_ptr(rhs)),

@@ -178,6 +178,15 @@ int dl4s_hip_exp_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int6
 int dl4s_hip_sqrt_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
 int dl4s_hip_relu_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
 int dl4s_hip_tanh_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+/* :369 log, :393 sin, :399 cos -- the element-wise maps PositionalEncoding (NN/Models/Transformer/
+ * PositionalEncoding.swift:52-69) and logSoftmax (Tensor/Operators/Unary.swift:198-204) add to the list */
+int dl4s_hip_log_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+int dl4s_hip_sin_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+int dl4s_hip_cos_f32(dl4s_hip_ctx *ctx, const float *values, float *result, int64_t count);
+/* :355 argmax(values:count:) -> (index, value): first index of the largest value, NaN never selected, (0, -inf) for an
+ * empty buffer (Engine/CPU/Numeric/CPUFloat.swift:294-318).  Synchronises the stream (the result is a host value), as
+ * Transformer's greedy decoding needs it (Transformer.swift:130). */
+int dl4s_hip_argmax_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, int64_t *out_index, float *out_value);
 /* :478 permuteAxes: source axis i becomes destination axis arrangement[i]
  * (Engine/CPU/CPUEngine.swift:897-935). */
 int dl4s_hip_permute_axes_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim,
@@ -185,6 +194,11 @@ int dl4s_hip_permute_axes_f32(dl4s_hip_ctx *ctx, const float *values, const int6
 /* :536 stack along axis 0 of `n` equally shaped buffers of `count` elements each
  * (Tensor/Operators/Stack.swift:79-98 as used by broadcastMatrixMultiplied). */
 int dl4s_hip_stack_f32(dl4s_hip_ctx *ctx, const float *const *buffers, int64_t n, int64_t count, float *result);
+/* :536 stack along any axis: buffer i is [outer, chunks[i]] (chunks[i] = its extent on the axis times the product of
+ * the trailing extents), result is [outer, sum of chunks] (Tensor/Operators/Stack.swift:79-98; PositionalEncoding
+ * interleaves sin and cos with it, PositionalEncoding.swift:59-65). */
+int dl4s_hip_stack_axis_f32(dl4s_hip_ctx *ctx, const float *const *buffers, const int64_t *chunks, int64_t n, int64_t outer,
+                            float *result);
 
 /* ------------------------------------------------ fused layer tails (next to the path) */
 /* NN/Layer/LayerNorm.swift:62-77 on x [B, rows, D] -> result, statistics over rows*D jointly per b:
@@ -196,6 +210,16 @@ int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *resid
  * (Dense bias, NN/Layer/Dense.swift:64-68). */
 int dl4s_hip_bias_gelu_f32(dl4s_hip_ctx *ctx, const float *x, const float *bias, float *result, int64_t rows,
                            int64_t D);
+/* Embedding lookup (NN/Layer/Embedding.swift:152-165: row token[t] of the table, a row of zeros for ignore_index)
+ * with the rest of Transformer.prepareInputs (Transformer.swift:86-92) folded in when the pointers are given:
+ *   result[b][l][:] = row * (*scale) + positions[l][:]
+ * table [vocab, D], tokens device int32 [batch, L], positions [L, D] or NULL, scale host pointer or NULL.  Each step
+ * is rounded like the separate engine calls.  Token values must lie in [0, vocab) or equal ignore_index. */
+int dl4s_hip_embed_positions_f32(dl4s_hip_ctx *ctx, const float *table, int64_t vocab, int64_t D, const int32_t *tokens,
+                                 int64_t batch, int64_t L, int32_t ignore_index, const float *scale, const float *positions,
+                                 float *result);
+/* logSoftmax over the last axis of x [rows, n] (Tensor/Operators/Unary.swift:198-204): (x - max) - log(sum(exp(x - max))). */
+int dl4s_hip_log_softmax_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t n, float *result);
 /* The Dense layer with its neighbours folded into the product's epilogue:
  *   result = act(x . weights + bias) + residual
  * x [rows, in], weights [in, out], bias [out] or NULL, residual [rows, out] or NULL, result [rows, out].

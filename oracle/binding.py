@@ -151,6 +151,38 @@ def gelu(x):
     return _unary("orc_gelu", x)
 
 
+def log(x):
+    return _unary("orc_log", x)
+
+
+def sin(x):
+    return _unary("orc_sin", x)
+
+
+def cos(x):
+    return _unary("orc_cos", x)
+
+
+def argmax(x):
+    x = _f32(x).reshape(-1)
+    v = C.c_float()
+    f = lib().orc_argmax
+    f.restype = C.c_int64
+    i = f(_p(x), C.c_int64(x.size), C.byref(v))
+    return int(i), float(v.value)
+
+
+def embedding(table, tokens, ignore_index=-1):
+    table = _f32(table)
+    tok = np.ascontiguousarray(tokens, np.int32).reshape(-1)
+    out = np.empty((tok.size, table.shape[1]), np.float32)
+    rc = lib().orc_embedding(_p(table), C.c_int64(table.shape[0]), C.c_int64(table.shape[1]),
+                             tok.ctypes.data_as(C.c_void_p), C.c_int64(tok.size), C.c_int32(ignore_index), _p(out))
+    if rc:
+        raise ValueError("orc_embedding: token out of range")
+    return out
+
+
 def permute(x, arrangement):
     x = _f32(x)
     dshape = [0] * x.ndim

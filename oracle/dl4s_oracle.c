@@ -28,6 +28,14 @@
  *   orc_encoder_block,
  *   orc_decoder_block        torch.nn.functional.multi_head_attention_forward in fp64 for the
  *                            attention core; an independent fp64 numpy model for the whole layer
+ *   orc_log, orc_sin, orc_cos  numpy fp64 log/sin/cos; the reference's log accuracy test
+ *                            Tests/DL4STests/VecTests.swift:242-258 (1e-4)
+ *   orc_argmax               numpy.argmax (first maximum), hand-written NaN / tie / empty vectors
+ *   orc_embedding            direct table indexing, zero rows for the ignore index
+ *   (oracle/transformer.py composes these with the functions above into PositionalEncoding,
+ *   prepareInputs, logSoftmax, the Transformer forward and its greedy decoding; pinned by the
+ *   closed form sin/cos(pos / 10000^(2i/d)), scipy.special.log_softmax, an independent fp64
+ *   numpy model of the whole network and the forward/greedy consistency check)
  * The reference's own tests hold no numeric vectors for softmax, masked attention, MHA,
  * LayerNorm or the transformer blocks (only a loss-convergence test), so beyond the checks
  * above those functions are pinned by mathematics, not by reference fixtures.
@@ -258,6 +266,36 @@ void orc_exp(const float *x, float *out, int64_t n)  { for (int64_t i = 0; i < n
 void orc_tanh(const float *x, float *out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = tanhf(x[i]); }
 void orc_sqrt(const float *x, float *out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = sqrtf(x[i]); }
 /* CPUFloat.swift relu arm: max(x, 0) */
+/* Engine/CPU/Numeric/CPUFloat.swift:471-483 (logf), :521-533 (sinf), :535-547 (cosf), generic branches */
+void orc_log(const float *x, float *out, int64_t n)  { for (int64_t i = 0; i < n; ++i) out[i] = logf(x[i]); }
+void orc_sin(const float *x, float *out, int64_t n)  { for (int64_t i = 0; i < n; ++i) out[i] = sinf(x[i]); }
+void orc_cos(const float *x, float *out, int64_t n)  { for (int64_t i = 0; i < n; ++i) out[i] = cosf(x[i]); }
+
+/* Engine/CPU/Numeric/CPUFloat.swift:294-318, generic branch: scan from (-inf, 0) with `v > maxV` */
+int64_t orc_argmax(const float *x, int64_t n, float *out_value) {
+    int64_t mi = 0;
+    float mv = -INFINITY;
+    for (int64_t i = 0; i < n; ++i) {
+        if (x[i] > mv) { mv = x[i]; mi = i; }
+    }
+    if (out_value) *out_value = mv;
+    return mi;
+}
+
+/* NN/Layer/Embedding.swift:152-165: row tokens[t] of the [vocab, D] table, zeros for ignore_index */
+int orc_embedding(const float *table, int64_t vocab, int64_t D, const int32_t *tokens, int64_t n,
+                  int32_t ignore_index, float *out) {
+    for (int64_t t = 0; t < n; ++t) {
+        if (tokens[t] == ignore_index) {
+            for (int64_t c = 0; c < D; ++c) out[t * D + c] = 0.0f;
+        } else {
+            if (tokens[t] < 0 || tokens[t] >= vocab) return -1;   /* the reference traps on the subscript */
+            memcpy(out + t * D, table + (int64_t)tokens[t] * D, (size_t)D * sizeof(float));
+        }
+    }
+    return 0;
+}
+
 void orc_relu(const float *x, float *out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = x[i] > 0.0f ? x[i] : 0.0f; }
 
 /* Tensor/Operators/Unary.swift:245-247 (gaussianErrorLinear) with sigmoid :184-186:

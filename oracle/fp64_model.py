@@ -72,3 +72,61 @@ def make_params(rng, D, H, dk, dv, F, trivial_affine=False):
     ffn = dict(W1=xavier_uniform(rng, D, F), b1=aff(F, 0.0), W2=xavier_uniform(rng, F, D), b2=aff(D, 0.0),
                ln_scale=aff(D, 1.0), ln_shift=aff(D, 0.0))
     return mha, ffn
+
+
+# ---- the Transformer wrapper, independently of the fp32 oracle (plain numpy, float64)
+def positional_encoding64(max_len, hidden):
+    pos = np.arange(max_len, dtype=np.float64)[:, None]
+    i = np.arange(hidden // 2, dtype=np.float64)[None, :]
+    angle = pos / np.power(10000.0, i / (hidden // 2))
+    out = np.empty((max_len, hidden))
+    out[:, 0::2], out[:, 1::2] = np.sin(angle), np.cos(angle)
+    return out
+
+
+def prepare_inputs64(params, tokens):
+    tokens = np.asarray(tokens)
+    E = f64(params["embedding"])
+    emb = np.where((tokens == -1)[..., None], 0.0, E[np.clip(tokens, 0, E.shape[0] - 1)])
+    return emb * np.sqrt(E.shape[1]) + positional_encoding64(tokens.shape[1], E.shape[1])
+
+
+def _enc_mask(lengths):
+    L = max(lengths)
+    return (np.arange(L)[None, None, None, :] >= np.asarray(lengths)[:, None, None, None]).astype(np.float64)
+
+
+def _dec_mask(lengths):
+    L = max(lengths)
+    i, j = np.indices((L, L))
+    return np.maximum(_enc_mask(lengths), (j > i)[None, None].astype(np.float64))
+
+
+def transformer64(params, enc_tokens, dec_tokens, enc_lengths, dec_lengths, log_probs=True):
+    H, dk, dv = params["heads"], params["dk"], params["dv"]
+    x = prepare_inputs64(params, enc_tokens)
+    for layer in params["encoder"]:
+        x = encoder_block64(x, _enc_mask(enc_lengths), layer["attn"], layer["ffn"], H, dk, dv)
+    y = prepare_inputs64(params, dec_tokens)
+    for layer in params["decoder"]:
+        y = decoder_block64(y, x, _dec_mask(dec_lengths), _enc_mask(enc_lengths), layer["self"], layer["cross"], layer["ffn"], H, dk, dv)
+    logits = y @ f64(params["embedding"]).T
+    if not log_probs:
+        return logits
+    logits = logits + f64(params["output_bias"])
+    m = logits.max(-1, keepdims=True)
+    return logits - m - np.log(np.exp(logits - m).sum(-1, keepdims=True))
+
+
+def make_transformer_params(rng, vocab, D, H, dk, dv, F, n_enc, n_dec):
+    p = {"embedding": (rng.standard_normal((vocab, D)) * (1.0 / np.sqrt(D))).astype(np.float32),
+         "output_bias": (rng.standard_normal(vocab) * 0.1).astype(np.float32), "heads": H, "dk": dk, "dv": dv,
+         "encoder": [], "decoder": []}
+    for _ in range(n_enc):
+        a, f = make_params(rng, D, H, dk, dv, F)
+        p["encoder"].append({"attn": a, "ffn": f})
+    for _ in range(n_dec):
+        a, f = make_params(rng, D, H, dk, dv, F)
+        c, _ = make_params(rng, D, H, dk, dv, F)
+        p["decoder"].append({"self": a, "cross": c, "ffn": f})
+    return p

@@ -382,3 +382,101 @@ def test_oracle_agrees_with_fp64_model_on_one_config3_token_block(orc):
     mask = (np.arange(L)[None, None, None, :] >= 30).astype(np.float32)
     assert np.allclose(orc.encoder_block(x, mask, attn, ffn, H, dk, dk), m64.encoder_block64(x, mask, attn, ffn, H, dk, dk),
                        rtol=1e-4, atol=1e-4)
+
+
+# ------------------------------------------------------------------ the Transformer wrapper (oracle/transformer.py)
+def test_log_sin_cos_against_numpy_fp64(orc):
+    rng = np.random.default_rng(5)
+    x = (rng.random(4096) * 600.0).astype(np.float32)
+    assert np.allclose(orc.sin(x), np.sin(x.astype(np.float64)), atol=2e-6)
+    assert np.allclose(orc.cos(x), np.cos(x.astype(np.float64)), atol=2e-6)
+    p = (rng.random(4096) * 1e4 + 1e-3).astype(np.float32)
+    assert np.allclose(orc.log(p), np.log(p.astype(np.float64)), rtol=1e-6, atol=1e-7)
+    # Tests/DL4STests/VecTests.swift:242-258 checks log against Foundation.log to 1e-4 on 1...16
+    v = np.arange(1, 17, dtype=np.float32)
+    assert np.abs(orc.log(v) - np.log(np.arange(1, 17))).max() < 1e-4
+
+
+def test_argmax_first_maximum_nan_and_empty(orc):
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal(1000).astype(np.float32)
+    assert orc.argmax(x) == (int(np.argmax(x)), float(x.max()))
+    assert orc.argmax(np.array([1, 3, 3, 2], np.float32)) == (1, 3.0)                 # ties: the first
+    assert orc.argmax(np.array([np.nan, -5, np.nan, -7], np.float32)) == (1, -5.0)    # NaN never selected
+    i, v = orc.argmax(np.array([np.nan, np.nan], np.float32))
+    assert i == 0 and v == -np.inf                                                     # nothing selected
+    i, v = orc.argmax(np.zeros(0, np.float32))
+    assert i == 0 and v == -np.inf
+
+
+def test_embedding_is_table_indexing_with_zero_rows_for_ignore(orc):
+    rng = np.random.default_rng(7)
+    E = rng.standard_normal((11, 6)).astype(np.float32)
+    tok = np.array([3, -1, 0, 10, 3], np.int32)
+    out = orc.embedding(E, tok, -1)
+    assert np.array_equal(out[[0, 2, 3, 4]], E[[3, 0, 10, 3]]) and not out[1].any()
+    with pytest.raises(ValueError):
+        orc.embedding(E, np.array([11], np.int32), -1)
+
+
+def test_positional_encoding_closed_form():
+    from oracle import transformer as T, fp64_model as m64
+    pe = T.positional_encoding(50, 16)
+    assert pe.shape == (50, 16) and pe.dtype == np.float32
+    # Attention Is All You Need, 3.5, with sin and cos interleaved and the exponent i / (d/2)
+    pos, i = np.arange(50)[:, None], np.arange(8)[None, :]
+    angle = pos / 10000.0 ** (i / 8.0)
+    assert np.allclose(pe[:, 0::2], np.sin(angle), atol=2e-5) and np.allclose(pe[:, 1::2], np.cos(angle), atol=2e-5)
+    assert np.allclose(pe, m64.positional_encoding64(50, 16), atol=2e-5)
+    assert np.array_equal(pe[0], np.tile([0.0, 1.0], 8).astype(np.float32))           # position 0: sin 0, cos 0
+
+
+def test_log_softmax_against_scipy():
+    import scipy.special
+    from oracle import transformer as T
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((3, 5, 37)) * 4).astype(np.float32)
+    got = T.log_softmax(x)
+    assert np.allclose(got, scipy.special.log_softmax(x.astype(np.float64), axis=-1), atol=2e-6)
+    assert np.allclose(np.exp(got.astype(np.float64)).sum(-1), 1.0, atol=1e-5)
+    assert np.allclose(T.log_softmax(x + np.float32(3.0)), got, atol=2e-6)            # shift invariance
+
+
+def _tiny_transformer(seed=9, vocab=13):
+    from oracle import fp64_model as m64
+    rng = np.random.default_rng(seed)
+    # the hyper-parameters of Tests/DL4STests/TransformerTests.swift:31: hidden 16, heads 4, key/value dim 8, ffn 32
+    return m64.make_transformer_params(rng, vocab, 16, 4, 8, 8, 32, 2, 2), rng
+
+
+def test_transformer_forward_against_independent_fp64_model():
+    from oracle import transformer as T, fp64_model as m64
+    params, rng = _tiny_transformer()
+    enc_len, dec_len = [7, 4, 6], [5, 3, 5]
+    enc = np.full((3, 7), -1, np.int32)
+    dec = np.full((3, 5), -1, np.int32)
+    for b in range(3):
+        enc[b, :enc_len[b]] = rng.integers(0, 13, enc_len[b])
+        dec[b, :dec_len[b]] = rng.integers(0, 13, dec_len[b])
+    got = T.forward(params, enc, dec, enc_len, dec_len)
+    ref = m64.transformer64(params, enc, dec, enc_len, dec_len)
+    assert got.shape == (3, 5, 13)
+    assert np.abs(got - ref).max() < 2e-4
+    assert np.allclose(np.exp(got.astype(np.float64)).sum(-1), 1.0, atol=1e-5)
+
+
+def test_greedy_decode_is_consistent_with_the_forward_pass():
+    """Token t of the greedy output is the argmax of the forward pass's distribution at the last position when the
+    decoder is fed start + tokens[:t] (bias zero: greedy decoding leaves the output bias out, Transformer.swift:127-130)."""
+    from oracle import transformer as T, fp64_model as m64
+    params, rng = _tiny_transformer(seed=10)
+    params["output_bias"] = np.zeros_like(params["output_bias"])
+    src = [int(t) for t in rng.integers(0, 13, 6)]
+    toks, logits = T.greedy_decode(params, src, 1, 2, 6, return_logits=True)
+    assert 1 <= len(toks) <= 6 and (toks[-1] == 2 or len(toks) == 6) and 2 not in toks[:-1]
+    for t, tok in enumerate(toks):
+        prefix = [[1] + toks[:t]]
+        lp = T.forward(params, [src], prefix, [len(src)], [t + 1])
+        assert int(np.argmax(lp[0, -1])) == tok
+        ref = m64.transformer64(params, np.array([src]), np.array(prefix), [len(src)], [t + 1], log_probs=False)
+        assert np.abs(logits[t] - ref[0, -1]).max() < 2e-4
