@@ -167,14 +167,29 @@ struct HIP {
                                             result.values.memory));
         }
         static void stack(const std::vector<ShapedBuffer> &buffers, const ShapedBuffer &result, int axis) {
-            precondition(axis == 0, "stack: only axis 0 is available for HIP");
             std::vector<const float *> ptrs;
-            for (auto &b : buffers) {
-                precondition(b.shape == buffers[0].shape, "stack: buffers must have equal shapes");
-                ptrs.push_back(b.values.memory);
+            for (auto &b : buffers) ptrs.push_back(b.values.memory);
+            bool equal = true;
+            for (auto &b : buffers) equal = equal && b.shape == buffers[0].shape;
+            if (axis == 0 && equal) {
+                check(dl4s_hip_stack_f32(context(), ptrs.data(), (int64_t)ptrs.size(), buffers.empty() ? 0 : buffers[0].count(),
+                                         result.values.memory));
+                return;
             }
-            check(dl4s_hip_stack_f32(context(), ptrs.data(), (int64_t)ptrs.size(), buffers.empty() ? 0 : buffers[0].count(),
-                                     result.values.memory));
+            int64_t outer = 1;
+            for (int i = 0; i < axis; ++i) outer *= result.shape[i];
+            std::vector<int64_t> chunks;
+            for (auto &b : buffers) chunks.push_back(outer == 0 ? 0 : b.count() / outer);
+            check(dl4s_hip_stack_axis_f32(context(), ptrs.data(), chunks.data(), (int64_t)ptrs.size(), outer, result.values.memory));
+        }
+        static void log(const ShapedBuffer &v, const ShapedBuffer &r) { check(dl4s_hip_log_f32(context(), v.values.memory, r.values.memory, v.count())); }
+        static void sin(const ShapedBuffer &v, const ShapedBuffer &r) { check(dl4s_hip_sin_f32(context(), v.values.memory, r.values.memory, v.count())); }
+        static void cos(const ShapedBuffer &v, const ShapedBuffer &r) { check(dl4s_hip_cos_f32(context(), v.values.memory, r.values.memory, v.count())); }
+        static std::pair<int64_t, float> argmax(Buffer values, int64_t count) {
+            int64_t i;
+            float v;
+            check(dl4s_hip_argmax_f32(context(), values.memory, count, &i, &v));
+            return {i, v};
         }
         // Fused entry points of this backend (no counterpart in EngineType).
         // tokenMajor: q, result are [B,Lq,H,d] and k, v [B,Lk,H,d] (the projections before their permutes)
@@ -214,6 +229,16 @@ struct HIP {
             const int64_t B = x.shape[0], D = scale.count();
             check(dl4s_hip_layernorm_f32(context(), x.values.memory, residual ? residual->values.memory : nullptr, scale.values.memory,
                                          shift.values.memory, result.values.memory, B, x.count() / (B * D), D));
+        }
+        // rows of `table` for device int32 tokens [batch, L], optionally * scale + positions[l]
+        static void embedPositions(const ShapedBuffer &table, const int32_t *tokens, int64_t batch, int64_t L, int32_t ignoreIndex,
+                                   const float *scale, const ShapedBuffer *positions, const ShapedBuffer &result) {
+            check(dl4s_hip_embed_positions_f32(context(), table.values.memory, table.shape[0], table.shape[1], tokens, batch, L, ignoreIndex,
+                                               scale, positions ? positions->values.memory : nullptr, result.values.memory));
+        }
+        static void logSoftmax(const ShapedBuffer &x, const ShapedBuffer &result) {
+            const int64_t n = x.shape.back();
+            check(dl4s_hip_log_softmax_f32(context(), x.values.memory, n == 0 ? 0 : x.count() / n, n, result.values.memory));
         }
         static void biasGelu(const ShapedBuffer &x, const ShapedBuffer &bias, const ShapedBuffer &result) {
             const int64_t D = bias.count();
@@ -343,6 +368,21 @@ class Tensor {
     Tensor tanh() const { return unary(Device::Engine::tanh); }        // :79-82
     Tensor sqrt() const { return unary(Device::Engine::sqrt); }
     Tensor rectifiedLinear() const { return unary(Device::Engine::relu); }
+    Tensor log() const { return unary(Device::Engine::log); }          // :60-77
+    Tensor sine() const { return unary(Device::Engine::sin); }         // :207-223
+    Tensor cosine() const { return unary(Device::Engine::cos); }       // :225-241
+    Tensor raised(const Tensor &power) const { return (log() * power).exp(); }                             // Binary.swift:408-410
+    Tensor logSoftmax(int axis = 1) const {                                                                // :198-204
+        if (Device::fused() && axis == dim() - 1) {
+            Tensor res(Device::Memory::allocateBuffer(shape));
+            Device::Engine::logSoftmax(values(), res.values());
+            return res;
+        }
+        Tensor norm = *this - reduceMax({axis}).unsqueezed(axis);
+        Tensor logSumExp = norm.exp().reduceSum({axis}).log().unsqueezed(axis);
+        return norm - logSumExp;
+    }
+    int64_t argmax() const { return Device::Engine::argmax(buffer(), count()).first; }                     // Reduce.swift:128-130
     Tensor sigmoid() const { return Tensor(0.5f) * (*this * Tensor(0.5f)).tanh() + Tensor(0.5f); }        // :184-186
     Tensor gaussianErrorLinear() const { return *this * (*this * Tensor(1.702f)).sigmoid(); }             // :245-247
     Tensor softmax(int axis = 1) const {                                                                   // :190-194
@@ -392,7 +432,26 @@ class Tensor {
         Device::Engine::permuteAxes(values(), res.values(), axes);
         return res;
     }
-    // Tensor(stacking:) along axis 0 (Tensor/Operators/Stack.swift:79-122)
+    // Tensor(stacking:along:) (Tensor/Operators/Stack.swift:79-122)
+    static Tensor stacking(const std::vector<Tensor> &tensors, int axis) {
+        if (axis == 0) return stacking(tensors);
+        precondition(!tensors.empty(), "cannot stack zero tensors");
+        precondition(axis >= 0 && axis < tensors[0].dim(), "Dimensionality of tensors must be in dimensionality range of source tensors");
+        Shape s = tensors[0].shape;
+        std::vector<ShapedBuffer> bufs;
+        int64_t extent = 0;
+        for (auto &t : tensors) {
+            precondition(t.dim() == tensors[0].dim(), "All vector shapes must match except on concatenation axis.");
+            for (int i = 0; i < t.dim(); ++i)
+                precondition(i == axis || t.shape[i] == s[i], "All vector shapes must match except on concatenation axis.");
+            extent += t.shape[axis];
+            bufs.push_back(t.values());
+        }
+        s[axis] = extent;
+        Tensor res(Device::Memory::allocateBuffer(s));
+        Device::Engine::stack(bufs, res.values(), axis);
+        return res;
+    }
     static Tensor stacking(const std::vector<Tensor> &tensors) {
         precondition(!tensors.empty(), "cannot stack zero tensors");
         Shape s = tensors[0].shape;
@@ -504,6 +563,9 @@ inline Tensor operator/(const Tensor &l, float r) { return l / Tensor(r); }
 inline Tensor sqrt(const Tensor &t) { return t.sqrt(); }
 inline Tensor relu(const Tensor &t) { return t.rectifiedLinear(); }
 inline Tensor softmax(const Tensor &t, int axis) { return t.softmax(axis); }
+inline Tensor logSoftmax(const Tensor &t, int axis) { return t.logSoftmax(axis); }
+inline Tensor sin(const Tensor &t) { return t.sine(); }
+inline Tensor cos(const Tensor &t) { return t.cosine(); }
 
 // ------------------------------------------------------------------------- layers
 // NN/Layer/LayerNorm.swift:29-78
@@ -601,29 +663,40 @@ struct MultiHeadAttention {
           qDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})), kDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})),
           vDense(Tensor::repeating(0.f, {hiddenDim_, valueDim_ * heads_})), fc(Tensor::repeating(0.f, {valueDim_ * heads_, hiddenDim_})),
           norm(Shape{hiddenDim_}), dropout(dropoutRate) {}
+    // fused mode, head dims 64: the key / value projections alone, [B,L,H,64], for callers that attend to the same keys
+    // and values repeatedly (the encoder states during greedy decoding)
+    bool canCacheProjections() const { return Device::fused() && keyDim == 64 && valueDim == 64; }
+    std::pair<Tensor, Tensor> projectKeysValues(const Tensor &k, const Tensor &v) const {
+        precondition(canCacheProjections() && k.dim() == 3 && v.dim() == 3 && k.shape[1] == v.shape[1], "Matmul operands must have matching shapes");
+        const int64_t B = k.shape[0], L = k.shape[1];
+        return {k.view({B * L, hiddenDim}).matrixMultiplied(kDense).view({B, L, heads, keyDim}),
+                v.view({B * L, hiddenDim}).matrixMultiplied(vDense).view({B, L, heads, valueDim})};
+    }
+    Tensor attendProjected(const Tensor &q, const Tensor &kp, const Tensor &vp, const Tensor *mask) const {
+        precondition(canCacheProjections() && q.dim() == 3 && kp.dim() == 4 && vp.dim() == 4, "Matmul operands must have matching shapes");
+        const int64_t batchSize = q.shape[0], queryCount = q.shape[1];
+        Tensor qp = q.view({batchSize * queryCount, hiddenDim}).matrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
+        Tensor a(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, heads, valueDim}));
+        ShapedBuffer mb;
+        if (mask) mb = mask->values();
+        Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true);
+        Tensor a2 = a.view({batchSize * queryCount, heads * valueDim});
+        if (!dropout.isActive) {
+            Tensor sum(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, hiddenDim}));
+            const ShapedBuffer rb = q.values();
+            Device::Engine::denseFused(a2.values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, sum.values());
+            return norm.normalize(sum, nullptr);
+        }
+        Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
+        return norm.normalize(out_drop, &q);
+    }
     Tensor operator()(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask) const {
         const int64_t batchSize = q.shape[0], queryCount = q.shape[1], keyCount = k.shape[1], valueCount = v.shape[1];
         const Tensor &res = q;
-        if (Device::fused() && keyDim == 64 && valueDim == 64) {
-            // the projections are read where they lie ([B,L,H,64]) and the attention output is written as
-            // [B,Lq,H,64] = [B,Lq,H*64]: no permuteAxes; the residual rides in the epilogue of the fc product
+        if (canCacheProjections()) {
             precondition(q.dim() == 3 && k.dim() == 3 && v.dim() == 3 && keyCount == valueCount, "Matmul operands must have matching shapes");
-            Tensor qp = q.view({batchSize * queryCount, hiddenDim}).matrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
-            Tensor kp = k.view({batchSize * keyCount, hiddenDim}).matrixMultiplied(kDense).view({batchSize, keyCount, heads, keyDim});
-            Tensor vp = v.view({batchSize * valueCount, hiddenDim}).matrixMultiplied(vDense).view({batchSize, valueCount, heads, valueDim});
-            Tensor a(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, heads, valueDim}));
-            ShapedBuffer mb;
-            if (mask) mb = mask->values();
-            Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true);
-            Tensor a2 = a.view({batchSize * queryCount, heads * valueDim});
-            if (!dropout.isActive) {
-                Tensor sum(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, hiddenDim}));
-                const ShapedBuffer rb = res.values();
-                Device::Engine::denseFused(a2.values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, sum.values());
-                return norm.normalize(sum, nullptr);
-            }
-            Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
-            return norm.normalize(out_drop, &res);
+            auto kv = projectKeysValues(k, v);
+            return attendProjected(q, kv.first, kv.second, mask);
         }
         Tensor q_prep = q.broadcastMatrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
         Tensor k_prep = k.broadcastMatrixMultiplied(kDense).view({batchSize, keyCount, heads, keyDim});
@@ -688,6 +761,13 @@ struct TransformerDecoderBlock {
         Tensor decAttn = selfAttention(decoderInput, decoderInput, decoderInput, &decoderMask);
         Tensor encAttn = encoderAttention(decAttn, encoderOutput, encoderOutput, &encoderMask);
         return pointwiseFeedForward(encAttn);
+    }    // the same block with the encoder-side key / value projections computed once by the caller
+    // (encoderAttention.projectKeysValues(encoderOutput, encoderOutput)): they do not depend on the decoder input
+    Tensor withProjectedEncoder(const Tensor &decoderInput, const Tensor &encKeys, const Tensor &encValues, const Tensor &encoderMask,
+                                const Tensor &decoderMask) const {
+        Tensor decAttn = selfAttention(decoderInput, decoderInput, decoderInput, &decoderMask);
+        Tensor encAttn = encoderAttention.attendProjected(decAttn, encKeys, encValues, &encoderMask);
+        return pointwiseFeedForward(encAttn);
     }
 };
 
@@ -712,5 +792,183 @@ inline Tensor makeDecoderMasks(const std::vector<int64_t> &sequenceLengths) {
     Tensor decoderCausalMask = Tensor::repeating(1.f, {maxLen, maxLen}).bandMatrix(-1, std::nullopt);
     return 1.f - relu(1.f - decoderSeqMask.view({batchSize, 1, 1, maxLen}) - decoderCausalMask);
 }
+
+// ------------------------------------------------------------------------- the model wrapper
+// NN/Layer/Embedding.swift:29-166 (forward only): row `token` of the embedding matrix, a row of zeros for ignoreIndex
+struct Embedding {
+    Tensor embeddingMatrix;   // [inputFeatures, outputSize]
+    int32_t ignoreIndex;
+    Embedding(int64_t inputFeatures, int64_t outputSize, int32_t ignoreIndex_ = -1)
+        : embeddingMatrix(Tensor::repeating(0.f, {inputFeatures, outputSize})), ignoreIndex(ignoreIndex_) {}
+    int64_t outputSize() const { return embeddingMatrix.shape[1]; }
+    // device copy of host tokens (Tensor<Int32, Device> in the reference)
+    static Tensor uploadTokens(const std::vector<int32_t> &tokens) {
+        Tensor t(Device::Memory::allocateBuffer(Shape{(int64_t)tokens.size()}));
+        Device::check(dl4s_hip_assign_h2d(Device::context(), t.buffer().memory, tokens.data(), tokens.size() * sizeof(int32_t)));
+        return t;
+    }
+    Tensor operator()(const std::vector<int32_t> &inputs) const {
+        for (int32_t idx : inputs)
+            precondition(idx == ignoreIndex || (idx >= 0 && idx < embeddingMatrix.shape[0]), "index out of bounds");
+        if (Device::fused()) {
+            Tensor tok = uploadTokens(inputs);
+            Tensor res(Device::Memory::allocateBuffer(Shape{(int64_t)inputs.size(), outputSize()}));
+            Device::Engine::embedPositions(embeddingMatrix.values(), reinterpret_cast<const int32_t *>(tok.buffer().memory), 1,
+                                           (int64_t)inputs.size(), ignoreIndex, nullptr, nullptr, res.values());
+            return res;
+        }
+        std::vector<Tensor> embedded;
+        for (int32_t idx : inputs) {
+            if (idx == ignoreIndex) embedded.push_back(Tensor::repeating(0.f, {1, outputSize()}));
+            else embedded.push_back(embeddingMatrix[{(int64_t)idx}].unsqueezed(0));
+        }
+        return Tensor::stacking(embedded, 0);
+    }
+};
+
+// NN/Models/Transformer/PositionalEncoding.swift:33-71
+struct PositionalEncoding {
+    int64_t hiddenSize;
+    explicit PositionalEncoding(int64_t hiddenSize_) : hiddenSize(hiddenSize_) {
+        precondition(hiddenSize % 2 == 0, "Hidden size must be multiple of 2");
+    }
+    Tensor operator()(int64_t maxLen) const {
+        std::vector<float> ir((size_t)maxLen), hr((size_t)(hiddenSize / 2));
+        std::iota(ir.begin(), ir.end(), 0.f);
+        std::iota(hr.begin(), hr.end(), 0.f);
+        Tensor inputRange(ir, {maxLen}), hiddenRange(hr, {hiddenSize / 2});
+        Tensor frequencies = Tensor(10000.f).raised(hiddenRange / Tensor((float)(hiddenSize / 2)));
+        Tensor samplePoints = inputRange.unsqueezed(1) / frequencies.unsqueezed(0);   // [seqlen, hiddenSize / 2]
+        return Tensor::stacking({sin(samplePoints).unsqueezed(2), cos(samplePoints).unsqueezed(2)}, 2).view({-1, hiddenSize});
+    }
+};
+
+// NN/Models/Transformer/TransformerEncoder.swift:29-72
+struct TransformerEncoder {
+    std::vector<TransformerEncoderBlock> encoderLayers;
+    TransformerEncoder(int64_t layerCount, int64_t heads, int64_t keyDim, int64_t valueDim, int64_t modelDim, int64_t forwardDim, float dropout) {
+        for (int64_t i = 0; i < layerCount; ++i) encoderLayers.emplace_back(modelDim, forwardDim, heads, keyDim, valueDim, dropout);
+    }
+    Tensor operator()(const Tensor &input, const std::vector<int64_t> &sequenceLengths) const {
+        const Tensor mask = makeEncoderMasks(sequenceLengths);
+        Tensor acc = input;
+        for (auto &layer : encoderLayers) acc = layer(acc, mask);
+        return acc;
+    }
+};
+
+// NN/Models/Transformer/TransformerDecoder.swift:29-63
+struct TransformerDecoder {
+    std::vector<TransformerDecoderBlock> decoderLayers;
+    TransformerDecoder(int64_t layerCount, int64_t heads, int64_t keyDim, int64_t valueDim, int64_t modelDim, int64_t forwardDim, float dropout) {
+        for (int64_t i = 0; i < layerCount; ++i) decoderLayers.emplace_back(modelDim, forwardDim, heads, keyDim, valueDim, dropout);
+    }
+    Tensor operator()(const Tensor &decoderInput, const Tensor &encoderStates, const std::vector<int64_t> &encoderInputLengths,
+                      const std::vector<int64_t> &decoderInputLengths) const {
+        const Tensor encoderMask = makeEncoderMasks(encoderInputLengths);
+        const Tensor decoderMask = makeDecoderMasks(decoderInputLengths);
+        Tensor acc = decoderInput;
+        for (auto &layer : decoderLayers) acc = layer(acc, encoderStates, encoderMask, decoderMask);
+        return acc;
+    }
+    // Encoder-side key / value projections of every layer, computed once per encoded sequence (fused mode, head dims 64)
+    bool canCacheEncoderProjections() const {
+        for (auto &l : decoderLayers)
+            if (!l.encoderAttention.canCacheProjections()) return false;
+        return !decoderLayers.empty();
+    }
+    std::vector<std::pair<Tensor, Tensor>> projectEncoderStates(const Tensor &encoderStates) const {
+        std::vector<std::pair<Tensor, Tensor>> kv;
+        for (auto &l : decoderLayers) kv.push_back(l.encoderAttention.projectKeysValues(encoderStates, encoderStates));
+        return kv;
+    }
+    Tensor withProjectedEncoder(const Tensor &decoderInput, const std::vector<std::pair<Tensor, Tensor>> &kv,
+                                const std::vector<int64_t> &encoderInputLengths, const std::vector<int64_t> &decoderInputLengths) const {
+        const Tensor encoderMask = makeEncoderMasks(encoderInputLengths);
+        const Tensor decoderMask = makeDecoderMasks(decoderInputLengths);
+        Tensor acc = decoderInput;
+        for (size_t i = 0; i < decoderLayers.size(); ++i)
+            acc = decoderLayers[i].withProjectedEncoder(acc, kv[i].first, kv[i].second, encoderMask, decoderMask);
+        return acc;
+    }
+};
+
+// NN/Models/Transformer/Transformer.swift:29-138
+struct Transformer {
+    Embedding embedding;
+    PositionalEncoding positionalEncoding;
+    Dropout dropout;
+    TransformerEncoder encoder;
+    TransformerDecoder decoder;
+    Tensor outputBias;
+    Transformer(int64_t encoderLayers, int64_t decoderLayers, int64_t vocabSize, int64_t hiddenDim, int64_t heads, int64_t keyDim,
+                int64_t valueDim, int64_t forwardDim, float dropoutRate = 0.1f)
+        : embedding(vocabSize, hiddenDim, -1), positionalEncoding(hiddenDim), dropout(dropoutRate),
+          encoder(encoderLayers, heads, keyDim, valueDim, hiddenDim, forwardDim, dropoutRate),
+          decoder(decoderLayers, heads, keyDim, valueDim, hiddenDim, forwardDim, dropoutRate),
+          outputBias(Tensor::repeating(0.f, {vocabSize})) {}
+
+    // inputs: [batchSize][maxLen] tokens, -1 = padding                                   (Transformer.swift:86-92)
+    Tensor prepareInputs(const std::vector<int32_t> &inputs, int64_t batchSize, int64_t maxLen) const {
+        precondition((int64_t)inputs.size() == batchSize * maxLen, "element count does not match shape");
+        const int64_t D = embedding.outputSize();
+        const Tensor encoderPositions = positionalEncoding(maxLen);          // [maxLen, embedDim]
+        const float scale = std::sqrt((float)D);
+        if (Device::fused()) {
+            for (int32_t idx : inputs)
+                precondition(idx == -1 || (idx >= 0 && idx < embedding.embeddingMatrix.shape[0]), "index out of bounds");
+            Tensor tok = Embedding::uploadTokens(inputs);
+            Tensor res(Device::Memory::allocateBuffer(Shape{batchSize, maxLen, D}));
+            const ShapedBuffer pb = encoderPositions.values();
+            Device::Engine::embedPositions(embedding.embeddingMatrix.values(), reinterpret_cast<const int32_t *>(tok.buffer().memory),
+                                           batchSize, maxLen, embedding.ignoreIndex, &scale, &pb, res.values());
+            return dropout(res);
+        }
+        Tensor embedded = embedding(inputs).view({batchSize, maxLen, -1});
+        return dropout(embedded * Tensor(scale) + encoderPositions);
+    }
+
+    // log-softmax distributions [batchSize, decLen, vocab]                               (Transformer.swift:101-115)
+    Tensor operator()(const std::vector<int32_t> &encoderInput, int64_t encLen, const std::vector<int32_t> &decoderInput, int64_t decLen,
+                      const std::vector<int64_t> &encInLens, const std::vector<int64_t> &decInLens) const {
+        const int64_t batchSize = (int64_t)encInLens.size();
+        Tensor encoderStates = encoder(prepareInputs(encoderInput, batchSize, encLen), encInLens);
+        Tensor decoded = decoder(prepareInputs(decoderInput, batchSize, decLen), encoderStates, encInLens, decInLens);
+        Tensor deembedded = decoded.broadcastMatrixMultiplied(embedding.embeddingMatrix, false, true) + outputBias;
+        return logSoftmax(deembedded, 2);
+    }
+
+    // greedy decoding                                                                    (Transformer.swift:118-137)
+    // The reference re-runs the decoder on the whole prefix at every step, and so does this: MultiHeadAttention
+    // normalises over (length, hidden) jointly, so the output at every earlier position changes as the prefix grows and a
+    // self-attention key/value cache would compute something else.  What does not change is the encoder side: in fused
+    // mode the cross-attention key / value projections of the encoder states are computed once, not once per step.
+    std::vector<int32_t> greedy(const std::vector<int32_t> &inputSequence, int32_t startToken, int32_t endToken, int64_t maxLength,
+                                std::vector<float> *lastLogits = nullptr) const {
+        const int64_t n = (int64_t)inputSequence.size();
+        Tensor encoded = encoder(prepareInputs(inputSequence, 1, n), {n});
+        const bool cached = decoder.canCacheEncoderProjections();
+        std::vector<std::pair<Tensor, Tensor>> kv;
+        if (cached) kv = decoder.projectEncoderStates(encoded);
+        std::vector<int32_t> tokens;
+        for (int64_t step = 0; step < maxLength; ++step) {
+            std::vector<int32_t> tokenInput{startToken};
+            tokenInput.insert(tokenInput.end(), tokens.begin(), tokens.end());
+            const int64_t len = (int64_t)tokenInput.size();
+            Tensor decIn = prepareInputs(tokenInput, 1, len);
+            Tensor output = cached ? decoder.withProjectedEncoder(decIn, kv, {n}, {len}) : decoder(decIn, encoded, {n}, {len});
+            Tensor deembedded = output.broadcastMatrixMultiplied(embedding.embeddingMatrix, false, true);
+            Tensor last = deembedded[{0, len - 1}];
+            if (lastLogits) {
+                const std::vector<float> row = last.elements();
+                lastLogits->insert(lastLogits->end(), row.begin(), row.end());
+            }
+            const int32_t nextToken = (int32_t)last.argmax();
+            tokens.push_back(nextToken);
+            if (nextToken == endToken) break;
+        }
+        return tokens;
+    }
+};
 
 }  // namespace dl4s

@@ -3,6 +3,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <chrono>
 #include <functional>
 
 #include "dl4s_host.hpp"
@@ -162,6 +163,91 @@ int dl4s_host_make_decoder_masks(dl4s_hip_ctx *ctx, const int64_t *lengths, int6
         if (!out) return;
         Tensor m = makeDecoderMasks(lens);
         HIP::Memory::assign(m.buffer(), out, m.count());
+    });
+}
+
+struct dl4s_host_transformer {
+    Transformer model;
+    dl4s_hip_ctx *ctx;
+};
+
+int dl4s_host_transformer_create(dl4s_hip_ctx *ctx, const dl4s_host_transformer_config *c, const dl4s_host_transformer_params *p,
+                                 dl4s_host_transformer **out) {
+    if (out) *out = nullptr;
+    return guarded(ctx, 1, [&] {
+        precondition(c && p && out, "NULL argument");
+        precondition(c->encoder_layers >= 0 && c->decoder_layers >= 0 && c->vocab_size > 0 && c->hidden_dim > 0 && c->heads > 0 &&
+                         c->key_dim > 0 && c->value_dim > 0 && c->forward_dim > 0,
+                     "bad transformer configuration");
+        auto *t = new dl4s_host_transformer{Transformer(c->encoder_layers, c->decoder_layers, c->vocab_size, c->hidden_dim, c->heads,
+                                                        c->key_dim, c->value_dim, c->forward_dim, 0.1f),
+                                            ctx};
+        try {
+            Transformer &m = t->model;
+            m.dropout.isActive = false;
+            m.embedding.embeddingMatrix = Tensor(p->embedding, m.embedding.embeddingMatrix.shape);
+            m.outputBias = Tensor(p->output_bias, m.outputBias.shape);
+            for (int64_t i = 0; i < c->encoder_layers; ++i) {
+                load(m.encoder.encoderLayers[i].selfAttention, &p->encoder_attention[i]);
+                load(m.encoder.encoderLayers[i].pointwiseFeedForward, &p->encoder_ffn[i]);
+            }
+            for (int64_t i = 0; i < c->decoder_layers; ++i) {
+                load(m.decoder.decoderLayers[i].selfAttention, &p->decoder_self_attention[i]);
+                load(m.decoder.decoderLayers[i].encoderAttention, &p->decoder_encoder_attention[i]);
+                load(m.decoder.decoderLayers[i].pointwiseFeedForward, &p->decoder_ffn[i]);
+            }
+        } catch (...) {
+            delete t;
+            throw;
+        }
+        *out = t;
+    });
+}
+
+void dl4s_host_transformer_destroy(dl4s_host_transformer *t) {
+    if (!t) return;
+    HIP::context() = t->ctx;
+    delete t;
+}
+
+int dl4s_host_transformer_forward(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *encoder_input,
+                                  int64_t enc_len, const int32_t *decoder_input, int64_t dec_len, const int64_t *encoder_lengths,
+                                  const int64_t *decoder_lengths, int64_t B, float *out, int iters, float *out_ms) {
+    return guarded(ctx, fused, [&] {
+        precondition(t && encoder_input && decoder_input && encoder_lengths && decoder_lengths && out, "NULL argument");
+        std::vector<int32_t> enc(encoder_input, encoder_input + B * enc_len), dec(decoder_input, decoder_input + B * dec_len);
+        std::vector<int64_t> el(encoder_lengths, encoder_lengths + B), dl(decoder_lengths, decoder_lengths + B);
+        // the masks are as long as the longest sequence (TransformerUtil.swift:30, :40): the token arrays must match
+        precondition(*std::max_element(el.begin(), el.end()) == enc_len && *std::max_element(dl.begin(), dl.end()) == dec_len,
+                     "the padded length must equal the longest sequence length");
+        Tensor r = timed(ctx, iters, out_ms, [&] { return t->model(enc, enc_len, dec, dec_len, el, dl); });
+        HIP::Memory::assign(r.buffer(), out, r.count());
+    });
+}
+
+int dl4s_host_transformer_greedy(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence, int64_t n,
+                                 int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens,
+                                 int64_t *out_count, float *out_logits, float *out_ms) {
+    return guarded(ctx, fused, [&] {
+        precondition(t && input_sequence && out_tokens && out_count && n > 0 && max_length >= 0, "bad argument");
+        std::vector<int32_t> in(input_sequence, input_sequence + n);
+        std::vector<float> logits;
+        HIP::check(dl4s_hip_sync(ctx));
+        const auto t0 = std::chrono::steady_clock::now();
+        std::vector<int32_t> toks = t->model.greedy(in, start_token, end_token, max_length, out_logits ? &logits : nullptr);
+        HIP::check(dl4s_hip_sync(ctx));
+        if (out_ms) *out_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        *out_count = (int64_t)toks.size();
+        std::copy(toks.begin(), toks.end(), out_tokens);
+        if (out_logits) std::copy(logits.begin(), logits.end(), out_logits);
+    });
+}
+
+int dl4s_host_positional_encoding(dl4s_hip_ctx *ctx, int fused, int64_t max_len, int64_t hidden, float *out) {
+    return guarded(ctx, fused, [&] {
+        precondition(out != nullptr && max_len >= 0, "bad argument");
+        Tensor r = PositionalEncoding(hidden)(max_len);
+        HIP::Memory::assign(r.buffer(), out, r.count());
     });
 }
 

@@ -166,3 +166,81 @@ def make_decoder_masks(ctx, lengths):
     out = np.empty((len(lens), 1, L, L), np.float32)
     _check(fn(ctx.handle, lp, _i64(len(lens)), _p(out), None))
     return out
+
+
+class TransformerConfig(C.Structure):
+    _fields_ = [(n, _i64) for n in ("encoder_layers", "decoder_layers", "vocab_size", "hidden_dim", "heads", "key_dim",
+                                    "value_dim", "forward_dim")]
+
+
+class TransformerParams(C.Structure):
+    _fields_ = [("embedding", _f), ("output_bias", _f), ("encoder_attention", C.POINTER(MhaParams)),
+                ("encoder_ffn", C.POINTER(FfnParams)), ("decoder_self_attention", C.POINTER(MhaParams)),
+                ("decoder_encoder_attention", C.POINTER(MhaParams)), ("decoder_ffn", C.POINTER(FfnParams))]
+
+
+class Transformer:
+    """Transformer (NN/Models/Transformer/Transformer.swift) with its weights resident on the device.  `params` is the
+    dictionary oracle.transformer documents."""
+
+    def __init__(self, ctx, params):
+        self.ctx = ctx
+        E = _a(params["embedding"])
+        ne, nd = len(params["encoder"]), len(params["decoder"])
+        first = (params["encoder"][0]["ffn"] if ne else params["decoder"][0]["ffn"])
+        self.vocab = E.shape[0]
+        cfg = TransformerConfig(ne, nd, E.shape[0], E.shape[1], params["heads"], params["dk"], params["dv"],
+                                np.asarray(first["W1"]).shape[1])
+        keep = [E, _a(params["output_bias"])]
+        st = TransformerParams()
+        st.embedding, st.output_bias = _p(keep[0]), _p(keep[1])
+        ea = (MhaParams * max(1, ne))(*[_mha(l["attn"], keep) for l in params["encoder"]])
+        ef = (FfnParams * max(1, ne))(*[_ffn(l["ffn"], keep) for l in params["encoder"]])
+        ds = (MhaParams * max(1, nd))(*[_mha(l["self"], keep) for l in params["decoder"]])
+        dc = (MhaParams * max(1, nd))(*[_mha(l["cross"], keep) for l in params["decoder"]])
+        df = (FfnParams * max(1, nd))(*[_ffn(l["ffn"], keep) for l in params["decoder"]])
+        st.encoder_attention, st.encoder_ffn = ea, ef
+        st.decoder_self_attention, st.decoder_encoder_attention, st.decoder_ffn = ds, dc, df
+        self.handle = C.c_void_p()
+        _check(load().dl4s_host_transformer_create(ctx.handle, C.byref(cfg), C.byref(st), C.byref(self.handle)))
+
+    def close(self):
+        if self.handle:
+            load().dl4s_host_transformer_destroy(self.handle)
+            self.handle = None
+
+    def forward(self, enc_tokens, dec_tokens, enc_lengths, dec_lengths, fused=True, iters=0):
+        enc = np.ascontiguousarray(enc_tokens, np.int32)
+        dec = np.ascontiguousarray(dec_tokens, np.int32)
+        el, dl = np.ascontiguousarray(enc_lengths, np.int64), np.ascontiguousarray(dec_lengths, np.int64)
+        B = enc.shape[0]
+        out = np.empty((B, dec.shape[1], self.vocab), np.float32)
+        tp, t = _timing(iters)
+        i32, i64p = C.POINTER(C.c_int32), C.POINTER(_i64)
+        _check(load().dl4s_host_transformer_forward(self.ctx.handle, int(fused), self.handle, enc.ctypes.data_as(i32),
+                                                    _i64(enc.shape[1]), dec.ctypes.data_as(i32), _i64(dec.shape[1]),
+                                                    el.ctypes.data_as(i64p), dl.ctypes.data_as(i64p), _i64(B), _p(out),
+                                                    max(1, iters), tp))
+        return (out, t.value) if iters else out
+
+    def greedy(self, input_sequence, start_token, end_token, max_length, fused=True, return_logits=False, timing=False):
+        src = np.ascontiguousarray(input_sequence, np.int32)
+        toks = np.empty(max(1, max_length), np.int32)
+        n = _i64()
+        logits = np.empty((max(1, max_length), self.vocab), np.float32) if return_logits else None
+        ms = C.c_float()
+        _check(load().dl4s_host_transformer_greedy(self.ctx.handle, int(fused), self.handle, src.ctypes.data_as(C.POINTER(C.c_int32)),
+                                                   _i64(len(src)), C.c_int32(start_token), C.c_int32(end_token), _i64(max_length),
+                                                   toks.ctypes.data_as(C.POINTER(C.c_int32)), C.byref(n), _p(logits), C.byref(ms)))
+        res = [[int(x) for x in toks[:n.value]]]
+        if return_logits:
+            res.append(logits[:n.value])
+        if timing:
+            res.append(ms.value)
+        return res[0] if len(res) == 1 else tuple(res)
+
+
+def positional_encoding(ctx, max_len, hidden, fused=True):
+    out = np.empty((max_len, hidden), np.float32)
+    _check(load().dl4s_host_positional_encoding(ctx.handle, int(fused), _i64(max_len), _i64(hidden), _p(out)))
+    return out

@@ -55,6 +55,38 @@ int dl4s_host_decoder_block(dl4s_hip_ctx *ctx, int fused, const float *dec, cons
 int dl4s_host_make_encoder_masks(dl4s_hip_ctx *ctx, const int64_t *lengths, int64_t B, float *out, int64_t *out_len);
 int dl4s_host_make_decoder_masks(dl4s_hip_ctx *ctx, const int64_t *lengths, int64_t B, float *out, int64_t *out_len);
 
+/* ---- the model wrapper: Transformer (NN/Models/Transformer/Transformer.swift:29-138), dropout inactive.
+ * The object keeps its weights on the device between calls. */
+typedef struct dl4s_host_transformer dl4s_host_transformer;
+typedef struct dl4s_host_transformer_config {
+    int64_t encoder_layers, decoder_layers, vocab_size, hidden_dim, heads, key_dim, value_dim, forward_dim;
+} dl4s_host_transformer_config;
+typedef struct dl4s_host_transformer_params {
+    const float *embedding;   /* [vocab, hidden]: Embedding.embeddingMatrix, shared with the output projection */
+    const float *output_bias; /* [vocab] */
+    const dl4s_host_mha_params *encoder_attention; /* [encoder_layers] */
+    const dl4s_host_ffn_params *encoder_ffn;       /* [encoder_layers] */
+    const dl4s_host_mha_params *decoder_self_attention, *decoder_encoder_attention; /* [decoder_layers] each */
+    const dl4s_host_ffn_params *decoder_ffn;       /* [decoder_layers] */
+} dl4s_host_transformer_params;
+
+int dl4s_host_transformer_create(dl4s_hip_ctx *ctx, const dl4s_host_transformer_config *config,
+                                 const dl4s_host_transformer_params *params, dl4s_host_transformer **out);
+void dl4s_host_transformer_destroy(dl4s_host_transformer *t);
+/* callAsFunction((encoderInput, decoderInput, encoderInputLengths, decoderInputLengths)) -- Transformer.swift:101-115.
+ * Tokens are [B, enc_len] / [B, dec_len] int32 with -1 as padding; out is [B, dec_len, vocab] log-probabilities. */
+int dl4s_host_transformer_forward(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *encoder_input,
+                                  int64_t enc_len, const int32_t *decoder_input, int64_t dec_len, const int64_t *encoder_lengths,
+                                  const int64_t *decoder_lengths, int64_t B, float *out, int iters, float *out_ms);
+/* callAsFunction(inputSequence:startToken:endToken:maxLength:) -- Transformer.swift:118-137.  out_tokens holds up to
+ * max_length tokens, *out_count how many were produced; out_logits (may be NULL) receives the [count, vocab] rows the
+ * argmax was taken over; out_ms (may be NULL) the wall time of the whole decode in milliseconds. */
+int dl4s_host_transformer_greedy(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence,
+                                 int64_t n, int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens,
+                                 int64_t *out_count, float *out_logits, float *out_ms);
+/* PositionalEncoding(hiddenSize)(maxLen) -> [maxLen, hiddenSize] -- PositionalEncoding.swift:52-69 */
+int dl4s_host_positional_encoding(dl4s_hip_ctx *ctx, int fused, int64_t max_len, int64_t hidden, float *out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,168 @@
+"""The callers on either side of the attention path: the engine additions the Transformer wrapper needs, and the wrapper
+itself (embedding, positional encoding, encoder / decoder stacks, log-softmax output, greedy decoding) through the C++
+host layer, against the CPU oracle.  Gate as everywhere: |gpu - oracle| <= 1e-4 + 1e-4 |oracle|; integer results exact."""
+import numpy as np
+import pytest
+
+from helpers import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from dl4s_amd import lib
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+def test_log_sin_cos(ctx, orc):
+    rng = np.random.default_rng(31)
+    n = 50001
+    x = (rng.random(n) * 600.0).astype(np.float32)
+    p = (rng.random(n) * 1e4 + 1e-3).astype(np.float32)
+    dx, dp, dy = ctx.to_device(x), ctx.to_device(p), ctx.empty((n,))
+    ctx.sin(dx, dy, n)
+    assert_parity(dy.numpy(), orc.sin(x), "sin")
+    ctx.cos(dx, dy, n)
+    assert_parity(dy.numpy(), orc.cos(x), "cos")
+    ctx.log(dp, dy, n)
+    assert_parity(dy.numpy(), orc.log(p), "log")
+    for b in (dx, dp, dy):
+        b.release()
+
+
+@pytest.mark.parametrize("n", [1, 7, 1024, 1025, 100003])
+def test_argmax_matches_the_reference_scan(ctx, orc, n):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal(n).astype(np.float32)
+    if n > 6:
+        x[[2, n - 3]] = x.max() + 1.0          # a tie far apart: the first wins
+        x[n // 2] = np.nan                      # NaN is never selected
+    d = ctx.to_device(x)
+    assert ctx.argmax(d, n) == orc.argmax(x)
+    d.release()
+
+
+def test_argmax_nothing_selected(ctx, orc):
+    for x in (np.array([np.nan, np.nan, np.nan], np.float32), np.full(2000, -np.inf, np.float32)):
+        d = ctx.to_device(x)
+        assert ctx.argmax(d, len(x)) == orc.argmax(x) == (0, -np.inf)
+        d.release()
+    d = ctx.empty((4,))
+    assert ctx.argmax(d, 0) == (0, -np.inf)
+    d.release()
+
+
+def test_stack_along_inner_axis(ctx):
+    rng = np.random.default_rng(32)
+    a, b, c = (rng.standard_normal(s).astype(np.float32) for s in ((5, 3, 4), (5, 2, 4), (5, 1, 4)))
+    da, db, dc, dy = ctx.to_device(a), ctx.to_device(b), ctx.to_device(c), ctx.empty((5, 6, 4))
+    ctx.stack_axis([da, db, dc], [12, 8, 4], 5, dy)
+    assert np.array_equal(dy.numpy(), np.concatenate([a, b, c], axis=1))
+    for x in (da, db, dc, dy):
+        x.release()
+
+
+def test_embedding_with_scale_and_positions(ctx, orc):
+    from oracle import transformer as T
+    rng = np.random.default_rng(33)
+    V, D, B, L = 29, 24, 3, 7
+    E = rng.standard_normal((V, D)).astype(np.float32)
+    tok = rng.integers(0, V, (B, L)).astype(np.int32)
+    tok[1, 4:] = -1
+    dE, dt, dy = ctx.to_device(E), ctx.to_device(tok, dtype=np.int32), ctx.empty((B, L, D))
+    ctx.embed_positions(dE, V, D, dt, B, L, -1, None, None, dy)
+    assert np.array_equal(dy.numpy(), orc.embedding(E, tok.reshape(-1), -1).reshape(B, L, D))
+    pos = T.positional_encoding(L, D)
+    dpos = ctx.to_device(pos)
+    scale = float(np.sqrt(np.float32(D)))
+    ctx.embed_positions(dE, V, D, dt, B, L, -1, scale, dpos, dy)
+    assert np.array_equal(dy.numpy(), T.prepare_inputs({"embedding": E}, tok))     # same roundings, same bits
+    for x in (dE, dt, dy, dpos):
+        x.release()
+
+
+def test_log_softmax_rows(ctx):
+    from oracle import transformer as T
+    rng = np.random.default_rng(34)
+    x = (rng.standard_normal((37, 1000)) * 5).astype(np.float32)
+    x[3, 10] = 80.0
+    dx, dy = ctx.to_device(x), ctx.empty(x.shape)
+    ctx.log_softmax(dx, 37, 1000, dy)
+    assert_parity(dy.numpy(), T.log_softmax(x), "logSoftmax")
+    dx.release()
+    dy.release()
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_positional_encoding_layer(ctx, fused):
+    from dl4s_amd import host_lib
+    from oracle import transformer as T
+    got = host_lib.positional_encoding(ctx, 300, 64, fused=fused)
+    assert_parity(got, T.positional_encoding(300, 64), "PositionalEncoding")
+
+
+def _model(seed, vocab, D, H, dk, F, n_enc, n_dec):
+    from oracle import fp64_model as m64
+    rng = np.random.default_rng(seed)
+    return m64.make_transformer_params(rng, vocab, D, H, dk, dk, F, n_enc, n_dec), rng
+
+
+CONFIGS = {  # vocab, hidden, heads, key/value dim, ffn, encoder layers, decoder layers
+    "transformer_tests_hyperparameters": (13, 16, 4, 8, 32, 2, 2),   # Tests/DL4STests/TransformerTests.swift:31
+    "head_dim_64": (40, 128, 2, 64, 256, 2, 2),
+}
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+@pytest.mark.parametrize("fused", [False, True])
+def test_transformer_forward(ctx, name, fused):
+    from dl4s_amd import host_lib
+    from oracle import transformer as T
+    vocab = CONFIGS[name][0]
+    params, rng = _model(41, *CONFIGS[name])
+    enc_len, dec_len = [9, 5, 7], [6, 6, 2]
+    enc = np.full((3, 9), -1, np.int32)
+    dec = np.full((3, 6), -1, np.int32)
+    for b in range(3):
+        enc[b, :enc_len[b]] = rng.integers(0, vocab, enc_len[b])
+        dec[b, :dec_len[b]] = rng.integers(0, vocab, dec_len[b])
+    model = host_lib.Transformer(ctx, params)
+    got = model.forward(enc, dec, enc_len, dec_len, fused=fused)
+    model.close()
+    ref = T.forward(params, enc, dec, enc_len, dec_len)
+    assert_parity(got, ref, "Transformer forward %s fused=%s" % (name, fused))
+    assert np.allclose(np.exp(got.astype(np.float64)).sum(-1), 1.0, atol=1e-4)
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_greedy_decoding(ctx, name):
+    """Same tokens as the oracle's decoding, logits within tolerance; fused mode (which keeps the encoder-side key / value
+    projections across steps when the head size allows) and primitive mode agree."""
+    from dl4s_amd import host_lib
+    from oracle import transformer as T
+    vocab = CONFIGS[name][0]
+    params, rng = _model(43, *CONFIGS[name])
+    src = [int(t) for t in rng.integers(0, vocab, 8)]
+    ref_tokens, ref_logits = T.greedy_decode(params, src, 1, 2, 7, return_logits=True)
+    top2 = np.sort(np.stack(ref_logits), axis=1)[:, -2:]
+    assert (top2[:, 1] - top2[:, 0]).min() > 1e-3, "the fixture must not sit on an argmax tie"
+    model = host_lib.Transformer(ctx, params)
+    for fused in (True, False):
+        toks, logits = model.greedy(src, 1, 2, 7, fused=fused, return_logits=True)
+        assert toks == ref_tokens
+        assert_parity(logits, np.stack(ref_logits), "greedy logits %s fused=%s" % (name, fused))
+    model.close()
+
+
+def test_transformer_argument_errors(ctx):
+    from dl4s_amd import host_lib
+    params, rng = _model(44, *CONFIGS["transformer_tests_hyperparameters"])
+    model = host_lib.Transformer(ctx, params)
+    with pytest.raises(host_lib.HostError):       # token outside the vocabulary: the reference traps on the subscript
+        model.forward([[99, 1]], [[1]], [2], [1])
+    with pytest.raises(host_lib.HostError):       # padded length differs from the longest sequence
+        model.forward([[3, 1, -1]], [[1]], [2], [1])
+    model.close()
