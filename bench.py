@@ -171,6 +171,28 @@ def other_configs(ctx, lib, cpu):
         res["config3_encoder_block_B8_L1024_D1024_H16_F4096_fused"]["cpu_baseline"] = {
             "tflops": fl1 / dt / 1e12, "cores": 1, "kind": "port",
             "sample": "one batch item cut to 256 tokens (%.1f s); extrapolated whole call %.0f s" % (dt, dt * fl / fl1)}
+    # the caller of the blocks: Transformer greedy decoding (batch 1; every step re-runs the decoder on the prefix, as the
+    # reference does).  6 + 6 layers, hidden 512, 8 heads of 64, ffn 2048, vocabulary 8000, 64 source tokens, 32 generated.
+    rng = np.random.Generator(np.random.PCG64(1006))
+    params = m64.make_transformer_params(rng, 8000, 512, 8, 64, 64, 2048, 6, 6)
+    src = [int(t) for t in rng.integers(0, 8000, 64)]
+    model = host_lib.Transformer(ctx, params)
+    entry = {"workload": "Transformer greedy decode, 6+6 layers, hidden 512, 8 heads x 64, ffn 2048, vocab 8000, 64 source tokens, "
+                         "32 generated tokens (prefix re-run every step)"}
+    for mode, fused in (("fused", True), ("primitive", False)):
+        model.greedy(src, 1, -5, 4, fused=fused)                       # warm the allocator pool
+        toks, ms = model.greedy(src, 1, -5, 32, fused=fused, timing=True)
+        entry["ms_per_token_" + mode] = ms / len(toks)
+        entry["tokens_per_s_" + mode] = len(toks) / ms * 1e3
+    model.close()
+    if cpu:
+        from oracle import transformer as orc_t
+        t0 = time.perf_counter()
+        n_cpu = len(orc_t.greedy_decode(params, src, 1, -5, 4))
+        dt = time.perf_counter() - t0
+        entry["cpu_baseline"] = {"ms_per_token": dt * 1e3 / n_cpu, "cores": 1, "kind": "port",
+                                 "sample": "encoder pass + the first %d generated tokens (%.1f s)" % (n_cpu, dt)}
+    res["transformer_greedy_decode"] = entry
     return res
 
 
