@@ -255,6 +255,23 @@ def sdpa(q, k, v, mask=None, temperature=None):
     return out
 
 
+def sdpa_backward(q, k, v, mask, dout, temperature=None):
+    """(dq, dk, dv) for the upstream gradient dout of sdpa(q, k, v, mask)."""
+    q, k, v, dout = _f32(q), _f32(k), _f32(v), _f32(dout)
+    B, H, Lq, dk = q.shape
+    Lk, dv = v.shape[2], v.shape[3]
+    assert dout.shape == (B, H, Lq, dv)
+    if temperature is None:
+        temperature = float(np.sqrt(np.float32(dk)))
+    dq, dkey, dval = np.empty_like(q), np.empty_like(k), np.empty_like(v)
+    mp, ms, md, keep = _mask_args(mask)
+    rc = lib().orc_sdpa_backward(_p(q), _p(k), _p(v), mp, ms, md, C.c_int64(B), C.c_int64(H), C.c_int64(Lq), C.c_int64(Lk),
+                                 C.c_int64(dk), C.c_int64(dv), C.c_float(temperature), _p(dout), _p(dq), _p(dkey), _p(dval))
+    if rc:
+        raise ValueError("orc_sdpa_backward rc=%d" % rc)
+    return dq, dkey, dval
+
+
 def sdpa_decode(q, kcache, vcache, T, temperature=None):
     q, kcache, vcache = _f32(q), _f32(kcache), _f32(vcache)
     B, H, Tcap, d = kcache.shape

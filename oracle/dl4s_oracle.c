@@ -28,6 +28,8 @@
  *   orc_encoder_block,
  *   orc_decoder_block        torch.nn.functional.multi_head_attention_forward in fp64 for the
  *                            attention core; an independent fp64 numpy model for the whole layer
+ *   orc_sdpa_backward        torch.autograd in fp64 through softmax(q k^T / T - 1e9 mask) v, central
+ *                            finite differences of the oracle's own forward in fp64 arithmetic
  *   orc_log, orc_sin, orc_cos  numpy fp64 log/sin/cos; the reference's log accuracy test
  *                            Tests/DL4STests/VecTests.swift:242-258 (1e-4)
  *   orc_argmax               numpy.argmax (first maximum), hand-written NaN / tie / empty vectors
@@ -440,6 +442,91 @@ int orc_sdpa(const float *q, const float *k, const float *v, const float *mask,
         rc = orc_bmm(P, ssh, v, vsh, 4, 0, 0, out);
     }
     free(qs); free(S); free(P);
+    return rc;
+}
+
+/* ------------------------------------------------------------- SDPA backward */
+/* Gradients of ScaledDotProductAttention with respect to q, k and v for an upstream gradient dout of its result, as
+ * the reference's reverse-mode closures produce them for the forward graph of ScaledDotProductAttention.swift:43-64:
+ *   o = p.bmm(v)            per slice dp = dout . v^T, dv = p^T . dout          Matrix.swift:139-174 (through the
+ *                           subscript views and the stack of broadcastMatrixMultiplied, Matrix.swift:79-117)
+ *   p = e / z               de = dp * (1/z);  dz = -sum_j((dp * e) * (1/(z*z)))   Binary.swift:235-300
+ *   z = reduceSum(e, 3)     de += dz (broadcast along the row)                    Reduce.swift:35-62
+ *   e = exp(d)              dd = de * e                                            Unary.swift:33-55
+ *   d = s2 - max (detached), s2 = s - mask*1e9: gradient passes unchanged          Unary.swift:190-194, Binary.swift:161-224
+ *   s = a.bmm(k^T)          da = ds . k, dk = (a^T . ds)^T                         Matrix.swift:139-174
+ *   a = q / T               dq = da * (1/T)                                        Binary.swift:259-277
+ * The mask takes no gradient.  Every product is the generic triple loop, every element-wise step one rounding. */
+int orc_sdpa_backward(const float *q, const float *k, const float *v, const float *mask,
+                      const int64_t *mshape, int mdim, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                      int64_t dk, int64_t dv, float temperature, const float *dout,
+                      float *dq, float *dkey, float *dval) {
+    int64_t nq = B * H * Lq * dk, ns = B * H * Lq * Lk;
+    float *qs = (float *)malloc(sizeof(float) * (size_t)(nq > 0 ? nq : 1));
+    float *S = (float *)malloc(sizeof(float) * (size_t)(ns > 0 ? ns : 1));
+    float *E = (float *)malloc(sizeof(float) * (size_t)(ns > 0 ? ns : 1));
+    float *Z = (float *)malloc(sizeof(float) * (size_t)(B * H * Lq > 0 ? B * H * Lq : 1));
+    float *G = (float *)malloc(sizeof(float) * (size_t)(Lq * Lk > 0 ? Lq * Lk : 1));
+    float *Pm = (float *)malloc(sizeof(float) * (size_t)(Lq * Lk > 0 ? Lq * Lk : 1));
+    float *da = (float *)malloc(sizeof(float) * (size_t)(Lq * dk > 0 ? Lq * dk : 1));
+    float *dkt = (float *)malloc(sizeof(float) * (size_t)(Lk * dk > 0 ? Lk * dk : 1));
+    int rc = (!qs || !S || !E || !Z || !G || !Pm || !da || !dkt) ? -2 : 0;
+    if (rc == 0) {
+        float rT = 1.0f / temperature;
+        for (int64_t i = 0; i < nq; ++i) qs[i] = q[i] * rT;
+        int64_t qsh[4] = {B, H, Lq, dk}, ksh[4] = {B, H, Lk, dk}, ssh[4] = {B, H, Lq, Lk};
+        rc = orc_bmm(qs, qsh, k, ksh, 4, 0, 1, S);
+        if (rc == 0 && mask) {
+            int64_t mn = orc_count(mshape, mdim);
+            float *M = (float *)malloc(sizeof(float) * (size_t)(mn > 0 ? mn : 1));
+            if (!M) rc = -2;
+            else {
+                for (int64_t i = 0; i < mn; ++i) M[i] = mask[i] * 1e9f;
+                rc = orc_broadcast(1, S, ssh, 4, M, mshape, mdim, E, NULL);
+                if (rc == 0) memcpy(S, E, sizeof(float) * (size_t)ns);
+                free(M);
+            }
+        }
+    }
+    if (rc == 0) {
+        /* forward intermediates of the softmax: e = exp(s - max), z = sum(e) */
+        for (int64_t r = 0; r < B * H * Lq; ++r) {
+            const float *p = S + r * Lk; float *e = E + r * Lk;
+            float mx = -INFINITY;
+            for (int64_t c = 0; c < Lk; ++c) if (p[c] > mx) mx = p[c];
+            float nmx = -mx, z = 0.0f;
+            for (int64_t c = 0; c < Lk; ++c) e[c] = expf(p[c] + nmx);
+            for (int64_t c = 0; c < Lk; ++c) z += e[c];
+            Z[r] = z;
+        }
+        float rT = 1.0f / temperature;
+        for (int64_t bh = 0; bh < B * H; ++bh) {
+            const float *e = E + bh * Lq * Lk, *z = Z + bh * Lq;
+            const float *go = dout + bh * Lq * dv, *vv = v + bh * Lk * dv, *kk = k + bh * Lk * dk;
+            /* p = e * (1/z) */
+            for (int64_t r = 0; r < Lq; ++r) {
+                float rz = 1.0f / z[r];
+                for (int64_t c = 0; c < Lk; ++c) Pm[r * Lk + c] = e[r * Lk + c] * rz;
+            }
+            orc_gemm(1, 0, Lk, dv, Lq, 1.0f, Pm, go, 0.0f, dval + bh * Lk * dv);   /* dv = p^T . dout */
+            orc_gemm(0, 1, Lq, Lk, dv, 1.0f, go, vv, 0.0f, G);                      /* dp = dout . v^T */
+            for (int64_t r = 0; r < Lq; ++r) {
+                float zr = z[r], rz = 1.0f / zr, rzz = 1.0f / (zr * zr), acc = 0.0f;
+                for (int64_t c = 0; c < Lk; ++c) acc += (G[r * Lk + c] * e[r * Lk + c]) * rzz;
+                float dz = -acc;
+                for (int64_t c = 0; c < Lk; ++c) {
+                    float de = G[r * Lk + c] * rz + dz;
+                    G[r * Lk + c] = de * e[r * Lk + c];                                        /* ds */
+                }
+            }
+            orc_gemm(0, 0, Lq, dk, Lk, 1.0f, G, kk, 0.0f, da);                      /* da = ds . k */
+            for (int64_t i = 0; i < Lq * dk; ++i) dq[bh * Lq * dk + i] = da[i] * rT;
+            orc_gemm(1, 0, dk, Lk, Lq, 1.0f, qs + bh * Lq * dk, G, 0.0f, dkt);      /* a^T . ds : [dk, Lk] */
+            for (int64_t c = 0; c < Lk; ++c)
+                for (int64_t l = 0; l < dk; ++l) dkey[bh * Lk * dk + c * dk + l] = dkt[l * Lk + c];
+        }
+    }
+    free(qs); free(S); free(E); free(Z); free(G); free(Pm); free(da); free(dkt);
     return rc;
 }
 

@@ -480,3 +480,49 @@ def test_greedy_decode_is_consistent_with_the_forward_pass():
         assert int(np.argmax(lp[0, -1])) == tok
         ref = m64.transformer64(params, np.array([src]), np.array(prefix), [len(src)], [t + 1], log_probs=False)
         assert np.abs(logits[t] - ref[0, -1]).max() < 2e-4
+
+
+# ------------------------------------------------------------------ SDPA backward
+@pytest.mark.parametrize("masked", [False, True])
+def test_sdpa_backward_against_torch_autograd_fp64(orc, masked):
+    import torch
+    rng = np.random.default_rng(12)
+    B, H, Lq, Lk, d = 2, 3, 9, 11, 8
+    q, k, v = (rng.standard_normal(s).astype(np.float32) for s in ((B, H, Lq, d), (B, H, Lk, d), (B, H, Lk, d)))
+    dout = rng.standard_normal((B, H, Lq, d)).astype(np.float32)
+    mask = (rng.random((B, 1, Lq, Lk)) < 0.3).astype(np.float32) if masked else None
+    if masked:
+        mask[0, 0, 2, :] = 1.0          # a fully blocked row: uniform weights, gradient still defined
+    dq, dk, dv = orc.sdpa_backward(q, k, v, mask, dout)
+    tq, tk, tv = (torch.tensor(x, dtype=torch.float64, requires_grad=True) for x in (q, k, v))
+    s = tq @ tk.transpose(-1, -2) / np.sqrt(d)
+    if masked:
+        # the value of a blocked score is what fp32 leaves of s - 1e9 (exactly -1e9 for |s| < 32, so a fully blocked row is
+        # uniform), while the reference's closures pass the gradient through the subtraction unchanged
+        collapsed = (s.detach().float() - torch.tensor(mask) * 1e9).double()
+        s = s + (collapsed - s).detach()
+    o = torch.softmax(s, dim=-1) @ tv
+    o.backward(torch.tensor(dout, dtype=torch.float64))
+    for got, ref, name in ((dq, tq.grad, "dq"), (dk, tk.grad, "dk"), (dv, tv.grad, "dv")):
+        assert np.abs(got - ref.numpy()).max() < 2e-5, name
+
+
+def test_sdpa_backward_against_finite_differences():
+    """Directional derivative of sum(out * dout) along random directions, central differences in fp64 (independent model)."""
+    from oracle import binding as orc, fp64_model as m64
+    rng = np.random.default_rng(13)
+    B, H, L, d = 1, 2, 6, 4
+    q, k, v, dout = (rng.standard_normal((B, H, L, d)).astype(np.float32) for _ in range(4))
+    i, j = np.indices((L, L))
+    mask = (j > i).astype(np.float32)
+    dq, dk, dv = orc.sdpa_backward(q, k, v, mask, dout)
+    f = lambda q_, k_, v_: float((m64.sdpa64(q_, k_, v_, mask) * dout).sum())
+    eps = 1e-6
+    for grad, idx in ((dq, 0), (dk, 1), (dv, 2)):
+        direction = rng.standard_normal((B, H, L, d))
+        args_p = [x.astype(np.float64) for x in (q, k, v)]
+        args_m = [x.astype(np.float64) for x in (q, k, v)]
+        args_p[idx] = args_p[idx] + eps * direction
+        args_m[idx] = args_m[idx] - eps * direction
+        fd = (f(*args_p) - f(*args_m)) / (2 * eps)
+        assert abs(fd - float((grad * direction).sum())) < 1e-4
