@@ -1,0 +1,460 @@
+// Gradients of the fused attention for gfx950 (head dim 64): given dout = d(loss)/d(out) of
+//   out = softmax((q * rT) . k^T - mask * 1e9) . v
+// compute dq, dk, dv.  With p = the softmax weights and D_i = sum_d dout[i][d] * out[i][d] (= sum_j dp_ij p_ij):
+//   dv = p^T . dout,   dp = dout . v^T,   ds = p * (dp - D),   dq = (ds . k) * rT,   dk = ds^T . (q * rT)
+// which is what the reference's reverse-mode closures compute for the forward graph of
+// NN/Models/Transformer/ScaledDotProductAttention.swift:43-64 (Tensor/Operators/Matrix.swift:139-174,
+// Binary.swift:235-300, Unary.swift:33-55, Reduce.swift:35-62), up to the order of the floating-point operations.
+//
+// The weights are not stored by the forward pass: they are recomputed tile by tile as p = 2^(s - m) / l, where s is the
+// base-2 score exactly as the forward kernel forms it and (m, 1/l) the two row statistics that
+// dl4s_hip_sdpa_fwd_stats_f32 leaves per row (the forward pass's reference maximum and the reciprocal of its row sum).
+// Two kernels, both deterministic (no atomics):
+//   sdpa_bwd_dq_f32_d64    a wavefront owns 32 queries and walks the keys like the forward kernel
+//                          (S^T, dP^T in the accumulator layout lane = query; dQ^T += K^T . dS^T)
+//   sdpa_bwd_dkv_f32_d64   a wavefront owns 32 keys and walks the queries (S, dP with lane = key;
+//                          dV^T += dO^T . P, dK^T += Q^T . dS)
+// All five products of each run on v_mfma_f32_32x32x2_f32 with the operand layouts of the forward kernel.
+#include "sdpa_common.h"
+
+namespace {
+
+constexpr float LN2 = 0.69314718055994530942f;
+
+// D[b,h,i] = sum_d dout[i][d] * out[i][d]; 16 lanes per row, four rows per wavefront
+__global__ __launch_bounds__(256) void sdpa_bwd_rowdot(const float *__restrict__ out, const float *__restrict__ dout,
+                                                       float *__restrict__ D, int H, int Lq, long long rows, int token_major) {
+    const long long r = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int c = (threadIdx.x & 15) * 4;
+    float acc = 0.f;
+    if (r < rows) {
+        const long long bh = r / Lq, qi = r % Lq;
+        const long long off = token_major ? (((bh / H) * Lq + qi) * H + bh % H) * HD : r * HD;
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(out + off + c);
+        const f32x4 g = *reinterpret_cast<const f32x4 *>(dout + off + c);
+        acc = a.x * g.x + a.y * g.y + a.z * g.z + a.w * g.w;
+    }
+    acc += __shfl_xor(acc, 8, 64);
+    acc += __shfl_xor(acc, 4, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    acc += __shfl_xor(acc, 1, 64);
+    if (r < rows && (threadIdx.x & 15) == 0) D[r] = acc;
+}
+
+// 32 x 32 product tile in the transposed accumulator layout of the forward kernel: A rows from LDS (lane reads row
+// lane % 32, 128-bit reads at columns half*32 + 4j), B from the lane's 32 registers.
+__device__ __forceinline__ f32x16 tile_product(const float *Ab, const float (&br)[32]) {
+    f32x16 acc;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Ab + 4 * j);
+        if (j == 0) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, br[0], zero, 0, 0, 0);
+        } else {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, br[4 * j + 0], acc, 0, 0, 0);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, br[4 * j + 1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, br[4 * j + 2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, br[4 * j + 3], acc, 0, 0, 0);
+    }
+    return acc;
+}
+
+// acc0/acc1 (rows d = 2m, 2m+1; column = the lane's query or key) += A^T . B where A is a [32][64] LDS tile read
+// through 64-bit loads (row 8(r/4) + r%4 + 4*half, columns 2*lane%32 + {0,1}: At already points there) and B the
+// accumulator-layout tile b.
+__device__ __forceinline__ void tile_accumulate_t(const float *At, const f32x16 &b, f32x16 &acc0, f32x16 &acc1) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const f32x2 a = *reinterpret_cast<const f32x2 *>(At + (8 * (r >> 2) + (r & 3)) * LSTR);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[r], acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[r], acc1, 0, 0, 0);
+    }
+}
+
+// Stores the transposed accumulators (register r of acc0/acc1 is d = 2*(8(r/4) + 4*half + r%4) + {0,1}) of the lane's
+// row to p[row][0..63], scaled.
+__device__ __forceinline__ void store_row_t(float *p, const f32x16 &acc0, const f32x16 &acc1, const float scale) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        f32x4 a, c;
+        a.x = acc0[4 * g + 0] * scale; a.y = acc1[4 * g + 0] * scale;
+        a.z = acc0[4 * g + 1] * scale; a.w = acc1[4 * g + 1] * scale;
+        c.x = acc0[4 * g + 2] * scale; c.y = acc1[4 * g + 2] * scale;
+        c.z = acc0[4 * g + 3] * scale; c.w = acc1[4 * g + 3] * scale;
+        *reinterpret_cast<f32x4 *>(p + 16 * g) = a;
+        *reinterpret_cast<f32x4 *>(p + 16 * g + 4) = c;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ dQ
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
+                                                               const float *__restrict__ v, const float *__restrict__ dout,
+                                                               const float *__restrict__ stats, const float *__restrict__ D,
+                                                               float *__restrict__ dq, int H, int Lq, int Lk, float rT,
+                                                               MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
+                                                               int token_major) {
+    extern __shared__ __align__(16) float lds[];
+    float *Ks = lds;                     // [2][BN][LSTR]
+    float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
+    int bh, unit;
+    if (!work_item(nqb, total_blocks, lpt, bh, unit)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int qb = nqb - 1 - unit;   // longest rows first
+    const int q0 = qb * BM + wave * 32;
+    const int qi = q0 + ln;
+    const int qic = qi < Lq ? qi : Lq - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * HD : HD;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+
+    // the same tiles as the forward pass visits (skipped tiles have weight exactly 0, hence gradient 0)
+    int kend = Lk, wkend = Lk;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
+        if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    float qr[32], gr[32];   // lane's Q fragment (scaled as in the forward pass) and dout fragment
+    {
+        const float *qp = q + q_base + (long long)qic * rs + half * 32;
+        const float *gp = dout + q_base + (long long)qic * rs + half * 32;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+            const f32x4 g = *reinterpret_cast<const f32x4 *>(gp + 4 * j);
+            qr[4 * j + 0] = (t.x * rT) * LOG2E; qr[4 * j + 1] = (t.y * rT) * LOG2E;
+            qr[4 * j + 2] = (t.z * rT) * LOG2E; qr[4 * j + 3] = (t.w * rT) * LOG2E;
+            gr[4 * j + 0] = g.x; gr[4 * j + 1] = g.y; gr[4 * j + 2] = g.z; gr[4 * j + 3] = g.w;
+        }
+    }
+    const float m_i = stats[2 * ((long long)bh * Lq + qic)];
+    const float rl_i = stats[2 * ((long long)bh * Lq + qic) + 1];
+    const float D_i = D[(long long)bh * Lq + qic];
+
+    const int ld_row = tid >> 4, ld_col = (tid & 15) * 4;
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + HD) * 4);
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
+    const unsigned ld_off0 = (unsigned)(ld_row * rs + ld_col) * 4u;
+    const unsigned ld_off1 = ld_off0 + 16u * rs * 4u;
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[2], vst[2];
+    auto load_tile = [&](int t) {
+        const int o0 = (int)(ld_off0 + t * tile_bytes), o1 = (int)(ld_off1 + t * tile_bytes);
+        kst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o0, 0, 0));
+        vst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o0, 0, 0));
+        kst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o1, 0, 0));
+        vst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o1, 0, 0));
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int off = buf * TILE_FLOATS + (i * 16 + ld_row) * LSTR + ld_col;
+            *reinterpret_cast<f32x4 *>(Ks + off) = kst[i];
+            *reinterpret_cast<f32x4 *>(Vs + off) = vst[i];
+        }
+    };
+
+    f32x16 a0, a1;   // dQ^T rows d = 2m + {0,1}
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { a0[i] = 0.f; a1[i] = 0.f; }
+
+    if (ntiles > 0) { load_tile(0); store_tile(0); }
+    __syncthreads();
+
+    const int row_lds = ln * LSTR + half * 32;        // row-fragment base (S^T and dP^T products)
+    const int col_lds = (4 * half) * LSTR + 2 * ln;   // transposed-fragment base (dQ^T product)
+    const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
+
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        const bool more = (t + 1 < ntiles);
+        if (more) load_tile(t + 1);
+        const int k0 = t * BN;
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk];
+        if (k0 < wkend) {
+            f32x16 p = masked_scores<KIND>(Ks + buf * TILE_FLOATS + row_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p[r] = fast_exp2(p[r] - m_i) * rl_i;                   // the forward pass's weights
+            const f32x16 dp = tile_product(Vs + buf * TILE_FLOATS + row_lds, gr);               // dP^T = V . dout^T
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p[r] = p[r] * (dp[r] - D_i);                           // dS^T
+            tile_accumulate_t(Ks + buf * TILE_FLOATS + col_lds, p, a0, a1);                     // dQ^T += K^T . dS^T
+        }
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+    if (qi < Lq) store_row_t(dq + q_base + (long long)qi * rs + 8 * half, a0, a1, rT);
+}
+
+// ------------------------------------------------------------------------------------------------ dK, dV
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
+                                                                const float *__restrict__ v, const float *__restrict__ dout,
+                                                                const float *__restrict__ stats, const float *__restrict__ D,
+                                                                float *__restrict__ dk, float *__restrict__ dv, int H, int Lq,
+                                                                int Lk, float rT, MaskArgs mask, int strict, int nkb,
+                                                                int total_blocks, int lpt, int token_major) {
+    extern __shared__ __align__(16) float lds[];
+    float *Qs = lds;                       // [2][BN][LSTR]  q * rT * log2(e)
+    float *Gs = lds + 2 * TILE_FLOATS;     // [2][BN][LSTR]  dout
+    float *Ss = lds + 4 * TILE_FLOATS;     // per query tile: [2][32] reference maxima, [2][32] 1 / row sums, [2][32] D
+    int bh, unit;
+    if (!work_item(nkb, total_blocks, lpt, bh, unit)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int kb = unit;                 // under a causal mask the first key block meets the most queries: longest first
+    const int kw0 = kb * BM + wave * 32; // first key of this wavefront
+    const int key = kw0 + ln;
+    const int keyc = key < Lk ? key : Lk - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * HD : HD;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+
+    // Query tiles this workgroup / wavefront has to visit: under a causal mask only queries at or after its first key;
+    // keys at or beyond the valid length have weight 0 everywhere.  Same exactness conditions as the forward pass.
+    const int nqt = (Lq + 31) / 32;
+    int t_begin = 0, wt_begin = 0;
+    bool wave_active = true;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) { t_begin = (kb * BM) / 32; wt_begin = kw0 / 32; }
+        if (LENS) {
+            if (kb * BM >= len) t_begin = nqt;
+            if (kw0 >= len) wave_active = false;
+        }
+    }
+
+    float kr[32], vr[32];   // the lane's key and value rows (columns half*32 ..)
+    {
+        const float *kp = k + kv_base + (long long)keyc * rs + half * 32;
+        const float *vp = v + kv_base + (long long)keyc * rs + half * 32;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const f32x4 a = *reinterpret_cast<const f32x4 *>(kp + 4 * j);
+            const f32x4 c = *reinterpret_cast<const f32x4 *>(vp + 4 * j);
+            kr[4 * j + 0] = a.x; kr[4 * j + 1] = a.y; kr[4 * j + 2] = a.z; kr[4 * j + 3] = a.w;
+            vr[4 * j + 0] = c.x; vr[4 * j + 1] = c.y; vr[4 * j + 2] = c.z; vr[4 * j + 3] = c.w;
+        }
+    }
+
+    // staging of one query tile: q (scaled when it is written to LDS), dout, and the tile's row statistics.  Rows at or
+    // beyond Lq read as zeros; their reciprocal row sum is taken as 0, which makes their weights 0.
+    const int ld_row = tid >> 4, ld_col = (tid & 15) * 4;
+    const int q_bytes = (int)(((long long)(Lq - 1) * rs + HD) * 4);
+    const __amdgpu_buffer_rsrc_t qrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(q + q_base), 0, q_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t grsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(dout + q_base), 0, q_bytes, 0x00020000);
+    const unsigned ld_off0 = (unsigned)(ld_row * rs + ld_col) * 4u;
+    const unsigned ld_off1 = ld_off0 + 16u * rs * 4u;
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 qst[2], gst[2];
+    float sst = 0.f;
+    auto load_tile = [&](int t) {
+        const int o0 = (int)(ld_off0 + t * tile_bytes), o1 = (int)(ld_off1 + t * tile_bytes);
+        qst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(qrsrc, o0, 0, 0));
+        gst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(grsrc, o0, 0, 0));
+        qst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(qrsrc, o1, 0, 0));
+        gst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(grsrc, o1, 0, 0));
+        if (tid < 96) {      // threads 0..31: reference maximum, 32..63: 1 / row sum, 64..95: D
+            const int row = t * 32 + (tid & 31);
+            const long long at = (long long)bh * Lq + row;
+            sst = 0.f;
+            if (row < Lq) sst = tid < 32 ? stats[2 * at] : (tid < 64 ? stats[2 * at + 1] : D[at]);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int off = buf * TILE_FLOATS + (i * 16 + ld_row) * LSTR + ld_col;
+            f32x4 s;
+            s.x = (qst[i].x * rT) * LOG2E; s.y = (qst[i].y * rT) * LOG2E;
+            s.z = (qst[i].z * rT) * LOG2E; s.w = (qst[i].w * rT) * LOG2E;
+            *reinterpret_cast<f32x4 *>(Qs + off) = s;
+            *reinterpret_cast<f32x4 *>(Gs + off) = gst[i];
+        }
+        if (tid < 96) Ss[(tid >> 5) * 64 + buf * 32 + (tid & 31)] = sst;
+    };
+
+    f32x16 k0a, k1a, v0a, v1a;   // dK^T and dV^T rows d = 2m + {0,1}
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { k0a[i] = 0.f; k1a[i] = 0.f; v0a[i] = 0.f; v1a[i] = 0.f; }
+
+    if (t_begin < nqt) { load_tile(t_begin); store_tile(0); }
+    __syncthreads();
+
+    const int row_lds = ln * LSTR + half * 32;
+    const int col_lds = (4 * half) * LSTR + 2 * ln;
+    const float PEN = __fmul_rn(1e9f, LOG2E);
+    const unsigned char *cls_col = nullptr;
+    if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
+    const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
+
+    for (int t = t_begin; t < nqt; ++t) {
+        const int buf = (t - t_begin) & 1;
+        const bool more = (t + 1 < nqt);
+        if (more) load_tile(t + 1);
+        const int qt0 = t * 32;
+        int cls = 2;
+        if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq];
+        if (wave_active && t >= wt_begin) {
+            // S[query, key] in the base-2 domain: rows = the tile's queries 8(r/4) + 4*half + r%4, column = the lane's key
+            f32x16 p = tile_product(Qs + buf * TILE_FLOATS + row_lds, kr);
+            if (DENSE) {
+                if (cls == 1) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[r] = __fsub_rn(p[r], PEN);
+                } else if (cls == 2) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        const int qc = qg < Lq ? qg : Lq - 1;
+                        p[r] = __fsub_rn(p[r], __fmul_rn(__fmul_rn(mcol[qc * mask.sq], 1e9f), LOG2E));
+                    }
+                }
+            } else if ((CAUSAL && (kw0 + 31 > qt0)) || (LENS && (kw0 + 32 > len))) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    bool blocked = false;
+                    if (CAUSAL) blocked = blocked || (key > qg);
+                    if (LENS) blocked = blocked || (key >= len);
+                    if (blocked) p[r] = __fsub_rn(p[r], PEN);
+                }
+            }
+            const float *st = Ss + buf * 32 + 4 * half;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 m4 = *reinterpret_cast<const f32x4 *>(st + 8 * g);
+                const f32x4 r4 = *reinterpret_cast<const f32x4 *>(st + 64 + 8 * g);
+                p[4 * g + 0] = fast_exp2(p[4 * g + 0] - m4.x) * r4.x;
+                p[4 * g + 1] = fast_exp2(p[4 * g + 1] - m4.y) * r4.y;
+                p[4 * g + 2] = fast_exp2(p[4 * g + 2] - m4.z) * r4.z;
+                p[4 * g + 3] = fast_exp2(p[4 * g + 3] - m4.w) * r4.w;
+            }
+            tile_accumulate_t(Gs + buf * TILE_FLOATS + col_lds, p, v0a, v1a);                   // dV^T += dout^T . P
+            const f32x16 dp = tile_product(Gs + buf * TILE_FLOATS + row_lds, vr);               // dP = dout . V^T
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 d4 = *reinterpret_cast<const f32x4 *>(st + 128 + 8 * g);
+                p[4 * g + 0] = p[4 * g + 0] * (dp[4 * g + 0] - d4.x);
+                p[4 * g + 1] = p[4 * g + 1] * (dp[4 * g + 1] - d4.y);
+                p[4 * g + 2] = p[4 * g + 2] * (dp[4 * g + 2] - d4.z);
+                p[4 * g + 3] = p[4 * g + 3] * (dp[4 * g + 3] - d4.w);
+            }
+            tile_accumulate_t(Qs + buf * TILE_FLOATS + col_lds, p, k0a, k1a);                   // dK^T += Q~^T . dS
+        }
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+    if (key < Lk) {
+        store_row_t(dv + kv_base + (long long)key * rs + 8 * half, v0a, v1a, 1.0f);
+        store_row_t(dk + kv_base + (long long)key * rs + 8 * half, k0a, k1a, LN2);   // Q~ carries log2(e): dK = Q~^T dS ln 2
+    }
+}
+
+template <int KIND>
+int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
+               const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
+               int strict, int token_major) {
+    constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    static bool attr_set[8] = {false};
+    const size_t lds_dq = 4 * TILE_FLOATS * sizeof(float);
+    const size_t lds_dkv = (4 * TILE_FLOATS + 192) * sizeof(float);
+    if (!attr_set[KIND]) {
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_f32_d64<KIND>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq));
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d64<KIND>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
+        attr_set[KIND] = true;
+    }
+    {
+        const int nqb = (Lq + BM - 1) / BM;
+        const long long total = (long long)nqb * B * H;
+        DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
+        const int lpt = (causal_kind && !strict && nqb >= 2) ? 1 : 0;
+        hipLaunchKernelGGL(sdpa_bwd_dq_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq, ctx->stream, q, k,
+                           v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major);
+        const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d64");
+        if (rc != DL4S_HIP_OK) return rc;
+    }
+    {
+        const int nkb = (Lk + BM - 1) / BM;
+        const long long total = (long long)nkb * B * H;
+        DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
+        const int lpt = (causal_kind && !strict && nkb >= 2) ? 1 : 0;
+        hipLaunchKernelGGL(sdpa_bwd_dkv_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
+                           k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total, lpt, token_major);
+        return dl4s::launch_status("sdpa_bwd_dkv_f32_d64");
+    }
+}
+
+}  // namespace
+
+extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *out,
+                                     const float *stats, const float *dout, float *dq, float *dk, float *dv, int64_t B,
+                                     int64_t H, int64_t Lq, int64_t Lk, int64_t d, float inv_temperature,
+                                     const dl4s_mask_desc *mask, uint32_t flags) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(B >= 0 && H >= 0 && Lq >= 0 && Lk >= 0 && d >= 0, DL4S_HIP_EINVALID_ARG, "sdpa backward: negative extent");
+    DL4S_REQUIRE(d == HD, DL4S_HIP_EUNSUPPORTED, "sdpa backward: head dim %lld is not implemented (64 only)", (long long)d);
+    DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR | DL4S_SDPA_NO_KEY_SPLIT)) == 0, DL4S_HIP_EINVALID_ARG,
+                 "sdpa backward: unknown flag bits 0x%x", flags);
+    if (B * H == 0 || (Lq == 0 && Lk == 0)) return DL4S_HIP_OK;
+    DL4S_REQUIRE(Lk > 0, DL4S_HIP_ESHAPE, "sdpa backward: keyCount is 0");
+    DL4S_REQUIRE(k && v && dk && dv, DL4S_HIP_EINVALID_ARG, "sdpa backward: NULL tensor pointer");
+    const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
+    if (Lq == 0) {   // no queries: the keys and values receive no gradient
+        if (token_major) return dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: empty query axis in the token-major layout");
+        const int rc = dl4s_hip_fill_f32(ctx, 0.f, dk, B * H * Lk * HD);
+        return rc != DL4S_HIP_OK ? rc : dl4s_hip_fill_f32(ctx, 0.f, dv, B * H * Lk * HD);
+    }
+    DL4S_REQUIRE(q && out && stats && dout && dq, DL4S_HIP_EINVALID_ARG, "sdpa backward: NULL tensor pointer");
+    DL4S_REQUIRE(B * H * (Lq > Lk ? Lq : Lk) * HD < (1ll << 40) && Lq < (1ll << 30) && Lk < (1ll << 30), DL4S_HIP_EUNSUPPORTED,
+                 "sdpa backward: extents too large");
+    DL4S_REQUIRE((Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
+                 "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB");
+    MaskArgs m{};
+    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, true, m);
+    if (rc != DL4S_HIP_OK) return rc;
+    const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
+    void *Dv = nullptr;
+    rc = dl4s_hip_alloc(ctx, (size_t)(B * H * Lq) * sizeof(float), &Dv);
+    if (rc != DL4S_HIP_OK) return rc;
+    float *D = static_cast<float *>(Dv);
+    const long long rows = B * H * Lq;
+    hipLaunchKernelGGL(sdpa_bwd_rowdot, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, ctx->stream, out, dout, D, (int)H, (int)Lq,
+                       rows, token_major);
+    rc = dl4s::launch_status("sdpa_bwd_rowdot");
+    if (rc == DL4S_HIP_OK) {
+        switch (m.kind) {
+            case DL4S_MASK_NONE: rc = launch_bwd<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
+            case DL4S_MASK_DENSE_F32: rc = launch_bwd<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
+            case DL4S_MASK_CAUSAL: rc = launch_bwd<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
+            case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
+            default: rc = launch_bwd<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
+        }
+    }
+    const int rc2 = dl4s_hip_free(ctx, Dv);   // stream-ordered: later users of the block queue behind these kernels
+    return rc != DL4S_HIP_OK ? rc : rc2;
+}

@@ -1,0 +1,210 @@
+// Shared by the attention forward and backward kernels for gfx950 (head dim 64): tile constants, the mask
+// descriptor as the kernels see it, the dense-mask tile classifier and the masked score tile.
+#pragma once
+#include "common.h"
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int HD = 64;       // head dim of the MFMA kernel
+constexpr int BM = 128;      // queries per workgroup
+constexpr int BN = 32;       // keys per LDS tile
+constexpr int LSTR = 68;     // LDS row stride in floats: 64 + 4 keeps 128-bit reads of 8 rows on distinct banks
+constexpr int TILE_FLOATS = BN * LSTR;
+constexpr float LOG2E = 1.44269504088896340736f;
+
+struct MaskArgs {
+    int kind;
+    const float *dense;
+    long long sb, sh, sq, sk;  // element strides of the dense mask, 0 on broadcast axes
+    const int *lengths;
+    // dense masks, optional: one class per 32-query x 32-key tile (0 = all zeros, 1 = all ones, 2 = anything else),
+    // laid out [slab][q tile][k tile] with slab / tile strides 0 on the mask's broadcast axes
+    const unsigned char *cls;
+    int cls_sb, cls_sh, cls_sq, cls_sk;
+};
+
+// Classifies the 32 x 32 tiles of a dense mask so that the attention kernel only reads mask values where a tile is
+// neither all zeros nor all ones.  One wavefront per tile; elements outside [Lq, Lk] count as matching.
+__global__ __launch_bounds__(256) void sdpa_mask_classify(MaskArgs m, int MB, int MH, int nqt, int nkt, int Lq, int Lk,
+                                                          long long total, unsigned char *cls) {
+    const long long tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (tile >= total) return;
+    const int lane = threadIdx.x & 63;
+    const int kt = (int)(tile % nkt);
+    const int qt = (int)((tile / nkt) % nqt);
+    const int hm = (int)((tile / nkt / nqt) % MH);
+    const int bm = (int)(tile / nkt / nqt / MH);
+    const int col = kt * 32 + (lane & 31);
+    const int nrow = m.sq ? 32 : 1, ncol_ok = (m.sk ? col < Lk : (lane & 31) == 0);
+    bool all0 = true, all1 = true;
+    const float *base = m.dense + bm * m.sb + hm * m.sh;
+    for (int r = lane >> 5; r < nrow; r += 2) {
+        const int row = qt * 32 + r;
+        if (ncol_ok && (!m.sq || row < Lq)) {
+            const float x = base[row * m.sq + col * m.sk];
+            all0 = all0 && (x == 0.0f);
+            all1 = all1 && (x == 1.0f);
+        }
+    }
+    const int z = __all(all0), o = __all(all1);
+    if (lane == 0) cls[tile] = z ? 0 : (o ? 1 : 2);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+
+// Work order of a launch of `total_blocks` = (batch*head pairs) x `nunits` workgroups.  Workgroups are handed to the 8
+// XCDs round-robin by index, so every XCD gets one contiguous run of the pair-major order (workgroups sharing a K/V pair
+// share an L2).  Inside the run the order is pair-major by default; with `lpt` the items are handed out by ascending
+// unit -- the callers number a pair's units longest first -- so that the hardware dispatcher does
+// longest-processing-time scheduling and the launch ends on the cheapest items.  Returns false for padding workgroups.
+__device__ __forceinline__ bool work_item(const int nunits, const int total_blocks, const int lpt, int &bh, int &unit) {
+    const int chunk = (total_blocks + 7) / 8;
+    const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
+    if (w >= total_blocks) return false;
+    bh = w / nunits;
+    unit = w % nunits;
+    if (lpt) {
+        // The run is w in [a, a + n).  Item `wl` of the run in (unit ascending, w ascending) order: every unit occurs c
+        // times, the `rem` units of the cyclic interval starting at s once more.
+        const int a = (blockIdx.x % 8) * chunk;
+        const int n = min(chunk, total_blocks - a);
+        const int wl = blockIdx.x / 8;
+        const int c = n / nunits, rem = n % nunits, s = a % nunits;
+        const int wrap = s + rem - nunits;   // > 0: the interval wraps around to units [0, wrap)
+        auto before = [&](int U) {           // items with unit < U
+            const int extra = wrap > 0 ? min(U, wrap) + max(0, U - s) : min(max(U - s, 0), rem);
+            return c * U + extra;
+        };
+        int lo = 0, hi = nunits - 1;         // largest U with before(U) <= wl
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (before(mid) <= wl) lo = mid; else hi = mid - 1;
+        }
+        unit = lo;
+        const int j = wl - before(lo);
+        bh = (a + (lo - s + nunits) % nunits + j * nunits) / nunits;
+    }
+    return true;
+}
+
+// S^T = K . Q^T for one 32-key tile of one wavefront (lane = query qi = q0 + lane % 32, 16 of the 32 keys per lane:
+// accumulator register r is key k0 + 8(r/4) + 4*half + r%4), then the mask, in registers.  Kb is the lane's K fragment
+// base in LDS; qr the lane's Q fragment, already scaled by (1/T) log2(e): the scores are in the base-2 exponent domain.
+template <int KIND>
+__device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&qr)[32], const int k0, const int q0, const int qi,
+                                                const int half, const int Lk, const int len, const float *mrow,
+                                                const long long msk, const int cls) {
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+    // ---- S^T = K . Q^T for one 32-key tile
+    // (one dependent accumulation chain keeps the matrix pipe full; the first MFMA takes a literal zero)
+    f32x16 s0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
+        if (j == 0) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[0], zero, 0, 0, 0);
+        } else {
+            s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
+        }
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s0, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, qr[4 * j + 2], s0, 0, 0, 0);
+        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s0, 0, 0, 0);
+    }
+
+    // ---- mask, in registers.  Accumulator register r is key k0 + 8(r/4) + 4*half + r%4.
+    if (DENSE) {
+        if (cls == 1) {           // every element of the tile is 1: the penalty is a constant
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+        } else if (cls == 2) {    // mixed tile: read the mask values (class 0 = all zeros needs nothing)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const int kc = kg < Lk ? kg : Lk - 1;
+                s0[r] = __fsub_rn(s0[r], __fmul_rn(__fmul_rn(mrow[kc * msk], 1e9f), LOG2E));
+            }
+        }
+    } else if ((CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len))) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+            bool blocked = false;
+            if (CAUSAL) blocked = blocked || (kg > qi);
+            if (LENS) blocked = blocked || (kg >= len);
+            if (blocked) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+        }
+    }
+    if (k0 + BN > Lk) {           // keys past the end of the tensor take no part
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
+            if (kg >= Lk) s0[r] = -INFINITY;
+        }
+    }
+    return s0;
+}
+
+// Validates a mask descriptor against [B,H,Lq,Lk], fills the kernels' view of it and, for dense masks on the MFMA
+// kernels, launches the tile classifier (its result lives in the context's scratch block until the next call that uses it).
+inline int build_mask_args(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                           bool classify, MaskArgs &m) {
+    m = MaskArgs{};
+    m.kind = mask ? mask->kind : DL4S_MASK_NONE;
+    switch (m.kind) {
+        case DL4S_MASK_NONE: break;
+        case DL4S_MASK_DENSE_F32: {
+            DL4S_REQUIRE(mask->dense, DL4S_HIP_EINVALID_ARG, "sdpa: dense mask pointer is NULL");
+            const int64_t full[4] = {B, H, Lq, Lk};
+            long long stride = 1, st[4];
+            for (int i = 3; i >= 0; --i) {
+                DL4S_REQUIRE(mask->shape[i] == 1 || mask->shape[i] == full[i], DL4S_HIP_ESHAPE,
+                             "sdpa: mask axis %d has size %lld, expected 1 or %lld", i, (long long)mask->shape[i],
+                             (long long)full[i]);
+                st[i] = mask->shape[i] == 1 ? 0 : stride;
+                stride *= mask->shape[i];
+            }
+            m.dense = mask->dense;
+            m.sb = st[0]; m.sh = st[1]; m.sq = st[2]; m.sk = st[3];
+            break;
+        }
+        case DL4S_MASK_KEY_LENGTHS:
+        case DL4S_MASK_CAUSAL_OR_KEY_LENGTHS:
+            DL4S_REQUIRE(mask->lengths, DL4S_HIP_EINVALID_ARG, "sdpa: lengths pointer is NULL");
+            m.lengths = mask->lengths;
+            break;
+        case DL4S_MASK_CAUSAL: break;
+        default: return dl4s::set_error(DL4S_HIP_EINVALID_ARG, "sdpa: unknown mask kind %d", m.kind);
+    }
+    if (m.kind == DL4S_MASK_DENSE_F32 && classify) {
+        const int64_t MB = m.sb ? B : 1, MH = m.sh ? H : 1;
+        const int64_t nqt = m.sq ? (Lq + 31) / 32 : 1, nkt = m.sk ? (Lk + 31) / 32 : 1;
+        const long long total = MB * MH * nqt * nkt;
+        if (total < (1ll << 31)) {
+            const int rc = dl4s::ensure_scratch(ctx, (size_t)total);
+            if (rc != DL4S_HIP_OK) return rc;
+            unsigned char *cls = static_cast<unsigned char *>(ctx->scratch);
+            hipLaunchKernelGGL(sdpa_mask_classify, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, ctx->stream, m, (int)MB,
+                               (int)MH, (int)nqt, (int)nkt, (int)Lq, (int)Lk, total, cls);
+            const int st = dl4s::launch_status("sdpa_mask_classify");
+            if (st != DL4S_HIP_OK) return st;
+            m.cls = cls;
+            m.cls_sk = m.sk ? 1 : 0;
+            m.cls_sq = m.sq ? (int)nkt : 0;
+            m.cls_sh = m.sh ? (int)(nqt * nkt) : 0;
+            m.cls_sb = m.sb ? (int)(MH * nqt * nkt) : 0;
+        }
+    }
+    return DL4S_HIP_OK;
+}
+
+}  // namespace

@@ -18,63 +18,9 @@
 // (NN/Models/Transformer/ScaledDotProductAttention.swift:53); the mask is applied in registers as
 // s - m * 1e9 (ibid. :55-57) before the running maximum; normalisation by the row sum is deferred
 // to the end.  Keys beyond Lk contribute nothing; queries beyond Lq are computed and not stored.
-#include "common.h"
+#include "sdpa_common.h"
 
 namespace {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-constexpr int HD = 64;       // head dim of the MFMA kernel
-constexpr int BM = 128;      // queries per workgroup
-constexpr int BN = 32;       // keys per LDS tile
-constexpr int LSTR = 68;     // LDS row stride in floats: 64 + 4 keeps 128-bit reads of 8 rows on distinct banks
-constexpr int TILE_FLOATS = BN * LSTR;
-constexpr float LOG2E = 1.44269504088896340736f;
-
-struct MaskArgs {
-    int kind;
-    const float *dense;
-    long long sb, sh, sq, sk;  // element strides of the dense mask, 0 on broadcast axes
-    const int *lengths;
-    // dense masks, optional: one class per 32-query x 32-key tile (0 = all zeros, 1 = all ones, 2 = anything else),
-    // laid out [slab][q tile][k tile] with slab / tile strides 0 on the mask's broadcast axes
-    const unsigned char *cls;
-    int cls_sb, cls_sh, cls_sq, cls_sk;
-};
-
-// Classifies the 32 x 32 tiles of a dense mask so that the attention kernel only reads mask values where a tile is
-// neither all zeros nor all ones.  One wavefront per tile; elements outside [Lq, Lk] count as matching.
-__global__ __launch_bounds__(256) void sdpa_mask_classify(MaskArgs m, int MB, int MH, int nqt, int nkt, int Lq, int Lk,
-                                                          long long total, unsigned char *cls) {
-    const long long tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (tile >= total) return;
-    const int lane = threadIdx.x & 63;
-    const int kt = (int)(tile % nkt);
-    const int qt = (int)((tile / nkt) % nqt);
-    const int hm = (int)((tile / nkt / nqt) % MH);
-    const int bm = (int)(tile / nkt / nqt / MH);
-    const int col = kt * 32 + (lane & 31);
-    const int nrow = m.sq ? 32 : 1, ncol_ok = (m.sk ? col < Lk : (lane & 31) == 0);
-    bool all0 = true, all1 = true;
-    const float *base = m.dense + bm * m.sb + hm * m.sh;
-    for (int r = lane >> 5; r < nrow; r += 2) {
-        const int row = qt * 32 + r;
-        if (ncol_ok && (!m.sq || row < Lq)) {
-            const float x = base[row * m.sq + col * m.sk];
-            all0 = all0 && (x == 0.0f);
-            all1 = all1 && (x == 1.0f);
-        }
-    }
-    const int z = __all(all0), o = __all(all1);
-    if (lane == 0) cls[tile] = z ? 0 : (o ? 1 : 2);
-}
-
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-__device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
 
 // One 32-key tile for one wavefront (32 queries): S^T = K.Q^T, mask, online softmax update, O^T += V^T.P^T.
 // Kb / Vb point at the lane's K and V fragment bases of the tile in LDS; mrow is the lane's row of a dense mask
@@ -84,56 +30,7 @@ __device__ __forceinline__ void attend_tile(const float *Kb, const float *Vb, co
                                             float &m_run, float &m_use, float &l_run, const int k0, const int q0, const int qi,
                                             const int half, const int Lk, const int len, const float *mrow, const long long msk,
                                             const int cls) {
-    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
-    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
-    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
-    // ---- S^T = K . Q^T for one 32-key tile
-    // (one dependent accumulation chain keeps the matrix pipe full; the first MFMA takes a literal zero)
-    f32x16 s0;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
-        if (j == 0) {
-            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[0], zero, 0, 0, 0);
-        } else {
-            s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, qr[4 * j + 0], s0, 0, 0, 0);
-        }
-        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, qr[4 * j + 1], s0, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, qr[4 * j + 2], s0, 0, 0, 0);
-        s0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, qr[4 * j + 3], s0, 0, 0, 0);
-    }
-
-    // ---- mask, in registers.  Accumulator register r is key k0 + 8(r/4) + 4*half + r%4.
-    if (DENSE) {
-        if (cls == 1) {           // every element of the tile is 1: the penalty is a constant
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
-        } else if (cls == 2) {    // mixed tile: read the mask values (class 0 = all zeros needs nothing)
-        #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                const int kc = kg < Lk ? kg : Lk - 1;
-                s0[r] = __fsub_rn(s0[r], __fmul_rn(__fmul_rn(mrow[kc * msk], 1e9f), LOG2E));
-            }
-        }
-    } else if ((CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len))) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-            bool blocked = false;
-            if (CAUSAL) blocked = blocked || (kg > qi);
-            if (LENS) blocked = blocked || (kg >= len);
-            if (blocked) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
-        }
-    }
-    if (k0 + BN > Lk) {           // keys past the end of the tensor take no part
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
-            if (kg >= Lk) s0[r] = -INFINITY;
-        }
-    }
+    f32x16 s0 = masked_scores<KIND>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
 
     // ---- online softmax: lane (query ln) sees 16 of the 32 keys, lane ^ 32 the other 16.
     // Vector-ALU instructions do not overlap the matrix pipe on a SIMD (measured: their cycles add to the MFMA
@@ -180,44 +77,14 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
                                                                 const float *__restrict__ v,
                                                                 float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict,
-                                                                int nqb, int total_blocks, int lpt, int token_major) {
+                                                                int nqb, int total_blocks, int lpt, int token_major,
+                                                                float *__restrict__ stats) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                     // [2][BN][LSTR]
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
 
-    // Workgroups are handed to the 8 XCDs round-robin by index: give every XCD one contiguous run of
-    // the (batch*head)-major work order so that the workgroups sharing a K/V pair share an L2.
-    const int chunk = (total_blocks + 7) / 8;
-    const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
-    if (w >= total_blocks) return;
-    // Work order.  By default (batch*head)-major, so that the workgroups resident on an XCD share few K/V pairs.
-    // With causal masks (`lpt`) the items of each XCD's run are instead handed out longest first -- the latest query
-    // block of every pair in the run, then the one before, ... -- so that the hardware dispatcher does
-    // longest-processing-time scheduling and the launch ends on the cheapest blocks.
-    int bh = w / nqb;
-    int unit = w % nqb;   // 0 = the last (longest) query block of the pair
-    if (lpt) {
-        // The run is w in [a, a + n).  Item `wl` of the run in (unit ascending, w ascending) order: every unit occurs c
-        // times, the `rem` units of the cyclic interval starting at s once more.
-        const int a = (blockIdx.x % 8) * chunk;
-        const int n = min(chunk, total_blocks - a);
-        const int wl = blockIdx.x / 8;
-        const int c = n / nqb, rem = n % nqb, s = a % nqb;
-        const int wrap = s + rem - nqb;   // > 0: the interval wraps around to units [0, wrap)
-        auto before = [&](int U) {        // items with unit < U
-            const int extra = wrap > 0 ? min(U, wrap) + max(0, U - s) : min(max(U - s, 0), rem);
-            return c * U + extra;
-        };
-        int lo = 0, hi = nqb - 1;         // largest U with before(U) <= wl
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (before(mid) <= wl) lo = mid; else hi = mid - 1;
-        }
-        unit = lo;
-        const int j = wl - before(lo);
-        const int w2 = a + (lo - s + nqb) % nqb + j * nqb;
-        bh = w2 / nqb;
-    }
+    int bh, unit;   // unit 0 = the last (longest) query block of the pair
+    if (!work_item(nqb, total_blocks, lpt, bh, unit)) return;
     const int b = bh / H;
     const int hh = bh % H;
 
@@ -345,6 +212,12 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     // ---- normalise and store.  Register r of o0/o1 is d = 2*(8(r/4) + 4*half + r%4) + {0,1}.
     const float l_tot = l_run + xor32(l_run);
     const float inv = 1.0f / l_tot;
+    // row statistics for the backward pass, [B,H,Lq,2]: the reference maximum m and 1 / sum_j 2^(s_j - m), so that a weight
+    // is 2^(s - m) * that (kept apart: m can be of the order of the 1e9 mask penalty, where a float cannot also hold log2 l)
+    if (stats && half == 0 && qi < Lq) {
+        stats[2 * ((long long)bh * Lq + qi)] = m_use;
+        stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
+    }
     if (qi < Lq) {
         float *op = out + q_base + (long long)qi * rs + 8 * half;
 #pragma unroll
@@ -371,7 +244,8 @@ template <int KIND>
 __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
                                                                       const float *__restrict__ v, float *__restrict__ out,
                                                                       int H, int Lq, int Lk, float rT, MaskArgs mask,
-                                                                      int strict, int nqb, int total_blocks, int token_major) {
+                                                                      int strict, int nqb, int total_blocks, int token_major,
+                                                                      float *__restrict__ stats) {
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -513,6 +387,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
             }
         }
         const float inv = 1.0f / l_tot;
+        if (stats && half == 0 && qi < Lq) {
+            stats[2 * ((long long)bh * Lq + qi)] = m_ref;
+            stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
+        }
         if (qi < Lq) {
             float *op = out + q_base + (long long)qi * rs + 8 * half;
 #pragma unroll
@@ -595,7 +473,7 @@ __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__
 
 template <int KIND>
 int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq,
-               int Lk, float rT, const MaskArgs &m, int strict, int token_major, int no_split) {
+               int Lk, float rT, const MaskArgs &m, int strict, int token_major, int no_split, float *stats) {
     // Too few 32-query wavefronts to give every SIMD about two: split the keys of each query block over 4 wavefronts.
     // The choice depends on the extents only, so every mask kind of one problem runs the same kernel.
     const long long waves = (long long)B * H * ((Lq + 31) / 32);
@@ -611,7 +489,7 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
             split_attr_set[KIND] = true;
         }
         hipLaunchKernelGGL(sdpa_prefill_split_f32_d64<KIND>, dim3((unsigned)((total32 + 7) / 8 * 8)), dim3(256), lds_split,
-                           ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major);
+                           ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major, stats);
         return dl4s::launch_status("sdpa_prefill_split_f32_d64");
     }
     const int nqb = (Lq + BM - 1) / BM;
@@ -632,16 +510,17 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         attr_set[KIND] = true;
     }
     hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
-                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major);
+                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats);
     return dl4s::launch_status("sdpa_prefill_f32_d64");
 }
 
 }  // namespace
 
-extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
-                                     int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
-                                     float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
+namespace {
+int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, float *stats, int64_t B, int64_t H,
+                 int64_t Lq, int64_t Lk, int64_t dk, int64_t dv, float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
     DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(!stats || (dk == HD && dv == HD), DL4S_HIP_EUNSUPPORTED, "sdpa: row statistics need head dims of 64");
     DL4S_REQUIRE(B >= 0 && H >= 0 && Lq >= 0 && Lk >= 0 && dk >= 0 && dv >= 0, DL4S_HIP_EINVALID_ARG,
                  "sdpa: negative extent");
     if (B * H * Lq * dv == 0) return DL4S_HIP_OK;  // nothing to write
@@ -651,50 +530,9 @@ extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     DL4S_REQUIRE(B * H * (Lq > Lk ? Lq : Lk) * (dk > dv ? dk : dv) < (1ll << 40) && Lq < (1ll << 30) && Lk < (1ll << 30),
                  DL4S_HIP_EUNSUPPORTED, "sdpa: extents too large");
     MaskArgs m{};
-    m.kind = mask ? mask->kind : DL4S_MASK_NONE;
-    switch (m.kind) {
-        case DL4S_MASK_NONE: break;
-        case DL4S_MASK_DENSE_F32: {
-            DL4S_REQUIRE(mask->dense, DL4S_HIP_EINVALID_ARG, "sdpa: dense mask pointer is NULL");
-            const int64_t full[4] = {B, H, Lq, Lk};
-            long long stride = 1, st[4];
-            for (int i = 3; i >= 0; --i) {
-                DL4S_REQUIRE(mask->shape[i] == 1 || mask->shape[i] == full[i], DL4S_HIP_ESHAPE,
-                             "sdpa: mask axis %d has size %lld, expected 1 or %lld", i, (long long)mask->shape[i],
-                             (long long)full[i]);
-                st[i] = mask->shape[i] == 1 ? 0 : stride;
-                stride *= mask->shape[i];
-            }
-            m.dense = mask->dense;
-            m.sb = st[0]; m.sh = st[1]; m.sq = st[2]; m.sk = st[3];
-            break;
-        }
-        case DL4S_MASK_KEY_LENGTHS:
-        case DL4S_MASK_CAUSAL_OR_KEY_LENGTHS:
-            DL4S_REQUIRE(mask->lengths, DL4S_HIP_EINVALID_ARG, "sdpa: lengths pointer is NULL");
-            m.lengths = mask->lengths;
-            break;
-        case DL4S_MASK_CAUSAL: break;
-        default: return dl4s::set_error(DL4S_HIP_EINVALID_ARG, "sdpa: unknown mask kind %d", m.kind);
-    }
-    if (m.kind == DL4S_MASK_DENSE_F32 && dk == HD && dv == HD) {
-        const int64_t MB = m.sb ? B : 1, MH = m.sh ? H : 1;
-        const int64_t nqt = m.sq ? (Lq + 31) / 32 : 1, nkt = m.sk ? (Lk + 31) / 32 : 1;
-        const long long total = MB * MH * nqt * nkt;
-        if (total < (1ll << 31)) {
-            const int rc = dl4s::ensure_scratch(ctx, (size_t)total);
-            if (rc != DL4S_HIP_OK) return rc;
-            unsigned char *cls = static_cast<unsigned char *>(ctx->scratch);
-            hipLaunchKernelGGL(sdpa_mask_classify, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, ctx->stream, m, (int)MB,
-                               (int)MH, (int)nqt, (int)nkt, (int)Lq, (int)Lk, total, cls);
-            const int st = dl4s::launch_status("sdpa_mask_classify");
-            if (st != DL4S_HIP_OK) return st;
-            m.cls = cls;
-            m.cls_sk = m.sk ? 1 : 0;
-            m.cls_sq = m.sq ? (int)nkt : 0;
-            m.cls_sh = m.sh ? (int)(nqt * nkt) : 0;
-            m.cls_sb = m.sb ? (int)(MH * nqt * nkt) : 0;
-        }
+    {
+        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, dk == HD && dv == HD, m);
+        if (rc != DL4S_HIP_OK) return rc;
     }
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
@@ -706,11 +544,11 @@ extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
         DL4S_REQUIRE(Lk * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
                      "sdpa: the K/V rows of one (batch, head) pair span more than 2 GiB");
         switch (m.kind) {
-            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
-            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
-            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
-            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
-            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split);
+            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
+            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
+            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
+            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
+            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
         }
     }
     DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs head dims of 64");
@@ -721,4 +559,18 @@ extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     hipLaunchKernelGGL(sdpa_generic_f32, dim3((unsigned)rows), dim3(64), 0, ctx->stream, q, k, v, out, (int)H, (int)Lq,
                        (int)Lk, (int)dk, (int)dv, inv_temperature, m);
     return dl4s::launch_status("sdpa_generic_f32");
+}
+}  // namespace
+
+extern "C" int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
+                                     int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
+                                     float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
+    return sdpa_forward(ctx, q, k, v, out, nullptr, B, H, Lq, Lk, dk, dv, inv_temperature, mask, flags);
+}
+
+extern "C" int dl4s_hip_sdpa_fwd_stats_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
+                                           float *stats, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t d,
+                                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
+    DL4S_REQUIRE(stats || B * H * Lq == 0, DL4S_HIP_EINVALID_ARG, "sdpa: stats pointer is NULL");
+    return sdpa_forward(ctx, q, k, v, out, stats, B, H, Lq, Lk, d, d, inv_temperature, mask, flags);
 }

@@ -147,6 +147,18 @@ class Context:
                                               _i64(Lq), _i64(Lk), _i64(dk), _i64(dv), C.c_float(inv_temperature),
                                               C.byref(mask) if mask is not None else None, C.c_uint32(flags)))
 
+    def sdpa_fwd_stats(self, q, k, v, out, stats, B, H, Lq, Lk, d, inv_temperature, mask=None, flags=0):
+        _check(self.lib.dl4s_hip_sdpa_fwd_stats_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(k)), _vp(_ptr(v)), _vp(_ptr(out)),
+                                                    _vp(_ptr(stats)), _i64(B), _i64(H), _i64(Lq), _i64(Lk), _i64(d),
+                                                    C.c_float(inv_temperature), C.byref(mask) if mask is not None else None,
+                                                    C.c_uint32(flags)))
+
+    def sdpa_bwd(self, q, k, v, out, stats, dout, dq, dk, dv, B, H, Lq, Lk, d, inv_temperature, mask=None, flags=0):
+        _check(self.lib.dl4s_hip_sdpa_bwd_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(k)), _vp(_ptr(v)), _vp(_ptr(out)), _vp(_ptr(stats)),
+                                              _vp(_ptr(dout)), _vp(_ptr(dq)), _vp(_ptr(dk)), _vp(_ptr(dv)), _i64(B), _i64(H), _i64(Lq),
+                                              _i64(Lk), _i64(d), C.c_float(inv_temperature),
+                                              C.byref(mask) if mask is not None else None, C.c_uint32(flags)))
+
     def sdpa_decode(self, q, kcache, vcache, out, B, H, T, Tcap, d, inv_temperature):
         _check(self.lib.dl4s_hip_sdpa_decode_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(kcache)), _vp(_ptr(vcache)), _vp(_ptr(out)),
                                                  _i64(B), _i64(H), _i64(T), _i64(Tcap), _i64(d), C.c_float(inv_temperature)))

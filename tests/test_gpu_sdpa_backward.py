@@ -1,0 +1,152 @@
+"""Gradients of the fused attention (dl4s_hip_sdpa_fwd_stats_f32 + dl4s_hip_sdpa_bwd_f32) against the CPU oracle's
+restatement of the reference's reverse-mode closures.  Gate: |gpu - oracle| <= 1e-4 + 1e-4 |oracle|."""
+import numpy as np
+import pytest
+
+from helpers import assert_parity, causal_mask, lengths_mask
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from dl4s_amd import lib
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+def rand(rng, *shape, scale=1.0):
+    return (rng.standard_normal(shape) * scale).astype(np.float32)
+
+
+def run_fwd_bwd(ctx, q, k, v, dout, mask=None, kind=None, lens=None, strict=False, token_major=False):
+    """Returns (out, stats, dq, dk, dv) in [B,H,L,64] order whatever layout the kernels were given."""
+    from dl4s_amd import lib
+    B, H, Lq, d = q.shape
+    Lk = k.shape[2]
+    tm = (lambda x: np.ascontiguousarray(x.transpose(0, 2, 1, 3))) if token_major else (lambda x: x)
+    back = (lambda x, L: np.ascontiguousarray(x.reshape(B, L, H, d).transpose(0, 2, 1, 3))) if token_major else (lambda x, L: x)
+    bufs = [ctx.to_device(tm(x)) for x in (q, k, v, dout)]
+    dq_, dk_, dv_, out, stats = ctx.empty((B, H, Lq, d)), ctx.empty((B, H, Lk, d)), ctx.empty((B, H, Lk, d)), ctx.empty((B, H, Lq, d)), ctx.empty((B, H, Lq, 2))
+    desc, extra = None, []
+    if kind is None:
+        kind = lib.MASK_NONE if mask is None else lib.MASK_DENSE
+    if kind == lib.MASK_DENSE:
+        extra.append(ctx.to_device(mask))
+        desc = ctx.mask_desc(lib.MASK_DENSE, dense=extra[0])
+    elif kind in (lib.MASK_KEY_LENGTHS, lib.MASK_CAUSAL_OR_KEY_LENGTHS):
+        extra.append(ctx.to_device(np.asarray(lens, np.int32), dtype=np.int32))
+        desc = ctx.mask_desc(kind, lengths=extra[0])
+    elif kind == lib.MASK_CAUSAL:
+        desc = ctx.mask_desc(lib.MASK_CAUSAL)
+    flags = (lib.SDPA_STRICT if strict else 0) | (lib.SDPA_TOKEN_MAJOR if token_major else 0)
+    ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], out, stats, B, H, Lq, Lk, d, 0.125, desc, flags)
+    ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], out, stats, bufs[3], dq_, dk_, dv_, B, H, Lq, Lk, d, 0.125, desc, flags)
+    res = (back(out.numpy(), Lq), stats.numpy(), back(dq_.numpy(), Lq), back(dk_.numpy(), Lk), back(dv_.numpy(), Lk))
+    for b in bufs + [dq_, dk_, dv_, out, stats] + extra:
+        b.release()
+    return res
+
+
+SHAPES = [(1, 2, 5, 7), (2, 3, 130, 70), (1, 2, 128, 128), (2, 2, 100, 300), (1, 3, 257, 257)]
+
+
+@pytest.mark.parametrize("B,H,Lq,Lk", SHAPES)
+@pytest.mark.parametrize("mask_kind", ["none", "dense", "lengths", "causal", "causal_lengths"])
+def test_gradients_match_the_oracle(ctx, orc, B, H, Lq, Lk, mask_kind):
+    from dl4s_amd import lib
+    if mask_kind.startswith("causal") and Lq != Lk:
+        pytest.skip("causal masks are square here")
+    rng = np.random.default_rng(Lq * 7 + Lk)
+    q, k, v, dout = rand(rng, B, H, Lq, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lq, 64)
+    lens = rng.integers(1, Lk + 1, size=B)
+    kw, mask = {}, None
+    if mask_kind == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.3).astype(np.float32)
+        mask[0, 0, Lq // 2, :] = 1.0          # one fully blocked row: uniform weights
+        kw = dict(mask=mask)
+    elif mask_kind == "lengths":
+        mask, kw = lengths_mask(lens, Lk), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    elif mask_kind == "causal":
+        mask, kw = causal_mask(Lq, Lq), dict(kind=lib.MASK_CAUSAL)
+    elif mask_kind == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lq)[None, None])
+        kw = dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens)
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, **kw)
+    assert_parity(out, orc.sdpa(q, k, v, mask), "forward with stats")
+    rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+    assert_parity(dq, rq, "dq %s" % mask_kind)
+    assert_parity(dk, rk, "dk %s" % mask_kind)
+    assert_parity(dv, rv, "dv %s" % mask_kind)
+    if mask_kind not in ("none", "dense"):
+        # the structured descriptor gives the bits of the dense mask it stands for (strict visits the same tiles),
+        # and the token-major layout the bits of the head-major one
+        dense = run_fwd_bwd(ctx, q, k, v, dout, mask=mask)
+        strict = run_fwd_bwd(ctx, q, k, v, dout, strict=True, **kw)
+        for a, b_ in zip(dense, strict):
+            assert np.array_equal(a, b_)
+        for a, b_ in zip(strict[2:], (dq, dk, dv)):
+            assert_parity(b_, a, "tile skipping")
+    tm = run_fwd_bwd(ctx, q, k, v, dout, token_major=True, **kw)
+    for a, b_ in zip(tm, (out, stats, dq, dk, dv)):
+        assert np.array_equal(a, b_)
+
+
+def test_forward_with_stats_is_the_plain_forward_and_stats_give_log_sum_exp(ctx):
+    from dl4s_amd import lib
+    from oracle import fp64_model as m64
+    import scipy.special
+    rng = np.random.default_rng(3)
+    B, H, L = 2, 2, 200
+    q, k, v = rand(rng, B, H, L, 64), rand(rng, B, H, L, 64), rand(rng, B, H, L, 64)
+    out, stats, *_ = run_fwd_bwd(ctx, q, k, v, np.zeros_like(q), kind=lib.MASK_CAUSAL)
+    dq_, dk_, dv_, o2 = ctx.to_device(q), ctx.to_device(k), ctx.to_device(v), ctx.empty(q.shape)
+    ctx.sdpa_fwd(dq_, dk_, dv_, o2, B, H, L, L, 64, 64, 0.125, ctx.mask_desc(lib.MASK_CAUSAL), 0)
+    assert np.array_equal(out, o2.numpy())
+    s = np.matmul(q.astype(np.float64), k.astype(np.float64).transpose(0, 1, 3, 2)) / 8.0 - causal_mask(L, L) * 1e9
+    lse2 = scipy.special.logsumexp(s, axis=-1) / np.log(2.0)
+    assert np.allclose(stats[..., 0] - np.log2(stats[..., 1]), lse2, atol=1e-4)      # (m, 1/l): m + log2 l = log2 sum 2^s
+    for b in (dq_, dk_, dv_, o2):
+        b.release()
+
+
+def test_zero_upstream_gradient_gives_zero_gradients(ctx):
+    rng = np.random.default_rng(4)
+    q, k, v = rand(rng, 1, 2, 70, 64), rand(rng, 1, 2, 90, 64), rand(rng, 1, 2, 90, 64)
+    _, _, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, np.zeros_like(q))
+    assert not dq.any() and not dk.any() and not dv.any()
+
+
+def test_config4_sized_gradients(ctx, orc):
+    """B8 H16 L2048 d64 causal: two (batch, head) slices against the oracle, and on every slice the identities that hold
+    whatever the inputs: sum over keys of dv = sum over queries of dout (every row's weights sum to 1), and
+    <q, dq> = <k, dk> (the scores are bilinear in q and k)."""
+    from dl4s_amd import lib
+    B, H, L = 8, 16, 2048
+    rng = np.random.Generator(np.random.PCG64(1004))
+    q, k, v = (rng.standard_normal((B, H, L, 64), dtype=np.float32) * np.float32(0.5) for _ in range(3))
+    dout = rng.standard_normal((B, H, L, 64), dtype=np.float32)
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, kind=lib.MASK_CAUSAL)
+    assert np.isfinite(dq).all() and np.isfinite(dk).all() and np.isfinite(dv).all()
+    assert np.allclose(dv.astype(np.float64).sum(2), dout.astype(np.float64).sum(2), atol=2e-3)
+    a = (q.astype(np.float64) * dq).sum((2, 3))
+    b_ = (k.astype(np.float64) * dk).sum((2, 3))
+    assert np.allclose(a, b_, rtol=1e-4, atol=1e-3)
+    m = causal_mask(L, L)
+    for (b, h) in [(0, 0), (5, 11)]:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        rq, rk, rv = orc.sdpa_backward(q[sl], k[sl], v[sl], m, dout[sl])
+        assert_parity(dq[sl], rq, "config 4 dq")
+        assert_parity(dk[sl], rk, "config 4 dk")
+        assert_parity(dv[sl], rv, "config 4 dv")
+
+
+def test_backward_argument_errors(ctx):
+    from dl4s_amd import lib
+    a = ctx.empty((1, 1, 4, 8))
+    with pytest.raises(lib.Dl4sHipError):       # head dim other than 64
+        ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5)
+    with pytest.raises(lib.Dl4sHipError):
+        ctx.sdpa_fwd_stats(a, a, a, a, a, 1, 1, 4, 4, 8, 0.5)
+    a.release()
