@@ -171,6 +171,38 @@ def other_configs(ctx, lib, cpu):
         res["config3_encoder_block_B8_L1024_D1024_H16_F4096_fused"]["cpu_baseline"] = {
             "tflops": fl1 / dt / 1e12, "cores": 1, "kind": "port",
             "sample": "one batch item cut to 256 tokens (%.1f s); extrapolated whole call %.0f s" % (dt, dt * fl / fl1)}
+    # gradients of the headline workload (config 4 shapes): forward with row statistics, then dq, dk, dv
+    B, H, L = 8, 16, 2048
+    rng = np.random.Generator(np.random.PCG64(1004))
+    bufs = [ctx.to_device(rng.standard_normal((B, H, L, 64), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
+    outs = [ctx.empty((B, H, L, 64)) for _ in range(4)]
+    st = ctx.empty((B, H, L, 2))
+    desc = ctx.mask_desc(lib.MASK_CAUSAL)
+    ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], outs[0], st, B, H, L, L, 64, 0.125, desc, 0)
+    bwd = lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, 64, 0.125, desc, 0)
+    for _ in range(20):
+        bwd()
+    ctx.sync()
+    ctx.timer_begin()
+    for _ in range(20):
+        bwd()
+    ms = ctx.timer_end() / 20
+    fl = 10.0 * 64 * B * H * (L * (L + 1) // 2)          # five products: dv, dp, dq, dk and the recomputed scores
+    res["config4_attention_backward_B8_H16_L2048_causal"] = {
+        "us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
+        "note": "algorithmic flops = 5 products; the two deterministic kernels issue 7 (scores and dp are formed in both)"}
+    if cpu:
+        from oracle import binding as orc
+        hq, hk, hv, hg = (b_.numpy()[:1, :2] for b_ in bufs)
+        i, j = np.indices((L, L))
+        t0 = time.perf_counter()
+        orc.sdpa_backward(hq, hk, hv, (j > i).astype(np.float32), hg)
+        dt = time.perf_counter() - t0
+        res["config4_attention_backward_B8_H16_L2048_causal"]["cpu_baseline"] = {
+            "tflops": fl * 2 / (B * H) / dt / 1e12, "cores": 1, "kind": "port",
+            "sample": "2 of 128 (batch, head) slices, dense causal mask (%.1f s)" % dt}
+    for b_ in bufs + outs + [st]:
+        b_.release()
     # the caller of the blocks: Transformer greedy decoding (batch 1; every step re-runs the decoder on the prefix, as the
     # reference does).  6 + 6 layers, hidden 512, 8 heads of 64, ffn 2048, vocabulary 8000, 64 source tokens, 32 generated.
     rng = np.random.Generator(np.random.PCG64(1006))
