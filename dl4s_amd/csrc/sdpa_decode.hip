@@ -94,7 +94,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
             const int kc = key < T ? key : T - 1;
             const float *kp = kcache + base + (long long)kc * HD;
             if (APPEND) kp = (kc == pos) ? kn_row : kp;
-            kk[i] = *reinterpret_cast<const f32x4 *>(kp);
+            kk[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(kp));
         }
 #pragma unroll
         for (int i = 0; i < KB / 4; ++i) {
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
             const int kc = key < T ? key : T - 1;
             const float *vp = vcache + base + (long long)kc * HD;
             if (APPEND) vp = (kc == pos) ? vn_row : vp;
-            vv[i] = *reinterpret_cast<const f32x4 *>(vp);
+            vv[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(vp));
         }
         float s[KB / 4];
         float bm = -INFINITY;
