@@ -555,6 +555,96 @@ class Tensor {
     }
 };
 
+// ---- Tensor: Codable (Tensor/TensorExt.swift:241-271) in the form Foundation's JSONEncoder gives it: an object with
+// "requiresGradient" (Bool), "shape" ([Int]) and "data" (the elements' bytes, little-endian fp32, base64 - the encoder's
+// default Data strategy).  Both directions go through Device.Memory.assign, like the reference.
+namespace codable {
+inline std::string base64(const unsigned char *p, size_t n) {
+    static const char *tbl = "ABCDEFGHIJKLMNOPQRSTUVWXYZabcdefghijklmnopqrstuvwxyz0123456789+/";
+    std::string out;
+    out.reserve((n + 2) / 3 * 4);
+    for (size_t i = 0; i < n; i += 3) {
+        const unsigned v = (p[i] << 16) | ((i + 1 < n ? p[i + 1] : 0) << 8) | (i + 2 < n ? p[i + 2] : 0);
+        out += tbl[(v >> 18) & 63];
+        out += tbl[(v >> 12) & 63];
+        out += i + 1 < n ? tbl[(v >> 6) & 63] : '=';
+        out += i + 2 < n ? tbl[v & 63] : '=';
+    }
+    return out;
+}
+inline std::vector<unsigned char> unbase64(const std::string &s) {
+    auto val = [](char c) -> int {
+        if (c >= 'A' && c <= 'Z') return c - 'A';
+        if (c >= 'a' && c <= 'z') return c - 'a' + 26;
+        if (c >= '0' && c <= '9') return c - '0' + 52;
+        if (c == '+') return 62;
+        if (c == '/') return 63;
+        return -1;
+    };
+    std::vector<unsigned char> out;
+    unsigned acc = 0;
+    int bits = 0;
+    for (char c : s) {
+        if (c == '=' || c == '\\') continue;       // padding; JSON may escape '/' as "\/"
+        const int v = val(c);
+        precondition(v >= 0, "The data couldn't be read because it isn't in the correct format.");
+        acc = (acc << 6) | (unsigned)v;
+        bits += 6;
+        if (bits >= 8) {
+            bits -= 8;
+            out.push_back((unsigned char)((acc >> bits) & 0xff));
+        }
+    }
+    return out;
+}
+// position just after `"key"` and the following colon, or npos
+inline size_t find_key(const std::string &json, const char *key) {
+    const std::string k = std::string("\"") + key + "\"";
+    size_t at = json.find(k);
+    if (at == std::string::npos) return at;
+    at = json.find(':', at + k.size());
+    return at == std::string::npos ? at : at + 1;
+}
+}  // namespace codable
+
+inline std::string encodeJSON(const Tensor &t, bool requiresGradient = false) {
+    const std::vector<float> e = t.elements();
+    std::string out = std::string("{\"requiresGradient\":") + (requiresGradient ? "true" : "false") + ",\"data\":\"" +
+                      codable::base64(reinterpret_cast<const unsigned char *>(e.data()), e.size() * sizeof(float)) + "\",\"shape\":[";
+    for (size_t i = 0; i < t.shape.size(); ++i) out += (i ? "," : "") + std::to_string(t.shape[i]);
+    return out + "]}";
+}
+
+inline Tensor decodeJSON(const std::string &json, bool *requiresGradient = nullptr) {
+    const char *bad = "The data couldn't be read because it is missing.";
+    size_t at = codable::find_key(json, "shape");
+    precondition(at != std::string::npos, bad);
+    at = json.find('[', at);
+    const size_t close = json.find(']', at);
+    precondition(at != std::string::npos && close != std::string::npos, bad);
+    Shape shape;
+    for (size_t i = at + 1; i < close;) {
+        while (i < close && (json[i] == ' ' || json[i] == ',' || json[i] == '\n')) ++i;
+        if (i >= close) break;
+        size_t used = 0;
+        shape.push_back(std::stoll(json.substr(i, close - i), &used));
+        precondition(shape.back() >= 0, "negative extent");
+        i += used;
+    }
+    at = codable::find_key(json, "data");
+    precondition(at != std::string::npos, bad);
+    const size_t q0 = json.find('"', at), q1 = json.find('"', q0 + 1);
+    precondition(q0 != std::string::npos && q1 != std::string::npos, bad);
+    const std::vector<unsigned char> bytes = codable::unbase64(json.substr(q0 + 1, q1 - q0 - 1));
+    precondition((int64_t)bytes.size() == count_of(shape) * (int64_t)sizeof(float), "element count does not match shape");
+    if (requiresGradient) {
+        at = codable::find_key(json, "requiresGradient");
+        precondition(at != std::string::npos, bad);
+        *requiresGradient = json.compare(json.find_first_not_of(" \n", at), 4, "true") == 0;
+    }
+    return Tensor(reinterpret_cast<const float *>(bytes.data()), shape);
+}
+
 inline Tensor operator*(const Tensor &l, float r) { return l * Tensor(r); }
 inline Tensor operator*(float l, const Tensor &r) { return Tensor(l) * r; }
 inline Tensor operator+(const Tensor &l, float r) { return l + Tensor(r); }

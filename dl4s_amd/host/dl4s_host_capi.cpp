@@ -251,4 +251,30 @@ int dl4s_host_positional_encoding(dl4s_hip_ctx *ctx, int fused, int64_t max_len,
     });
 }
 
+int dl4s_host_tensor_encode_json(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim, char *out, size_t capacity,
+                                 size_t *needed) {
+    return guarded(ctx, 1, [&] {
+        precondition((values || dim >= 0) && dim >= 0 && dim <= DL4S_HIP_MAX_DIM && (dim == 0 || shape), "bad argument");
+        Tensor t(values, Shape(shape, shape + dim));
+        const std::string js = encodeJSON(t);
+        if (needed) *needed = js.size() + 1;
+        if (out) {
+            precondition(capacity >= js.size() + 1, "output buffer too small");
+            std::memcpy(out, js.c_str(), js.size() + 1);
+        }
+    });
+}
+
+int dl4s_host_tensor_decode_json(dl4s_hip_ctx *ctx, const char *json, float *out_values, int64_t *out_count, int64_t *out_shape,
+                                 int *out_dim) {
+    return guarded(ctx, 1, [&] {
+        precondition(json != nullptr, "bad argument");
+        Tensor t = decodeJSON(json);
+        if (out_count) *out_count = t.count();
+        if (out_dim) *out_dim = t.dim();
+        if (out_shape) std::copy(t.shape.begin(), t.shape.end(), out_shape);
+        if (out_values) HIP::Memory::assign(t.buffer(), out_values, t.count());
+    });
+}
+
 }  // extern "C"

@@ -244,3 +244,25 @@ def positional_encoding(ctx, max_len, hidden, fused=True):
     out = np.empty((max_len, hidden), np.float32)
     _check(load().dl4s_host_positional_encoding(ctx.handle, int(fused), _i64(max_len), _i64(hidden), _p(out)))
     return out
+
+
+def tensor_encode_json(ctx, values):
+    """Tensor -> the JSON text the reference's Codable conformance produces (through a device tensor)."""
+    v = np.require(values, np.float32, "C")        # keeps a 0-d array 0-d (a scalar tensor has shape [])
+    shp = (_i64 * max(1, v.ndim))(*v.shape)
+    need = C.c_size_t()
+    _check(load().dl4s_host_tensor_encode_json(ctx.handle, _p(v), shp, v.ndim, None, C.c_size_t(0), C.byref(need)))
+    buf = C.create_string_buffer(need.value)
+    _check(load().dl4s_host_tensor_encode_json(ctx.handle, _p(v), shp, v.ndim, buf, C.c_size_t(need.value), None))
+    return buf.value.decode()
+
+
+def tensor_decode_json(ctx, text):
+    """JSON text of an encoded Tensor -> numpy array (through a device tensor)."""
+    js = text.encode()
+    n, dim = _i64(), C.c_int()
+    shp = (_i64 * 8)()
+    _check(load().dl4s_host_tensor_decode_json(ctx.handle, js, None, C.byref(n), shp, C.byref(dim)))
+    out = np.empty(tuple(shp[i] for i in range(dim.value)), np.float32)
+    _check(load().dl4s_host_tensor_decode_json(ctx.handle, js, _p(out) if out.size else None, None, None, None))
+    return out

@@ -87,6 +87,15 @@ int dl4s_host_transformer_greedy(dl4s_hip_ctx *ctx, int fused, dl4s_host_transfo
 /* PositionalEncoding(hiddenSize)(maxLen) -> [maxLen, hiddenSize] -- PositionalEncoding.swift:52-69 */
 int dl4s_host_positional_encoding(dl4s_hip_ctx *ctx, int fused, int64_t max_len, int64_t hidden, float *out);
 
+/* Tensor: Codable (Tensor/TensorExt.swift:241-271) as Foundation's JSONEncoder writes it:
+ * {"requiresGradient":Bool,"data":"<base64 of the little-endian fp32 elements>","shape":[Int]}.
+ * encode: host values -> device tensor -> JSON text (out may be NULL to query *needed, which includes the NUL);
+ * decode: JSON text -> device tensor -> host values (out_values / out_shape may be NULL to query *out_count, *out_dim). */
+int dl4s_host_tensor_encode_json(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim, char *out, size_t capacity,
+                                 size_t *needed);
+int dl4s_host_tensor_decode_json(dl4s_hip_ctx *ctx, const char *json, float *out_values, int64_t *out_count, int64_t *out_shape,
+                                 int *out_dim);
+
 #ifdef __cplusplus
 }
 #endif

@@ -40,3 +40,17 @@ def test_null_context_is_rejected_not_crashed():
     assert rc == -1 and b"ctx is NULL" in l.dl4s_hip_last_error()
     rc = l.dl4s_hip_create(0, None)
     assert rc == -1
+
+
+def test_host_library_exports_every_symbol_its_header_declares():
+    from dl4s_amd import host_lib, lib
+    text = open(os.path.join(ROOT, "include", "dl4s_host.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(dl4s_host_[a-z0-9_]+)\s*\(", text)))
+    assert "dl4s_host_transformer_greedy" in declared and "dl4s_host_mha" in declared
+    ctypes.CDLL(lib.LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    so = ctypes.CDLL(host_lib.HOST_LIB_PATH)
+    missing = [s for s in declared if not hasattr(so, s)]
+    assert not missing, missing
+    # a NULL context is an error return, never a crash
+    assert so.dl4s_host_positional_encoding(None, 1, ctypes.c_int64(4), ctypes.c_int64(4), None) == -1

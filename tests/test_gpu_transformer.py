@@ -166,3 +166,27 @@ def test_transformer_argument_errors(ctx):
     with pytest.raises(host_lib.HostError):       # padded length differs from the longest sequence
         model.forward([[3, 1, -1]], [[1]], [2], [1])
     model.close()
+
+
+def test_tensor_codable_json_round_trip(ctx):
+    """Tensor: Codable (Tensor/TensorExt.swift:241-271) as JSONEncoder writes it: requiresGradient, base64 data, shape."""
+    import base64
+    import json
+    from dl4s_amd import host_lib
+    rng = np.random.default_rng(51)
+    x = rng.standard_normal((3, 5, 7)).astype(np.float32)
+    x[0, 0, 0], x[1, 2, 3] = np.inf, -0.0
+    text = host_lib.tensor_encode_json(ctx, x)
+    obj = json.loads(text)
+    assert obj["shape"] == [3, 5, 7] and obj["requiresGradient"] is False
+    assert base64.b64decode(obj["data"]) == x.tobytes()
+    assert np.array_equal(host_lib.tensor_decode_json(ctx, text), x)
+    # a document written elsewhere: other key order, whitespace, Foundation's escaped slashes
+    doc = json.dumps({"shape": [5, 21], "data": base64.b64encode(x.tobytes()).decode(), "requiresGradient": True}, indent=1)
+    doc = doc.replace("/", "\\/")
+    assert np.array_equal(host_lib.tensor_decode_json(ctx, doc), x.reshape(5, 21))
+    for bad in ('{"shape":[2,2],"data":"AAAA","requiresGradient":false}', '{"data":"AAAA"}'):
+        with pytest.raises(host_lib.HostError):
+            host_lib.tensor_decode_json(ctx, bad)
+    s = host_lib.tensor_decode_json(ctx, host_lib.tensor_encode_json(ctx, np.float32(2.5)))      # scalar: shape []
+    assert s.shape == () and s == np.float32(2.5)
