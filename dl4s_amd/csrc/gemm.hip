@@ -1,11 +1,12 @@
-// fp32 GEMM on v_mfma_f32_32x32x2_f32 for gfx950:  C = alpha * op(A) . op(B) + beta * C, row-major,
-// optional strided batch.  A workgroup (4 wavefronts, 2x2) computes a 128x128 tile of C; each
-// wavefront holds a 64x64 sub-tile as 2x2 MFMA accumulators.  K is walked in steps of 16 through
-// LDS tiles stored k-major ([k][m] and [k][n]) so that the MFMA operand reads (lane l wants row
-// l % 32 at k = l / 32) are consecutive 32-bit words, and the next K step is prefetched into
-// registers while the current one is multiplied.  Transposes are handled by the loader only: the
-// operand is addressed through (row stride, column stride), and the thread-to-element mapping is
-// chosen so that the unit-stride direction runs along the lanes.
+// fp32 GEMM on v_mfma_f32_32x32x2_f32 for gfx950:  C = alpha * op(A) . op(B) + beta * C, row-major, optional strided
+// batch, optional epilogue act(. + bias[n]) + residual[m][n] (the fused Dense forms).  A workgroup (4 wavefronts, 2x2)
+// computes a 128x128 (or 64x64) tile of C; the next K step is prefetched into registers while the current one is
+// multiplied.  Two kernels:
+//   gemm_f32_mfma      any (row stride, column stride) operands, i.e. every transpose combination: scalar loads, LDS
+//                      tiles stored k-major ([k][m] and [k][n]) so that the MFMA operand reads (lane l wants row l % 32
+//                      at k = l / 32) are consecutive 32-bit words; the thread-to-element mapping of the loader is
+//                      chosen so that the unit-stride direction runs along the lanes
+//   gemm_f32_mfma_nn   row-major A and B (the layers' products): 128-bit buffer loads, A kept [m][k] in LDS
 #include "common.h"
 
 namespace {

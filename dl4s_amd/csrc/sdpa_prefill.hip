@@ -15,9 +15,14 @@
 // therefore 16 in-lane operations plus one exchange with lane l ^ 32.
 //
 // The scale is applied to Q once (q * rT), as the reference does before its first matrix product
-// (NN/Models/Transformer/ScaledDotProductAttention.swift:53); the mask is applied in registers as
-// s - m * 1e9 (ibid. :55-57) before the running maximum; normalisation by the row sum is deferred
-// to the end.  Keys beyond Lk contribute nothing; queries beyond Lq are computed and not stored.
+// (NN/Models/Transformer/ScaledDotProductAttention.swift:53), followed by a factor log2(e) so that the scores live in
+// the base-2 exponent domain; the mask is applied in registers (the base-2 image of s - m * 1e9, ibid. :55-57) before
+// the running maximum; normalisation by the row sum is deferred to the end.  Keys beyond Lk contribute nothing;
+// queries beyond Lq are computed and not stored.
+//
+// Kernels in this file: sdpa_prefill_f32_d64 (above), sdpa_prefill_split_f32_d64 (small launches: the keys of a
+// 32-query block split over the 4 wavefronts of a workgroup), sdpa_generic_f32 (head dims other than 64).  Both MFMA
+// kernels can also leave the two row statistics the backward pass needs (sdpa_backward.hip).
 #include "sdpa_common.h"
 
 namespace {
