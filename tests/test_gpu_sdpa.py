@@ -415,3 +415,46 @@ def test_dense_mask_with_uniform_and_mixed_tiles(ctx, orc, mshape):
     assert_parity(got, ref, "dense mask tiles " + mshape)
     got_tm = run_sdpa(ctx, q, k, v, full, token_major=True)
     assert np.array_equal(got, got_tm)
+
+
+def test_tensors_beyond_2_31_elements(ctx, orc):
+    """32768 (batch, head) pairs of 1024 x 64: every tensor holds 2^31 elements (8 GiB), so any 32-bit element index in
+    the kernels or their launch arithmetic would wrap.  The tensors are filled on the device from one 64-pair block
+    (with the last pair made distinct); the first, a middle and the last pair are checked against the oracle, and the
+    output of every block of 64 pairs but the last must repeat the first block bit for bit."""
+    import ctypes as C
+    from dl4s_amd import lib
+    if NO_SPLIT_DEFAULT[0]:
+        pytest.skip("one run is enough: the launch is far beyond the key-split range")
+    B, H, L, d = 2048, 16, 1024, 64
+    blk = 64                                     # pairs per host block
+    rng = np.random.default_rng(99)
+    hq, hk, hv = (rand(rng, blk, L, d) for _ in range(3))
+    last = [rand(rng, 1, L, d) for _ in range(3)]
+    nbytes_pair = L * d * 4
+    bufs = [lib.DeviceBuffer(ctx, B * H * nbytes_pair, (B, H, L, d)) for _ in range(4)]
+    for buf, host, tail in zip(bufs, (hq, hk, hv), last):
+        for i in range(B * H // blk):
+            lib._check(ctx.lib.dl4s_hip_assign_h2d(ctx.handle, C.c_void_p(buf.offset(i * blk * nbytes_pair)),
+                                                   host.ctypes.data_as(C.c_void_p), C.c_size_t(host.nbytes)))
+        lib._check(ctx.lib.dl4s_hip_assign_h2d(ctx.handle, C.c_void_p(buf.offset((B * H - 1) * nbytes_pair)),
+                                               tail.ctypes.data_as(C.c_void_p), C.c_size_t(tail.nbytes)))
+    ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], bufs[3], B, H, L, L, d, d, 0.125, ctx.mask_desc(lib.MASK_CAUSAL), 0)
+
+    def pair(i):
+        out = np.empty((1, 1, L, d), np.float32)
+        lib._check(ctx.lib.dl4s_hip_assign_d2h(ctx.handle, out.ctypes.data_as(C.c_void_p), C.c_void_p(bufs[3].offset(i * nbytes_pair)),
+                                               C.c_size_t(out.nbytes)))
+        return out
+    m = causal_mask(L, L)
+    for i, (q_, k_, v_) in ((0, (hq[0], hk[0], hv[0])), (B * H // 2 + 5, (hq[5], hk[5], hv[5])), (B * H - 1, [t[0] for t in last])):
+        assert_parity(pair(i), orc.sdpa(q_[None, None], k_[None, None], v_[None, None], m), "pair %d of %d" % (i, B * H))
+    first = np.empty((blk, L, d), np.float32)
+    other = np.empty_like(first)
+    lib._check(ctx.lib.dl4s_hip_assign_d2h(ctx.handle, first.ctypes.data_as(C.c_void_p), C.c_void_p(bufs[3].ptr), C.c_size_t(first.nbytes)))
+    for i in (1, 255, B * H // blk - 2):
+        lib._check(ctx.lib.dl4s_hip_assign_d2h(ctx.handle, other.ctypes.data_as(C.c_void_p),
+                                               C.c_void_p(bufs[3].offset(i * blk * nbytes_pair)), C.c_size_t(other.nbytes)))
+        assert np.array_equal(first, other)
+    for b in bufs:
+        b.release()
