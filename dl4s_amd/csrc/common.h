@@ -27,6 +27,9 @@ struct dl4s_hip_ctx {
     // scratch owned by the library for split-K partial results (grown on demand, never shrunk)
     void *scratch = nullptr;
     size_t scratch_bytes = 0;
+    // Held by an entry point from the launch that fills the scratch block to the launch that reads it, so that calls
+    // from several host threads cannot interleave their use of it (the kernels themselves are ordered by the stream).
+    std::mutex scratch_mu;
 };
 
 namespace dl4s {

@@ -543,6 +543,7 @@ int dl4s_hip_argmax_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, i
     *out_value = -INFINITY;            // the reference's result for an empty buffer
     if (count == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(values, DL4S_HIP_EINVALID_ARG, "argmax: NULL pointer");
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     int rc = dl4s::ensure_scratch(ctx, 16);
     if (rc) return rc;
     float *dv = reinterpret_cast<float *>(ctx->scratch);
@@ -597,6 +598,7 @@ int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *resid
     DL4S_REQUIRE(B <= 65535, DL4S_HIP_EUNSUPPORTED, "layernorm: batch above 65535 with long rows");
     long long want = n / (TPB * 8);
     int nblk = (int)(want < 1 ? 1 : (want > 256 ? 256 : want));
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     int rc = dl4s::ensure_scratch(ctx, (size_t)B * nblk * 2 * sizeof(float));
     if (rc) return rc;
     float *part = reinterpret_cast<float *>(ctx->scratch);

@@ -434,6 +434,7 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                  "sdpa backward: extents too large");
     DL4S_REQUIRE((Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB");
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     MaskArgs m{};
     int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, true, m);
     if (rc != DL4S_HIP_OK) return rc;

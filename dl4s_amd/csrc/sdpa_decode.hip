@@ -221,7 +221,9 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     chunk = (chunk + KB - 1) / KB * KB;
     const int nsplit = (int)((T + chunk - 1) / chunk);
     float *part = nullptr;
+    std::unique_lock<std::mutex> scratch_lock(ctx->scratch_mu, std::defer_lock);
     if (nsplit > 1) {
+        scratch_lock.lock();
         int rc = dl4s::ensure_scratch(ctx, (size_t)BH * nsplit * PSTR * sizeof(float));
         if (rc) return rc;
         part = reinterpret_cast<float *>(ctx->scratch);

@@ -526,6 +526,7 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
                  int64_t Lq, int64_t Lk, int64_t dk, int64_t dv, float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
     DL4S_CHECK_CTX(ctx);
     DL4S_REQUIRE(!stats || (dk == HD && dv == HD), DL4S_HIP_EUNSUPPORTED, "sdpa: row statistics need head dims of 64");
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     DL4S_REQUIRE(B >= 0 && H >= 0 && Lq >= 0 && Lk >= 0 && dk >= 0 && dv >= 0, DL4S_HIP_EINVALID_ARG,
                  "sdpa: negative extent");
     if (B * H * Lq * dv == 0) return DL4S_HIP_OK;  // nothing to write
