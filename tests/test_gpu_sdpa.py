@@ -458,3 +458,32 @@ def test_tensors_beyond_2_31_elements(ctx, orc):
         assert np.array_equal(first, other)
     for b in bufs:
         b.release()
+
+
+def test_concurrent_callers_on_one_context(ctx, orc):
+    """Four host threads issue dense-mask attention calls (which stage mask tile classes in the context's scratch block)
+    on the same context at once; every result must be its own problem's."""
+    import threading
+    rng = np.random.default_rng(77)
+    problems = []
+    for i in range(4):
+        Lq, Lk = 96 + 32 * i, 200 - 24 * i
+        q, k, v = rand(rng, 1, 2, Lq, 64), rand(rng, 1, 2, Lk, 64), rand(rng, 1, 2, Lk, 64)
+        mask = (rng.random((1, 1, Lq, Lk)) < 0.5).astype(np.float32)
+        mask[..., : Lk // 2] = float(i % 2)          # uniform tiles of both kinds plus mixed ones
+        problems.append((q, k, v, mask, orc.sdpa(q, k, v, mask)))
+    results = [[] for _ in problems]
+
+    def work(i):
+        q, k, v, mask, _ = problems[i]
+        for _ in range(10):
+            results[i].append(run_sdpa(ctx, q, k, v, mask))
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(problems))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for i, (_, _, _, _, ref) in enumerate(problems):
+        for got in results[i]:
+            assert_parity(got, ref, "thread %d" % i)
+            assert np.array_equal(got, results[i][0])
