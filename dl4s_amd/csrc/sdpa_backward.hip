@@ -373,6 +373,118 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
     }
 }
 
+// ------------------------------------------------------------------------------------------------ other head dims
+// Plain gradient kernels for head dims other than 64 (up to 256, key dim = value dim = d), the counterpart of the plain
+// forward kernel: correctness paths for small models, one wavefront per query row (dq) and per key row (dk, dv).
+// Weights are recomputed as exp(s - mx) * inv from the statistics the plain forward kernel leaves.
+__global__ __launch_bounds__(64) void sdpa_bwd_rowdot_plain(const float *__restrict__ out, const float *__restrict__ dout,
+                                                             float *__restrict__ D, int d) {
+    const long long row = blockIdx.x;
+    float acc = 0.f;
+    for (int c = threadIdx.x; c < d; c += 64) acc += out[row * d + c] * dout[row * d + c];
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (threadIdx.x == 0) D[row] = acc;
+}
+
+__global__ __launch_bounds__(64) void sdpa_bwd_dq_plain(const float *__restrict__ q, const float *__restrict__ k,
+                                                         const float *__restrict__ v, const float *__restrict__ dout,
+                                                         const float *__restrict__ stats, const float *__restrict__ D,
+                                                         float *__restrict__ dq, int H, int Lq, int Lk, int d, float rT,
+                                                         MaskArgs mask) {
+    __shared__ float qs[GEN_MAXD], go[GEN_MAXD], ds[64];
+    const int row = blockIdx.x;   // over B*H*Lq
+    const int qi = row % Lq, bh = row / Lq, b = bh / H, hh = bh % H, lane = threadIdx.x;
+    for (int c = lane; c < d; c += 64) {
+        qs[c] = q[(long long)row * d + c] * rT;
+        go[c] = dout[(long long)row * d + c];
+    }
+    __syncthreads();
+    const float *kp = k + (long long)bh * Lk * d, *vp = v + (long long)bh * Lk * d;
+    int len = Lk;
+    if (mask.kind == DL4S_MASK_KEY_LENGTHS || mask.kind == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS) len = mask.lengths[b];
+    const float mx = stats[2 * (long long)row], inv = stats[2 * (long long)row + 1], Di = D[row];
+    float acc[GEN_MAXD / 64];
+    for (int i = 0; i < GEN_MAXD / 64; ++i) acc[i] = 0.f;
+    for (int j0 = 0; j0 < Lk; j0 += 64) {
+        const int j = j0 + lane;
+        float g = 0.f;
+        if (j < Lk) {
+            const float p = expf(plain_score(qs, kp + (long long)j * d, d, mask, b, hh, qi, j, len) - mx) * inv;
+            float dp = 0.f;
+            for (int c = 0; c < d; ++c) dp += go[c] * vp[(long long)j * d + c];
+            g = p * (dp - Di);
+        }
+        ds[lane] = g;
+        __syncthreads();
+        const int n = min(64, Lk - j0);
+        for (int i = 0; i < GEN_MAXD / 64; ++i) {
+            const int c = lane + 64 * i;
+            if (c < d)
+                for (int jj = 0; jj < n; ++jj) acc[i] += ds[jj] * kp[(long long)(j0 + jj) * d + c];
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < GEN_MAXD / 64; ++i) {
+        const int c = lane + 64 * i;
+        if (c < d) dq[(long long)row * d + c] = acc[i] * rT;
+    }
+}
+
+__global__ __launch_bounds__(64) void sdpa_bwd_dkv_plain(const float *__restrict__ q, const float *__restrict__ k,
+                                                          const float *__restrict__ v, const float *__restrict__ dout,
+                                                          const float *__restrict__ stats, const float *__restrict__ D,
+                                                          float *__restrict__ dk, float *__restrict__ dv, int H, int Lq, int Lk,
+                                                          int d, float rT, MaskArgs mask) {
+    __shared__ float kj[GEN_MAXD], vj[GEN_MAXD], ps[64], ds[64];
+    const int row = blockIdx.x;   // over B*H*Lk
+    const int j = row % Lk, bh = row / Lk, b = bh / H, hh = bh % H, lane = threadIdx.x;
+    for (int c = lane; c < d; c += 64) {
+        kj[c] = k[(long long)row * d + c];
+        vj[c] = v[(long long)row * d + c];
+    }
+    __syncthreads();
+    const float *qp = q + (long long)bh * Lq * d, *gp = dout + (long long)bh * Lq * d;
+    int len = Lk;
+    if (mask.kind == DL4S_MASK_KEY_LENGTHS || mask.kind == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS) len = mask.lengths[b];
+    float acck[GEN_MAXD / 64], accv[GEN_MAXD / 64];
+    for (int i = 0; i < GEN_MAXD / 64; ++i) { acck[i] = 0.f; accv[i] = 0.f; }
+    for (int i0 = 0; i0 < Lq; i0 += 64) {
+        const int qi = i0 + lane;
+        float p = 0.f, g = 0.f;
+        if (qi < Lq) {
+            // the score with the forward kernel's roundings: (q * rT) . k accumulated in order, then the mask
+            float s = 0.f;
+            for (int c = 0; c < d; ++c) s = __fadd_rn(s, __fmul_rn(qp[(long long)qi * d + c] * rT, kj[c]));
+            s = plain_masked(s, mask, b, hh, qi, j, len);
+            const long long r = (long long)bh * Lq + qi;
+            p = expf(s - stats[2 * r]) * stats[2 * r + 1];
+            float dp = 0.f;
+            for (int c = 0; c < d; ++c) dp += gp[(long long)qi * d + c] * vj[c];
+            g = p * (dp - D[r]);
+        }
+        ps[lane] = p;
+        ds[lane] = g;
+        __syncthreads();
+        const int n = min(64, Lq - i0);
+        for (int i = 0; i < GEN_MAXD / 64; ++i) {
+            const int c = lane + 64 * i;
+            if (c < d)
+                for (int ii = 0; ii < n; ++ii) {
+                    accv[i] += ps[ii] * gp[(long long)(i0 + ii) * d + c];
+                    acck[i] += ds[ii] * (qp[(long long)(i0 + ii) * d + c] * rT);
+                }
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < GEN_MAXD / 64; ++i) {
+        const int c = lane + 64 * i;
+        if (c < d) {
+            dv[(long long)row * d + c] = accv[i];
+            dk[(long long)row * d + c] = acck[i];
+        }
+    }
+}
+
 template <int KIND>
 int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
                const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
@@ -417,7 +529,8 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                                      const dl4s_mask_desc *mask, uint32_t flags) {
     DL4S_CHECK_CTX(ctx);
     DL4S_REQUIRE(B >= 0 && H >= 0 && Lq >= 0 && Lk >= 0 && d >= 0, DL4S_HIP_EINVALID_ARG, "sdpa backward: negative extent");
-    DL4S_REQUIRE(d == HD, DL4S_HIP_EUNSUPPORTED, "sdpa backward: head dim %lld is not implemented (64 only)", (long long)d);
+    DL4S_REQUIRE(d > 0 && d <= GEN_MAXD, DL4S_HIP_EUNSUPPORTED, "sdpa backward: head dim %lld is not implemented (1..%d)",
+                 (long long)d, GEN_MAXD);
     DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR | DL4S_SDPA_NO_KEY_SPLIT)) == 0, DL4S_HIP_EINVALID_ARG,
                  "sdpa backward: unknown flag bits 0x%x", flags);
     if (B * H == 0 || (Lq == 0 && Lk == 0)) return DL4S_HIP_OK;
@@ -426,17 +539,17 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
     if (Lq == 0) {   // no queries: the keys and values receive no gradient
         if (token_major) return dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: empty query axis in the token-major layout");
-        const int rc = dl4s_hip_fill_f32(ctx, 0.f, dk, B * H * Lk * HD);
-        return rc != DL4S_HIP_OK ? rc : dl4s_hip_fill_f32(ctx, 0.f, dv, B * H * Lk * HD);
+        const int rc = dl4s_hip_fill_f32(ctx, 0.f, dk, B * H * Lk * d);
+        return rc != DL4S_HIP_OK ? rc : dl4s_hip_fill_f32(ctx, 0.f, dv, B * H * Lk * d);
     }
     DL4S_REQUIRE(q && out && stats && dout && dq, DL4S_HIP_EINVALID_ARG, "sdpa backward: NULL tensor pointer");
-    DL4S_REQUIRE(B * H * (Lq > Lk ? Lq : Lk) * HD < (1ll << 40) && Lq < (1ll << 30) && Lk < (1ll << 30), DL4S_HIP_EUNSUPPORTED,
+    DL4S_REQUIRE(B * H * (Lq > Lk ? Lq : Lk) * d < (1ll << 40) && Lq < (1ll << 30) && Lk < (1ll << 30), DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: extents too large");
-    DL4S_REQUIRE((Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
+    DL4S_REQUIRE(d != HD || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB");
     std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     MaskArgs m{};
-    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, true, m);
+    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, d == HD, m);
     if (rc != DL4S_HIP_OK) return rc;
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     void *Dv = nullptr;
@@ -444,6 +557,21 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     if (rc != DL4S_HIP_OK) return rc;
     float *D = static_cast<float *>(Dv);
     const long long rows = B * H * Lq;
+    if (d != HD) {   // plain kernels
+        rc = DL4S_HIP_OK;
+        if (token_major) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: the token-major layout needs head dims of 64");
+        else if (rows >= (1ll << 31) || B * H * Lk >= (1ll << 31)) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: too many rows for the plain kernels");
+        if (rc == DL4S_HIP_OK) {
+            hipLaunchKernelGGL(sdpa_bwd_rowdot_plain, dim3((unsigned)rows), dim3(64), 0, ctx->stream, out, dout, D, (int)d);
+            hipLaunchKernelGGL(sdpa_bwd_dq_plain, dim3((unsigned)rows), dim3(64), 0, ctx->stream, q, k, v, dout, stats, D, dq, (int)H,
+                               (int)Lq, (int)Lk, (int)d, inv_temperature, m);
+            hipLaunchKernelGGL(sdpa_bwd_dkv_plain, dim3((unsigned)(B * H * Lk)), dim3(64), 0, ctx->stream, q, k, v, dout, stats, D, dk,
+                               dv, (int)H, (int)Lq, (int)Lk, (int)d, inv_temperature, m);
+            rc = dl4s::launch_status("sdpa_bwd_plain");
+        }
+        const int rcf = dl4s_hip_free(ctx, Dv);
+        return rc != DL4S_HIP_OK ? rc : rcf;
+    }
     hipLaunchKernelGGL(sdpa_bwd_rowdot, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, ctx->stream, out, dout, D, (int)H, (int)Lq,
                        rows, token_major);
     rc = dl4s::launch_status("sdpa_bwd_rowdot");

@@ -154,6 +154,31 @@ __device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&q
     return s0;
 }
 
+// Plain kernels (head dims other than 64).  The score of (query qi, key j) is the sequential dot product of the scaled
+// query row with the key row, then the mask, every step rounded like the reference's generic engine.
+constexpr int GEN_MAXD = 256;
+__device__ __forceinline__ float plain_masked(float s, const MaskArgs &mask, const int b, const int hh, const int qi, const int j,
+                                              const int len) {
+    switch (mask.kind) {
+        case DL4S_MASK_DENSE_F32: {
+            const float mval = mask.dense[b * mask.sb + hh * mask.sh + qi * mask.sq + j * mask.sk];
+            s = __fsub_rn(s, __fmul_rn(mval, 1e9f));
+            break;
+        }
+        case DL4S_MASK_CAUSAL: if (j > qi) s = __fsub_rn(s, 1e9f); break;
+        case DL4S_MASK_KEY_LENGTHS: if (j >= len) s = __fsub_rn(s, 1e9f); break;
+        case DL4S_MASK_CAUSAL_OR_KEY_LENGTHS: if (j > qi || j >= len) s = __fsub_rn(s, 1e9f); break;
+        default: break;
+    }
+    return s;
+}
+__device__ __forceinline__ float plain_score(const float *qs, const float *krow, const int dk, const MaskArgs &mask, const int b,
+                                             const int hh, const int qi, const int j, const int len) {
+    float s = 0.f;
+    for (int c = 0; c < dk; ++c) s = __fadd_rn(s, __fmul_rn(qs[c], krow[c]));
+    return plain_masked(s, mask, b, hh, qi, j, len);
+}
+
 // Validates a mask descriptor against [B,H,Lq,Lk], fills the kernels' view of it and, for dense masks on the MFMA
 // kernels, launches the tile classifier (its result lives in the context's scratch block until the next call that uses it).
 inline int build_mask_args(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,

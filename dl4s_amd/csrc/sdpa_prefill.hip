@@ -414,10 +414,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
 
 // Plain fused kernel for head dims other than 64 (up to 256): one wavefront per query row, two passes over
 // the keys like the reference's softmax (max, then exp / sum), keys handled 64 at a time through LDS.
-constexpr int GEN_MAXD = 256;
 __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__ q, const float *__restrict__ k,
                                                         const float *__restrict__ v, float *__restrict__ out, int H,
-                                                        int Lq, int Lk, int dk, int dv, float rT, MaskArgs mask) {
+                                                        int Lq, int Lk, int dk, int dv, float rT, MaskArgs mask,
+                                                        float *__restrict__ stats) {
     __shared__ float qs[GEN_MAXD];
     __shared__ float ps[64];
     const int row = blockIdx.x;  // over B*H*Lq
@@ -431,22 +431,7 @@ __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__
     const float *vp = v + (long long)bh * Lk * dv;
     int len = Lk;
     if (mask.kind == DL4S_MASK_KEY_LENGTHS || mask.kind == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS) len = mask.lengths[b];
-    auto score = [&](int j) {
-        float s = 0.f;
-        for (int c = 0; c < dk; ++c) s = __fadd_rn(s, __fmul_rn(qs[c], kp[(long long)j * dk + c]));
-        switch (mask.kind) {
-            case DL4S_MASK_DENSE_F32: {
-                float mval = mask.dense[b * mask.sb + hh * mask.sh + qi * mask.sq + j * mask.sk];
-                s = __fsub_rn(s, __fmul_rn(mval, 1e9f));
-                break;
-            }
-            case DL4S_MASK_CAUSAL: if (j > qi) s = __fsub_rn(s, 1e9f); break;
-            case DL4S_MASK_KEY_LENGTHS: if (j >= len) s = __fsub_rn(s, 1e9f); break;
-            case DL4S_MASK_CAUSAL_OR_KEY_LENGTHS: if (j > qi || j >= len) s = __fsub_rn(s, 1e9f); break;
-            default: break;
-        }
-        return s;
-    };
+    auto score = [&](int j) { return plain_score(qs, kp + (long long)j * dk, dk, mask, b, hh, qi, j, len); };
     float mx = -INFINITY;
     for (int j = lane; j < Lk; j += 64) mx = fmaxf(mx, score(j));
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
@@ -473,6 +458,10 @@ __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__
     for (int i = 0; i < GEN_MAXD / 64; ++i) {
         const int c = lane + 64 * i;
         if (c < dv) out[(long long)row * dv + c] = acc[i] * inv;
+    }
+    if (stats && lane == 0) {     // row statistics for the backward pass: a weight is exp(s - mx) * inv
+        stats[2 * (long long)row] = mx;
+        stats[2 * (long long)row + 1] = inv;
     }
 }
 
@@ -525,7 +514,6 @@ namespace {
 int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, float *stats, int64_t B, int64_t H,
                  int64_t Lq, int64_t Lk, int64_t dk, int64_t dv, float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
     DL4S_CHECK_CTX(ctx);
-    DL4S_REQUIRE(!stats || (dk == HD && dv == HD), DL4S_HIP_EUNSUPPORTED, "sdpa: row statistics need head dims of 64");
     std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     DL4S_REQUIRE(B >= 0 && H >= 0 && Lq >= 0 && Lk >= 0 && dk >= 0 && dv >= 0, DL4S_HIP_EINVALID_ARG,
                  "sdpa: negative extent");
@@ -563,7 +551,7 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
     const long long rows = B * H * Lq;
     DL4S_REQUIRE(rows < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "sdpa: too many rows for the plain kernel");
     hipLaunchKernelGGL(sdpa_generic_f32, dim3((unsigned)rows), dim3(64), 0, ctx->stream, q, k, v, out, (int)H, (int)Lq,
-                       (int)Lk, (int)dk, (int)dv, inv_temperature, m);
+                       (int)Lk, (int)dk, (int)dv, inv_temperature, m, stats);
     return dl4s::launch_status("sdpa_generic_f32");
 }
 }  // namespace

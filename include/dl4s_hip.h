@@ -120,7 +120,7 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
                           int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
 
-/* Training form of the fused attention (head dims 64).  The reference differentiates ScaledDotProductAttention through
+/* Training form of the fused attention (key dim = value dim = d; MFMA kernels for d = 64, plain kernels up to 256).  The reference differentiates ScaledDotProductAttention through
  * the backward closures of its primitive operators (Tensor/Operators/Matrix.swift:139-174 for the products through the
  * subscript views and the stack of broadcastMatrixMultiplied :79-117, Binary.swift:235-300 for e / sum,
  * Reduce.swift:35-62, Unary.swift:33-55 for exp, Binary.swift:161-224 for the subtractions); a backend that fuses the
@@ -130,7 +130,7 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
  *                                opaque to the caller)
  *   dl4s_hip_sdpa_bwd_f32        dq, dk, dv for the upstream gradient dout of out, from q, k, v, out, stats and the
  *                                same mask and flags as the forward call (the mask takes no gradient)
- * Layouts follow the forward call ([B,H,L,64], or [B,L,H,64] with DL4S_SDPA_TOKEN_MAJOR; stats is always [B,H,Lq,2]).
+ * Layouts follow the forward call ([B,H,L,d], or [B,L,H,64] with DL4S_SDPA_TOKEN_MAJOR; stats is always [B,H,Lq,2]).
  * Deterministic: no atomics, the same bits on every run. */
 int dl4s_hip_sdpa_fwd_stats_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, float *stats,
                                 int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t d, float inv_temperature,

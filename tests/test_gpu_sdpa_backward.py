@@ -142,11 +142,47 @@ def test_config4_sized_gradients(ctx, orc):
         assert_parity(dv[sl], rv, "config 4 dv")
 
 
+@pytest.mark.parametrize("d", [4, 8, 40, 130])
+@pytest.mark.parametrize("mask_kind", ["none", "dense", "causal_lengths"])
+def test_gradients_for_other_head_dims(ctx, orc, d, mask_kind):
+    """The plain kernels (head dims other than 64), e.g. the key size 8 of Tests/DL4STests/TransformerTests.swift:31."""
+    from dl4s_amd import lib
+    B, H, L = 2, 3, 70
+    rng = np.random.default_rng(d)
+    q, k, v, dout = (rand(rng, B, H, L, d) for _ in range(4))
+    lens = rng.integers(1, L + 1, size=B)
+    desc, mask, keep = None, None, []
+    if mask_kind == "dense":
+        mask = (rng.random((B, 1, L, L)) < 0.3).astype(np.float32)
+        mask[1, 0, 3, :] = 1.0
+        keep.append(ctx.to_device(mask))
+        desc = ctx.mask_desc(lib.MASK_DENSE, dense=keep[0])
+    elif mask_kind == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, L), causal_mask(L, L)[None, None])
+        keep.append(ctx.to_device(np.asarray(lens, np.int32), dtype=np.int32))
+        desc = ctx.mask_desc(lib.MASK_CAUSAL_OR_KEY_LENGTHS, lengths=keep[0])
+    bufs = [ctx.to_device(x) for x in (q, k, v, dout)]
+    out, dq, dk, dv = (ctx.empty((B, H, L, d)) for _ in range(4))
+    st = ctx.empty((B, H, L, 2))
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+    ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], out, st, B, H, L, L, d, rT, desc, 0)
+    ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], out, st, bufs[3], dq, dk, dv, B, H, L, L, d, rT, desc, 0)
+    assert_parity(out.numpy(), orc.sdpa(q, k, v, mask), "forward d=%d" % d)
+    rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+    assert_parity(dq.numpy(), rq, "dq d=%d" % d)
+    assert_parity(dk.numpy(), rk, "dk d=%d" % d)
+    assert_parity(dv.numpy(), rv, "dv d=%d" % d)
+    for b in bufs + [out, dq, dk, dv, st] + keep:
+        b.release()
+
+
 def test_backward_argument_errors(ctx):
     from dl4s_amd import lib
-    a = ctx.empty((1, 1, 4, 8))
-    with pytest.raises(lib.Dl4sHipError):       # head dim other than 64
-        ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5)
-    with pytest.raises(lib.Dl4sHipError):
-        ctx.sdpa_fwd_stats(a, a, a, a, a, 1, 1, 4, 4, 8, 0.5)
+    a = ctx.empty((1, 1, 4, 300))
+    with pytest.raises(lib.Dl4sHipError):       # head dim above 256
+        ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 300, 0.5)
+    with pytest.raises(lib.Dl4sHipError):       # token-major needs head dims of 64
+        ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5, None, lib.SDPA_TOKEN_MAJOR)
+    with pytest.raises(lib.Dl4sHipError):       # unknown flag
+        ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5, None, 128)
     a.release()
