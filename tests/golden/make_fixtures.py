@@ -1,4 +1,5 @@
-"""Writes tests/golden/attention_fixtures.npz: small inputs and the CPU oracle's outputs for them.
+"""Writes tests/golden/attention_fixtures.npz and tests/golden/model_fixtures.npz: small inputs and the CPU oracle's
+outputs for them.
 
 The vectors come from this repository's oracle (oracle/dl4s_oracle.c), never from the reference (which is Swift and
 cannot run here); they freeze the oracle's behaviour so that a later change to it shows up, and give the GPU tests a
@@ -58,5 +59,48 @@ def main():
     print("wrote %d arrays" % len(out))
 
 
+def flatten_transformer(params):
+    flat = {"embedding": params["embedding"], "output_bias": params["output_bias"]}
+    for side, parts in (("encoder", ("attn", "ffn")), ("decoder", ("self", "cross", "ffn"))):
+        for i, layer in enumerate(params[side]):
+            for part in parts:
+                for name, val in layer[part].items():
+                    flat["%s%d_%s_%s" % (side, i, part, name)] = val
+    return flat
+
+
+def model_fixtures():
+    """Gradients of attention on the tiny attention fixture, and the Transformer wrapper (forward log-probabilities and
+    greedy decoding) at the hyper-parameters of Tests/DL4STests/TransformerTests.swift:31."""
+    from oracle import transformer as orc_t
+    fix = np.load(os.path.join(ROOT, "tests", "golden", "attention_fixtures.npz"))
+    rng = np.random.default_rng(20241)
+    out = {}
+    q, k, v = fix["sdpa_q"], fix["sdpa_k"], fix["sdpa_v"]
+    dout = rng.standard_normal(q.shape).astype(np.float32)
+    out["bwd_dout"] = dout
+    for name in ("none", "dense", "causal", "blocked_row"):
+        m = None if name == "none" else fix["sdpa_mask_" + name]
+        dq, dk, dv = orc.sdpa_backward(q, k, v, m, dout)
+        out.update({"bwd_dq_" + name: dq, "bwd_dk_" + name: dk, "bwd_dv_" + name: dv})
+    vocab = 13
+    params = m64.make_transformer_params(rng, vocab, 16, 4, 8, 8, 32, 2, 2)
+    for name, val in flatten_transformer(params).items():
+        out["tf_" + name] = val
+    enc_len, dec_len = [7, 4], [5, 3]
+    enc, dec = np.full((2, 7), -1, np.int32), np.full((2, 5), -1, np.int32)
+    for b in range(2):
+        enc[b, :enc_len[b]] = rng.integers(0, vocab, enc_len[b])
+        dec[b, :dec_len[b]] = rng.integers(0, vocab, dec_len[b])
+    src = rng.integers(0, vocab, 6).astype(np.int32)
+    toks, logits = orc_t.greedy_decode(params, [int(t) for t in src], 1, 2, 6, return_logits=True)
+    out.update(tf_enc_tokens=enc, tf_dec_tokens=dec, tf_enc_lengths=np.array(enc_len), tf_dec_lengths=np.array(dec_len),
+               tf_log_probs=orc_t.forward(params, enc, dec, enc_len, dec_len), tf_positions=orc_t.positional_encoding(9, 16),
+               tf_greedy_source=src, tf_greedy_tokens=np.array(toks, np.int32), tf_greedy_logits=np.stack(logits))
+    np.savez_compressed(os.path.join(ROOT, "tests", "golden", "model_fixtures.npz"), **out)
+    print("wrote %d arrays" % len(out))
+
+
 if __name__ == "__main__":
     main()
+    model_fixtures()

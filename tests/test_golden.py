@@ -1,5 +1,5 @@
-"""Golden fixtures (tests/golden/attention_fixtures.npz, written by tests/golden/make_fixtures.py from the CPU
-oracle): the oracle must still reproduce them bit for bit (CPU), and the HIP path must match them (GPU)."""
+"""Golden fixtures (tests/golden/attention_fixtures.npz and model_fixtures.npz, written by tests/golden/make_fixtures.py
+from the CPU oracle): the oracle must still reproduce them bit for bit (CPU), and the HIP path must match them (GPU)."""
 import os
 
 import numpy as np
@@ -72,5 +72,81 @@ def test_hip_matches_fixtures():
             ctx.sdpa_decode_step(dq, dk_, dv_, kn, vn, out, 1, 2, 9 + t, 12, 64, 0.125)
             assert_parity(out.numpy(), FIX["dec_out"][t], "decode step %d" % t)
         assert np.array_equal(dk_.numpy(), FIX["dec_k"]) and np.array_equal(dv_.numpy(), FIX["dec_v"])
+    finally:
+        ctx.close()
+
+
+# ------------------------------------------------------------------ gradients and the Transformer wrapper
+MFIX = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "model_fixtures.npz"))
+BWD_MASKS = ["none", "dense", "causal", "blocked_row"]
+
+
+def _transformer_params():
+    p = {"embedding": MFIX["tf_embedding"], "output_bias": MFIX["tf_output_bias"], "heads": 4, "dk": 8, "dv": 8, "encoder": [], "decoder": []}
+    for side, parts in (("encoder", ("attn", "ffn")), ("decoder", ("self", "cross", "ffn"))):
+        for i in range(2):
+            layer = {}
+            for part in parts:
+                pre = "tf_%s%d_%s_" % (side, i, part)
+                layer[part] = {k[len(pre):]: MFIX[k] for k in MFIX.files if k.startswith(pre)}
+            p[side].append(layer)
+    return p
+
+
+def test_oracle_reproduces_model_fixtures(orc):
+    from oracle import transformer as T
+    q, k, v = FIX["sdpa_q"], FIX["sdpa_k"], FIX["sdpa_v"]
+    for name in BWD_MASKS:
+        got = orc.sdpa_backward(q, k, v, _mask(name), MFIX["bwd_dout"])
+        for g, key in zip(got, ("dq", "dk", "dv")):
+            assert np.array_equal(g, MFIX["bwd_%s_%s" % (key, name)]), (key, name)
+    params = _transformer_params()
+    assert np.array_equal(T.positional_encoding(9, 16), MFIX["tf_positions"])
+    lp = T.forward(params, MFIX["tf_enc_tokens"], MFIX["tf_dec_tokens"], list(MFIX["tf_enc_lengths"]), list(MFIX["tf_dec_lengths"]))
+    assert np.array_equal(lp, MFIX["tf_log_probs"])
+    toks, logits = T.greedy_decode(params, [int(t) for t in MFIX["tf_greedy_source"]], 1, 2, 6, return_logits=True)
+    assert toks == list(MFIX["tf_greedy_tokens"]) and np.array_equal(np.stack(logits), MFIX["tf_greedy_logits"])
+
+
+def test_model_fixture_invariants():
+    # every softmax row sums to 1, so the value gradient sums to the upstream gradient, whatever the mask
+    for name in BWD_MASKS:
+        assert np.allclose(MFIX["bwd_dv_" + name].sum(2), MFIX["bwd_dout"].sum(2), atol=1e-5)
+    assert np.allclose(np.exp(MFIX["tf_log_probs"].astype(np.float64)).sum(-1), 1.0, atol=1e-5)
+    top2 = np.sort(MFIX["tf_greedy_logits"], axis=1)[:, -2:]
+    assert (top2[:, 1] - top2[:, 0]).min() > 1e-3                  # the greedy fixture does not sit on a tie
+
+
+@pytest.mark.gpu
+def test_hip_matches_model_fixtures():
+    from dl4s_amd import host_lib, lib
+    ctx = lib.Context(0)
+    try:
+        q, k, v, dout = FIX["sdpa_q"], FIX["sdpa_k"], FIX["sdpa_v"], MFIX["bwd_dout"]
+        B, H, Lq, d = q.shape
+        Lk = k.shape[2]
+        bufs = [ctx.to_device(x) for x in (q, k, v, dout)]
+        out, dq, st = ctx.empty(q.shape), ctx.empty(q.shape), ctx.empty((B, H, Lq, 2))
+        dk_, dv_ = ctx.empty(k.shape), ctx.empty(v.shape)
+        for name in BWD_MASKS:
+            desc, keep = None, None
+            if name != "none":
+                keep = ctx.to_device(_mask(name))
+                desc = ctx.mask_desc(lib.MASK_DENSE, dense=keep)
+            ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], out, st, B, H, Lq, Lk, d, 0.5, desc, 0)
+            ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], out, st, bufs[3], dq, dk_, dv_, B, H, Lq, Lk, d, 0.5, desc, 0)
+            assert_parity(out.numpy(), FIX["sdpa_out_" + name], "forward " + name)
+            for got, key in ((dq, "dq"), (dk_, "dk"), (dv_, "dv")):
+                assert_parity(got.numpy(), MFIX["bwd_%s_%s" % (key, name)], key + " " + name)
+        params = _transformer_params()
+        model = host_lib.Transformer(ctx, params)
+        for fused in (False, True):
+            assert_parity(host_lib.positional_encoding(ctx, 9, 16, fused=fused), MFIX["tf_positions"], "positions")
+            lp = model.forward(MFIX["tf_enc_tokens"], MFIX["tf_dec_tokens"], MFIX["tf_enc_lengths"], MFIX["tf_dec_lengths"], fused=fused)
+            assert_parity(lp, MFIX["tf_log_probs"], "log-probabilities")
+            toks, logits = model.greedy(MFIX["tf_greedy_source"], 1, 2, 6, fused=fused, return_logits=True)
+            assert toks == list(MFIX["tf_greedy_tokens"])
+            assert_parity(logits, MFIX["tf_greedy_logits"], "greedy logits")
+        model.close()
     finally:
         ctx.close()
