@@ -237,28 +237,53 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
             for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < NI; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s8 >> 2][s8 & 3], bv[j], acc[i][j], 0, 0, 0);
+                    // operands swapped: the accumulator is the TRANSPOSED tile (lane = row m, registers = columns n), so
+                    // that a lane holds four consecutive columns and the epilogue moves 128 bits per access
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], af[i][s8 >> 2][s8 & 3], acc[i][j], 0, 0, 0);
         }
         if (more) store(buf ^ 1);
         __syncthreads();
     }
 
+    // accumulator register r of a transposed 32x32 tile: row m = lane % 32, column n = 8*(r/4) + 4*half + r%4
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < MI; ++i) {
+        const int gm = m0 + wm * 32 * MI + i * 32 + ln;
+        if (gm >= g.M) continue;
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            const int gn = n0 + wn * 32 * NI + j * 32 + ln;
+        for (int j = 0; j < NI; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int gm = m0 + wm * 32 * MI + i * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (gm < g.M && gn < g.N) {
-                    float *cp = C + (long long)gm * g.N + gn;
-                    float val = g.alpha * acc[i][j][r];
-                    if (g.beta != 0.f) val = val + g.beta * (*cp);
-                    *cp = EPI ? epilogue(g, val, gm, gn) : val;
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int gn = n0 + wn * 32 * NI + j * 32 + 8 * q4 + 4 * half;
+                if (gn >= g.N) continue;      // N is a multiple of 4: a quad is inside or outside as a whole
+                float *cp = C + (long long)gm * g.N + gn;
+                f32x4 val;
+                val.x = g.alpha * acc[i][j][4 * q4 + 0]; val.y = g.alpha * acc[i][j][4 * q4 + 1];
+                val.z = g.alpha * acc[i][j][4 * q4 + 2]; val.w = g.alpha * acc[i][j][4 * q4 + 3];
+                if (g.beta != 0.f) {
+                    const f32x4 old = *reinterpret_cast<const f32x4 *>(cp);
+                    val.x = val.x + g.beta * old.x; val.y = val.y + g.beta * old.y;
+                    val.z = val.z + g.beta * old.z; val.w = val.w + g.beta * old.w;
                 }
+                if (EPI) {
+                    if (g.bias) {
+                        const f32x4 bq = *reinterpret_cast<const f32x4 *>(g.bias + gn);
+                        val.x = __fadd_rn(val.x, bq.x); val.y = __fadd_rn(val.y, bq.y);
+                        val.z = __fadd_rn(val.z, bq.z); val.w = __fadd_rn(val.w, bq.w);
+                    }
+                    if (g.act == 1) {
+                        val.x = gelu_sigmoid(val.x); val.y = gelu_sigmoid(val.y);
+                        val.z = gelu_sigmoid(val.z); val.w = gelu_sigmoid(val.w);
+                    }
+                    if (g.residual) {
+                        const f32x4 rq = *reinterpret_cast<const f32x4 *>(g.residual + (long long)blockIdx.z * g.c_bs + (long long)gm * g.N + gn);
+                        val.x = __fadd_rn(val.x, rq.x); val.y = __fadd_rn(val.y, rq.y);
+                        val.z = __fadd_rn(val.z, rq.z); val.w = __fadd_rn(val.w, rq.w);
+                    }
+                }
+                *reinterpret_cast<f32x4 *>(cp) = val;
             }
-        }
+    }
 }
 
 int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int64_t lbs, const float *rhs, int64_t rr,
@@ -284,7 +309,8 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     // the fast kernels address A within a tile's rows and B as a whole through 32-bit byte offsets below 2^31
     const bool fast = !ta && !tb && K % 4 == 0 && N % 4 == 0 && K > 0 && aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 &&
-                      rbs % 4 == 0 && K < (1ll << 21) && K * N * 4 < (1ll << 31);
+                      rbs % 4 == 0 && K < (1ll << 21) && K * N * 4 < (1ll << 31) && aligned16(result) && cbs % 4 == 0 &&
+                      aligned16(bias) && aligned16(residual);
     long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
     // small products: 64x64 tiles, so that there are at least about two workgroups per CU
     const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;
