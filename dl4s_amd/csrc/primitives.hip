@@ -270,6 +270,24 @@ int launch_binary(dl4s_hip_ctx *ctx, const float *a, const float *b, float *y, i
     hipLaunchKernelGGL(binary_f32<OP>, dim3(grid_for(n)), dim3(TPB), 0, ctx->stream, a, b, y, (long long)n);
     return dl4s::launch_status(name);
 }
+// stack along axis 0: up to 64 equally sized source buffers per launch (their addresses travel as kernel arguments),
+// blockIdx.y = buffer, the grid-stride loop copies 128 bits per thread where the addresses allow
+struct StackSrc {
+    const float *p[64];
+};
+__global__ void stack_f32(StackSrc src, float *__restrict__ dst, long long count, int vec) {
+    const float *s = src.p[blockIdx.y];
+    float *d = dst + (long long)blockIdx.y * count;
+    const long long stride = (long long)gridDim.x * blockDim.x, i0 = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec) {
+        const long long n4 = count >> 2;
+        for (long long i = i0; i < n4; i += stride) reinterpret_cast<float4 *>(d)[i] = reinterpret_cast<const float4 *>(s)[i];
+        for (long long i = (n4 << 2) + i0; i < count; i += stride) d[i] = s[i];
+    } else {
+        for (long long i = i0; i < count; i += stride) d[i] = s[i];
+    }
+}
+
 // First index of the largest value, scanning like `if v > maxV` from (-inf, index 0): NaN is never selected, ties keep
 // the earliest index (Engine/CPU/Numeric/CPUFloat.swift:294-318, generic branch).  One workgroup; out = {value, index}.
 __global__ __launch_bounds__(1024) void argmax_f32(const float *__restrict__ x, long long n, float *out_value, long long *out_index) {
@@ -507,9 +525,23 @@ int dl4s_hip_stack_f32(dl4s_hip_ctx *ctx, const float *const *buffers, int64_t n
     DL4S_REQUIRE(n >= 0 && count >= 0, DL4S_HIP_EINVALID_ARG, "stack: negative extent");
     if (n * count == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(buffers && result, DL4S_HIP_EINVALID_ARG, "stack: NULL pointer");
-    for (int64_t i = 0; i < n; ++i) {
-        DL4S_REQUIRE(buffers[i], DL4S_HIP_EINVALID_ARG, "stack: buffer %lld is NULL", (long long)i);
-        DL4S_HIP_TRY(hipMemcpyAsync(result + i * count, buffers[i], (size_t)count * sizeof(float), hipMemcpyDeviceToDevice, ctx->stream));
+    for (int64_t i = 0; i < n; ++i) DL4S_REQUIRE(buffers[i], DL4S_HIP_EINVALID_ARG, "stack: buffer %lld is NULL", (long long)i);
+    // one launch per 64 buffers instead of one copy per buffer (the reference stacks B*H score slices per attention call)
+    for (int64_t at = 0; at < n; at += 64) {
+        const int m = (int)(n - at < 64 ? n - at : 64);
+        StackSrc src{};
+        int vec = ((reinterpret_cast<uintptr_t>(result + at * count) & 15) == 0 && count % 4 == 0) ? 1 : 0;
+        for (int i = 0; i < m; ++i) {
+            src.p[i] = buffers[at + i];
+            if (reinterpret_cast<uintptr_t>(buffers[at + i]) & 15) vec = 0;
+        }
+        long long want = (count / (vec ? 4 : 1) + TPB * 4 - 1) / (TPB * 4);
+        if (want < 1) want = 1;
+        if (want > 1024) want = 1024;
+        hipLaunchKernelGGL(stack_f32, dim3((unsigned)want, (unsigned)m), dim3(TPB), 0, ctx->stream, src, result + at * count,
+                           (long long)count, vec);
+        const int rc = dl4s::launch_status("stack");
+        if (rc != DL4S_HIP_OK) return rc;
     }
     return DL4S_HIP_OK;
 }

@@ -280,3 +280,19 @@ def test_dense_fused_errors(ctx):
     with pytest.raises(lib.Dl4sHipError):
         ctx.dense_fused(a, -1, 4, a, 4, None, 0, None, a)
     a.release()
+
+
+@pytest.mark.parametrize("nbuf,count", [(1, 5), (3, 1000), (70, 333), (130, 64), (65, 4099)])
+def test_stack_many_buffers(ctx, nbuf, count):
+    """Tensor(stacking:) along axis 0 (Tensor/Operators/Stack.swift:79-98): more buffers than one launch carries, counts
+    that are not multiples of four, sources at unaligned offsets."""
+    rng = np.random.default_rng(nbuf * 100 + count)
+    parts = [rng.standard_normal(count + 1).astype(np.float32) for _ in range(nbuf)]
+    dev = [ctx.to_device(p) for p in parts]
+    dst = ctx.empty((nbuf, count))
+    srcs = [d.offset(4) if i % 2 else d for i, d in enumerate(dev)]      # every other source starts one float in
+    ctx.stack(srcs, count, dst)
+    ref = np.stack([p[1:count + 1] if i % 2 else p[:count] for i, p in enumerate(parts)])
+    assert np.array_equal(dst.numpy(), ref)
+    for d in dev + [dst]:
+        d.release()
