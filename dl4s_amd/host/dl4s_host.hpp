@@ -209,6 +209,17 @@ struct HIP {
                                         1.0f / temperature, mask ? &md : nullptr,
                                         DL4S_SDPA_STRICT | (tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u)));
         }
+        // the same with a structured mask descriptor (kind + device int32 lengths) instead of a dense mask tensor
+        static void fusedAttentionStructured(const ShapedBuffer &q, const ShapedBuffer &k, const ShapedBuffer &v, int kind,
+                                             const int32_t *lengths, const ShapedBuffer &result, float temperature, bool tokenMajor) {
+            dl4s_mask_desc md{};
+            md.kind = kind;
+            md.lengths = lengths;
+            const int h = tokenMajor ? 2 : 1, l = tokenMajor ? 1 : 2;
+            check(dl4s_hip_sdpa_fwd_f32(context(), q.values.memory, k.values.memory, v.values.memory, result.values.memory,
+                                        q.shape[0], q.shape[h], q.shape[l], k.shape[l], q.shape[3], v.shape[3], 1.0f / temperature,
+                                        kind == DL4S_MASK_NONE ? nullptr : &md, tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u));
+        }
         // result = act(x . weights + bias) + residual  (bias, residual optional)
         static void denseFused(const ShapedBuffer &x, const ShapedBuffer &weights, const ShapedBuffer *bias, int activation,
                                const ShapedBuffer *residual, const ShapedBuffer &result) {
@@ -718,6 +729,26 @@ struct Dense {
     }
 };
 
+// A mask whose structure the caller knows - the two families TransformerUtil.swift:29-50 builds: keys at or beyond each
+// sequence's length blocked, optionally together with the causal triangle.  In fused mode the model-level layers hand it
+// to the attention kernel as a descriptor instead of materialising the dense tensor: the same bits as the dense mask
+// it stands for, and key tiles it blocks entirely are not visited (exact because activations are finite and every row
+// keeps at least its first key; a sequence of length 0 - all keys blocked, uniform weights - is computed in full).
+struct AttentionMask {
+    int kind = DL4S_MASK_NONE;
+    Tensor lengths;   // device int32 [batchSize], viewed through a float buffer of the same byte size
+    static AttentionMask forLengths(const std::vector<int64_t> &sequenceLengths, bool causal) {
+        AttentionMask m;
+        m.kind = causal ? DL4S_MASK_CAUSAL_OR_KEY_LENGTHS : DL4S_MASK_KEY_LENGTHS;
+        std::vector<int32_t> l32(sequenceLengths.begin(), sequenceLengths.end());
+        for (int32_t v : l32) precondition(v >= 0, "sequence lengths must not be negative");
+        m.lengths = Tensor(Device::Memory::allocateBuffer(Shape{(int64_t)l32.size()}));
+        Device::check(dl4s_hip_assign_h2d(Device::context(), m.lengths.buffer().memory, l32.data(), l32.size() * sizeof(int32_t)));
+        return m;
+    }
+    const int32_t *lengthsPointer() const { return reinterpret_cast<const int32_t *>(lengths.buffer().memory); }
+};
+
 // NN/Models/Transformer/ScaledDotProductAttention.swift:29-65
 struct ScaledDotProductAttention {
     float temperature;
@@ -762,14 +793,19 @@ struct MultiHeadAttention {
         return {k.view({B * L, hiddenDim}).matrixMultiplied(kDense).view({B, L, heads, keyDim}),
                 v.view({B * L, hiddenDim}).matrixMultiplied(vDense).view({B, L, heads, valueDim})};
     }
-    Tensor attendProjected(const Tensor &q, const Tensor &kp, const Tensor &vp, const Tensor *mask) const {
+    Tensor attendProjected(const Tensor &q, const Tensor &kp, const Tensor &vp, const Tensor *mask,
+                           const AttentionMask *structured = nullptr) const {
         precondition(canCacheProjections() && q.dim() == 3 && kp.dim() == 4 && vp.dim() == 4, "Matmul operands must have matching shapes");
         const int64_t batchSize = q.shape[0], queryCount = q.shape[1];
         Tensor qp = q.view({batchSize * queryCount, hiddenDim}).matrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
         Tensor a(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, heads, valueDim}));
         ShapedBuffer mb;
         if (mask) mb = mask->values();
-        Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true);
+        if (structured)
+            Device::Engine::fusedAttentionStructured(qp.values(), kp.values(), vp.values(), structured->kind, structured->lengthsPointer(),
+                                                     a.values(), attn.temperature, true);
+        else
+            Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true);
         Tensor a2 = a.view({batchSize * queryCount, heads * valueDim});
         if (!dropout.isActive) {
             Tensor sum(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, hiddenDim}));
@@ -779,6 +815,11 @@ struct MultiHeadAttention {
         }
         Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
         return norm.normalize(out_drop, &q);
+    }
+    // self- or cross-attention with a structured mask (fused mode, head dims 64)
+    Tensor structured(const Tensor &q, const Tensor &k, const Tensor &v, const AttentionMask &mask) const {
+        auto kv = projectKeysValues(k, v);
+        return attendProjected(q, kv.first, kv.second, nullptr, &mask);
     }
     Tensor operator()(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask) const {
         const int64_t batchSize = q.shape[0], queryCount = q.shape[1], keyCount = k.shape[1], valueCount = v.shape[1];
@@ -838,6 +879,9 @@ struct TransformerEncoderBlock {
         Tensor attn = selfAttention(inputs, inputs, inputs, &mask);
         return pointwiseFeedForward(attn);
     }
+    Tensor operator()(const Tensor &inputs, const AttentionMask &mask) const {
+        return pointwiseFeedForward(selfAttention.structured(inputs, inputs, inputs, mask));
+    }
 };
 
 // NN/Models/Transformer/TransformerDecoderBlock.swift:29-69
@@ -857,6 +901,12 @@ struct TransformerDecoderBlock {
                                 const Tensor &decoderMask) const {
         Tensor decAttn = selfAttention(decoderInput, decoderInput, decoderInput, &decoderMask);
         Tensor encAttn = encoderAttention.attendProjected(decAttn, encKeys, encValues, &encoderMask);
+        return pointwiseFeedForward(encAttn);
+    }
+    Tensor withProjectedEncoder(const Tensor &decoderInput, const Tensor &encKeys, const Tensor &encValues, const AttentionMask &encoderMask,
+                                const AttentionMask &decoderMask) const {
+        Tensor decAttn = selfAttention.structured(decoderInput, decoderInput, decoderInput, decoderMask);
+        Tensor encAttn = encoderAttention.attendProjected(decAttn, encKeys, encValues, nullptr, &encoderMask);
         return pointwiseFeedForward(encAttn);
     }
 };
@@ -939,9 +989,19 @@ struct TransformerEncoder {
     TransformerEncoder(int64_t layerCount, int64_t heads, int64_t keyDim, int64_t valueDim, int64_t modelDim, int64_t forwardDim, float dropout) {
         for (int64_t i = 0; i < layerCount; ++i) encoderLayers.emplace_back(modelDim, forwardDim, heads, keyDim, valueDim, dropout);
     }
+    bool canUseStructuredMasks() const {
+        for (auto &l : encoderLayers)
+            if (!l.selfAttention.canCacheProjections()) return false;
+        return !encoderLayers.empty();
+    }
     Tensor operator()(const Tensor &input, const std::vector<int64_t> &sequenceLengths) const {
-        const Tensor mask = makeEncoderMasks(sequenceLengths);
         Tensor acc = input;
+        if (canUseStructuredMasks()) {      // fused mode: the mask as a descriptor, never materialised
+            const AttentionMask mask = AttentionMask::forLengths(sequenceLengths, false);
+            for (auto &layer : encoderLayers) acc = layer(acc, mask);
+            return acc;
+        }
+        const Tensor mask = makeEncoderMasks(sequenceLengths);
         for (auto &layer : encoderLayers) acc = layer(acc, mask);
         return acc;
     }
@@ -955,6 +1015,8 @@ struct TransformerDecoder {
     }
     Tensor operator()(const Tensor &decoderInput, const Tensor &encoderStates, const std::vector<int64_t> &encoderInputLengths,
                       const std::vector<int64_t> &decoderInputLengths) const {
+        if (canCacheEncoderProjections())   // fused mode, head dims 64: structured masks, encoder projections per call
+            return withProjectedEncoder(decoderInput, projectEncoderStates(encoderStates), encoderInputLengths, decoderInputLengths);
         const Tensor encoderMask = makeEncoderMasks(encoderInputLengths);
         const Tensor decoderMask = makeDecoderMasks(decoderInputLengths);
         Tensor acc = decoderInput;
@@ -964,7 +1026,7 @@ struct TransformerDecoder {
     // Encoder-side key / value projections of every layer, computed once per encoded sequence (fused mode, head dims 64)
     bool canCacheEncoderProjections() const {
         for (auto &l : decoderLayers)
-            if (!l.encoderAttention.canCacheProjections()) return false;
+            if (!l.encoderAttention.canCacheProjections() || !l.selfAttention.canCacheProjections()) return false;
         return !decoderLayers.empty();
     }
     std::vector<std::pair<Tensor, Tensor>> projectEncoderStates(const Tensor &encoderStates) const {
@@ -974,8 +1036,8 @@ struct TransformerDecoder {
     }
     Tensor withProjectedEncoder(const Tensor &decoderInput, const std::vector<std::pair<Tensor, Tensor>> &kv,
                                 const std::vector<int64_t> &encoderInputLengths, const std::vector<int64_t> &decoderInputLengths) const {
-        const Tensor encoderMask = makeEncoderMasks(encoderInputLengths);
-        const Tensor decoderMask = makeDecoderMasks(decoderInputLengths);
+        const AttentionMask encoderMask = AttentionMask::forLengths(encoderInputLengths, false);
+        const AttentionMask decoderMask = AttentionMask::forLengths(decoderInputLengths, true);
         Tensor acc = decoderInput;
         for (size_t i = 0; i < decoderLayers.size(); ++i)
             acc = decoderLayers[i].withProjectedEncoder(acc, kv[i].first, kv[i].second, encoderMask, decoderMask);
@@ -999,10 +1061,12 @@ struct Transformer {
           outputBias(Tensor::repeating(0.f, {vocabSize})) {}
 
     // inputs: [batchSize][maxLen] tokens, -1 = padding                                   (Transformer.swift:86-92)
-    Tensor prepareInputs(const std::vector<int32_t> &inputs, int64_t batchSize, int64_t maxLen) const {
+    // positions: optional precomputed encoding with at least maxLen rows (row l does not depend on the length)
+    Tensor prepareInputs(const std::vector<int32_t> &inputs, int64_t batchSize, int64_t maxLen, const Tensor *positions = nullptr) const {
         precondition((int64_t)inputs.size() == batchSize * maxLen, "element count does not match shape");
         const int64_t D = embedding.outputSize();
-        const Tensor encoderPositions = positionalEncoding(maxLen);          // [maxLen, embedDim]
+        precondition(!positions || (Device::fused() && positions->shape[0] >= maxLen), "bad positions");
+        const Tensor encoderPositions = positions ? *positions : positionalEncoding(maxLen);          // [maxLen, embedDim]
         const float scale = std::sqrt((float)D);
         if (Device::fused()) {
             for (int32_t idx : inputs)
@@ -1040,12 +1104,14 @@ struct Transformer {
         const bool cached = decoder.canCacheEncoderProjections();
         std::vector<std::pair<Tensor, Tensor>> kv;
         if (cached) kv = decoder.projectEncoderStates(encoded);
+        Tensor positions;     // fused mode: one encoding for the longest prefix instead of one per step
+        if (Device::fused()) positions = positionalEncoding(maxLength);
         std::vector<int32_t> tokens;
         for (int64_t step = 0; step < maxLength; ++step) {
             std::vector<int32_t> tokenInput{startToken};
             tokenInput.insert(tokenInput.end(), tokens.begin(), tokens.end());
             const int64_t len = (int64_t)tokenInput.size();
-            Tensor decIn = prepareInputs(tokenInput, 1, len);
+            Tensor decIn = prepareInputs(tokenInput, 1, len, Device::fused() ? &positions : nullptr);
             Tensor output = cached ? decoder.withProjectedEncoder(decIn, kv, {n}, {len}) : decoder(decIn, encoded, {n}, {len});
             Tensor deembedded = output.broadcastMatrixMultiplied(embedding.embeddingMatrix, false, true);
             Tensor last = deembedded[{0, len - 1}];
