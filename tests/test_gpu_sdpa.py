@@ -487,3 +487,22 @@ def test_concurrent_callers_on_one_context(ctx, orc):
         for got in results[i]:
             assert_parity(got, ref, "thread %d" % i)
             assert np.array_equal(got, results[i][0])
+
+
+@pytest.mark.parametrize("kind_name", ["lens", "causal_lens"])
+def test_sequence_of_length_zero_gives_uniform_rows(ctx, orc, kind_name):
+    """A valid length of 0 blocks every key of that batch item: all rows are uniform (the mean of V), exactly as with
+    the dense mask; the other batch items are unaffected."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(123)
+    B, H, L = 3, 2, 160
+    q, k, v = rand(rng, B, H, L, 64), rand(rng, B, H, L, 64), rand(rng, B, H, L, 64)
+    lens = np.array([0, 97, 160])
+    kind = lib.MASK_KEY_LENGTHS if kind_name == "lens" else lib.MASK_CAUSAL_OR_KEY_LENGTHS
+    mask = lengths_mask(lens, L)
+    if kind_name == "causal_lens":
+        mask = np.maximum(mask, causal_mask(L, L)[None, None])
+    got = run_sdpa(ctx, q, k, v, kind=kind, lens=lens)
+    assert_parity(got, orc.sdpa(q, k, v, mask), kind_name)
+    assert np.allclose(got[0], v[0].mean(axis=1, keepdims=True), atol=1e-5)
+    assert np.array_equal(got, run_sdpa(ctx, q, k, v, mask))
