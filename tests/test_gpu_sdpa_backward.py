@@ -186,3 +186,42 @@ def test_backward_argument_errors(ctx):
     with pytest.raises(lib.Dl4sHipError):       # unknown flag
         ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5, None, 128)
     a.release()
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_forward_and_backward(ctx, orc, seed):
+    """Seeded random extents, mask kinds, layouts and flags: forward and gradients against the oracle."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(1000 + seed)
+    B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+    Lq, Lk = int(rng.integers(1, 330)), int(rng.integers(1, 330))
+    kind_name = ["none", "dense", "dense_bcast", "lengths", "causal", "causal_lengths"][int(rng.integers(0, 6))]
+    if kind_name.startswith("causal"):
+        Lk = Lq
+    scale = float(rng.choice([0.3, 1.0, 3.0]))
+    q, k, v, dout = rand(rng, B, H, Lq, 64, scale=scale), rand(rng, B, H, Lk, 64, scale=scale), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lq, 64)
+    lens = rng.integers(1, Lk + 1, size=B)
+    kw, mask = {}, None
+    if kind_name == "dense":
+        mask = (rng.random((B, H, Lq, Lk)) < rng.choice([0.1, 0.5, 0.9])).astype(np.float32)
+        kw = dict(mask=mask)
+    elif kind_name == "dense_bcast":
+        mask = (rng.random((1, H, 1, Lk)) < 0.5).astype(np.float32)
+        mask[..., 0] = 0.0
+        kw = dict(mask=mask)
+    elif kind_name == "lengths":
+        mask, kw = lengths_mask(lens, Lk), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    elif kind_name == "causal":
+        mask, kw = causal_mask(Lq, Lq), dict(kind=lib.MASK_CAUSAL)
+    elif kind_name == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lq)[None, None])
+        kw = dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens)
+    kw["token_major"] = bool(rng.integers(0, 2))
+    kw["strict"] = bool(rng.integers(0, 2))
+    out, _, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, **kw)
+    what = "seed %d: B%d H%d Lq%d Lk%d %s %s" % (seed, B, H, Lq, Lk, kind_name, kw)
+    assert_parity(out, orc.sdpa(q, k, v, mask), "out " + what)
+    rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+    assert_parity(dq, rq, "dq " + what)
+    assert_parity(dk, rk, "dk " + what)
+    assert_parity(dv, rv, "dv " + what)
