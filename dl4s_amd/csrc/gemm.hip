@@ -6,7 +6,10 @@
 //                      tiles stored k-major ([k][m] and [k][n]) so that the MFMA operand reads (lane l wants row l % 32
 //                      at k = l / 32) are consecutive 32-bit words; the thread-to-element mapping of the loader is
 //                      chosen so that the unit-stride direction runs along the lanes
-//   gemm_f32_mfma_nn   row-major A and B (the layers' products): 128-bit buffer loads, A kept [m][k] in LDS
+//   gemm_f32_mfma_fast every transpose combination of aligned operands with extents that are multiples of 4 (the layers'
+//                      products and their gradients): 128-bit buffer loads, see below
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -23,6 +26,7 @@ struct GemmArgs {
     long long a_rs, a_cs;  // element strides of op(A)[m][k]
     long long b_rs, b_cs;  // element strides of op(B)[k][n]
     long long a_bs, b_bs, c_bs;  // batch strides
+    long long lda, ldb;          // row strides of A and B as stored (the fast kernels)
     float alpha, beta;
     int tiles_n;
     // epilogue of the fused Dense forms: C = act(alpha * A.B + bias[n]) + residual[m][n]
@@ -136,74 +140,106 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_mfma(GemmArgs g) {
         }
 }
 
-// Fast path for the layers' matrix products: op(A) = A row-major (unit stride along k), op(B) = B row-major (unit stride
-// along n), K and N multiples of 4 and 16-byte aligned operands.  Same 128x128 tile and 2x2 wavefront layout; the
-// differences are 128-bit global loads and LDS stores, A kept [m][k] in LDS (row stride 20 floats: 128-bit operand
-// reads of 8 rows fall on distinct banks) so that one LDS read feeds four MFMA steps, and three workgroups per CU.
-// MFMA step s of a K tile takes k = 8*half + s from both operands (any bijection of k works as long as A and B agree).
-constexpr int ALS = GBK + 4;   // A LDS row stride (floats)
+// Fast kernels: 128-bit buffer loads, K and the unit-stride extents multiples of 4, 16-byte aligned operands.  Same
+// 2x2 wavefront layout as above.  An operand is staged in one of two ways, chosen by how it lies in memory:
+//   rows x K, K contiguous (A, or B when transposeSecond)   kept [row][k] in LDS on a 20-float row stride, so that
+//                                                           128-bit operand reads of 8 rows fall on distinct banks
+//                                                           and one LDS read feeds four MFMA steps
+//   K x rows, rows contiguous (B, or A when transposeFirst) kept [k][row] in LDS, read one word per MFMA step
+// Both go through buffer loads with the whole byte offset in the (range-checked) vector operand: rows past the extent,
+// K rows past K and -- through an offset beyond any descriptor -- columns past the extent read as zeros, so a K step
+// costs one add per load and no predication.  MFMA step s of a K tile takes k = 8*half + s from both operands (any
+// bijection of k works as long as A and B agree).
+constexpr int ALS = GBK + 4;   // LDS row stride of a [row][k] tile (floats)
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned OUTSIDE = 0x80000000u;   // an offset beyond every descriptor (the host keeps them below 2^31 bytes)
+
+// One operand of the fast kernels.  XI = MFMA tiles per wavefront along this operand's extent (tile extent T = 64*XI);
+// KROWS = true for the K x rows memory layout.
+template <int XI, bool KROWS>
+struct FastOperand {
+    static constexpr int T = 64 * XI;
+    static constexpr int LDS_FLOATS = KROWS ? 2 * GBK * (T + 4) : 2 * T * ALS;
+    static constexpr int Q = T / 4, PASS_ROWS = 256 / Q;   // K x rows: float4 per K row, K rows covered per pass
+    float *lds;
+    __amdgpu_buffer_rsrc_t rsrc;
+    unsigned off[XI];
+    unsigned step;          // byte step of one K tile
+    f32x4 st[XI];
+    int kq;                 // rows x K: the thread's k quad
+    bool ragged_k;
+    int K;
+
+    // base: the operand's matrix (batch applied); extent rows, row stride rs (elements), first row / column r0 of the tile
+    __device__ __forceinline__ void init(float *lds_, const float *base, int extent, long long rs, int r0, int K_, int tid) {
+        lds = lds_;
+        K = K_;
+        ragged_k = (K % GBK) != 0;
+        if (KROWS) {
+            const int krow = tid / Q, rq = (tid % Q) * 4;
+            rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(base + r0), 0, (int)((((long long)K - 1) * rs + (extent - r0)) * 4), 0x00020000);
+#pragma unroll
+            for (int i = 0; i < XI; ++i) off[i] = (r0 + rq < extent) ? (unsigned)((krow + PASS_ROWS * i) * (int)rs + rq) * 4u : OUTSIDE;
+            step = (unsigned)GBK * (unsigned)rs * 4u;
+            kq = 0;
+        } else {
+            const int row = tid >> 2;
+            kq = (tid & 3) * 4;
+            const long long rem = ((long long)(extent - r0 - 1) * rs + K) * 4;
+            rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(base + (long long)r0 * rs), 0, (int)(rem < 0x7fffffffll ? rem : 0x7fffffffll), 0x00020000);
+#pragma unroll
+            for (int i = 0; i < XI; ++i) off[i] = (r0 + row + 64 * i < extent) ? (unsigned)((row + 64 * i) * (int)rs + kq) * 4u : OUTSIDE;
+            step = (unsigned)GBK * 4u;
+        }
+    }
+    __device__ __forceinline__ void load(int kt) {
+        // rows x K on the last K step of a ragged K: quads at or past K lie inside the next row, so they are sent outside
+        const bool past = !KROWS && ragged_k && (kt * GBK + kq >= K);
+#pragma unroll
+        for (int i = 0; i < XI; ++i)
+            st[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(past ? OUTSIDE : off[i] + kt * step), 0, 0));
+    }
+    __device__ __forceinline__ void store(int buf, int tid) {
+        if (KROWS) {
+            const int krow = tid / Q, rq = (tid % Q) * 4;
+#pragma unroll
+            for (int i = 0; i < XI; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * GBK + krow + PASS_ROWS * i) * (T + 4) + rq) = st[i];
+        } else {
+            const int row = tid >> 2;
+#pragma unroll
+            for (int i = 0; i < XI; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * T + row + 64 * i) * ALS + kq) = st[i];
+        }
+    }
+    // rows x K: the lane's fragment of tile x for the whole K tile (k = 8*half .. 8*half + 7)
+    __device__ __forceinline__ void fragment(int buf, int row, int half, f32x4 (&f)[2]) const {
+        f[0] = *reinterpret_cast<const f32x4 *>(lds + (buf * T + row) * ALS + 8 * half);
+        f[1] = *reinterpret_cast<const f32x4 *>(lds + (buf * T + row) * ALS + 8 * half + 4);
+    }
+    // K x rows: the lane's value for MFMA step s8
+    __device__ __forceinline__ float word(int buf, int row, int half, int s8) const { return lds[(buf * GBK + 8 * half + s8) * (T + 4) + row]; }
+};
 
 // MI x NI = MFMA tiles per wavefront (2x2: 128x128 workgroup tile for large products, 1x1: 64x64 so that small
-// products still put a workgroup on every CU).
-template <int MI, int NI, bool EPI>
-__global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
+// products still put a workgroup on every CU).  TA / TB: the operand is stored transposed (transposeFirst / Second).
+template <int MI, int NI, bool EPI, bool TA, bool TB>
+__global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
     constexpr int TM = 64 * MI, TN = 64 * NI;       // workgroup tile
-    constexpr int BLS = TN + 4;                      // B LDS row stride (floats)
-    __shared__ __align__(16) float As[2][TM][ALS];
-    __shared__ __align__(16) float Bs[2][GBK][BLS];
+    using OpA = FastOperand<MI, TA>;                 // A is M x K in memory unless transposed
+    using OpB = FastOperand<NI, !TB>;                // B is K x N in memory unless transposed
+    __shared__ __align__(16) float As[OpA::LDS_FLOATS];
+    __shared__ __align__(16) float Bs[OpB::LDS_FLOATS];
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int half = lane >> 5, ln = lane & 31;
     const int wm = wave >> 1, wn = wave & 1;
     const int tile_m = blockIdx.x / g.tiles_n, tile_n = blockIdx.x % g.tiles_n;
     const int m0 = tile_m * TM, n0 = tile_n * TN;
-    const float *A = g.A + (long long)blockIdx.z * g.a_bs;
-    const float *B = g.B + (long long)blockIdx.z * g.b_bs;
     float *C = g.C + (long long)blockIdx.z * g.c_bs;
 
-    // loaders: A tile TM x 16 = TM*4 float4: thread -> rows (tid/4 + 64*i), k quad tid%4;
-    //          B tile 16 x TN = 4*TN float4: thread -> row (tid / (TN/4) + (1024/TN)*i), n quad tid % (TN/4).
-    // Both through buffer loads with the whole byte offset in the (range-checked) vector operand: rows of A past M,
-    // rows of B past K and -- through an offset beyond any descriptor -- columns of B past N read as zeros, so a K step
-    // costs one add per load and no predication.
-    constexpr int BQ = TN / 4, BROWS = 256 / BQ;     // float4 per B row, B rows covered per pass
-    constexpr unsigned OUTSIDE = 0x80000000u;        // the host keeps every descriptor below 2^31 bytes
-    const int a_row = tid >> 2, a_kq = (tid & 3) * 4;
-    const int b_row = tid / BQ, b_nq = (tid % BQ) * 4;
-    const long long a_rem = ((long long)(g.M - m0 - 1) * g.a_rs + g.K) * 4;
-    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(A + (long long)m0 * g.a_rs), 0, (int)(a_rem < 0x7fffffffll ? a_rem : 0x7fffffffll), 0x00020000);
-    const __amdgpu_buffer_rsrc_t brsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(B + n0), 0, (int)((((long long)g.K - 1) * g.b_rs + (g.N - n0)) * 4), 0x00020000);
-    unsigned a_off[MI], b_off[NI];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-        a_off[i] = (m0 + a_row + 64 * i < g.M) ? (unsigned)((a_row + 64 * i) * (int)g.a_rs + a_kq) * 4u : OUTSIDE;
-#pragma unroll
-    for (int i = 0; i < NI; ++i)
-        b_off[i] = (n0 + b_nq < g.N) ? (unsigned)((b_row + BROWS * i) * (int)g.b_rs + b_nq) * 4u : OUTSIDE;
-    const bool ragged_k = (g.K % GBK) != 0;
-    const unsigned b_step = (unsigned)GBK * (unsigned)g.b_rs * 4u;
-    f32x4 ast[MI], bst[NI];
-    auto load = [&](int kt) {
-        const int k0 = kt * GBK;
-        // the last K step of a ragged K: quads at or past K lie inside the next row of A, so they are sent outside
-        const bool a_past = ragged_k && (k0 + a_kq >= g.K);
-#pragma unroll
-        for (int i = 0; i < MI; ++i)
-            ast[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                   arsrc, (int)(a_past ? OUTSIDE : a_off[i] + (unsigned)k0 * 4u), 0, 0));
-#pragma unroll
-        for (int i = 0; i < NI; ++i)
-            bst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(brsrc, (int)(b_off[i] + kt * b_step), 0, 0));
-    };
-    auto store = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < MI; ++i) *reinterpret_cast<f32x4 *>(&As[buf][a_row + 64 * i][a_kq]) = ast[i];
-#pragma unroll
-        for (int i = 0; i < NI; ++i) *reinterpret_cast<f32x4 *>(&Bs[buf][b_row + BROWS * i][b_nq]) = bst[i];
-    };
+    OpA opa;
+    OpB opb;
+    opa.init(As, g.A + (long long)blockIdx.z * g.a_bs, g.M, g.lda, m0, g.K, tid);
+    opb.init(Bs, g.B + (long long)blockIdx.z * g.b_bs, g.N, g.ldb, n0, g.K, tid);
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -214,35 +250,47 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_nn(GemmArgs g) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const int ktiles = (g.K + GBK - 1) / GBK;
-    load(0);
-    store(0);
+    opa.load(0);
+    opb.load(0);
+    opa.store(0, tid);
+    opb.store(0, tid);
     __syncthreads();
-    for (int kt = 0; kt < ktiles; ++kt) {
-        const int buf = kt & 1;
+    // one K step; the LDS buffer index is a compile-time constant (the loop below is unrolled by two) so that every LDS
+    // address is a per-thread base plus a literal
+    auto k_step = [&](const int kt, auto buf_c) {
+        constexpr int buf = decltype(buf_c)::value;
         const bool more = kt + 1 < ktiles;
-        if (more) load(kt + 1);
-        // A fragments of this K tile: row (wm*32*MI + i*32 + ln), k = 8*half .. 8*half+7
-        f32x4 af[MI][2];
+        if (more) { opa.load(kt + 1); opb.load(kt + 1); }
+        f32x4 af[MI][2], bf[NI][2];
+        if (!TA) {
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-            af[i][0] = *reinterpret_cast<const f32x4 *>(&As[buf][wm * 32 * MI + i * 32 + ln][8 * half]);
-            af[i][1] = *reinterpret_cast<const f32x4 *>(&As[buf][wm * 32 * MI + i * 32 + ln][8 * half + 4]);
+            for (int i = 0; i < MI; ++i) opa.fragment(buf, wm * 32 * MI + i * 32 + ln, half, af[i]);
+        }
+        if (TB) {
+#pragma unroll
+            for (int j = 0; j < NI; ++j) opb.fragment(buf, wn * 32 * NI + j * 32 + ln, half, bf[j]);
         }
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) {
-            float bv[NI];
+            float av[MI], bv[NI];
 #pragma unroll
-            for (int j = 0; j < NI; ++j) bv[j] = Bs[buf][8 * half + s8][wn * 32 * NI + j * 32 + ln];
+            for (int i = 0; i < MI; ++i) av[i] = TA ? opa.word(buf, wm * 32 * MI + i * 32 + ln, half, s8) : af[i][s8 >> 2][s8 & 3];
+#pragma unroll
+            for (int j = 0; j < NI; ++j) bv[j] = TB ? bf[j][s8 >> 2][s8 & 3] : opb.word(buf, wn * 32 * NI + j * 32 + ln, half, s8);
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
                 for (int j = 0; j < NI; ++j)
                     // operands swapped: the accumulator is the TRANSPOSED tile (lane = row m, registers = columns n), so
                     // that a lane holds four consecutive columns and the epilogue moves 128 bits per access
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], af[i][s8 >> 2][s8 & 3], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
         }
-        if (more) store(buf ^ 1);
+        if (more) { opa.store(buf ^ 1, tid); opb.store(buf ^ 1, tid); }
         __syncthreads();
+    };
+    for (int kt = 0; kt < ktiles; kt += 2) {
+        k_step(kt, std::integral_constant<int, 0>{});
+        if (kt + 1 < ktiles) k_step(kt + 1, std::integral_constant<int, 1>{});
     }
 
     // accumulator register r of a transposed 32x32 tile: row m = lane % 32, column n = 8*(r/4) + 4*half + r%4
@@ -303,14 +351,18 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.a_rs = ta ? 1 : lc; g.a_cs = ta ? lc : 1;
     g.b_rs = tb ? 1 : rc; g.b_cs = tb ? rc : 1;
     g.a_bs = lbs; g.b_bs = rbs; g.c_bs = cbs;
+    g.lda = lc; g.ldb = rc;
     g.alpha = alpha; g.beta = beta;
     g.bias = bias; g.residual = residual; g.act = act;
     const bool epi = bias || residual || act;
     const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    // the fast kernels address A within a tile's rows and B as a whole through 32-bit byte offsets below 2^31
-    const bool fast = !ta && !tb && K % 4 == 0 && N % 4 == 0 && K > 0 && aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 &&
-                      rbs % 4 == 0 && K < (1ll << 21) && K * N * 4 < (1ll << 31) && aligned16(result) && cbs % 4 == 0 &&
-                      aligned16(bias) && aligned16(residual);
+    // The fast kernels: every unit-stride extent a multiple of 4 (128-bit accesses), 16-byte aligned operands, and 32-bit
+    // byte offsets below 2^31 (an operand stored rows x K is addressed within a tile's 128 rows, one stored K x rows as a whole).
+    const auto rows_by_k_ok = [&](int64_t ld) { return K % 4 == 0 && ld < (1ll << 21); };
+    const auto k_by_rows_ok = [&](int64_t extent, int64_t ld) { return extent % 4 == 0 && K * ld * 4 < (1ll << 31); };
+    const bool fast = K > 0 && N % 4 == 0 && (ta ? k_by_rows_ok(M, lc) : rows_by_k_ok(lc)) && (tb ? rows_by_k_ok(rc) : k_by_rows_ok(N, rc)) &&
+                      aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 && rbs % 4 == 0 && aligned16(result) && cbs % 4 == 0 &&
+                      aligned16(bias) && aligned16(residual) && !(epi && (ta || tb));
     long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
     // small products: 64x64 tiles, so that there are at least about two workgroups per CU
     const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;
@@ -318,10 +370,23 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.tiles_n = (int)tn;
     DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
     const dim3 grid((unsigned)(tm * tn), 1, (unsigned)batch);
-    if (small && epi) hipLaunchKernelGGL((gemm_f32_mfma_nn<1, 1, true>), grid, dim3(256), 0, ctx->stream, g);
-    else if (small) hipLaunchKernelGGL((gemm_f32_mfma_nn<1, 1, false>), grid, dim3(256), 0, ctx->stream, g);
-    else if (fast && epi) hipLaunchKernelGGL((gemm_f32_mfma_nn<2, 2, true>), grid, dim3(256), 0, ctx->stream, g);
-    else if (fast) hipLaunchKernelGGL((gemm_f32_mfma_nn<2, 2, false>), grid, dim3(256), 0, ctx->stream, g);
+#define DL4S_GEMM_FAST(MI_, EPI_, TA_, TB_) hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_>), grid, dim3(256), 0, ctx->stream, g)
+    if (fast) {
+        const int variant = (small ? 0 : 8) + (epi ? 4 : 0) + (ta ? 2 : 0) + (tb ? 1 : 0);
+        switch (variant) {
+            case 0: DL4S_GEMM_FAST(1, false, false, false); break;
+            case 1: DL4S_GEMM_FAST(1, false, false, true); break;
+            case 2: DL4S_GEMM_FAST(1, false, true, false); break;
+            case 3: DL4S_GEMM_FAST(1, false, true, true); break;
+            case 4: DL4S_GEMM_FAST(1, true, false, false); break;
+            case 8: DL4S_GEMM_FAST(2, false, false, false); break;
+            case 9: DL4S_GEMM_FAST(2, false, false, true); break;
+            case 10: DL4S_GEMM_FAST(2, false, true, false); break;
+            case 11: DL4S_GEMM_FAST(2, false, true, true); break;
+            default: DL4S_GEMM_FAST(2, true, false, false); break;   // 12: epilogue forms are never transposed
+        }
+    }
+#undef DL4S_GEMM_FAST
     else hipLaunchKernelGGL(gemm_f32_mfma, grid, dim3(256), 0, ctx->stream, g);
     return dl4s::launch_status("gemm_f32_mfma");
 }

@@ -83,7 +83,8 @@ def test_elementwise_bit_exact(ctx, orc):
 
 @pytest.mark.parametrize("ta", [False, True])
 @pytest.mark.parametrize("tb", [False, True])
-@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 7, 6), (128, 128, 16), (130, 70, 33), (257, 129, 100), (64, 512, 512)])
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (5, 7, 6), (128, 128, 16), (130, 70, 33), (257, 129, 100), (64, 512, 512),
+                                   (260, 132, 100), (516, 260, 36), (8, 4, 4), (1028, 1284, 520)])   # the last four: ragged tiles on the fast kernels
 def test_gemm(ctx, orc, ta, tb, M, N, K):
     A = rnd(K, M) if ta else rnd(M, K)
     B = rnd(N, K) if tb else rnd(K, N)
