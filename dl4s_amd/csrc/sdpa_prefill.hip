@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     const int hh = bh % H;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: lets the per-wavefront tile conditions branch on scalars
     const int lane = tid & 63;
     const int half = lane >> 5;
     const int ln = lane & 31;
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
                                                                       float *__restrict__ stats) {
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: lets the per-wavefront tile conditions branch on scalars
     const int lane = tid & 63;
     const int half = lane >> 5;
     const int ln = lane & 31;
