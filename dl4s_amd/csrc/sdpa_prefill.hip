@@ -23,6 +23,8 @@
 // Kernels in this file: sdpa_prefill_f32_d64 (above), sdpa_prefill_split_f32_d64 (small launches: the keys of a
 // 32-query block split over the 4 wavefronts of a workgroup), sdpa_generic_f32 (head dims other than 64).  Both MFMA
 // kernels can also leave the two row statistics the backward pass needs (sdpa_backward.hip).
+#include <type_traits>
+
 #include "sdpa_common.h"
 
 namespace {
@@ -197,8 +199,10 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;   // wavefronts past Lq store nothing
 
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
+    // one key tile; the LDS buffer index is a compile-time constant (the loop is unrolled by two), so every LDS address
+    // in the step is a per-thread base plus a literal
+    auto tile_step = [&](const int t, auto buf_c) {
+        constexpr int buf = decltype(buf_c)::value;
         const bool more = (t + 1 < ntiles);
         if (more) load_tile(t + 1);
         const int k0 = t * BN;
@@ -212,6 +216,10 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
 
         if (more) store_tile(buf ^ 1);
         __syncthreads();
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        tile_step(t, std::integral_constant<int, 0>{});
+        if (t + 1 < ntiles) tile_step(t + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- normalise and store.  Register r of o0/o1 is d = 2*(8(r/4) + 4*half + r%4) + {0,1}.
