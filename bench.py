@@ -93,6 +93,13 @@ def decode(ctx, lib, repeats):
         ctx.timer_begin()
         run()
         per_step_us.append(ctx.timer_end() * 1e3 / steps)
+    # the distribution over single steps: every step of one more pass bracketed by its own pair of events
+    single_us = []
+    for t in range(steps):
+        ctx.timer_begin()
+        ctx.sdpa_decode_step(qs.offset(t * sb), kc, vc, kn.offset(t * sb), vn.offset(t * sb), out.offset(t * sb),
+                             B, H, T0 + t, Tcap, d, 0.125)
+        single_us.append(ctx.timer_end() * 1e3)
     o = out.numpy()
     if not np.isfinite(o).all():
         raise RuntimeError("decode output failed its sanity check")
@@ -103,6 +110,7 @@ def decode(ctx, lib, repeats):
     Tavg = T0 + (steps + 1) / 2.0
     bytes_step = 2 * B * H * Tavg * d * 4 + 2 * B * H * d * 4 + 2 * B * H * d * 4
     return {"us_per_step": us, "us_per_step_min": float(np.min(per_step_us)), "tokens_per_s": B / (us * 1e-6),
+            "single_step_us_p50": float(np.percentile(single_us, 50)), "single_step_us_p99": float(np.percentile(single_us, 99)),
             "bytes_per_step": bytes_step, "gbs": bytes_step / (us * 1e-6) / 1e9,
             "shape": {"B": B, "H": H, "d": d, "T0": T0, "steps": steps}}
 
@@ -323,6 +331,7 @@ def main():
         line["decode"] = {"workload": "incremental decode B=16 H=16 d=64, KV cache 4096 rows + 64 append+attend steps "
                                       "(BASELINE config 5)",
                           "us_per_step": dec["us_per_step"], "tokens_per_s": dec["tokens_per_s"],
+                          "single_step_us_p50": dec["single_step_us_p50"], "single_step_us_p99": dec["single_step_us_p99"],
                           "roofline": {"bound": "hbm", "achieved": dec["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                        "frac": dec["gbs"] / HBM_PEAK_GBS, "traffic": DECODE_TRAFFIC_BYTES,
                                        "kernel": "sdpa_decode_splitk_f32", "bytes_per_step": dec["bytes_per_step"]}}
