@@ -271,6 +271,26 @@ def cpu_baseline_prefill(q, k, v, pairs):
                                                                              os.cpu_count() or 0)}
 
 
+def cpu_blas_proxy_prefill(q, k, v, pairs):
+    """The same materialised-score structure with the products handed to the host's threaded BLAS (numpy): a stand-in for
+    the reference built against MKL (-DMKL_ENABLE), NOT the reference binary and not the parity oracle."""
+    L, d = q.shape[2], q.shape[3]
+    i, j = np.indices((L, L))
+    pen = (j > i).astype(np.float32) * np.float32(1e9)
+    t0 = time.perf_counter()
+    for p in range(pairs):
+        b, h = divmod(p, q.shape[1])
+        s = (q[b, h] * np.float32(0.125)) @ k[b, h].T - pen
+        s -= s.max(axis=1, keepdims=True)
+        np.exp(s, out=s)
+        s *= np.float32(1.0) / s.sum(axis=1, keepdims=True)
+        s @ v[b, h]
+    dt = time.perf_counter() - t0
+    flops = 4.0 * d * pairs * (L * (L + 1) // 2)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": os.cpu_count() or 0, "kind": "proxy (numpy + threaded BLAS)",
+            "sample": "%d (batch, head) slices, %.1f s" % (pairs, dt)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -338,6 +358,7 @@ def main():
     if args.cpu_pairs > 0:
         q, k, v = pre["inputs"]
         line["cpu_baseline"] = cpu_baseline_prefill(q, k, v, args.cpu_pairs)
+        line["cpu_blas_proxy"] = cpu_blas_proxy_prefill(q, k, v, min(32, q.shape[0] * q.shape[1]))
         if dec:
             line["decode"]["cpu_baseline"] = cpu_baseline_decode()
     if others is not None:
