@@ -96,24 +96,36 @@ struct Reduce {
     long long rcount;
 };
 
+// One workgroup per (output element, part): blockIdx.x = output, blockIdx.y = part of the reduced range
+// [part * chunk, min(rcount, (part + 1) * chunk)); the result goes to y[output * gridDim.y + part].
 template <bool IS_MAX>
-__global__ __launch_bounds__(TPB) void reduce_f32(const float *__restrict__ x, float *__restrict__ y, Reduce rd) {
+__global__ __launch_bounds__(TPB) void reduce_f32(const float *__restrict__ x, float *__restrict__ y, Reduce rd, long long chunk) {
     __shared__ float sm[TPB / 64];
     long long o = blockIdx.x, base = 0;
     for (int i = rd.kdim - 1; i >= 0; --i) {
         base += (o % rd.kshape[i]) * rd.kstride[i];
         o /= rd.kshape[i];
     }
+    const long long j0 = (long long)blockIdx.y * chunk, j1 = min(rd.rcount, j0 + chunk);
     float acc = IS_MAX ? -INFINITY : 0.f;
-    for (long long j = threadIdx.x; j < rd.rcount; j += TPB) {
-        long long rem = j, off = base;
-        for (int i = rd.rdim - 1; i >= 0; --i) {
-            off += (rem % rd.rshape[i]) * rd.rstride[i];
-            rem /= rd.rshape[i];
+    if (rd.rdim == 1) {     // one (merged) reduced axis: no index arithmetic beyond a multiply
+        const long long rs = rd.rstride[0];
+        for (long long j = j0 + threadIdx.x; j < j1; j += TPB) {
+            const float v = x[base + j * rs];
+            if (IS_MAX) acc = fmaxf(acc, v);   // NaN never selected, like the reference's "v > max" scan
+            else acc += v;
         }
-        const float v = x[off];
-        if (IS_MAX) acc = fmaxf(acc, v);   // NaN never selected, like the reference's "v > max" scan
-        else acc += v;
+    } else {
+        for (long long j = j0 + threadIdx.x; j < j1; j += TPB) {
+            long long rem = j, off = base;
+            for (int i = rd.rdim - 1; i >= 0; --i) {
+                off += (rem % rd.rshape[i]) * rd.rstride[i];
+                rem /= rd.rshape[i];
+            }
+            const float v = x[off];
+            if (IS_MAX) acc = fmaxf(acc, v);
+            else acc += v;
+        }
     }
     for (int s = 32; s > 0; s >>= 1) {
         const float t = __shfl_xor(acc, s, 64);
@@ -124,7 +136,7 @@ __global__ __launch_bounds__(TPB) void reduce_f32(const float *__restrict__ x, f
     if (threadIdx.x == 0) {
         float r = sm[0];
         for (int w = 1; w < TPB / 64; ++w) r = IS_MAX ? fmaxf(r, sm[w]) : r + sm[w];
-        y[blockIdx.x] = r;
+        y[(long long)blockIdx.x * gridDim.y + blockIdx.y] = r;
     }
 }
 
@@ -457,15 +469,55 @@ static int reduce_common(dl4s_hip_ctx *ctx, bool is_max, const float *values, co
         s *= shape[i];
     }
     rd.rcount = 1;
+    // neighbouring axes of the same kind are merged (the tensor is contiguous), so that e.g. LayerNorm's sum over
+    // (length, hidden) is one reduced axis of stride 1
     for (int i = 0; i < dim; ++i) {
-        if (red[i]) { rd.rshape[rd.rdim] = shape[i]; rd.rstride[rd.rdim] = stride[i]; rd.rcount *= shape[i]; ++rd.rdim; }
-        else { rd.kshape[rd.kdim] = shape[i]; rd.kstride[rd.kdim] = stride[i]; nout *= shape[i]; ++rd.kdim; }
+        if (shape[i] == 1) continue;    // extent 1 contributes nothing to either index
+        if (red[i]) {
+            if (rd.rdim > 0 && i > 0 && red[i - 1] && shape[i - 1] != 1) { rd.rshape[rd.rdim - 1] *= shape[i]; rd.rstride[rd.rdim - 1] = stride[i]; }
+            else { rd.rshape[rd.rdim] = shape[i]; rd.rstride[rd.rdim] = stride[i]; ++rd.rdim; }
+            rd.rcount *= shape[i];
+        } else {
+            if (rd.kdim > 0 && i > 0 && !red[i - 1] && shape[i - 1] != 1) { rd.kshape[rd.kdim - 1] *= shape[i]; rd.kstride[rd.kdim - 1] = stride[i]; }
+            else { rd.kshape[rd.kdim] = shape[i]; rd.kstride[rd.kdim] = stride[i]; ++rd.kdim; }
+            nout *= shape[i];
+        }
     }
+    for (int i = 0; i < dim; ++i)
+        if (shape[i] == 0) { if (red[i]) rd.rcount = 0; else nout = 0; }
     if (nout == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(values && result, DL4S_HIP_EINVALID_ARG, "reduce: NULL pointer");
     DL4S_REQUIRE(nout < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "reduce: too many output elements");
-    if (is_max) hipLaunchKernelGGL(reduce_f32<true>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, values, result, rd);
-    else hipLaunchKernelGGL(reduce_f32<false>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, values, result, rd);
+    // few outputs with long reduced ranges (LayerNorm statistics: one per batch item): split every range over several
+    // workgroups, partial results in the scratch block, then reduce the parts
+    long long parts = 1;
+    if (nout < 2ll * ctx->cu_count && rd.rcount >= 64ll * TPB) {
+        parts = (4ll * ctx->cu_count + nout - 1) / nout;
+        const long long most = rd.rcount / (8ll * TPB);
+        if (parts > most) parts = most;
+        if (parts > 1024) parts = 1024;
+        if (parts < 1) parts = 1;
+    }
+    if (parts == 1) {
+        if (is_max) hipLaunchKernelGGL(reduce_f32<true>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, values, result, rd, rd.rcount);
+        else hipLaunchKernelGGL(reduce_f32<false>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, values, result, rd, rd.rcount);
+        return dl4s::launch_status("reduce");
+    }
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
+    int rc = dl4s::ensure_scratch(ctx, (size_t)(nout * parts) * sizeof(float));
+    if (rc) return rc;
+    float *part = reinterpret_cast<float *>(ctx->scratch);
+    const long long chunk = (rd.rcount + parts - 1) / parts;
+    Reduce fin{};
+    fin.kdim = 1; fin.kshape[0] = nout; fin.kstride[0] = parts;
+    fin.rdim = 1; fin.rshape[0] = parts; fin.rstride[0] = 1; fin.rcount = parts;
+    if (is_max) {
+        hipLaunchKernelGGL(reduce_f32<true>, dim3((unsigned)nout, (unsigned)parts), dim3(TPB), 0, ctx->stream, values, part, rd, chunk);
+        hipLaunchKernelGGL(reduce_f32<true>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, part, result, fin, parts);
+    } else {
+        hipLaunchKernelGGL(reduce_f32<false>, dim3((unsigned)nout, (unsigned)parts), dim3(TPB), 0, ctx->stream, values, part, rd, chunk);
+        hipLaunchKernelGGL(reduce_f32<false>, dim3((unsigned)nout), dim3(TPB), 0, ctx->stream, part, result, fin, parts);
+    }
     return dl4s::launch_status("reduce");
 }
 

@@ -165,7 +165,9 @@ def test_broadcast_shape_error(ctx):
 
 
 @pytest.mark.parametrize("shape,axes", [((3, 4, 5), [2]), ((3, 4, 5), [1, 2]), ((3, 4, 5), [0]), ((2, 3, 4, 50), [3]),
-                                        ((2, 300, 70), [1, 2]), ((6,), [0]), ((4, 5), [0, 1])])
+                                        ((2, 300, 70), [1, 2]), ((6,), [0]), ((4, 5), [0, 1]), ((4, 512, 512), [1, 2]),
+                                        ((3, 1, 7, 1, 5), [1, 2]), ((2, 3, 4, 5), [0, 2]), ((2, 3, 4, 5), [1, 3]), ((1, 1), [0]),
+                                        ((700000,), [0]), ((2, 200, 1, 300), [1, 2, 3])])
 def test_reduce_sum(ctx, orc, shape, axes):
     x = rnd(*shape)
     ref = orc.reduce_sum(x, axes)
