@@ -180,6 +180,30 @@ __device__ __forceinline__ void block_sum2(float &a, float &b, float *sm) {
     for (int i = 0; i < TPB / 64; ++i) { a += sm[2 * i]; b += sm[2 * i + 1]; }
 }
 
+// LayerNorm kernels.  VEC: rows, D and the pointers allow 128-bit accesses (n % 4 == 0, D % 4 == 0, 16-byte alignment);
+// the arithmetic per element is the same either way.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 ln_load4(const float *xp, const float *rp, long long i) {
+    f32x4 v = *reinterpret_cast<const f32x4 *>(xp + i);
+    if (rp) {
+        const f32x4 r = *reinterpret_cast<const f32x4 *>(rp + i);
+        v.x = __fadd_rn(v.x, r.x); v.y = __fadd_rn(v.y, r.y); v.z = __fadd_rn(v.z, r.z); v.w = __fadd_rn(v.w, r.w);
+    }
+    return v;
+}
+
+__device__ __forceinline__ f32x4 ln_norm4(f32x4 v, float mean, float rden, const float *scale, const float *shift, long long d) {
+    const f32x4 sc = *reinterpret_cast<const f32x4 *>(scale + d), sh = *reinterpret_cast<const f32x4 *>(shift + d);
+    f32x4 y;
+    y.x = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.x, -mean), rden), sc.x), sh.x);
+    y.y = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.y, -mean), rden), sc.y), sh.y);
+    y.z = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.z, -mean), rden), sc.z), sh.z);
+    y.w = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.w, -mean), rden), sc.w), sh.w);
+    return y;
+}
+
+template <bool VEC>
 __global__ __launch_bounds__(TPB) void ln_partial_f32(const float *__restrict__ x, const float *__restrict__ res,
                                                        float *__restrict__ part, long long n, int nblk) {
     __shared__ float sm[2 * TPB / 64];
@@ -187,16 +211,25 @@ __global__ __launch_bounds__(TPB) void ln_partial_f32(const float *__restrict__ 
     const float *xp = x + b * n;
     const float *rp = res ? res + b * n : nullptr;
     float s = 0.f, ss = 0.f;
-    for (long long i = (long long)blockIdx.x * TPB + threadIdx.x; i < n; i += (long long)nblk * TPB) {
-        float v = xp[i];
-        if (rp) v = __fadd_rn(v, rp[i]);
-        s += v;
-        ss += __fmul_rn(v, v);
+    if (VEC) {
+        for (long long i = ((long long)blockIdx.x * TPB + threadIdx.x) * 4; i < n; i += (long long)nblk * TPB * 4) {
+            const f32x4 v = ln_load4(xp, rp, i);
+            s += (v.x + v.y) + (v.z + v.w);
+            ss += (__fmul_rn(v.x, v.x) + __fmul_rn(v.y, v.y)) + (__fmul_rn(v.z, v.z) + __fmul_rn(v.w, v.w));
+        }
+    } else {
+        for (long long i = (long long)blockIdx.x * TPB + threadIdx.x; i < n; i += (long long)nblk * TPB) {
+            float v = xp[i];
+            if (rp) v = __fadd_rn(v, rp[i]);
+            s += v;
+            ss += __fmul_rn(v, v);
+        }
     }
     block_sum2(s, ss, sm);
     if (threadIdx.x == 0) { part[(b * nblk + blockIdx.x) * 2] = s; part[(b * nblk + blockIdx.x) * 2 + 1] = ss; }
 }
 
+template <bool VEC>
 __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x, const float *__restrict__ res,
                                                      const float *__restrict__ scale, const float *__restrict__ shift,
                                                      float *__restrict__ y, const float *__restrict__ part, long long n,
@@ -211,17 +244,29 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     const float *xp = x + b * n;
     const float *rp = res ? res + b * n : nullptr;
     float *yp = y + b * n;
-    for (long long i = (long long)blockIdx.x * TPB + threadIdx.x; i < n; i += (long long)gridDim.x * TPB) {
-        float v = xp[i];
-        if (rp) v = __fadd_rn(v, rp[i]);
-        const float c = __fadd_rn(v, -mean);
-        const float nrm = __fmul_rn(c, rden);
-        const long long d = i % D;
-        yp[i] = __fadd_rn(__fmul_rn(nrm, scale[d]), shift[d]);
+    if (VEC) {
+        // the column of element i advances by a constant per iteration: no division in the loop
+        const long long step = (long long)gridDim.x * TPB * 4, dstep = step % D;
+        long long i = ((long long)blockIdx.x * TPB + threadIdx.x) * 4, d = i % D;
+        for (; i < n; i += step) {
+            *reinterpret_cast<f32x4 *>(yp + i) = ln_norm4(ln_load4(xp, rp, i), mean, rden, scale, shift, d);
+            d += dstep;
+            if (d >= D) d -= D;
+        }
+    } else {
+        for (long long i = (long long)blockIdx.x * TPB + threadIdx.x; i < n; i += (long long)gridDim.x * TPB) {
+            float v = xp[i];
+            if (rp) v = __fadd_rn(v, rp[i]);
+            const float c = __fadd_rn(v, -mean);
+            const float nrm = __fmul_rn(c, rden);
+            const long long d = i % D;
+            yp[i] = __fadd_rn(__fmul_rn(nrm, scale[d]), shift[d]);
+        }
     }
 }
 
 // one workgroup per batch item, for short rows (per-token LayerNorm of the feed-forward block)
+template <bool VEC>
 __global__ __launch_bounds__(TPB) void ln_small_f32(const float *__restrict__ x, const float *__restrict__ res,
                                                      const float *__restrict__ scale, const float *__restrict__ shift,
                                                      float *__restrict__ y, long long n, long long D) {
@@ -229,25 +274,48 @@ __global__ __launch_bounds__(TPB) void ln_small_f32(const float *__restrict__ x,
     const long long b = blockIdx.x;
     const float *xp = x + b * n;
     const float *rp = res ? res + b * n : nullptr;
-    float s = 0.f, ss = 0.f;
-    for (long long i = threadIdx.x; i < n; i += TPB) {
-        float v = xp[i];
-        if (rp) v = __fadd_rn(v, rp[i]);
-        s += v;
-        ss += __fmul_rn(v, v);
-    }
-    block_sum2(s, ss, sm);
-    const float rN = __fdiv_rn(1.0f, (float)n);
-    const float mean = __fmul_rn(s, rN);
-    const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
-    const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
     float *yp = y + b * n;
-    for (long long i = threadIdx.x; i < n; i += TPB) {
-        float v = xp[i];
-        if (rp) v = __fadd_rn(v, rp[i]);
-        const float nrm = __fmul_rn(__fadd_rn(v, -mean), rden);
-        const long long d = i % D;
-        yp[i] = __fadd_rn(__fmul_rn(nrm, scale[d]), shift[d]);
+    float s = 0.f, ss = 0.f;
+    if (VEC) {
+        const bool one = n <= (long long)TPB * 4;      // the whole row in one 128-bit access per thread: keep it in registers
+        f32x4 keep = {0.f, 0.f, 0.f, 0.f};
+        for (long long i = (long long)threadIdx.x * 4; i < n; i += (long long)TPB * 4) {
+            const f32x4 v = ln_load4(xp, rp, i);
+            if (one) keep = v;
+            s += (v.x + v.y) + (v.z + v.w);
+            ss += (__fmul_rn(v.x, v.x) + __fmul_rn(v.y, v.y)) + (__fmul_rn(v.z, v.z) + __fmul_rn(v.w, v.w));
+        }
+        block_sum2(s, ss, sm);
+        const float rN = __fdiv_rn(1.0f, (float)n);
+        const float mean = __fmul_rn(s, rN);
+        const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
+        const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
+        const long long step = (long long)TPB * 4, dstep = step % D;
+        long long i = (long long)threadIdx.x * 4, d = i % D;
+        for (; i < n; i += step) {
+            *reinterpret_cast<f32x4 *>(yp + i) = ln_norm4(one ? keep : ln_load4(xp, rp, i), mean, rden, scale, shift, d);
+            d += dstep;
+            if (d >= D) d -= D;
+        }
+    } else {
+        for (long long i = threadIdx.x; i < n; i += TPB) {
+            float v = xp[i];
+            if (rp) v = __fadd_rn(v, rp[i]);
+            s += v;
+            ss += __fmul_rn(v, v);
+        }
+        block_sum2(s, ss, sm);
+        const float rN = __fdiv_rn(1.0f, (float)n);
+        const float mean = __fmul_rn(s, rN);
+        const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
+        const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
+        for (long long i = threadIdx.x; i < n; i += TPB) {
+            float v = xp[i];
+            if (rp) v = __fadd_rn(v, rp[i]);
+            const float nrm = __fmul_rn(__fadd_rn(v, -mean), rden);
+            const long long d = i % D;
+            yp[i] = __fadd_rn(__fmul_rn(nrm, scale[d]), shift[d]);
+        }
     }
 }
 
@@ -675,8 +743,11 @@ int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *resid
     if (B * n == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(x && scale && shift && result, DL4S_HIP_EINVALID_ARG, "layernorm: NULL pointer");
     DL4S_REQUIRE(B < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "layernorm: batch too large");
+    const auto a16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool vec = n % 4 == 0 && D % 4 == 0 && a16(x) && a16(residual) && a16(scale) && a16(shift) && a16(result);
     if (n <= 16384) {
-        hipLaunchKernelGGL(ln_small_f32, dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+        if (vec) hipLaunchKernelGGL(ln_small_f32<true>, dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+        else hipLaunchKernelGGL(ln_small_f32<false>, dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
         return dl4s::launch_status("layernorm");
     }
     DL4S_REQUIRE(B <= 65535, DL4S_HIP_EUNSUPPORTED, "layernorm: batch above 65535 with long rows");
@@ -686,9 +757,15 @@ int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *resid
     int rc = dl4s::ensure_scratch(ctx, (size_t)B * nblk * 2 * sizeof(float));
     if (rc) return rc;
     float *part = reinterpret_cast<float *>(ctx->scratch);
-    hipLaunchKernelGGL(ln_partial_f32, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, part, n, nblk);
-    hipLaunchKernelGGL(ln_apply_f32, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, part, n,
-                       (long long)D, nblk);
+    if (vec) {
+        hipLaunchKernelGGL(ln_partial_f32<true>, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, part, n, nblk);
+        hipLaunchKernelGGL(ln_apply_f32<true>, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, part,
+                           n, (long long)D, nblk);
+    } else {
+        hipLaunchKernelGGL(ln_partial_f32<false>, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, part, n, nblk);
+        hipLaunchKernelGGL(ln_apply_f32<false>, dim3(nblk, (unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, part,
+                           n, (long long)D, nblk);
+    }
     return dl4s::launch_status("layernorm");
 }
 

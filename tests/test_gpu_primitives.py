@@ -215,7 +215,8 @@ def test_band_and_decoder_mask_recipe(ctx, orc):
     dy.release()
 
 
-@pytest.mark.parametrize("B,rows,D", [(3, 7, 16), (5, 1, 1024), (4, 512, 512), (2, 1, 33)])
+@pytest.mark.parametrize("B,rows,D", [(3, 7, 16), (5, 1, 1024), (4, 512, 512), (2, 1, 33), (3, 1, 4096), (2, 300, 68), (2, 2000, 33),
+                                       (6, 1, 12), (2, 40, 1028)])   # vector and scalar paths, short and long rows, D not dividing the stride
 def test_layernorm(ctx, orc, B, rows, D):
     x, res = rnd(B, rows, D) * 2 + np.float32(0.3), rnd(B, rows, D)
     scale, shift = rnd(D), rnd(D)
