@@ -291,6 +291,55 @@ def cpu_blas_proxy_prefill(q, k, v, pairs):
             "sample": "%d (batch, head) slices, %.1f s" % (pairs, dt)}
 
 
+def kernel_sample(ctx, lib, iters):
+    """A short fixed sequence of the kernels behind configs 3 and 4 that the headline run does not time one by one (the
+    fused Dense products, the dense-mask attention of config 3, the attention gradients), `iters` launches each, for
+    counter runs of a profiler: no pre-heat loops, a few dozen launches in all.  Returns the mean event time of each."""
+    rng = np.random.Generator(np.random.PCG64(1007))
+    res = {}
+
+    def timed(name, fn):
+        fn()
+        ctx.sync()
+        ctx.timer_begin()
+        for _ in range(iters):
+            fn()
+        res[name] = {"us_per_launch": ctx.timer_end() * 1e3 / iters}
+    M, D, F = 8192, 1024, 4096
+    x, h = ctx.to_device(rng.standard_normal((M, D), dtype=np.float32)), ctx.empty((M, F))
+    w1, w2 = ctx.to_device(rng.standard_normal((D, F), dtype=np.float32) * 0.03), ctx.to_device(rng.standard_normal((F, D), dtype=np.float32) * 0.03)
+    wq, b1, b2, y = ctx.to_device(rng.standard_normal((D, D), dtype=np.float32) * 0.03), ctx.empty((F,)), ctx.empty((D,)), ctx.empty((M, D))
+    ctx.fill(0.0, b1, F)
+    ctx.fill(0.0, b2, D)
+    timed("projection_8192x1024x1024", lambda: ctx.gemm(x, (M, D), wq, (D, D), y))
+    timed("ffn_up_gelu_8192x1024x4096", lambda: ctx.dense_fused(x, M, D, w1, F, b1, lib.ACT_GELU, None, h))
+    timed("ffn_down_residual_8192x4096x1024", lambda: ctx.dense_fused(h, M, F, w2, D, b2, lib.ACT_NONE, x, y))
+    timed("fc_residual_8192x1024x1024", lambda: ctx.dense_fused(x, M, D, wq, D, None, lib.ACT_NONE, x, y))
+    for b_ in (x, h, w1, w2, wq, b1, b2, y):
+        b_.release()
+    B, H, L = 8, 16, 1024
+    q, k, v = (ctx.to_device(rng.standard_normal((B, L, H, 64), dtype=np.float32)) for _ in range(3))
+    lens = rng.integers(512, 1025, size=B)
+    mask = ctx.to_device((np.arange(L)[None, None, None, :] >= lens[:, None, None, None]).astype(np.float32))
+    out = ctx.empty((B, L, H, 64))
+    desc = ctx.mask_desc(lib.MASK_DENSE, dense=mask)
+    timed("attention_config3_dense_padding_mask_token_major",
+          lambda: ctx.sdpa_fwd(q, k, v, out, B, H, L, L, 64, 64, 0.125, desc, lib.SDPA_STRICT | lib.SDPA_TOKEN_MAJOR))
+    for b_ in (q, k, v, mask, out):
+        b_.release()
+    B, H, L = 8, 16, 2048
+    bufs = [ctx.to_device(rng.standard_normal((B, H, L, 64), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
+    outs = [ctx.empty((B, H, L, 64)) for _ in range(4)]
+    st = ctx.empty((B, H, L, 2))
+    desc = ctx.mask_desc(lib.MASK_CAUSAL)
+    ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], outs[0], st, B, H, L, L, 64, 0.125, desc, 0)
+    timed("attention_backward_config4_causal",
+          lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, 64, 0.125, desc, 0))
+    for b_ in bufs + outs + [st]:
+        b_.release()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -303,6 +352,10 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one streaming kernel (negate, 1 GiB read + 1 GiB written) so that a counter run of "
                          "this command can scale FETCH_SIZE / WRITE_SIZE by a kernel of known traffic")
+    ap.add_argument("--kernel-sample", type=int, default=0, metavar="N",
+                    help="instead of the benchmark, launch the kernels behind configs 3 and 4 (fused Dense products, dense-mask "
+                         "attention, attention gradients) N times each and print their mean event times: a short command for "
+                         "profiler counter runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (every attention problem fits one MI355X); --gpus %d is not "
@@ -312,6 +365,10 @@ def main():
     from dl4s_amd import lib
     ctx = lib.Context(0)
     info = ctx.device_info()
+    if args.kernel_sample > 0:
+        print(json.dumps({"kernel_sample": kernel_sample(ctx, lib, args.kernel_sample)}))
+        ctx.close()
+        return
     pre = prefill(ctx, lib, args.steps, args.warmup)
     dec = decode(ctx, lib, args.decode_repeats) if args.decode_repeats > 0 else None
     if args.copy_calibration:
