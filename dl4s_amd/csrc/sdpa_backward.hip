@@ -23,13 +23,13 @@ constexpr float LN2 = 0.69314718055994530942f;
 
 // D[b,h,i] = sum_d dout[i][d] * out[i][d]; 16 lanes per row, four rows per wavefront
 __global__ __launch_bounds__(256) void sdpa_bwd_rowdot(const float *__restrict__ out, const float *__restrict__ dout,
-                                                       float *__restrict__ D, int H, int Lq, long long rows, int token_major) {
+                                                       float *__restrict__ D, int H, int Lq, long long rows, int token_major, int hd) {
     const long long r = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
     const int c = (threadIdx.x & 15) * 4;
     float acc = 0.f;
-    if (r < rows) {
+    if (r < rows && c < hd) {
         const long long bh = r / Lq, qi = r % Lq;
-        const long long off = token_major ? (((bh / H) * Lq + qi) * H + bh % H) * HD : r * HD;
+        const long long off = token_major ? (((bh / H) * Lq + qi) * H + bh % H) * hd : r * hd;
         const f32x4 a = *reinterpret_cast<const f32x4 *>(out + off + c);
         const f32x4 g = *reinterpret_cast<const f32x4 *>(dout + off + c);
         acc = a.x * g.x + a.y * g.y + a.z * g.z + a.w * g.w;
@@ -74,8 +74,8 @@ __device__ __forceinline__ void tile_accumulate_t(const float *At, const f32x16 
 }
 
 // Stores the transposed accumulators (register r of acc0/acc1 is d = 2*(8(r/4) + 4*half + r%4) + {0,1}) of the lane's
-// row to p[row][0..63], scaled.
-__device__ __forceinline__ void store_row_t(float *p, const f32x16 &acc0, const f32x16 &acc1, const float scale) {
+// row to p[row][0..63], scaled; p points at the lane's first column, of which ncols (a multiple of 4, may be <= 0) exist.
+__device__ __forceinline__ void store_row_t(float *p, const f32x16 &acc0, const f32x16 &acc1, const float scale, const int ncols) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         f32x4 a, c;
@@ -83,8 +83,8 @@ __device__ __forceinline__ void store_row_t(float *p, const f32x16 &acc0, const 
         a.z = acc0[4 * g + 1] * scale; a.w = acc1[4 * g + 1] * scale;
         c.x = acc0[4 * g + 2] * scale; c.y = acc1[4 * g + 2] * scale;
         c.z = acc0[4 * g + 3] * scale; c.w = acc1[4 * g + 3] * scale;
-        *reinterpret_cast<f32x4 *>(p + 16 * g) = a;
-        *reinterpret_cast<f32x4 *>(p + 16 * g + 4) = c;
+        if (16 * g < ncols) *reinterpret_cast<f32x4 *>(p + 16 * g) = a;
+        if (16 * g + 4 < ncols) *reinterpret_cast<f32x4 *>(p + 16 * g + 4) = c;
     }
 }
 
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
                                                                const float *__restrict__ stats, const float *__restrict__ D,
                                                                float *__restrict__ dq, int H, int Lq, int Lk, float rT,
                                                                MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
-                                                               int token_major) {
+                                                               int token_major, int hd) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                     // [2][BN][LSTR]
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
@@ -114,9 +114,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
     const int qic = qi < Lq ? qi : Lq - 1;
     int len = Lk;
     if (LENS) len = mask.lengths[b];
-    const int rs = token_major ? H * HD : HD;
-    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
-    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+    const int rs = token_major ? H * hd : hd;   // hd: the tensors' head dim, a multiple of 4 up to 64; tiles are zero beyond it
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
 
     // the same tiles as the forward pass visits (skipped tiles have weight exactly 0, hence gradient 0)
     int kend = Lk, wkend = Lk;
@@ -132,8 +132,11 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
         const float *gp = dout + q_base + (long long)qic * rs + half * 32;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
-            const f32x4 g = *reinterpret_cast<const f32x4 *>(gp + 4 * j);
+            f32x4 t = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
+            if (half * 32 + 4 * j < hd) {
+                t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+                g = *reinterpret_cast<const f32x4 *>(gp + 4 * j);
+            }
             qr[4 * j + 0] = (t.x * rT) * LOG2E; qr[4 * j + 1] = (t.y * rT) * LOG2E;
             qr[4 * j + 2] = (t.z * rT) * LOG2E; qr[4 * j + 3] = (t.w * rT) * LOG2E;
             gr[4 * j + 0] = g.x; gr[4 * j + 1] = g.y; gr[4 * j + 2] = g.z; gr[4 * j + 3] = g.w;
@@ -144,10 +147,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
     const float D_i = D[(long long)bh * Lq + qic];
 
     const int ld_row = tid >> 4, ld_col = (tid & 15) * 4;
-    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + HD) * 4);
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
-    const unsigned ld_off0 = (unsigned)(ld_row * rs + ld_col) * 4u;
+    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;   // beyond hd: outside the descriptor, zeros
     const unsigned ld_off1 = ld_off0 + 16u * rs * 4u;
     const unsigned tile_bytes = (unsigned)BN * rs * 4u;
     f32x4 kst[2], vst[2];
@@ -199,7 +202,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
-    if (qi < Lq) store_row_t(dq + q_base + (long long)qi * rs + 8 * half, a0, a1, rT);
+    if (qi < Lq) store_row_t(dq + q_base + (long long)qi * rs + 8 * half, a0, a1, rT, hd - 8 * half);
 }
 
 // ------------------------------------------------------------------------------------------------ dK, dV
@@ -209,7 +212,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
                                                                 const float *__restrict__ stats, const float *__restrict__ D,
                                                                 float *__restrict__ dk, float *__restrict__ dv, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict, int nkb,
-                                                                int total_blocks, int lpt, int token_major) {
+                                                                int total_blocks, int lpt, int token_major, int hd) {
     extern __shared__ __align__(16) float lds[];
     float *Qs = lds;                       // [2][BN][LSTR]  q * rT * log2(e)
     float *Gs = lds + 2 * TILE_FLOATS;     // [2][BN][LSTR]  dout
@@ -229,9 +232,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
     const int keyc = key < Lk ? key : Lk - 1;
     int len = Lk;
     if (LENS) len = mask.lengths[b];
-    const int rs = token_major ? H * HD : HD;
-    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
-    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+    const int rs = token_major ? H * hd : hd;   // hd: the tensors' head dim, a multiple of 4 up to 64; tiles are zero beyond it
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
 
     // Query tiles this workgroup / wavefront has to visit: under a causal mask only queries at or after its first key;
     // keys at or beyond the valid length have weight 0 everywhere.  Same exactness conditions as the forward pass.
@@ -252,8 +255,11 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
         const float *vp = v + kv_base + (long long)keyc * rs + half * 32;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const f32x4 a = *reinterpret_cast<const f32x4 *>(kp + 4 * j);
-            const f32x4 c = *reinterpret_cast<const f32x4 *>(vp + 4 * j);
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
+            if (half * 32 + 4 * j < hd) {
+                a = *reinterpret_cast<const f32x4 *>(kp + 4 * j);
+                c = *reinterpret_cast<const f32x4 *>(vp + 4 * j);
+            }
             kr[4 * j + 0] = a.x; kr[4 * j + 1] = a.y; kr[4 * j + 2] = a.z; kr[4 * j + 3] = a.w;
             vr[4 * j + 0] = c.x; vr[4 * j + 1] = c.y; vr[4 * j + 2] = c.z; vr[4 * j + 3] = c.w;
         }
@@ -262,10 +268,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
     // staging of one query tile: q (scaled when it is written to LDS), dout, and the tile's row statistics.  Rows at or
     // beyond Lq read as zeros; their reciprocal row sum is taken as 0, which makes their weights 0.
     const int ld_row = tid >> 4, ld_col = (tid & 15) * 4;
-    const int q_bytes = (int)(((long long)(Lq - 1) * rs + HD) * 4);
+    const int q_bytes = (int)(((long long)(Lq - 1) * rs + hd) * 4);
     const __amdgpu_buffer_rsrc_t qrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(q + q_base), 0, q_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t grsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(dout + q_base), 0, q_bytes, 0x00020000);
-    const unsigned ld_off0 = (unsigned)(ld_row * rs + ld_col) * 4u;
+    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;   // beyond hd: outside the descriptor, zeros
     const unsigned ld_off1 = ld_off0 + 16u * rs * 4u;
     const unsigned tile_bytes = (unsigned)BN * rs * 4u;
     f32x4 qst[2], gst[2];
@@ -368,8 +374,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
         __syncthreads();
     }
     if (key < Lk) {
-        store_row_t(dv + kv_base + (long long)key * rs + 8 * half, v0a, v1a, 1.0f);
-        store_row_t(dk + kv_base + (long long)key * rs + 8 * half, k0a, k1a, LN2);   // Q~ carries log2(e): dK = Q~^T dS ln 2
+        store_row_t(dv + kv_base + (long long)key * rs + 8 * half, v0a, v1a, 1.0f, hd - 8 * half);
+        store_row_t(dk + kv_base + (long long)key * rs + 8 * half, k0a, k1a, LN2, hd - 8 * half);   // Q~ carries log2(e): dK = Q~^T dS ln 2
     }
 }
 
@@ -488,7 +494,7 @@ __global__ __launch_bounds__(64) void sdpa_bwd_dkv_plain(const float *__restrict
 template <int KIND>
 int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
                const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
-               int strict, int token_major) {
+               int strict, int token_major, int hd) {
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     static bool attr_set[8] = {false};
     const size_t lds_dq = 4 * TILE_FLOATS * sizeof(float);
@@ -506,7 +512,7 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
         const int lpt = (causal_kind && !strict && nqb >= 2) ? 1 : 0;
         hipLaunchKernelGGL(sdpa_bwd_dq_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq, ctx->stream, q, k,
-                           v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major);
+                           v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, hd);
         const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d64");
         if (rc != DL4S_HIP_OK) return rc;
     }
@@ -516,7 +522,7 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
         const int lpt = (causal_kind && !strict && nkb >= 2) ? 1 : 0;
         hipLaunchKernelGGL(sdpa_bwd_dkv_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
-                           k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total, lpt, token_major);
+                           k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total, lpt, token_major, hd);
         return dl4s::launch_status("sdpa_bwd_dkv_f32_d64");
     }
 }
@@ -545,11 +551,18 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     DL4S_REQUIRE(q && out && stats && dout && dq, DL4S_HIP_EINVALID_ARG, "sdpa backward: NULL tensor pointer");
     DL4S_REQUIRE(B * H * (Lq > Lk ? Lq : Lk) * d < (1ll << 40) && Lq < (1ll << 30) && Lk < (1ll << 30), DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: extents too large");
-    DL4S_REQUIRE(d != HD || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
-                 "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB");
+    // head dims that are multiples of 4 up to 64 run on the MFMA kernels (tiles padded with zero columns) when every row
+    // starts on a 16-byte boundary
+    const bool mfma_path = d > 0 && d <= HD && d % 4 == 0 &&
+                           ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                             reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dout) | reinterpret_cast<uintptr_t>(dq) |
+                             reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
+    DL4S_REQUIRE(!mfma_path || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * d * 4 < (d == HD ? (1ll << 31) : (1ll << 30)),
+                 DL4S_HIP_EUNSUPPORTED,
+                 "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB (1 GiB for head dims below 64)");
     std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     MaskArgs m{};
-    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, d == HD, m);
+    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path, m);
     if (rc != DL4S_HIP_OK) return rc;
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     void *Dv = nullptr;
@@ -557,9 +570,9 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     if (rc != DL4S_HIP_OK) return rc;
     float *D = static_cast<float *>(Dv);
     const long long rows = B * H * Lq;
-    if (d != HD) {   // plain kernels
+    if (!mfma_path) {   // plain kernels
         rc = DL4S_HIP_OK;
-        if (token_major) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: the token-major layout needs head dims of 64");
+        if (token_major) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: the token-major layout needs a head dim that is a multiple of 4, at most 64, and 16-byte aligned tensors");
         else if (rows >= (1ll << 31) || B * H * Lk >= (1ll << 31)) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: too many rows for the plain kernels");
         if (rc == DL4S_HIP_OK) {
             hipLaunchKernelGGL(sdpa_bwd_rowdot_plain, dim3((unsigned)rows), dim3(64), 0, ctx->stream, out, dout, D, (int)d);
@@ -573,15 +586,15 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
         return rc != DL4S_HIP_OK ? rc : rcf;
     }
     hipLaunchKernelGGL(sdpa_bwd_rowdot, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, ctx->stream, out, dout, D, (int)H, (int)Lq,
-                       rows, token_major);
+                       rows, token_major, (int)d);
     rc = dl4s::launch_status("sdpa_bwd_rowdot");
     if (rc == DL4S_HIP_OK) {
         switch (m.kind) {
-            case DL4S_MASK_NONE: rc = launch_bwd<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
-            case DL4S_MASK_DENSE_F32: rc = launch_bwd<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
-            case DL4S_MASK_CAUSAL: rc = launch_bwd<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
-            case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
-            default: rc = launch_bwd<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major); break;
+            case DL4S_MASK_NONE: rc = launch_bwd<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+            case DL4S_MASK_DENSE_F32: rc = launch_bwd<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+            case DL4S_MASK_CAUSAL: rc = launch_bwd<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+            case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+            default: rc = launch_bwd<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
         }
     }
     const int rc2 = dl4s_hip_free(ctx, Dv);   // stream-ordered: later users of the block queue behind these kernels

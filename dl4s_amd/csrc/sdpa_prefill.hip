@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
                                                                 float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict,
                                                                 int nqb, int total_blocks, int lpt, int token_major,
-                                                                float *__restrict__ stats) {
+                                                                float *__restrict__ stats, int hd) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                     // [2][BN][LSTR]
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
@@ -115,9 +115,11 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
 
     // Tensor layout: [B,H,L,64] (row stride 64) or, token-major, [B,L,H,64] (row stride H*64): the projections of
     // MultiHeadAttention come out token-major, so reading them in place saves the four permuteAxes copies.
-    const int rs = token_major ? H * HD : HD;
-    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
-    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+    // hd = the tensors' head dim (a multiple of 4, at most 64): rows are hd floats long; columns hd..63 of every tile are
+    // zeros, which leaves scores and outputs unchanged
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
 
     // Keys this workgroup / wavefront has to visit.  Skipping is exact when every row keeps at least one
     // unblocked key (true unless len == 0) and K, V are finite at blocked keys.
@@ -142,7 +144,8 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
         const float *qp = q + q_base + (long long)qic * rs + half * 32;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            if (half * 32 + 4 * j < hd) t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
             qr[4 * j + 0] = (t.x * rT) * LOG2E;
             qr[4 * j + 1] = (t.y * rT) * LOG2E;
             qr[4 * j + 2] = (t.z * rT) * LOG2E;
@@ -156,10 +159,11 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     // bound below), so the loop needs neither address arithmetic beyond one add nor clamps.
     const int ld_row = tid >> 4;
     const int ld_col = (tid & 15) * 4;
-    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + HD) * 4);   // extent of this pair's rows; the host keeps it below 2^31
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);   // extent of this pair's rows; the host keeps it below 2^31
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
-    const unsigned ld_off0 = (unsigned)(ld_row * rs + ld_col) * 4u;   // unsigned: the last tile may step past 2^31
+    // columns at or beyond hd: an offset outside every descriptor (they stay below 2^31 bytes), i.e. zeros
+    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;   // unsigned: sums may pass 2^31
     const unsigned ld_off1 = ld_off0 + 16u * rs * 4u;
     const unsigned tile_bytes = (unsigned)BN * rs * 4u;
     f32x4 kst[2], vst[2];
@@ -240,8 +244,8 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
             a.z = o0[4 * g + 1] * inv; a.w = o1[4 * g + 1] * inv;
             c.x = o0[4 * g + 2] * inv; c.y = o1[4 * g + 2] * inv;
             c.z = o0[4 * g + 3] * inv; c.w = o1[4 * g + 3] * inv;
-            *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
-            *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
+            if (8 * half + 16 * g < hd) *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
+            if (8 * half + 16 * g + 4 < hd) *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
         }
     }
 }
@@ -258,7 +262,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
                                                                       const float *__restrict__ v, float *__restrict__ out,
                                                                       int H, int Lq, int Lk, float rT, MaskArgs mask,
                                                                       int strict, int nqb, int total_blocks, int token_major,
-                                                                      float *__restrict__ stats) {
+                                                                      float *__restrict__ stats, int hd) {
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: lets the per-wavefront tile conditions branch on scalars
@@ -285,9 +289,11 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
     const int qic = qi < Lq ? qi : Lq - 1;
     int len = Lk;
     if (LENS) len = mask.lengths[b];
-    const int rs = token_major ? H * HD : HD;
-    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * HD : (long long)bh * Lq * HD;
-    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * HD : (long long)bh * Lk * HD;
+    // hd = the tensors' head dim (a multiple of 4, at most 64): rows are hd floats long; columns hd..63 of every tile are
+    // zeros, which leaves scores and outputs unchanged
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
 
     int kend = Lk;
     if (!strict && !(LENS && len <= 0)) {
@@ -301,7 +307,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
         const float *qp = q + q_base + (long long)qic * rs + half * 32;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            f32x4 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            if (half * 32 + 4 * j < hd) t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
             qr[4 * j + 0] = (t.x * rT) * LOG2E;
             qr[4 * j + 1] = (t.y * rT) * LOG2E;
             qr[4 * j + 2] = (t.z * rT) * LOG2E;
@@ -312,10 +319,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
     // the wavefront stages its own tiles: lane covers rows (i*4 + lane/16), 4 floats at column (lane%16)*4
     const int ld_row = lane >> 4;
     const int ld_col = (lane & 15) * 4;
-    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + HD) * 4);
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
-    const unsigned ld_off = (unsigned)(ld_row * rs + ld_col) * 4u;
+    const unsigned ld_off = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
     const unsigned row4_bytes = 4u * rs * 4u;
     const unsigned tile_bytes = (unsigned)BN * rs * 4u;
     f32x4 kst[8], vst[8];
@@ -413,8 +420,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
                 a.z = o0[4 * g + 1] * inv; a.w = o1[4 * g + 1] * inv;
                 c.x = o0[4 * g + 2] * inv; c.y = o1[4 * g + 2] * inv;
                 c.z = o0[4 * g + 3] * inv; c.w = o1[4 * g + 3] * inv;
-                *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
-                *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
+                if (8 * half + 16 * g < hd) *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
+                if (8 * half + 16 * g + 4 < hd) *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
             }
         }
     }
@@ -475,7 +482,7 @@ __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__
 
 template <int KIND>
 int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq,
-               int Lk, float rT, const MaskArgs &m, int strict, int token_major, int no_split, float *stats) {
+               int Lk, float rT, const MaskArgs &m, int strict, int token_major, int no_split, float *stats, int hd) {
     // Too few 32-query wavefronts to give every SIMD about two: split the keys of each query block over 4 wavefronts.
     // The choice depends on the extents only, so every mask kind of one problem runs the same kernel.
     const long long waves = (long long)B * H * ((Lq + 31) / 32);
@@ -491,7 +498,7 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
             split_attr_set[KIND] = true;
         }
         hipLaunchKernelGGL(sdpa_prefill_split_f32_d64<KIND>, dim3((unsigned)((total32 + 7) / 8 * 8)), dim3(256), lds_split,
-                           ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major, stats);
+                           ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major, stats, hd);
         return dl4s::launch_status("sdpa_prefill_split_f32_d64");
     }
     const int nqb = (Lq + BM - 1) / BM;
@@ -512,7 +519,7 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         attr_set[KIND] = true;
     }
     hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
-                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats);
+                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_d64");
 }
 
@@ -531,9 +538,14 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
     DL4S_REQUIRE(dk > 0, DL4S_HIP_ESHAPE, "sdpa: keyDim is 0");
     DL4S_REQUIRE(B * H * (Lq > Lk ? Lq : Lk) * (dk > dv ? dk : dv) < (1ll << 40) && Lq < (1ll << 30) && Lk < (1ll << 30),
                  DL4S_HIP_EUNSUPPORTED, "sdpa: extents too large");
+    // head dims that are multiples of 4 up to 64 run on the MFMA kernels (tiles padded with zero columns), as long as
+    // every row starts on a 16-byte boundary
+    const bool mfma_path = dk == dv && dk <= HD && dk % 4 == 0 &&
+                           ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                             reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     MaskArgs m{};
     {
-        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, dk == HD && dv == HD, m);
+        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path, m);
         if (rc != DL4S_HIP_OK) return rc;
     }
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
@@ -541,19 +553,20 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
     const int no_split = (flags & DL4S_SDPA_NO_KEY_SPLIT) ? 1 : 0;
     DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR | DL4S_SDPA_NO_KEY_SPLIT)) == 0, DL4S_HIP_EINVALID_ARG,
                  "sdpa: unknown flag bits 0x%x", flags);
-    if (dk == HD && dv == HD) {
+    if (mfma_path) {
         // the MFMA kernel addresses one (batch, head) pair's K/V rows through a 32-bit byte offset
-        DL4S_REQUIRE(Lk * (token_major ? H : 1) * HD * 4 < (1ll << 31), DL4S_HIP_EUNSUPPORTED,
-                     "sdpa: the K/V rows of one (batch, head) pair span more than 2 GiB");
+        // (half of that for head dims below 64, whose padding columns use offsets from 2^31 up that must not wrap)
+        DL4S_REQUIRE(Lk * (token_major ? H : 1) * dk * 4 < (dk == HD ? (1ll << 31) : (1ll << 30)), DL4S_HIP_EUNSUPPORTED,
+                     "sdpa: the K/V rows of one (batch, head) pair span more than 2 GiB (1 GiB for head dims below 64)");
         switch (m.kind) {
-            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
-            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
-            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
-            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
-            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats);
+            case DL4S_MASK_NONE: return launch_d64<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
+            case DL4S_MASK_DENSE_F32: return launch_d64<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
+            case DL4S_MASK_CAUSAL: return launch_d64<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
+            case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
+            default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
         }
     }
-    DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs head dims of 64");
+    DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 64, and 16-byte aligned tensors");
     DL4S_REQUIRE(dk <= GEN_MAXD && dv <= GEN_MAXD && dv > 0, DL4S_HIP_EUNSUPPORTED,
                  "sdpa: head dims (%lld, %lld) above %d are not implemented", (long long)dk, (long long)dv, GEN_MAXD);
     const long long rows = B * H * Lq;

@@ -784,9 +784,10 @@ struct MultiHeadAttention {
           qDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})), kDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})),
           vDense(Tensor::repeating(0.f, {hiddenDim_, valueDim_ * heads_})), fc(Tensor::repeating(0.f, {valueDim_ * heads_, hiddenDim_})),
           norm(Shape{hiddenDim_}), dropout(dropoutRate) {}
-    // fused mode, head dims 64: the key / value projections alone, [B,L,H,64], for callers that attend to the same keys
-    // and values repeatedly (the encoder states during greedy decoding)
-    bool canCacheProjections() const { return Device::fused() && keyDim == 64 && valueDim == 64; }
+    // fused mode, equal head dims that are a multiple of 4 up to 64 (what the token-major attention kernels take): the
+    // key / value projections alone, [B,L,H,d], for callers that attend to the same keys and values repeatedly (the
+    // encoder states during greedy decoding)
+    bool canCacheProjections() const { return Device::fused() && keyDim == valueDim && keyDim <= 64 && keyDim % 4 == 0; }
     std::pair<Tensor, Tensor> projectKeysValues(const Tensor &k, const Tensor &v) const {
         precondition(canCacheProjections() && k.dim() == 3 && v.dim() == 3 && k.shape[1] == v.shape[1], "Matmul operands must have matching shapes");
         const int64_t B = k.shape[0], L = k.shape[1];
@@ -816,7 +817,7 @@ struct MultiHeadAttention {
         Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
         return norm.normalize(out_drop, &q);
     }
-    // self- or cross-attention with a structured mask (fused mode, head dims 64)
+    // self- or cross-attention with a structured mask (fused mode, head dims as for canCacheProjections)
     Tensor structured(const Tensor &q, const Tensor &k, const Tensor &v, const AttentionMask &mask) const {
         auto kv = projectKeysValues(k, v);
         return attendProjected(q, kv.first, kv.second, nullptr, &mask);
@@ -1015,7 +1016,7 @@ struct TransformerDecoder {
     }
     Tensor operator()(const Tensor &decoderInput, const Tensor &encoderStates, const std::vector<int64_t> &encoderInputLengths,
                       const std::vector<int64_t> &decoderInputLengths) const {
-        if (canCacheEncoderProjections())   // fused mode, head dims 64: structured masks, encoder projections per call
+        if (canCacheEncoderProjections())   // fused mode, head dims the MFMA kernels take: structured masks, encoder projections per call
             return withProjectedEncoder(decoderInput, projectEncoderStates(encoderStates), encoderInputLengths, decoderInputLengths);
         const Tensor encoderMask = makeEncoderMasks(encoderInputLengths);
         const Tensor decoderMask = makeDecoderMasks(decoderInputLengths);
@@ -1023,7 +1024,7 @@ struct TransformerDecoder {
         for (auto &layer : decoderLayers) acc = layer(acc, encoderStates, encoderMask, decoderMask);
         return acc;
     }
-    // Encoder-side key / value projections of every layer, computed once per encoded sequence (fused mode, head dims 64)
+    // Encoder-side key / value projections of every layer, computed once per encoded sequence (fused mode, head dims the MFMA kernels take)
     bool canCacheEncoderProjections() const {
         for (auto &l : decoderLayers)
             if (!l.encoderAttention.canCacheProjections() || !l.selfAttention.canCacheProjections()) return false;

@@ -100,10 +100,11 @@ typedef struct dl4s_mask_desc {
                                fully blocked tiles are skipped, which is exact as long as K and V hold finite
                                values at blocked positions (the reference computes 0 * v there, so a NaN/Inf in
                                V or K at a blocked key reaches the output only in strict mode). */
-#define DL4S_SDPA_TOKEN_MAJOR 2u /* q, out are [B,Lq,H,64] and k, v are [B,Lk,H,64] (the layout the projections of
+#define DL4S_SDPA_TOKEN_MAJOR 2u /* q, out are [B,Lq,H,d] and k, v are [B,Lk,H,d] (the layout the projections of
                                     MultiHeadAttention produce, NN/Models/Transformer/MultiHeadAttention.swift:105-107
                                     before its permutes :109-111, and the layout its output permute :117 produces), so a
-                                    caller can drop the four permuteAxes copies.  Head dims of 64 only. */
+                                    caller can drop the four permuteAxes copies.  Needs the MFMA kernel's conditions (see
+                                    dl4s_hip_sdpa_fwd_f32). */
 #define DL4S_SDPA_NO_KEY_SPLIT 4u /* small launches (fewer 32-query blocks than about two per SIMD) normally split each
                                      block's keys over the 4 wavefronts of a workgroup and merge the partial softmax
                                      results; this flag keeps the one-wavefront-per-block kernel.  The two agree within
@@ -114,13 +115,14 @@ typedef struct dl4s_mask_desc {
  * NN/Models/Transformer/ScaledDotProductAttention.swift:43-64.  q [B,H,Lq,dk], k [B,H,Lk,dk],
  * v [B,H,Lk,dv], out [B,H,Lq,dv], all row-major contiguous device fp32.  inv_temperature is the
  * fp32 reciprocal the reference forms once (Engine/CPU/CPUEngine.swift:635).  mask may be NULL
- * (= DL4S_MASK_NONE).  dk = dv = 64 runs the fused MFMA kernel; other sizes up to 256 run a
- * plain fused kernel. */
+ * (= DL4S_MASK_NONE).  dk = dv, a multiple of 4 and at most 64, with 16-byte aligned tensors runs
+ * the fused MFMA kernel (written for 64; smaller head dims are padded with zero columns on the
+ * fly and cost as much as 64); other sizes up to 256 run a plain fused kernel. */
 int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
                           int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
 
-/* Training form of the fused attention (key dim = value dim = d; MFMA kernels for d = 64, plain kernels up to 256).  The reference differentiates ScaledDotProductAttention through
+/* Training form of the fused attention (key dim = value dim = d; MFMA kernels under the forward call's conditions, plain kernels up to 256).  The reference differentiates ScaledDotProductAttention through
  * the backward closures of its primitive operators (Tensor/Operators/Matrix.swift:139-174 for the products through the
  * subscript views and the stack of broadcastMatrixMultiplied :79-117, Binary.swift:235-300 for e / sum,
  * Reduce.swift:35-62, Unary.swift:33-55 for exp, Binary.swift:161-224 for the subtractions); a backend that fuses the
@@ -130,7 +132,7 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
  *                                opaque to the caller)
  *   dl4s_hip_sdpa_bwd_f32        dq, dk, dv for the upstream gradient dout of out, from q, k, v, out, stats and the
  *                                same mask and flags as the forward call (the mask takes no gradient)
- * Layouts follow the forward call ([B,H,L,d], or [B,L,H,64] with DL4S_SDPA_TOKEN_MAJOR; stats is always [B,H,Lq,2]).
+ * Layouts follow the forward call ([B,H,L,d], or [B,L,H,d] with DL4S_SDPA_TOKEN_MAJOR; stats is always [B,H,Lq,2]).
  * Deterministic: no atomics, the same bits on every run. */
 int dl4s_hip_sdpa_fwd_stats_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, float *stats,
                                 int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t d, float inv_temperature,

@@ -71,8 +71,13 @@ def rand(rng, *shape, scale=1.0):
 
 # ------------------------------------------------------------------ small shapes, every mask kind
 SHAPES = [  # B, H, Lq, Lk, d
-    (1, 2, 5, 7, 4),        # the golden-fixture shape: plain kernel
-    (2, 3, 9, 11, 8),
+    (1, 2, 5, 7, 4),        # the golden-fixture shape: MFMA kernel with 60 padding columns
+    (2, 3, 9, 11, 8),       # key size of Tests/DL4STests/TransformerTests.swift:31
+    (2, 3, 9, 11, 6),       # not a multiple of 4: plain kernel
+    (1, 2, 40, 50, 96),     # above 64: plain kernel
+    (2, 3, 130, 70, 32),    # padded MFMA tiles, ragged
+    (2, 2, 200, 333, 40),
+    (1, 2, 100, 100, 60),
     (1, 2, 5, 7, 64),       # MFMA kernel, ragged single tile
     (2, 3, 130, 70, 64),    # ragged: Lq and Lk cross tile edges
     (1, 2, 128, 128, 64),
@@ -118,16 +123,24 @@ def test_sdpa_matches_oracle(ctx, orc, shape, mk):
         assert_parity(got, dense, "skip vs dense")
 
 
+def test_different_key_and_value_dims(ctx, orc):
+    rng = np.random.default_rng(77)
+    for dk, dv in [(8, 16), (64, 32), (5, 70)]:
+        q, k, v = rand(rng, 2, 2, 40, dk), rand(rng, 2, 2, 55, dk), rand(rng, 2, 2, 55, dv)
+        mask = (rng.random((40, 55)) < 0.3).astype(np.float32)
+        assert_parity(run_sdpa(ctx, q, k, v, mask), orc.sdpa(q, k, v, mask), "dk %d dv %d" % (dk, dv))
+
+
 def test_nil_mask_equals_zero_mask_bitwise(ctx):
     rng = np.random.default_rng(3)
-    for d in (8, 64):
+    for d in (8, 10, 64):
         q, k, v = rand(rng, 2, 2, 70, d), rand(rng, 2, 2, 90, d), rand(rng, 2, 2, 90, d)
         a = run_sdpa(ctx, q, k, v, None)
         b = run_sdpa(ctx, q, k, v, np.zeros((70, 90), np.float32))
         assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("d", [8, 64])
+@pytest.mark.parametrize("d", [8, 10, 64])
 def test_blocked_keys_have_exactly_zero_weight_and_blocked_rows_are_uniform(ctx, orc, d):
     rng = np.random.default_rng(5)
     B, H, Lq, Lk = 1, 2, 70, 100
@@ -148,7 +161,7 @@ def test_blocked_keys_have_exactly_zero_weight_and_blocked_rows_are_uniform(ctx,
     assert not np.isnan(base).any()
 
 
-@pytest.mark.parametrize("d", [8, 64])
+@pytest.mark.parametrize("d", [8, 10, 64])
 def test_nan_inf_placement_matches_oracle(ctx, orc, d):
     rng = np.random.default_rng(9)
     B, H, Lq, Lk = 1, 1, 40, 150
@@ -358,13 +371,14 @@ def test_config5_incremental_decode_append_then_attend(ctx, orc):
         buf.release()
 
 
+@pytest.mark.parametrize("d", [64, 8, 36])
 @pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 70), (1, 2, 5, 7), (2, 4, 256, 256), (1, 5, 33, 161)])
-def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk):
-    """[B,L,H,64] operands (what the projections of MultiHeadAttention produce before its permutes,
-    NN/Models/Transformer/MultiHeadAttention.swift:105-117) give the same bits as the permuted [B,H,L,64] ones."""
+def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk, d):
+    """[B,L,H,d] operands (what the projections of MultiHeadAttention produce before its permutes,
+    NN/Models/Transformer/MultiHeadAttention.swift:105-117) give the same bits as the permuted [B,H,L,d] ones."""
     from dl4s_amd import lib
-    rng = np.random.default_rng(B * 1000 + Lq)
-    q, k, v = rand(rng, B, H, Lq, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lk, 64)
+    rng = np.random.default_rng(B * 1000 + Lq + d)
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
     lens = rng.integers(1, Lk + 1, size=B)
     dense = (rng.random((B, 1, Lq, Lk)) < 0.3).astype(np.float32)
     cases = [dict(), dict(mask=dense), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)]
@@ -378,9 +392,12 @@ def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk):
 
 def test_token_major_rejected_for_other_head_dims_and_unknown_flags(ctx):
     from dl4s_amd import lib
-    q = ctx.empty((1, 2, 4, 8))
-    with pytest.raises(lib.Dl4sHipError):
-        ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, 8, 8, 0.5, None, lib.SDPA_TOKEN_MAJOR)
+    q = ctx.empty((1, 2, 4, 128))
+    for d in (6, 72, 128):      # neither a multiple of 4 up to 64
+        with pytest.raises(lib.Dl4sHipError):
+            ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, d, d, 0.5, None, lib.SDPA_TOKEN_MAJOR)
+    with pytest.raises(lib.Dl4sHipError):       # different key and value dims
+        ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, 8, 16, 0.5, None, lib.SDPA_TOKEN_MAJOR)
     with pytest.raises(lib.Dl4sHipError):
         ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, 8, 8, 0.5, None, 64)
     q.release()

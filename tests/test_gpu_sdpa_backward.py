@@ -21,7 +21,7 @@ def rand(rng, *shape, scale=1.0):
 
 
 def run_fwd_bwd(ctx, q, k, v, dout, mask=None, kind=None, lens=None, strict=False, token_major=False):
-    """Returns (out, stats, dq, dk, dv) in [B,H,L,64] order whatever layout the kernels were given."""
+    """Returns (out, stats, dq, dk, dv) in [B,H,L,d] order whatever layout the kernels were given."""
     from dl4s_amd import lib
     B, H, Lq, d = q.shape
     Lk = k.shape[2]
@@ -41,8 +41,9 @@ def run_fwd_bwd(ctx, q, k, v, dout, mask=None, kind=None, lens=None, strict=Fals
     elif kind == lib.MASK_CAUSAL:
         desc = ctx.mask_desc(lib.MASK_CAUSAL)
     flags = (lib.SDPA_STRICT if strict else 0) | (lib.SDPA_TOKEN_MAJOR if token_major else 0)
-    ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], out, stats, B, H, Lq, Lk, d, 0.125, desc, flags)
-    ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], out, stats, bufs[3], dq_, dk_, dv_, B, H, Lq, Lk, d, 0.125, desc, flags)
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))   # 0.125 for d = 64
+    ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], out, stats, B, H, Lq, Lk, d, rT, desc, flags)
+    ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], out, stats, bufs[3], dq_, dk_, dv_, B, H, Lq, Lk, d, rT, desc, flags)
     res = (back(out.numpy(), Lq), stats.numpy(), back(dq_.numpy(), Lq), back(dk_.numpy(), Lk), back(dv_.numpy(), Lk))
     for b in bufs + [dq_, dk_, dv_, out, stats] + extra:
         b.release()
@@ -142,10 +143,11 @@ def test_config4_sized_gradients(ctx, orc):
         assert_parity(dv[sl], rv, "config 4 dv")
 
 
-@pytest.mark.parametrize("d", [4, 8, 40, 130])
+@pytest.mark.parametrize("d", [4, 8, 40, 60, 6, 130])
 @pytest.mark.parametrize("mask_kind", ["none", "dense", "causal_lengths"])
 def test_gradients_for_other_head_dims(ctx, orc, d, mask_kind):
-    """The plain kernels (head dims other than 64), e.g. the key size 8 of Tests/DL4STests/TransformerTests.swift:31."""
+    """Head dims other than 64: multiples of 4 below it on the MFMA kernels with zero padding columns (e.g. the key size
+    8 of Tests/DL4STests/TransformerTests.swift:31), the others on the plain kernels."""
     from dl4s_amd import lib
     B, H, L = 2, 3, 70
     rng = np.random.default_rng(d)
@@ -181,8 +183,8 @@ def test_backward_argument_errors(ctx):
     a = ctx.empty((1, 1, 4, 300))
     with pytest.raises(lib.Dl4sHipError):       # head dim above 256
         ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 300, 0.5)
-    with pytest.raises(lib.Dl4sHipError):       # token-major needs head dims of 64
-        ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5, None, lib.SDPA_TOKEN_MAJOR)
+    with pytest.raises(lib.Dl4sHipError):       # token-major needs a head dim that is a multiple of 4, at most 64
+        ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 10, 0.5, None, lib.SDPA_TOKEN_MAJOR)
     with pytest.raises(lib.Dl4sHipError):       # unknown flag
         ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5, None, 128)
     a.release()
@@ -199,7 +201,8 @@ def test_random_shapes_forward_and_backward(ctx, orc, seed):
     if kind_name.startswith("causal"):
         Lk = Lq
     scale = float(rng.choice([0.3, 1.0, 3.0]))
-    q, k, v, dout = rand(rng, B, H, Lq, 64, scale=scale), rand(rng, B, H, Lk, 64, scale=scale), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lq, 64)
+    d = 64 if seed % 3 else int(rng.choice([4, 8, 20, 32, 48]))     # every third case on padded tiles
+    q, k, v, dout = rand(rng, B, H, Lq, d, scale=scale), rand(rng, B, H, Lk, d, scale=scale), rand(rng, B, H, Lk, d), rand(rng, B, H, Lq, d)
     lens = rng.integers(1, Lk + 1, size=B)
     kw, mask = {}, None
     if kind_name == "dense":
@@ -219,7 +222,7 @@ def test_random_shapes_forward_and_backward(ctx, orc, seed):
     kw["token_major"] = bool(rng.integers(0, 2))
     kw["strict"] = bool(rng.integers(0, 2))
     out, _, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, **kw)
-    what = "seed %d: B%d H%d Lq%d Lk%d %s %s" % (seed, B, H, Lq, Lk, kind_name, kw)
+    what = "seed %d: B%d H%d Lq%d Lk%d d%d %s %s" % (seed, B, H, Lq, Lk, d, kind_name, kw)
     assert_parity(out, orc.sdpa(q, k, v, mask), "out " + what)
     rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
     assert_parity(dq, rq, "dq " + what)
