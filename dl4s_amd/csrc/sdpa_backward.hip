@@ -120,9 +120,25 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
 
     // the same tiles as the forward pass visits (skipped tiles have weight exactly 0, hence gradient 0)
     int kend = Lk, wkend = Lk;
+    bool skip_ones = false;   // dense masks: this wavefront's all-ones tiles have weight exactly zero
     if (!strict && !(LENS && len <= 0)) {
         if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
         if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
+        if (DENSE && mask.cls) {   // trailing all-ones tiles of open blocks
+            const unsigned char *cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
+            int kmax = 0;
+#pragma unroll
+            for (int w = 0; w < BM / 32; ++w) {
+                const int blk = min(qb * BM + w * 32, Lq - 1) >> 5;
+                const int bound = dense_key_bound(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, Lk);
+                kmax = max(kmax, bound);
+                if (w == wave) {
+                    wkend = bound;
+                    skip_ones = dense_block_open(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, (Lk + 31) >> 5);
+                }
+            }
+            kend = kmax;
+        }
     }
     const int ntiles = (kend + BN - 1) / BN;
 
@@ -189,8 +205,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
         if (more) load_tile(t + 1);
         const int k0 = t * BN;
         int cls = 2;
-        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk];
-        if (k0 < wkend) {
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
             f32x16 p = masked_scores<KIND>(Ks + buf * TILE_FLOATS + row_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
 #pragma unroll
             for (int r = 0; r < 16; ++r) p[r] = fast_exp2(p[r] - m_i) * rl_i;                   // the forward pass's weights
@@ -241,11 +257,24 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
     const int nqt = (Lq + 31) / 32;
     int t_begin = 0, wt_begin = 0;
     bool wave_active = true;
+    const unsigned char *skip_cls0 = nullptr;   // dense masks with tile skipping: the (batch, head) slab's tile classes
     if (!strict && !(LENS && len <= 0)) {
         if (CAUSAL) { t_begin = (kb * BM) / 32; wt_begin = kw0 / 32; }
         if (LENS) {
             if (kb * BM >= len) t_begin = nqt;
             if (kw0 >= len) wave_active = false;
+        }
+        if (DENSE && mask.cls) {   // leading all-ones tiles of open query blocks
+            skip_cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
+            int tmin = nqt;
+#pragma unroll
+            for (int w = 0; w < BM / 32; ++w) {
+                const int kt = min(kb * BM + w * 32, Lk - 1) >> 5;
+                const int first = dense_query_begin(mask, skip_cls0, kt, nqt, (Lk + 31) >> 5);
+                tmin = min(tmin, first);
+                if (w == wave) wt_begin = first;
+            }
+            t_begin = tmin;
         }
     }
 
@@ -322,8 +351,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
         if (more) load_tile(t + 1);
         const int qt0 = t * 32;
         int cls = 2;
-        if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq];
-        if (wave_active && t >= wt_begin) {
+        if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq] & 3;
+        if (wave_active && t >= wt_begin &&
+            !(DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5))) {
             // S[query, key] in the base-2 domain: rows = the tile's queries 8(r/4) + 4*half + r%4, column = the lane's key
             f32x16 p = tile_product(Qs + buf * TILE_FLOATS + row_lds, kr);
             if (DENSE) {
@@ -510,7 +540,7 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         const int nqb = (Lq + BM - 1) / BM;
         const long long total = (long long)nqb * B * H;
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
-        const int lpt = (causal_kind && !strict && nqb >= 2) ? 1 : 0;
+        const int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
         hipLaunchKernelGGL(sdpa_bwd_dq_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq, ctx->stream, q, k,
                            v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, hd);
         const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d64");
@@ -520,7 +550,7 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         const int nkb = (Lk + BM - 1) / BM;
         const long long total = (long long)nkb * B * H;
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
-        const int lpt = (causal_kind && !strict && nkb >= 2) ? 1 : 0;
+        const int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nkb >= 2) ? 1 : 0;
         hipLaunchKernelGGL(sdpa_bwd_dkv_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
                            k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total, lpt, token_major, hd);
         return dl4s::launch_status("sdpa_bwd_dkv_f32_d64");

@@ -24,12 +24,16 @@ struct MaskArgs {
     const int *lengths;
     // dense masks, optional: one class per 32-query x 32-key tile (0 = all zeros, 1 = all ones, 2 = anything else),
     // laid out [slab][q tile][k tile] with slab / tile strides 0 on the mask's broadcast axes
+    // Bit 2 (value 4) of a class: every query row of the tile has a zero among the tile's 32 keys.  A 32-query block with
+    // such a tile is "open": each of its rows keeps an unblocked key, so its all-ones tiles have weight exactly zero (like
+    // the tiles a structured mask blocks) and may be skipped.
     const unsigned char *cls;
     int cls_sb, cls_sh, cls_sq, cls_sk;
 };
 
 // Classifies the 32 x 32 tiles of a dense mask so that the attention kernel only reads mask values where a tile is
-// neither all zeros nor all ones.  One wavefront per tile; elements outside [Lq, Lk] count as matching.
+// neither all zeros nor all ones.  One wavefront per tile; elements outside [Lq, Lk] count as matching.  Bit 2 of the
+// class says that every row of the tile (inside Lq) has a zero in this tile.
 __global__ __launch_bounds__(256) void sdpa_mask_classify(MaskArgs m, int MB, int MH, int nqt, int nkt, int Lq, int Lk,
                                                           long long total, unsigned char *cls) {
     const long long tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -41,18 +45,68 @@ __global__ __launch_bounds__(256) void sdpa_mask_classify(MaskArgs m, int MB, in
     const int bm = (int)(tile / nkt / nqt / MH);
     const int col = kt * 32 + (lane & 31);
     const int nrow = m.sq ? 32 : 1, ncol_ok = (m.sk ? col < Lk : (lane & 31) == 0);
-    bool all0 = true, all1 = true;
+    bool all0 = true, all1 = true, rows_open = true;
     const float *base = m.dense + bm * m.sb + hm * m.sh;
-    for (int r = lane >> 5; r < nrow; r += 2) {
+    for (int it = 0; 2 * it < nrow; ++it) {           // lanes 0..31 take row 2*it, lanes 32..63 row 2*it + 1
+        const int r = 2 * it + (lane >> 5);
         const int row = qt * 32 + r;
-        if (ncol_ok && (!m.sq || row < Lq)) {
+        bool zero = false;
+        if (r < nrow && ncol_ok && (!m.sq || row < Lq)) {
             const float x = base[row * m.sq + col * m.sk];
             all0 = all0 && (x == 0.0f);
             all1 = all1 && (x == 1.0f);
+            zero = (x == 0.0f);
         }
+        const unsigned long long zeros = __ballot(zero);
+        const bool row0 = !m.sq || qt * 32 + 2 * it < Lq, row1 = 2 * it + 1 < nrow && (!m.sq || qt * 32 + 2 * it + 1 < Lq);
+        if (row0 && (unsigned)zeros == 0u) rows_open = false;
+        if (row1 && (unsigned)(zeros >> 32) == 0u) rows_open = false;
     }
     const int z = __all(all0), o = __all(all1);
-    if (lane == 0) cls[tile] = z ? 0 : (o ? 1 : 2);
+    if (lane == 0) cls[tile] = (unsigned char)((z ? 0 : (o ? 1 : 2)) | (rows_open ? 4 : 0));
+}
+
+// Whether a 32-query block is known to be open (see MaskArgs): looked up in its first key tile and in the tile on the
+// diagonal, which covers causal, padding and band masks.  cls_row: the block's row of tile classes.
+__device__ __forceinline__ bool dense_block_open(const unsigned char *cls_row, const int cls_sk, const int qt, const int nkt) {
+    if (!cls_row || !cls_sk) return false;
+    return ((cls_row[0] | cls_row[min(qt, nkt - 1)]) & 4) != 0;
+}
+
+// Dense masks, tile skipping: how many leading keys a 32-query block has to visit.  Its key tiles from there on are all
+// ones while the block is open, so their weights are exactly zero.  cls_row: the block's row of tile classes, qt: its
+// index.  The same value in every lane.
+__device__ __forceinline__ int dense_key_bound(const unsigned char *cls_row, const int cls_sk, const int qt, const int Lk) {
+    const int nkt = (Lk + 31) >> 5;
+    if (!dense_block_open(cls_row, cls_sk, qt, nkt)) return Lk;
+    const int lane = threadIdx.x & 63;
+    for (int base = (nkt - 1) & ~63; base >= 0; base -= 64) {
+        const int t = base + lane;
+        const bool need = t < nkt && (cls_row[t] & 3) != 1;
+        const unsigned long long bal = __ballot(need);
+        if (bal) return __builtin_amdgcn_readfirstlane(min(Lk, (base + 64 - (int)__builtin_clzll(bal)) * 32));
+    }
+    return min(Lk, 32);   // not reached: an open block has a tile that is not all ones
+}
+
+// Dense masks, tile skipping, seen from a 32-key block (key tile kt): the first 32-query tile it has to visit; the
+// tiles before are all ones in open query blocks.  nqt when no tile needs a visit.  cls0: the (batch, head) slab's
+// classes.
+__device__ __forceinline__ int dense_query_begin(const MaskArgs &m, const unsigned char *cls0, const int kt, const int nqt, const int nkt) {
+    if (!cls0 || !m.cls_sk) return 0;
+    if (!m.cls_sq) return (dense_block_open(cls0, m.cls_sk, 0, nkt) && (cls0[kt] & 3) == 1) ? nqt : 0;   // one mask row for every query
+    const int lane = threadIdx.x & 63;
+    for (int base = 0; base < nqt; base += 64) {
+        const int t = base + lane;
+        bool need = false;
+        if (t < nqt) {
+            const unsigned char *row = cls0 + (long long)t * m.cls_sq;
+            need = !(dense_block_open(row, m.cls_sk, t, nkt) && (row[kt] & 3) == 1);
+        }
+        const unsigned long long bal = __ballot(need);
+        if (bal) return __builtin_amdgcn_readfirstlane(base + (int)__builtin_ctzll(bal));
+    }
+    return nqt;
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -65,6 +119,17 @@ __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); 
 // unit -- the callers number a pair's units longest first -- so that the hardware dispatcher does
 // longest-processing-time scheduling and the launch ends on the cheapest items.  Returns false for padding workgroups.
 __device__ __forceinline__ bool work_item(const int nunits, const int total_blocks, const int lpt, int &bh, int &unit) {
+    const int npairs = total_blocks / nunits;
+    if ((npairs & 7) == 0) {
+        // A pair count that divides by 8: XCD x takes the pairs x, x + 8, ... instead of a contiguous run.  Work that
+        // depends on the batch element (valid lengths, padding masks) then spreads evenly over the XCDs, whose runs
+        // would otherwise each hold a few whole batch elements.
+        const int x = blockIdx.x & 7, wl = blockIdx.x >> 3, cnt = npairs >> 3;
+        if (wl >= cnt * nunits) return false;
+        if (lpt) { unit = wl / cnt; bh = x + 8 * (wl % cnt); }
+        else { bh = x + 8 * (wl / nunits); unit = wl % nunits; }
+        return true;
+    }
     const int chunk = (total_blocks + 7) / 8;
     const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
     if (w >= total_blocks) return false;

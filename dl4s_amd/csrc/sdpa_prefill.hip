@@ -124,6 +124,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     // Keys this workgroup / wavefront has to visit.  Skipping is exact when every row keeps at least one
     // unblocked key (true unless len == 0) and K, V are finite at blocked keys.
     int kend = Lk, wkend = Lk;
+    bool skip_ones = false;   // dense masks: this wavefront's all-ones tiles have weight exactly zero
     if (!strict && !(LENS && len <= 0)) {
         if (CAUSAL) {
             kend = min(kend, qb * BM + BM);
@@ -132,6 +133,21 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
         if (LENS) {
             kend = min(kend, len);
             wkend = min(wkend, len);
+        }
+        if (DENSE && mask.cls) {   // trailing all-ones tiles of open blocks
+            const unsigned char *cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
+            int kmax = 0;
+#pragma unroll
+            for (int w = 0; w < BM / 32; ++w) {
+                const int blk = min(qb * BM + w * 32, Lq - 1) >> 5;
+                const int bound = dense_key_bound(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, Lk);
+                kmax = max(kmax, bound);
+                if (w == wave) {
+                    wkend = bound;
+                    skip_ones = dense_block_open(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, (Lk + 31) >> 5);
+                }
+            }
+            kend = kmax;
         }
     }
     const int ntiles = (kend + BN - 1) / BN;
@@ -211,9 +227,9 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
         if (more) load_tile(t + 1);
         const int k0 = t * BN;
         int cls = 2;
-        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk];
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
 
-        if (k0 < wkend) {
+        if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
             attend_tile<KIND>(Ks + buf * TILE_FLOATS + k_lds, Vs + buf * TILE_FLOATS + v_lds, qr, o0, o1, m_run, m_use, l_run, k0, q0,
                               qi, half, Lk, len, mrow, mask.sk, cls);
         }
@@ -296,7 +312,14 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
     const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
 
     int kend = Lk;
+    bool skip_ones = false;   // dense masks: the block's all-ones tiles have weight exactly zero
     if (!strict && !(LENS && len <= 0)) {
+        if (DENSE && mask.cls) {   // trailing all-ones tiles of an open block
+            const int blk = min(q0, Lq - 1) >> 5;
+            const unsigned char *row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)blk * mask.cls_sq;
+            skip_ones = dense_block_open(row, mask.cls_sk, blk, (Lk + 31) >> 5);
+            kend = dense_key_bound(row, mask.cls_sk, blk, Lk);
+        }
         if (CAUSAL) kend = min(kend, q0 + 32);
         if (LENS) kend = min(kend, len);
     }
@@ -364,8 +387,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
         const bool more = (t + SPLIT_WAVES < ntiles);
         if (more) load_tile(t + SPLIT_WAVES);
         int cls = 2;
-        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk];
-        attend_tile<KIND>(Ks + k_lds, Vs + v_lds, qr, o0, o1, m_run, m_use, l_run, t * BN, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        if (!(DENSE && skip_ones && cls == 1))
+            attend_tile<KIND>(Ks + k_lds, Vs + v_lds, qr, o0, o1, m_run, m_use, l_run, t * BN, q0, qi, half, Lk, len, mrow, mask.sk, cls);
         if (more) store_tile();
     }
 
@@ -507,7 +531,7 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
     // 16 (= the whole run) / 8 / 4 / 1 pairs: 120 / 111 / 107 / 87 TFLOP/s and 754 / 391 / 263 / 248 MiB of L2 fills
     // (the floor is 192 MiB): the kernel is MFMA-bound, the fills stay far below what the memory side delivers, so
     // balance wins over L2 reuse.
-    const int lpt = (causal_kind && !strict && nqb >= 2) ? 1 : 0;
+    const int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int chunk = (int)((total + 7) / 8);

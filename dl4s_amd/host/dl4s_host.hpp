@@ -86,6 +86,12 @@ struct HIP {
         static bool f = true;
         return f;
     }
+    // Fused attention only.  false: key tiles that the mask blocks entirely are skipped (their weights are exactly zero;
+    // the reference's 0 * v at such keys only differs when k or v hold NaN / Inf there).  true: every tile is visited.
+    static bool &strictMasks() {
+        static bool f = false;
+        return f;
+    }
     static void check(int rc) {
         if (rc != DL4S_HIP_OK) throw Trap(std::string("dl4s_hip: ") + dl4s_hip_last_error());
     }
@@ -207,7 +213,7 @@ struct HIP {
             check(dl4s_hip_sdpa_fwd_f32(context(), q.values.memory, k.values.memory, v.values.memory, result.values.memory,
                                         q.shape[0], q.shape[h], q.shape[l], k.shape[l], q.shape[3], v.shape[3],
                                         1.0f / temperature, mask ? &md : nullptr,
-                                        DL4S_SDPA_STRICT | (tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u)));
+                                        (strictMasks() ? DL4S_SDPA_STRICT : 0u) | (tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u)));
         }
         // the same with a structured mask descriptor (kind + device int32 lengths) instead of a dense mask tensor
         static void fusedAttentionStructured(const ShapedBuffer &q, const ShapedBuffer &k, const ShapedBuffer &v, int kind,
@@ -218,7 +224,8 @@ struct HIP {
             const int h = tokenMajor ? 2 : 1, l = tokenMajor ? 1 : 2;
             check(dl4s_hip_sdpa_fwd_f32(context(), q.values.memory, k.values.memory, v.values.memory, result.values.memory,
                                         q.shape[0], q.shape[h], q.shape[l], k.shape[l], q.shape[3], v.shape[3], 1.0f / temperature,
-                                        kind == DL4S_MASK_NONE ? nullptr : &md, tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u));
+                                        kind == DL4S_MASK_NONE ? nullptr : &md,
+                                        (strictMasks() ? DL4S_SDPA_STRICT : 0u) | (tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u)));
         }
         // result = act(x . weights + bias) + residual  (bias, residual optional)
         static void denseFused(const ShapedBuffer &x, const ShapedBuffer &weights, const ShapedBuffer *bias, int activation,

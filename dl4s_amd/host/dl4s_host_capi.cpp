@@ -21,6 +21,7 @@ int guarded(dl4s_hip_ctx *ctx, int fused, const std::function<void()> &body) {
     }
     HIP::context() = ctx;
     HIP::fused() = fused != 0;
+    HIP::strictMasks() = fused == 2;
     try {
         body();
         return 0;

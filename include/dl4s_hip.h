@@ -96,10 +96,12 @@ typedef struct dl4s_mask_desc {
 } dl4s_mask_desc;
 
 /* flags for dl4s_hip_sdpa_fwd_f32 */
-#define DL4S_SDPA_STRICT 1u /* visit every key tile even where a structured mask blocks all of it.  Without it
-                               fully blocked tiles are skipped, which is exact as long as K and V hold finite
-                               values at blocked positions (the reference computes 0 * v there, so a NaN/Inf in
-                               V or K at a blocked key reaches the output only in strict mode). */
+#define DL4S_SDPA_STRICT 1u /* visit every key tile even where the mask blocks all of it.  Without it fully blocked
+                               tiles are skipped - those a structured mask describes, and the all-ones 32 x 32 tiles
+                               of a dense mask in query blocks whose every row keeps an unblocked key (a zero) - which
+                               is exact as long as K and V hold finite values at blocked positions (the reference
+                               computes 0 * v there, so a NaN/Inf in V or K at a blocked key reaches the output only
+                               in strict mode).  Fully blocked rows are never skipped: they come out uniform. */
 #define DL4S_SDPA_TOKEN_MAJOR 2u /* q, out are [B,Lq,H,d] and k, v are [B,Lk,H,d] (the layout the projections of
                                     MultiHeadAttention produce, NN/Models/Transformer/MultiHeadAttention.swift:105-107
                                     before its permutes :109-111, and the layout its output permute :117 produces), so a

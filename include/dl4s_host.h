@@ -6,7 +6,9 @@
  * downloads the last result and returns 0, or -1 with the text in dl4s_host_last_error().
  *
  * `fused` selects the execution mode of the host layer: 0 issues exactly the engine primitive calls the
- * reference's tensor operators issue; 1 lets the layers use the backend's fused entry points.
+ * reference's tensor operators issue; 1 lets the layers use the backend's fused entry points; 2 is 1 with
+ * DL4S_SDPA_STRICT on every attention call (no tile skipping: NaN / Inf in keys or values at blocked
+ * positions then reach the output as in the reference).
  * A mask pointer may be NULL (no mask); mshape/mdim describe the mask tensor handed to the layer
  * (float, 1 = blocked), which must be broadcastable to [B,H,Lq,Lk].
  */

@@ -28,7 +28,7 @@ def host():
     return host_lib
 
 
-MODES = [pytest.param(False, id="primitive"), pytest.param(True, id="fused")]
+MODES = [pytest.param(False, id="primitive"), pytest.param(True, id="fused"), pytest.param(2, id="fused_strict")]
 
 
 def test_mask_builders_match_oracle_exactly(ctx, host, orc):
@@ -47,6 +47,26 @@ def test_sdpa_layer(ctx, host, orc, fused, shape):
         assert_parity(host.sdpa(ctx, q, k, v, mask, fused=fused), orc.sdpa(q, k, v, mask), "SDPA layer")
     pad = (np.arange(Lk)[None, None, None, :] >= np.array([3, Lk, 1][:B])[:, None, None, None]).astype(np.float32)
     assert_parity(host.sdpa(ctx, q, k, v, pad, fused=fused), orc.sdpa(q, k, v, pad), "SDPA layer padding mask")
+
+
+def test_nan_at_a_blocked_key_follows_the_mode(ctx, host, orc):
+    """The reference multiplies a NaN value at a blocked key by its zero weight (NaN).  The primitive and fused-strict modes
+    do the same; the fused mode skips key tiles its mask blocks entirely and documents that it differs there."""
+    B, H, L, d = 1, 2, 128, 64
+    rng = np.random.default_rng(33)
+    q, k, v = (rng.standard_normal((B, H, L, d)).astype(np.float32) for _ in range(3))
+    v[0, 1, 127, 3] = np.nan
+    mask = causal_mask(L, L)
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa(q, k, v, mask)
+    assert np.isnan(ref[0, 1, :, 3]).all() and not np.isnan(ref[0, 0]).any()
+    for mode in (False, 2):
+        assert_parity(host.sdpa(ctx, q, k, v, mask, fused=mode), ref, "mode %s" % mode)
+    got = host.sdpa(ctx, q, k, v, mask, fused=True)
+    assert not np.isnan(got[0, 1, :96]).any()             # key 127 lies in a tile these rows never visit
+    assert np.isnan(got[0, 1, 96:, 3]).all()              # rows of the last tile row read it (weight 0 times NaN)
+    keep = ~np.isnan(ref)
+    assert_parity(np.where(keep, got, 0), np.where(keep, ref, 0), "fused, finite part")
 
 
 @pytest.mark.parametrize("fused", MODES)

@@ -117,10 +117,14 @@ def test_sdpa_matches_oracle(ctx, orc, shape, mk):
     assert_parity(got, ref, "sdpa %s %s" % (shape, mk))
     if kind is not None:
         # structured descriptor == the dense mask it stands for, bit for bit (strict visits the same tiles)
-        dense = run_sdpa(ctx, q, k, v, mask)
+        dense = run_sdpa(ctx, q, k, v, mask, strict=True)
         strict = run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=True)
         assert np.array_equal(strict, dense)
         assert_parity(got, dense, "skip vs dense")
+    if mask is not None:
+        # a dense mask without the strict flag skips the all-ones tiles of query blocks whose rows all keep a key:
+        # zero weights either way, the same bits
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask), run_sdpa(ctx, q, k, v, mask, strict=True))
 
 
 def test_different_key_and_value_dims(ctx, orc):
@@ -195,10 +199,12 @@ def test_nan_in_v_at_blocked_key_reaches_output_only_in_strict_mode(ctx, orc):
     assert np.isnan(ref[0, 0, :, 5]).all()
     strict = run_sdpa(ctx, q, k, v, mask, kind=lib.MASK_CAUSAL, strict=True)
     assert_parity(strict, ref, "strict NaN")
-    dense = run_sdpa(ctx, q, k, v, mask)
+    dense = run_sdpa(ctx, q, k, v, mask, strict=True)
     assert_parity(dense, ref, "dense NaN")
     fast = run_sdpa(ctx, q, k, v, mask, kind=lib.MASK_CAUSAL)
     assert not np.isnan(fast[0, 0, :128]).any()     # documented: skipped tiles do not propagate it
+    fast_dense = run_sdpa(ctx, q, k, v, mask)       # the same for the all-ones tiles of a dense mask
+    assert not np.isnan(fast_dense[0, 0, :128]).any()
 
 
 def test_temperature_is_a_reciprocal_multiply_on_q(ctx, orc):

@@ -83,12 +83,18 @@ def test_gradients_match_the_oracle(ctx, orc, B, H, Lq, Lk, mask_kind):
     if mask_kind not in ("none", "dense"):
         # the structured descriptor gives the bits of the dense mask it stands for (strict visits the same tiles),
         # and the token-major layout the bits of the head-major one
-        dense = run_fwd_bwd(ctx, q, k, v, dout, mask=mask)
+        dense = run_fwd_bwd(ctx, q, k, v, dout, mask=mask, strict=True)
         strict = run_fwd_bwd(ctx, q, k, v, dout, strict=True, **kw)
         for a, b_ in zip(dense, strict):
             assert np.array_equal(a, b_)
         for a, b_ in zip(strict[2:], (dq, dk, dv)):
             assert_parity(b_, a, "tile skipping")
+    if mask is not None:
+        # dense masks without the strict flag skip all-ones tiles of query blocks whose rows all keep a key
+        skipping = run_fwd_bwd(ctx, q, k, v, dout, mask=mask)
+        visiting = run_fwd_bwd(ctx, q, k, v, dout, mask=mask, strict=True)
+        for a, b_ in zip(skipping, visiting):
+            assert np.array_equal(a, b_)
     tm = run_fwd_bwd(ctx, q, k, v, dout, token_major=True, **kw)
     for a, b_ in zip(tm, (out, stats, dq, dk, dv)):
         assert np.array_equal(a, b_)
@@ -228,3 +234,59 @@ def test_random_shapes_forward_and_backward(ctx, orc, seed):
     assert_parity(dq, rq, "dq " + what)
     assert_parity(dk, rk, "dk " + what)
     assert_parity(dv, rv, "dv " + what)
+
+
+@pytest.mark.parametrize("pattern", ["band", "left_padding", "block_sparse", "causal_rect", "blocked_rows", "per_head"])
+def test_dense_mask_tile_skipping_patterns(ctx, orc, pattern):
+    """Dense masks with whole 32 x 32 tiles of ones in different places.  Without the strict flag such tiles are skipped in
+    query blocks that are known to keep an unblocked key in every row (looked up in the block's first and diagonal tile);
+    forward results and gradients must not move by a bit, and must match the oracle."""
+    rng = np.random.default_rng(len(pattern))
+    B, H, Lq, Lk = 2, 2, 200, 200
+    i, j = np.indices((Lq, Lk))
+    if pattern == "band":                  # sliding window of 40 keys: ones on both sides of the diagonal band
+        mask = ((j > i) | (j < i - 40)).astype(np.float32)
+    elif pattern == "left_padding":        # the first keys blocked: no row has an open key in the first tile
+        mask = np.broadcast_to((np.arange(Lk) < np.array([70, 33])[:, None, None, None]), (B, 1, 1, Lk)).astype(np.float32)
+    elif pattern == "block_sparse":        # interior all-ones tiles between open ones
+        tiles = rng.random((7, 7)) < 0.5
+        tiles[:, 0] = False
+        mask = np.kron(tiles, np.ones((32, 32)))[:Lq, :Lk].astype(np.float32)
+    elif pattern == "causal_rect":         # more keys than queries
+        Lk = 300
+        i, j = np.indices((Lq, Lk))
+        mask = (j > i + 50).astype(np.float32)
+    elif pattern == "blocked_rows":        # causal, with some rows blocked entirely: their blocks must not skip
+        mask = (j > i).astype(np.float32)
+        mask[[0, 77, 199], :] = 1.0
+    else:                                  # a different structure per head
+        mask = np.stack([(j > i), (j < i - 64) | (j > i + 3)]).astype(np.float32)[None]
+    q, k, v, dout = rand(rng, B, H, Lq, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lq, 64)
+    skipping = run_fwd_bwd(ctx, q, k, v, dout, mask=mask)
+    visiting = run_fwd_bwd(ctx, q, k, v, dout, mask=mask, strict=True)
+    for a, b_ in zip(skipping, visiting):
+        assert np.array_equal(a, b_)
+    tm = run_fwd_bwd(ctx, q, k, v, dout, mask=mask, token_major=True)
+    for a, b_ in zip(skipping, tm):
+        assert np.array_equal(a, b_)
+    assert_parity(skipping[0], orc.sdpa(q, k, v, mask), "out " + pattern)
+    rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+    assert_parity(skipping[2], rq, "dq " + pattern)
+    assert_parity(skipping[3], rk, "dk " + pattern)
+    assert_parity(skipping[4], rv, "dv " + pattern)
+
+
+def test_dense_mask_tile_skipping_is_active(ctx):
+    """A NaN value at a key that lies in all-ones tiles only: with tile skipping neither the output nor any gradient sees
+    it; the strict flag brings back the reference's 0 * NaN."""
+    rng = np.random.default_rng(8)
+    B, H, L = 1, 2, 256
+    q, k, v, dout = (rand(rng, B, H, L, 64) for _ in range(4))
+    lens = np.array([130])
+    mask = lengths_mask(lens, L)           # keys 130.. blocked: tiles 5..7 are all ones
+    v[0, 0, 200, 7] = np.nan
+    out, _, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, mask=mask)
+    assert not np.isnan(out).any() and not np.isnan(dq).any() and not np.isnan(dk).any() and not np.isnan(dv).any()
+    out_s, _, dq_s, _, _ = run_fwd_bwd(ctx, q, k, v, dout, mask=mask, strict=True)
+    assert np.isnan(out_s[0, 0, :, 7]).all() and not np.isnan(out_s[0, 1]).any()
+    assert np.isnan(dq_s[0, 0]).all()
