@@ -26,6 +26,10 @@ struct GemmArgs {
     long long a_rs, a_cs;  // element strides of op(A)[m][k]
     long long b_rs, b_cs;  // element strides of op(B)[k][n]
     long long a_bs, b_bs, c_bs;  // batch strides
+    // grouped launches (groups > 0): blockIdx.z selects one of up to 4 products of the same shape whose operands lie at
+    // these element offsets from A, B, C
+    int groups;
+    long long a_off[4], b_off[4], c_off[4];
     long long lda, ldb;          // row strides of A and B as stored (the fast kernels)
     float alpha, beta;
     int tiles_n;
@@ -57,9 +61,9 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_mfma(GemmArgs g) {
     const int wm = wave >> 1, wn = wave & 1;
     const int tile_m = blockIdx.x / g.tiles_n, tile_n = blockIdx.x % g.tiles_n;
     const int m0 = tile_m * GBM, n0 = tile_n * GBN;
-    const float *A = g.A + (long long)blockIdx.z * g.a_bs;
-    const float *B = g.B + (long long)blockIdx.z * g.b_bs;
-    float *C = g.C + (long long)blockIdx.z * g.c_bs;
+    const float *A = g.A + (g.groups ? g.a_off[blockIdx.z] : (long long)blockIdx.z * g.a_bs);
+    const float *B = g.B + (g.groups ? g.b_off[blockIdx.z] : (long long)blockIdx.z * g.b_bs);
+    float *C = g.C + (g.groups ? g.c_off[blockIdx.z] : (long long)blockIdx.z * g.c_bs);
 
     // loader mappings: unit stride along k -> 16 lanes walk k; otherwise 128 threads walk m (or n)
     const bool a_kfast = (g.a_cs == 1);
@@ -234,12 +238,13 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
     const int wm = wave >> 1, wn = wave & 1;
     const int tile_m = blockIdx.x / g.tiles_n, tile_n = blockIdx.x % g.tiles_n;
     const int m0 = tile_m * TM, n0 = tile_n * TN;
-    float *C = g.C + (long long)blockIdx.z * g.c_bs;
+    const long long c_at = g.groups ? g.c_off[blockIdx.z] : (long long)blockIdx.z * g.c_bs;
+    float *C = g.C + c_at;
 
     OpA opa;
     OpB opb;
-    opa.init(As, g.A + (long long)blockIdx.z * g.a_bs, g.M, g.lda, m0, g.K, tid);
-    opb.init(Bs, g.B + (long long)blockIdx.z * g.b_bs, g.N, g.ldb, n0, g.K, tid);
+    opa.init(As, g.A + (g.groups ? g.a_off[blockIdx.z] : (long long)blockIdx.z * g.a_bs), g.M, g.lda, m0, g.K, tid);
+    opb.init(Bs, g.B + (g.groups ? g.b_off[blockIdx.z] : (long long)blockIdx.z * g.b_bs), g.N, g.ldb, n0, g.K, tid);
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -324,7 +329,7 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
                         val.z = gelu_sigmoid(val.z); val.w = gelu_sigmoid(val.w);
                     }
                     if (g.residual) {
-                        const f32x4 rq = *reinterpret_cast<const f32x4 *>(g.residual + (long long)blockIdx.z * g.c_bs + (long long)gm * g.N + gn);
+                        const f32x4 rq = *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
                         val.x = __fadd_rn(val.x, rq.x); val.y = __fadd_rn(val.y, rq.y);
                         val.z = __fadd_rn(val.z, rq.z); val.w = __fadd_rn(val.w, rq.w);
                     }
@@ -336,7 +341,9 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
 
 int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int64_t lbs, const float *rhs, int64_t rr,
                 int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb,
-                const float *bias = nullptr, const float *residual = nullptr, int act = 0) {
+                const float *bias = nullptr, const float *residual = nullptr, int act = 0, const float *const *group_lhs = nullptr,
+                const float *const *group_rhs = nullptr, float *const *group_result = nullptr) {
+    // group_*: `batch` (at most 4) products of one shape with unrelated operand addresses, in one launch
     DL4S_REQUIRE(lr >= 0 && lc >= 0 && rr >= 0 && rc >= 0 && batch >= 0, DL4S_HIP_EINVALID_ARG, "gemm: negative extent");
     const int64_t M = ta ? lc : lr, K = ta ? lr : lc;
     const int64_t K2 = tb ? rc : rr, N = tb ? rr : rc;
@@ -351,6 +358,16 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.a_rs = ta ? 1 : lc; g.a_cs = ta ? lc : 1;
     g.b_rs = tb ? 1 : rc; g.b_cs = tb ? rc : 1;
     g.a_bs = lbs; g.b_bs = rbs; g.c_bs = cbs;
+    bool group_aligned = true;
+    if (group_lhs) {
+        g.groups = (int)batch;
+        for (int i = 0; i < g.groups; ++i) {
+            g.a_off[i] = group_lhs[i] - lhs;
+            g.b_off[i] = group_rhs[i] - rhs;
+            g.c_off[i] = group_result[i] - result;
+            group_aligned = group_aligned && ((g.a_off[i] | g.b_off[i] | g.c_off[i]) & 3) == 0;
+        }
+    }
     g.lda = lc; g.ldb = rc;
     g.alpha = alpha; g.beta = beta;
     g.bias = bias; g.residual = residual; g.act = act;
@@ -362,7 +379,7 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     const auto k_by_rows_ok = [&](int64_t extent, int64_t ld) { return extent % 4 == 0 && K * ld * 4 < (1ll << 31); };
     const bool fast = K > 0 && N % 4 == 0 && (ta ? k_by_rows_ok(M, lc) : rows_by_k_ok(lc)) && (tb ? rows_by_k_ok(rc) : k_by_rows_ok(N, rc)) &&
                       aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 && rbs % 4 == 0 && aligned16(result) && cbs % 4 == 0 &&
-                      aligned16(bias) && aligned16(residual) && !(epi && (ta || tb));
+                      aligned16(bias) && aligned16(residual) && !(epi && (ta || tb)) && group_aligned;
     long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
     // small products: 64x64 tiles, so that there are at least about two workgroups per CU
     const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;
@@ -411,6 +428,19 @@ int dl4s_hip_gemm_batched_f32(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_r
     DL4S_REQUIRE(lhs_stride >= 0 && rhs_stride >= 0 && result_stride >= 0, DL4S_HIP_EINVALID_ARG, "gemm: negative batch stride");
     return gemm_launch(ctx, lhs, lhs_rows, lhs_cols, lhs_stride, rhs, rhs_rows, rhs_cols, rhs_stride, result, result_stride,
                        batch, alpha, beta, transpose_first, transpose_second);
+}
+
+int dl4s_hip_gemm_grouped_f32(dl4s_hip_ctx *ctx, int count, const float *const *lhs, int64_t lhs_rows, int64_t lhs_cols,
+                              const float *const *rhs, int64_t rhs_rows, int64_t rhs_cols, float *const *result, float alpha,
+                              float beta, int transpose_first, int transpose_second) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(count >= 0 && count <= 4, DL4S_HIP_EINVALID_ARG, "gemm: a group holds at most 4 products, got %d", count);
+    if (count == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(lhs && rhs && result, DL4S_HIP_EINVALID_ARG, "gemm: NULL pointer array");
+    for (int i = 0; i < count; ++i)
+        DL4S_REQUIRE(result[i] && lhs[i] && rhs[i], DL4S_HIP_EINVALID_ARG, "gemm: NULL pointer in group entry %d", i);
+    return gemm_launch(ctx, lhs[0], lhs_rows, lhs_cols, 0, rhs[0], rhs_rows, rhs_cols, 0, result[0], 0, count, alpha, beta,
+                       transpose_first, transpose_second, nullptr, nullptr, 0, lhs, rhs, result);
 }
 
 int dl4s_hip_dense_fused_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t in_features, const float *weights,

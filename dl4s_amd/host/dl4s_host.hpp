@@ -242,6 +242,21 @@ struct HIP {
                                             rhs.values.memory, rhs.shape[rd - 2], rhs.shape[rd - 1], rstride, result.values.memory,
                                             result.shape[od - 2] * result.shape[od - 1], batch, 1.0f, 0.0f, tA, tB));
         }
+        // up to 4 products [rows, in] . [in, out] of one shape in one launch (operands anywhere)
+        static void gemmGrouped(const std::vector<ShapedBuffer> &lhs, int64_t rows, const std::vector<ShapedBuffer> &rhs,
+                                const std::vector<ShapedBuffer> &results) {
+            const float *a[4], *b[4];
+            float *c[4];
+            precondition(lhs.size() == rhs.size() && lhs.size() == results.size() && lhs.size() <= 4, "bad group");
+            for (size_t i = 0; i < lhs.size(); ++i) {
+                precondition(lhs[i].count() == rows * rhs[i].shape[0] && rhs[i].shape == rhs[0].shape, "Matmul operands must have matching shapes");
+                a[i] = lhs[i].values.memory;
+                b[i] = rhs[i].values.memory;
+                c[i] = results[i].values.memory;
+            }
+            check(dl4s_hip_gemm_grouped_f32(context(), (int)lhs.size(), a, rows, rhs[0].shape[0], b, rhs[0].shape[0], rhs[0].shape[1], c,
+                                            1.0f, 0.0f, 0, 0));
+        }
         static void layerNorm(const ShapedBuffer &x, const ShapedBuffer *residual, const ShapedBuffer &scale,
                               const ShapedBuffer &shift, const ShapedBuffer &result) {
             const int64_t B = x.shape[0], D = scale.count();
@@ -795,17 +810,29 @@ struct MultiHeadAttention {
     // key / value projections alone, [B,L,H,d], for callers that attend to the same keys and values repeatedly (the
     // encoder states during greedy decoding)
     bool canCacheProjections() const { return Device::fused() && keyDim == valueDim && keyDim <= 64 && keyDim % 4 == 0; }
-    std::pair<Tensor, Tensor> projectKeysValues(const Tensor &k, const Tensor &v) const {
+    // The projections are separate products in the reference (MultiHeadAttention.swift:105-107); the key and value ones
+    // (and the query one, when all three inputs have one length) go out as one grouped launch.
+    std::pair<Tensor, Tensor> projectKeysValues(const Tensor &k, const Tensor &v, const Tensor *q = nullptr, Tensor *qp = nullptr) const {
         precondition(canCacheProjections() && k.dim() == 3 && v.dim() == 3 && k.shape[1] == v.shape[1], "Matmul operands must have matching shapes");
         const int64_t B = k.shape[0], L = k.shape[1];
-        return {k.view({B * L, hiddenDim}).matrixMultiplied(kDense).view({B, L, heads, keyDim}),
-                v.view({B * L, hiddenDim}).matrixMultiplied(vDense).view({B, L, heads, valueDim})};
+        precondition(k.shape[2] == hiddenDim && v.shape[2] == hiddenDim && k.shape[0] == v.shape[0], "Matmul operands must have matching shapes");
+        Tensor kp(Device::Memory::allocateBuffer(Shape{B, L, heads, keyDim})), vp(Device::Memory::allocateBuffer(Shape{B, L, heads, valueDim}));
+        std::vector<ShapedBuffer> lhs{k.values(), v.values()}, rhs{kDense.values(), vDense.values()}, res{kp.values(), vp.values()};
+        if (q && qp && q->shape == k.shape) {
+            *qp = Tensor(Device::Memory::allocateBuffer(Shape{B, L, heads, keyDim}));
+            lhs.push_back(q->values());
+            rhs.push_back(qDense.values());
+            res.push_back(qp->values());
+        }
+        Device::Engine::gemmGrouped(lhs, B * L, rhs, res);
+        return {kp, vp};
     }
     Tensor attendProjected(const Tensor &q, const Tensor &kp, const Tensor &vp, const Tensor *mask,
-                           const AttentionMask *structured = nullptr) const {
+                           const AttentionMask *structured = nullptr, const Tensor *qProjected = nullptr) const {
         precondition(canCacheProjections() && q.dim() == 3 && kp.dim() == 4 && vp.dim() == 4, "Matmul operands must have matching shapes");
         const int64_t batchSize = q.shape[0], queryCount = q.shape[1];
-        Tensor qp = q.view({batchSize * queryCount, hiddenDim}).matrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
+        Tensor qp = qProjected ? *qProjected
+                               : q.view({batchSize * queryCount, hiddenDim}).matrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
         Tensor a(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, heads, valueDim}));
         ShapedBuffer mb;
         if (mask) mb = mask->values();
@@ -826,16 +853,18 @@ struct MultiHeadAttention {
     }
     // self- or cross-attention with a structured mask (fused mode, head dims as for canCacheProjections)
     Tensor structured(const Tensor &q, const Tensor &k, const Tensor &v, const AttentionMask &mask) const {
-        auto kv = projectKeysValues(k, v);
-        return attendProjected(q, kv.first, kv.second, nullptr, &mask);
+        Tensor qp;
+        auto kv = projectKeysValues(k, v, &q, &qp);
+        return attendProjected(q, kv.first, kv.second, nullptr, &mask, qp.dim() ? &qp : nullptr);
     }
     Tensor operator()(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask) const {
         const int64_t batchSize = q.shape[0], queryCount = q.shape[1], keyCount = k.shape[1], valueCount = v.shape[1];
         const Tensor &res = q;
         if (canCacheProjections()) {
             precondition(q.dim() == 3 && k.dim() == 3 && v.dim() == 3 && keyCount == valueCount, "Matmul operands must have matching shapes");
-            auto kv = projectKeysValues(k, v);
-            return attendProjected(q, kv.first, kv.second, mask);
+            Tensor qp;
+            auto kv = projectKeysValues(k, v, &q, &qp);
+            return attendProjected(q, kv.first, kv.second, mask, nullptr, qp.dim() ? &qp : nullptr);
         }
         Tensor q_prep = q.broadcastMatrixMultiplied(qDense).view({batchSize, queryCount, heads, keyDim});
         Tensor k_prep = k.broadcastMatrixMultiplied(kDense).view({batchSize, keyCount, heads, keyDim});

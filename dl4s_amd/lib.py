@@ -227,6 +227,14 @@ class Context:
                                                   _vp(_ptr(result)), _i64(cstride), _i64(batch), C.c_float(alpha),
                                                   C.c_float(beta), int(ta), int(tb)))
 
+    def gemm_grouped(self, lhs, lshape, rhs, rshape, results, alpha=1.0, beta=0.0, ta=False, tb=False):
+        """len(lhs) (at most 4) products of one shape, operands anywhere, in one launch."""
+        n = len(lhs)
+        arr = lambda xs: (C.c_void_p * max(1, n))(*[_ptr(x) for x in xs])
+        _check(self.lib.dl4s_hip_gemm_grouped_f32(self.handle, n, arr(lhs), _i64(lshape[0]), _i64(lshape[1]), arr(rhs),
+                                                  _i64(rshape[0]), _i64(rshape[1]), arr(results), C.c_float(alpha),
+                                                  C.c_float(beta), int(ta), int(tb)))
+
     def band(self, x, y, rows, cols, below, above):
         _check(self.lib.dl4s_hip_band_f32(self.handle, _vp(_ptr(x)), _vp(_ptr(y)), _i64(rows), _i64(cols),
                                           int(below is not None), _i64(below or 0), int(above is not None), _i64(above or 0)))

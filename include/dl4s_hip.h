@@ -181,6 +181,13 @@ int dl4s_hip_gemm_batched_f32(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_r
                               int64_t lhs_stride, const float *rhs, int64_t rhs_rows, int64_t rhs_cols,
                               int64_t rhs_stride, float *result, int64_t result_stride, int64_t batch,
                               float alpha, float beta, int transpose_first, int transpose_second);
+/* Grouped form: `count` (at most 4) products of one shape whose operands lie anywhere (host arrays of
+ * device pointers; entries may repeat), in one launch - the three projections of
+ * NN/Models/Transformer/MultiHeadAttention.swift:105-107, which the reference issues as three
+ * broadcastMatrixMultiplied calls.  Every product gets the bits the single call gives. */
+int dl4s_hip_gemm_grouped_f32(dl4s_hip_ctx *ctx, int count, const float *const *lhs, int64_t lhs_rows, int64_t lhs_cols,
+                              const float *const *rhs, int64_t rhs_rows, int64_t rhs_cols, float *const *result,
+                              float alpha, float beta, int transpose_first, int transpose_second);
 /* :233 band: copies columns max(0,i-below) .. min(cols,i+above+1)-1 of each row i; other elements of
  * result are left untouched (the caller zero-fills first, Tensor/Operators/UtilOps.swift:117-121).
  * has_below / has_above == 0 stand for nil. */

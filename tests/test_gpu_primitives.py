@@ -140,6 +140,39 @@ def test_gemm_batched_equals_loop_and_stack(ctx, orc):
         x.release()
 
 
+@pytest.mark.parametrize("M,N,K,ta,tb", [(256, 128, 64, False, False), (2048, 512, 512, False, False), (70, 40, 30, False, False),
+                                          (128, 64, 96, True, False), (96, 200, 64, False, True), (5, 7, 3, True, True)])
+@pytest.mark.parametrize("count", [1, 2, 3, 4])
+def test_gemm_grouped_gives_the_bits_of_single_calls(ctx, orc, M, N, K, ta, tb, count):
+    """The three projections of NN/Models/Transformer/MultiHeadAttention.swift:105-107 as one launch: same bits as one call
+    each, whatever tile size either launch picks; operands may repeat within a group."""
+    As = [rnd(K, M) if ta else rnd(M, K) for _ in range(count)]
+    Bs = [rnd(N, K) if tb else rnd(K, N) for _ in range(count)]
+    dA, dB = [ctx.to_device(a) for a in As], [ctx.to_device(b) for b in Bs]
+    if count >= 3:
+        dA[2], As[2] = dA[0], As[0]          # a shared left operand, like q = k = v
+    single, grouped = [ctx.empty((M, N)) for _ in range(count)], [ctx.empty((M, N)) for _ in range(count)]
+    for i in range(count):
+        ctx.gemm(dA[i], As[i].shape, dB[i], Bs[i].shape, single[i], 1.0, 0.0, ta, tb)
+    ctx.gemm_grouped(dA, As[0].shape, dB, Bs[0].shape, grouped, 1.0, 0.0, ta, tb)
+    for i in range(count):
+        assert np.array_equal(single[i].numpy(), grouped[i].numpy())
+        assert_parity(grouped[i].numpy(), orc.gemm(As[i], Bs[i], ta, tb), "grouped gemm %d" % i)
+    for x in set(dA) | set(dB) | set(single) | set(grouped):
+        x.release()
+
+
+def test_gemm_grouped_argument_errors(ctx):
+    from dl4s_amd import lib
+    a = ctx.empty((4, 4))
+    with pytest.raises(lib.Dl4sHipError):
+        ctx.gemm_grouped([a] * 5, (4, 4), [a] * 5, (4, 4), [a] * 5)
+    with pytest.raises(lib.Dl4sHipError):
+        ctx.gemm_grouped([a, 0], (4, 4), [a, a], (4, 4), [a, a])
+    ctx.gemm_grouped([], (4, 4), [], (4, 4), [])
+    a.release()
+
+
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
 @pytest.mark.parametrize("sa,sb", [((2, 3, 4), (4,)), ((2, 3, 4), (3, 1)), ((2, 3, 4), ()), ((), (2, 3)), ((2, 1, 4), (1, 3, 1)),
                                    ((2, 3, 4, 5), (2, 1, 1, 5)), ((3, 4), (3, 4)), ((2, 2, 33, 33), (33, 33)), ((40, 1), (1, 50)),
