@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
     float *Ks = lds;                     // [2][BN][LSTR]
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
     int bh, unit;
-    if (!work_item(nqb, total_blocks, lpt, bh, unit)) return;
+    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
 
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
     float *Gs = lds + 2 * TILE_FLOATS;     // [2][BN][LSTR]  dout
     float *Ss = lds + 4 * TILE_FLOATS;     // per query tile: [2][32] reference maxima, [2][32] 1 / row sums, [2][32] D
     int bh, unit;
-    if (!work_item(nkb, total_blocks, lpt, bh, unit)) return;
+    if (!work_item(nkb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
 
@@ -540,7 +540,10 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         const int nqb = (Lq + BM - 1) / BM;
         const long long total = (long long)nqb * B * H;
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
-        const int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
+        // longest first; in a launch that fits the chip at once (two workgroups per CU) also every second round of the CUs
+        // reversed, which pairs long items with short ones on a CU
+        int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
+        if (lpt && total <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
         hipLaunchKernelGGL(sdpa_bwd_dq_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq, ctx->stream, q, k,
                            v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, hd);
         const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d64");
@@ -550,7 +553,8 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         const int nkb = (Lk + BM - 1) / BM;
         const long long total = (long long)nkb * B * H;
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
-        const int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nkb >= 2) ? 1 : 0;
+        int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nkb >= 2) ? 1 : 0;
+        if (lpt && total <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
         hipLaunchKernelGGL(sdpa_bwd_dkv_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
                            k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total, lpt, token_major, hd);
         return dl4s::launch_status("sdpa_bwd_dkv_f32_d64");

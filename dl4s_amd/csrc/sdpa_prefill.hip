@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
     float *Vs = lds + 2 * TILE_FLOATS;   // [2][BN][LSTR]
 
     int bh, unit;   // unit 0 = the last (longest) query block of the pair
-    if (!work_item(nqb, total_blocks, lpt, bh, unit)) return;
+    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H;
     const int hh = bh % H;
 
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
                                                                       const float *__restrict__ v, float *__restrict__ out,
                                                                       int H, int Lq, int Lk, float rT, MaskArgs mask,
                                                                       int strict, int nqb, int total_blocks, int token_major,
-                                                                      float *__restrict__ stats, int hd) {
+                                                                      float *__restrict__ stats, int hd, int order) {
     extern __shared__ __align__(16) float lds[];
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: lets the per-wavefront tile conditions branch on scalars
@@ -288,11 +288,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
     float *Ks = lds + wave * 2 * TILE_FLOATS;   // this wavefront's K tile, then its V tile
     float *Vs = Ks + TILE_FLOATS;
 
-    const int chunk = (total_blocks + 7) / 8;   // one contiguous run of the (batch*head)-major order per XCD
-    const int w = (blockIdx.x % 8) * chunk + blockIdx.x / 8;
-    if (w >= total_blocks) return;
-    const int bh = w / nqb;
-    const int qb = nqb - 1 - w % nqb;
+    int bh, unit;
+    if (!work_item(nqb, total_blocks, order & 1, bh, unit, order >> 1)) return;
+    const int qb = nqb - 1 - unit;   // longest rows first
     const int b = bh / H;
     const int hh = bh % H;
 
@@ -521,8 +519,15 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_split));
             split_attr_set[KIND] = true;
         }
+        // Rows of different length (causal masks, dense masks with tile skipping): longest first, and when the launch fits
+        // the chip at once (two workgroups per CU) every second round of the CUs reversed, which pairs long rows with
+        // short ones on a CU.  B4 H8 L512 causal: 24.3 us pair-major, 19.5 us longest first, 17.6 us with the reversal.
+        constexpr bool causal_kind32 = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+        int split_order = 0;
+        if ((causal_kind32 || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb32 >= 2)
+            split_order = 1 | (total32 <= 2ll * ctx->cu_count ? (ctx->cu_count / 8) << 1 : 0);
         hipLaunchKernelGGL(sdpa_prefill_split_f32_d64<KIND>, dim3((unsigned)((total32 + 7) / 8 * 8)), dim3(256), lds_split,
-                           ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major, stats, hd);
+                           ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major, stats, hd, split_order);
         return dl4s::launch_status("sdpa_prefill_split_f32_d64");
     }
     const int nqb = (Lq + BM - 1) / BM;
@@ -542,8 +547,11 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
         attr_set[KIND] = true;
     }
+    // a launch that fits the chip at once (three workgroups per CU): every second round of the CUs reversed as well
+    // (B2 H16 L2048 causal: 203 -> 161 us, B4 H16 L1024: 106 -> 88 us)
+    const int lpt_arg = lpt | ((lpt && total <= 3ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
     hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
-                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd);
+                       Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_d64");
 }
 
