@@ -339,6 +339,140 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
     }
 }
 
+// ---- Skinny products: few rows (a handful of tokens) against a whole weight matrix, e.g. the decoder's projections
+// during greedy decoding (NN/Models/Transformer/Transformer.swift:118-137 re-runs the decoder on the prefix for every
+// generated token).  The tiled kernels above would put such a product on a handful of workgroups of four wavefronts
+// that each walk all of K, one latency-bound step after the other.  Here a workgroup of SKW wavefronts owns a
+// 32 x 32 output block: each wavefront contracts one SKW-th of K straight from global memory (no staging: every
+// element of B is used once), the partial blocks are added up in LDS in wavefront order, and the block is finished
+// with alpha, beta and the fused Dense epilogue.  For very long K the contraction is also cut into S slices over
+// workgroups, which write part[z][s][M][N]; a second small kernel then adds the slices in order and finishes.  No
+// atomics anywhere: the same bits on every run.
+// op(A) is rows x K with K contiguous; B is K x N (TB = false) or N x K (TB = true).  K % 4 == 0.
+constexpr int SKW = 16;
+template <bool TB>
+__global__ __launch_bounds__(64 * SKW) void gemm_f32_skinny(GemmArgs g, float *__restrict__ part, int kslice, int nbn, int S) {
+    __shared__ float red[SKW][32][32];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+    const int cb = blockIdx.x % nbn, rb = blockIdx.x / nbn, s = blockIdx.y, z = blockIdx.z;
+    const float *A = g.A + (g.groups ? g.a_off[z] : (long long)z * g.a_bs);
+    const float *B = g.B + (g.groups ? g.b_off[z] : (long long)z * g.b_bs);
+    const int m = rb * 32 + ln, n = cb * 32 + ln;
+    const int share = kslice / SKW;   // a multiple of 8
+    const int k_begin = s * kslice + wave * share;
+    const int k_end = min(g.K, k_begin + share);
+    const float *arow = A + (long long)min(m, g.M - 1) * g.lda;
+    const int nc = min(n, g.N - 1);   // rows >= M and columns >= N compute on clamped addresses and are never stored
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    // One block = 8 of K: lanes 0..31 contract k = kb .. kb+3, lanes 32..63 k = kb+4 .. kb+7 (the order inside the
+    // contraction is free as long as both operands use it).  Loads are unconditional - out-of-range rows, columns and
+    // blocks read a valid address and are zeroed or dropped afterwards - and run one batch of SKU blocks ahead of the
+    // MFMAs, so that a wavefront has up to 2 * SKU blocks in flight instead of waiting for each (a kernel starts on a cold
+    // L2: every first touch pays the full memory latency, and little else limits these products).
+    constexpr int SKU = 4;
+    const int nblk = (k_end - k_begin + 7) / 8;
+    if (nblk > 0) {
+        auto fetch = [&](const int blk, f32x4 &a, f32x4 &b) {
+            const int kb = k_begin + 8 * min(blk, nblk - 1);
+            int k0 = kb + 4 * half;
+            if (k0 >= k_end) k0 = kb;
+            a = *reinterpret_cast<const f32x4 *>(arow + k0);
+            if (TB) {
+                b = *reinterpret_cast<const f32x4 *>(B + (long long)nc * g.ldb + k0);
+            } else {
+                const float *bp = B + (long long)k0 * g.ldb + nc;
+                b.x = bp[0]; b.y = bp[g.ldb]; b.z = bp[2 * g.ldb]; b.w = bp[3 * g.ldb];
+            }
+        };
+        auto contract = [&](const int base, const f32x4 (&a)[SKU], const f32x4 (&b)[SKU]) {
+#pragma unroll
+            for (int u = 0; u < SKU; ++u) {
+                // blocks past the end contribute nothing (both operands zeroed: the clamped loads hold real data)
+                const bool ok = base + u < nblk && k_begin + 8 * (base + u) + 4 * half < k_end;
+                const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                const f32x4 av = ok ? a[u] : zero, bv = ok ? b[u] : zero;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc, 0, 0, 0);
+            }
+        };
+        // two register sets taken in turn: the loads of one are in flight while the other is contracted
+        f32x4 a0[SKU], b0[SKU], a1[SKU], b1[SKU];
+#pragma unroll
+        for (int u = 0; u < SKU; ++u) fetch(u, a0[u], b0[u]);
+        for (int base = 0; base < nblk; base += 2 * SKU) {
+            if (base + SKU < nblk) {
+#pragma unroll
+                for (int u = 0; u < SKU; ++u) fetch(base + SKU + u, a1[u], b1[u]);
+            }
+            contract(base, a0, b0);
+            if (base + 2 * SKU < nblk) {
+#pragma unroll
+                for (int u = 0; u < SKU; ++u) fetch(base + 2 * SKU + u, a0[u], b0[u]);
+            }
+            if (base + SKU < nblk) contract(base + SKU, a1, b1);
+        }
+    }
+    // accumulator register r: row 8*(r/4) + 4*half + r%4, column ln
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[wave][8 * (r >> 2) + 4 * half + (r & 3)][ln] = acc[r];
+    __syncthreads();
+    const long long c_at = g.groups ? g.c_off[z] : (long long)z * g.c_bs;
+    float *pz = part ? part + ((long long)z * S + s) * g.M * g.N : nullptr;
+#pragma unroll
+    for (int i = 0; i < 1024 / (64 * SKW); ++i) {
+        const int e = tid + 64 * SKW * i, row = e >> 5, col = e & 31;
+        const int gm = rb * 32 + row, gn = cb * 32 + col;
+        if (gm < g.M && gn < g.N) {
+            float sum = red[0][row][col];
+#pragma unroll
+            for (int w = 1; w < SKW; ++w) sum += red[w][row][col];
+            const long long at = (long long)gm * g.N + gn;
+            if (pz) {
+                pz[at] = sum;
+            } else {
+                float *cp = g.C + c_at + at;
+                float val = g.alpha * sum;
+                if (g.beta != 0.f) val = val + g.beta * (*cp);
+                if (g.bias) val = __fadd_rn(val, g.bias[gn]);
+                if (g.act == 1) val = gelu_sigmoid(val);
+                if (g.residual) val = __fadd_rn(val, g.residual[c_at + at]);
+                *cp = val;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void gemm_f32_skinny_finish(GemmArgs g, const float *__restrict__ part, int S) {
+    const long long mn = (long long)g.M * g.N;
+    const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int z = blockIdx.z;
+    if (e >= mn) return;
+    const float *pz = part + (long long)z * S * mn + e;
+    float sum = 0.f;   // slices in order, eight loads in flight at a time
+    for (int s0 = 0; s0 < S; s0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = pz[(long long)min(s0 + i, S - 1) * mn];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (s0 + i < S) sum = (s0 + i == 0) ? v[i] : sum + v[i];
+    }
+    const long long c_at = g.groups ? g.c_off[z] : (long long)z * g.c_bs;
+    float *cp = g.C + c_at + e;
+    float val = g.alpha * sum;
+    if (g.beta != 0.f) val = val + g.beta * (*cp);
+    const long long gm = e / g.N;
+    const int gn = (int)(e - gm * g.N);
+    if (g.bias) val = __fadd_rn(val, g.bias[gn]);
+    if (g.act == 1) val = gelu_sigmoid(val);
+    if (g.residual) val = __fadd_rn(val, g.residual[c_at + e]);
+    *cp = val;
+}
+
 int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int64_t lbs, const float *rhs, int64_t rr,
                 int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb,
                 const float *bias = nullptr, const float *residual = nullptr, int act = 0, const float *const *group_lhs = nullptr,
@@ -380,6 +514,37 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     const bool fast = K > 0 && N % 4 == 0 && (ta ? k_by_rows_ok(M, lc) : rows_by_k_ok(lc)) && (tb ? rows_by_k_ok(rc) : k_by_rows_ok(N, rc)) &&
                       aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 && rbs % 4 == 0 && aligned16(result) && cbs % 4 == 0 &&
                       aligned16(bias) && aligned16(residual) && !(epi && (ta || tb)) && group_aligned;
+    // Skinny products (see gemm_f32_skinny): up to 128 rows, and too few 64 x 64 tiles to give every CU one.  The
+    // rule looks at one product's shape only, so a product gets the same bits alone, in a batch, in a group and with the
+    // fused Dense epilogue.
+    const auto rows_by_k_any = [&](int64_t ld) { return K % 4 == 0 && ld % 4 == 0; };
+    const bool skinny = !ta && K >= 64 && M <= 128 && ((M + 63) / 64) * ((N + 63) / 64) < ctx->cu_count && rows_by_k_any(lc) &&
+                        (tb ? rows_by_k_any(rc) : true) && aligned16(lhs) && (!tb || aligned16(rhs)) && lbs % 4 == 0 &&
+                        (!tb || rbs % 4 == 0) && group_aligned && M * N * batch < (1ll << 31) && K * (tb ? 1 : rc) < (1ll << 31);
+    if (skinny) {
+        const int nbn = (int)((N + 31) / 32), nbm = (int)((M + 31) / 32);
+        // One slice up to K = 1024; beyond, slices of 512 (one batch of loads per wavefront), since a single workgroup per
+        // column block pulls a long K through one CU: M16 N512 K2048 8.9 us against 15.3 us unsliced, K4096 8.9 against
+        // 26.9.  The slicing depends on K alone, so a product gets the same summation order alone, batched and grouped.
+        const int unit = 8 * SKW;
+        const long long S = K <= 1024 ? 1 : (K + 511) / 512;
+        const int kslice = (int)((((K + S - 1) / S) + unit - 1) / unit * unit);
+        const dim3 pgrid((unsigned)(nbn * nbm), (unsigned)S, (unsigned)batch);
+        if (S == 1) {
+            if (tb) hipLaunchKernelGGL(gemm_f32_skinny<true>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, (float *)nullptr, kslice, nbn, 1);
+            else hipLaunchKernelGGL(gemm_f32_skinny<false>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, (float *)nullptr, kslice, nbn, 1);
+            return dl4s::launch_status("gemm_f32_skinny");
+        }
+        std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
+        const int rc_s = dl4s::ensure_scratch(ctx, (size_t)(batch * S * M * N) * sizeof(float));
+        if (rc_s != DL4S_HIP_OK) return rc_s;
+        float *part = static_cast<float *>(ctx->scratch);
+        if (tb) hipLaunchKernelGGL(gemm_f32_skinny<true>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, part, kslice, nbn, (int)S);
+        else hipLaunchKernelGGL(gemm_f32_skinny<false>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, part, kslice, nbn, (int)S);
+        hipLaunchKernelGGL(gemm_f32_skinny_finish, dim3((unsigned)((M * N + 255) / 256), 1, (unsigned)batch), dim3(256), 0, ctx->stream, g,
+                           part, (int)S);
+        return dl4s::launch_status("gemm_f32_skinny");
+    }
     long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
     // small products: 64x64 tiles, so that there are at least about two workgroups per CU
     const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;

@@ -234,9 +234,14 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
                                                      const float *__restrict__ scale, const float *__restrict__ shift,
                                                      float *__restrict__ y, const float *__restrict__ part, long long n,
                                                      long long D, int nblk) {
+    __shared__ float sm[2 * TPB / 64];
     const long long b = blockIdx.y;
     float s = 0.f, ss = 0.f;
-    for (int i = 0; i < nblk; ++i) { s += part[(b * nblk + i) * 2]; ss += part[(b * nblk + i) * 2 + 1]; }
+    if ((int)threadIdx.x < nblk) {      // nblk <= TPB: one partial pair per thread, summed in a fixed order
+        s = part[(b * nblk + threadIdx.x) * 2];
+        ss = part[(b * nblk + threadIdx.x) * 2 + 1];
+    }
+    block_sum2(s, ss, sm);
     const float rN = __fdiv_rn(1.0f, (float)n);
     const float mean = __fmul_rn(s, rN);
     const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));

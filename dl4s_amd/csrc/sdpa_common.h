@@ -47,18 +47,26 @@ __global__ __launch_bounds__(256) void sdpa_mask_classify(MaskArgs m, int MB, in
     const int nrow = m.sq ? 32 : 1, ncol_ok = (m.sk ? col < Lk : (lane & 31) == 0);
     bool all0 = true, all1 = true, rows_open = true;
     const float *base = m.dense + bm * m.sb + hm * m.sh;
-    for (int it = 0; 2 * it < nrow; ++it) {           // lanes 0..31 take row 2*it, lanes 32..63 row 2*it + 1
+    // lanes 0..31 take row 2*it, lanes 32..63 row 2*it + 1; all 16 loads are issued before the first is looked at
+    float x[16];
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
         const int r = 2 * it + (lane >> 5);
         const int row = qt * 32 + r;
-        bool zero = false;
-        if (r < nrow && ncol_ok && (!m.sq || row < Lq)) {
-            const float x = base[row * m.sq + col * m.sk];
-            all0 = all0 && (x == 0.0f);
-            all1 = all1 && (x == 1.0f);
-            zero = (x == 0.0f);
+        x[it] = __builtin_nanf("");     // neither 0 nor 1: an element that does not exist
+        if (r < nrow && ncol_ok && (!m.sq || row < Lq)) x[it] = base[row * m.sq + col * m.sk];
+    }
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+        const int r = 2 * it + (lane >> 5);
+        const bool exists = r < nrow && ncol_ok && (!m.sq || qt * 32 + r < Lq);
+        const bool zero = exists && x[it] == 0.0f;
+        if (exists) {
+            all0 = all0 && zero;
+            all1 = all1 && (x[it] == 1.0f);
         }
         const unsigned long long zeros = __ballot(zero);
-        const bool row0 = !m.sq || qt * 32 + 2 * it < Lq, row1 = 2 * it + 1 < nrow && (!m.sq || qt * 32 + 2 * it + 1 < Lq);
+        const bool row0 = 2 * it < nrow && (!m.sq || qt * 32 + 2 * it < Lq), row1 = 2 * it + 1 < nrow && (!m.sq || qt * 32 + 2 * it + 1 < Lq);
         if (row0 && (unsigned)zeros == 0u) rows_open = false;
         if (row1 && (unsigned)(zeros >> 32) == 0u) rows_open = false;
     }

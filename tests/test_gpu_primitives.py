@@ -100,6 +100,57 @@ def test_gemm(ctx, orc, ta, tb, M, N, K):
         x.release()
 
 
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("M,N,K", [(1, 512, 512), (5, 2048, 512), (32, 512, 2048), (33, 70, 64), (100, 8000, 512), (128, 33, 100),
+                                   (17, 512, 68), (3, 5, 4096)])
+def test_gemm_skinny_products(ctx, orc, M, N, K, tb):
+    """Few rows against a whole weight matrix (the products of greedy decoding): the contraction is cut into slices over
+    workgroups and added up in a fixed order.  Parity with the oracle, alpha / beta, and the same bits alone, batched and
+    grouped."""
+    A = rnd(M, K)
+    B = (rnd(N, K) if tb else rnd(K, N)) * np.float32(0.2)     # weight-like magnitudes: two summation orders over 4096
+    C0 = rnd(M, N)                                               # unit-variance terms differ by more than the gate
+    dA, dB, dC = ctx.to_device(A), ctx.to_device(B), ctx.empty((M, N))
+    ctx.gemm(dA, A.shape, dB, B.shape, dC, 1.0, 0.0, False, tb)
+    ref = orc.gemm(A, B, False, tb)
+    assert_parity(dC.numpy(), ref, "skinny gemm %s" % ((M, N, K, tb),))
+    first = dC.numpy()
+    ctx.gemm(dA, A.shape, dB, B.shape, dC, 1.0, 0.0, False, tb)
+    assert np.array_equal(dC.numpy(), first)                      # no atomics: the same bits again
+    dD = ctx.to_device(C0)
+    ctx.gemm(dA, A.shape, dB, B.shape, dD, 2.0, 1.0, False, tb)  # beta accumulates
+    assert_parity(dD.numpy(), 2.0 * ref + C0, "skinny alpha beta")
+    # batched (shared right operand) and grouped launches give each product the bits of the single call
+    A3 = np.stack([A, rnd(M, K), A])
+    dA3, dC3 = ctx.to_device(A3), ctx.empty((3, M, N))
+    ctx.gemm_batched(dA3, (M, K), M * K, dB, B.shape, 0, dC3, M * N, 3, 1.0, 0.0, False, tb)
+    assert np.array_equal(dC3.numpy()[0], first) and np.array_equal(dC3.numpy()[2], first)
+    assert_parity(dC3.numpy()[1], orc.gemm(A3[1], B, False, tb), "skinny batched")
+    outs = [ctx.empty((M, N)) for _ in range(2)]
+    ctx.gemm_grouped([dA, dA3.offset(M * K * 4)], A.shape, [dB, dB], B.shape, outs, 1.0, 0.0, False, tb)
+    assert np.array_equal(outs[0].numpy(), first) and np.array_equal(outs[1].numpy(), dC3.numpy()[1])
+    for x in [dA, dB, dC, dD, dA3, dC3] + outs:
+        x.release()
+
+
+@pytest.mark.parametrize("tb", [False, True])
+def test_gemm_skinny_products_with_a_sliced_contraction(ctx, orc, tb):
+    """K long enough that the skinny form also cuts the contraction over workgroups (partial blocks in scratch, added up
+    by a second kernel): parity, and the bits of the single call when batched."""
+    M, N, K, batch = 3, 70, 16400, 3
+    A = rnd(batch, M, K)
+    B = (rnd(N, K) if tb else rnd(K, N)) * np.float32(0.05)
+    dA, dB, dC, d1 = ctx.to_device(A), ctx.to_device(B), ctx.empty((batch, M, N)), ctx.empty((M, N))
+    ctx.gemm_batched(dA, (M, K), M * K, dB, B.shape, 0, dC, M * N, batch, 1.0, 0.0, False, tb)
+    got = dC.numpy()
+    for b in range(batch):
+        ctx.gemm(dA.offset(b * M * K * 4), (M, K), dB, B.shape, d1, 1.0, 0.0, False, tb)
+        assert np.array_equal(d1.numpy(), got[b])
+        assert_parity(got[b], orc.gemm(A[b], B, False, tb), "sliced skinny %d" % b)
+    for x in (dA, dB, dC, d1):
+        x.release()
+
+
 def test_gemm_known_answers_and_beta(ctx):
     # Tests/DL4STests/VecTests.swift:127-156
     c = np.array([[1, 2, 3], [4, 5, 6]], np.float32)
@@ -274,7 +325,8 @@ def test_bias_gelu(ctx, orc):
         t.release()
 
 
-@pytest.mark.parametrize("M,K,N", [(130, 64, 72), (256, 128, 256), (64, 512, 1024), (7, 5, 3), (300, 100, 260)])
+@pytest.mark.parametrize("M,K,N", [(130, 64, 72), (256, 128, 256), (64, 512, 1024), (7, 5, 3), (300, 100, 260),
+                                   (5, 512, 2048), (31, 2048, 512), (100, 68, 70)])      # the last three: skinny products
 @pytest.mark.parametrize("act", [0, 1])
 @pytest.mark.parametrize("with_bias,with_res", [(True, False), (False, True), (True, True)])
 def test_dense_fused_equals_separate_engine_calls(ctx, orc, M, K, N, act, with_bias, with_res):
