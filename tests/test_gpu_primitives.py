@@ -102,7 +102,7 @@ def test_gemm(ctx, orc, ta, tb, M, N, K):
 
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("M,N,K", [(1, 512, 512), (5, 2048, 512), (32, 512, 2048), (33, 70, 64), (100, 8000, 512), (128, 33, 100),
-                                   (17, 512, 68), (3, 5, 4096)])
+                                   (17, 512, 68), (3, 5, 4096), (512, 64, 512), (300, 40, 100), (1000, 33, 64)])
 def test_gemm_skinny_products(ctx, orc, M, N, K, tb):
     """Few rows against a whole weight matrix (the products of greedy decoding): the contraction is cut into slices over
     workgroups and added up in a fixed order.  Parity with the oracle, alpha / beta, and the same bits alone, batched and
