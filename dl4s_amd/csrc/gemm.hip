@@ -515,13 +515,15 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
                       aligned16(lhs) && aligned16(rhs) && lbs % 4 == 0 && rbs % 4 == 0 && aligned16(result) && cbs % 4 == 0 &&
                       aligned16(bias) && aligned16(residual) && !(epi && (ta || tb)) && group_aligned;
     // Skinny products (see gemm_f32_skinny): up to 128 rows and too few 64 x 64 tiles to give every CU one, or any shape
-    // with so few 32 x 32 output blocks that half the CUs would get none (e.g. the weights . values product of one
-    // (batch, head) pair, [512,512] . [512,64], which the reference issues pair by pair, Tensor/Operators/Matrix.swift:
-    // 106-116).  The rule looks at one product's shape only, so a product gets the same bits alone, in a batch, in a
+    // with at most two 32 x 32 output blocks per CU (e.g. the weights . values product of one (batch, head) pair,
+    // [512,512] . [512,64], which the reference issues pair by pair, Tensor/Operators/Matrix.swift:106-116): the tiled
+    // kernels would run such a product one wavefront per SIMD or less.  Measured against the 64 x 64 tiles:
+    // [512,512].[512,512] 6.6 against 14.5 us, [1024,512].[512,512] 11.1 against 14.7 us; from [2048,512].[512,512]
+    // (1024 blocks) on the tiles win (16.6 against 21.0 us).  The rule looks at one product's shape only, so a product gets the same bits alone, in a batch, in a
     // group and with the fused Dense epilogue.
     const auto rows_by_k_any = [&](int64_t ld) { return K % 4 == 0 && ld % 4 == 0; };
     const bool few_rows = M <= 128 && ((M + 63) / 64) * ((N + 63) / 64) < ctx->cu_count;
-    const bool few_blocks = ((M + 31) / 32) * ((N + 31) / 32) <= ctx->cu_count / 2;
+    const bool few_blocks = ((M + 31) / 32) * ((N + 31) / 32) <= 2 * ctx->cu_count;
     const bool skinny = !ta && K >= 64 && (few_rows || few_blocks) && rows_by_k_any(lc) &&
                         (tb ? rows_by_k_any(rc) : true) && aligned16(lhs) && (!tb || aligned16(rhs)) && lbs % 4 == 0 &&
                         (!tb || rbs % 4 == 0) && group_aligned && M * N * batch < (1ll << 31) && K * (tb ? 1 : rc) < (1ll << 31);
