@@ -385,3 +385,44 @@ def test_stack_many_buffers(ctx, nbuf, count):
     assert np.array_equal(dst.numpy(), ref)
     for d in dev + [dst]:
         d.release()
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_gemm_random_shapes_and_forms(ctx, seed):
+    """Seeded random extents around the boundaries between the tiled, skinny and scalar-load kernels, every transpose
+    combination, alone / batched / grouped, against an fp64 product (the bound scales with the size of the sums)."""
+    rng = np.random.default_rng(7000 + seed)
+    pick = lambda: int(rng.choice([1, 3, 4, 8, 31, 32, 33, 64, 100, 128, 129, 260, 512, 1000]))
+    M, N, K = pick(), pick(), int(rng.choice([1, 4, 6, 60, 64, 68, 100, 256, 516, 1028, 2048]))
+    ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    form = ["single", "batched", "grouped"][int(rng.integers(0, 3))]
+    count = 1 if form == "single" else int(rng.integers(2, 5))
+    As = [(rng.standard_normal((K, M) if ta else (M, K))).astype(np.float32) for _ in range(count)]
+    Bs = [(rng.standard_normal((N, K) if tb else (K, N)) * 0.1).astype(np.float32) for _ in range(count)]
+    what = "seed %d: M%d N%d K%d ta%d tb%d %s x%d" % (seed, M, N, K, ta, tb, form, count)
+    refs = [(a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64) for a, b in zip(As, Bs)]
+    outs = [ctx.empty((M, N)) for _ in range(count)]
+    keep = []
+    if form == "batched":
+        dA, dB, dC = ctx.to_device(np.stack(As)), ctx.to_device(np.stack(Bs)), ctx.empty((count, M, N))
+        keep = [dA, dB, dC]
+        ctx.gemm_batched(dA, As[0].shape, As[0].size, dB, Bs[0].shape, Bs[0].size, dC, M * N, count, 1.0, 0.0, ta, tb)
+        got = list(dC.numpy())
+    else:
+        dA, dB = [ctx.to_device(a) for a in As], [ctx.to_device(b) for b in Bs]
+        keep = dA + dB
+        if form == "grouped":
+            ctx.gemm_grouped(dA, As[0].shape, dB, Bs[0].shape, outs, 1.0, 0.0, ta, tb)
+        else:
+            ctx.gemm(dA[0], As[0].shape, dB[0], Bs[0].shape, outs[0], 1.0, 0.0, ta, tb)
+        got = [o.numpy() for o in outs]
+    for g, r in zip(got, refs):
+        bound = 2e-6 * np.sqrt(K) * (np.abs(r).max() + 1.0) + 1e-6
+        assert np.abs(g - r).max() <= bound, "%s: max |d| %.3e > %.3e" % (what, np.abs(g - r).max(), bound)
+    # every form gives the bits of the single call
+    single = ctx.empty((M, N))
+    a0, b0 = ctx.to_device(As[-1]), ctx.to_device(Bs[-1])
+    ctx.gemm(a0, As[-1].shape, b0, Bs[-1].shape, single, 1.0, 0.0, ta, tb)
+    assert np.array_equal(single.numpy(), got[-1]), what
+    for x in keep + outs + [single, a0, b0]:
+        x.release()
