@@ -184,8 +184,9 @@ __device__ __forceinline__ bool work_item(const int nunits, const int total_bloc
 // S^T = K . Q^T for one 32-key tile of one wavefront (lane = query qi = q0 + lane % 32, 16 of the 32 keys per lane:
 // accumulator register r is key k0 + 8(r/4) + 4*half + r%4), then the mask, in registers.  Kb is the lane's K fragment
 // base in LDS; qr the lane's Q fragment, already scaled by (1/T) log2(e): the scores are in the base-2 exponent domain.
-template <int KIND>
-__device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&qr)[32], const int k0, const int q0, const int qi,
+// NJ: 128-bit reads per K row fragment (head dim / 8: 8 for the 64-wide kernels, 16 for the 128-wide one)
+template <int KIND, int NJ = 8>
+__device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&qr)[4 * NJ], const int k0, const int q0, const int qi,
                                                 const int half, const int Lk, const int len, const float *mrow,
                                                 const long long msk, const int cls) {
     constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
@@ -195,7 +196,7 @@ __device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&q
     // (one dependent accumulation chain keeps the matrix pipe full; the first MFMA takes a literal zero)
     f32x16 s0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < NJ; ++j) {
         const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Kb + 4 * j);
         if (j == 0) {
             const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};

@@ -21,11 +21,13 @@
 // queries beyond Lq are computed and not stored.
 //
 // Kernels in this file: sdpa_prefill_f32_d64 (above), sdpa_prefill_split_f32_d64 (small launches: the keys of a
-// 32-query block split over the 4 wavefronts of a workgroup), sdpa_generic_f32 (head dims other than 64).  Both MFMA
-// kernels can also leave the two row statistics the backward pass needs (sdpa_backward.hip).
+// 32-query block split over the 4 wavefronts of a workgroup), sdpa_generic_f32 (head dims the MFMA kernels do not take);
+// sdpa_prefill_f32_d128 for head dims above 64 up to 128 is in sdpa_prefill_d128.h.  The two 64-wide MFMA kernels can
+// also leave the two row statistics the backward pass needs (sdpa_backward.hip).
 #include <type_traits>
 
 #include "sdpa_common.h"
+#include "sdpa_prefill_d128.h"
 
 namespace {
 
@@ -575,9 +577,14 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
     const bool mfma_path = dk == dv && dk <= HD && dk % 4 == 0 &&
                            ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                              reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    // head dims above 64 up to 128: the 128-wide MFMA kernel.  Not when row statistics are wanted: the gradient kernels
+    // for these head dims are the plain ones, which read the plain forward kernel's statistics.
+    const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                           reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const bool mfma128_path = dk == dv && dk > HD && dk <= HD2 && dk % 4 == 0 && aligned && !stats;
     MaskArgs m{};
     {
-        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path, m);
+        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path, m);
         if (rc != DL4S_HIP_OK) return rc;
     }
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
@@ -598,7 +605,18 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
             default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
         }
     }
-    DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 64, and 16-byte aligned tensors");
+    if (mfma128_path) {
+        DL4S_REQUIRE(Lk * (token_major ? H : 1) * dk * 4 < (dk == HD2 ? (1ll << 31) : (1ll << 30)), DL4S_HIP_EUNSUPPORTED,
+                     "sdpa: the K/V rows of one (batch, head) pair span more than 2 GiB (1 GiB for padded head dims)");
+        switch (m.kind) {
+            case DL4S_MASK_NONE: return launch_d128<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+            case DL4S_MASK_DENSE_F32: return launch_d128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+            case DL4S_MASK_CAUSAL: return launch_d128<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+            case DL4S_MASK_KEY_LENGTHS: return launch_d128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+            default: return launch_d128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+        }
+    }
+    DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 128 (64 with row statistics), and 16-byte aligned tensors");
     DL4S_REQUIRE(dk <= GEN_MAXD && dv <= GEN_MAXD && dv > 0, DL4S_HIP_EUNSUPPORTED,
                  "sdpa: head dims (%lld, %lld) above %d are not implemented", (long long)dk, (long long)dv, GEN_MAXD);
     const long long rows = B * H * Lq;

@@ -74,7 +74,12 @@ SHAPES = [  # B, H, Lq, Lk, d
     (1, 2, 5, 7, 4),        # the golden-fixture shape: MFMA kernel with 60 padding columns
     (2, 3, 9, 11, 8),       # key size of Tests/DL4STests/TransformerTests.swift:31
     (2, 3, 9, 11, 6),       # not a multiple of 4: plain kernel
-    (1, 2, 40, 50, 96),     # above 64: plain kernel
+    (1, 2, 40, 50, 96),     # above 64: the 128-wide MFMA kernel with padding columns
+    (2, 2, 200, 333, 128),
+    (2, 3, 130, 70, 72),
+    (1, 2, 100, 100, 100),
+    (1, 2, 40, 50, 130),    # not a multiple of 4 / above 128: plain kernel
+    (1, 1, 33, 40, 200),
     (2, 3, 130, 70, 32),    # padded MFMA tiles, ragged
     (2, 2, 200, 333, 40),
     (1, 2, 100, 100, 60),
@@ -137,14 +142,14 @@ def test_different_key_and_value_dims(ctx, orc):
 
 def test_nil_mask_equals_zero_mask_bitwise(ctx):
     rng = np.random.default_rng(3)
-    for d in (8, 10, 64):
+    for d in (8, 10, 64, 128, 100):
         q, k, v = rand(rng, 2, 2, 70, d), rand(rng, 2, 2, 90, d), rand(rng, 2, 2, 90, d)
         a = run_sdpa(ctx, q, k, v, None)
         b = run_sdpa(ctx, q, k, v, np.zeros((70, 90), np.float32))
         assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("d", [8, 10, 64])
+@pytest.mark.parametrize("d", [8, 10, 64, 128, 88])
 def test_blocked_keys_have_exactly_zero_weight_and_blocked_rows_are_uniform(ctx, orc, d):
     rng = np.random.default_rng(5)
     B, H, Lq, Lk = 1, 2, 70, 100
@@ -165,7 +170,7 @@ def test_blocked_keys_have_exactly_zero_weight_and_blocked_rows_are_uniform(ctx,
     assert not np.isnan(base).any()
 
 
-@pytest.mark.parametrize("d", [8, 10, 64])
+@pytest.mark.parametrize("d", [8, 10, 64, 128, 88])
 def test_nan_inf_placement_matches_oracle(ctx, orc, d):
     rng = np.random.default_rng(9)
     B, H, Lq, Lk = 1, 1, 40, 150
@@ -377,7 +382,7 @@ def test_config5_incremental_decode_append_then_attend(ctx, orc):
         buf.release()
 
 
-@pytest.mark.parametrize("d", [64, 8, 36])
+@pytest.mark.parametrize("d", [64, 8, 36, 128, 80])
 @pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 70), (1, 2, 5, 7), (2, 4, 256, 256), (1, 5, 33, 161)])
 def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk, d):
     """[B,L,H,d] operands (what the projections of MultiHeadAttention produce before its permutes,
@@ -398,8 +403,8 @@ def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk, d):
 
 def test_token_major_rejected_for_other_head_dims_and_unknown_flags(ctx):
     from dl4s_amd import lib
-    q = ctx.empty((1, 2, 4, 128))
-    for d in (6, 72, 128):      # neither a multiple of 4 up to 64
+    q = ctx.empty((1, 2, 4, 256))
+    for d in (6, 130, 200):     # not a multiple of 4 up to 128
         with pytest.raises(lib.Dl4sHipError):
             ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, d, d, 0.5, None, lib.SDPA_TOKEN_MAJOR)
     with pytest.raises(lib.Dl4sHipError):       # different key and value dims
