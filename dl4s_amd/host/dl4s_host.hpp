@@ -806,10 +806,10 @@ struct MultiHeadAttention {
           qDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})), kDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})),
           vDense(Tensor::repeating(0.f, {hiddenDim_, valueDim_ * heads_})), fc(Tensor::repeating(0.f, {valueDim_ * heads_, hiddenDim_})),
           norm(Shape{hiddenDim_}), dropout(dropoutRate) {}
-    // fused mode, equal head dims that are a multiple of 4 up to 64 (what the token-major attention kernels take): the
+    // fused mode, equal head dims that are a multiple of 4 up to 128 (what the token-major attention kernels take): the
     // key / value projections alone, [B,L,H,d], for callers that attend to the same keys and values repeatedly (the
     // encoder states during greedy decoding)
-    bool canCacheProjections() const { return Device::fused() && keyDim == valueDim && keyDim <= 64 && keyDim % 4 == 0; }
+    bool canCacheProjections() const { return Device::fused() && keyDim == valueDim && keyDim <= 128 && keyDim % 4 == 0; }
     // The projections are separate products in the reference (MultiHeadAttention.swift:105-107); the key and value ones
     // (and the query one, when all three inputs have one length) go out as one grouped launch.
     std::pair<Tensor, Tensor> projectKeysValues(const Tensor &k, const Tensor &v, const Tensor *q = nullptr, Tensor *qp = nullptr) const {

@@ -100,6 +100,23 @@ def test_tiny_transformer_layers(ctx, host, orc, fused):
                   orc.decoder_block(x, enc, dec_mask, enc_mask, attn, attn2, ffn, H, dk, dk), "decoder block")
 
 
+@pytest.mark.parametrize("fused", MODES)
+@pytest.mark.parametrize("dk", [96, 128, 12])
+def test_mha_with_other_head_dims(ctx, host, orc, fused, dk):
+    """Head dims other than 64: in fused mode the token-major attention kernels take every multiple of 4 up to 128 (the
+    64-wide and 128-wide MFMA kernels with padding columns)."""
+    B, L, Le, D, H = 2, 40, 50, 32, 2
+    rng = np.random.default_rng(dk)
+    attn, _ = m64.make_params(rng, D, H, dk, dk, 8)
+    x = rng.standard_normal((B, L, D)).astype(np.float32)
+    enc = rng.standard_normal((B, Le, D)).astype(np.float32)
+    enc_mask = orc.make_encoder_masks([33, Le])
+    assert_parity(host.mha(ctx, x, enc, enc, enc_mask, attn, H, dk, dk, fused=fused),
+                  orc.mha(x, enc, enc, enc_mask, attn, H, dk, dk), "MHA cross dk=%d" % dk)
+    cm = causal_mask(L, L)
+    assert_parity(host.mha(ctx, x, x, x, cm, attn, H, dk, dk, fused=fused), orc.mha(x, x, x, cm, attn, H, dk, dk), "MHA self dk=%d" % dk)
+
+
 def _config2():
     B, L, D, H, dk = 4, 512, 512, 8, 64
     rng = np.random.Generator(np.random.PCG64(1002))
