@@ -216,6 +216,33 @@ def other_configs(ctx, lib, cpu):
             "sample": "2 of 128 (batch, head) slices, dense causal mask (%.1f s)" % dt}
     for b_ in bufs + outs + [st]:
         b_.release()
+    # the headline shape with the mask as an unmodified DL4S passes it (a dense [L,L] tensor): all-ones tiles skipped
+    # (default) and every tile visited (DL4S_SDPA_STRICT); and the same shape with head dim 128 (causal descriptor)
+    B, H, L = 8, 16, 2048
+    rng = np.random.Generator(np.random.PCG64(1008))
+    i, j = np.indices((L, L))
+    dmask = ctx.to_device((j > i).astype(np.float32))
+    for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal")):
+        qkv = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(3)]
+        o = ctx.empty((B, H, L, d))
+        rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+        fl = 4.0 * d * B * H * (L * (L + 1) // 2)
+        entry = {"flops": fl}
+        variants = (("tile_skipping", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), 0), ("strict", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), lib.SDPA_STRICT)) \
+            if d == 64 else (("causal_descriptor", ctx.mask_desc(lib.MASK_CAUSAL), 0),)
+        for vname, desc, flags in variants:
+            for _ in range(100):
+                ctx.sdpa_fwd(qkv[0], qkv[1], qkv[2], o, B, H, L, L, d, d, rT, desc, flags)
+            ctx.sync()
+            ctx.timer_begin()
+            for _ in range(30):
+                ctx.sdpa_fwd(qkv[0], qkv[1], qkv[2], o, B, H, L, L, d, d, rT, desc, flags)
+            ms = ctx.timer_end() / 30
+            entry[vname] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS}
+        res[name] = entry
+        for b_ in qkv + [o]:
+            b_.release()
+    dmask.release()
     # the caller of the blocks: Transformer greedy decoding (batch 1; every step re-runs the decoder on the prefix, as the
     # reference does).  6 + 6 layers, hidden 512, 8 heads of 64, ffn 2048, vocabulary 8000, 64 source tokens, 32 generated.
     rng = np.random.Generator(np.random.PCG64(1006))
