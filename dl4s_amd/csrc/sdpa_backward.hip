@@ -409,6 +409,341 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
     }
 }
 
+// ------------------------------------------------------------------------------------------------ small launches
+// Too few 32-row blocks to give every SIMD about two wavefronts (the forward pass's rule): a workgroup is ONE 32-query
+// block (dQ) or ONE 32-key block (dK, dV) whose tiles along the other axis are dealt round-robin to its 4 wavefronts.
+// Each wavefront stages its own tiles in its own LDS region (the LDS operations of one wavefront execute in order, so
+// the loop has no workgroup barrier); the four partial gradient blocks are added in wavefront order at the end.
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_split_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
+                                                                     const float *__restrict__ v, const float *__restrict__ dout,
+                                                                     const float *__restrict__ stats, const float *__restrict__ D,
+                                                                     float *__restrict__ dq, int H, int Lq, int Lk, float rT,
+                                                                     MaskArgs mask, int strict, int nqb, int total_blocks, int order,
+                                                                     int token_major, int hd) {
+    extern __shared__ __align__(16) float lds[];
+    int bh, unit;
+    if (!work_item(nqb, total_blocks, order & 1, bh, unit, order >> 1)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    float *Ks = lds + wave * 2 * TILE_FLOATS, *Vs = Ks + TILE_FLOATS;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int qb = nqb - 1 - unit;   // longest rows first
+    const int q0 = qb * 32;
+    const int qi = q0 + ln;
+    const int qic = qi < Lq ? qi : Lq - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
+
+    int kend = Lk;
+    bool skip_ones = false;
+    if (!strict && !(LENS && len <= 0)) {
+        if (DENSE && mask.cls) {
+            const int blk = min(q0, Lq - 1) >> 5;
+            const unsigned char *row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)blk * mask.cls_sq;
+            skip_ones = dense_block_open(row, mask.cls_sk, blk, (Lk + 31) >> 5);
+            kend = dense_key_bound(row, mask.cls_sk, blk, Lk);
+        }
+        if (CAUSAL) kend = min(kend, q0 + 32);
+        if (LENS) kend = min(kend, len);
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    float qr[32], gr[32];
+    {
+        const float *qp = q + q_base + (long long)qic * rs + half * 32;
+        const float *gp = dout + q_base + (long long)qic * rs + half * 32;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
+            if (half * 32 + 4 * j < hd) {
+                t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+                g = *reinterpret_cast<const f32x4 *>(gp + 4 * j);
+            }
+            qr[4 * j + 0] = (t.x * rT) * LOG2E; qr[4 * j + 1] = (t.y * rT) * LOG2E;
+            qr[4 * j + 2] = (t.z * rT) * LOG2E; qr[4 * j + 3] = (t.w * rT) * LOG2E;
+            gr[4 * j + 0] = g.x; gr[4 * j + 1] = g.y; gr[4 * j + 2] = g.z; gr[4 * j + 3] = g.w;
+        }
+    }
+    const float m_i = stats[2 * ((long long)bh * Lq + qic)];
+    const float rl_i = stats[2 * ((long long)bh * Lq + qic) + 1];
+    const float D_i = D[(long long)bh * Lq + qic];
+
+    // the wavefront stages its own tiles: lane covers rows (i*4 + lane/16), 4 floats at column (lane%16)*4
+    const int ld_row = lane >> 4, ld_col = (lane & 15) * 4;
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
+    const unsigned ld_off = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
+    const unsigned row4_bytes = 4u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[8], vst[8];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int o = (int)(ld_off + t * tile_bytes + i * row4_bytes);
+            kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o, 0, 0));
+            vst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o, 0, 0));
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int off = (i * 4 + ld_row) * LSTR + ld_col;
+            *reinterpret_cast<f32x4 *>(Ks + off) = kst[i];
+            *reinterpret_cast<f32x4 *>(Vs + off) = vst[i];
+        }
+    };
+
+    f32x16 a0, a1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { a0[i] = 0.f; a1[i] = 0.f; }
+    const int row_lds = ln * LSTR + half * 32;
+    const int col_lds = (4 * half) * LSTR + 2 * ln;
+    const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
+
+    if (wave < ntiles) { load_tile(wave); store_tile(); }
+    for (int t = wave; t < ntiles; t += 4) {
+        const bool more = (t + 4 < ntiles);
+        if (more) load_tile(t + 4);
+        const int k0 = t * BN;
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        if (!(DENSE && skip_ones && cls == 1)) {
+            f32x16 p = masked_scores<KIND>(Ks + row_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p[r] = fast_exp2(p[r] - m_i) * rl_i;
+            const f32x16 dp = tile_product(Vs + row_lds, gr);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p[r] = p[r] * (dp[r] - D_i);
+            tile_accumulate_t(Ks + col_lds, p, a0, a1);
+        }
+        if (more) store_tile();
+    }
+
+    // add the four partial dQ^T blocks in wavefront order
+    __syncthreads();
+    float *mine = lds + wave * 2 * TILE_FLOATS;   // [32][64]
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { mine[(2 * r) * 64 + lane] = a0[r]; mine[(2 * r + 1) * 64 + lane] = a1[r]; }
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int x = 1; x < 4; ++x) {
+            const float *other = lds + x * 2 * TILE_FLOATS;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { a0[r] += other[(2 * r) * 64 + lane]; a1[r] += other[(2 * r + 1) * 64 + lane]; }
+        }
+        if (qi < Lq) store_row_t(dq + q_base + (long long)qi * rs + 8 * half, a0, a1, rT, hd - 8 * half);
+    }
+}
+
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_split_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
+                                                                      const float *__restrict__ v, const float *__restrict__ dout,
+                                                                      const float *__restrict__ stats, const float *__restrict__ D,
+                                                                      float *__restrict__ dk, float *__restrict__ dv, int H, int Lq,
+                                                                      int Lk, float rT, MaskArgs mask, int strict, int nkb,
+                                                                      int total_blocks, int order, int token_major, int hd) {
+    extern __shared__ __align__(16) float lds[];
+    int bh, unit;
+    if (!work_item(nkb, total_blocks, order & 1, bh, unit, order >> 1)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int REGION = 2 * TILE_FLOATS + 96;   // q tile, dout tile, the tile's (m, 1/l, D)
+    float *Qs = lds + wave * REGION, *Gs = Qs + TILE_FLOATS, *Ss = Gs + TILE_FLOATS;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int kb = unit;                 // under a causal mask the first key block meets the most queries
+    const int kw0 = kb * 32;
+    const int key = kw0 + ln;
+    const int keyc = key < Lk ? key : Lk - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
+
+    const int nqt = (Lq + 31) / 32;
+    int t_begin = 0;
+    const unsigned char *skip_cls0 = nullptr;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) t_begin = kw0 / 32;
+        if (LENS && kw0 >= len) t_begin = nqt;
+        if (DENSE && mask.cls) {
+            skip_cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
+            t_begin = dense_query_begin(mask, skip_cls0, min(kw0, Lk - 1) >> 5, nqt, (Lk + 31) >> 5);
+        }
+    }
+
+    float kr[32], vr[32];
+    {
+        const float *kp = k + kv_base + (long long)keyc * rs + half * 32;
+        const float *vp = v + kv_base + (long long)keyc * rs + half * 32;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
+            if (half * 32 + 4 * j < hd) {
+                a = *reinterpret_cast<const f32x4 *>(kp + 4 * j);
+                c = *reinterpret_cast<const f32x4 *>(vp + 4 * j);
+            }
+            kr[4 * j + 0] = a.x; kr[4 * j + 1] = a.y; kr[4 * j + 2] = a.z; kr[4 * j + 3] = a.w;
+            vr[4 * j + 0] = c.x; vr[4 * j + 1] = c.y; vr[4 * j + 2] = c.z; vr[4 * j + 3] = c.w;
+        }
+    }
+
+    const int ld_row = lane >> 4, ld_col = (lane & 15) * 4;
+    const int q_bytes = (int)(((long long)(Lq - 1) * rs + hd) * 4);
+    const __amdgpu_buffer_rsrc_t qrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(q + q_base), 0, q_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t grsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(dout + q_base), 0, q_bytes, 0x00020000);
+    const unsigned ld_off = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
+    const unsigned row4_bytes = 4u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
+    // a query tile in two halves of 16 rows, so that the staging registers stay few
+    f32x4 qst[4], gst[4];
+    float s_ml = 0.f, s_d = 0.f;   // lanes 0..31: reference maximum and D of the tile's query ln; lanes 32..63: 1 / row sum
+    auto load_half = [&](int t, int h) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int o = (int)(ld_off + t * tile_bytes + (4 * h + i) * row4_bytes);
+            qst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(qrsrc, o, 0, 0));
+            gst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(grsrc, o, 0, 0));
+        }
+        if (h == 0) {
+            const int row = t * 32 + ln;
+            const long long at = (long long)bh * Lq + row;
+            s_ml = 0.f; s_d = 0.f;
+            if (row < Lq) {
+                s_ml = stats[2 * at + half];
+                if (half == 0) s_d = D[at];
+            }
+        }
+    };
+    auto store_half = [&](int h) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int off = ((4 * h + i) * 4 + ld_row) * LSTR + ld_col;
+            f32x4 sc;
+            sc.x = (qst[i].x * rT) * LOG2E; sc.y = (qst[i].y * rT) * LOG2E;
+            sc.z = (qst[i].z * rT) * LOG2E; sc.w = (qst[i].w * rT) * LOG2E;
+            *reinterpret_cast<f32x4 *>(Qs + off) = sc;
+            *reinterpret_cast<f32x4 *>(Gs + off) = gst[i];
+        }
+        if (h == 0) {
+            Ss[half * 32 + ln] = s_ml;           // [0..31] m, [32..63] 1 / l
+            if (half == 0) Ss[64 + ln] = s_d;    // [64..95] D
+        }
+    };
+
+    f32x16 k0a, k1a, v0a, v1a;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { k0a[i] = 0.f; k1a[i] = 0.f; v0a[i] = 0.f; v1a[i] = 0.f; }
+    const int row_lds = ln * LSTR + half * 32;
+    const int col_lds = (4 * half) * LSTR + 2 * ln;
+    const float PEN = __fmul_rn(1e9f, LOG2E);
+    const unsigned char *cls_col = nullptr;
+    if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
+    const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
+
+    // query tile t belongs to wavefront t % 4 whatever t_begin is, so that skipping tiles does not change which partial
+    // sum a tile goes into (the same bits with and without skipping)
+    for (int t = t_begin + ((wave - t_begin) & 3); t < nqt; t += 4) {
+        load_half(t, 0);
+        store_half(0);
+        load_half(t, 1);
+        store_half(1);
+        const int qt0 = t * 32;
+        int cls = 2;
+        if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq] & 3;
+        if (DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5)) continue;
+        f32x16 p = tile_product(Qs + row_lds, kr);
+        if (DENSE) {
+            if (cls == 1) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = __fsub_rn(p[r], PEN);
+            } else if (cls == 2) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    const int qc = qg < Lq ? qg : Lq - 1;
+                    p[r] = __fsub_rn(p[r], __fmul_rn(__fmul_rn(mcol[qc * mask.sq], 1e9f), LOG2E));
+                }
+            }
+        } else if ((CAUSAL && (kw0 + 31 > qt0)) || (LENS && (kw0 + 32 > len))) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                bool blocked = false;
+                if (CAUSAL) blocked = blocked || (key > qg);
+                if (LENS) blocked = blocked || (key >= len);
+                if (blocked) p[r] = __fsub_rn(p[r], PEN);
+            }
+        }
+        const float *st = Ss + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 m4 = *reinterpret_cast<const f32x4 *>(st + 8 * g);
+            const f32x4 r4 = *reinterpret_cast<const f32x4 *>(st + 32 + 8 * g);
+            p[4 * g + 0] = fast_exp2(p[4 * g + 0] - m4.x) * r4.x;
+            p[4 * g + 1] = fast_exp2(p[4 * g + 1] - m4.y) * r4.y;
+            p[4 * g + 2] = fast_exp2(p[4 * g + 2] - m4.z) * r4.z;
+            p[4 * g + 3] = fast_exp2(p[4 * g + 3] - m4.w) * r4.w;
+        }
+        tile_accumulate_t(Gs + col_lds, p, v0a, v1a);
+        const f32x16 dp = tile_product(Gs + row_lds, vr);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(st + 64 + 8 * g);
+            p[4 * g + 0] = p[4 * g + 0] * (dp[4 * g + 0] - d4.x);
+            p[4 * g + 1] = p[4 * g + 1] * (dp[4 * g + 1] - d4.y);
+            p[4 * g + 2] = p[4 * g + 2] * (dp[4 * g + 2] - d4.z);
+            p[4 * g + 3] = p[4 * g + 3] * (dp[4 * g + 3] - d4.w);
+        }
+        tile_accumulate_t(Qs + col_lds, p, k0a, k1a);
+    }
+
+    // add the four partial dK^T / dV^T blocks in wavefront order
+    __syncthreads();
+    float *mine = lds + wave * REGION;   // [64][64]
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            mine[(4 * r + 0) * 64 + lane] = k0a[r]; mine[(4 * r + 1) * 64 + lane] = k1a[r];
+            mine[(4 * r + 2) * 64 + lane] = v0a[r]; mine[(4 * r + 3) * 64 + lane] = v1a[r];
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+        for (int x = 1; x < 4; ++x) {
+            const float *other = lds + x * REGION;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                k0a[r] += other[(4 * r + 0) * 64 + lane]; k1a[r] += other[(4 * r + 1) * 64 + lane];
+                v0a[r] += other[(4 * r + 2) * 64 + lane]; v1a[r] += other[(4 * r + 3) * 64 + lane];
+            }
+        }
+        if (key < Lk) {
+            store_row_t(dv + kv_base + (long long)key * rs + 8 * half, v0a, v1a, 1.0f, hd - 8 * half);
+            store_row_t(dk + kv_base + (long long)key * rs + 8 * half, k0a, k1a, LN2, hd - 8 * half);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ other head dims
 // Plain gradient kernels for head dims other than 64 (up to 256, key dim = value dim = d), the counterpart of the plain
 // forward kernel: correctness paths for small models, one wavefront per query row (dq) and per key row (dk, dv).
@@ -524,19 +859,37 @@ __global__ __launch_bounds__(64) void sdpa_bwd_dkv_plain(const float *__restrict
 template <int KIND>
 int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
                const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
-               int strict, int token_major, int hd) {
+               int strict, int token_major, int hd, int no_split) {
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     static bool attr_set[8] = {false};
     const size_t lds_dq = 4 * TILE_FLOATS * sizeof(float);
     const size_t lds_dkv = (4 * TILE_FLOATS + 192) * sizeof(float);
+    const size_t lds_dq_split = 8 * TILE_FLOATS * sizeof(float);
+    const size_t lds_dkv_split = 4 * (2 * TILE_FLOATS + 96) * sizeof(float);
     if (!attr_set[KIND]) {
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_f32_d64<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq));
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d64<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_split_f32_d64<KIND>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq_split));
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_split_f32_d64<KIND>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv_split));
         attr_set[KIND] = true;
     }
-    {
+    const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
+    // Small launches (the forward pass's rule, from the extents only): one 32-row block per workgroup, the tiles along the
+    // other axis split over its four wavefronts.
+    if (!no_split && (long long)B * H * ((Lq + 31) / 32) < 8ll * ctx->cu_count && Lk >= 2 * BN) {
+        const int nqb32 = (Lq + 31) / 32;
+        const long long total = (long long)nqb32 * B * H;
+        int order = (uneven && nqb32 >= 2) ? 1 : 0;
+        if (order && total <= 2ll * ctx->cu_count) order |= (ctx->cu_count / 8) << 1;
+        hipLaunchKernelGGL(sdpa_bwd_dq_split_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq_split, ctx->stream,
+                           q, k, v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb32, (int)total, order, token_major, hd);
+        const int rc = dl4s::launch_status("sdpa_bwd_dq_split_f32_d64");
+        if (rc != DL4S_HIP_OK) return rc;
+    } else {
         const int nqb = (Lq + BM - 1) / BM;
         const long long total = (long long)nqb * B * H;
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
@@ -548,6 +901,15 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                            v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, hd);
         const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d64");
         if (rc != DL4S_HIP_OK) return rc;
+    }
+    if (!no_split && (long long)B * H * ((Lk + 31) / 32) < 8ll * ctx->cu_count && Lq >= 2 * BN) {
+        const int nkb32 = (Lk + 31) / 32;
+        const long long total = (long long)nkb32 * B * H;
+        int order = (uneven && nkb32 >= 2) ? 1 : 0;
+        if (order && total <= 2ll * ctx->cu_count) order |= (ctx->cu_count / 8) << 1;
+        hipLaunchKernelGGL(sdpa_bwd_dkv_split_f32_d64<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv_split, ctx->stream,
+                           q, k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb32, (int)total, order, token_major, hd);
+        return dl4s::launch_status("sdpa_bwd_dkv_split_f32_d64");
     }
     {
         const int nkb = (Lk + BM - 1) / BM;
@@ -599,6 +961,7 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path, m);
     if (rc != DL4S_HIP_OK) return rc;
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
+    const int no_split = (flags & DL4S_SDPA_NO_KEY_SPLIT) ? 1 : 0;
     void *Dv = nullptr;
     rc = dl4s_hip_alloc(ctx, (size_t)(B * H * Lq) * sizeof(float), &Dv);
     if (rc != DL4S_HIP_OK) return rc;
@@ -624,11 +987,11 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     rc = dl4s::launch_status("sdpa_bwd_rowdot");
     if (rc == DL4S_HIP_OK) {
         switch (m.kind) {
-            case DL4S_MASK_NONE: rc = launch_bwd<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-            case DL4S_MASK_DENSE_F32: rc = launch_bwd<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-            case DL4S_MASK_CAUSAL: rc = launch_bwd<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-            case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-            default: rc = launch_bwd<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+            case DL4S_MASK_NONE: rc = launch_bwd<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, no_split); break;
+            case DL4S_MASK_DENSE_F32: rc = launch_bwd<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, no_split); break;
+            case DL4S_MASK_CAUSAL: rc = launch_bwd<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, no_split); break;
+            case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, no_split); break;
+            default: rc = launch_bwd<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, no_split); break;
         }
     }
     const int rc2 = dl4s_hip_free(ctx, Dv);   // stream-ordered: later users of the block queue behind these kernels

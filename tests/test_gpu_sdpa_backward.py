@@ -20,6 +20,17 @@ def rand(rng, *shape, scale=1.0):
     return (rng.standard_normal(shape) * scale).astype(np.float32)
 
 
+# Small launches run the split kernels unless DL4S_SDPA_NO_KEY_SPLIT is set; the module's tests run once per variant.
+NO_SPLIT_DEFAULT = [False]
+
+
+@pytest.fixture(autouse=True, params=["split_auto", "no_split"])
+def kernel_variant(request):
+    NO_SPLIT_DEFAULT[0] = request.param == "no_split"
+    yield
+    NO_SPLIT_DEFAULT[0] = False
+
+
 def run_fwd_bwd(ctx, q, k, v, dout, mask=None, kind=None, lens=None, strict=False, token_major=False):
     """Returns (out, stats, dq, dk, dv) in [B,H,L,d] order whatever layout the kernels were given."""
     from dl4s_amd import lib
@@ -40,7 +51,7 @@ def run_fwd_bwd(ctx, q, k, v, dout, mask=None, kind=None, lens=None, strict=Fals
         desc = ctx.mask_desc(kind, lengths=extra[0])
     elif kind == lib.MASK_CAUSAL:
         desc = ctx.mask_desc(lib.MASK_CAUSAL)
-    flags = (lib.SDPA_STRICT if strict else 0) | (lib.SDPA_TOKEN_MAJOR if token_major else 0)
+    flags = (lib.SDPA_STRICT if strict else 0) | (lib.SDPA_TOKEN_MAJOR if token_major else 0) | (lib.SDPA_NO_KEY_SPLIT if NO_SPLIT_DEFAULT[0] else 0)
     rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))   # 0.125 for d = 64
     ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], out, stats, B, H, Lq, Lk, d, rT, desc, flags)
     ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], out, stats, bufs[3], dq_, dk_, dv_, B, H, Lq, Lk, d, rT, desc, flags)
@@ -109,7 +120,7 @@ def test_forward_with_stats_is_the_plain_forward_and_stats_give_log_sum_exp(ctx)
     q, k, v = rand(rng, B, H, L, 64), rand(rng, B, H, L, 64), rand(rng, B, H, L, 64)
     out, stats, *_ = run_fwd_bwd(ctx, q, k, v, np.zeros_like(q), kind=lib.MASK_CAUSAL)
     dq_, dk_, dv_, o2 = ctx.to_device(q), ctx.to_device(k), ctx.to_device(v), ctx.empty(q.shape)
-    ctx.sdpa_fwd(dq_, dk_, dv_, o2, B, H, L, L, 64, 64, 0.125, ctx.mask_desc(lib.MASK_CAUSAL), 0)
+    ctx.sdpa_fwd(dq_, dk_, dv_, o2, B, H, L, L, 64, 64, 0.125, ctx.mask_desc(lib.MASK_CAUSAL), lib.SDPA_NO_KEY_SPLIT if NO_SPLIT_DEFAULT[0] else 0)
     assert np.array_equal(out, o2.numpy())
     s = np.matmul(q.astype(np.float64), k.astype(np.float64).transpose(0, 1, 3, 2)) / 8.0 - causal_mask(L, L) * 1e9
     lse2 = scipy.special.logsumexp(s, axis=-1) / np.log(2.0)
