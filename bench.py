@@ -375,7 +375,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--cpu-pairs", type=int, default=24, help="(batch, head) slices timed on the CPU oracle; 0 disables")
+    ap.add_argument("--cpu-pairs", type=int, default=64, help="(batch, head) slices timed on the CPU oracle; 0 disables")
     ap.add_argument("--decode-repeats", type=int, default=5)
     ap.add_argument("--no-other-configs", dest="other_configs", action="store_false",
                     help="skip configs 1-3 (SDPA, MHA layer, encoder block) that are reported beside the headline")
