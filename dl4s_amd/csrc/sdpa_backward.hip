@@ -1,4 +1,4 @@
-// Gradients of the fused attention for gfx950 (head dim 64): given dout = d(loss)/d(out) of
+// Gradients of the fused attention for gfx950 (64-wide tiles: head dims up to 64, padded with zero columns): given dout = d(loss)/d(out) of
 //   out = softmax((q * rT) . k^T - mask * 1e9) . v
 // compute dq, dk, dv.  With p = the softmax weights and D_i = sum_d dout[i][d] * out[i][d] (= sum_j dp_ij p_ij):
 //   dv = p^T . dout,   dp = dout . v^T,   ds = p * (dp - D),   dq = (ds . k) * rT,   dk = ds^T . (q * rT)
@@ -14,7 +14,9 @@
 //                          (S^T, dP^T in the accumulator layout lane = query; dQ^T += K^T . dS^T)
 //   sdpa_bwd_dkv_f32_d64   a wavefront owns 32 keys and walks the queries (S, dP with lane = key;
 //                          dV^T += dO^T . P, dK^T += Q^T . dS)
-// All five products of each run on v_mfma_f32_32x32x2_f32 with the operand layouts of the forward kernel.
+// All five products of each run on v_mfma_f32_32x32x2_f32 with the operand layouts of the forward kernel.  Small launches
+// run the _split_ forms of the two (one 32-row block per workgroup, its tiles split over the four wavefronts); head dims
+// the MFMA kernels do not take run the plain kernels at the end of the file.
 #include "sdpa_common.h"
 
 namespace {

@@ -1,5 +1,5 @@
-// Shared by the attention forward and backward kernels for gfx950 (head dim 64): tile constants, the mask
-// descriptor as the kernels see it, the dense-mask tile classifier and the masked score tile.
+// Shared by the attention forward and backward kernels for gfx950: tile constants of the 64-wide kernels, the mask
+// descriptor as the kernels see it, the dense-mask tile classifier, the masked score tile and the plain-kernel helpers.
 #pragma once
 #include "common.h"
 #include "work_order.h"

@@ -1,6 +1,6 @@
 // Fused attention forward for gfx950: out = softmax((q * rT) . k^T - mask * 1e9) . v
 //
-// sdpa_prefill_f32_d64 is the hot kernel (head dim 64).  One workgroup = 4 wavefronts = 128
+// sdpa_prefill_f32_d64 is the hot kernel (head dim 64; smaller head dims padded with zero columns).  One workgroup = 4 wavefronts = 128
 // queries of one (batch, head); each wavefront owns 32 queries and walks the keys in LDS tiles of
 // 32.  Both contractions run on v_mfma_f32_32x32x2_f32 and are set up TRANSPOSED so that the
 // probabilities never leave the registers they were computed in:
