@@ -8,6 +8,7 @@
 //                      chosen so that the unit-stride direction runs along the lanes
 //   gemm_f32_mfma_fast every transpose combination of aligned operands with extents that are multiples of 4 (the layers'
 //                      products and their gradients): 128-bit buffer loads, see below
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
@@ -533,7 +534,10 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
         // column block pulls a long K through one CU: M16 N512 K2048 8.9 us against 15.3 us unsliced, K4096 8.9 against
         // 26.9.  The slicing depends on K alone, so a product gets the same summation order alone, batched and grouped.
         const int unit = 8 * SKW;
-        const long long S = K <= 1024 ? 1 : (K + 511) / 512;
+        // (not more slices than it takes to give every CU two workgroups: with many column blocks the launch is wide
+        // enough already, and a workgroup that lives for a single batch of loads spends its time starting and finishing)
+        const long long want = (2ll * ctx->cu_count + (long long)nbn * nbm - 1) / ((long long)nbn * nbm);
+        const long long S = K <= 1024 ? 1 : std::max(1ll, std::min((long long)((K + 511) / 512), want));
         const int kslice = (int)((((K + S - 1) / S) + unit - 1) / unit * unit);
         const dim3 pgrid((unsigned)(nbn * nbm), (unsigned)S, (unsigned)batch);
         if (S == 1) {
