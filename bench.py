@@ -115,156 +115,167 @@ def decode(ctx, lib, repeats):
             "shape": {"B": B, "H": H, "d": d, "T0": T0, "steps": steps}}
 
 
-def other_configs(ctx, lib, cpu):
+def other_configs(ctx, lib, cpu, only=None):
     """Configs 1-3 of the baseline: us/call, TFLOP/s on the algorithmic flops, fraction of the fp32 MFMA peak; the
     CPU oracle beside each (whole call for configs 1 and 2, one batch item of config 3), single thread."""
     from dl4s_amd import host_lib
     from oracle import fp64_model as m64
+    if cpu:
+        from oracle import binding as orc
     res = {}
-    # config 1: SDPA B1 H8 L128 d64, no mask
-    rng = np.random.Generator(np.random.PCG64(1001))
-    q, k, v = (rng.standard_normal((1, 8, 128, 64), dtype=np.float32) for _ in range(3))
-    dq, dk, dv, out = ctx.to_device(q), ctx.to_device(k), ctx.to_device(v), ctx.empty((1, 8, 128, 64))
-    for _ in range(5):
-        ctx.sdpa_fwd(dq, dk, dv, out, 1, 8, 128, 128, 64, 64, 0.125, None, 0)
-    ctx.sync()
-    ctx.timer_begin()
-    for _ in range(200):
-        ctx.sdpa_fwd(dq, dk, dv, out, 1, 8, 128, 128, 64, 64, 0.125, None, 0)
-    us = ctx.timer_end() * 1e3 / 200
-    fl = 4.0 * 64 * 8 * 128 * 128
-    res["config1_sdpa_B1_H8_L128_d64"] = {"us_per_call": us, "tflops": fl / us / 1e6, "frac_mfma_peak": fl / us / 1e6 / MFMA_FP32_PEAK_TFLOPS,
-                                          "flops": fl, "note": "launch-latency bound (33.6 MFLOP)"}
-    for b in (dq, dk, dv, out):
-        b.release()
-    if cpu:
-        from oracle import binding as orc
-        t0 = time.perf_counter()
-        orc.sdpa(q, k, v, None)
-        dt = time.perf_counter() - t0
-        res["config1_sdpa_B1_H8_L128_d64"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
-    # config 2: MHA layer B4 L512 D512 H8 causal (dense mask tensor, as the layer receives it)
-    B, L, D, H, dk_ = 4, 512, 512, 8, 64
-    rng = np.random.Generator(np.random.PCG64(1002))
-    x = rng.standard_normal((B, L, D), dtype=np.float32)
-    attn, _ = m64.make_params(rng, D, H, dk_, dk_, 8, trivial_affine=True)
-    i, j = np.indices((L, L))
-    mask = (j > i).astype(np.float32)
-    fl = 4.0 * 64 * B * H * (L * (L + 1) // 2) + 4 * 2.0 * B * L * D * D
-    # fused: tiles the mask blocks entirely are skipped; fused_strict: every tile visited (NaN / Inf at blocked keys as in
-    # the reference); primitive: the reference's engine calls one by one
-    for mode, fused in (("fused", 1), ("fused_strict", 2), ("primitive", 0)):
-        host_lib.mha(ctx, x, x, x, mask, attn, H, dk_, dk_, fused=fused, iters=1500 if fused else 60)   # ~0.2 s: clocks up
-        _, ms = host_lib.mha(ctx, x, x, x, mask, attn, H, dk_, dk_, fused=fused, iters=100 if fused else 20)
-        res["config2_mha_B4_L512_D512_H8_causal_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
-                                                            "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
-    if cpu:
-        t0 = time.perf_counter()
-        orc.mha(x, x, x, mask, attn, H, dk_, dk_)
-        dt = time.perf_counter() - t0
-        res["config2_mha_B4_L512_D512_H8_causal_fused"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
-    # config 3: encoder block B8 L1024 D1024 H16 F4096, key-length mask
-    B, L, D, H, F = 8, 1024, 1024, 16, 4096
-    rng = np.random.Generator(np.random.PCG64(1003))
-    x = rng.standard_normal((B, L, D), dtype=np.float32)
-    attn, ffn = m64.make_params(rng, D, H, 64, 64, F, trivial_affine=True)
-    lens = rng.integers(512, 1025, size=B)
-    mask = (np.arange(L)[None, None, None, :] >= lens[:, None, None, None]).astype(np.float32)
-    fl = 4.0 * 64 * H * L * float(lens.sum()) + 4 * 2.0 * B * L * D * D + 2 * 2.0 * B * L * D * F
-    for mode, fused in (("fused", 1), ("fused_strict", 2)):
-        host_lib.encoder_block(ctx, x, mask, attn, ffn, H, 64, 64, fused=fused, iters=100)                   # ~0.2 s: clocks up
-        _, ms = host_lib.encoder_block(ctx, x, mask, attn, ffn, H, 64, 64, fused=fused, iters=20)
-        res["config3_encoder_block_B8_L1024_D1024_H16_F4096_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
-                                                                         "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
-    if cpu:
-        t0 = time.perf_counter()
-        orc.encoder_block(x[:1, :256], mask[:1, :, :, :256], attn, ffn, H, 64, 64)
-        dt = time.perf_counter() - t0
-        fl1 = 4.0 * 64 * H * 256 * min(int(lens[0]), 256) + 4 * 2.0 * 256 * D * D + 2 * 2.0 * 256 * D * F
-        res["config3_encoder_block_B8_L1024_D1024_H16_F4096_fused"]["cpu_baseline"] = {
-            "tflops": fl1 / dt / 1e12, "cores": 1, "kind": "port",
-            "sample": "one batch item cut to 256 tokens (%.1f s); extrapolated whole call %.0f s" % (dt, dt * fl / fl1)}
-    # gradients of the headline workload (config 4 shapes): forward with row statistics, then dq, dk, dv
-    B, H, L = 8, 16, 2048
-    rng = np.random.Generator(np.random.PCG64(1004))
-    bufs = [ctx.to_device(rng.standard_normal((B, H, L, 64), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
-    outs = [ctx.empty((B, H, L, 64)) for _ in range(4)]
-    st = ctx.empty((B, H, L, 2))
-    desc = ctx.mask_desc(lib.MASK_CAUSAL)
-    ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], outs[0], st, B, H, L, L, 64, 0.125, desc, 0)
-    bwd = lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, 64, 0.125, desc, 0)
-    for _ in range(20):
-        bwd()
-    ctx.sync()
-    ctx.timer_begin()
-    for _ in range(20):
-        bwd()
-    ms = ctx.timer_end() / 20
-    fl = 10.0 * 64 * B * H * (L * (L + 1) // 2)          # five products: dv, dp, dq, dk and the recomputed scores
-    res["config4_attention_backward_B8_H16_L2048_causal"] = {
-        "us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
-        "note": "algorithmic flops = 5 products; the two deterministic kernels issue 7 (scores and dp are formed in both)"}
-    if cpu:
-        from oracle import binding as orc
-        hq, hk, hv, hg = (b_.numpy()[:1, :2] for b_ in bufs)
+    want = lambda name: only is None or name in only
+    if want("config1"):
+        # config 1: SDPA B1 H8 L128 d64, no mask
+        rng = np.random.Generator(np.random.PCG64(1001))
+        q, k, v = (rng.standard_normal((1, 8, 128, 64), dtype=np.float32) for _ in range(3))
+        dq, dk, dv, out = ctx.to_device(q), ctx.to_device(k), ctx.to_device(v), ctx.empty((1, 8, 128, 64))
+        for _ in range(5):
+            ctx.sdpa_fwd(dq, dk, dv, out, 1, 8, 128, 128, 64, 64, 0.125, None, 0)
+        ctx.sync()
+        ctx.timer_begin()
+        for _ in range(200):
+            ctx.sdpa_fwd(dq, dk, dv, out, 1, 8, 128, 128, 64, 64, 0.125, None, 0)
+        us = ctx.timer_end() * 1e3 / 200
+        fl = 4.0 * 64 * 8 * 128 * 128
+        res["config1_sdpa_B1_H8_L128_d64"] = {"us_per_call": us, "tflops": fl / us / 1e6, "frac_mfma_peak": fl / us / 1e6 / MFMA_FP32_PEAK_TFLOPS,
+                                              "flops": fl, "note": "launch-latency bound (33.6 MFLOP)"}
+        for b in (dq, dk, dv, out):
+            b.release()
+        if cpu:
+            from oracle import binding as orc
+            t0 = time.perf_counter()
+            orc.sdpa(q, k, v, None)
+            dt = time.perf_counter() - t0
+            res["config1_sdpa_B1_H8_L128_d64"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
+    if want("config2"):
+        # config 2: MHA layer B4 L512 D512 H8 causal (dense mask tensor, as the layer receives it)
+        B, L, D, H, dk_ = 4, 512, 512, 8, 64
+        rng = np.random.Generator(np.random.PCG64(1002))
+        x = rng.standard_normal((B, L, D), dtype=np.float32)
+        attn, _ = m64.make_params(rng, D, H, dk_, dk_, 8, trivial_affine=True)
         i, j = np.indices((L, L))
-        t0 = time.perf_counter()
-        orc.sdpa_backward(hq, hk, hv, (j > i).astype(np.float32), hg)
-        dt = time.perf_counter() - t0
-        res["config4_attention_backward_B8_H16_L2048_causal"]["cpu_baseline"] = {
-            "tflops": fl * 2 / (B * H) / dt / 1e12, "cores": 1, "kind": "port",
-            "sample": "2 of 128 (batch, head) slices, dense causal mask (%.1f s)" % dt}
-    for b_ in bufs + outs + [st]:
-        b_.release()
-    # the headline shape with the mask as an unmodified DL4S passes it (a dense [L,L] tensor): all-ones tiles skipped
-    # (default) and every tile visited (DL4S_SDPA_STRICT); and the same shape with head dim 128 (causal descriptor)
-    B, H, L = 8, 16, 2048
-    rng = np.random.Generator(np.random.PCG64(1008))
-    i, j = np.indices((L, L))
-    dmask = ctx.to_device((j > i).astype(np.float32))
-    for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal")):
-        qkv = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(3)]
-        o = ctx.empty((B, H, L, d))
-        rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
-        fl = 4.0 * d * B * H * (L * (L + 1) // 2)
-        entry = {"flops": fl}
-        variants = (("tile_skipping", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), 0), ("strict", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), lib.SDPA_STRICT)) \
-            if d == 64 else (("causal_descriptor", ctx.mask_desc(lib.MASK_CAUSAL), 0),)
-        for vname, desc, flags in variants:
-            for _ in range(100):
-                ctx.sdpa_fwd(qkv[0], qkv[1], qkv[2], o, B, H, L, L, d, d, rT, desc, flags)
-            ctx.sync()
-            ctx.timer_begin()
-            for _ in range(30):
-                ctx.sdpa_fwd(qkv[0], qkv[1], qkv[2], o, B, H, L, L, d, d, rT, desc, flags)
-            ms = ctx.timer_end() / 30
-            entry[vname] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS}
-        res[name] = entry
-        for b_ in qkv + [o]:
+        mask = (j > i).astype(np.float32)
+        fl = 4.0 * 64 * B * H * (L * (L + 1) // 2) + 4 * 2.0 * B * L * D * D
+        # fused: tiles the mask blocks entirely are skipped; fused_strict: every tile visited (NaN / Inf at blocked keys as in
+        # the reference); primitive: the reference's engine calls one by one
+        for mode, fused in (("fused", 1), ("fused_strict", 2), ("primitive", 0)):
+            host_lib.mha(ctx, x, x, x, mask, attn, H, dk_, dk_, fused=fused, iters=1500 if fused else 60)   # ~0.2 s: clocks up
+            _, ms = host_lib.mha(ctx, x, x, x, mask, attn, H, dk_, dk_, fused=fused, iters=100 if fused else 20)
+            res["config2_mha_B4_L512_D512_H8_causal_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
+                                                                "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
+        if cpu:
+            t0 = time.perf_counter()
+            orc.mha(x, x, x, mask, attn, H, dk_, dk_)
+            dt = time.perf_counter() - t0
+            res["config2_mha_B4_L512_D512_H8_causal_fused"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
+    if want("config3"):
+        # config 3: encoder block B8 L1024 D1024 H16 F4096, key-length mask
+        B, L, D, H, F = 8, 1024, 1024, 16, 4096
+        rng = np.random.Generator(np.random.PCG64(1003))
+        x = rng.standard_normal((B, L, D), dtype=np.float32)
+        attn, ffn = m64.make_params(rng, D, H, 64, 64, F, trivial_affine=True)
+        lens = rng.integers(512, 1025, size=B)
+        mask = (np.arange(L)[None, None, None, :] >= lens[:, None, None, None]).astype(np.float32)
+        fl = 4.0 * 64 * H * L * float(lens.sum()) + 4 * 2.0 * B * L * D * D + 2 * 2.0 * B * L * D * F
+        for mode, fused in (("fused", 1), ("fused_strict", 2)):
+            host_lib.encoder_block(ctx, x, mask, attn, ffn, H, 64, 64, fused=fused, iters=100)                   # ~0.2 s: clocks up
+            _, ms = host_lib.encoder_block(ctx, x, mask, attn, ffn, H, 64, 64, fused=fused, iters=20)
+            res["config3_encoder_block_B8_L1024_D1024_H16_F4096_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
+                                                                             "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
+        if cpu:
+            t0 = time.perf_counter()
+            orc.encoder_block(x[:1, :256], mask[:1, :, :, :256], attn, ffn, H, 64, 64)
+            dt = time.perf_counter() - t0
+            fl1 = 4.0 * 64 * H * 256 * min(int(lens[0]), 256) + 4 * 2.0 * 256 * D * D + 2 * 2.0 * 256 * D * F
+            res["config3_encoder_block_B8_L1024_D1024_H16_F4096_fused"]["cpu_baseline"] = {
+                "tflops": fl1 / dt / 1e12, "cores": 1, "kind": "port",
+                "sample": "one batch item cut to 256 tokens (%.1f s); extrapolated whole call %.0f s" % (dt, dt * fl / fl1)}
+    if want("backward"):
+        # gradients of the headline workload (config 4 shapes): forward with row statistics, then dq, dk, dv
+        B, H, L = 8, 16, 2048
+        rng = np.random.Generator(np.random.PCG64(1004))
+        bufs = [ctx.to_device(rng.standard_normal((B, H, L, 64), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
+        outs = [ctx.empty((B, H, L, 64)) for _ in range(4)]
+        st = ctx.empty((B, H, L, 2))
+        desc = ctx.mask_desc(lib.MASK_CAUSAL)
+        ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], outs[0], st, B, H, L, L, 64, 0.125, desc, 0)
+        bwd = lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, 64, 0.125, desc, 0)
+        for _ in range(20):
+            bwd()
+        ctx.sync()
+        ctx.timer_begin()
+        for _ in range(20):
+            bwd()
+        ms = ctx.timer_end() / 20
+        fl = 10.0 * 64 * B * H * (L * (L + 1) // 2)          # five products: dv, dp, dq, dk and the recomputed scores
+        res["config4_attention_backward_B8_H16_L2048_causal"] = {
+            "us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
+            "note": "algorithmic flops = 5 products; the two deterministic kernels issue 7 (scores and dp are formed in both)"}
+        if cpu:
+            from oracle import binding as orc
+            hq, hk, hv, hg = (b_.numpy()[:1, :2] for b_ in bufs)
+            i, j = np.indices((L, L))
+            t0 = time.perf_counter()
+            orc.sdpa_backward(hq, hk, hv, (j > i).astype(np.float32), hg)
+            dt = time.perf_counter() - t0
+            res["config4_attention_backward_B8_H16_L2048_causal"]["cpu_baseline"] = {
+                "tflops": fl * 2 / (B * H) / dt / 1e12, "cores": 1, "kind": "port",
+                "sample": "2 of 128 (batch, head) slices, dense causal mask (%.1f s)" % dt}
+        for b_ in bufs + outs + [st]:
             b_.release()
-    dmask.release()
-    # the caller of the blocks: Transformer greedy decoding (batch 1; every step re-runs the decoder on the prefix, as the
-    # reference does).  6 + 6 layers, hidden 512, 8 heads of 64, ffn 2048, vocabulary 8000, 64 source tokens, 32 generated.
-    rng = np.random.Generator(np.random.PCG64(1006))
-    params = m64.make_transformer_params(rng, 8000, 512, 8, 64, 64, 2048, 6, 6)
-    src = [int(t) for t in rng.integers(0, 8000, 64)]
-    model = host_lib.Transformer(ctx, params)
-    entry = {"workload": "Transformer greedy decode, 6+6 layers, hidden 512, 8 heads x 64, ffn 2048, vocab 8000, 64 source tokens, "
-                         "32 generated tokens (prefix re-run every step)"}
-    for mode, fused in (("fused", True), ("primitive", False)):
-        model.greedy(src, 1, -5, 4, fused=fused)                       # warm the allocator pool
-        toks, ms = model.greedy(src, 1, -5, 32, fused=fused, timing=True)
-        entry["ms_per_token_" + mode] = ms / len(toks)
-        entry["tokens_per_s_" + mode] = len(toks) / ms * 1e3
-    model.close()
-    if cpu:
-        from oracle import transformer as orc_t
-        t0 = time.perf_counter()
-        n_cpu = len(orc_t.greedy_decode(params, src, 1, -5, 4))
-        dt = time.perf_counter() - t0
-        entry["cpu_baseline"] = {"ms_per_token": dt * 1e3 / n_cpu, "cores": 1, "kind": "port",
-                                 "sample": "encoder pass + the first %d generated tokens (%.1f s)" % (n_cpu, dt)}
-    res["transformer_greedy_decode"] = entry
+    if want("masks_and_head_dim"):
+        # the headline shape with the mask as an unmodified DL4S passes it (a dense [L,L] tensor): all-ones tiles skipped
+        # (default) and every tile visited (DL4S_SDPA_STRICT); and the same shape with head dim 128 (causal descriptor)
+        B, H, L = 8, 16, 2048
+        rng = np.random.Generator(np.random.PCG64(1008))
+        i, j = np.indices((L, L))
+        dmask = ctx.to_device((j > i).astype(np.float32))
+        for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal")):
+            qkv = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(3)]
+            o = ctx.empty((B, H, L, d))
+            rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+            fl = 4.0 * d * B * H * (L * (L + 1) // 2)
+            entry = {"flops": fl}
+            variants = (("tile_skipping", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), 0), ("strict", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), lib.SDPA_STRICT)) \
+                if d == 64 else (("causal_descriptor", ctx.mask_desc(lib.MASK_CAUSAL), 0),)
+            for vname, desc, flags in variants:
+                for _ in range(100):
+                    ctx.sdpa_fwd(qkv[0], qkv[1], qkv[2], o, B, H, L, L, d, d, rT, desc, flags)
+                ctx.sync()
+                ctx.timer_begin()
+                for _ in range(30):
+                    ctx.sdpa_fwd(qkv[0], qkv[1], qkv[2], o, B, H, L, L, d, d, rT, desc, flags)
+                ms = ctx.timer_end() / 30
+                entry[vname] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS}
+            res[name] = entry
+            for b_ in qkv + [o]:
+                b_.release()
+        dmask.release()
+    if want("greedy") or want("greedy_fused") or want("greedy_primitive"):
+        # the caller of the blocks: Transformer greedy decoding (batch 1; every step re-runs the decoder on the prefix, as the
+        # reference does).  6 + 6 layers, hidden 512, 8 heads of 64, ffn 2048, vocabulary 8000, 64 source tokens, 32 generated.
+        rng = np.random.Generator(np.random.PCG64(1006))
+        params = m64.make_transformer_params(rng, 8000, 512, 8, 64, 64, 2048, 6, 6)
+        src = [int(t) for t in rng.integers(0, 8000, 64)]
+        model = host_lib.Transformer(ctx, params)
+        entry = {"workload": "Transformer greedy decode, 6+6 layers, hidden 512, 8 heads x 64, ffn 2048, vocab 8000, 64 source tokens, "
+                             "32 generated tokens (prefix re-run every step)"}
+        for mode, fused in (("fused", True), ("primitive", False)):
+            if not (want("greedy") or want("greedy_" + mode)):
+                continue
+            model.greedy(src, 1, -5, 4, fused=fused)                       # warm the allocator pool
+            toks, ms = model.greedy(src, 1, -5, 32, fused=fused, timing=True)
+            entry["ms_per_token_" + mode] = ms / len(toks)
+            entry["tokens_per_s_" + mode] = len(toks) / ms * 1e3
+        model.close()
+        if cpu:
+            from oracle import transformer as orc_t
+            t0 = time.perf_counter()
+            n_cpu = len(orc_t.greedy_decode(params, src, 1, -5, 4))
+            dt = time.perf_counter() - t0
+            entry["cpu_baseline"] = {"ms_per_token": dt * 1e3 / n_cpu, "cores": 1, "kind": "port",
+                                     "sample": "encoder pass + the first %d generated tokens (%.1f s)" % (n_cpu, dt)}
+        res["transformer_greedy_decode"] = entry
     return res
 
 
@@ -386,6 +397,10 @@ def main():
                     help="instead of the benchmark, launch the kernels behind configs 3 and 4 (fused Dense products, dense-mask "
                          "attention, attention gradients) N times each and print their mean event times: a short command for "
                          "profiler counter runs")
+    ap.add_argument("--only", default="", metavar="NAMES",
+                    help="instead of the benchmark, run only these of the workloads reported beside the headline (comma "
+                         "separated: config1, config2, config3, backward, masks_and_head_dim, greedy, greedy_fused, greedy_primitive) and print their entries: "
+                         "short commands for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (every attention problem fits one MI355X); --gpus %d is not "
@@ -397,6 +412,10 @@ def main():
     info = ctx.device_info()
     if args.kernel_sample > 0:
         print(json.dumps({"kernel_sample": kernel_sample(ctx, lib, args.kernel_sample)}))
+        ctx.close()
+        return
+    if args.only:
+        print(json.dumps({"only": other_configs(ctx, lib, args.cpu_pairs > 0, set(args.only.split(",")))}))
         ctx.close()
         return
     pre = prefill(ctx, lib, args.steps, args.warmup)
