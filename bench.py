@@ -65,7 +65,7 @@ def prefill(ctx, lib, steps, warmup):
     for b in (dq, dk, dv, out):
         b.release()
     return {"flops": flops, "wall_s": wall, "event_ms_per_launch": ev_ms / steps,
-            "shape": {"B": B, "H": H, "L": L, "d": d}, "inputs": (q, k, v)}
+            "shape": {"B": B, "H": H, "L": L, "d": d}, "inputs": (q, k, v), "output": o}
 
 
 def decode(ctx, lib, repeats):
@@ -294,19 +294,31 @@ def cpu_baseline_decode(steps_sample=1):
     return {"us_per_step": dt * 1e6, "tokens_per_s": B / dt, "cores": 1, "kind": "port", "sample": "%d whole step(s) at T=4097" % steps_sample}
 
 
-def cpu_baseline_prefill(q, k, v, pairs):
+def cpu_baseline_prefill(q, k, v, pairs, gpu_out=None):
+    """The CPU oracle timed on `pairs` (batch, head) slices of the headline workload, single thread; its results also
+    check the GPU output of the same slices (raw maxima of the absolute and the relative difference)."""
     from oracle import binding as orc
     L, d = q.shape[2], q.shape[3]
     i, j = np.indices((L, L))
     mask = (j > i).astype(np.float32)
     orc.lib()
-    t0 = time.perf_counter()
+    dt, max_abs, max_ref = 0.0, 0.0, 0.0
     for p in range(pairs):
         b, h = divmod(p, q.shape[1])
-        orc.sdpa(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mask)
-    dt = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        ref = orc.sdpa(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mask)
+        dt += time.perf_counter() - t0
+        if gpu_out is not None:
+            diff = np.abs(gpu_out[b:b + 1, h:h + 1].astype(np.float64) - ref.astype(np.float64))
+            if not (diff <= 1e-4 + 1e-4 * np.abs(ref)).all():
+                raise RuntimeError("prefill output differs from the CPU oracle on slice (%d, %d): max |d| = %g" % (b, h, diff.max()))
+            max_abs = max(max_abs, float(diff.max()))
+            max_ref = max(max_ref, float(np.abs(ref).max()))
     flops = 4.0 * d * pairs * (L * (L + 1) // 2)
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+    parity = {} if gpu_out is None else {"parity": {"gate": "|gpu - oracle| <= 1e-4 + 1e-4 |oracle| on every element of the sample",
+                                                    "max_abs_diff": max_abs, "max_abs_oracle": max_ref,
+                                                    "max_abs_diff_over_max_abs_oracle": max_abs / max(max_ref, 1e-30)}}
+    return {**parity, "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
             "sample": "%d of %d (batch, head) slices of the headline workload (L=%d, d=%d, dense causal mask), "
                       "%.1f s of single-thread CPU time; host has %d cores" % (pairs, q.shape[0] * q.shape[1], L, d, dt,
                                                                              os.cpu_count() or 0)}
@@ -463,7 +475,7 @@ def main():
                                        "kernel": "sdpa_decode_splitk_f32", "bytes_per_step": dec["bytes_per_step"]}}
     if args.cpu_pairs > 0:
         q, k, v = pre["inputs"]
-        line["cpu_baseline"] = cpu_baseline_prefill(q, k, v, args.cpu_pairs)
+        line["cpu_baseline"] = cpu_baseline_prefill(q, k, v, args.cpu_pairs, pre["output"])
         line["cpu_blas_proxy"] = cpu_blas_proxy_prefill(q, k, v, min(32, q.shape[0] * q.shape[1]))
         if dec:
             line["decode"]["cpu_baseline"] = cpu_baseline_decode()
