@@ -170,6 +170,7 @@ __global__ void band_f32(const float *__restrict__ x, float *__restrict__ y, lon
 }
 
 // ---- LayerNorm over rows*D elements per batch item (NN/Layer/LayerNorm.swift:62-77)
+template <int NT = TPB>
 __device__ __forceinline__ void block_sum2(float &a, float &b, float *sm) {
     for (int s = 32; s > 0; s >>= 1) { a += __shfl_xor(a, s, 64); b += __shfl_xor(b, s, 64); }
     const int w = threadIdx.x >> 6;
@@ -177,7 +178,7 @@ __device__ __forceinline__ void block_sum2(float &a, float &b, float *sm) {
     if ((threadIdx.x & 63) == 0) { sm[2 * w] = a; sm[2 * w + 1] = b; }
     __syncthreads();
     a = 0.f; b = 0.f;
-    for (int i = 0; i < TPB / 64; ++i) { a += sm[2 * i]; b += sm[2 * i + 1]; }
+    for (int i = 0; i < NT / 64; ++i) { a += sm[2 * i]; b += sm[2 * i + 1]; }
 }
 
 // LayerNorm kernels.  VEC: rows, D and the pointers allow 128-bit accesses (n % 4 == 0, D % 4 == 0, 16-byte alignment);
@@ -270,32 +271,32 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     }
 }
 
-// one workgroup per batch item, for short rows (per-token LayerNorm of the feed-forward block)
-template <bool VEC>
-__global__ __launch_bounds__(TPB) void ln_small_f32(const float *__restrict__ x, const float *__restrict__ res,
+// one workgroup (of NT threads: 256, or 1024 when a row is longer than 4096) per batch item, for short rows (per-token LayerNorm of the feed-forward block)
+template <bool VEC, int NT>
+__global__ __launch_bounds__(NT) void ln_small_f32(const float *__restrict__ x, const float *__restrict__ res,
                                                      const float *__restrict__ scale, const float *__restrict__ shift,
                                                      float *__restrict__ y, long long n, long long D) {
-    __shared__ float sm[2 * TPB / 64];
+    __shared__ float sm[2 * NT / 64];
     const long long b = blockIdx.x;
     const float *xp = x + b * n;
     const float *rp = res ? res + b * n : nullptr;
     float *yp = y + b * n;
     float s = 0.f, ss = 0.f;
     if (VEC) {
-        const bool one = n <= (long long)TPB * 4;      // the whole row in one 128-bit access per thread: keep it in registers
+        const bool one = n <= (long long)NT * 4;      // the whole row in one 128-bit access per thread: keep it in registers
         f32x4 keep = {0.f, 0.f, 0.f, 0.f};
-        for (long long i = (long long)threadIdx.x * 4; i < n; i += (long long)TPB * 4) {
+        for (long long i = (long long)threadIdx.x * 4; i < n; i += (long long)NT * 4) {
             const f32x4 v = ln_load4(xp, rp, i);
             if (one) keep = v;
             s += (v.x + v.y) + (v.z + v.w);
             ss += (__fmul_rn(v.x, v.x) + __fmul_rn(v.y, v.y)) + (__fmul_rn(v.z, v.z) + __fmul_rn(v.w, v.w));
         }
-        block_sum2(s, ss, sm);
+        block_sum2<NT>(s, ss, sm);
         const float rN = __fdiv_rn(1.0f, (float)n);
         const float mean = __fmul_rn(s, rN);
         const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
         const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
-        const long long step = (long long)TPB * 4, dstep = step % D;
+        const long long step = (long long)NT * 4, dstep = step % D;
         long long i = (long long)threadIdx.x * 4, d = i % D;
         for (; i < n; i += step) {
             *reinterpret_cast<f32x4 *>(yp + i) = ln_norm4(one ? keep : ln_load4(xp, rp, i), mean, rden, scale, shift, d);
@@ -303,18 +304,18 @@ __global__ __launch_bounds__(TPB) void ln_small_f32(const float *__restrict__ x,
             if (d >= D) d -= D;
         }
     } else {
-        for (long long i = threadIdx.x; i < n; i += TPB) {
+        for (long long i = threadIdx.x; i < n; i += NT) {
             float v = xp[i];
             if (rp) v = __fadd_rn(v, rp[i]);
             s += v;
             ss += __fmul_rn(v, v);
         }
-        block_sum2(s, ss, sm);
+        block_sum2<NT>(s, ss, sm);
         const float rN = __fdiv_rn(1.0f, (float)n);
         const float mean = __fmul_rn(s, rN);
         const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
         const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
-        for (long long i = threadIdx.x; i < n; i += TPB) {
+        for (long long i = threadIdx.x; i < n; i += NT) {
             float v = xp[i];
             if (rp) v = __fadd_rn(v, rp[i]);
             const float nrm = __fmul_rn(__fadd_rn(v, -mean), rden);
@@ -751,8 +752,15 @@ int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *resid
     const auto a16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     const bool vec = n % 4 == 0 && D % 4 == 0 && a16(x) && a16(residual) && a16(scale) && a16(shift) && a16(result);
     if (n <= 16384) {
-        if (vec) hipLaunchKernelGGL(ln_small_f32<true>, dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
-        else hipLaunchKernelGGL(ln_small_f32<false>, dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+        // rows beyond 4096 elements (the joint (L, D) LayerNorm of a short decoded prefix): 1024 threads, so that a thread's
+        // loads are few enough to be in flight together
+        if (n > 4096) {
+            if (vec) hipLaunchKernelGGL((ln_small_f32<true, 1024>), dim3((unsigned)B), dim3(1024), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+            else hipLaunchKernelGGL((ln_small_f32<false, 1024>), dim3((unsigned)B), dim3(1024), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+        } else {
+            if (vec) hipLaunchKernelGGL((ln_small_f32<true, TPB>), dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+            else hipLaunchKernelGGL((ln_small_f32<false, TPB>), dim3((unsigned)B), dim3(TPB), 0, ctx->stream, x, residual, scale, shift, result, n, (long long)D);
+        }
         return dl4s::launch_status("layernorm");
     }
     DL4S_REQUIRE(B <= 65535, DL4S_HIP_EUNSUPPORTED, "layernorm: batch above 65535 with long rows");

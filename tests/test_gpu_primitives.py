@@ -300,7 +300,8 @@ def test_band_and_decoder_mask_recipe(ctx, orc):
 
 
 @pytest.mark.parametrize("B,rows,D", [(3, 7, 16), (5, 1, 1024), (4, 512, 512), (2, 1, 33), (3, 1, 4096), (2, 300, 68), (2, 2000, 33),
-                                       (6, 1, 12), (2, 40, 1028)])   # vector and scalar paths, short and long rows, D not dividing the stride
+                                       (6, 1, 12), (2, 40, 1028), (1, 20, 512), (2, 16, 1024), (3, 150, 33), (1, 32, 512)])
+# vector and scalar paths, short and long rows (one workgroup of 256 or of 1024 threads, or two kernels), D not dividing the stride
 def test_layernorm(ctx, orc, B, rows, D):
     x, res = rnd(B, rows, D) * 2 + np.float32(0.3), rnd(B, rows, D)
     scale, shift = rnd(D), rnd(D)
