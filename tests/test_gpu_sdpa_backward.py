@@ -301,3 +301,28 @@ def test_dense_mask_tile_skipping_is_active(ctx):
     out_s, _, dq_s, _, _ = run_fwd_bwd(ctx, q, k, v, dout, mask=mask, strict=True)
     assert np.isnan(out_s[0, 0, :, 7]).all() and not np.isnan(out_s[0, 1]).any()
     assert np.isnan(dq_s[0, 0]).all()
+
+
+@pytest.mark.parametrize("d", [8, 64])
+def test_gradient_descent_through_the_fused_gradients_converges(ctx, d):
+    """The role the gradient has in the reference's Tests/DL4STests/TransformerTests.swift:30-69 (a loss driven down by
+    gradient steps), reduced to the attention operator itself: q, k, v are fitted so that the causal attention output
+    matches a target, with dq, dk, dv from dl4s_hip_sdpa_bwd_f32 only.  A sign, scale or transposition mistake in any of
+    the three gradients stops the loss from falling."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(42 + d)
+    B, H, L = 1, 2, 48
+    q, k, v = (rand(rng, B, H, L, d, scale=0.5) for _ in range(3))
+    tq, tk, tv = (rand(rng, B, H, L, d, scale=0.5) for _ in range(3))
+    dummy = np.zeros_like(q)
+    target = run_fwd_bwd(ctx, tq, tk, tv, dummy, kind=lib.MASK_CAUSAL)[0]       # reachable by construction
+    eta, losses = 0.3, []        # loss = sum |out - target|^2 / 2, so dout = out - target
+    for step in range(300):
+        out = run_fwd_bwd(ctx, q, k, v, dummy, kind=lib.MASK_CAUSAL)[0]
+        diff = out - target
+        losses.append(float((diff.astype(np.float64) ** 2).mean()))
+        _, _, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, diff, kind=lib.MASK_CAUSAL)
+        q, k, v = q - eta * dq, k - eta * dk, v - eta * dv
+    assert np.isfinite(losses).all()
+    assert losses[-1] < 0.02 * losses[0], (losses[0], losses[-1])       # the CPU oracle's gradients give 0.01
+    assert losses[-1] < losses[100] < 0.1 * losses[0]
