@@ -16,8 +16,10 @@
 //                          dV^T += dO^T . P, dK^T += Q^T . dS)
 // All five products of each run on v_mfma_f32_32x32x2_f32 with the operand layouts of the forward kernel.  Small launches
 // run the _split_ forms of the two (one 32-row block per workgroup, its tiles split over the four wavefronts); head dims
-// the MFMA kernels do not take run the plain kernels at the end of the file.
+// above 64 up to 128 run the 128-wide forms in sdpa_backward_d128.h; head dims the MFMA kernels do not take run the
+// plain kernels at the end of the file.
 #include "sdpa_common.h"
+#include "sdpa_backward_d128.h"
 
 namespace {
 
@@ -955,12 +957,19 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                            ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                              reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dout) | reinterpret_cast<uintptr_t>(dq) |
                              reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
+    const bool mfma128_path = d > HD && d <= HD2 && d % 4 == 0 &&
+                              ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                                reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dout) | reinterpret_cast<uintptr_t>(dq) |
+                                reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
+    DL4S_REQUIRE(!mfma128_path || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * d * 4 < (d == HD2 ? (1ll << 31) : (1ll << 30)),
+                 DL4S_HIP_EUNSUPPORTED,
+                 "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB (1 GiB for padded head dims)");
     DL4S_REQUIRE(!mfma_path || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * d * 4 < (d == HD ? (1ll << 31) : (1ll << 30)),
                  DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB (1 GiB for head dims below 64)");
     std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     MaskArgs m{};
-    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path, m);
+    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path, m);
     if (rc != DL4S_HIP_OK) return rc;
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     const int no_split = (flags & DL4S_SDPA_NO_KEY_SPLIT) ? 1 : 0;
@@ -969,9 +978,25 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     if (rc != DL4S_HIP_OK) return rc;
     float *D = static_cast<float *>(Dv);
     const long long rows = B * H * Lq;
+    if (mfma128_path) {
+        hipLaunchKernelGGL(sdpa_bwd_rowdot128, dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, ctx->stream, out, dout, D, (int)H, (int)Lq,
+                           rows, token_major, (int)d);
+        rc = dl4s::launch_status("sdpa_bwd_rowdot128");
+        if (rc == DL4S_HIP_OK) {
+            switch (m.kind) {
+                case DL4S_MASK_NONE: rc = launch_bwd128<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+                case DL4S_MASK_DENSE_F32: rc = launch_bwd128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+                case DL4S_MASK_CAUSAL: rc = launch_bwd128<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+                case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+                default: rc = launch_bwd128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+            }
+        }
+        const int rcf = dl4s_hip_free(ctx, Dv);
+        return rc != DL4S_HIP_OK ? rc : rcf;
+    }
     if (!mfma_path) {   // plain kernels
         rc = DL4S_HIP_OK;
-        if (token_major) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: the token-major layout needs a head dim that is a multiple of 4, at most 64, and 16-byte aligned tensors");
+        if (token_major) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: the token-major layout needs a head dim that is a multiple of 4, at most 128, and 16-byte aligned tensors");
         else if (rows >= (1ll << 31) || B * H * Lk >= (1ll << 31)) rc = dl4s::set_error(DL4S_HIP_EUNSUPPORTED, "sdpa backward: too many rows for the plain kernels");
         if (rc == DL4S_HIP_OK) {
             hipLaunchKernelGGL(sdpa_bwd_rowdot_plain, dim3((unsigned)rows), dim3(64), 0, ctx->stream, out, dout, D, (int)d);

@@ -1,0 +1,440 @@
+// Gradients of the fused attention for head dims above 64 and up to 128 (multiples of 4): the two deterministic kernels
+// of sdpa_backward.hip on 128-wide tiles.  Included by sdpa_backward.hip only; needs sdpa_prefill_d128.h's constants.
+//
+// The operand layouts follow the 128-wide forward kernel: a score product contracts d = 64*half + j over 64 MFMA steps;
+// a transposed accumulation (dQ^T, dK^T, dV^T) uses four accumulators whose rows interleave (accumulator c row i is
+// d = 4*i + c), fed by one 128-bit LDS read per key (query) and stored 128 bits at a time.  The row fragments of two
+// operands (2 x 64 registers) and up to eight accumulators leave room for one wavefront per SIMD only, so these kernels
+// run at a lower MFMA rate than the 64-wide ones; they are there so that training with such head dims stays on the
+// matrix cores at all (the plain kernels are some 40 times slower).
+#pragma once
+#include "sdpa_common.h"
+
+namespace {
+
+// D[b,h,i] = sum_d dout[i][d] * out[i][d] for head dims up to 128: 32 lanes per row, eight rows per workgroup
+__global__ __launch_bounds__(256) void sdpa_bwd_rowdot128(const float *__restrict__ out, const float *__restrict__ dout,
+                                                          float *__restrict__ D, int H, int Lq, long long rows, int token_major, int hd) {
+    const long long r = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int c = (threadIdx.x & 31) * 4;
+    float acc = 0.f;
+    if (r < rows && c < hd) {
+        const long long bh = r / Lq, qi = r % Lq;
+        const long long off = token_major ? (((bh / H) * Lq + qi) * H + bh % H) * hd : r * hd;
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(out + off + c);
+        const f32x4 g = *reinterpret_cast<const f32x4 *>(dout + off + c);
+        acc = a.x * g.x + a.y * g.y + a.z * g.z + a.w * g.w;
+    }
+    acc += __shfl_xor(acc, 16, 64);
+    acc += __shfl_xor(acc, 8, 64);
+    acc += __shfl_xor(acc, 4, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    acc += __shfl_xor(acc, 1, 64);
+    if (r < rows && (threadIdx.x & 31) == 0) D[r] = acc;
+}
+
+// 32 x 32 product tile over a 128-wide contraction: A rows from LDS (row lane % 32, columns 64*half + 4j), B from the
+// lane's 64 registers
+__device__ __forceinline__ f32x16 tile_product128(const float *Ab, const float (&br)[64]) {
+    f32x16 acc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Ab + 4 * j);
+        if (j == 0) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, br[0], zero, 0, 0, 0);
+        } else {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, br[4 * j + 0], acc, 0, 0, 0);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, br[4 * j + 1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, br[4 * j + 2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, br[4 * j + 3], acc, 0, 0, 0);
+    }
+    return acc;
+}
+
+// acc[c] (row i is d = 4*i + c; column = the lane's query or key) += A^T . B where A is a [32][128] LDS tile read through
+// 128-bit loads (row 8(r/4) + r%4 + 4*half, columns 4*(lane%32) ..: At already points there) and B the accumulator-layout
+// tile b
+__device__ __forceinline__ void tile_accumulate_t128(const float *At, const f32x16 &b, f32x16 (&acc)[4]) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const f32x4 a = *reinterpret_cast<const f32x4 *>(At + (8 * (r >> 2) + (r & 3)) * LSTR2);
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[r], acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[r], acc[1], 0, 0, 0);
+        acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b[r], acc[2], 0, 0, 0);
+        acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b[r], acc[3], 0, 0, 0);
+    }
+}
+
+// stores the lane's row of four interleaved transposed accumulators to p[row][0 .. hd-1], scaled
+__device__ __forceinline__ void store_row_t128(float *p, const f32x16 (&acc)[4], const float scale, const int half, const int hd) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int d0 = 4 * (8 * (r >> 2) + 4 * half + (r & 3));
+        f32x4 a;
+        a.x = acc[0][r] * scale; a.y = acc[1][r] * scale; a.z = acc[2][r] * scale; a.w = acc[3][r] * scale;
+        if (d0 < hd) *reinterpret_cast<f32x4 *>(p + d0) = a;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ dQ
+template <int KIND>
+__global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
+                                                                const float *__restrict__ v, const float *__restrict__ dout,
+                                                                const float *__restrict__ stats, const float *__restrict__ D,
+                                                                float *__restrict__ dq, int H, int Lq, int Lk, float rT,
+                                                                MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
+                                                                int token_major, int hd) {
+    extern __shared__ __align__(16) float lds[];
+    float *Ks = lds;                      // [2][BN][LSTR2]
+    float *Vs = lds + 2 * TILE2_FLOATS;   // [2][BN][LSTR2]
+    int bh, unit;
+    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int qb = nqb - 1 - unit;   // longest rows first
+    const int q0 = qb * BM + wave * 32;
+    const int qi = q0 + ln;
+    const int qic = qi < Lq ? qi : Lq - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
+
+    int kend = Lk, wkend = Lk;
+    bool skip_ones = false;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
+        if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
+        if (DENSE && mask.cls) {
+            const unsigned char *cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
+            int kmax = 0;
+#pragma unroll
+            for (int w = 0; w < BM / 32; ++w) {
+                const int blk = min(qb * BM + w * 32, Lq - 1) >> 5;
+                const int bound = dense_key_bound(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, Lk);
+                kmax = max(kmax, bound);
+                if (w == wave) {
+                    wkend = bound;
+                    skip_ones = dense_block_open(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, (Lk + 31) >> 5);
+                }
+            }
+            kend = kmax;
+        }
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    float qr[64], gr[64];   // the lane's Q fragment (scaled as in the forward pass) and dout fragment, columns 64*half ..
+    {
+        const float *qp = q + q_base + (long long)qic * rs + half * 64;
+        const float *gp = dout + q_base + (long long)qic * rs + half * 64;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
+            if (half * 64 + 4 * j < hd) {
+                t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+                g = *reinterpret_cast<const f32x4 *>(gp + 4 * j);
+            }
+            qr[4 * j + 0] = (t.x * rT) * LOG2E; qr[4 * j + 1] = (t.y * rT) * LOG2E;
+            qr[4 * j + 2] = (t.z * rT) * LOG2E; qr[4 * j + 3] = (t.w * rT) * LOG2E;
+            gr[4 * j + 0] = g.x; gr[4 * j + 1] = g.y; gr[4 * j + 2] = g.z; gr[4 * j + 3] = g.w;
+        }
+    }
+    const float m_i = stats[2 * ((long long)bh * Lq + qic)];
+    const float rl_i = stats[2 * ((long long)bh * Lq + qic) + 1];
+    const float D_i = D[(long long)bh * Lq + qic];
+
+    const int ld_row = tid >> 5, ld_col = (tid & 31) * 4;
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
+    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
+    const unsigned row8_bytes = 8u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[4], vst[4];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int o = (int)(ld_off0 + t * tile_bytes + i * row8_bytes);
+            kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o, 0, 0));
+            vst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o, 0, 0));
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int off = buf * TILE2_FLOATS + (i * 8 + ld_row) * LSTR2 + ld_col;
+            *reinterpret_cast<f32x4 *>(Ks + off) = kst[i];
+            *reinterpret_cast<f32x4 *>(Vs + off) = vst[i];
+        }
+    };
+
+    f32x16 acc[4];   // dQ^T, accumulator c row i is d = 4*i + c
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
+
+    if (ntiles > 0) { load_tile(0); store_tile(0); }
+    __syncthreads();
+
+    const int row_lds = ln * LSTR2 + half * 64;        // row-fragment base (S^T and dP^T products)
+    const int col_lds = (4 * half) * LSTR2 + 4 * ln;   // transposed-fragment base (dQ^T product)
+    const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
+
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        const bool more = (t + 1 < ntiles);
+        if (more) load_tile(t + 1);
+        const int k0 = t * BN;
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
+            f32x16 p = masked_scores<KIND, 16>(Ks + buf * TILE2_FLOATS + row_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p[r] = fast_exp2(p[r] - m_i) * rl_i;                    // the forward pass's weights
+            const f32x16 dp = tile_product128(Vs + buf * TILE2_FLOATS + row_lds, gr);            // dP^T = V . dout^T
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p[r] = p[r] * (dp[r] - D_i);                            // dS^T
+            tile_accumulate_t128(Ks + buf * TILE2_FLOATS + col_lds, p, acc);                     // dQ^T += K^T . dS^T
+        }
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+    if (qi < Lq) store_row_t128(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
+}
+
+// ------------------------------------------------------------------------------------------------ dK, dV
+template <int KIND>
+__global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
+                                                                 const float *__restrict__ v, const float *__restrict__ dout,
+                                                                 const float *__restrict__ stats, const float *__restrict__ D,
+                                                                 float *__restrict__ dk, float *__restrict__ dv, int H, int Lq,
+                                                                 int Lk, float rT, MaskArgs mask, int strict, int nkb,
+                                                                 int total_blocks, int lpt, int token_major, int hd) {
+    extern __shared__ __align__(16) float lds[];
+    float *Qs = lds;                        // [2][BN][LSTR2]  q * rT * log2(e)
+    float *Gs = lds + 2 * TILE2_FLOATS;     // [2][BN][LSTR2]  dout
+    float *Ss = lds + 4 * TILE2_FLOATS;     // per query tile: [2][32] reference maxima, [2][32] 1 / row sums, [2][32] D
+    int bh, unit;
+    if (!work_item(nkb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int kb = unit;
+    const int kw0 = kb * BM + wave * 32;
+    const int key = kw0 + ln;
+    const int keyc = key < Lk ? key : Lk - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
+
+    const int nqt = (Lq + 31) / 32;
+    int t_begin = 0, wt_begin = 0;
+    bool wave_active = true;
+    const unsigned char *skip_cls0 = nullptr;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) { t_begin = (kb * BM) / 32; wt_begin = kw0 / 32; }
+        if (LENS) {
+            if (kb * BM >= len) t_begin = nqt;
+            if (kw0 >= len) wave_active = false;
+        }
+        if (DENSE && mask.cls) {
+            skip_cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
+            int tmin = nqt;
+#pragma unroll
+            for (int w = 0; w < BM / 32; ++w) {
+                const int kt = min(kb * BM + w * 32, Lk - 1) >> 5;
+                const int first = dense_query_begin(mask, skip_cls0, kt, nqt, (Lk + 31) >> 5);
+                tmin = min(tmin, first);
+                if (w == wave) wt_begin = first;
+            }
+            t_begin = tmin;
+        }
+    }
+
+    float kr[64], vr[64];   // the lane's key and value rows (columns 64*half ..)
+    {
+        const float *kp = k + kv_base + (long long)keyc * rs + half * 64;
+        const float *vp = v + kv_base + (long long)keyc * rs + half * 64;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
+            if (half * 64 + 4 * j < hd) {
+                a = *reinterpret_cast<const f32x4 *>(kp + 4 * j);
+                c = *reinterpret_cast<const f32x4 *>(vp + 4 * j);
+            }
+            kr[4 * j + 0] = a.x; kr[4 * j + 1] = a.y; kr[4 * j + 2] = a.z; kr[4 * j + 3] = a.w;
+            vr[4 * j + 0] = c.x; vr[4 * j + 1] = c.y; vr[4 * j + 2] = c.z; vr[4 * j + 3] = c.w;
+        }
+    }
+
+    const int ld_row = tid >> 5, ld_col = (tid & 31) * 4;
+    const int q_bytes = (int)(((long long)(Lq - 1) * rs + hd) * 4);
+    const __amdgpu_buffer_rsrc_t qrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(q + q_base), 0, q_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t grsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(dout + q_base), 0, q_bytes, 0x00020000);
+    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
+    const unsigned row8_bytes = 8u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 qst[4], gst[4];
+    float sst = 0.f;
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int o = (int)(ld_off0 + t * tile_bytes + i * row8_bytes);
+            qst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(qrsrc, o, 0, 0));
+            gst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(grsrc, o, 0, 0));
+        }
+        if (tid < 96) {      // threads 0..31: reference maximum, 32..63: 1 / row sum, 64..95: D
+            const int row = t * 32 + (tid & 31);
+            const long long at = (long long)bh * Lq + row;
+            sst = 0.f;
+            if (row < Lq) sst = tid < 32 ? stats[2 * at] : (tid < 64 ? stats[2 * at + 1] : D[at]);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int off = buf * TILE2_FLOATS + (i * 8 + ld_row) * LSTR2 + ld_col;
+            f32x4 s;
+            s.x = (qst[i].x * rT) * LOG2E; s.y = (qst[i].y * rT) * LOG2E;
+            s.z = (qst[i].z * rT) * LOG2E; s.w = (qst[i].w * rT) * LOG2E;
+            *reinterpret_cast<f32x4 *>(Qs + off) = s;
+            *reinterpret_cast<f32x4 *>(Gs + off) = gst[i];
+        }
+        if (tid < 96) Ss[(tid >> 5) * 64 + buf * 32 + (tid & 31)] = sst;
+    };
+
+    f32x16 ka[4], va[4];   // dK^T and dV^T, accumulator c row i is d = 4*i + c
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { ka[c][i] = 0.f; va[c][i] = 0.f; }
+
+    if (t_begin < nqt) { load_tile(t_begin); store_tile(0); }
+    __syncthreads();
+
+    const int row_lds = ln * LSTR2 + half * 64;
+    const int col_lds = (4 * half) * LSTR2 + 4 * ln;
+    const float PEN = __fmul_rn(1e9f, LOG2E);
+    const unsigned char *cls_col = nullptr;
+    if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
+    const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
+
+    for (int t = t_begin; t < nqt; ++t) {
+        const int buf = (t - t_begin) & 1;
+        const bool more = (t + 1 < nqt);
+        if (more) load_tile(t + 1);
+        const int qt0 = t * 32;
+        int cls = 2;
+        if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq] & 3;
+        if (wave_active && t >= wt_begin &&
+            !(DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5))) {
+            // S[query, key] in the base-2 domain: rows = the tile's queries 8(r/4) + 4*half + r%4, column = the lane's key
+            f32x16 p = tile_product128(Qs + buf * TILE2_FLOATS + row_lds, kr);
+            if (DENSE) {
+                if (cls == 1) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[r] = __fsub_rn(p[r], PEN);
+                } else if (cls == 2) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        const int qc = qg < Lq ? qg : Lq - 1;
+                        p[r] = __fsub_rn(p[r], __fmul_rn(__fmul_rn(mcol[qc * mask.sq], 1e9f), LOG2E));
+                    }
+                }
+            } else if ((CAUSAL && (kw0 + 31 > qt0)) || (LENS && (kw0 + 32 > len))) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    bool blocked = false;
+                    if (CAUSAL) blocked = blocked || (key > qg);
+                    if (LENS) blocked = blocked || (key >= len);
+                    if (blocked) p[r] = __fsub_rn(p[r], PEN);
+                }
+            }
+            const float *st = Ss + buf * 32 + 4 * half;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 m4 = *reinterpret_cast<const f32x4 *>(st + 8 * g);
+                const f32x4 r4 = *reinterpret_cast<const f32x4 *>(st + 64 + 8 * g);
+                p[4 * g + 0] = fast_exp2(p[4 * g + 0] - m4.x) * r4.x;
+                p[4 * g + 1] = fast_exp2(p[4 * g + 1] - m4.y) * r4.y;
+                p[4 * g + 2] = fast_exp2(p[4 * g + 2] - m4.z) * r4.z;
+                p[4 * g + 3] = fast_exp2(p[4 * g + 3] - m4.w) * r4.w;
+            }
+            tile_accumulate_t128(Gs + buf * TILE2_FLOATS + col_lds, p, va);                      // dV^T += dout^T . P
+            const f32x16 dp = tile_product128(Gs + buf * TILE2_FLOATS + row_lds, vr);            // dP = dout . V^T
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 d4 = *reinterpret_cast<const f32x4 *>(st + 128 + 8 * g);
+                p[4 * g + 0] = p[4 * g + 0] * (dp[4 * g + 0] - d4.x);
+                p[4 * g + 1] = p[4 * g + 1] * (dp[4 * g + 1] - d4.y);
+                p[4 * g + 2] = p[4 * g + 2] * (dp[4 * g + 2] - d4.z);
+                p[4 * g + 3] = p[4 * g + 3] * (dp[4 * g + 3] - d4.w);
+            }
+            tile_accumulate_t128(Qs + buf * TILE2_FLOATS + col_lds, p, ka);                      // dK^T += Q~^T . dS
+        }
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+    if (key < Lk) {
+        store_row_t128(dv + kv_base + (long long)key * rs, va, 1.0f, half, hd);
+        store_row_t128(dk + kv_base + (long long)key * rs, ka, 0.69314718055994530942f, half, hd);   // Q~ carries log2(e)
+    }
+}
+
+template <int KIND>
+int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
+                  const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
+                  int strict, int token_major, int hd) {
+    constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    static bool attr_set[8] = {false};
+    const size_t lds_dq = 4 * TILE2_FLOATS * sizeof(float);
+    const size_t lds_dkv = (4 * TILE2_FLOATS + 192) * sizeof(float);
+    if (!attr_set[KIND]) {
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_f32_d128<KIND>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq));
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
+        attr_set[KIND] = true;
+    }
+    const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
+    {
+        const int nqb = (Lq + BM - 1) / BM;
+        const long long total = (long long)nqb * B * H;
+        DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
+        int lpt = (uneven && nqb >= 2) ? 1 : 0;
+        if (lpt && total <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+        hipLaunchKernelGGL(sdpa_bwd_dq_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq, ctx->stream, q, k,
+                           v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, hd);
+        const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d128");
+        if (rc != DL4S_HIP_OK) return rc;
+    }
+    {
+        const int nkb = (Lk + BM - 1) / BM;
+        const long long total = (long long)nkb * B * H;
+        DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
+        int lpt = (uneven && nkb >= 2) ? 1 : 0;
+        if (lpt && total <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+        hipLaunchKernelGGL(sdpa_bwd_dkv_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
+                           k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total, lpt, token_major, hd);
+        return dl4s::launch_status("sdpa_bwd_dkv_f32_d128");
+    }
+}
+
+}  // namespace

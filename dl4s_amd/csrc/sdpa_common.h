@@ -17,6 +17,10 @@ constexpr int BN = 32;       // keys per LDS tile
 constexpr int LSTR = 68;     // LDS row stride in floats: 64 + 4 keeps 128-bit reads of 8 rows on distinct banks
 constexpr int TILE_FLOATS = BN * LSTR;
 constexpr float LOG2E = 1.44269504088896340736f;
+// the 128-wide kernels (head dims above 64 up to 128)
+constexpr int HD2 = 128;
+constexpr int LSTR2 = HD2 + 4;   // 132 = 4 mod 32: the same bank spread as LSTR
+constexpr int TILE2_FLOATS = BN * LSTR2;
 
 struct MaskArgs {
     int kind;

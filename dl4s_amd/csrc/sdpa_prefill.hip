@@ -577,11 +577,10 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
     const bool mfma_path = dk == dv && dk <= HD && dk % 4 == 0 &&
                            ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                              reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-    // head dims above 64 up to 128: the 128-wide MFMA kernel.  Not when row statistics are wanted: the gradient kernels
-    // for these head dims are the plain ones, which read the plain forward kernel's statistics.
+    // head dims above 64 up to 128: the 128-wide MFMA kernel
     const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                            reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-    const bool mfma128_path = dk == dv && dk > HD && dk <= HD2 && dk % 4 == 0 && aligned && !stats;
+    const bool mfma128_path = dk == dv && dk > HD && dk <= HD2 && dk % 4 == 0 && aligned;
     MaskArgs m{};
     {
         const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path, m);
@@ -616,7 +615,7 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
             default: return launch_d128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
         }
     }
-    DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 128 (64 with row statistics), and 16-byte aligned tensors");
+    DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 128, and 16-byte aligned tensors");
     DL4S_REQUIRE(dk <= GEN_MAXD && dv <= GEN_MAXD && dv > 0, DL4S_HIP_EUNSUPPORTED,
                  "sdpa: head dims (%lld, %lld) above %d are not implemented", (long long)dk, (long long)dv, GEN_MAXD);
     const long long rows = B * H * Lq;

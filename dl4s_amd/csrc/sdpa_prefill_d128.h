@@ -16,10 +16,6 @@
 
 namespace {
 
-constexpr int HD2 = 128;
-constexpr int LSTR2 = HD2 + 4;
-constexpr int TILE2_FLOATS = BN * LSTR2;
-
 template <int KIND>
 __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
                                                                  const float *__restrict__ v, float *__restrict__ out, int H,

@@ -125,7 +125,7 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
                           int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
 
-/* Training form of the fused attention (key dim = value dim = d; MFMA kernels under the forward call's conditions, plain kernels up to 256).  The reference differentiates ScaledDotProductAttention through
+/* Training form of the fused attention (key dim = value dim = d; MFMA kernels for d a multiple of 4 up to 128 and 16-byte aligned tensors, plain kernels up to 256).  The reference differentiates ScaledDotProductAttention through
  * the backward closures of its primitive operators (Tensor/Operators/Matrix.swift:139-174 for the products through the
  * subscript views and the stack of broadcastMatrixMultiplied :79-117, Binary.swift:235-300 for e / sum,
  * Reduce.swift:35-62, Unary.swift:33-55 for exp, Binary.swift:161-224 for the subtractions); a backend that fuses the

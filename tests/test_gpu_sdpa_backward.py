@@ -160,10 +160,10 @@ def test_config4_sized_gradients(ctx, orc):
         assert_parity(dv[sl], rv, "config 4 dv")
 
 
-@pytest.mark.parametrize("d", [4, 8, 40, 60, 6, 130])
+@pytest.mark.parametrize("d", [4, 8, 40, 60, 6, 130, 72, 96, 128, 200])
 @pytest.mark.parametrize("mask_kind", ["none", "dense", "causal_lengths"])
 def test_gradients_for_other_head_dims(ctx, orc, d, mask_kind):
-    """Head dims other than 64: multiples of 4 below it on the MFMA kernels with zero padding columns (e.g. the key size
+    """Head dims other than 64: multiples of 4 up to 128 on the MFMA kernels with zero padding columns (e.g. the key size
     8 of Tests/DL4STests/TransformerTests.swift:31), the others on the plain kernels."""
     from dl4s_amd import lib
     B, H, L = 2, 3, 70
@@ -218,7 +218,7 @@ def test_random_shapes_forward_and_backward(ctx, orc, seed):
     if kind_name.startswith("causal"):
         Lk = Lq
     scale = float(rng.choice([0.3, 1.0, 3.0]))
-    d = 64 if seed % 3 else int(rng.choice([4, 8, 20, 32, 48]))     # every third case on padded tiles
+    d = 64 if seed % 3 else int(rng.choice([4, 8, 20, 32, 48, 96, 128]))     # every third case on padded or 128-wide tiles
     q, k, v, dout = rand(rng, B, H, Lq, d, scale=scale), rand(rng, B, H, Lk, d, scale=scale), rand(rng, B, H, Lk, d), rand(rng, B, H, Lq, d)
     lens = rng.integers(1, Lk + 1, size=B)
     kw, mask = {}, None
@@ -326,3 +326,42 @@ def test_gradient_descent_through_the_fused_gradients_converges(ctx, d):
     assert np.isfinite(losses).all()
     assert losses[-1] < 0.02 * losses[0], (losses[0], losses[-1])       # the CPU oracle's gradients give 0.01
     assert losses[-1] < losses[100] < 0.1 * losses[0]
+
+
+@pytest.mark.parametrize("d", [128, 80])
+@pytest.mark.parametrize("mask_kind", ["none", "dense", "lengths", "causal", "causal_lengths"])
+def test_gradients_on_the_128_wide_kernels(ctx, orc, d, mask_kind):
+    """Head dims above 64: parity with the oracle for every mask kind, the structured descriptors bit-identical to the
+    dense masks they describe (strict), tile skipping and the token-major layout bit-identical too."""
+    from dl4s_amd import lib
+    B, H, L = 2, 2, 200
+    rng = np.random.default_rng(d * 10 + len(mask_kind))
+    q, k, v, dout = (rand(rng, B, H, L, d) for _ in range(4))
+    lens = np.array([L, 77])
+    kw, mask = {}, None
+    if mask_kind == "dense":
+        mask = (rng.random((B, 1, L, L)) < 0.3).astype(np.float32)
+        mask[0, 0, 5, :] = 1.0
+        kw = dict(mask=mask)
+    elif mask_kind == "lengths":
+        mask, kw = lengths_mask(lens, L), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    elif mask_kind == "causal":
+        mask, kw = causal_mask(L, L), dict(kind=lib.MASK_CAUSAL)
+    elif mask_kind == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, L), causal_mask(L, L)[None, None])
+        kw = dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens)
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, **kw)
+    assert_parity(out, orc.sdpa(q, k, v, mask), "forward with stats d=%d" % d)
+    rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+    assert_parity(dq, rq, "dq d=%d %s" % (d, mask_kind))
+    assert_parity(dk, rk, "dk d=%d %s" % (d, mask_kind))
+    assert_parity(dv, rv, "dv d=%d %s" % (d, mask_kind))
+    if mask is not None:
+        dense_strict = run_fwd_bwd(ctx, q, k, v, dout, mask=mask, strict=True)
+        if mask_kind != "dense":
+            for a, b_ in zip(dense_strict, run_fwd_bwd(ctx, q, k, v, dout, strict=True, **kw)):
+                assert np.array_equal(a, b_)
+        for a, b_ in zip(dense_strict, run_fwd_bwd(ctx, q, k, v, dout, mask=mask)):
+            assert np.array_equal(a, b_)
+    for a, b_ in zip(run_fwd_bwd(ctx, q, k, v, dout, token_major=True, **kw), (out, stats, dq, dk, dv)):
+        assert np.array_equal(a, b_)
