@@ -128,21 +128,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
     if (!strict && !(LENS && len <= 0)) {
         if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
         if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
-        if (DENSE && mask.cls) {   // trailing all-ones tiles of open blocks
-            const unsigned char *cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
-            int kmax = 0;
-#pragma unroll
-            for (int w = 0; w < BM / 32; ++w) {
-                const int blk = min(qb * BM + w * 32, Lq - 1) >> 5;
-                const int bound = dense_key_bound(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, Lk);
-                kmax = max(kmax, bound);
-                if (w == wave) {
-                    wkend = bound;
-                    skip_ones = dense_block_open(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, (Lk + 31) >> 5);
-                }
-            }
-            kend = kmax;
-        }
+        if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
     }
     const int ntiles = (kend + BN - 1) / BN;
 
@@ -268,18 +254,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
             if (kb * BM >= len) t_begin = nqt;
             if (kw0 >= len) wave_active = false;
         }
-        if (DENSE && mask.cls) {   // leading all-ones tiles of open query blocks
-            skip_cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
-            int tmin = nqt;
-#pragma unroll
-            for (int w = 0; w < BM / 32; ++w) {
-                const int kt = min(kb * BM + w * 32, Lk - 1) >> 5;
-                const int first = dense_query_begin(mask, skip_cls0, kt, nqt, (Lk + 31) >> 5);
-                tmin = min(tmin, first);
-                if (w == wave) wt_begin = first;
-            }
-            t_begin = tmin;
-        }
+        if (DENSE && mask.cls) skip_cls0 = dense_query_bounds(mask, b, hh, kb * BM, wave, nqt, Lk, t_begin, wt_begin);
     }
 
     float kr[32], vr[32];   // the lane's key and value rows (columns half*32 ..)

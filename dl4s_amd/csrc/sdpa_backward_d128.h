@@ -1,5 +1,5 @@
 // Gradients of the fused attention for head dims above 64 and up to 128 (multiples of 4): the two deterministic kernels
-// of sdpa_backward.hip on 128-wide tiles.  Included by sdpa_backward.hip only; needs sdpa_prefill_d128.h's constants.
+// of sdpa_backward.hip on 128-wide tiles.  Included by sdpa_backward.hip only.
 //
 // The operand layouts follow the 128-wide forward kernel: a score product contracts d = 64*half + j over 64 MFMA steps;
 // a transposed accumulation (dQ^T, dK^T, dV^T) uses four accumulators whose rows interleave (accumulator c row i is
@@ -113,21 +113,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
     if (!strict && !(LENS && len <= 0)) {
         if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
         if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
-        if (DENSE && mask.cls) {
-            const unsigned char *cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
-            int kmax = 0;
-#pragma unroll
-            for (int w = 0; w < BM / 32; ++w) {
-                const int blk = min(qb * BM + w * 32, Lq - 1) >> 5;
-                const int bound = dense_key_bound(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, Lk);
-                kmax = max(kmax, bound);
-                if (w == wave) {
-                    wkend = bound;
-                    skip_ones = dense_block_open(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, (Lk + 31) >> 5);
-                }
-            }
-            kend = kmax;
-        }
+        if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
     }
     const int ntiles = (kend + BN - 1) / BN;
 
@@ -253,18 +239,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
             if (kb * BM >= len) t_begin = nqt;
             if (kw0 >= len) wave_active = false;
         }
-        if (DENSE && mask.cls) {
-            skip_cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
-            int tmin = nqt;
-#pragma unroll
-            for (int w = 0; w < BM / 32; ++w) {
-                const int kt = min(kb * BM + w * 32, Lk - 1) >> 5;
-                const int first = dense_query_begin(mask, skip_cls0, kt, nqt, (Lk + 31) >> 5);
-                tmin = min(tmin, first);
-                if (w == wave) wt_begin = first;
-            }
-            t_begin = tmin;
-        }
+        if (DENSE && mask.cls) skip_cls0 = dense_query_bounds(mask, b, hh, kb * BM, wave, nqt, Lk, t_begin, wt_begin);
     }
 
     float kr[64], vr[64];   // the lane's key and value rows (columns 64*half ..)

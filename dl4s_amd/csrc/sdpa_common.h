@@ -122,6 +122,45 @@ __device__ __forceinline__ int dense_query_begin(const MaskArgs &m, const unsign
     return nqt;
 }
 
+// Dense masks, tile skipping, for a workgroup of BM / 32 wavefronts that owns the queries first .. first + BM - 1 (one
+// 32-query block per wavefront; `sub` = this wavefront's block): kend = the keys the workgroup has to visit (the largest
+// bound of its blocks), wkend = this wavefront's own bound, skip_ones = whether its all-ones tiles may be skipped.
+__device__ __forceinline__ void dense_key_bounds(const MaskArgs &m, const int b, const int hh, const int first, const int sub,
+                                                 const int Lq, const int Lk, int &kend, int &wkend, bool &skip_ones) {
+    const unsigned char *cls0 = m.cls + (long long)b * m.cls_sb + hh * m.cls_sh;
+    int kmax = 0;
+#pragma unroll
+    for (int w = 0; w < BM / 32; ++w) {
+        const int blk = min(first + w * 32, Lq - 1) >> 5;
+        const unsigned char *row = cls0 + (long long)blk * m.cls_sq;
+        const int bound = dense_key_bound(row, m.cls_sk, blk, Lk);
+        kmax = max(kmax, bound);
+        if (w == sub) {
+            wkend = bound;
+            skip_ones = dense_block_open(row, m.cls_sk, blk, (Lk + 31) >> 5);
+        }
+    }
+    kend = kmax;
+}
+
+// The same seen from a workgroup that owns the keys first .. first + BM - 1: t_begin = the first query tile the workgroup
+// has to visit, wt_begin = this wavefront's own.  Returns the (batch, head) slab's tile classes for the per-tile test.
+__device__ __forceinline__ const unsigned char *dense_query_bounds(const MaskArgs &m, const int b, const int hh, const int first,
+                                                                   const int sub, const int nqt, const int Lk, int &t_begin,
+                                                                   int &wt_begin) {
+    const unsigned char *cls0 = m.cls + (long long)b * m.cls_sb + hh * m.cls_sh;
+    int tmin = nqt;
+#pragma unroll
+    for (int w = 0; w < BM / 32; ++w) {
+        const int kt = min(first + w * 32, Lk - 1) >> 5;
+        const int begin = dense_query_begin(m, cls0, kt, nqt, (Lk + 31) >> 5);
+        tmin = min(tmin, begin);
+        if (w == sub) wt_begin = begin;
+    }
+    t_begin = tmin;
+    return cls0;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }

@@ -136,21 +136,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_prefill_f32_d64(const float *__re
             kend = min(kend, len);
             wkend = min(wkend, len);
         }
-        if (DENSE && mask.cls) {   // trailing all-ones tiles of open blocks
-            const unsigned char *cls0 = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh;
-            int kmax = 0;
-#pragma unroll
-            for (int w = 0; w < BM / 32; ++w) {
-                const int blk = min(qb * BM + w * 32, Lq - 1) >> 5;
-                const int bound = dense_key_bound(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, Lk);
-                kmax = max(kmax, bound);
-                if (w == wave) {
-                    wkend = bound;
-                    skip_ones = dense_block_open(cls0 + (long long)blk * mask.cls_sq, mask.cls_sk, blk, (Lk + 31) >> 5);
-                }
-            }
-            kend = kmax;
-        }
+        if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
     }
     const int ntiles = (kend + BN - 1) / BN;
 
