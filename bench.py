@@ -168,6 +168,74 @@ def other_configs(ctx, lib, cpu, only=None):
             orc.mha(x, x, x, mask, attn, H, dk_, dk_)
             dt = time.perf_counter() - t0
             res["config2_mha_B4_L512_D512_H8_causal_fused"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
+    if want("recorded"):
+        # Calls recorded into a HIP graph and replayed, against the same calls issued one by one.
+        B, L, D, H, dk_ = 4, 512, 512, 8, 64
+        rng = np.random.Generator(np.random.PCG64(1012))
+        x = rng.standard_normal((B, L, D), dtype=np.float32)
+        i, j = np.indices((L, L))
+        mask = (j > i).astype(np.float32)
+        fl = 4.0 * 64 * B * H * (L * (L + 1) // 2) + 4 * 2.0 * B * L * D * D
+        # config 2's fused layer (projections in one launch, attention, output product + residual, layer norm) on
+        # fixed buffers through the C ABI: issued one by one, and recorded once into a graph and replayed
+        r = lambda *sh: ctx.to_device(rng.standard_normal(sh, dtype=np.float32) * np.float32(0.05))
+        dx, dmask, w4 = ctx.to_device(x.reshape(B * L, D)), ctx.to_device(mask), [r(D, D) for _ in range(4)]
+        dscale, dshift = r(L, D), r(L, D)
+        t = [ctx.empty((B * L, D)) for _ in range(6)]
+        md = ctx.mask_desc(lib.MASK_DENSE, dense=dmask)
+
+        def layer_calls():
+            ctx.gemm_grouped([dx, dx, dx], (B * L, D), w4[:3], (D, D), t[:3])
+            ctx.sdpa_fwd(t[0], t[1], t[2], t[3], B, H, L, L, dk_, dk_, 0.125, mask=md, flags=lib.SDPA_TOKEN_MAJOR)
+            ctx.dense_fused(t[3], B * L, D, w4[3], D, None, lib.ACT_NONE, dx, t[4])
+            ctx.layernorm(t[4], None, dscale, dshift, t[5], B, L, D)
+
+        def timed(fn, n):
+            for _ in range(n * 10):
+                fn()
+            ctx.sync()
+            ctx.timer_begin()
+            for _ in range(n):
+                fn()
+            return ctx.timer_end() / n
+
+        ms_calls = timed(layer_calls, 100)
+        y_calls = t[5].numpy()
+        ctx.graph_begin()
+        layer_calls()
+        graph = ctx.graph_end()
+        ctx.fill(0.0, t[5], B * L * D)
+        ms_graph = timed(graph.replay, 100)
+        same = bool(np.array_equal(t[5].numpy(), y_calls))
+        res["config2_mha_B4_L512_D512_H8_causal_c_abi_calls_recorded"] = {
+            "us_per_call_issued_one_by_one": ms_calls * 1e3, "us_per_call_replayed": ms_graph * 1e3, "graph_nodes": graph.nodes,
+            "replay_equals_calls_bitwise": same, "tflops": fl / ms_graph / 1e9,
+            "frac_mfma_peak": fl / ms_graph / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
+        graph.destroy()
+        for b_ in [dx, dmask, dscale, dshift] + w4 + t:
+            b_.release()
+        # a chain of 32 dependent element-wise calls on 4096 floats: nothing but launch latency
+        n = 4096
+        a_, b_ = ctx.empty((n,)), ctx.empty((n,))
+        ctx.fill(1.0, a_, n)
+        ctx.fill(0.0, b_, n)
+
+        def chain():
+            for _ in range(16):
+                ctx.vadd(a_, b_, b_, n)
+                ctx.vmul(a_, b_, b_, n)
+
+        ms_calls = timed(chain, 50)
+        ctx.graph_begin()
+        chain()
+        graph = ctx.graph_end()
+        ms_graph = timed(graph.replay, 50)
+        res["chain_of_32_dependent_small_kernels_recorded"] = {
+            "us_per_kernel_issued_one_by_one": ms_calls * 1e3 / 32, "us_per_kernel_replayed": ms_graph * 1e3 / 32,
+            "graph_nodes": graph.nodes}
+        graph.destroy()
+        a_.release()
+        b_.release()
     if want("config3"):
         # config 3: encoder block B8 L1024 D1024 H16 F4096, key-length mask
         B, L, D, H, F = 8, 1024, 1024, 16, 4096
@@ -411,7 +479,7 @@ def main():
                          "profiler counter runs")
     ap.add_argument("--only", default="", metavar="NAMES",
                     help="instead of the benchmark, run only these of the workloads reported beside the headline (comma "
-                         "separated: config1, config2, config3, backward, masks_and_head_dim, greedy, greedy_fused, greedy_primitive) and print their entries: "
+                         "separated: config1, config2, recorded, config3, backward, masks_and_head_dim, greedy, greedy_fused, greedy_primitive) and print their entries: "
                          "short commands for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:

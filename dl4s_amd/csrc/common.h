@@ -30,6 +30,19 @@ struct dl4s_hip_ctx {
     // Held by an entry point from the launch that fills the scratch block to the launch that reads it, so that calls
     // from several host threads cannot interleave their use of it (the kernels themselves are ordered by the stream).
     std::mutex scratch_mu;
+    // Stream capture (dl4s_hip_graph_begin .. dl4s_hip_graph_end): entry points that would wait for the stream, copy to or
+    // from host memory or change device allocations refuse to run while it is set.  scratch_generation counts the
+    // regrowths of the scratch block; a captured graph holds the block's address and is refused once it has moved.
+    bool capturing = false;
+    unsigned long long scratch_generation = 0;
+};
+
+struct dl4s_hip_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    dl4s_hip_ctx *owner = nullptr;
+    size_t nodes = 0;
+    unsigned long long scratch_generation = 0;
 };
 
 namespace dl4s {
@@ -44,6 +57,15 @@ int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes);
         if (!(ctx)) return dl4s::set_error(DL4S_HIP_EINVALID_ARG, "%s: ctx is NULL", __func__); \
         hipError_t e__ = hipSetDevice((ctx)->device);                              \
         if (e__ != hipSuccess) return dl4s::hip_error(e__, "hipSetDevice");        \
+    } while (0)
+
+// For entry points that cannot be recorded into a graph.
+#define DL4S_NOT_WHILE_CAPTURING(ctx)                                                                       \
+    do {                                                                                                    \
+        if ((ctx)->capturing)                                                                               \
+            return dl4s::set_error(DL4S_HIP_EUNSUPPORTED,                                                   \
+                                   "%s cannot be recorded into a graph (it waits for the stream, copies to or from " \
+                                   "host memory or allocates)", __func__);                                  \
     } while (0)
 
 #define DL4S_HIP_TRY(expr)                                               \

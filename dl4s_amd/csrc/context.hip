@@ -33,6 +33,9 @@ static size_t round_size(size_t bytes) {
 int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes) {
     std::lock_guard<std::mutex> g(ctx->mu);
     if (bytes <= ctx->scratch_bytes) return DL4S_HIP_OK;
+    DL4S_REQUIRE(!ctx->capturing, DL4S_HIP_EUNSUPPORTED,
+                 "a call recorded into a graph needs %zu bytes of library scratch and %zu are there: run the same calls "
+                 "once before recording them", bytes, ctx->scratch_bytes);
     // the old block may still be read by enqueued kernels: wait before releasing it
     if (ctx->scratch) {
         DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -43,6 +46,7 @@ int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes) {
     size_t want = round_size(bytes);
     DL4S_HIP_TRY(hipMalloc(&ctx->scratch, want));
     ctx->scratch_bytes = want;
+    ++ctx->scratch_generation;
     return DL4S_HIP_OK;
 }
 
@@ -103,6 +107,7 @@ int dl4s_hip_destroy(dl4s_hip_ctx *ctx) {
 
 int dl4s_hip_sync(dl4s_hip_ctx *ctx) {
     DL4S_CHECK_CTX(ctx);
+    DL4S_NOT_WHILE_CAPTURING(ctx);
     DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
     return DL4S_HIP_OK;
 }
@@ -117,6 +122,7 @@ int dl4s_hip_device_info(dl4s_hip_ctx *ctx, int *out_cu_count, int *out_clock_kh
 
 int dl4s_hip_timer_begin(dl4s_hip_ctx *ctx) {
     DL4S_CHECK_CTX(ctx);
+    DL4S_NOT_WHILE_CAPTURING(ctx);
     DL4S_HIP_TRY(hipEventRecord(ctx->ev_begin, ctx->stream));
     return DL4S_HIP_OK;
 }
@@ -124,9 +130,90 @@ int dl4s_hip_timer_begin(dl4s_hip_ctx *ctx) {
 int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms) {
     DL4S_CHECK_CTX(ctx);
     DL4S_REQUIRE(out_ms, DL4S_HIP_EINVALID_ARG, "dl4s_hip_timer_end: out_ms is NULL");
+    DL4S_NOT_WHILE_CAPTURING(ctx);
     DL4S_HIP_TRY(hipEventRecord(ctx->ev_end, ctx->stream));
     DL4S_HIP_TRY(hipEventSynchronize(ctx->ev_end));
     DL4S_HIP_TRY(hipEventElapsedTime(out_ms, ctx->ev_begin, ctx->ev_end));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_graph_begin(dl4s_hip_ctx *ctx) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(!ctx->capturing, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_begin: a graph is being recorded already");
+    // thread-local mode: calls of other host threads on other streams are left alone
+    DL4S_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_graph_end(dl4s_hip_ctx *ctx, dl4s_hip_graph **out_graph) {
+    DL4S_CHECK_CTX(ctx);
+    if (out_graph) *out_graph = nullptr;
+    DL4S_REQUIRE(ctx->capturing, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_end: no graph is being recorded");
+    ctx->capturing = false;
+    hipGraph_t recorded = nullptr;
+    DL4S_HIP_TRY(hipStreamEndCapture(ctx->stream, &recorded));
+    if (!out_graph) {  // the caller gives the recording up
+        if (recorded) (void)hipGraphDestroy(recorded);
+        return DL4S_HIP_OK;
+    }
+    dl4s_hip_graph *g = new (std::nothrow) dl4s_hip_graph();
+    if (!g) {
+        (void)hipGraphDestroy(recorded);
+        return set_error(DL4S_HIP_EOOM, "dl4s_hip_graph_end: host allocation failed");
+    }
+    g->graph = recorded;
+    hipError_t e = hipGraphInstantiate(&g->exec, recorded, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(recorded);
+        delete g;
+        return hip_error(e, "hipGraphInstantiate");
+    }
+    size_t nodes = 0;
+    (void)hipGraphGetNodes(recorded, nullptr, &nodes);
+    g->nodes = nodes;
+    g->owner = ctx;
+    {
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        g->scratch_generation = ctx->scratch_generation;
+    }
+    *out_graph = g;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_graph_launch(dl4s_hip_ctx *ctx, dl4s_hip_graph *graph) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(graph && graph->owner == ctx, DL4S_HIP_EINVALID_ARG,
+                 "dl4s_hip_graph_launch: the graph is NULL or was recorded on another context");
+    DL4S_REQUIRE(!ctx->capturing, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_launch: a graph is being recorded");
+    // the mutex orders the replay against a host thread whose call regrows the scratch block
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
+    {
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        DL4S_REQUIRE(graph->scratch_generation == ctx->scratch_generation, DL4S_HIP_EUNSUPPORTED,
+                     "dl4s_hip_graph_launch: the library's scratch block has been regrown since the graph was recorded; "
+                     "record it again");
+    }
+    DL4S_HIP_TRY(hipGraphLaunch(graph->exec, ctx->stream));
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_graph_node_count(dl4s_hip_ctx *ctx, const dl4s_hip_graph *graph, size_t *out_nodes) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(graph && out_nodes, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_node_count: NULL argument");
+    *out_nodes = graph->nodes;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_graph_destroy(dl4s_hip_ctx *ctx, dl4s_hip_graph *graph) {
+    DL4S_CHECK_CTX(ctx);
+    if (!graph) return DL4S_HIP_OK;
+    DL4S_REQUIRE(graph->owner == ctx, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_destroy: recorded on another context");
+    // a replay that is still running reads the executable graph
+    DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    (void)hipGraphExecDestroy(graph->exec);
+    (void)hipGraphDestroy(graph->graph);
+    delete graph;
     return DL4S_HIP_OK;
 }
 
@@ -143,6 +230,9 @@ int dl4s_hip_alloc(dl4s_hip_ctx *ctx, size_t bytes, void **out_ptr) {
         it->second.pop_back();
         ctx->bytes_pooled -= sz;
     } else {
+        DL4S_REQUIRE(!ctx->capturing, DL4S_HIP_EUNSUPPORTED,
+                     "dl4s_hip_alloc: no pooled block of %zu bytes while a graph is being recorded; allocate before "
+                     "dl4s_hip_graph_begin", sz);
         hipError_t e = hipMalloc(&p, sz);
         if (e == hipErrorOutOfMemory) {
             // give the pooled blocks back to the driver and try once more
@@ -203,6 +293,7 @@ int dl4s_hip_assign_h2d(dl4s_hip_ctx *ctx, void *dst_dev, const void *src_host, 
     DL4S_CHECK_CTX(ctx);
     if (bytes == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(dst_dev && src_host, DL4S_HIP_EINVALID_ARG, "dl4s_hip_assign_h2d: NULL pointer");
+    DL4S_NOT_WHILE_CAPTURING(ctx);
     // pageable source: the async copy stages the data before returning only for small sizes, so wait
     DL4S_HIP_TRY(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
     DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
@@ -221,6 +312,7 @@ int dl4s_hip_assign_d2h(dl4s_hip_ctx *ctx, void *dst_host, const void *src_dev, 
     DL4S_CHECK_CTX(ctx);
     if (bytes == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(dst_host && src_dev, DL4S_HIP_EINVALID_ARG, "dl4s_hip_assign_d2h: NULL pointer");
+    DL4S_NOT_WHILE_CAPTURING(ctx);
     DL4S_HIP_TRY(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
     return DL4S_HIP_OK;

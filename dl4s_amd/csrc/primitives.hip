@@ -701,6 +701,7 @@ int dl4s_hip_argmax_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, i
     *out_value = -INFINITY;            // the reference's result for an empty buffer
     if (count == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(values, DL4S_HIP_EINVALID_ARG, "argmax: NULL pointer");
+    DL4S_NOT_WHILE_CAPTURING(ctx);
     std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     int rc = dl4s::ensure_scratch(ctx, 16);
     if (rc) return rc;

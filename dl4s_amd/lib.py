@@ -82,6 +82,27 @@ def _shape_arr(shape):
     return (_i64 * max(1, len(shape)))(*shape)
 
 
+class Graph:
+    """A recorded sequence of calls (dl4s_hip_graph_*); replay() enqueues it on the context's stream."""
+
+    def __init__(self, ctx, handle):
+        self.ctx, self.handle = ctx, handle
+
+    def replay(self):
+        _check(self.ctx.lib.dl4s_hip_graph_launch(self.ctx.handle, self.handle))
+
+    @property
+    def nodes(self):
+        n = C.c_size_t()
+        _check(self.ctx.lib.dl4s_hip_graph_node_count(self.ctx.handle, self.handle, C.byref(n)))
+        return n.value
+
+    def destroy(self):
+        if self.handle is not None and self.ctx.handle is not None:
+            _check(self.ctx.lib.dl4s_hip_graph_destroy(self.ctx.handle, self.handle))
+        self.handle = None
+
+
 class Context:
     """One GPU, one stream, one pooled allocator (dl4s_hip_ctx)."""
 
@@ -117,6 +138,19 @@ class Context:
         ms = C.c_float()
         _check(self.lib.dl4s_hip_timer_end(self.handle, C.byref(ms)))
         return ms.value
+
+    # ---- recorded call sequences
+    def graph_begin(self):
+        _check(self.lib.dl4s_hip_graph_begin(self.handle))
+
+    def graph_end(self, keep=True):
+        """Ends the recording; returns a Graph, or None when keep is False (the recording is given up)."""
+        if not keep:
+            _check(self.lib.dl4s_hip_graph_end(self.handle, None))
+            return None
+        g = _vp()
+        _check(self.lib.dl4s_hip_graph_end(self.handle, C.byref(g)))
+        return Graph(self, g)
 
     def device_info(self):
         cu, khz = C.c_int(), C.c_int()

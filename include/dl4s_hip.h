@@ -52,6 +52,33 @@ int dl4s_hip_device_info(dl4s_hip_ctx *ctx, int *out_cu_count, int *out_clock_kh
 int dl4s_hip_timer_begin(dl4s_hip_ctx *ctx);
 int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms);
 
+/* ------------------------------------------------------------------ recorded call sequences (HIP graphs)
+ * No counterpart in the reference.  A fixed sequence of calls on fixed buffers (one layer, one decode step at a fixed
+ * length) costs about 3 us of launch latency per kernel when it is issued call by call and about 1.8 us when it is
+ * replayed from a graph.  Between dl4s_hip_graph_begin and dl4s_hip_graph_end the calls on this context are recorded
+ * instead of run; dl4s_hip_graph_launch replays them, in stream order with everything else on the context.
+ *
+ * What can be recorded: every entry point that only enqueues kernels or device-to-device copies.  Entry points that
+ * wait for the stream, copy to or from host memory (dl4s_hip_sync, the timer, dl4s_hip_assign_h2d / _d2h, the single
+ * value getters and setters, dl4s_hip_argmax_f32) or that would have to allocate (dl4s_hip_alloc without a pooled
+ * block of that size, a call that needs more library scratch than is there) return DL4S_HIP_EUNSUPPORTED and leave the
+ * recording open.  Run the same calls once before recording them: that sizes the scratch block.
+ *
+ * A graph holds the addresses it was recorded with.  Every buffer that the recorded calls read or write, temporaries
+ * included, must stay allocated (not handed back with dl4s_hip_free and allocated again for something else) for as
+ * long as the graph is replayed; inputs are read at replay time, so new data in the same buffers gives new results.
+ * Some calls use the library's scratch block: if a later call regrows it, dl4s_hip_graph_launch refuses the graph
+ * (DL4S_HIP_EUNSUPPORTED) and it has to be recorded again.  One recording at a time per context, made and replayed
+ * from one host thread at a time.
+ *
+ * dl4s_hip_graph_end with out_graph == NULL gives the recording up. */
+typedef struct dl4s_hip_graph dl4s_hip_graph;
+int dl4s_hip_graph_begin(dl4s_hip_ctx *ctx);
+int dl4s_hip_graph_end(dl4s_hip_ctx *ctx, dl4s_hip_graph **out_graph);
+int dl4s_hip_graph_launch(dl4s_hip_ctx *ctx, dl4s_hip_graph *graph);
+int dl4s_hip_graph_node_count(dl4s_hip_ctx *ctx, const dl4s_hip_graph *graph, size_t *out_nodes);
+int dl4s_hip_graph_destroy(dl4s_hip_ctx *ctx, dl4s_hip_graph *graph);
+
 /* ------------------------------------------------------- MemoryOperatorsType subset */
 /* Engine/Engine.swift:49,55 allocateBuffer.  Memory is NOT zeroed (the reference's is not either,
  * Engine/CPU/CPU.swift:71-96).  bytes == 0 yields a valid unique pointer. */
