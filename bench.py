@@ -526,7 +526,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "long-context prefill B=8 H=16 L=2048 d=64 causal, q/k/v=0.5*N(0,1) (BASELINE config 4)",
+        "config": {"workload": "long-context prefill B=8 H=16 L=2048 d=64 causal, q/k/v=0.5*N(0,1) (benchmark config 4)",
                    "flops_per_step": pre["flops"], "device": info["name"], "cu_count": info["cu_count"]},
         "roofline": {"bound": "mfma", "achieved": ach, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": ach / MFMA_FP32_PEAK_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
@@ -535,7 +535,7 @@ def main():
     }
     if dec:
         line["decode"] = {"workload": "incremental decode B=16 H=16 d=64, KV cache 4096 rows + 64 append+attend steps "
-                                      "(BASELINE config 5)",
+                                      "(benchmark config 5)",
                           "us_per_step": dec["us_per_step"], "tokens_per_s": dec["tokens_per_s"],
                           "single_step_us_p50": dec["single_step_us_p50"], "single_step_us_p99": dec["single_step_us_p99"],
                           "roofline": {"bound": "hbm", "achieved": dec["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -93,6 +93,12 @@ int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx) {
 
 int dl4s_hip_destroy(dl4s_hip_ctx *ctx) {
     DL4S_CHECK_CTX(ctx);
+    if (ctx->capturing) {   // an open recording is given up
+        hipGraph_t recorded = nullptr;
+        if (hipStreamEndCapture(ctx->stream, &recorded) == hipSuccess && recorded) (void)hipGraphDestroy(recorded);
+        (void)hipGetLastError();
+        ctx->capturing = false;
+    }
     (void)hipStreamSynchronize(ctx->stream);
     for (auto &kv : ctx->pool)
         for (void *p : kv.second) (void)hipFree(p);

@@ -71,7 +71,8 @@ int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms);
  * (DL4S_HIP_EUNSUPPORTED) and it has to be recorded again.  One recording at a time per context, made and replayed
  * from one host thread at a time.
  *
- * dl4s_hip_graph_end with out_graph == NULL gives the recording up. */
+ * dl4s_hip_graph_end with out_graph == NULL gives the recording up, and so does dl4s_hip_destroy.  Destroy a context's
+ * graphs before the context. */
 typedef struct dl4s_hip_graph dl4s_hip_graph;
 int dl4s_hip_graph_begin(dl4s_hip_ctx *ctx);
 int dl4s_hip_graph_end(dl4s_hip_ctx *ctx, dl4s_hip_graph **out_graph);

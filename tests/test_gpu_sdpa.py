@@ -237,7 +237,7 @@ def test_error_paths(ctx):
     bad.release()
 
 
-# ------------------------------------------------------------------ the BASELINE configurations
+# ------------------------------------------------------------------ the benchmark configurations
 def test_config1_sdpa_b1_h8_l128_d64(ctx, orc):
     rng = np.random.Generator(np.random.PCG64(1001))
     q, k, v = (rng.standard_normal((1, 8, 128, 64), dtype=np.float32) for _ in range(3))
