@@ -227,6 +227,21 @@ struct HIP {
                                         kind == DL4S_MASK_NONE ? nullptr : &md,
                                         (strictMasks() ? DL4S_SDPA_STRICT : 0u) | (tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u)));
         }
+        // one query row per (batch, head) over a key / value cache [B,H,Tcap,d]: q, result [B,H,1,d] (equally [B,1,H,d])
+        static void decodeAttention(const ShapedBuffer &q, const ShapedBuffer &keyCache, const ShapedBuffer &valueCache, int64_t rows,
+                                    const ShapedBuffer &result, float temperature) {
+            check(dl4s_hip_sdpa_decode_f32(context(), q.values.memory, keyCache.values.memory, valueCache.values.memory,
+                                           result.values.memory, keyCache.shape[0], keyCache.shape[1], rows, keyCache.shape[2],
+                                           keyCache.shape[3], 1.0f / temperature));
+        }
+        // the same after writing newKey, newValue [B,H,1,d] into row `position` of the caches (rows 0 ... position attended)
+        static void decodeAttentionAppending(const ShapedBuffer &q, const ShapedBuffer &keyCache, const ShapedBuffer &valueCache,
+                                             const ShapedBuffer &newKey, const ShapedBuffer &newValue, int64_t position,
+                                             const ShapedBuffer &result, float temperature) {
+            check(dl4s_hip_sdpa_decode_step_f32(context(), q.values.memory, keyCache.values.memory, valueCache.values.memory,
+                                                newKey.values.memory, newValue.values.memory, result.values.memory, keyCache.shape[0],
+                                                keyCache.shape[1], position, keyCache.shape[2], keyCache.shape[3], 1.0f / temperature));
+        }
         // result = act(x . weights + bias) + residual  (bias, residual optional)
         static void denseFused(const ShapedBuffer &x, const ShapedBuffer &weights, const ShapedBuffer *bias, int activation,
                                const ShapedBuffer *residual, const ShapedBuffer &result) {
@@ -801,6 +816,18 @@ struct MultiHeadAttention {
     Tensor qDense, kDense, vDense, fc;
     LayerNorm norm;
     Dropout dropout;
+    // Not in the reference.  false: the reference's normalisation, over (length, hidden) jointly, because the layer hands
+    // LayerNorm a 3-D tensor (MultiHeadAttention.swift:123-124, LayerNorm.swift:62-77).  true: every token normalised by
+    // itself (the input viewed as [batch * length, hidden], as PointwiseFeedForward.swift:68 does) - the conventional
+    // Transformer, whose output at a position does not depend on later positions, which cached decoding needs.
+    bool normalizesPerToken = false;
+    Tensor normalized(const Tensor &x, const Tensor *residual) const {
+        if (!normalizesPerToken || x.dim() != 3) return norm.normalize(x, residual);
+        const Shape flat{x.shape[0] * x.shape[1], x.shape[2]};
+        if (!residual) return norm.normalize(x.view(flat), nullptr).view(x.shape);
+        const Tensor r = residual->view(flat);
+        return norm.normalize(x.view(flat), &r).view(x.shape);
+    }
     MultiHeadAttention(int64_t heads_, int64_t hiddenDim_, int64_t keyDim_, int64_t valueDim_, float dropoutRate = 0.1f)
         : heads(heads_), keyDim(keyDim_), valueDim(valueDim_), hiddenDim(hiddenDim_), attn(std::sqrt((float)keyDim_)),
           qDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})), kDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})),
@@ -846,10 +873,48 @@ struct MultiHeadAttention {
             Tensor sum(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, hiddenDim}));
             const ShapedBuffer rb = q.values();
             Device::Engine::denseFused(a2.values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, sum.values());
-            return norm.normalize(sum, nullptr);
+            return normalized(sum, nullptr);
         }
         Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
-        return norm.normalize(out_drop, &q);
+        return normalized(out_drop, &q);
+    }
+    // ---- one new position against cached keys and values (no counterpart in the reference; fused mode, head dim 64,
+    // dropout inactive).  x [B,1,hidden].  With a single position the joint normalisation and the per-token one coincide.
+    bool canDecodeIncrementally() const { return canCacheProjections() && keyDim == 64 && !dropout.isActive; }
+    Tensor finishStep(const Tensor &x, const Tensor &attended) const {
+        const int64_t B = x.shape[0];
+        Tensor sum(Device::Memory::allocateBuffer(Shape{B, 1, hiddenDim}));
+        const ShapedBuffer rb = x.values();
+        Device::Engine::denseFused(attended.view({B, heads * valueDim}).values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, sum.values());
+        return norm.normalize(sum, nullptr);
+    }
+    // self-attention: projects x, writes its key / value row into row `position` of the caches [B,H,capacity,64], attends
+    // to rows 0 ... position
+    Tensor stepAppending(const Tensor &x, const Tensor &keyCache, const Tensor &valueCache, int64_t position) const {
+        precondition(canDecodeIncrementally() && x.dim() == 3 && x.shape[1] == 1 && x.shape[2] == hiddenDim && keyCache.dim() == 4 &&
+                         keyCache.shape == valueCache.shape && keyCache.shape[0] == x.shape[0] && keyCache.shape[1] == heads &&
+                         position >= 0 && position < keyCache.shape[2],
+                     "cached attention step: bad shapes");
+        const int64_t B = x.shape[0];
+        const Shape ps{B, heads, 1, keyDim};
+        Tensor qp(Device::Memory::allocateBuffer(ps)), kp(Device::Memory::allocateBuffer(ps)), vp(Device::Memory::allocateBuffer(ps));
+        Device::Engine::gemmGrouped({x.values(), x.values(), x.values()}, B, {qDense.values(), kDense.values(), vDense.values()},
+                                    {qp.values(), kp.values(), vp.values()});
+        Tensor a(Device::Memory::allocateBuffer(ps));
+        Device::Engine::decodeAttentionAppending(qp.values(), keyCache.values(), valueCache.values(), kp.values(), vp.values(), position,
+                                                 a.values(), attn.temperature);
+        return finishStep(x, a);
+    }
+    // attention to `rows` cached rows that do not change (the projected encoder states, head-major [B,H,rows,64])
+    Tensor stepAttending(const Tensor &x, const Tensor &keys, const Tensor &values) const {
+        precondition(canDecodeIncrementally() && x.dim() == 3 && x.shape[1] == 1 && x.shape[2] == hiddenDim && keys.dim() == 4 &&
+                         keys.shape == values.shape && keys.shape[0] == x.shape[0] && keys.shape[1] == heads && keys.shape[2] >= 1,
+                     "cached attention step: bad shapes");
+        const int64_t B = x.shape[0];
+        Tensor qp = x.view({B, hiddenDim}).matrixMultiplied(qDense);
+        Tensor a(Device::Memory::allocateBuffer(Shape{B, heads, 1, keyDim}));
+        Device::Engine::decodeAttention(qp.values(), keys.values(), values.values(), keys.shape[2], a.values(), attn.temperature);
+        return finishStep(x, a);
     }
     // self- or cross-attention with a structured mask (fused mode, head dims as for canCacheProjections)
     Tensor structured(const Tensor &q, const Tensor &k, const Tensor &v, const AttentionMask &mask) const {
@@ -875,9 +940,9 @@ struct MultiHeadAttention {
         Tensor q_attn = attn(q_trans, k_trans, v_trans, mask);
         Tensor out = q_attn.permuted({0, 2, 1, 3}).view({batchSize, queryCount, -1}).broadcastMatrixMultiplied(fc);
         Tensor out_drop = dropout(out);
-        if (Device::fused()) return norm.normalize(out_drop, &res);
+        if (Device::fused()) return normalized(out_drop, &res);
         Tensor q_res = out_drop + res;
-        return norm(q_res);
+        return normalized(q_res, nullptr);
     }
 };
 
@@ -938,6 +1003,13 @@ struct TransformerDecoderBlock {
                                 const Tensor &decoderMask) const {
         Tensor decAttn = selfAttention(decoderInput, decoderInput, decoderInput, &decoderMask);
         Tensor encAttn = encoderAttention.attendProjected(decAttn, encKeys, encValues, &encoderMask);
+        return pointwiseFeedForward(encAttn);
+    }
+    // one new position: decoderInput [B,1,hidden], self-attention caches [B,H,capacity,64], encoder keys / values [B,H,n,64]
+    Tensor step(const Tensor &decoderInput, const Tensor &keyCache, const Tensor &valueCache, int64_t position, const Tensor &encKeys,
+                const Tensor &encValues) const {
+        Tensor decAttn = selfAttention.stepAppending(decoderInput, keyCache, valueCache, position);
+        Tensor encAttn = encoderAttention.stepAttending(decAttn, encKeys, encValues);
         return pointwiseFeedForward(encAttn);
     }
     Tensor withProjectedEncoder(const Tensor &decoderInput, const Tensor &encKeys, const Tensor &encValues, const AttentionMask &encoderMask,
@@ -1127,6 +1199,62 @@ struct Transformer {
         Tensor decoded = decoder(prepareInputs(decoderInput, batchSize, decLen), encoderStates, encInLens, decInLens);
         Tensor deembedded = decoded.broadcastMatrixMultiplied(embedding.embeddingMatrix, false, true) + outputBias;
         return logSoftmax(deembedded, 2);
+    }
+
+    // every attention layer normalised per token (see MultiHeadAttention::normalizesPerToken; not in the reference)
+    void setNormalizesPerToken(bool perToken) {
+        for (auto &l : encoder.encoderLayers) l.selfAttention.normalizesPerToken = perToken;
+        for (auto &l : decoder.decoderLayers) l.selfAttention.normalizesPerToken = l.encoderAttention.normalizesPerToken = perToken;
+    }
+    bool canDecodeIncrementally() const {
+        if (!Device::fused() || decoder.decoderLayers.empty() || dropout.isActive) return false;
+        for (auto &l : decoder.decoderLayers)
+            if (!l.selfAttention.normalizesPerToken || !l.encoderAttention.normalizesPerToken || !l.selfAttention.canDecodeIncrementally() ||
+                !l.encoderAttention.canDecodeIncrementally() || l.pointwiseFeedForward.dropout.isActive)
+                return false;
+        return true;
+    }
+
+    // Greedy decoding with key / value caches: no counterpart in the reference, which re-runs the whole prefix at every
+    // step (greedy() below).  A step runs the decoder on the one new position: every layer appends the position's
+    // self-attention key / value row to its cache [1,H,maxLength,64] and attends to the rows so far, then to the encoder
+    // states' keys / values, projected once and stored head-major [1,H,n,64].  Only a model whose attention layers
+    // normalise per token computes the same function this way (the prefix re-run of such a model gives the same tokens and
+    // the same logits up to summation order): with the reference's joint normalisation every earlier position's output
+    // changes as the prefix grows, and the precondition refuses the model.
+    std::vector<int32_t> greedyCached(const std::vector<int32_t> &inputSequence, int32_t startToken, int32_t endToken, int64_t maxLength,
+                                      std::vector<float> *lastLogits = nullptr) const {
+        precondition(canDecodeIncrementally(),
+                     "cached decoding needs fused mode, inactive dropout, head dim 64 and attention layers that normalise per token");
+        const int64_t n = (int64_t)inputSequence.size(), D = embedding.outputSize();
+        std::vector<int32_t> tokens;
+        if (maxLength <= 0) return tokens;
+        Tensor encoded = encoder(prepareInputs(inputSequence, 1, n), {n});
+        struct LayerState { Tensor encKeys, encValues, keyCache, valueCache; };
+        std::vector<LayerState> state;
+        for (auto &l : decoder.decoderLayers) {
+            auto kv = l.encoderAttention.projectKeysValues(encoded, encoded);                       // [1,n,H,64]
+            const Shape cache{1, l.selfAttention.heads, maxLength, l.selfAttention.keyDim};
+            state.push_back({kv.first.permuted({0, 2, 1, 3}), kv.second.permuted({0, 2, 1, 3}),    // [1,H,n,64]
+                             Tensor(Device::Memory::allocateBuffer(cache)), Tensor(Device::Memory::allocateBuffer(cache))});
+        }
+        const Tensor positions = positionalEncoding(maxLength);
+        int32_t current = startToken;
+        for (int64_t step = 0; step < maxLength; ++step) {
+            const Tensor position = positions[{step}].view({1, D});
+            Tensor acc = prepareInputs({current}, 1, 1, &position);                                   // [1,1,hidden]
+            for (size_t i = 0; i < state.size(); ++i)
+                acc = decoder.decoderLayers[i].step(acc, state[i].keyCache, state[i].valueCache, step, state[i].encKeys, state[i].encValues);
+            Tensor last = acc.view({1, D}).matrixMultiplied(embedding.embeddingMatrix, false, true).view({-1});
+            if (lastLogits) {
+                const std::vector<float> row = last.elements();
+                lastLogits->insert(lastLogits->end(), row.begin(), row.end());
+            }
+            current = (int32_t)last.argmax();
+            tokens.push_back(current);
+            if (current == endToken) break;
+        }
+        return tokens;
     }
 
     // greedy decoding                                                                    (Transformer.swift:118-137)

@@ -226,22 +226,43 @@ int dl4s_host_transformer_forward(dl4s_hip_ctx *ctx, int fused, dl4s_host_transf
     });
 }
 
-int dl4s_host_transformer_greedy(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence, int64_t n,
-                                 int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens,
-                                 int64_t *out_count, float *out_logits, float *out_ms) {
+static int greedy_decode(dl4s_hip_ctx *ctx, int fused, bool cached, dl4s_host_transformer *t, const int32_t *input_sequence, int64_t n,
+                         int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens, int64_t *out_count,
+                         float *out_logits, float *out_ms) {
     return guarded(ctx, fused, [&] {
         precondition(t && input_sequence && out_tokens && out_count && n > 0 && max_length >= 0, "bad argument");
         std::vector<int32_t> in(input_sequence, input_sequence + n);
         std::vector<float> logits;
         HIP::check(dl4s_hip_sync(ctx));
         const auto t0 = std::chrono::steady_clock::now();
-        std::vector<int32_t> toks = t->model.greedy(in, start_token, end_token, max_length, out_logits ? &logits : nullptr);
+        std::vector<int32_t> toks = cached ? t->model.greedyCached(in, start_token, end_token, max_length, out_logits ? &logits : nullptr)
+                                           : t->model.greedy(in, start_token, end_token, max_length, out_logits ? &logits : nullptr);
         HIP::check(dl4s_hip_sync(ctx));
         if (out_ms) *out_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
         *out_count = (int64_t)toks.size();
         std::copy(toks.begin(), toks.end(), out_tokens);
         if (out_logits) std::copy(logits.begin(), logits.end(), out_logits);
     });
+}
+
+int dl4s_host_transformer_greedy(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence, int64_t n,
+                                 int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens,
+                                 int64_t *out_count, float *out_logits, float *out_ms) {
+    return greedy_decode(ctx, fused, false, t, input_sequence, n, start_token, end_token, max_length, out_tokens, out_count, out_logits,
+                         out_ms);
+}
+
+int dl4s_host_transformer_greedy_cached(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence,
+                                        int64_t n, int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens,
+                                        int64_t *out_count, float *out_logits, float *out_ms) {
+    return greedy_decode(ctx, fused, true, t, input_sequence, n, start_token, end_token, max_length, out_tokens, out_count, out_logits,
+                         out_ms);
+}
+
+int dl4s_host_transformer_set_norm_per_token(dl4s_host_transformer *t, int per_token) {
+    if (!t) return DL4S_HIP_EINVALID_ARG;
+    t->model.setNormalizesPerToken(per_token != 0);
+    return DL4S_HIP_OK;
 }
 
 int dl4s_host_positional_encoding(dl4s_hip_ctx *ctx, int fused, int64_t max_len, int64_t hidden, float *out) {

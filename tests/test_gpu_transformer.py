@@ -157,6 +157,57 @@ def test_greedy_decoding(ctx, name):
     model.close()
 
 
+def test_cached_greedy_decoding(ctx):
+    """Decoding with key / value caches (one new position per step through the decode kernels) against the oracle's
+    prefix re-run of the same model.  Only a model that normalises per token can be cached: the reference's joint
+    normalisation is refused, and the per-token model's uncached paths are checked against the oracle as well."""
+    from dl4s_amd import host_lib
+    from oracle import transformer as T
+    name = "head_dim_64"
+    vocab = CONFIGS[name][0]
+    params, rng = _model(47, *CONFIGS[name])
+    src = [int(t) for t in rng.integers(0, vocab, 11)]
+    steps = 12
+    ref_tokens, ref_logits = T.greedy_decode(params, src, 1, -5, steps, return_logits=True, norm_per_token=True)
+    assert len(ref_tokens) == steps
+    top2 = np.sort(np.stack(ref_logits), axis=1)[:, -2:]
+    assert (top2[:, 1] - top2[:, 0]).min() > 1e-3, "the fixture must not sit on an argmax tie"
+    model = host_lib.Transformer(ctx, params)
+    with pytest.raises(host_lib.HostError, match="normalise per token"):
+        model.greedy(src, 1, -5, steps, cached=True)
+    model.set_norm_per_token(True)
+    for fused in (True, False):                      # the prefix re-run of the per-token model
+        toks, logits = model.greedy(src, 1, -5, steps, fused=fused, return_logits=True)
+        assert toks == ref_tokens
+        assert_parity(logits, np.stack(ref_logits), "per-token greedy logits fused=%s" % fused)
+    toks, logits = model.greedy(src, 1, -5, steps, cached=True, return_logits=True)
+    assert toks == ref_tokens
+    assert_parity(logits, np.stack(ref_logits), "cached greedy logits")
+    # stops at the end token like the uncached loop
+    assert model.greedy(src, 1, ref_tokens[3], steps, cached=True) == ref_tokens[:ref_tokens.index(ref_tokens[3]) + 1]
+    assert model.greedy(src, 1, -5, 0, cached=True) == []
+    with pytest.raises(host_lib.HostError, match="fused mode"):
+        model.greedy(src, 1, -5, steps, fused=False, cached=True)
+    # forward pass of the per-token model, and back to the reference's normalisation
+    enc = np.array([src[:9], src[:5] + [-1] * 4], np.int32)
+    dec = np.array([[1, 4, 7, 9, 3, 2], [1, 5, -1, -1, -1, -1]], np.int32)
+    assert_parity(model.forward(enc, dec, [9, 5], [6, 2]), T.forward(params, enc, dec, [9, 5], [6, 2], norm_per_token=True),
+                  "per-token forward")
+    model.set_norm_per_token(False)
+    assert_parity(model.forward(enc, dec, [9, 5], [6, 2]), T.forward(params, enc, dec, [9, 5], [6, 2]), "joint forward")
+    model.close()
+
+
+def test_cached_decoding_needs_head_dim_64(ctx):
+    from dl4s_amd import host_lib
+    params, rng = _model(48, *CONFIGS["transformer_tests_hyperparameters"])
+    model = host_lib.Transformer(ctx, params)
+    model.set_norm_per_token(True)
+    with pytest.raises(host_lib.HostError, match="head dim 64"):
+        model.greedy([3, 4, 5], 1, 2, 4, cached=True)
+    model.close()
+
+
 def test_transformer_argument_errors(ctx):
     from dl4s_amd import host_lib
     params, rng = _model(44, *CONFIGS["transformer_tests_hyperparameters"])

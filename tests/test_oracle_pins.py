@@ -526,3 +526,32 @@ def test_sdpa_backward_against_finite_differences():
         args_m[idx] = args_m[idx] - eps * direction
         fd = (f(*args_p) - f(*args_m)) / (2 * eps)
         assert abs(fd - float((grad * direction).sum())) < 1e-4
+
+
+def test_per_token_attention_variant_of_the_transformer_oracle(orc):
+    """oracle.transformer.mha_per_token is not the reference's layer; it is pinned by two properties.  With a single
+    position the joint normalisation and the per-token one are the same computation (bit for bit against the pinned
+    layer).  And a decoder built from it is causal: its output at a position does not depend on later positions, bit for
+    bit - which the reference's jointly normalised decoder is not, the reason its decoding cannot be cached."""
+    from oracle import fp64_model as m64
+    from oracle import transformer as T
+    rng = np.random.default_rng(71)
+    params = m64.make_transformer_params(rng, 13, 16, 4, 8, 8, 32, 2, 2)
+    p = params["decoder"][0]["self"]
+    x = rng.standard_normal((3, 1, 16)).astype(np.float32)
+    kv = rng.standard_normal((3, 5, 16)).astype(np.float32)
+    assert np.array_equal(T.mha_per_token(x, kv, kv, None, p, 4, 8, 8), orc.mha(x, kv, kv, None, p, 4, 8, 8))
+    # several positions: each output row equals the jointly normalised layer applied to that row alone
+    xs = rng.standard_normal((2, 4, 16)).astype(np.float32)
+    whole = T.mha_per_token(xs, kv[:2], kv[:2], None, p, 4, 8, 8)
+    for i in range(4):
+        assert np.array_equal(whole[:, i:i + 1], orc.mha(xs[:, i:i + 1], kv[:2], kv[:2], None, p, 4, 8, 8))
+    src = [3, 4, 5, 6]
+    for per_token in (True, False):
+        enc = T.encoder(params, T.prepare_inputs(params, [src]), [4], per_token)
+        long = T.decoder(params, T.prepare_inputs(params, [[1, 3, 4, 5, 6]]), enc, [4], [5], per_token)
+        short = T.decoder(params, T.prepare_inputs(params, [[1, 3, 4]]), enc, [4], [3], per_token)
+        if per_token:
+            assert np.array_equal(long[:, :3], short)
+        else:
+            assert np.abs(long[:, :3] - short).max() > 1e-3
