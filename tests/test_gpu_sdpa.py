@@ -313,7 +313,8 @@ def run_decode(ctx, q, kc, vc, T):
     return out
 
 
-@pytest.mark.parametrize("B,H,T,Tcap", [(1, 1, 1, 1), (2, 3, 9, 12), (2, 2, 256, 256), (1, 4, 257, 300), (3, 2, 1000, 1024),
+@pytest.mark.parametrize("B,H,T,Tcap", [(1, 1, 1, 1), (2, 3, 9, 12), (2, 2, 128, 128), (2, 2, 129, 140), (2, 2, 256, 256),
+                                        (1, 4, 257, 300), (1, 8, 512, 512), (1, 8, 513, 600), (3, 2, 1000, 1024),
                                         (2, 2, 4097, 4160)])
 def test_decode_matches_oracle(ctx, orc, B, H, T, Tcap):
     rng = np.random.default_rng(T)
