@@ -774,8 +774,16 @@ struct Dense {
 struct AttentionMask {
     int kind = DL4S_MASK_NONE;
     Tensor lengths;   // device int32 [batchSize], viewed through a float buffer of the same byte size
-    static AttentionMask forLengths(const std::vector<int64_t> &sequenceLengths, bool causal) {
+    // keyCount: the padded length of the keys.  When no sequence is shorter the mask blocks nothing by length and the
+    // descriptor needs no lengths on the device (the kernels give the same bits for either description of a mask).
+    static AttentionMask forLengths(const std::vector<int64_t> &sequenceLengths, bool causal, int64_t keyCount) {
         AttentionMask m;
+        bool allFull = true;
+        for (int64_t v : sequenceLengths) allFull = allFull && v >= keyCount;
+        if (allFull) {
+            m.kind = causal ? DL4S_MASK_CAUSAL : DL4S_MASK_NONE;
+            return m;
+        }
         m.kind = causal ? DL4S_MASK_CAUSAL_OR_KEY_LENGTHS : DL4S_MASK_KEY_LENGTHS;
         std::vector<int32_t> l32(sequenceLengths.begin(), sequenceLengths.end());
         for (int32_t v : l32) precondition(v >= 0, "sequence lengths must not be negative");
@@ -783,7 +791,10 @@ struct AttentionMask {
         Device::check(dl4s_hip_assign_h2d(Device::context(), m.lengths.buffer().memory, l32.data(), l32.size() * sizeof(int32_t)));
         return m;
     }
-    const int32_t *lengthsPointer() const { return reinterpret_cast<const int32_t *>(lengths.buffer().memory); }
+    const int32_t *lengthsPointer() const {
+        const bool needed = kind == DL4S_MASK_KEY_LENGTHS || kind == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS;
+        return needed ? reinterpret_cast<const int32_t *>(lengths.buffer().memory) : nullptr;
+    }
 };
 
 // NN/Models/Transformer/ScaledDotProductAttention.swift:29-65
@@ -1106,7 +1117,7 @@ struct TransformerEncoder {
     Tensor operator()(const Tensor &input, const std::vector<int64_t> &sequenceLengths) const {
         Tensor acc = input;
         if (canUseStructuredMasks()) {      // fused mode: the mask as a descriptor, never materialised
-            const AttentionMask mask = AttentionMask::forLengths(sequenceLengths, false);
+            const AttentionMask mask = AttentionMask::forLengths(sequenceLengths, false, input.shape[1]);
             for (auto &layer : encoderLayers) acc = layer(acc, mask);
             return acc;
         }
@@ -1145,8 +1156,9 @@ struct TransformerDecoder {
     }
     Tensor withProjectedEncoder(const Tensor &decoderInput, const std::vector<std::pair<Tensor, Tensor>> &kv,
                                 const std::vector<int64_t> &encoderInputLengths, const std::vector<int64_t> &decoderInputLengths) const {
-        const AttentionMask encoderMask = AttentionMask::forLengths(encoderInputLengths, false);
-        const AttentionMask decoderMask = AttentionMask::forLengths(decoderInputLengths, true);
+        precondition(!kv.empty() && kv.size() == decoderLayers.size(), "one projected key / value pair per decoder layer");
+        const AttentionMask encoderMask = AttentionMask::forLengths(encoderInputLengths, false, kv[0].first.shape[1]);
+        const AttentionMask decoderMask = AttentionMask::forLengths(decoderInputLengths, true, decoderInput.shape[1]);
         Tensor acc = decoderInput;
         for (size_t i = 0; i < decoderLayers.size(); ++i)
             acc = decoderLayers[i].withProjectedEncoder(acc, kv[i].first, kv[i].second, encoderMask, decoderMask);
