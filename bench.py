@@ -319,7 +319,7 @@ def other_configs(ctx, lib, cpu, only=None):
             for b_ in qkv + [o]:
                 b_.release()
         dmask.release()
-    if want("greedy") or want("greedy_fused") or want("greedy_primitive") or want("greedy_cached"):
+    if want("greedy") or want("greedy_fused") or want("greedy_primitive") or want("greedy_cached") or want("greedy_cached_only"):
         # the caller of the blocks: Transformer greedy decoding (batch 1; every step re-runs the decoder on the prefix, as the
         # reference does).  6 + 6 layers, hidden 512, 8 heads of 64, ffn 2048, vocabulary 8000, 64 source tokens, 32 generated.
         rng = np.random.Generator(np.random.PCG64(1006))
@@ -335,6 +335,13 @@ def other_configs(ctx, lib, cpu, only=None):
             toks, ms = model.greedy(src, 1, -5, 32, fused=fused, timing=True)
             entry["ms_per_token_" + mode] = ms / len(toks)
             entry["tokens_per_s_" + mode] = len(toks) / ms * 1e3
+        if only is not None and "greedy_cached_only" in only:
+            # the cached decode of 512 tokens alone (for a kernel trace of just that loop)
+            model.set_norm_per_token(True)
+            model.greedy(src, 1, -5, 4, cached=True)
+            toks_c, ms_c = model.greedy(src, 1, -5, 512, cached=True, timing=True)
+            entry["per_token_normalisation"] = {"512_tokens": {"cached": ms_c / len(toks_c)}}
+            model.set_norm_per_token(False)
         if want("greedy") or want("greedy_cached"):
             # The same model with per-token normalisation in its attention layers (not the reference's model: its joint
             # normalisation cannot be cached), decoded by re-running the prefix and with key / value caches, 32 and 512 tokens.
@@ -344,8 +351,10 @@ def other_configs(ctx, lib, cpu, only=None):
             for count in (32, 512):
                 toks_r, ms_r = model.greedy(src, 1, -5, count, timing=True)
                 toks_c, ms_c = model.greedy(src, 1, -5, count, cached=True, timing=True)
-                per_token["%d_tokens" % count] = {"prefix_rerun": ms_r / len(toks_r), "cached": ms_c / len(toks_c),
-                                                  "same_tokens": toks_r == toks_c}
+                toks_s, ms_s = model.greedy(src, 1, -5, count, cached="stepwise", timing=True)
+                per_token["%d_tokens" % count] = {"prefix_rerun": ms_r / len(toks_r), "cached_step_recorded_and_replayed": ms_c / len(toks_c),
+                                                  "cached_calls_issued_one_by_one": ms_s / len(toks_s),
+                                                  "same_tokens": toks_r == toks_c == toks_s}
             entry["per_token_normalisation"] = per_token
             model.set_norm_per_token(False)
         model.close()
@@ -492,7 +501,7 @@ def main():
                          "profiler counter runs")
     ap.add_argument("--only", default="", metavar="NAMES",
                     help="instead of the benchmark, run only these of the workloads reported beside the headline (comma "
-                         "separated: config1, config2, recorded, config3, backward, masks_and_head_dim, greedy, greedy_fused, greedy_primitive, greedy_cached) and print their entries: "
+                         "separated: config1, config2, recorded, config3, backward, masks_and_head_dim, greedy, greedy_fused, greedy_primitive, greedy_cached, greedy_cached_only) and print their entries: "
                          "short commands for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -35,6 +35,11 @@ struct dl4s_hip_ctx {
     // regrowths of the scratch block; a captured graph holds the block's address and is refused once it has moved.
     bool capturing = false;
     unsigned long long scratch_generation = 0;
+    // Blocks handed back with dl4s_hip_free while a graph is being recorded: the recorded kernels still use them on every
+    // replay, so they stay out of the pool until the graph is destroyed (dl4s_hip_graph_end moves the list to the graph).
+    // Allocations made later in the same recording may take them.
+    std::vector<std::pair<void *, size_t>> held_by_recording;
+    size_t bytes_held = 0;
 };
 
 struct dl4s_hip_graph {
@@ -43,6 +48,7 @@ struct dl4s_hip_graph {
     dl4s_hip_ctx *owner = nullptr;
     size_t nodes = 0;
     unsigned long long scratch_generation = 0;
+    std::vector<std::pair<void *, size_t>> held;   // temporaries freed during the recording, returned to the pool on destroy
 };
 
 namespace dl4s {

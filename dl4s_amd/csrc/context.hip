@@ -100,6 +100,7 @@ int dl4s_hip_destroy(dl4s_hip_ctx *ctx) {
         ctx->capturing = false;
     }
     (void)hipStreamSynchronize(ctx->stream);
+    for (auto &b : ctx->held_by_recording) (void)hipFree(b.first);
     for (auto &kv : ctx->pool)
         for (void *p : kv.second) (void)hipFree(p);
     for (auto &kv : ctx->live) (void)hipFree(reinterpret_cast<void *>(kv.first));
@@ -143,6 +144,16 @@ int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms) {
     return DL4S_HIP_OK;
 }
 
+static void release_held(dl4s_hip_ctx *ctx, std::vector<std::pair<void *, size_t>> &held) {
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    for (auto &b : held) {
+        ctx->pool[b.second].push_back(b.first);
+        ctx->bytes_pooled += b.second;
+        ctx->bytes_held -= b.second;
+    }
+    held.clear();
+}
+
 int dl4s_hip_graph_begin(dl4s_hip_ctx *ctx) {
     DL4S_CHECK_CTX(ctx);
     DL4S_REQUIRE(!ctx->capturing, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_begin: a graph is being recorded already");
@@ -158,14 +169,22 @@ int dl4s_hip_graph_end(dl4s_hip_ctx *ctx, dl4s_hip_graph **out_graph) {
     DL4S_REQUIRE(ctx->capturing, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_end: no graph is being recorded");
     ctx->capturing = false;
     hipGraph_t recorded = nullptr;
-    DL4S_HIP_TRY(hipStreamEndCapture(ctx->stream, &recorded));
+    {
+        const hipError_t e = hipStreamEndCapture(ctx->stream, &recorded);
+        if (e != hipSuccess) {
+            release_held(ctx, ctx->held_by_recording);
+            return hip_error(e, "hipStreamEndCapture");
+        }
+    }
     if (!out_graph) {  // the caller gives the recording up
         if (recorded) (void)hipGraphDestroy(recorded);
+        release_held(ctx, ctx->held_by_recording);
         return DL4S_HIP_OK;
     }
     dl4s_hip_graph *g = new (std::nothrow) dl4s_hip_graph();
     if (!g) {
         (void)hipGraphDestroy(recorded);
+        release_held(ctx, ctx->held_by_recording);
         return set_error(DL4S_HIP_EOOM, "dl4s_hip_graph_end: host allocation failed");
     }
     g->graph = recorded;
@@ -173,7 +192,12 @@ int dl4s_hip_graph_end(dl4s_hip_ctx *ctx, dl4s_hip_graph **out_graph) {
     if (e != hipSuccess) {
         (void)hipGraphDestroy(recorded);
         delete g;
+        release_held(ctx, ctx->held_by_recording);
         return hip_error(e, "hipGraphInstantiate");
+    }
+    {
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        g->held.swap(ctx->held_by_recording);
     }
     size_t nodes = 0;
     (void)hipGraphGetNodes(recorded, nullptr, &nodes);
@@ -219,6 +243,7 @@ int dl4s_hip_graph_destroy(dl4s_hip_ctx *ctx, dl4s_hip_graph *graph) {
     DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
     (void)hipGraphExecDestroy(graph->exec);
     (void)hipGraphDestroy(graph->graph);
+    release_held(ctx, graph->held);
     delete graph;
     return DL4S_HIP_OK;
 }
@@ -231,7 +256,18 @@ int dl4s_hip_alloc(dl4s_hip_ctx *ctx, size_t bytes, void **out_ptr) {
     std::lock_guard<std::mutex> g(ctx->mu);
     void *p = nullptr;
     auto it = ctx->pool.find(sz);
-    if (it != ctx->pool.end() && !it->second.empty()) {
+    // While recording, a block freed earlier in the same recording is taken first: inside one graph the recorded calls run
+    // in order, so such reuse is as safe as it is between calls issued one by one.
+    auto held = ctx->held_by_recording.end();
+    if (ctx->capturing)
+        for (auto h = ctx->held_by_recording.begin(); h != ctx->held_by_recording.end(); ++h)
+            if (h->second == sz) { held = h; break; }
+    if (held != ctx->held_by_recording.end()) {
+        p = held->first;
+        ctx->bytes_held -= sz;
+        *held = ctx->held_by_recording.back();
+        ctx->held_by_recording.pop_back();
+    } else if (it != ctx->pool.end() && !it->second.empty()) {
         p = it->second.back();
         it->second.pop_back();
         ctx->bytes_pooled -= sz;
@@ -269,6 +305,11 @@ int dl4s_hip_free(dl4s_hip_ctx *ctx, void *ptr) {
     size_t sz = it->second;
     ctx->live.erase(it);
     ctx->bytes_in_use -= sz;
+    if (ctx->capturing) {   // the recorded kernels use the block on every replay: not reusable before the graph is gone
+        ctx->held_by_recording.emplace_back(ptr, sz);
+        ctx->bytes_held += sz;
+        return DL4S_HIP_OK;
+    }
     ctx->pool[sz].push_back(ptr);
     ctx->bytes_pooled += sz;
     return DL4S_HIP_OK;

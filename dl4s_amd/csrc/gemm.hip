@@ -447,6 +447,98 @@ __global__ __launch_bounds__(64 * SKW) void gemm_f32_skinny(GemmArgs g, float *_
     }
 }
 
+// The same for products of at most 16 rows (a single token of cached decoding, the first steps of a prefix re-run): a
+// workgroup owns a 16 x 16 output block and contracts with v_mfma_f32_16x16x4_f32.  A 32 x 32 block costs K/2 MFMAs of 64
+// cycles whatever the row count - 4096 cycles per SIMD at K = 512, 1.7 us of the 5 us such a launch takes - and leaves
+// N/32 workgroups; here the block costs K/4 MFMAs of 32 cycles (1024 cycles per SIMD) on N/16 workgroups.
+// One block = 16 of K: the 16-lane group q of a wavefront contracts k = kb + 4q .. kb + 4q + 3.
+template <bool TB>
+__global__ __launch_bounds__(64 * SKW) void gemm_f32_skinny16(GemmArgs g, float *__restrict__ part, int kslice, int nbn, int S) {
+    __shared__ float red[SKW][16][16];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, q = lane >> 4, ln = lane & 15;
+    const int cb = blockIdx.x % nbn, rb = blockIdx.x / nbn, s = blockIdx.y, z = blockIdx.z;
+    const float *A = g.A + (g.groups ? g.a_off[z] : (long long)z * g.a_bs);
+    const float *B = g.B + (g.groups ? g.b_off[z] : (long long)z * g.b_bs);
+    const int m = rb * 16 + ln, n = cb * 16 + ln;
+    const int share = kslice / SKW;   // a multiple of 16
+    const int k_begin = s * kslice + wave * share;
+    const int k_end = min(g.K, k_begin + share);
+    const float *arow = A + (long long)min(m, g.M - 1) * g.lda;
+    const int nc = min(n, g.N - 1);   // rows >= M and columns >= N compute on clamped addresses and are never stored
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    constexpr int SKU = 2;
+    const int nblk = (k_end - k_begin + 15) / 16;
+    if (nblk > 0) {
+        auto fetch = [&](const int blk, f32x4 &a, f32x4 &b) {
+            const int kb = k_begin + 16 * min(blk, nblk - 1);
+            int k0 = kb + 4 * q;
+            if (k0 >= k_end) k0 = kb;
+            a = *reinterpret_cast<const f32x4 *>(arow + k0);
+            if (TB) {
+                b = *reinterpret_cast<const f32x4 *>(B + (long long)nc * g.ldb + k0);
+            } else {
+                const float *bp = B + (long long)k0 * g.ldb + nc;
+                b.x = bp[0]; b.y = bp[g.ldb]; b.z = bp[2 * g.ldb]; b.w = bp[3 * g.ldb];
+            }
+        };
+        auto contract = [&](const int base, const f32x4 (&a)[SKU], const f32x4 (&b)[SKU]) {
+#pragma unroll
+            for (int u = 0; u < SKU; ++u) {
+                // blocks past the end contribute nothing (both operands zeroed: the clamped loads hold real data)
+                const bool ok = base + u < nblk && k_begin + 16 * (base + u) + 4 * q < k_end;
+                const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                const f32x4 av = ok ? a[u] : zero, bv = ok ? b[u] : zero;
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, bv.x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, bv.y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, bv.z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, bv.w, acc, 0, 0, 0);
+            }
+        };
+        f32x4 a0[SKU], b0[SKU], a1[SKU], b1[SKU];
+#pragma unroll
+        for (int u = 0; u < SKU; ++u) fetch(u, a0[u], b0[u]);
+        for (int base = 0; base < nblk; base += 2 * SKU) {
+            if (base + SKU < nblk) {
+#pragma unroll
+                for (int u = 0; u < SKU; ++u) fetch(base + SKU + u, a1[u], b1[u]);
+            }
+            contract(base, a0, b0);
+            if (base + 2 * SKU < nblk) {
+#pragma unroll
+                for (int u = 0; u < SKU; ++u) fetch(base + 2 * SKU + u, a0[u], b0[u]);
+            }
+            if (base + SKU < nblk) contract(base + SKU, a1, b1);
+        }
+    }
+    // accumulator register r: row 4*q + r, column ln
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][4 * q + r][ln] = acc[r];
+    __syncthreads();
+    if (tid < 256) {
+        const int row = tid >> 4, col = tid & 15;
+        const int gm = rb * 16 + row, gn = cb * 16 + col;
+        if (gm < g.M && gn < g.N) {
+            float sum = red[0][row][col];
+#pragma unroll
+            for (int w = 1; w < SKW; ++w) sum += red[w][row][col];
+            const long long c_at = g.groups ? g.c_off[z] : (long long)z * g.c_bs;
+            const long long at = (long long)gm * g.N + gn;
+            if (part) {
+                part[((long long)z * S + s) * g.M * g.N + at] = sum;
+            } else {
+                float *cp = g.C + c_at + at;
+                float val = g.alpha * sum;
+                if (g.beta != 0.f) val = val + g.beta * (*cp);
+                if (g.bias) val = __fadd_rn(val, g.bias[gn]);
+                if (g.act == 1) val = gelu_sigmoid(val);
+                if (g.residual) val = __fadd_rn(val, g.residual[c_at + at]);
+                *cp = val;
+            }
+        }
+    }
+}
+
+
 __global__ __launch_bounds__(256) void gemm_f32_skinny_finish(GemmArgs g, const float *__restrict__ part, int S) {
     const long long mn = (long long)g.M * g.N;
     const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -529,28 +621,43 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
                         (tb ? rows_by_k_any(rc) : true) && aligned16(lhs) && (!tb || aligned16(rhs)) && lbs % 4 == 0 &&
                         (!tb || rbs % 4 == 0) && group_aligned && M * N * batch < (1ll << 31) && K * (tb ? 1 : rc) < (1ll << 31);
     if (skinny) {
-        const int nbn = (int)((N + 31) / 32), nbm = (int)((M + 31) / 32);
+        // 16 x 16 output blocks (gemm_f32_skinny16) for up to 16 rows, and beyond for an unsliced K while that grid stays
+        // within two workgroups per CU ([32,512].[512,512] 5.7 -> 3.7 us, [128,512].[512,512] 5.8 -> 4.0 us,
+        // [64,1024].[1024,1024] 10.6 -> 6.4 us); else 32 x 32 blocks ([32,512].[8000,512]^T: 8.5 us, against 11.3 us on a
+        // thousand 16 x 16 blocks that read the weights twice; [96,2048].[2048,512] in slices: 9.5 against 12.8 us)
+        const bool rows16 = M <= 16 || (K <= 1024 && ((M + 15) / 16) * ((N + 15) / 16) <= 2 * ctx->cu_count);
+        const int blk = rows16 ? 16 : 32;
+        const int nbn = (int)((N + blk - 1) / blk), nbm = (int)((M + blk - 1) / blk);
         // One slice up to K = 1024; beyond, slices of 512 (one batch of loads per wavefront), since a single workgroup per
         // column block pulls a long K through one CU: M16 N512 K2048 8.9 us against 15.3 us unsliced, K4096 8.9 against
         // 26.9.  The slicing depends on K alone, so a product gets the same summation order alone, batched and grouped.
-        const int unit = 8 * SKW;
+        const int unit = (rows16 ? 16 : 8) * SKW;
         // (not more slices than it takes to give every CU two workgroups: with many column blocks the launch is wide
         // enough already, and a workgroup that lives for a single batch of loads spends its time starting and finishing)
         const long long want = (2ll * ctx->cu_count + (long long)nbn * nbm - 1) / ((long long)nbn * nbm);
         const long long S = K <= 1024 ? 1 : std::max(1ll, std::min((long long)((K + 511) / 512), want));
         const int kslice = (int)((((K + S - 1) / S) + unit - 1) / unit * unit);
         const dim3 pgrid((unsigned)(nbn * nbm), (unsigned)S, (unsigned)batch);
+        const auto launch = [&](float *partials) {
+            const int variant = (rows16 ? 2 : 0) | (tb ? 1 : 0);
+#define DL4S_SKINNY(KERNEL) hipLaunchKernelGGL(KERNEL, pgrid, dim3(64 * SKW), 0, ctx->stream, g, partials, kslice, nbn, (int)S)
+            switch (variant) {
+                case 0: DL4S_SKINNY(gemm_f32_skinny<false>); break;
+                case 1: DL4S_SKINNY(gemm_f32_skinny<true>); break;
+                case 2: DL4S_SKINNY(gemm_f32_skinny16<false>); break;
+                default: DL4S_SKINNY(gemm_f32_skinny16<true>); break;
+            }
+#undef DL4S_SKINNY
+        };
         if (S == 1) {
-            if (tb) hipLaunchKernelGGL(gemm_f32_skinny<true>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, (float *)nullptr, kslice, nbn, 1);
-            else hipLaunchKernelGGL(gemm_f32_skinny<false>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, (float *)nullptr, kslice, nbn, 1);
+            launch(nullptr);
             return dl4s::launch_status("gemm_f32_skinny");
         }
         std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
         const int rc_s = dl4s::ensure_scratch(ctx, (size_t)(batch * S * M * N) * sizeof(float));
         if (rc_s != DL4S_HIP_OK) return rc_s;
         float *part = static_cast<float *>(ctx->scratch);
-        if (tb) hipLaunchKernelGGL(gemm_f32_skinny<true>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, part, kslice, nbn, (int)S);
-        else hipLaunchKernelGGL(gemm_f32_skinny<false>, pgrid, dim3(64 * SKW), 0, ctx->stream, g, part, kslice, nbn, (int)S);
+        launch(part);
         hipLaunchKernelGGL(gemm_f32_skinny_finish, dim3((unsigned)((M * N + 255) / 256), 1, (unsigned)batch), dim3(256), 0, ctx->stream, g,
                            part, (int)S);
         return dl4s::launch_status("gemm_f32_skinny");

@@ -376,7 +376,10 @@ __global__ void stack_f32(StackSrc src, float *__restrict__ dst, long long count
 
 // First index of the largest value, scanning like `if v > maxV` from (-inf, index 0): NaN is never selected, ties keep
 // the earliest index (Engine/CPU/Numeric/CPUFloat.swift:294-318, generic branch).  One workgroup; out = {value, index}.
-__global__ __launch_bounds__(1024) void argmax_f32(const float *__restrict__ x, long long n, float *out_value, long long *out_index) {
+// out_token / counter (either may be NULL): the index as int32 and a counter advanced by one, both in device memory, for
+// decoding loops that keep the chosen token and the position on the device
+__global__ __launch_bounds__(1024) void argmax_f32(const float *__restrict__ x, long long n, float *out_value, long long *out_index,
+                                                   int *out_token = nullptr, int *counter = nullptr) {
     __shared__ float sv[1024];
     __shared__ long long si[1024];
     float bv = -INFINITY;
@@ -401,7 +404,27 @@ __global__ __launch_bounds__(1024) void argmax_f32(const float *__restrict__ x, 
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) { *out_value = sv[0]; *out_index = si[0]; }
+    if (threadIdx.x == 0) {
+        if (out_value) *out_value = sv[0];
+        if (out_index) *out_index = si[0];
+        if (out_token) *out_token = (int)si[0];
+        if (counter) *counter += 1;
+    }
+}
+
+// One token whose id and position are in device memory: out[c] = table[token][c] * scale + pos[position][c].  A token
+// outside [0, vocab) (the ignore index included) embeds as zeros; a position outside [0, pos_rows) adds nothing.
+__global__ void embed_at_f32(const float *__restrict__ table, const int *__restrict__ token_dev, const float *__restrict__ pos,
+                             const int *__restrict__ position_dev, float *__restrict__ out, long long vocab, long long D, long long pos_rows,
+                             float scale, int has_scale) {
+    const int tok = *token_dev;
+    const int at = position_dev ? *position_dev : 0;
+    for (long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x; c < D; c += (long long)gridDim.x * blockDim.x) {
+        float v = (tok >= 0 && tok < vocab) ? table[(long long)tok * D + c] : 0.0f;
+        if (has_scale) v = __fmul_rn(v, scale);
+        if (pos && at >= 0 && at < pos_rows) v = __fadd_rn(v, pos[(long long)at * D + c]);
+        out[c] = v;
+    }
 }
 
 // Embedding lookup with the scale and positional term of Transformer.prepareInputs folded in:
@@ -716,6 +739,27 @@ int dl4s_hip_argmax_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, i
     *out_index = host.i;
     *out_value = host.v;
     return DL4S_HIP_OK;
+}
+
+int dl4s_hip_argmax_to_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, int32_t *out_index_dev, int32_t *counter_dev) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(values && out_index_dev && count > 0 && count < (1ll << 31), DL4S_HIP_EINVALID_ARG,
+                 "argmax_to: NULL pointer or count outside [1, 2^31)");
+    hipLaunchKernelGGL(argmax_f32, dim3(1), dim3(1024), 0, ctx->stream, values, (long long)count, (float *)nullptr, (long long *)nullptr,
+                       out_index_dev, counter_dev);
+    return dl4s::launch_status("argmax_to");
+}
+
+int dl4s_hip_embed_at_f32(dl4s_hip_ctx *ctx, const float *table, int64_t vocab, int64_t D, const int32_t *token_dev,
+                          const float *scale, const float *positions, int64_t position_rows, const int32_t *position_dev,
+                          float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(vocab >= 0 && D >= 0 && position_rows >= 0, DL4S_HIP_EINVALID_ARG, "embed_at: negative extent");
+    if (D == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(table && token_dev && result && (!positions || position_dev), DL4S_HIP_EINVALID_ARG, "embed_at: NULL pointer");
+    hipLaunchKernelGGL(embed_at_f32, dim3(grid_for(D)), dim3(TPB), 0, ctx->stream, table, token_dev, positions, position_dev, result,
+                       (long long)vocab, (long long)D, (long long)position_rows, scale ? *scale : 1.0f, scale ? 1 : 0);
+    return dl4s::launch_status("embed_at");
 }
 
 int dl4s_hip_embed_positions_f32(dl4s_hip_ctx *ctx, const float *table, int64_t vocab, int64_t D, const int32_t *tokens,

@@ -43,14 +43,22 @@ __device__ __forceinline__ float row16_sum(float x) {
 // [split*chunk, split*chunk + chunk) round-robin.  Inside a wavefront each 16-lane group keeps its own running
 // (max, sum, 4 output columns per lane), so the loop has no cross-lane traffic beyond the 16-lane dot-product
 // reduction; groups, wavefronts and (through the scratch records) workgroups are merged once at the end.
-template <bool APPEND, int NW>
+// DEVPOS: the row to append comes from device memory (*pos_dev) and T = row + 1, for callers that replay one recorded
+// step at successive positions; a value outside [0, Tcap) leaves caches and output untouched.
+template <bool APPEND, int NW, bool DEVPOS = false>
 __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
                                                                    float *vcache, const float *__restrict__ k_new,
                                                                    const float *__restrict__ v_new,
                                                                    float *__restrict__ out, float *part, int T, int Tcap,
-                                                                   int pos, float rT, int nsplit, int chunk) {
+                                                                   int pos, float rT, int nsplit, int chunk,
+                                                                   const int *__restrict__ pos_dev = nullptr) {
     __shared__ float sm_o[NW][HD];
     __shared__ float sm_m[NW], sm_l[NW];
+    if (DEVPOS) {
+        pos = *pos_dev;
+        if (pos < 0 || pos >= Tcap) return;   // uniform over the grid
+        T = pos + 1;
+    }
     const int split = blockIdx.x;
     const int bh = blockIdx.y;
     const int tid = threadIdx.x;
@@ -279,6 +287,24 @@ int dl4s_hip_sdpa_decode_step_f32(dl4s_hip_ctx *ctx, const float *q, float *kcac
     DL4S_REQUIRE(pos >= 0 && pos < Tcap, DL4S_HIP_ESHAPE, "sdpa_decode_step: row %lld outside the cache capacity %lld",
                  (long long)pos, (long long)Tcap);
     return decode_launch(ctx, q, kcache, vcache, k_new, v_new, out, B, H, pos + 1, Tcap, pos, d, inv_temperature, true);
+}
+
+int dl4s_hip_sdpa_decode_step_at_f32(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcache, const float *k_new,
+                                     const float *v_new, float *out, int64_t B, int64_t H, const int32_t *pos_dev, int64_t Tcap,
+                                     int64_t d, float inv_temperature) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(B >= 0 && H >= 0, DL4S_HIP_EINVALID_ARG, "sdpa_decode_step_at: negative extent");
+    const int64_t BH = B * H;
+    if (BH == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(q && kcache && vcache && out && k_new && v_new && pos_dev, DL4S_HIP_EINVALID_ARG, "sdpa_decode_step_at: NULL pointer");
+    DL4S_REQUIRE(d == HD, DL4S_HIP_EUNSUPPORTED, "sdpa_decode_step_at: head dim %lld (only 64 is implemented)", (long long)d);
+    DL4S_REQUIRE(Tcap >= 1 && Tcap < (1ll << 30) && BH <= 65535, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa_decode_step_at: capacity %lld or B*H=%lld out of range", (long long)Tcap, (long long)BH);
+    // the row count is not known on the host: one workgroup of 16 wavefronts per pair walks whatever rows there are
+    const int chunk = (int)((Tcap + KB - 1) / KB * KB);
+    hipLaunchKernelGGL((sdpa_decode_splitk_f32<true, 16, true>), dim3(1, (unsigned)BH), dim3(16 * 64), 0, ctx->stream, q, kcache, vcache,
+                       k_new, v_new, out, (float *)nullptr, 0, (int)Tcap, 0, inv_temperature, 1, chunk, pos_dev);
+    return dl4s::launch_status("sdpa_decode_splitk_f32");
 }
 
 }  // extern "C"

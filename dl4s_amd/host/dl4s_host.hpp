@@ -242,6 +242,25 @@ struct HIP {
                                                 newKey.values.memory, newValue.values.memory, result.values.memory, keyCache.shape[0],
                                                 keyCache.shape[1], position, keyCache.shape[2], keyCache.shape[3], 1.0f / temperature));
         }
+        // the same with the row position read from device memory (a step that is recorded once and replayed)
+        static void decodeAttentionAppendingAt(const ShapedBuffer &q, const ShapedBuffer &keyCache, const ShapedBuffer &valueCache,
+                                               const ShapedBuffer &newKey, const ShapedBuffer &newValue, const int32_t *positionOnDevice,
+                                               const ShapedBuffer &result, float temperature) {
+            check(dl4s_hip_sdpa_decode_step_at_f32(context(), q.values.memory, keyCache.values.memory, valueCache.values.memory,
+                                                   newKey.values.memory, newValue.values.memory, result.values.memory, keyCache.shape[0],
+                                                   keyCache.shape[1], positionOnDevice, keyCache.shape[2], keyCache.shape[3],
+                                                   1.0f / temperature));
+        }
+        // result[D] = table[*token] * scale + positions[*position], token and position in device memory
+        static void embedAt(const ShapedBuffer &table, const int32_t *tokenOnDevice, const float *scale, const ShapedBuffer &positions,
+                            const int32_t *positionOnDevice, const ShapedBuffer &result) {
+            check(dl4s_hip_embed_at_f32(context(), table.values.memory, table.shape[0], table.shape[1], tokenOnDevice, scale,
+                                        positions.values.memory, positions.shape[0], positionOnDevice, result.values.memory));
+        }
+        // *tokenOnDevice = argmax(values); *counterOnDevice += 1
+        static void argmaxTo(const ShapedBuffer &values, int32_t *tokenOnDevice, int32_t *counterOnDevice) {
+            check(dl4s_hip_argmax_to_f32(context(), values.values.memory, values.count(), tokenOnDevice, counterOnDevice));
+        }
         // result = act(x . weights + bias) + residual  (bias, residual optional)
         static void denseFused(const ShapedBuffer &x, const ShapedBuffer &weights, const ShapedBuffer *bias, int activation,
                                const ShapedBuffer *residual, const ShapedBuffer &result) {
@@ -296,6 +315,41 @@ struct HIP {
 };
 
 using Device = HIP;
+
+// A sequence of engine calls recorded into a HIP graph (dl4s_hip_graph_*; no counterpart in the reference).  Tensors
+// created and released inside the recorded function stay reserved for the graph until it is destroyed.
+class RecordedCalls {
+    dl4s_hip_graph *graph_ = nullptr;
+    dl4s_hip_ctx *ctx_ = nullptr;
+
+   public:
+    RecordedCalls() = default;
+    RecordedCalls(const RecordedCalls &) = delete;
+    RecordedCalls &operator=(const RecordedCalls &) = delete;
+    ~RecordedCalls() { reset(); }
+    explicit operator bool() const { return graph_ != nullptr; }
+    void reset() {
+        if (graph_) (void)dl4s_hip_graph_destroy(ctx_, graph_);
+        graph_ = nullptr;
+    }
+    template <class F>
+    void record(F &&calls) {
+        reset();
+        ctx_ = Device::context();
+        Device::check(dl4s_hip_graph_begin(ctx_));
+        try {
+            calls();
+        } catch (...) {
+            (void)dl4s_hip_graph_end(ctx_, nullptr);
+            throw;
+        }
+        Device::check(dl4s_hip_graph_end(ctx_, &graph_));
+    }
+    void replay() const {
+        precondition(graph_ != nullptr, "nothing recorded");
+        Device::check(dl4s_hip_graph_launch(ctx_, graph_));
+    }
+};
 
 // ------------------------------------------------------------------------- Tensor.swift
 // Owns a buffer; a handle with a parent is a view into the parent's allocation and frees nothing
@@ -901,10 +955,12 @@ struct MultiHeadAttention {
     }
     // self-attention: projects x, writes its key / value row into row `position` of the caches [B,H,capacity,64], attends
     // to rows 0 ... position
-    Tensor stepAppending(const Tensor &x, const Tensor &keyCache, const Tensor &valueCache, int64_t position) const {
+    // (positionOnDevice != nullptr: the row index is read from device memory instead, see Transformer::greedyCached)
+    Tensor stepAppending(const Tensor &x, const Tensor &keyCache, const Tensor &valueCache, int64_t position,
+                         const int32_t *positionOnDevice = nullptr) const {
         precondition(canDecodeIncrementally() && x.dim() == 3 && x.shape[1] == 1 && x.shape[2] == hiddenDim && keyCache.dim() == 4 &&
                          keyCache.shape == valueCache.shape && keyCache.shape[0] == x.shape[0] && keyCache.shape[1] == heads &&
-                         position >= 0 && position < keyCache.shape[2],
+                         (positionOnDevice || (position >= 0 && position < keyCache.shape[2])),
                      "cached attention step: bad shapes");
         const int64_t B = x.shape[0];
         const Shape ps{B, heads, 1, keyDim};
@@ -912,8 +968,12 @@ struct MultiHeadAttention {
         Device::Engine::gemmGrouped({x.values(), x.values(), x.values()}, B, {qDense.values(), kDense.values(), vDense.values()},
                                     {qp.values(), kp.values(), vp.values()});
         Tensor a(Device::Memory::allocateBuffer(ps));
-        Device::Engine::decodeAttentionAppending(qp.values(), keyCache.values(), valueCache.values(), kp.values(), vp.values(), position,
-                                                 a.values(), attn.temperature);
+        if (positionOnDevice)
+            Device::Engine::decodeAttentionAppendingAt(qp.values(), keyCache.values(), valueCache.values(), kp.values(), vp.values(),
+                                                       positionOnDevice, a.values(), attn.temperature);
+        else
+            Device::Engine::decodeAttentionAppending(qp.values(), keyCache.values(), valueCache.values(), kp.values(), vp.values(), position,
+                                                     a.values(), attn.temperature);
         return finishStep(x, a);
     }
     // attention to `rows` cached rows that do not change (the projected encoder states, head-major [B,H,rows,64])
@@ -1018,8 +1078,8 @@ struct TransformerDecoderBlock {
     }
     // one new position: decoderInput [B,1,hidden], self-attention caches [B,H,capacity,64], encoder keys / values [B,H,n,64]
     Tensor step(const Tensor &decoderInput, const Tensor &keyCache, const Tensor &valueCache, int64_t position, const Tensor &encKeys,
-                const Tensor &encValues) const {
-        Tensor decAttn = selfAttention.stepAppending(decoderInput, keyCache, valueCache, position);
+                const Tensor &encValues, const int32_t *positionOnDevice = nullptr) const {
+        Tensor decAttn = selfAttention.stepAppending(decoderInput, keyCache, valueCache, position, positionOnDevice);
         Tensor encAttn = encoderAttention.stepAttending(decAttn, encKeys, encValues);
         return pointwiseFeedForward(encAttn);
     }
@@ -1235,10 +1295,11 @@ struct Transformer {
     // the same logits up to summation order): with the reference's joint normalisation every earlier position's output
     // changes as the prefix grows, and the precondition refuses the model.
     std::vector<int32_t> greedyCached(const std::vector<int32_t> &inputSequence, int32_t startToken, int32_t endToken, int64_t maxLength,
-                                      std::vector<float> *lastLogits = nullptr) const {
+                                      std::vector<float> *lastLogits = nullptr, bool recorded = true) const {
         precondition(canDecodeIncrementally(),
                      "cached decoding needs fused mode, inactive dropout, head dim 64 and attention layers that normalise per token");
-        const int64_t n = (int64_t)inputSequence.size(), D = embedding.outputSize();
+        const int64_t n = (int64_t)inputSequence.size(), D = embedding.outputSize(), vocab = embedding.embeddingMatrix.shape[0];
+        precondition(startToken >= 0 && startToken < vocab, "index out of bounds");
         std::vector<int32_t> tokens;
         if (maxLength <= 0) return tokens;
         Tensor encoded = encoder(prepareInputs(inputSequence, 1, n), {n});
@@ -1251,20 +1312,40 @@ struct Transformer {
                              Tensor(Device::Memory::allocateBuffer(cache)), Tensor(Device::Memory::allocateBuffer(cache))});
         }
         const Tensor positions = positionalEncoding(maxLength);
-        int32_t current = startToken;
-        for (int64_t step = 0; step < maxLength; ++step) {
-            const Tensor position = positions[{step}].view({1, D});
-            Tensor acc = prepareInputs({current}, 1, 1, &position);                                   // [1,1,hidden]
+        const float scale = std::sqrt((float)D);
+        Tensor logits(Device::Memory::allocateBuffer(Shape{1, vocab}));
+        // The step's token and position live in device memory (two int32 in a float buffer of the same size): the calls of a
+        // step are then the same at every position, and are recorded once and replayed (about 80 launches per token at
+        // about 2 us each instead of 3 us issued one by one).
+        Tensor cursor(Device::Memory::allocateBuffer(Shape{2}));
+        int32_t *token = reinterpret_cast<int32_t *>(cursor.buffer().memory), *position = token + 1;
+        const int32_t first[2] = {startToken, 0};
+        Device::check(dl4s_hip_assign_h2d(Device::context(), token, first, sizeof(first)));
+        auto step = [&] {
+            Tensor acc(Device::Memory::allocateBuffer(Shape{1, 1, D}));
+            Device::Engine::embedAt(embedding.embeddingMatrix.values(), token, &scale, positions.values(), position, acc.values());
             for (size_t i = 0; i < state.size(); ++i)
-                acc = decoder.decoderLayers[i].step(acc, state[i].keyCache, state[i].valueCache, step, state[i].encKeys, state[i].encValues);
-            Tensor last = acc.view({1, D}).matrixMultiplied(embedding.embeddingMatrix, false, true).view({-1});
+                acc = decoder.decoderLayers[i].step(acc, state[i].keyCache, state[i].valueCache, -1, state[i].encKeys, state[i].encValues,
+                                                    position);
+            Device::Engine::gemm(acc.view({1, D}).values(), embedding.embeddingMatrix.values(), logits.values(), 1.0f, 0.0f, false, true);
+            Device::Engine::argmaxTo(logits.values(), token, position);
+        };
+        RecordedCalls replayable;
+        for (int64_t i = 0; i < maxLength; ++i) {
+            if (i == 0 || !recorded) {
+                step();                       // the first step also sizes the library's scratch block
+            } else {
+                if (!replayable) replayable.record(step);
+                replayable.replay();
+            }
+            int32_t chosen = 0;
+            Device::check(dl4s_hip_assign_d2h(Device::context(), &chosen, token, sizeof(chosen)));
             if (lastLogits) {
-                const std::vector<float> row = last.elements();
+                const std::vector<float> row = logits.elements();
                 lastLogits->insert(lastLogits->end(), row.begin(), row.end());
             }
-            current = (int32_t)last.argmax();
-            tokens.push_back(current);
-            if (current == endToken) break;
+            tokens.push_back(chosen);
+            if (chosen == endToken) break;
         }
         return tokens;
     }

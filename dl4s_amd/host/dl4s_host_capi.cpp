@@ -226,7 +226,7 @@ int dl4s_host_transformer_forward(dl4s_hip_ctx *ctx, int fused, dl4s_host_transf
     });
 }
 
-static int greedy_decode(dl4s_hip_ctx *ctx, int fused, bool cached, dl4s_host_transformer *t, const int32_t *input_sequence, int64_t n,
+static int greedy_decode(dl4s_hip_ctx *ctx, int fused, bool cached, bool recorded, dl4s_host_transformer *t, const int32_t *input_sequence, int64_t n,
                          int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens, int64_t *out_count,
                          float *out_logits, float *out_ms) {
     return guarded(ctx, fused, [&] {
@@ -235,7 +235,7 @@ static int greedy_decode(dl4s_hip_ctx *ctx, int fused, bool cached, dl4s_host_tr
         std::vector<float> logits;
         HIP::check(dl4s_hip_sync(ctx));
         const auto t0 = std::chrono::steady_clock::now();
-        std::vector<int32_t> toks = cached ? t->model.greedyCached(in, start_token, end_token, max_length, out_logits ? &logits : nullptr)
+        std::vector<int32_t> toks = cached ? t->model.greedyCached(in, start_token, end_token, max_length, out_logits ? &logits : nullptr, recorded)
                                            : t->model.greedy(in, start_token, end_token, max_length, out_logits ? &logits : nullptr);
         HIP::check(dl4s_hip_sync(ctx));
         if (out_ms) *out_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -248,14 +248,14 @@ static int greedy_decode(dl4s_hip_ctx *ctx, int fused, bool cached, dl4s_host_tr
 int dl4s_host_transformer_greedy(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence, int64_t n,
                                  int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens,
                                  int64_t *out_count, float *out_logits, float *out_ms) {
-    return greedy_decode(ctx, fused, false, t, input_sequence, n, start_token, end_token, max_length, out_tokens, out_count, out_logits,
+    return greedy_decode(ctx, fused, false, false, t, input_sequence, n, start_token, end_token, max_length, out_tokens, out_count, out_logits,
                          out_ms);
 }
 
 int dl4s_host_transformer_greedy_cached(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence,
-                                        int64_t n, int32_t start_token, int32_t end_token, int64_t max_length, int32_t *out_tokens,
-                                        int64_t *out_count, float *out_logits, float *out_ms) {
-    return greedy_decode(ctx, fused, true, t, input_sequence, n, start_token, end_token, max_length, out_tokens, out_count, out_logits,
+                                        int64_t n, int32_t start_token, int32_t end_token, int64_t max_length, int recorded,
+                                        int32_t *out_tokens, int64_t *out_count, float *out_logits, float *out_ms) {
+    return greedy_decode(ctx, fused, true, recorded != 0, t, input_sequence, n, start_token, end_token, max_length, out_tokens, out_count, out_logits,
                          out_ms);
 }
 

@@ -228,16 +228,20 @@ class Transformer:
         _check(load().dl4s_host_transformer_set_norm_per_token(self.handle, int(bool(per_token))))
 
     def greedy(self, input_sequence, start_token, end_token, max_length, fused=True, return_logits=False, timing=False, cached=False):
-        """cached=True: key / value caches, one new position per step (models set to normalise per token only)."""
+        """cached=True: key / value caches, one new position per step (models set to normalise per token only), the step
+        recorded into a HIP graph and replayed; cached="stepwise": the same calls issued one by one."""
         src = np.ascontiguousarray(input_sequence, np.int32)
         toks = np.empty(max(1, max_length), np.int32)
         n = _i64()
         logits = np.empty((max(1, max_length), self.vocab), np.float32) if return_logits else None
         ms = C.c_float()
-        entry = load().dl4s_host_transformer_greedy_cached if cached else load().dl4s_host_transformer_greedy
-        _check(entry(self.ctx.handle, int(fused), self.handle, src.ctypes.data_as(C.POINTER(C.c_int32)), _i64(len(src)),
-                     C.c_int32(start_token), C.c_int32(end_token), _i64(max_length), toks.ctypes.data_as(C.POINTER(C.c_int32)),
-                     C.byref(n), _p(logits), C.byref(ms)))
+        head = (self.ctx.handle, int(fused), self.handle, src.ctypes.data_as(C.POINTER(C.c_int32)), _i64(len(src)),
+                C.c_int32(start_token), C.c_int32(end_token), _i64(max_length))
+        tail = (toks.ctypes.data_as(C.POINTER(C.c_int32)), C.byref(n), _p(logits), C.byref(ms))
+        if cached:
+            _check(load().dl4s_host_transformer_greedy_cached(*head, C.c_int(0 if cached == "stepwise" else 1), *tail))
+        else:
+            _check(load().dl4s_host_transformer_greedy(*head, *tail))
         res = [[int(x) for x in toks[:n.value]]]
         if return_logits:
             res.append(logits[:n.value])

@@ -64,9 +64,10 @@ int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms);
  * block of that size, a call that needs more library scratch than is there) return DL4S_HIP_EUNSUPPORTED and leave the
  * recording open.  Run the same calls once before recording them: that sizes the scratch block.
  *
- * A graph holds the addresses it was recorded with.  Every buffer that the recorded calls read or write, temporaries
- * included, must stay allocated (not handed back with dl4s_hip_free and allocated again for something else) for as
- * long as the graph is replayed; inputs are read at replay time, so new data in the same buffers gives new results.
+ * A graph holds the addresses it was recorded with.  Every buffer that the recorded calls read or write must stay
+ * allocated for as long as the graph is replayed; inputs are read at replay time, so new data in the same buffers gives
+ * new results.  Temporaries may be allocated and freed inside the recording as usual: a block handed to dl4s_hip_free
+ * while recording stays reserved for the graph and returns to the pool when the graph is destroyed.
  * Some calls use the library's scratch block: if a later call regrows it, dl4s_hip_graph_launch refuses the graph
  * (DL4S_HIP_EUNSUPPORTED) and it has to be recorded again.  One recording at a time per context, made and replayed
  * from one host thread at a time.
@@ -187,6 +188,24 @@ int dl4s_hip_kv_append_f32(dl4s_hip_ctx *ctx, float *kcache, float *vcache, cons
 int dl4s_hip_sdpa_decode_step_f32(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcache,
                                   const float *k_new, const float *v_new, float *out, int64_t B, int64_t H,
                                   int64_t pos, int64_t Tcap, int64_t d, float inv_temperature);
+/* ---- a decoding step whose token and position live in device memory (no counterpart in the reference).
+ * A step of cached decoding has the same shapes at every position; with the position and the chosen token kept in device
+ * memory the calls of one step can be recorded once (dl4s_hip_graph_begin) and replayed for every later position.
+ *   dl4s_hip_embed_at_f32            result[D] = table[*token_dev] * (*scale) + positions[*position_dev]; a token outside
+ *                                    [0, vocab) embeds as zeros, a position outside [0, position_rows) adds nothing
+ *   dl4s_hip_sdpa_decode_step_at_f32 dl4s_hip_sdpa_decode_step_f32 with pos = *pos_dev (one workgroup per (batch, head)
+ *                                    pair, no key split); a value outside [0, Tcap) leaves caches and output untouched
+ *   dl4s_hip_argmax_to_f32           index of the first maximum of values[0..count) written to *out_index_dev (what
+ *                                    dl4s_hip_argmax_f32 returns), then *counter_dev += 1 when counter_dev != NULL
+ * scale is a host pointer (or NULL), read when the call is made. */
+int dl4s_hip_embed_at_f32(dl4s_hip_ctx *ctx, const float *table, int64_t vocab, int64_t D, const int32_t *token_dev,
+                          const float *scale, const float *positions, int64_t position_rows, const int32_t *position_dev,
+                          float *result);
+int dl4s_hip_sdpa_decode_step_at_f32(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcache, const float *k_new,
+                                     const float *v_new, float *out, int64_t B, int64_t H, const int32_t *pos_dev,
+                                     int64_t Tcap, int64_t d, float inv_temperature);
+int dl4s_hip_argmax_to_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, int32_t *out_index_dev,
+                           int32_t *counter_dev);
 
 /* ------------------------------------------------------------------ EngineType subset */
 /* The primitives the layers on the path call (Engine/Engine.swift:143-581); fp32 only.

@@ -92,13 +92,16 @@ int dl4s_host_transformer_greedy(dl4s_hip_ctx *ctx, int fused, dl4s_host_transfo
  * decoding can be cached.  Applies to forward and greedy as well. */
 int dl4s_host_transformer_set_norm_per_token(dl4s_host_transformer *t, int per_token);
 /* No counterpart in the reference.  Greedy decoding with key / value caches: each step runs the decoder on the one new
- * position (dl4s_hip_sdpa_decode_step_f32 over the layer's cache, dl4s_hip_sdpa_decode_f32 over the encoder states'
- * projections) instead of re-running the prefix.  Same arguments as dl4s_host_transformer_greedy.  Requires fused mode,
+ * position (dl4s_hip_sdpa_decode_step_at_f32 over the layer's cache, dl4s_hip_sdpa_decode_f32 over the encoder states'
+ * projections) instead of re-running the prefix.  The step's token and position stay in device memory, so every step
+ * issues the same calls: with recorded != 0 they are recorded into a HIP graph at the second step and replayed from
+ * then on, with recorded == 0 issued one by one (same results, bit for bit).  Other arguments as
+ * dl4s_host_transformer_greedy.  Requires fused mode,
  * head dim 64 and a model set to normalise per token (error otherwise: with the reference's joint normalisation a cache
  * computes a different function).  For such a model it returns the tokens of dl4s_host_transformer_greedy, and the same
  * logits up to summation order. */
 int dl4s_host_transformer_greedy_cached(dl4s_hip_ctx *ctx, int fused, dl4s_host_transformer *t, const int32_t *input_sequence,
-                                        int64_t n, int32_t start_token, int32_t end_token, int64_t max_length,
+                                        int64_t n, int32_t start_token, int32_t end_token, int64_t max_length, int recorded,
                                         int32_t *out_tokens, int64_t *out_count, float *out_logits, float *out_ms);
 /* PositionalEncoding(hiddenSize)(maxLen) -> [maxLen, hiddenSize] -- PositionalEncoding.swift:52-69 */
 int dl4s_host_positional_encoding(dl4s_hip_ctx *ctx, int fused, int64_t max_len, int64_t hidden, float *out);

@@ -183,6 +183,12 @@ def test_cached_greedy_decoding(ctx):
     toks, logits = model.greedy(src, 1, -5, steps, cached=True, return_logits=True)
     assert toks == ref_tokens
     assert_parity(logits, np.stack(ref_logits), "cached greedy logits")
+    # the recorded step replayed at every position computes what the same calls issued one by one compute, and a second
+    # decode (a new recording, the pool holding the first one's blocks again) repeats the first
+    toks_s, logits_s = model.greedy(src, 1, -5, steps, cached="stepwise", return_logits=True)
+    assert toks_s == toks and np.array_equal(logits_s, logits)
+    toks_2, logits_2 = model.greedy(src, 1, -5, steps, cached=True, return_logits=True)
+    assert toks_2 == toks and np.array_equal(logits_2, logits)
     # stops at the end token like the uncached loop
     assert model.greedy(src, 1, ref_tokens[3], steps, cached=True) == ref_tokens[:ref_tokens.index(ref_tokens[3]) + 1]
     assert model.greedy(src, 1, -5, 0, cached=True) == []
