@@ -206,6 +206,12 @@ class Context:
                                                       _vp(_ptr(k_new)), _vp(_ptr(v_new)), _vp(_ptr(out)), _i64(B), _i64(H),
                                                       _i64(pos), _i64(Tcap), _i64(d), C.c_float(inv_temperature)))
 
+    def sdpa_decode_step_at(self, q, kcache, vcache, k_new, v_new, out, B, H, pos_dev, Tcap, d, inv_temperature):
+        """pos_dev: device address of the int32 row index."""
+        _check(self.lib.dl4s_hip_sdpa_decode_step_at_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(kcache)), _vp(_ptr(vcache)),
+                                                         _vp(_ptr(k_new)), _vp(_ptr(v_new)), _vp(_ptr(out)), _i64(B), _i64(H),
+                                                         _vp(_ptr(pos_dev)), _i64(Tcap), _i64(d), C.c_float(inv_temperature)))
+
     # ---- engine primitives
     def fill(self, value, result, count):
         _check(self.lib.dl4s_hip_fill_f32(self.handle, C.c_float(value), _vp(_ptr(result)), _i64(count)))
@@ -234,6 +240,17 @@ class Context:
         idx, val = C.c_int64(), C.c_float()
         _check(self.lib.dl4s_hip_argmax_f32(self.handle, _vp(_ptr(x)), _i64(count), C.byref(idx), C.byref(val)))
         return idx.value, val.value
+
+    def argmax_to(self, x, count, out_index_dev, counter_dev=None):
+        """Index of the first maximum to device int32 *out_index_dev; *counter_dev += 1 when given."""
+        _check(self.lib.dl4s_hip_argmax_to_f32(self.handle, _vp(_ptr(x)), _i64(count), _vp(_ptr(out_index_dev)),
+                                               _vp(_ptr(counter_dev)) if counter_dev is not None else None))
+
+    def embed_at(self, table, vocab, D, token_dev, scale, positions, position_rows, position_dev, y):
+        sc = C.byref(C.c_float(scale)) if scale is not None else None
+        _check(self.lib.dl4s_hip_embed_at_f32(self.handle, _vp(_ptr(table)), _i64(vocab), _i64(D), _vp(_ptr(token_dev)), sc,
+                                              _vp(_ptr(positions)) if positions is not None else None, _i64(position_rows),
+                                              _vp(_ptr(position_dev)) if position_dev is not None else None, _vp(_ptr(y))))
 
     def stack_axis(self, buffers, chunks, outer, y):
         arr = (_vp * max(1, len(buffers)))(*[_ptr(b) for b in buffers])

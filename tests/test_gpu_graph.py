@@ -140,3 +140,52 @@ def test_scratch_growth_is_refused_while_recording_and_outdates_graphs(ctx):
     with pytest.raises(lib.Dl4sHipError, match="regrown"):
         graph.replay()
     graph.destroy()
+
+
+def test_blocks_freed_while_recording_stay_reserved_for_the_graph(ctx):
+    """A recorded sequence may allocate and free its temporaries as usual: the freed blocks serve later allocations of the
+    same recording, are kept out of the pool while the graph lives (an allocation made afterwards must not alias what a
+    replay overwrites) and return to the pool when the graph is destroyed."""
+    n = 4096
+    x = ctx.to_device(np.arange(n, dtype=np.float32))
+    y = ctx.empty((n,))
+
+    def calls():
+        t1 = ctx.empty((n,))
+        ctx.vneg(x, t1, n)
+        t2 = ctx.empty((n,))
+        ctx.vadd(t1, t1, t2, n)
+        p1 = t1.ptr
+        t1.release()
+        t3 = ctx.empty((n,))              # takes the block t1 gave back, inside the recording as outside
+        ctx.vmul(t2, t2, t3, n)
+        ctx.vadd(t3, x, y, n)
+        ptrs = (p1, t2.ptr, t3.ptr)
+        t2.release()
+        t3.release()
+        return ptrs
+
+    eager = calls()
+    assert eager[0] == eager[2]
+    want = y.numpy()
+    assert np.array_equal(want, 4.0 * np.arange(n, dtype=np.float32) ** 2 + np.arange(n, dtype=np.float32))
+    used0, pooled0 = ctx.mem_stats()
+    ctx.graph_begin()
+    rec = calls()
+    graph = ctx.graph_end()
+    assert rec[0] == rec[2]
+    used1, pooled1 = ctx.mem_stats()
+    assert used1 == used0 and pooled1 == pooled0 - 2 * n * 4       # two blocks of the pool now belong to the graph
+    others = [ctx.empty((n,)) for _ in range(4)]                    # same size class: must come from elsewhere
+    assert not {o.ptr for o in others} & set(rec)
+    for o in others:
+        ctx.fill(7.0, o, n)
+    ctx.fill(0.0, y, n)
+    graph.replay()
+    assert np.array_equal(y.numpy(), want)
+    for o in others:
+        assert np.array_equal(o.numpy(), np.full(n, 7.0, np.float32))
+        o.release()
+    graph.destroy()
+    _, pooled2 = ctx.mem_stats()
+    assert pooled2 >= pooled0                                        # the graph's blocks are back (plus the four others)

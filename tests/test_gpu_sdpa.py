@@ -383,6 +383,43 @@ def test_config5_incremental_decode_append_then_attend(ctx, orc):
         buf.release()
 
 
+def test_decode_step_with_the_position_in_device_memory(ctx, orc):
+    """dl4s_hip_sdpa_decode_step_at_f32 reads the row to append from device memory: a sequence of steps driven by a
+    device counter (advanced by dl4s_hip_argmax_to_f32, as cached decoding does) fills the cache and attends like the
+    by-value entry point; a position outside the cache leaves cache and output alone."""
+    B, H, d, Tcap, steps = 2, 3, 64, 300, 260
+    rng = np.random.default_rng(5150)
+    qs, kn, vn = (rng.standard_normal((steps, B, H, 1, d)).astype(np.float32) for _ in range(3))
+    dq, dkn, dvn = ctx.to_device(qs), ctx.to_device(kn), ctx.to_device(vn)
+    dk_, dv_ = ctx.empty((B, H, Tcap, d)), ctx.empty((B, H, Tcap, d))
+    ctx.fill(float("nan"), dk_, B * H * Tcap * d)          # rows never appended must never be read
+    ctx.fill(float("nan"), dv_, B * H * Tcap * d)
+    dout = ctx.empty((steps, B, H, 1, d))
+    cursor = ctx.to_device(np.zeros(2, np.int32), dtype=np.int32)      # [token (unused here), position]
+    scores = ctx.to_device(np.arange(7, dtype=np.float32))
+    step_bytes = B * H * d * 4
+    for t in range(steps):
+        ctx.sdpa_decode_step_at(dq.offset(t * step_bytes), dk_, dv_, dkn.offset(t * step_bytes), dvn.offset(t * step_bytes),
+                                dout.offset(t * step_bytes), B, H, cursor.offset(4), Tcap, d, 0.125)
+        ctx.argmax_to(scores, 7, cursor, cursor.offset(4))               # position += 1
+    assert list(cursor.numpy()) == [6, steps]
+    out, kfin, vfin = dout.numpy(), dk_.numpy(), dv_.numpy()
+    assert np.array_equal(kfin[:, :, :steps], np.moveaxis(kn[:, :, :, 0], 0, 2)) and np.isnan(kfin[:, :, steps:]).all()
+    assert np.array_equal(vfin[:, :, :steps], np.moveaxis(vn[:, :, :, 0], 0, 2))
+    for t in (0, 1, 127, 128, 129, 259):
+        ref = orc.sdpa_decode(qs[t], kfin, vfin, t + 1)
+        assert_parity(out[t], ref, "decode step at device position %d" % t)
+    # positions outside the cache: nothing is written
+    before = dout.numpy().copy()
+    for bad in (-1, Tcap, 1 << 20):
+        cur = ctx.to_device(np.array([0, bad], np.int32), dtype=np.int32)
+        ctx.sdpa_decode_step_at(dq, dk_, dv_, dkn, dvn, dout, B, H, cur.offset(4), Tcap, d, 0.125)
+        assert np.array_equal(dout.numpy(), before, equal_nan=True) and np.array_equal(dk_.numpy(), kfin, equal_nan=True)
+        cur.release()
+    for buf in (dq, dkn, dvn, dk_, dv_, dout, cursor, scores):
+        buf.release()
+
+
 @pytest.mark.parametrize("d", [64, 8, 36, 128, 80])
 @pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 70), (1, 2, 5, 7), (2, 4, 256, 256), (1, 5, 33, 161)])
 def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk, d):

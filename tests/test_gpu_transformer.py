@@ -96,6 +96,49 @@ def test_log_softmax_rows(ctx):
     dy.release()
 
 
+def test_embedding_of_a_token_held_in_device_memory(ctx, orc):
+    """dl4s_hip_embed_at_f32: token and position come from device memory; same rounding as the host-token entry point;
+    a token outside the vocabulary embeds as zeros, a position outside the table adds nothing."""
+    from oracle import transformer as T
+    rng = np.random.default_rng(34)
+    V, D, rows = 29, 24, 9
+    E = rng.standard_normal((V, D)).astype(np.float32)
+    pos = T.positional_encoding(rows, D)
+    scale = float(np.sqrt(np.float32(D)))
+    dE, dpos, dy = ctx.to_device(E), ctx.to_device(pos), ctx.empty((D,))
+    for token, at in ((0, 0), (17, 5), (28, 8)):
+        cur = ctx.to_device(np.array([token, at], np.int32), dtype=np.int32)
+        ctx.embed_at(dE, V, D, cur, scale, dpos, rows, cur.offset(4), dy)
+        want = orc.broadcast("add", orc.broadcast("mul", E[token], np.float32(scale)), pos[at])
+        assert np.array_equal(dy.numpy(), want)
+        ctx.embed_at(dE, V, D, cur, None, None, 0, None, dy)
+        assert np.array_equal(dy.numpy(), E[token])
+        cur.release()
+    for token, at, want in ((-1, 2, pos[2]), (V, 2, pos[2]), (3, rows, E[3] * np.float32(scale)), (3, -1, E[3] * np.float32(scale))):
+        cur = ctx.to_device(np.array([token, at], np.int32), dtype=np.int32)
+        ctx.embed_at(dE, V, D, cur, scale, dpos, rows, cur.offset(4), dy)
+        assert np.array_equal(dy.numpy(), want.astype(np.float32))
+        cur.release()
+    for b in (dE, dpos, dy):
+        b.release()
+
+
+@pytest.mark.parametrize("n", [1, 7, 1025, 100003])
+def test_argmax_to_device_memory(ctx, orc, n):
+    rng = np.random.default_rng(n + 1)
+    x = rng.standard_normal(n).astype(np.float32)
+    if n > 6:
+        x[[2, n - 3]] = x.max() + 1.0
+    d = ctx.to_device(x)
+    cur = ctx.to_device(np.array([-7, 41], np.int32), dtype=np.int32)
+    ctx.argmax_to(d, n, cur, cur.offset(4))
+    assert list(cur.numpy()) == [orc.argmax(x)[0], 42]
+    ctx.argmax_to(d, n, cur.offset(4))                  # no counter
+    assert list(cur.numpy()) == [orc.argmax(x)[0]] * 2
+    d.release()
+    cur.release()
+
+
 @pytest.mark.parametrize("fused", [False, True])
 def test_positional_encoding_layer(ctx, fused):
     from dl4s_amd import host_lib
