@@ -115,6 +115,12 @@ def decode(ctx, lib, repeats):
             "shape": {"B": B, "H": H, "d": d, "T0": T0, "steps": steps}}
 
 
+def under_rocprof():
+    """rocprofv3's queue interception aborts the queue on a HIP graph launch (HSA_STATUS_ERROR_INVALID_PACKET_FORMAT) and
+    then does not exit: the sections that replay recorded calls are left out when the process runs under it."""
+    return any(k.startswith(("ROCPROF", "ROCP_")) or "rocprofiler-sdk" in v for k, v in os.environ.items())
+
+
 def other_configs(ctx, lib, cpu, only=None):
     """Configs 1-3 of the baseline: us/call, TFLOP/s on the algorithmic flops, fraction of the fp32 MFMA peak; the
     CPU oracle beside each (whole call for configs 1 and 2, one batch item of config 3), single thread."""
@@ -168,7 +174,9 @@ def other_configs(ctx, lib, cpu, only=None):
             orc.mha(x, x, x, mask, attn, H, dk_, dk_)
             dt = time.perf_counter() - t0
             res["config2_mha_B4_L512_D512_H8_causal_fused"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
-    if want("recorded"):
+    if want("recorded") and under_rocprof():
+        res["recorded"] = "skipped under rocprofv3 (graph launches abort its intercepted queue)"
+    elif want("recorded"):
         # Calls recorded into a HIP graph and replayed, against the same calls issued one by one.
         B, L, D, H, dk_ = 4, 512, 512, 8, 64
         rng = np.random.Generator(np.random.PCG64(1012))
@@ -336,21 +344,22 @@ def other_configs(ctx, lib, cpu, only=None):
             entry["ms_per_token_" + mode] = ms / len(toks)
             entry["tokens_per_s_" + mode] = len(toks) / ms * 1e3
         if only is not None and "greedy_cached_only" in only:
-            # the cached decode of 512 tokens alone (for a kernel trace of just that loop)
+            # the cached decode of 512 tokens alone, its calls issued one by one (for a kernel trace of just that loop)
             model.set_norm_per_token(True)
-            model.greedy(src, 1, -5, 4, cached=True)
-            toks_c, ms_c = model.greedy(src, 1, -5, 512, cached=True, timing=True)
-            entry["per_token_normalisation"] = {"512_tokens": {"cached": ms_c / len(toks_c)}}
+            model.greedy(src, 1, -5, 4, cached="stepwise")
+            toks_c, ms_c = model.greedy(src, 1, -5, 512, cached="stepwise", timing=True)
+            entry["per_token_normalisation"] = {"512_tokens": {"cached_calls_issued_one_by_one": ms_c / len(toks_c)}}
             model.set_norm_per_token(False)
         if want("greedy") or want("greedy_cached"):
             # The same model with per-token normalisation in its attention layers (not the reference's model: its joint
             # normalisation cannot be cached), decoded by re-running the prefix and with key / value caches, 32 and 512 tokens.
             model.set_norm_per_token(True)
-            model.greedy(src, 1, -5, 4, cached=True)
+            replay = "stepwise" if under_rocprof() else True
+            model.greedy(src, 1, -5, 4, cached=replay)
             per_token = {"note": "attention layers normalise per token (not the reference's model); ms per generated token"}
             for count in (32, 512):
                 toks_r, ms_r = model.greedy(src, 1, -5, count, timing=True)
-                toks_c, ms_c = model.greedy(src, 1, -5, count, cached=True, timing=True)
+                toks_c, ms_c = model.greedy(src, 1, -5, count, cached=replay, timing=True)
                 toks_s, ms_s = model.greedy(src, 1, -5, count, cached="stepwise", timing=True)
                 per_token["%d_tokens" % count] = {"prefix_rerun": ms_r / len(toks_r), "cached_step_recorded_and_replayed": ms_c / len(toks_c),
                                                   "cached_calls_issued_one_by_one": ms_s / len(toks_s),
