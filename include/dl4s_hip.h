@@ -72,6 +72,9 @@ int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms);
  * (DL4S_HIP_EUNSUPPORTED) and it has to be recorded again.  One recording at a time per context, made and replayed
  * from one host thread at a time.
  *
+ * Do not replay graphs under rocprofv3: its queue interception rejects the packets of a graph launch
+ * (HSA_STATUS_ERROR_INVALID_PACKET_FORMAT, ROCm 7.2) and the queue is aborted.
+ *
  * dl4s_hip_graph_end with out_graph == NULL gives the recording up, and so does dl4s_hip_destroy.  Destroy a context's
  * graphs before the context. */
 typedef struct dl4s_hip_graph dl4s_hip_graph;
