@@ -337,6 +337,53 @@ __global__ void bias_gelu_f32(const float *__restrict__ x, const float *__restri
     }
 }
 
+// The same for operands whose axes merge into at most three groups (outer, middle, inner), each group taken whole by
+// both operands or broadcast whole by one of them - every broadcast of the attention path: scores - mask ([B,H,L,L] -
+// [L,L]), x - max and x / sum ([.., L] against [.., 1]), LayerNorm's [B,L,D] against [B,1,1] and [D].  32-bit index
+// arithmetic with two divisions per V elements (the general kernel spends two 64-bit divisions per axis and element:
+// 2.4 TB/s on the mask subtraction of config 2), 128-bit accesses when the inner group allows.
+// A_IN / B_IN: the operand runs along the inner group (else it is one value per inner row).  e2v = inner extent / V.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+template <int OP>
+__device__ __forceinline__ float broadcast_op(const float x, const float z, const int mode) {
+    if (OP == DL4S_OP_ADD) return __fadd_rn(x, z);
+    if (OP == DL4S_OP_MUL) return __fmul_rn(x, z);
+    if (OP == DL4S_OP_SUB) {
+        if (mode == 2) return __fadd_rn(x, -z);             // x + (-s)
+        if (mode == 1) return -__fadd_rn(z, -x);            // -(x + (-s))
+        return __fsub_rn(x, z);
+    }
+    if (mode == 2) return __fmul_rn(x, __fdiv_rn(1.0f, z));  // x * (1/s)
+    return __fdiv_rn(x, z);
+}
+template <int OP, int V, bool A_IN, bool B_IN>
+__global__ void broadcast3_f32(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ y, unsigned e1,
+                               unsigned e2v, unsigned sa0, unsigned sa1, unsigned sb0, unsigned sb1, int mode, unsigned nvec) {
+    for (unsigned v = blockIdx.x * blockDim.x + threadIdx.x; v < nvec; v += gridDim.x * blockDim.x) {
+        const unsigned i2 = v % e2v, t = v / e2v, i1 = t % e1, i0 = t / e1;
+        const unsigned ao = i0 * sa0 + i1 * sa1 + (A_IN ? i2 * V : 0u), bo = i0 * sb0 + i1 * sb1 + (B_IN ? i2 * V : 0u);
+        if (V == 4) {
+            f32x4_t x, z, r;
+            if (A_IN) x = *reinterpret_cast<const f32x4_t *>(a + ao);
+            else { const float s = a[ao]; x = f32x4_t{s, s, s, s}; }
+            if (B_IN) z = *reinterpret_cast<const f32x4_t *>(b + bo);
+            else { const float s = b[bo]; z = f32x4_t{s, s, s, s}; }
+            r.x = broadcast_op<OP>(x.x, z.x, mode); r.y = broadcast_op<OP>(x.y, z.y, mode);
+            r.z = broadcast_op<OP>(x.z, z.z, mode); r.w = broadcast_op<OP>(x.w, z.w, mode);
+            *reinterpret_cast<f32x4_t *>(y + (size_t)v * 4) = r;
+        } else {
+            y[v] = broadcast_op<OP>(a[ao], b[bo], mode);
+        }
+    }
+}
+template <int OP, int V>
+void launch_broadcast3(hipStream_t stream, const int inner_type, const float *a, const float *b, float *y, unsigned e1, unsigned e2v,
+                       unsigned sa0, unsigned sa1, unsigned sb0, unsigned sb1, int mode, unsigned nvec) {
+    const dim3 g(grid_for((long long)nvec, 2)), blk(TPB);
+    if (inner_type == 3) hipLaunchKernelGGL((broadcast3_f32<OP, V, true, true>), g, blk, 0, stream, a, b, y, e1, e2v, sa0, sa1, sb0, sb1, mode, nvec);
+    else if (inner_type == 1) hipLaunchKernelGGL((broadcast3_f32<OP, V, true, false>), g, blk, 0, stream, a, b, y, e1, e2v, sa0, sa1, sb0, sb1, mode, nvec);
+    else hipLaunchKernelGGL((broadcast3_f32<OP, V, false, true>), g, blk, 0, stream, a, b, y, e1, e2v, sa0, sa1, sb0, sb1, mode, nvec);
+}
 template <int OP>
 int launch_unary(dl4s_hip_ctx *ctx, const float *x, float *y, int64_t n, const char *name) {
     DL4S_CHECK_CTX(ctx);
@@ -538,6 +585,42 @@ int dl4s_hip_broadcast_f32(dl4s_hip_ctx *ctx, int op, const float *lhs, const in
             if (ls[i] > rs[i]) { mode = 2; break; }
             if (rs[i] > ls[i]) { mode = 1; break; }
         }
+    // Merge neighbouring axes that both operands treat alike (1 = only lhs runs along it, 2 = only rhs, 3 = both; axes of
+    // extent 1 drop out).  Up to three groups and fewer than 2^31 elements: the fast kernel.
+    long long ge[DL4S_HIP_MAX_DIM];
+    int gt[DL4S_HIP_MAX_DIM], groups = 0;
+    for (int i = 0; i < dim; ++i) {
+        if (bc.oshape[i] == 1) continue;
+        const int t = (ls[i] > 1 ? 1 : 0) | (rs[i] > 1 ? 2 : 0);
+        if (groups && gt[groups - 1] == t) ge[groups - 1] *= bc.oshape[i];
+        else { ge[groups] = bc.oshape[i]; gt[groups] = t; ++groups; }
+    }
+    if (groups >= 1 && groups <= 3 && n < (1ll << 31)) {
+        long long e[3] = {1, 1, 1};
+        int t[3] = {0, 0, 0};
+        for (int i = 0; i < groups; ++i) { e[3 - groups + i] = ge[i]; t[3 - groups + i] = gt[i]; }
+        // element strides of the two (dense) operands over the groups they run along
+        unsigned sa[3] = {0, 0, 0}, sb[3] = {0, 0, 0};
+        long long as = 1, bs = 1;
+        for (int i = 2; i >= 0; --i) {
+            if (t[i] & 1) { sa[i] = (unsigned)as; as *= e[i]; }
+            if (t[i] & 2) { sb[i] = (unsigned)bs; bs *= e[i]; }
+        }
+        const auto al16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+        const bool vec = e[2] % 4 == 0 && al16(result) && (!(t[2] & 1) || al16(lhs)) && (!(t[2] & 2) || al16(rhs));
+        const unsigned e2v = (unsigned)(vec ? e[2] / 4 : e[2]), nvec = (unsigned)(vec ? n / 4 : n);
+#define DL4S_BCAST3(OP_)                                                                                                               \
+    if (vec) launch_broadcast3<OP_, 4>(ctx->stream, t[2], lhs, rhs, result, (unsigned)e[1], e2v, sa[0], sa[1], sb[0], sb[1], mode, nvec); \
+    else launch_broadcast3<OP_, 1>(ctx->stream, t[2], lhs, rhs, result, (unsigned)e[1], e2v, sa[0], sa[1], sb[0], sb[1], mode, nvec)
+        switch (op) {
+            case DL4S_OP_ADD: DL4S_BCAST3(DL4S_OP_ADD); break;
+            case DL4S_OP_SUB: DL4S_BCAST3(DL4S_OP_SUB); break;
+            case DL4S_OP_MUL: DL4S_BCAST3(DL4S_OP_MUL); break;
+            default: DL4S_BCAST3(DL4S_OP_DIV); break;
+        }
+#undef DL4S_BCAST3
+        return dl4s::launch_status("broadcast");
+    }
     const dim3 g(grid_for(n, 2)), b(TPB);
     switch (op) {
         case DL4S_OP_ADD: hipLaunchKernelGGL(broadcast_f32<DL4S_OP_ADD>, g, b, 0, ctx->stream, lhs, rhs, result, bc, mode, n); break;

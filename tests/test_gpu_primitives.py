@@ -227,7 +227,12 @@ def test_gemm_grouped_argument_errors(ctx):
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
 @pytest.mark.parametrize("sa,sb", [((2, 3, 4), (4,)), ((2, 3, 4), (3, 1)), ((2, 3, 4), ()), ((), (2, 3)), ((2, 1, 4), (1, 3, 1)),
                                    ((2, 3, 4, 5), (2, 1, 1, 5)), ((3, 4), (3, 4)), ((2, 2, 33, 33), (33, 33)), ((40, 1), (1, 50)),
-                                   ((2, 3, 7, 9), (2, 3, 7, 1))])
+                                   ((2, 3, 7, 9), (2, 3, 7, 1)),
+                                   # 128-bit paths of the merged-axes kernel: inner group taken by both, by lhs only, by rhs only
+                                   ((2, 3, 64, 64), (64, 64)), ((4, 8, 16), (4, 8, 1)), ((8, 1), (8, 12)), ((5, 16), (1, 16)),
+                                   ((3, 1, 8), (1, 5, 1)), ((6, 40), ()),
+                                   # more than three groups: the general kernel
+                                   ((2, 3, 4, 5, 6), (2, 1, 4, 1, 6)), ((2, 1, 4, 1, 6), (2, 3, 1, 5, 1))])
 def test_broadcast_bit_exact(ctx, orc, op, sa, sb):
     from dl4s_amd import lib
     a, b = rnd(*sa), rnd(*sb) + np.float32(2.5)
@@ -235,6 +240,19 @@ def test_broadcast_bit_exact(ctx, orc, op, sa, sb):
     da, db, dy = ctx.to_device(a), ctx.to_device(b), ctx.empty(ref.shape)
     ctx.broadcast({"add": lib.OP_ADD, "sub": lib.OP_SUB, "mul": lib.OP_MUL, "div": lib.OP_DIV}[op], da, sa, db, sb, dy)
     assert np.array_equal(dy.numpy(), ref)          # includes x*(1/s) and x+(-s) roundings of the scalar forms
+    for x in (da, db, dy):
+        x.release()
+
+
+def test_broadcast_on_operands_that_are_not_16_byte_aligned(ctx, orc):
+    """Offset views (a row of a larger tensor starting at an odd element) take the element-wise path of the same kernel."""
+    from dl4s_amd import lib
+    a, b = rnd(3 * 64 + 1), rnd(64 + 3)
+    da, db, dy = ctx.to_device(a), ctx.to_device(b), ctx.empty((3 * 64 + 1,))
+    ctx.broadcast(lib.OP_SUB, da.offset(4), (3, 64), db.offset(12), (64,), dy.offset(4))
+    assert np.array_equal(dy.numpy()[1:].reshape(3, 64), orc.broadcast("sub", a[1:].reshape(3, 64), b[3:]))
+    ctx.broadcast(lib.OP_MUL, da, (3, 64), db.offset(12), (64,), dy)        # only rhs off the grid
+    assert np.array_equal(dy.numpy()[:192].reshape(3, 64), orc.broadcast("mul", a[:192].reshape(3, 64), b[3:]))
     for x in (da, db, dy):
         x.release()
 
