@@ -300,10 +300,15 @@ int dl4s_hip_sdpa_decode_step_at_f32(dl4s_hip_ctx *ctx, const float *q, float *k
     DL4S_REQUIRE(d == HD, DL4S_HIP_EUNSUPPORTED, "sdpa_decode_step_at: head dim %lld (only 64 is implemented)", (long long)d);
     DL4S_REQUIRE(Tcap >= 1 && Tcap < (1ll << 30) && BH <= 65535, DL4S_HIP_EUNSUPPORTED,
                  "sdpa_decode_step_at: capacity %lld or B*H=%lld out of range", (long long)Tcap, (long long)BH);
-    // the row count is not known on the host: one workgroup of 16 wavefronts per pair walks whatever rows there are
+    // the row count is not known on the host: one workgroup per pair walks whatever rows there are (16 wavefronts, 4 for a
+    // cache of up to 128 rows, where one 32-row block per wavefront covers it)
     const int chunk = (int)((Tcap + KB - 1) / KB * KB);
-    hipLaunchKernelGGL((sdpa_decode_splitk_f32<true, 16, true>), dim3(1, (unsigned)BH), dim3(16 * 64), 0, ctx->stream, q, kcache, vcache,
-                       k_new, v_new, out, (float *)nullptr, 0, (int)Tcap, 0, inv_temperature, 1, chunk, pos_dev);
+    if (Tcap > 128)
+        hipLaunchKernelGGL((sdpa_decode_splitk_f32<true, 16, true>), dim3(1, (unsigned)BH), dim3(16 * 64), 0, ctx->stream, q, kcache,
+                           vcache, k_new, v_new, out, (float *)nullptr, 0, (int)Tcap, 0, inv_temperature, 1, chunk, pos_dev);
+    else
+        hipLaunchKernelGGL((sdpa_decode_splitk_f32<true, 4, true>), dim3(1, (unsigned)BH), dim3(4 * 64), 0, ctx->stream, q, kcache,
+                           vcache, k_new, v_new, out, (float *)nullptr, 0, (int)Tcap, 0, inv_temperature, 1, chunk, pos_dev);
     return dl4s::launch_status("sdpa_decode_splitk_f32");
 }
 

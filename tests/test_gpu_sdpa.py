@@ -383,11 +383,12 @@ def test_config5_incremental_decode_append_then_attend(ctx, orc):
         buf.release()
 
 
-def test_decode_step_with_the_position_in_device_memory(ctx, orc):
+@pytest.mark.parametrize("Tcap,steps", [(300, 260), (100, 90)])      # workgroups of 16 and of 4 wavefronts
+def test_decode_step_with_the_position_in_device_memory(ctx, orc, Tcap, steps):
     """dl4s_hip_sdpa_decode_step_at_f32 reads the row to append from device memory: a sequence of steps driven by a
     device counter (advanced by dl4s_hip_argmax_to_f32, as cached decoding does) fills the cache and attends like the
     by-value entry point; a position outside the cache leaves cache and output alone."""
-    B, H, d, Tcap, steps = 2, 3, 64, 300, 260
+    B, H, d = 2, 3, 64
     rng = np.random.default_rng(5150)
     qs, kn, vn = (rng.standard_normal((steps, B, H, 1, d)).astype(np.float32) for _ in range(3))
     dq, dkn, dvn = ctx.to_device(qs), ctx.to_device(kn), ctx.to_device(vn)
@@ -406,7 +407,7 @@ def test_decode_step_with_the_position_in_device_memory(ctx, orc):
     out, kfin, vfin = dout.numpy(), dk_.numpy(), dv_.numpy()
     assert np.array_equal(kfin[:, :, :steps], np.moveaxis(kn[:, :, :, 0], 0, 2)) and np.isnan(kfin[:, :, steps:]).all()
     assert np.array_equal(vfin[:, :, :steps], np.moveaxis(vn[:, :, :, 0], 0, 2))
-    for t in (0, 1, 127, 128, 129, 259):
+    for t in sorted({0, 1, 31, 32, min(127, steps - 1), min(128, steps - 1), min(129, steps - 1), steps - 1}):
         ref = orc.sdpa_decode(qs[t], kfin, vfin, t + 1)
         assert_parity(out[t], ref, "decode step at device position %d" % t)
     # positions outside the cache: nothing is written
