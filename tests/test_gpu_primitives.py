@@ -269,7 +269,10 @@ def test_broadcast_shape_error(ctx):
 @pytest.mark.parametrize("shape,axes", [((3, 4, 5), [2]), ((3, 4, 5), [1, 2]), ((3, 4, 5), [0]), ((2, 3, 4, 50), [3]),
                                         ((2, 300, 70), [1, 2]), ((6,), [0]), ((4, 5), [0, 1]), ((4, 512, 512), [1, 2]),
                                         ((3, 1, 7, 1, 5), [1, 2]), ((2, 3, 4, 5), [0, 2]), ((2, 3, 4, 5), [1, 3]), ((1, 1), [0]),
-                                        ((700000,), [0]), ((2, 200, 1, 300), [1, 2, 3])])
+                                        ((700000,), [0]), ((2, 200, 1, 300), [1, 2, 3]),
+                                        # many short contiguous rows: one wavefront per row
+                                        ((4, 300, 70), [2]), ((2, 8, 128, 130), [3]), ((1200, 3, 5), [1, 2]), ((1025, 1), [1]),
+                                        ((1100, 4096), [1])])
 def test_reduce_sum(ctx, orc, shape, axes):
     x = rnd(*shape)
     ref = orc.reduce_sum(x, axes)
@@ -280,7 +283,8 @@ def test_reduce_sum(ctx, orc, shape, axes):
     dy.release()
 
 
-@pytest.mark.parametrize("shape,axis", [((3, 4, 5), 2), ((3, 4, 5), 1), ((3, 4, 5), 0), ((2, 2, 9, 1000), 3)])
+@pytest.mark.parametrize("shape,axis", [((3, 4, 5), 2), ((3, 4, 5), 1), ((3, 4, 5), 0), ((2, 2, 9, 1000), 3),
+                                        ((2, 8, 128, 130), 3), ((1100, 7), 1)])
 def test_reduce_max_exact_and_nan_skipping(ctx, orc, shape, axis):
     x = rnd(*shape)
     x.flat[3] = np.nan
