@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # streaming kernel (--copy-calibration: x2.00 and x1.00).  The runs and their figures are summarised in
 # profiles/bench_prefill_config4_decode_config5.md; they are constants here because a counter run cannot be part of
 # the timed process.
-PREFILL_TRAFFIC_BYTES = (396584 * 2.00 + 65536 * 1.00) * 1024      # L2 fills (K/V re-reads included) + writes
-DECODE_TRAFFIC_BYTES = (264293 * 2.00 + 192 * 1.00) * 1024
+PREFILL_TRAFFIC_BYTES = (397295 * 2.00 + 65536 * 1.00) * 1024      # L2 fills (K/V re-reads included) + writes
+DECODE_TRAFFIC_BYTES = (264295 * 2.00 + 192 * 1.00) * 1024
 PREHEAT_S = 0.25
 
 
