@@ -118,7 +118,8 @@ def decode(ctx, lib, repeats):
 def under_rocprof():
     """rocprofv3's queue interception aborts the queue on a HIP graph launch (HSA_STATUS_ERROR_INVALID_PACKET_FORMAT) and
     then does not exit: the sections that replay recorded calls are left out when the process runs under it."""
-    return any(k.startswith(("ROCPROF", "ROCP_")) or "rocprofiler-sdk" in v for k, v in os.environ.items())
+    from dl4s_amd import lib
+    return not lib.graph_supported()
 
 
 def other_configs(ctx, lib, cpu, only=None):

@@ -1,6 +1,7 @@
 // Context, pooled allocator, copies and the stream timer of libdl4s_hip.so.
 #include "common.h"
 
+#include <cstdlib>
 #include <cstring>
 
 namespace dl4s {
@@ -154,9 +155,17 @@ static void release_held(dl4s_hip_ctx *ctx, std::vector<std::pair<void *, size_t
     held.clear();
 }
 
+int dl4s_hip_graph_supported(void) {
+    // rocprofv3 (ROCm 7.2) intercepts the queues of the process; a graph launch then ends in
+    // HSA_STATUS_ERROR_INVALID_PACKET_FORMAT and an aborted queue.  Its launcher exports these variables.
+    return !(getenv("ROCP_TOOL_LIBRARIES") || getenv("ROCPROFILER_LIBRARY_CTOR"));
+}
+
 int dl4s_hip_graph_begin(dl4s_hip_ctx *ctx) {
     DL4S_CHECK_CTX(ctx);
     DL4S_REQUIRE(!ctx->capturing, DL4S_HIP_EINVALID_ARG, "dl4s_hip_graph_begin: a graph is being recorded already");
+    DL4S_REQUIRE(dl4s_hip_graph_supported(), DL4S_HIP_EUNSUPPORTED,
+                 "dl4s_hip_graph_begin: the process runs under rocprofv3, whose queue interception aborts the queue on a graph launch");
     // thread-local mode: calls of other host threads on other streams are left alone
     DL4S_HIP_TRY(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;

@@ -1332,7 +1332,7 @@ struct Transformer {
         };
         RecordedCalls replayable;
         for (int64_t i = 0; i < maxLength; ++i) {
-            if (i == 0 || !recorded) {
+            if (i == 0 || !recorded || !dl4s_hip_graph_supported()) {
                 step();                       // the first step also sizes the library's scratch block
             } else {
                 if (!replayable) replayable.record(step);

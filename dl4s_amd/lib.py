@@ -82,6 +82,11 @@ def _shape_arr(shape):
     return (_i64 * max(1, len(shape)))(*shape)
 
 
+def graph_supported():
+    """False when the process runs under rocprofv3 (graph launches abort its intercepted queue)."""
+    return bool(load().dl4s_hip_graph_supported())
+
+
 class Graph:
     """A recorded sequence of calls (dl4s_hip_graph_*); replay() enqueues it on the context's stream."""
 

@@ -72,12 +72,14 @@ int dl4s_hip_timer_end(dl4s_hip_ctx *ctx, float *out_ms);
  * (DL4S_HIP_EUNSUPPORTED) and it has to be recorded again.  One recording at a time per context, made and replayed
  * from one host thread at a time.
  *
- * Do not replay graphs under rocprofv3: its queue interception rejects the packets of a graph launch
- * (HSA_STATUS_ERROR_INVALID_PACKET_FORMAT, ROCm 7.2) and the queue is aborted.
+ * Graphs cannot be replayed under rocprofv3: its queue interception rejects the packets of a graph launch
+ * (HSA_STATUS_ERROR_INVALID_PACKET_FORMAT, ROCm 7.2) and the queue is aborted.  dl4s_hip_graph_supported returns 0 when
+ * the process was started by rocprofv3, and dl4s_hip_graph_begin then refuses with DL4S_HIP_EUNSUPPORTED.
  *
  * dl4s_hip_graph_end with out_graph == NULL gives the recording up, and so does dl4s_hip_destroy.  Destroy a context's
  * graphs before the context. */
 typedef struct dl4s_hip_graph dl4s_hip_graph;
+int dl4s_hip_graph_supported(void);
 int dl4s_hip_graph_begin(dl4s_hip_ctx *ctx);
 int dl4s_hip_graph_end(dl4s_hip_ctx *ctx, dl4s_hip_graph **out_graph);
 int dl4s_hip_graph_launch(dl4s_hip_ctx *ctx, dl4s_hip_graph *graph);

@@ -15,6 +15,8 @@ HD = D // H
 @pytest.fixture()
 def ctx():
     from dl4s_amd import lib
+    if not lib.graph_supported():
+        pytest.skip("graph launches abort the queue under rocprofv3")
     c = lib.Context(0)
     yield c
     c.close()
