@@ -259,9 +259,12 @@ __device__ __forceinline__ float plain_score(const float *qs, const float *krow,
 
 // Validates a mask descriptor against [B,H,Lq,Lk], fills the kernels' view of it and, for dense masks on the MFMA
 // kernels, launches the tile classifier (its result lives in the context's scratch block until the next call that uses it).
+// extra_bytes / extra: the caller's own share of the scratch block (partial results), placed behind the mask classes so
+// that one sizing of the block covers both (growing it later would move the classes away from under m.cls).
 inline int build_mask_args(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
-                           bool classify, MaskArgs &m) {
+                           bool classify, MaskArgs &m, size_t extra_bytes = 0, void **extra = nullptr) {
     m = MaskArgs{};
+    if (extra) *extra = nullptr;
     m.kind = mask ? mask->kind : DL4S_MASK_NONE;
     switch (m.kind) {
         case DL4S_MASK_NONE: break;
@@ -293,9 +296,11 @@ inline int build_mask_args(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_
         const int64_t nqt = m.sq ? (Lq + 31) / 32 : 1, nkt = m.sk ? (Lk + 31) / 32 : 1;
         const long long total = MB * MH * nqt * nkt;
         if (total < (1ll << 31)) {
-            const int rc = dl4s::ensure_scratch(ctx, (size_t)total);
+            const size_t cls_bytes = ((size_t)total + 255) / 256 * 256;
+            const int rc = dl4s::ensure_scratch(ctx, cls_bytes + extra_bytes);
             if (rc != DL4S_HIP_OK) return rc;
             unsigned char *cls = static_cast<unsigned char *>(ctx->scratch);
+            if (extra && extra_bytes) { *extra = cls + cls_bytes; extra_bytes = 0; }
             hipLaunchKernelGGL(sdpa_mask_classify, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, ctx->stream, m, (int)MB,
                                (int)MH, (int)nqt, (int)nkt, (int)Lq, (int)Lk, total, cls);
             const int st = dl4s::launch_status("sdpa_mask_classify");
@@ -306,6 +311,11 @@ inline int build_mask_args(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_
             m.cls_sh = m.sh ? (int)(nqt * nkt) : 0;
             m.cls_sb = m.sb ? (int)(MH * nqt * nkt) : 0;
         }
+    }
+    if (extra && extra_bytes) {   // no classes in the block: the caller's share starts at its base
+        const int rc = dl4s::ensure_scratch(ctx, extra_bytes);
+        if (rc != DL4S_HIP_OK) return rc;
+        *extra = ctx->scratch;
     }
     return DL4S_HIP_OK;
 }

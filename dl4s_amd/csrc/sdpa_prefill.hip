@@ -570,14 +570,29 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
     const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                            reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     const bool mfma128_path = dk == dv && dk > HD && dk <= HD2 && dk % 4 == 0 && aligned;
-    MaskArgs m{};
-    {
-        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path, m);
-        if (rc != DL4S_HIP_OK) return rc;
-    }
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
     const int no_split = (flags & DL4S_SDPA_NO_KEY_SPLIT) ? 1 : 0;
+    // The 128-wide kernel on a launch that leaves CUs without their two workgroups: the key tiles of every block are dealt
+    // to several workgroups, whose partial results a second kernel adds up (B4 H8 L512 d128: 73 us unsplit).  The count
+    // depends on the extents only.
+    int nsplit128 = 1;
+    size_t part_bytes = 0;
+    if (mfma128_path && !no_split) {
+        const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
+        if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
+            long long want = (2ll * ctx->cu_count + blocks - 1) / blocks;
+            want = std::min(want, std::min(8ll, nkt / 2));
+            const size_t bytes = (size_t)want * B * H * Lq * PART2_STRIDE * sizeof(float);
+            if (want > 1 && bytes <= (size_t(256) << 20)) { nsplit128 = (int)want; part_bytes = bytes; }
+        }
+    }
+    MaskArgs m{};
+    void *part128 = nullptr;
+    {
+        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path, m, part_bytes, &part128);
+        if (rc != DL4S_HIP_OK) return rc;
+    }
     DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR | DL4S_SDPA_NO_KEY_SPLIT)) == 0, DL4S_HIP_EINVALID_ARG,
                  "sdpa: unknown flag bits 0x%x", flags);
     if (mfma_path) {
@@ -597,11 +612,11 @@ int sdpa_forward(dl4s_hip_ctx *ctx, const float *q, const float *k, const float 
         DL4S_REQUIRE(Lk * (token_major ? H : 1) * dk * 4 < (dk == HD2 ? (1ll << 31) : (1ll << 30)), DL4S_HIP_EUNSUPPORTED,
                      "sdpa: the K/V rows of one (batch, head) pair span more than 2 GiB (1 GiB for padded head dims)");
         switch (m.kind) {
-            case DL4S_MASK_NONE: return launch_d128<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
-            case DL4S_MASK_DENSE_F32: return launch_d128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
-            case DL4S_MASK_CAUSAL: return launch_d128<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
-            case DL4S_MASK_KEY_LENGTHS: return launch_d128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
-            default: return launch_d128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+            case DL4S_MASK_NONE: return launch_d128<DL4S_MASK_NONE>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, static_cast<float *>(part128));
+            case DL4S_MASK_DENSE_F32: return launch_d128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, static_cast<float *>(part128));
+            case DL4S_MASK_CAUSAL: return launch_d128<DL4S_MASK_CAUSAL>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, static_cast<float *>(part128));
+            case DL4S_MASK_KEY_LENGTHS: return launch_d128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, static_cast<float *>(part128));
+            default: return launch_d128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, static_cast<float *>(part128));
         }
     }
     DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 128, and 16-byte aligned tensors");

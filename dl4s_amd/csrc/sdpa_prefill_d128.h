@@ -10,23 +10,63 @@
 // One workgroup = 4 wavefronts = 128 queries of one (batch, head), K/V in double-buffered LDS tiles of 32 keys on a
 // 132-float row stride (2 x 2 x 32 x 132 floats = 66 KiB: two workgroups per CU).  Head dims below 128 are padded with
 // zero columns on the fly like the 64-wide kernels do.  Mask kinds, tile skipping, the token-major layout, the work
-// order and the row statistics are those of the 64-wide kernel.
+// order and the row statistics are those of the 64-wide kernel.  Small launches are split over the keys across
+// workgroups (grid.y shares per block, partial results in a scratch buffer, sdpa_prefill_merge_d128 adds them up).
 #pragma once
 #include "sdpa_common.h"
 
 namespace {
+
+constexpr int PART2_STRIDE = HD2 + 4;   // floats per partial row: 128 weighted sums, reference maximum, row sum, padding
+
+// Adds up the nsplit partial results of every query row (32 lanes per row, four columns each), normalises and stores.
+// A partial result whose reference maximum is -inf has seen no finite score: its sums are zeros (or NaN, which must
+// survive), so it is added with factor 1.
+__global__ __launch_bounds__(256) void sdpa_prefill_merge_d128(const float *__restrict__ part, float *__restrict__ out,
+                                                               float *__restrict__ stats, int nsplit, long long rows, int H, int Lq,
+                                                               int hd, int token_major) {
+    const long long row = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int c = threadIdx.x & 31;
+    if (row >= rows) return;
+    float m_all = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) m_all = fmaxf(m_all, part[((long long)s * rows + row) * PART2_STRIDE + HD2]);
+    const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
+    float l_tot = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < nsplit; ++s) {
+        const float *p = part + ((long long)s * rows + row) * PART2_STRIDE;
+        const float ms = p[HD2];
+        const float f = (ms == -INFINITY) ? 1.0f : fast_exp2(ms - m_ref);
+        l_tot += p[HD2 + 1] * f;
+        const f32x4 x = *reinterpret_cast<const f32x4 *>(p + 4 * c);
+        acc.x += x.x * f; acc.y += x.y * f; acc.z += x.z * f; acc.w += x.w * f;
+    }
+    const float inv = 1.0f / l_tot;
+    if (stats && c == 0) { stats[2 * row] = m_ref; stats[2 * row + 1] = inv; }
+    if (4 * c < hd) {
+        const long long bh = row / Lq, qi = row % Lq, b = bh / H, hh = bh % H;
+        const long long at = token_major ? (((b * Lq + qi) * H + hh) * hd) : (row * hd);
+        acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+        *reinterpret_cast<f32x4 *>(out + at + 4 * c) = acc;
+    }
+}
 
 template <int KIND>
 __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
                                                                  const float *__restrict__ v, float *__restrict__ out, int H,
                                                                  int Lq, int Lk, float rT, MaskArgs mask, int strict, int nqb,
                                                                  int total_blocks, int lpt, int token_major,
-                                                                 float *__restrict__ stats, int hd) {
+                                                                 float *__restrict__ stats, int hd, int nsplit,
+                                                                 float *__restrict__ part) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                      // [2][BN][LSTR2]
     float *Vs = lds + 2 * TILE2_FLOATS;   // [2][BN][LSTR2]
     int bh, unit;
-    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    // Key split with blocks of different length: the workgroups of an odd share walk the block order backwards, so that the
+    // CU that got the longest block's first share gets the shortest block's second (the dispatcher deals both rounds out
+    // in the same order).
+    const int blk = ((lpt & 1) && (blockIdx.y & 1)) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    if (!dl4s_work_order::work_item_at(blk, nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -104,7 +144,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__r
         for (int i = 0; i < 16; ++i) o[c][i] = 0.f;
     float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
 
-    if (ntiles > 0) { load_tile(0); store_tile(0); }
+    // Key split over workgroups (small launches): workgroup blockIdx.y of nsplit takes the key tiles y, y + nsplit, ... -
+    // an assignment that does not depend on how many tiles the mask lets the block skip, so skipping keeps the bits.
+    const int sp = blockIdx.y;
+    if (sp < ntiles) { load_tile(sp); store_tile(0); }
     __syncthreads();
 
     const int k_lds = ln * LSTR2 + half * 64;        // K fragment base: row ln, columns 64*half ..
@@ -113,10 +156,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__r
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
 
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        const bool more = (t + 1 < ntiles);
-        if (more) load_tile(t + 1);
+    for (int t = sp, it = 0; t < ntiles; t += nsplit, ++it) {
+        const int buf = it & 1;
+        const bool more = (t + nsplit < ntiles);
+        if (more) load_tile(t + nsplit);
         const int k0 = t * BN;
         int cls = 2;
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
@@ -163,6 +206,20 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__r
 
     // ---- normalise and store.  Register r of accumulator c is d = 4*(8(r/4) + 4*half + r%4) + c.
     const float l_tot = l_run + xor32(l_run);
+    if (part) {   // this workgroup's share of the keys: the weighted sums as they are, with their reference maximum and row sum
+        if (qi < Lq) {
+            const long long pairs = total_blocks / nqb;
+            float *pp = part + (((long long)sp * pairs + bh) * Lq + qi) * PART2_STRIDE;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int d0 = 4 * (8 * (r >> 2) + 4 * half + (r & 3));
+                const f32x4 a = {o[0][r], o[1][r], o[2][r], o[3][r]};
+                *reinterpret_cast<f32x4 *>(pp + d0) = a;
+            }
+            if (half == 0) { pp[HD2] = m_run; pp[HD2 + 1] = l_tot; }
+        }
+        return;
+    }
     const float inv = 1.0f / l_tot;
     if (stats && half == 0 && qi < Lq) {
         stats[2 * ((long long)bh * Lq + qi)] = m_use;
@@ -182,7 +239,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__r
 
 template <int KIND>
 int launch_d128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
-                float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+                float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit, float *part) {
     const int nqb = (Lq + BM - 1) / BM;
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
@@ -196,9 +253,15 @@ int launch_d128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
         attr_set[KIND] = true;
     }
-    hipLaunchKernelGGL(sdpa_prefill_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_bytes, ctx->stream, q, k, v,
-                       out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd);
-    return dl4s::launch_status("sdpa_prefill_f32_d128");
+    if (nsplit <= 1 || !part) { nsplit = 1; part = nullptr; }
+    hipLaunchKernelGGL(sdpa_prefill_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
+                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part);
+    int st = dl4s::launch_status("sdpa_prefill_f32_d128");
+    if (st != DL4S_HIP_OK || nsplit == 1) return st;
+    const long long rows = (long long)B * H * Lq;
+    hipLaunchKernelGGL(sdpa_prefill_merge_d128, dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, ctx->stream, part, out, stats, nsplit, rows,
+                       H, Lq, hd, token_major);
+    return dl4s::launch_status("sdpa_prefill_merge_d128");
 }
 
 }  // namespace
