@@ -142,10 +142,10 @@ typedef struct dl4s_mask_desc {
                                     caller can drop the four permuteAxes copies.  Needs the MFMA kernel's conditions (see
                                     dl4s_hip_sdpa_fwd_f32). */
 #define DL4S_SDPA_NO_KEY_SPLIT 4u /* small launches (fewer 32-query blocks than about two per SIMD) normally split each
-                                     block's keys over the 4 wavefronts of a workgroup and merge the partial softmax
-                                     results; this flag keeps the one-wavefront-per-block kernel.  The two agree within
-                                     rounding (different summation order over keys), each well inside the parity
-                                     tolerance. */
+                                     block's keys over the 4 wavefronts of a workgroup (head dims up to 64) or over
+                                     several workgroups (head dims above 64) and merge the partial softmax results;
+                                     this flag keeps the unsplit kernel.  The two agree within rounding (different
+                                     summation order over keys), each well inside the parity tolerance. */
 
 /* out = softmax((q * inv_temperature) . k^T - mask * 1e9, axis = keys) . v
  * NN/Models/Transformer/ScaledDotProductAttention.swift:43-64.  q [B,H,Lq,dk], k [B,H,Lk,dk],
