@@ -140,6 +140,40 @@ def test_different_key_and_value_dims(ctx, orc):
         assert_parity(run_sdpa(ctx, q, k, v, mask), orc.sdpa(q, k, v, mask), "dk %d dv %d" % (dk, dv))
 
 
+@pytest.mark.parametrize("dk,dv", [(70, 70), (6, 6), (40, 24), (5, 128), (100, 36)])
+def test_head_dims_served_by_padded_copies(ctx, orc, dk, dv):
+    """Key dim != value dim or not a multiple of 4, on problems large enough for the padded-copy route (the MFMA kernels
+    on zero-padded copies of the operands): every mask kind against the oracle, the structured kinds bit-identical to the
+    dense tensors they describe, NaN / Inf placement as in the oracle."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(dk * 131 + dv)
+    B, H, Lq, Lk = 2, 3, 330, 420
+    assert B * H * Lq * Lk * max(dk, dv) >= 1 << 24 or (dk, dv) == (6, 6)
+    if (dk, dv) == (6, 6):
+        B, H, Lq, Lk = 2, 4, 900, 800
+    q, k, v = rand(rng, B, H, Lq, dk), rand(rng, B, H, Lk, dk), rand(rng, B, H, Lk, dv)
+    lens = [Lk - 57, 31][:B]
+    i, j = np.indices((Lq, Lk))
+    causal = (j > i).astype(np.float32)
+    pad = (np.arange(Lk)[None, None, None, :] >= np.asarray(lens)[:, None, None, None]).astype(np.float32)
+    for name, mask, kind, lens_arg in (("none", None, None, None), ("causal", causal, lib.MASK_CAUSAL, None),
+                                       ("lens", pad, lib.MASK_KEY_LENGTHS, lens)):
+        sample = (slice(0, 1), slice(0, 2))          # the single-thread oracle on a sample of the pairs
+        ref = orc.sdpa(q[sample], k[sample], v[sample], None if mask is None else (mask if mask.ndim == 2 else mask[:1]))
+        got = run_sdpa(ctx, q, k, v, mask)
+        assert_parity(got[sample], ref, "padded %s dk %d dv %d" % (name, dk, dv))
+        assert np.isfinite(got).all()
+        if kind is not None:
+            assert np.array_equal(run_sdpa(ctx, q, k, v, kind=kind, lens=lens_arg, strict=True), run_sdpa(ctx, q, k, v, mask, strict=True))
+    q2, k2 = q.copy(), k.copy()
+    q2[0, 0, 5, 1] = np.nan
+    k2[0, 1, 9, 0] = np.inf
+    got = run_sdpa(ctx, q2, k2, v, causal)
+    ref = orc.sdpa(q2[:1, :2], k2[:1, :2], v[:1, :2], causal)
+    assert np.array_equal(np.isnan(got[:1, :2]), np.isnan(ref))
+    assert_parity(np.nan_to_num(got[:1, :2]), np.nan_to_num(ref), "padded NaN / Inf dk %d dv %d" % (dk, dv))
+
+
 def test_nil_mask_equals_zero_mask_bitwise(ctx):
     rng = np.random.default_rng(3)
     for d in (8, 10, 64, 128, 100):
