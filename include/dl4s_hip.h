@@ -153,8 +153,10 @@ typedef struct dl4s_mask_desc {
  * fp32 reciprocal the reference forms once (Engine/CPU/CPUEngine.swift:635).  mask may be NULL
  * (= DL4S_MASK_NONE).  dk = dv, a multiple of 4 and at most 128, with 16-byte aligned tensors runs
  * a fused MFMA kernel (one written for 64, one for 128; smaller head dims are padded with zero
- * columns on the fly and cost as much as the width they are padded to); other sizes up to 256 run a
- * plain fused kernel. */
+ * columns on the fly and cost as much as the width they are padded to).  Other head dims up to 128
+ * (dk != dv, not a multiple of 4, unaligned tensors) run the same kernels on zero-padded copies of the
+ * operands, which the call allocates from the context's pool, when the problem is large enough to pay
+ * for the copies; small problems and head dims up to 256 run a plain fused kernel. */
 int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
                           int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
