@@ -302,12 +302,14 @@ def other_configs(ctx, lib, cpu, only=None):
             b_.release()
     if want("masks_and_head_dim"):
         # the headline shape with the mask as an unmodified DL4S passes it (a dense [L,L] tensor): all-ones tiles skipped
-        # (default) and every tile visited (DL4S_SDPA_STRICT); and the same shape with head dim 128 (causal descriptor)
+        # (default) and every tile visited (DL4S_SDPA_STRICT); the same shape with head dim 128 (causal descriptor); and with
+        # head dim 70, which the MFMA kernels take through zero-padded copies of the operands
         B, H, L = 8, 16, 2048
         rng = np.random.Generator(np.random.PCG64(1008))
         i, j = np.indices((L, L))
         dmask = ctx.to_device((j > i).astype(np.float32))
-        for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal")):
+        for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal"),
+                        (70, "config4_shape_head_dim_70_causal_on_padded_copies")):
             qkv = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(3)]
             o = ctx.empty((B, H, L, d))
             rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
