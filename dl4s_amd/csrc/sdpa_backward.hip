@@ -928,14 +928,18 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                  "sdpa backward: extents too large");
     // head dims that are multiples of 4 up to 64 run on the MFMA kernels (tiles padded with zero columns) when every row
     // starts on a 16-byte boundary
-    const bool mfma_path = d > 0 && d <= HD && d % 4 == 0 &&
-                           ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
-                             reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dout) | reinterpret_cast<uintptr_t>(dq) |
-                             reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
-    const bool mfma128_path = d > HD && d <= HD2 && d % 4 == 0 &&
-                              ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
-                                reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dout) | reinterpret_cast<uintptr_t>(dq) |
-                                reinterpret_cast<uintptr_t>(dk) | reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
+    // The route follows the forward pass's rule (head dim, alignment of q, k, v, out): the two kinds of kernels keep the
+    // row statistics in different forms (base-2 and natural exponent), so the gradient call must land where the forward
+    // call landed.  On the MFMA route the gradient tensors have to be aligned as well.
+    const bool fwd_aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                               reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const bool grads_aligned = ((reinterpret_cast<uintptr_t>(dout) | reinterpret_cast<uintptr_t>(dq) | reinterpret_cast<uintptr_t>(dk) |
+                                 reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
+    const bool mfma_path = d > 0 && d <= HD && d % 4 == 0 && fwd_aligned;
+    const bool mfma128_path = d > HD && d <= HD2 && d % 4 == 0 && fwd_aligned;
+    DL4S_REQUIRE(!(mfma_path || mfma128_path) || grads_aligned, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa backward: dout, dq, dk and dv must be 16-byte aligned when q, k, v and out are (the forward pass ran on "
+                 "the MFMA kernels and left its row statistics in their form)");
     DL4S_REQUIRE(!mfma128_path || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * d * 4 < (d == HD2 ? (1ll << 31) : (1ll << 30)),
                  DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB (1 GiB for padded head dims)");

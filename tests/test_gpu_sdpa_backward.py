@@ -204,6 +204,12 @@ def test_backward_argument_errors(ctx):
         ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 10, 0.5, None, lib.SDPA_TOKEN_MAJOR)
     with pytest.raises(lib.Dl4sHipError):       # unknown flag
         ctx.sdpa_bwd(a, a, a, a, a, a, a, a, a, 1, 1, 4, 4, 8, 0.5, None, 128)
+    # aligned q, k, v, out mean the forward pass ran on the MFMA kernels: a gradient tensor off the 16-byte grid is refused
+    # rather than sent to the plain kernels, which read the row statistics in another form
+    with pytest.raises(lib.Dl4sHipError, match="16-byte aligned"):
+        ctx.sdpa_bwd(a, a, a, a, a, a.offset(4), a, a, a, 1, 1, 4, 4, 8, 0.5)
+    with pytest.raises(lib.Dl4sHipError, match="16-byte aligned"):
+        ctx.sdpa_bwd(a, a, a, a, a, a, a.offset(8), a, a, 1, 1, 4, 4, 64, 0.5)
     a.release()
 
 
