@@ -1331,8 +1331,10 @@ struct Transformer {
             Device::Engine::argmaxTo(logits.values(), token, position);
         };
         RecordedCalls replayable;
+        // recording and instantiating the step costs a few eager steps: not for short decodes
+        const bool replay = recorded && maxLength >= 16 && dl4s_hip_graph_supported();
         for (int64_t i = 0; i < maxLength; ++i) {
-            if (i == 0 || !recorded || !dl4s_hip_graph_supported()) {
+            if (i == 0 || !replay) {
                 step();                       // the first step also sizes the library's scratch block
             } else {
                 if (!replayable) replayable.record(step);

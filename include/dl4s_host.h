@@ -94,8 +94,9 @@ int dl4s_host_transformer_set_norm_per_token(dl4s_host_transformer *t, int per_t
 /* No counterpart in the reference.  Greedy decoding with key / value caches: each step runs the decoder on the one new
  * position (dl4s_hip_sdpa_decode_step_at_f32 over the layer's cache, dl4s_hip_sdpa_decode_f32 over the encoder states'
  * projections) instead of re-running the prefix.  The step's token and position stay in device memory, so every step
- * issues the same calls: with recorded != 0 they are recorded into a HIP graph at the second step and replayed from
- * then on, with recorded == 0 issued one by one (same results, bit for bit).  Other arguments as
+ * issues the same calls: with recorded != 0 (and max_length of at least 16: recording costs a few steps) they are
+ * recorded into a HIP graph at the second step and replayed from then on, with recorded == 0 issued one by one (same
+ * results, bit for bit).  Other arguments as
  * dl4s_host_transformer_greedy.  Requires fused mode,
  * head dim 64 and a model set to normalise per token (error otherwise: with the reference's joint normalisation a cache
  * computes a different function).  For such a model it returns the tokens of dl4s_host_transformer_greedy, and the same

@@ -210,7 +210,7 @@ def test_cached_greedy_decoding(ctx):
     vocab = CONFIGS[name][0]
     params, rng = _model(47, *CONFIGS[name])
     src = [int(t) for t in rng.integers(0, vocab, 11)]
-    steps = 12
+    steps = 20          # long enough for the recorded step (decodes of 16 tokens or more)
     ref_tokens, ref_logits = T.greedy_decode(params, src, 1, -5, steps, return_logits=True, norm_per_token=True)
     assert len(ref_tokens) == steps
     top2 = np.sort(np.stack(ref_logits), axis=1)[:, -2:]
