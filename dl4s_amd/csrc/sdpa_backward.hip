@@ -937,6 +937,31 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                                  reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
     const bool mfma_path = d > 0 && d <= HD && d % 4 == 0 && fwd_aligned;
     const bool mfma128_path = d > HD && d <= HD2 && d % 4 == 0 && fwd_aligned;
+    // the forward pass ran on zero-padded copies (sdpa_padded_route): so does this call, gradients included
+    if (!token_major && sdpa_padded_route(mfma_path || mfma128_path, B, H, Lq, Lk, d, d)) {
+        const int64_t dp = (d + 3) / 4 * 4, qrows = B * H * Lq, krows = B * H * Lk;
+        const int64_t rows_of[8] = {qrows, krows, krows, qrows, qrows, qrows, krows, krows};   // q k v out dout dq dk dv
+        void *bufs[8] = {nullptr};
+        for (int i = 0; i < 8; ++i)
+            if (dl4s_hip_alloc(ctx, (size_t)(rows_of[i] * dp) * sizeof(float), &bufs[i]) != DL4S_HIP_OK) {
+                for (int j = 0; j < i; ++j) (void)dl4s_hip_free(ctx, bufs[j]);
+                return DL4S_HIP_EOOM;
+            }
+        float *p[8];
+        for (int i = 0; i < 8; ++i) p[i] = static_cast<float *>(bufs[i]);
+        const float *src[5] = {q, k, v, out, dout};
+        for (int i = 0; i < 5; ++i) launch_copy_rows(ctx, src[i], p[i], rows_of[i], d, dp);
+        int rc = dl4s::launch_status("copy_rows_f32");
+        if (rc == DL4S_HIP_OK)
+            rc = dl4s_hip_sdpa_bwd_f32(ctx, p[0], p[1], p[2], p[3], stats, p[4], p[5], p[6], p[7], B, H, Lq, Lk, dp, inv_temperature, mask, flags);
+        if (rc == DL4S_HIP_OK) {
+            float *dst[3] = {dq, dk, dv};
+            for (int i = 0; i < 3; ++i) launch_copy_rows(ctx, p[5 + i], dst[i], rows_of[5 + i], dp, d);
+            rc = dl4s::launch_status("copy_rows_f32");
+        }
+        for (int i = 0; i < 8; ++i) (void)dl4s_hip_free(ctx, bufs[i]);
+        return rc;
+    }
     DL4S_REQUIRE(!(mfma_path || mfma128_path) || grads_aligned, DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: dout, dq, dk and dv must be 16-byte aligned when q, k, v and out are (the forward pass ran on "
                  "the MFMA kernels and left its row statistics in their form)");

@@ -2,6 +2,8 @@
 // descriptor as the kernels see it, the dense-mask tile classifier, the masked score tile and the plain-kernel helpers.
 #pragma once
 #include "common.h"
+
+#include <algorithm>
 #include "work_order.h"
 
 namespace {
@@ -259,6 +261,30 @@ __device__ __forceinline__ float plain_score(const float *qs, const float *krow,
 
 // Validates a mask descriptor against [B,H,Lq,Lk], fills the kernels' view of it and, for dense masks on the MFMA
 // kernels, launches the tile classifier (its result lives in the context's scratch block until the next call that uses it).
+// Head dims the MFMA kernels do not take as they are (not a multiple of 4, key dim != value dim, q / k / v / out off the
+// 16-byte grid), up to 128, on a problem large enough to pay for streaming copies: the kernels run on zero-padded copies.
+// The forward call that leaves row statistics and the gradient call evaluate this on the same arguments, so both land
+// on the same kind of kernel.
+inline bool sdpa_padded_route(bool mfma_as_is, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv) {
+    const int64_t dmax = dk > dv ? dk : dv;
+    return !mfma_as_is && dk > 0 && dv > 0 && dmax <= HD2 && (double)B * H * Lq * Lk * (double)dmax >= (double)(1ll << 24);
+}
+
+// rows x d_src -> rows x d_dst: the common columns copied, the rest of a wider destination zeroed
+__global__ void copy_rows_f32(const float *__restrict__ src, float *__restrict__ dst, long long rows, int d_src, int d_dst) {
+    const long long n = rows * d_dst;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        const long long r = i / d_dst;
+        const int c = (int)(i - r * d_dst);
+        dst[i] = c < d_src ? src[r * d_src + c] : 0.0f;
+    }
+}
+inline void launch_copy_rows(dl4s_hip_ctx *ctx, const float *src, float *dst, long long rows, int64_t d_src, int64_t d_dst) {
+    const long long n = rows * d_dst;
+    const unsigned grid = (unsigned)std::min<long long>((n + 1023) / 1024, 65536);
+    hipLaunchKernelGGL(copy_rows_f32, dim3(grid), dim3(256), 0, ctx->stream, src, dst, rows, (int)d_src, (int)d_dst);
+}
+
 // extra_bytes / extra: the caller's own share of the scratch block (partial results), placed behind the mask classes so
 // that one sizing of the block covers both (growing it later would move the classes away from under m.cls).
 inline int build_mask_args(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,

@@ -549,16 +549,6 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
 }  // namespace
 
 namespace {
-// rows x d_src -> rows x d_dst: the common columns copied, the rest of a wider destination zeroed
-__global__ void copy_rows_f32(const float *__restrict__ src, float *__restrict__ dst, long long rows, int d_src, int d_dst) {
-    const long long n = rows * d_dst;
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
-        const long long r = i / d_dst;
-        const int c = (int)(i - r * d_dst);
-        dst[i] = c < d_src ? src[r * d_src + c] : 0.0f;
-    }
-}
-
 int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, float *stats, int64_t B,
                         int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv, float inv_temperature, const dl4s_mask_desc *mask,
                         uint32_t flags);
@@ -583,9 +573,7 @@ int sdpa_forward_padded(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     float *qp = static_cast<float *>(bufs[0]), *kp = static_cast<float *>(bufs[1]), *vp = static_cast<float *>(bufs[2]),
           *op = static_cast<float *>(bufs[3]);
     const auto copy = [&](const float *src, float *dst, long long rows, int64_t ds, int64_t dd) {
-        const long long n = rows * dd;
-        const unsigned grid = (unsigned)std::min<long long>((n + 1023) / 1024, 65536);
-        hipLaunchKernelGGL(copy_rows_f32, dim3(grid), dim3(256), 0, ctx->stream, src, dst, rows, (int)ds, (int)dd);
+        launch_copy_rows(ctx, src, dst, rows, ds, dd);
     };
     copy(q, qp, qrows, dk, dp);
     copy(k, kp, krows, dk, dp);
@@ -679,11 +667,12 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
         }
     }
     DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 128, and 16-byte aligned tensors");
-    // Large enough to pay for four copies: the MFMA kernels on padded copies of the operands.  Not when row statistics
-    // are asked for: the gradient kernels for these head dims read them in the plain kernel's (natural exponent) form.
-    if (!stats && dk <= HD2 && dv <= HD2 && dv > 0 && (double)B * H * Lq * Lk * (double)std::max(dk, dv) >= (double)(1ll << 24)) {
+    // Large enough to pay for four copies: the MFMA kernels on padded copies of the operands.  When row statistics are
+    // asked for there is no falling back to the plain kernel: the gradient call decides by the same rule and reads the
+    // statistics in the MFMA kernels' form.
+    if (sdpa_padded_route(false, B, H, Lq, Lk, dk, dv)) {
         const int rc = sdpa_forward_padded(ctx, q, k, v, out, stats, B, H, Lq, Lk, dk, dv, inv_temperature, mask, flags);
-        if (rc != DL4S_HIP_EOOM && rc != DL4S_HIP_EUNSUPPORTED) return rc;   // else: the plain kernel below
+        if (stats || (rc != DL4S_HIP_EOOM && rc != DL4S_HIP_EUNSUPPORTED)) return rc;   // else: the plain kernel below
     }
     DL4S_REQUIRE(dk <= GEN_MAXD && dv <= GEN_MAXD && dv > 0, DL4S_HIP_EUNSUPPORTED,
                  "sdpa: head dims (%lld, %lld) above %d are not implemented", (long long)dk, (long long)dv, GEN_MAXD);

@@ -173,8 +173,10 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
  *                                same mask and flags as the forward call (the mask takes no gradient)
  * Layouts follow the forward call ([B,H,L,d], or [B,L,H,d] with DL4S_SDPA_TOKEN_MAJOR; stats is always [B,H,Lq,2]).
  * The gradient call takes the route the forward call took (MFMA kernels for d a multiple of 4 up to 128 with 16-byte
- * aligned q, k, v, out; the plain kernels otherwise) because the two keep the statistics in different forms; on the MFMA
- * route dout, dq, dk, dv must be 16-byte aligned too (DL4S_HIP_EUNSUPPORTED otherwise).
+ * aligned q, k, v, out; the same kernels on zero-padded copies for other d up to 128 on large problems; the plain
+ * kernels otherwise) because the two kinds of kernels keep the statistics in different forms: pass both calls the same
+ * tensors and extents.  On the direct MFMA route dout, dq, dk, dv must be 16-byte aligned too (DL4S_HIP_EUNSUPPORTED
+ * otherwise).
  * Deterministic: no atomics, the same bits on every run. */
 int dl4s_hip_sdpa_fwd_stats_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, float *stats,
                                 int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t d, float inv_temperature,
