@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -33,13 +34,17 @@ struct dl4s_hip_ctx {
     // Stream capture (dl4s_hip_graph_begin .. dl4s_hip_graph_end): entry points that would wait for the stream, copy to or
     // from host memory or change device allocations refuse to run while it is set.  scratch_generation counts the
     // regrowths of the scratch block; a captured graph holds the block's address and is refused once it has moved.
-    bool capturing = false;
+    std::atomic<bool> capturing{false};
     unsigned long long scratch_generation = 0;
     // Blocks handed back with dl4s_hip_free while a graph is being recorded: the recorded kernels still use them on every
     // replay, so they stay out of the pool until the graph is destroyed (dl4s_hip_graph_end moves the list to the graph).
     // Allocations made later in the same recording may take them.
     std::vector<std::pair<void *, size_t>> held_by_recording;
     size_t bytes_held = 0;
+    // One bit per (kernel family, mask kind): the dynamic-LDS limit of those kernels has been raised on this context's
+    // device (hipFuncSetAttribute is per device; two host threads that both find a bit clear both set the attribute, which
+    // is harmless, and then the bit).
+    std::atomic<unsigned long long> lds_limit_raised{0};
 };
 
 struct dl4s_hip_graph {
@@ -84,6 +89,15 @@ int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes);
     do {                                                                 \
         if (!(cond)) return dl4s::set_error((code), __VA_ARGS__);        \
     } while (0)
+
+// Kernel families of dl4s_hip_ctx::lds_limit_raised.
+enum { LDS_PREFILL_SPLIT = 0, LDS_PREFILL = 1, LDS_PREFILL_D128 = 2, LDS_BWD = 3, LDS_BWD_D128 = 4 };
+inline bool lds_limit_pending(const dl4s_hip_ctx *ctx, int family, int kind) {
+    return !(ctx->lds_limit_raised.load(std::memory_order_acquire) & (1ull << (family * 8 + kind)));
+}
+inline void lds_limit_done(dl4s_hip_ctx *ctx, int family, int kind) {
+    ctx->lds_limit_raised.fetch_or(1ull << (family * 8 + kind), std::memory_order_release);
+}
 
 inline int launch_status(const char *kernel) {
     hipError_t e = hipGetLastError();

@@ -43,6 +43,8 @@ int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes) {
         DL4S_HIP_TRY(hipFree(ctx->scratch));
         ctx->scratch = nullptr;
         ctx->scratch_bytes = 0;
+        // graphs recorded so far hold the freed address: they are refused from here on, whether or not the new block comes
+        ++ctx->scratch_generation;
     }
     size_t want = round_size(bytes);
     DL4S_HIP_TRY(hipMalloc(&ctx->scratch, want));

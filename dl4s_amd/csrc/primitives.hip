@@ -498,14 +498,17 @@ __global__ void embed_at_f32(const float *__restrict__ table, const int *__restr
 
 // Embedding lookup with the scale and positional term of Transformer.prepareInputs folded in:
 // out[t][:] = (token[t] == ignore ? 0 : table[token[t]][:]) * scale + positions[t % L][:]
+// A token outside [0, vocab) that is not the ignore index is a caller's mistake (the reference's subscript traps on it); the
+// table is never read out of bounds for it: such a token embeds as a row of NaN, which no later step can hide.
 __global__ void embed_positions_f32(const float *__restrict__ table, const int *__restrict__ tokens, const float *__restrict__ pos,
-                                    float *__restrict__ out, long long ntok, long long L, long long D, int ignore, float scale,
-                                    int has_scale) {
+                                    float *__restrict__ out, long long ntok, long long L, long long D, long long vocab, int ignore,
+                                    float scale, int has_scale) {
     const long long n = ntok * D;
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
         const long long t = i / D, c = i % D;
         const int tok = tokens[t];
-        float v = tok == ignore ? 0.0f : table[(long long)tok * D + c];
+        float v = 0.0f;
+        if (tok != ignore) v = (tok >= 0 && tok < vocab) ? table[(long long)tok * D + c] : __builtin_nanf("");
         if (has_scale) v = __fmul_rn(v, scale);
         if (pos) v = __fadd_rn(v, pos[(t % L) * D + c]);
         out[i] = v;
@@ -885,9 +888,9 @@ int dl4s_hip_embed_positions_f32(dl4s_hip_ctx *ctx, const float *table, int64_t 
     const long long n = batch * L * D;
     if (n == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(table && tokens && result, DL4S_HIP_EINVALID_ARG, "embedding: NULL pointer");
-    // token values are not checked on the device: the caller (like the reference's subscript) must keep them in range
     hipLaunchKernelGGL(embed_positions_f32, dim3(grid_for(n)), dim3(TPB), 0, ctx->stream, table, tokens, positions, result,
-                       (long long)(batch * L), (long long)L, (long long)D, (int)ignore_index, scale ? *scale : 1.0f, scale ? 1 : 0);
+                       (long long)(batch * L), (long long)L, (long long)D, (long long)vocab, (int)ignore_index,
+                       scale ? *scale : 1.0f, scale ? 1 : 0);
     return dl4s::launch_status("embedding");
 }
 

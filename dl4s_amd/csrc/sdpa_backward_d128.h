@@ -329,7 +329,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                     for (int r = 0; r < 16; ++r) {
                         const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
                         const int qc = qg < Lq ? qg : Lq - 1;
-                        p[r] = __fsub_rn(p[r], __fmul_rn(__fmul_rn(mcol[qc * mask.sq], 1e9f), LOG2E));
+                        p[r] = __fsub_rn(p[r], dense_penalty2(mcol[qc * mask.sq]));
                     }
                 }
             } else if ((CAUSAL && (kw0 + 31 > qt0)) || (LENS && (kw0 + 32 > len))) {
@@ -378,15 +378,14 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
                   const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
                   int strict, int token_major, int hd) {
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
-    static bool attr_set[8] = {false};
     const size_t lds_dq = 4 * TILE2_FLOATS * sizeof(float);
     const size_t lds_dkv = (4 * TILE2_FLOATS + 192) * sizeof(float);
-    if (!attr_set[KIND]) {
+    if (dl4s::lds_limit_pending(ctx, dl4s::LDS_BWD_D128, KIND)) {
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_f32_d128<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq));
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
-        attr_set[KIND] = true;
+        dl4s::lds_limit_done(ctx, dl4s::LDS_BWD_D128, KIND);
     }
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
     {

@@ -173,6 +173,17 @@ __device__ __forceinline__ bool work_item(const int nunits, const int total_bloc
     return dl4s_work_order::work_item_at((int)blockIdx.x, nunits, total_blocks, lpt, bh, unit, snake);
 }
 
+// The penalty of a dense mask value in the base-2 exponent domain, fl(fl(m * 1e9) * log2 e).  The reference subtracts
+// fl(m * 1e9) from the natural-domain score (ScaledDotProductAttention.swift:55-57).  Where that is finite but its product
+// with log2 e is not (|m * 1e9| above 2.36e38) the penalty stays at the largest finite float: a row blocked by such values
+// then comes out uniform, as the reference's does, instead of NaN.  (Different penalties in that last sliver of the float
+// range count as equal here.)
+__device__ __forceinline__ float dense_penalty2(const float mval) {
+    const float pen = __fmul_rn(mval, 1e9f);
+    const float pen2 = __fmul_rn(pen, LOG2E);
+    return (__builtin_isinf(pen2) && !__builtin_isinf(pen)) ? __builtin_copysignf(3.402823466e38f, pen) : pen2;
+}
+
 // S^T = K . Q^T for one 32-key tile of one wavefront (lane = query qi = q0 + lane % 32, 16 of the 32 keys per lane:
 // accumulator register r is key k0 + 8(r/4) + 4*half + r%4), then the mask, in registers.  Kb is the lane's K fragment
 // base in LDS; qr the lane's Q fragment, already scaled by (1/T) log2(e): the scores are in the base-2 exponent domain.
@@ -211,7 +222,7 @@ __device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&q
             for (int r = 0; r < 16; ++r) {
                 const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
                 const int kc = kg < Lk ? kg : Lk - 1;
-                s0[r] = __fsub_rn(s0[r], __fmul_rn(__fmul_rn(mrow[kc * msk], 1e9f), LOG2E));
+                s0[r] = __fsub_rn(s0[r], dense_penalty2(mrow[kc * msk]));
             }
         }
     } else if ((CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len))) {

@@ -112,6 +112,11 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
             if (APPEND) vp = (kc == pos) ? vn_row : vp;
             vv[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(vp));
         }
+        if (kb + KB > c1) {     // the range's last block: lanes past its end re-read row T-1 and must add nothing, not 0 * Inf
+#pragma unroll
+            for (int i = 0; i < KB / 4; ++i)
+                if (kb + 4 * i + g >= c1) vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
         float s[KB / 4];
         float bm = -INFINITY;
 #pragma unroll

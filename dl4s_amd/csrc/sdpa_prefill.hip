@@ -504,11 +504,10 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         const long long total32 = (long long)nqb32 * B * H;
         DL4S_REQUIRE(total32 < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total32);
         const size_t lds_split = (size_t)SPLIT_WAVES * 2 * TILE_FLOATS * sizeof(float);
-        static bool split_attr_set[8] = {false};
-        if (!split_attr_set[KIND]) {
+        if (dl4s::lds_limit_pending(ctx, dl4s::LDS_PREFILL_SPLIT, KIND)) {
             DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_prefill_split_f32_d64<KIND>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_split));
-            split_attr_set[KIND] = true;
+            dl4s::lds_limit_done(ctx, dl4s::LDS_PREFILL_SPLIT, KIND);
         }
         // Rows of different length (causal masks, dense masks with tile skipping): longest first, and when the launch fits
         // the chip at once (two workgroups per CU) every second round of the CUs reversed, which pairs long rows with
@@ -532,11 +531,10 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int chunk = (int)((total + 7) / 8);
     const size_t lds_bytes = 4 * TILE_FLOATS * sizeof(float);
-    static bool attr_set[8] = {false};
-    if (!attr_set[KIND]) {
+    if (dl4s::lds_limit_pending(ctx, dl4s::LDS_PREFILL, KIND)) {
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_prefill_f32_d64<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        attr_set[KIND] = true;
+        dl4s::lds_limit_done(ctx, dl4s::LDS_PREFILL, KIND);
     }
     // a launch that fits the chip at once (three workgroups per CU): every second round of the CUs reversed as well
     // (B2 H16 L2048 causal: 203 -> 161 us, B4 H16 L1024: 106 -> 88 us)

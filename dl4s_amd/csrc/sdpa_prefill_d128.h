@@ -247,11 +247,10 @@ int launch_d128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *
     int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
     if (lpt && total <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
     const size_t lds_bytes = 4 * TILE2_FLOATS * sizeof(float);
-    static bool attr_set[8] = {false};
-    if (!attr_set[KIND]) {
+    if (dl4s::lds_limit_pending(ctx, dl4s::LDS_PREFILL_D128, KIND)) {
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_prefill_f32_d128<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-        attr_set[KIND] = true;
+        dl4s::lds_limit_done(ctx, dl4s::LDS_PREFILL_D128, KIND);
     }
     if (nsplit <= 1 || !part) { nsplit = 1; part = nullptr; }
     hipLaunchKernelGGL(sdpa_prefill_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,

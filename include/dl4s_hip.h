@@ -304,7 +304,8 @@ int dl4s_hip_bias_gelu_f32(dl4s_hip_ctx *ctx, const float *x, const float *bias,
  * with the rest of Transformer.prepareInputs (Transformer.swift:86-92) folded in when the pointers are given:
  *   result[b][l][:] = row * (*scale) + positions[l][:]
  * table [vocab, D], tokens device int32 [batch, L], positions [L, D] or NULL, scale host pointer or NULL.  Each step
- * is rounded like the separate engine calls.  Token values must lie in [0, vocab) or equal ignore_index. */
+ * is rounded like the separate engine calls.  Token values must lie in [0, vocab) or equal ignore_index (the reference's
+ * subscript traps otherwise); the table is never read for a value outside that range: its row of the result is NaN. */
 int dl4s_hip_embed_positions_f32(dl4s_hip_ctx *ctx, const float *table, int64_t vocab, int64_t D, const int32_t *tokens,
                                  int64_t batch, int64_t L, int32_t ignore_index, const float *scale, const float *positions,
                                  float *result);

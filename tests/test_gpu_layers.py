@@ -4,6 +4,8 @@ execution modes, against the CPU oracle (small and config-2 shapes) and the inde
 mode "primitive": every tensor operator issues the engine calls the reference issues (drop-in behaviour);
 mode "fused": ScaledDotProductAttention, batched matmul, residual+LayerNorm and bias+GELU use fused entries.
 """
+import sys
+
 import numpy as np
 import pytest
 
@@ -142,7 +144,8 @@ def test_config2_mha_layer_causal(ctx, host, orc, fused):
 def test_config3_encoder_block_padding_mask(ctx, host, orc):
     """TransformerEncoderBlock fp32, B8 L1024 D1024 H16 F4096, sigmoid-GELU, LayerNorm, key-length mask U[512,1024].
     The fused mode is checked against the fp64 model on the whole batch (the single-threaded oracle needs
-    minutes at this size) and the primitive mode against the fused mode on two batch items."""
+    minutes at this size), the primitive mode against the fused mode on two batch items, and all three modes against
+    the C oracle on one whole batch item."""
     B, L, D, H, dk, F = 8, 1024, 1024, 16, 64, 4096
     rng = np.random.Generator(np.random.PCG64(1003))
     x = rng.standard_normal((B, L, D), dtype=np.float32)
@@ -154,3 +157,15 @@ def test_config3_encoder_block_padding_mask(ctx, host, orc):
     assert_parity(got, ref.astype(np.float32), "config 3 vs fp64")
     prim = host.encoder_block(ctx, x[:2], mask[:2], attn, ffn, H, dk, dk, fused=False)
     assert_parity(prim, got[:2], "config 3 primitive vs fused")
+    # One whole batch item against the C oracle.  MultiHeadAttention's LayerNorm runs over (L, D) of a batch item and the
+    # feed-forward one over D of a token, so a batch item is a self-contained problem: the oracle on item b alone computes
+    # what the reference computes for item b of the batch (about 90 s of single-threaded CPU at these widths).
+    b = int(np.argmin(lens))
+    sys.__stdout__.write("\n[config 3] CPU oracle on batch item %d (%d valid keys) ...\n" % (b, lens[b]))
+    sys.__stdout__.flush()
+    ref_b = orc.encoder_block(x[b:b + 1], mask[b:b + 1], attn, ffn, H, dk, dk)
+    assert_parity(got[b:b + 1], ref_b, "config 3, batch item %d, fused vs oracle" % b)
+    strict_b = host.encoder_block(ctx, x[b:b + 1], mask[b:b + 1], attn, ffn, H, dk, dk, fused=2)
+    assert_parity(strict_b, ref_b, "config 3, batch item %d, fused strict vs oracle" % b)
+    assert_parity(prim[b:b + 1] if b < 2 else host.encoder_block(ctx, x[b:b + 1], mask[b:b + 1], attn, ffn, H, dk, dk, fused=False),
+                  ref_b, "config 3, batch item %d, primitive vs oracle" % b)

@@ -4,6 +4,8 @@ Gate: |gpu - oracle| <= 1e-4 + 1e-4 * |oracle| element-wise (fp32), NaN/Inf at e
 positions, structured masks bit-identical to the dense mask they describe, mask == nil bit-identical
 to an all-zero mask.
 """
+import zlib
+
 import numpy as np
 import pytest
 
@@ -97,7 +99,7 @@ SHAPES = [  # B, H, Lq, Lk, d
 def test_sdpa_matches_oracle(ctx, orc, shape, mk):
     from dl4s_amd import lib
     B, H, Lq, Lk, d = shape
-    rng = np.random.default_rng(hash((shape, mk)) % (2 ** 32))
+    rng = np.random.default_rng(zlib.crc32(repr((shape, mk)).encode()))   # the same inputs in every process
     q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
     lens = rng.integers(0, Lk + 1, size=B)
     lens[0] = max(1, Lk // 2)
@@ -224,6 +226,30 @@ def test_nan_inf_placement_matches_oracle(ctx, orc, d):
     assert np.isnan(ref[0, 0, 3]).all() and np.isnan(ref[0, 0, 5]).all() and np.isnan(ref[0, 0, 7]).all()
     assert not np.isnan(ref[0, 0, 9]).any() and not np.isnan(ref[0, 0, 11]).any()
     assert_parity(got, ref, "nan/inf d=%d" % d)
+
+
+@pytest.mark.parametrize("d", [8, 10, 64, 128])
+def test_mask_penalties_at_the_top_of_the_float_range(ctx, orc, d):
+    """mask * 1e9 is finite up to a mask value of 3.4e29 (the reference then subtracts about 3e38 and the row, if every key
+    has that value, comes out uniform); the kernels hold penalties in the base-2 exponent domain, where the same penalty
+    times log2(e) would be infinite and the row NaN.  Beyond 3.4e29 the reference's product is infinite as well."""
+    rng = np.random.default_rng(31)
+    B, H, Lq, Lk = 1, 2, 40, 75
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    mask = (rng.random((Lq, Lk)) < 0.3).astype(np.float32)
+    mask[3, :] = 3e29            # every key: uniform row
+    mask[5, 10:] = 3e29          # some keys: weight zero there
+    mask[7, :] = 2e29            # finite in both domains
+    mask[9, :] = 3.5e29          # mask * 1e9 overflows in the reference too: -inf everywhere, NaN row
+    mask[11, :] = -3e29          # a bonus of 3e38 on every key: uniform again
+    mask[13, 40] = -3e29         # one key takes all the weight
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa(q, k, v, mask)
+    assert np.isnan(ref[:, :, 9]).all() and np.isnan(ref).sum() == B * H * d
+    assert np.allclose(ref[:, :, 3], v.mean(axis=2), atol=1e-5) and np.array_equal(ref[:, :, 13], v[:, :, 40])
+    for strict in (False, True):
+        got = run_sdpa(ctx, q, k, v, mask, strict=strict)
+        assert_parity(got, ref, "huge mask values d=%d strict=%d" % (d, strict))
 
 
 def test_nan_in_v_at_blocked_key_reaches_output_only_in_strict_mode(ctx, orc):
@@ -375,6 +401,24 @@ def test_decode_nan_inf(ctx, orc):
     got = run_decode(ctx, q, kc, vc, T)
     assert np.isnan(ref[0, 0]).all() and np.isnan(ref[1, 1]).all() and not np.isnan(ref[0, 1]).any()
     assert_parity(got, ref, "decode nan/inf")
+
+
+@pytest.mark.parametrize("T", [1, 9, 45, 300, 1000, 2077])      # none a multiple of 32: the last block has lanes past the end
+def test_decode_non_finite_values_in_the_last_cached_row(ctx, orc, T):
+    """Lanes past the end of the cache re-read row T-1 with weight zero; they must add nothing (0 * Inf would be NaN)."""
+    rng = np.random.default_rng(T)
+    B, H = 2, 3
+    q, kc, vc = rand(rng, B, H, 1, 64), rand(rng, B, H, T + 5, 64), rand(rng, B, H, T + 5, 64)
+    vc[0, 0, T - 1, 7] = np.inf          # a valid row: weight > 0 times Inf = Inf in that column, in the reference too
+    vc[0, 1, T - 1, 9] = -np.inf
+    vc[1, 2, T - 1, 11] = np.nan
+    kc[1, 0, T - 1, :] = 0
+    kc[1, 0, T - 1, 3] = 3e38            # the last row's score overflows for this pair
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa_decode(q, kc, vc, T)
+    assert np.isposinf(ref[0, 0, 0, 7]) and np.isneginf(ref[0, 1, 0, 9]) and np.isnan(ref[1, 2, 0, 11])
+    assert np.isfinite(ref[0, 0, 0, :7]).all() and np.isfinite(ref[0, 2]).all()
+    assert_parity(run_decode(ctx, q, kc, vc, T), ref, "decode, non-finite last row, T=%d" % T)
 
 
 def test_config5_incremental_decode_append_then_attend(ctx, orc):

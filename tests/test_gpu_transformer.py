@@ -84,6 +84,30 @@ def test_embedding_with_scale_and_positions(ctx, orc):
         x.release()
 
 
+def test_embedding_never_reads_the_table_for_a_token_out_of_range(ctx):
+    """The reference's subscript traps on a token outside [0, vocab).  The kernel does not read the table for one: the
+    token's row of the result is NaN and every other row is what it would be without it.  The table sits at the end of
+    its own small allocation, so an unchecked index of 10**9 or -7 would read far outside it."""
+    rng = np.random.default_rng(35)
+    V, D, B, L = 11, 8, 2, 5
+    E = rng.standard_normal((V, D)).astype(np.float32)
+    tok = rng.integers(0, V, (B, L)).astype(np.int32)
+    good = tok.copy()
+    tok[0, 1], tok[1, 3], tok[1, 4] = V, -7, 10 ** 9
+    pos = rng.standard_normal((L, D)).astype(np.float32)
+    dE, dt, dg, dpos = ctx.to_device(E), ctx.to_device(tok, dtype=np.int32), ctx.to_device(good, dtype=np.int32), ctx.to_device(pos)
+    dy, dyg = ctx.empty((B, L, D)), ctx.empty((B, L, D))
+    for scale, dp in ((None, None), (3.0, dpos)):
+        ctx.embed_positions(dE, V, D, dt, B, L, -1, scale, dp, dy)
+        ctx.embed_positions(dE, V, D, dg, B, L, -1, scale, dp, dyg)
+        got, want = dy.numpy(), dyg.numpy()
+        bad = np.zeros((B, L), bool)
+        bad[0, 1] = bad[1, 3] = bad[1, 4] = True
+        assert np.isnan(got[bad]).all() and np.array_equal(got[~bad], want[~bad])
+    for x in (dE, dt, dg, dpos, dy, dyg):
+        x.release()
+
+
 def test_log_softmax_rows(ctx):
     from oracle import transformer as T
     rng = np.random.default_rng(34)
