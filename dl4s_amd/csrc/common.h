@@ -31,6 +31,8 @@ struct dl4s_hip_ctx {
     // Held by an entry point from the launch that fills the scratch block to the launch that reads it, so that calls
     // from several host threads cannot interleave their use of it (the kernels themselves are ordered by the stream).
     std::mutex scratch_mu;
+    // Device address, on this context's GPU, of the fixed block dl4s_hip_sdpa_decode_noalloc_f32 keeps its partial records in.
+    float *static_scratch = nullptr;
     // Stream capture (dl4s_hip_graph_begin .. dl4s_hip_graph_end): entry points that would wait for the stream, copy to or
     // from host memory or change device allocations refuse to run while it is set.  scratch_generation counts the
     // regrowths of the scratch block; a captured graph holds the block's address and is refused once it has moved.
@@ -62,6 +64,8 @@ int set_error(int code, const char *fmt, ...);
 int hip_error(hipError_t e, const char *what);
 // Grows ctx->scratch to at least `bytes`; returns 0 or a status.
 int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes);
+// Looks up the device address of the decode kernels' fixed scratch block (sdpa_decode.hip) for the current GPU.
+int decode_static_scratch_init(dl4s_hip_ctx *ctx);
 
 #define DL4S_CHECK_CTX(ctx)                                                        \
     do {                                                                           \

@@ -90,6 +90,16 @@ int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx) {
         delete c;
         return hip_error(e, "dl4s_hip_create");
     }
+    {
+        const int rc = decode_static_scratch_init(c);
+        if (rc) {
+            (void)hipEventDestroy(c->ev_end);
+            (void)hipEventDestroy(c->ev_begin);
+            (void)hipStreamDestroy(c->stream);
+            delete c;
+            return rc;
+        }
+    }
     *out_ctx = c;
     return DL4S_HIP_OK;
 }

@@ -15,6 +15,14 @@
 // an order of magnitude slower than the two launches.)
 #include "common.h"
 
+// Partial records of dl4s_hip_sdpa_decode_noalloc_f32: a fixed block in the code object's own device memory (one copy per
+// GPU, held until the process ends), so that entry point never asks the driver for memory.  Host code must not pass this
+// name to a kernel: it uses the device address hipGetSymbolAddress returns (dl4s::decode_static_scratch_init).
+constexpr size_t NOALLOC_SCRATCH_FLOATS = size_t(1) << 19;   // 2 MiB
+static __device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
+// Serialises the two launches of a split decode on the fixed block between host threads (whatever their context).
+static std::mutex g_static_scratch_mu;
+
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -214,7 +222,7 @@ __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restr
 
 int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcache, const float *k_new,
                   const float *v_new, float *out, int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t pos,
-                  int64_t d, float rT, bool append) {
+                  int64_t d, float rT, bool append, bool fixed_scratch = false) {
     const int64_t BH = B * H;
     if (BH == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(q && kcache && vcache && out, DL4S_HIP_EINVALID_ARG, "sdpa_decode: NULL tensor pointer");
@@ -237,12 +245,22 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     chunk = (chunk + KB - 1) / KB * KB;
     const int nsplit = (int)((T + chunk - 1) / chunk);
     float *part = nullptr;
-    std::unique_lock<std::mutex> scratch_lock(ctx->scratch_mu, std::defer_lock);
+    std::unique_lock<std::mutex> scratch_lock(fixed_scratch ? g_static_scratch_mu : ctx->scratch_mu, std::defer_lock);
     if (nsplit > 1) {
+        const size_t need = (size_t)BH * nsplit * PSTR;
         scratch_lock.lock();
-        int rc = dl4s::ensure_scratch(ctx, (size_t)BH * nsplit * PSTR * sizeof(float));
-        if (rc) return rc;
-        part = reinterpret_cast<float *>(ctx->scratch);
+        if (fixed_scratch) {
+            DL4S_REQUIRE(ctx->static_scratch, DL4S_HIP_EHIP, "sdpa_decode_noalloc: the fixed scratch block has no device address");
+            DL4S_REQUIRE(need <= NOALLOC_SCRATCH_FLOATS, DL4S_HIP_EUNSUPPORTED,
+                         "sdpa_decode_noalloc: B*H=%lld pairs split %d ways need %zu bytes of partial records, the fixed block "
+                         "holds %zu: use dl4s_hip_sdpa_decode_f32", (long long)BH, nsplit, need * sizeof(float),
+                         NOALLOC_SCRATCH_FLOATS * sizeof(float));
+            part = ctx->static_scratch;
+        } else {
+            int rc = dl4s::ensure_scratch(ctx, need * sizeof(float));
+            if (rc) return rc;
+            part = reinterpret_cast<float *>(ctx->scratch);
+        }
     }
     dim3 grid(nsplit, (unsigned)BH);
 #define DL4S_DECODE_LAUNCH(AP, NW_)                                                                                    \
@@ -259,6 +277,19 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
 
 }  // namespace
 
+namespace dl4s {
+
+// Device address of the fixed scratch block on the context's GPU (each GPU holds its own copy at its own address).
+// Called by dl4s_hip_create with that GPU current.
+int decode_static_scratch_init(dl4s_hip_ctx *ctx) {
+    void *p = nullptr;
+    DL4S_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    ctx->static_scratch = reinterpret_cast<float *>(p);
+    return DL4S_HIP_OK;
+}
+
+}  // namespace dl4s
+
 extern "C" {
 
 int dl4s_hip_sdpa_decode_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache, float *out,
@@ -267,6 +298,14 @@ int dl4s_hip_sdpa_decode_f32(dl4s_hip_ctx *ctx, const float *q, const float *kca
     DL4S_REQUIRE(B >= 0 && H >= 0, DL4S_HIP_EINVALID_ARG, "sdpa_decode: negative extent");
     return decode_launch(ctx, q, const_cast<float *>(kcache), const_cast<float *>(vcache), nullptr, nullptr, out, B, H, T,
                          Tcap, -1, d, inv_temperature, false);
+}
+
+int dl4s_hip_sdpa_decode_noalloc_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache, float *out,
+                                     int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d, float inv_temperature) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(B >= 0 && H >= 0, DL4S_HIP_EINVALID_ARG, "sdpa_decode_noalloc: negative extent");
+    return decode_launch(ctx, q, const_cast<float *>(kcache), const_cast<float *>(vcache), nullptr, nullptr, out, B, H, T,
+                         Tcap, -1, d, inv_temperature, false, true);
 }
 
 int dl4s_hip_kv_append_f32(dl4s_hip_ctx *ctx, float *kcache, float *vcache, const float *k_new, const float *v_new,

@@ -202,6 +202,12 @@ class Context:
         _check(self.lib.dl4s_hip_sdpa_decode_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(kcache)), _vp(_ptr(vcache)), _vp(_ptr(out)),
                                                  _i64(B), _i64(H), _i64(T), _i64(Tcap), _i64(d), C.c_float(inv_temperature)))
 
+    def sdpa_decode_noalloc(self, q, kcache, vcache, out, B, H, T, Tcap, d, inv_temperature):
+        """sdpa_decode with its partial records in the library's fixed device block (no allocation)."""
+        _check(self.lib.dl4s_hip_sdpa_decode_noalloc_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(kcache)), _vp(_ptr(vcache)),
+                                                         _vp(_ptr(out)), _i64(B), _i64(H), _i64(T), _i64(Tcap), _i64(d),
+                                                         C.c_float(inv_temperature)))
+
     def kv_append(self, kcache, vcache, k_new, v_new, B, H, pos, Tcap, d):
         _check(self.lib.dl4s_hip_kv_append_f32(self.handle, _vp(_ptr(kcache)), _vp(_ptr(vcache)), _vp(_ptr(k_new)), _vp(_ptr(v_new)),
                                                _i64(B), _i64(H), _i64(pos), _i64(Tcap), _i64(d)))
