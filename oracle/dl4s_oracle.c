@@ -21,8 +21,14 @@
  *   orc_softmax_last         scipy.special.softmax in fp64, shift invariance, NaN/Inf table
  *   orc_sdpa                 torch.nn.functional.scaled_dot_product_attention in fp64 (additive
  *                            -1e9 mask), blocked-weight and fully-blocked-row invariants
- *   orc_layernorm            torch.nn.functional.layer_norm in fp64 (eps placement differs by
- *                            O(eps); tolerance says so) and an fp64 closed form with the quirks
+ *   orc_layernorm            torch.nn.functional.layer_norm in fp64; an fp64 closed form with the quirks,
+ *                            each on an input where the plausible mistake fails: eps outside the root on
+ *                            a low-variance input (the other placement is off by 3x), the biased variance
+ *                            on four elements, the one-pass variance on two-element rows where it is
+ *                            negative in fp32 (NaN row; a two-pass variance never is).  Far from a zero
+ *                            mean the formula's fp32 value is noise of the summation order: only the
+ *                            order this file uses (the generic engine's) is restated, and no GPU kernel
+ *                            is held to it there
  *   orc_gelu                 x * scipy.special.expit(1.702 x)
  *   orc_mha, orc_ffn,
  *   orc_encoder_block,

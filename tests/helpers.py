@@ -29,3 +29,19 @@ def causal_mask(Lq, Lk):
 
 def lengths_mask(lens, Lk):
     return (np.arange(Lk)[None, None, None, :] >= np.asarray(lens)[:, None, None, None]).astype(np.float32)
+
+
+def negative_variance_pairs(count=6):
+    """Two-element rows [a, b] whose variance by the one-pass formula E[x^2] - E[x]^2 is negative in fp32.  With two
+    elements every step has one possible order, so the fp32 value is fixed by the formula alone."""
+    f = np.float32
+    rng = np.random.default_rng(0)
+    rows = []
+    while len(rows) < count:
+        a = f(rng.uniform(1, 2))
+        b = f(a + f(rng.integers(-3, 4)) * np.spacing(a))
+        mean = f(f(a + b) * f(0.5))
+        var = f(f(f(f(a * a) + f(b * b)) * f(0.5)) - f(mean * mean))
+        if var < 0:
+            rows.append((a, b))
+    return np.array(rows, f)

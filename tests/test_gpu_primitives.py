@@ -3,7 +3,7 @@ arithmetic is a single IEEE operation, 1e-4 tolerance where summation order or l
 import numpy as np
 import pytest
 
-from helpers import assert_parity
+from helpers import assert_parity, negative_variance_pairs
 
 pytestmark = pytest.mark.gpu
 
@@ -334,6 +334,60 @@ def test_layernorm(ctx, orc, B, rows, D):
     assert_parity(dy.numpy(), orc.layernorm(x + res, scale, shift), "layernorm+residual")
     for t in (dx, dr, ds, dh, dy):
         t.release()
+
+
+def _ln(ctx, x, scale, shift):
+    B, rows, D = x.shape
+    dx, ds, dh, dy = ctx.to_device(x), ctx.to_device(scale), ctx.to_device(shift), ctx.empty((B, rows, D))
+    ctx.layernorm(dx, None, ds, dh, dy, B, rows, D)
+    y = dy.numpy()
+    for t in (dx, ds, dh, dy):
+        t.release()
+    return y
+
+
+@pytest.mark.parametrize("B,rows,D", [(3, 5, 64), (15, 1, 64), (2, 300, 68), (4, 1, 1024), (2, 1, 33)])
+def test_layernorm_low_variance_input(ctx, orc, B, rows, D):
+    """Standard deviation 1e-3: eps = 1e-5 outside the root (NN/Layer/LayerNorm.swift:75) is 1 % of the denominator;
+    inside the root it would be 3.2e-3, three times the standard deviation."""
+    x = rnd(B, rows, D) * np.float32(1e-3)
+    scale, shift = rnd(D), rnd(D)
+    got = _ln(ctx, x, scale, shift)
+    assert_parity(got, orc.layernorm(x, scale, shift), "layernorm, low variance")
+    x64 = x.astype(np.float64)
+    mean = x64.mean(axis=(1, 2), keepdims=True)
+    std = np.sqrt((x64 * x64).mean(axis=(1, 2), keepdims=True) - mean * mean)
+    assert np.allclose(got, (x64 - mean) / (std + 1e-5) * scale + shift, rtol=1e-3, atol=1e-4)
+
+
+def test_layernorm_negative_one_pass_variance_gives_nan_rows(ctx, orc):
+    """var = E[x^2] - E[x]^2 in fp32 (Tensor/Operators/Reduce.swift:106-110) is negative for some rows, the root is NaN
+    and so is the row.  On two-element rows every sum has one possible order, so the kernel must agree with the oracle on
+    which rows those are."""
+    bad = negative_variance_pairs(8)
+    good = np.array([[1.5, 2.5], [-3.0, 3.0], [0.1, 0.7]], np.float32)
+    x = np.concatenate([bad[:4], good, bad[4:]]).reshape(-1, 1, 2)
+    scale, shift = np.array([2.0, -1.0], np.float32), np.array([0.5, 0.25], np.float32)
+    with np.errstate(invalid="ignore"):
+        ref = orc.layernorm(x, scale, shift)
+    assert np.isnan(ref[:4]).all() and np.isnan(ref[7:]).all() and np.isfinite(ref[4:7]).all()
+    assert_parity(_ln(ctx, x, scale, shift), ref, "layernorm, negative variance")
+
+
+@pytest.mark.parametrize("rows,D", [(1, 1024), (64, 512)])
+def test_layernorm_off_centre_input(ctx, orc, rows, D):
+    """The one-pass variance loses (mean / std)^2 * 2^-24 of relative precision per rounding of the sums.  Up to a mean
+    of 3 standard deviations the kernel's tree sums and the oracle's sequential sums agree inside the parity gate.  At
+    1000 standard deviations the formula's fp32 value is rounding noise of whichever summation order is used (the
+    oracle pins show the same formula with pairwise sums as far from the sequential sums as from the exact result), so
+    only what every order shares is asserted: a row is NaN as a whole or not at all."""
+    scale, shift = np.ones(D, np.float32), np.zeros(D, np.float32)
+    near = rnd(8, rows, D) + np.float32(3)
+    assert_parity(_ln(ctx, near, scale, shift), orc.layernorm(near, scale, shift), "layernorm, mean = 3 std")
+    far = rnd(8, rows, D) + np.float32(1000)
+    got = _ln(ctx, far, scale, shift)
+    nan_rows = np.isnan(got).any(axis=(1, 2))
+    assert np.array_equal(nan_rows, np.isnan(got).all(axis=(1, 2)))
 
 
 def test_bias_gelu(ctx, orc):

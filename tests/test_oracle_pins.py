@@ -6,6 +6,8 @@ import numpy as np
 import pytest
 import scipy.special
 
+from helpers import negative_variance_pairs
+
 RNG = np.random.default_rng(7)
 
 
@@ -286,6 +288,81 @@ def test_layernorm_vs_torch_and_closed_form(orc):
     x2 = x.reshape(21, 16)
     lib2 = torch.nn.functional.layer_norm(torch.from_numpy(x2.astype(np.float64)), (16,), eps=0.0).numpy()
     assert np.allclose(orc.layernorm(x2, ones, zeros), lib2, rtol=1e-4, atol=1e-4)
+
+
+def test_layernorm_eps_sits_outside_the_root(orc):
+    """NN/Layer/LayerNorm.swift:75: (x - mean) / (sqrt(var) + eps).  On an input of standard deviation 1e-3 the two
+    placements of eps differ by a factor of about three, so the wrong one cannot pass."""
+    x = (RNG.standard_normal((3, 5, 64)) * 1e-3).astype(np.float32)
+    ones, zeros = np.ones(64, np.float32), np.zeros(64, np.float32)
+    x64 = x.astype(np.float64)
+    mean = x64.mean(axis=(1, 2), keepdims=True)
+    var = (x64 * x64).mean(axis=(1, 2), keepdims=True) - mean * mean
+    outside = (x64 - mean) / (np.sqrt(var) + 1e-5)
+    inside = (x64 - mean) / np.sqrt(var + 1e-5)
+    got = orc.layernorm(x, ones, zeros)
+    assert np.allclose(got, outside, rtol=2e-4, atol=1e-6)
+    assert np.abs(outside).max() > 2.5 * np.abs(inside).max()          # what the wrong placement would give
+    # per token (2-D input), same rule
+    x2 = x.reshape(15, 64)
+    x264 = x2.astype(np.float64)
+    m2 = x264.mean(axis=1, keepdims=True)
+    v2 = (x264 * x264).mean(axis=1, keepdims=True) - m2 * m2
+    assert np.allclose(orc.layernorm(x2, ones, zeros), (x264 - m2) / (np.sqrt(v2) + 1e-5), rtol=2e-4, atol=1e-6)
+
+
+def test_layernorm_variance_is_the_biased_one(orc):
+    """Tensor/Operators/Reduce.swift:106-110 divides by N, not N - 1: on four elements the two differ by 15 %."""
+    x = np.array([[1.0, 2.0, 4.0, 9.0]], np.float32)
+    got = orc.layernorm(x, np.ones(4, np.float32), np.zeros(4, np.float32))
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean()) / (x64.std(ddof=0) + 1e-5)
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
+    assert np.abs(got - (x64 - x64.mean()) / (x64.std(ddof=1) + 1e-5)).max() > 0.1
+
+
+def test_layernorm_variance_is_one_pass_and_can_go_negative(orc):
+    """Reduce.swift:106-110: var = E[x^2] - E[x]^2, evaluated in fp32.  A variance formed from squared deviations is
+    never negative; the one-pass form is, for some rows, and then sqrt gives NaN and the whole row is NaN.  Two-element
+    rows fix the fp32 value whatever the summation order."""
+    rows = negative_variance_pairs()
+    ones, zeros = np.ones(2, np.float32), np.zeros(2, np.float32)
+    with np.errstate(invalid="ignore"):
+        got = orc.layernorm(rows, ones, zeros)                       # 2-D input: one row per token
+    assert np.isnan(got).all()
+    ok = np.array([[1.5, 2.5], [-3.0, 3.0]], np.float32)            # exact in fp32: var = 0.25 and 9
+    want = np.array([[-1.0, 1.0], [-1.0, 1.0]]) / (1 + 1e-5 / np.array([[0.5], [3.0]]))
+    assert np.allclose(orc.layernorm(ok, ones, zeros), want, rtol=1e-6)
+
+
+def test_layernorm_far_from_zero_mean_depends_on_the_summation_order(orc):
+    """With |mean| = 1000 standard deviations, E[x^2] and E[x]^2 agree to six digits and fp32 keeps seven: what is left
+    of the variance is rounding noise of the sums.  The oracle (sequential sums, Engine/CPU/CPUEngine.swift:306-378,
+    CPUFloat.swift:239-261) is therefore far from the exact result there, and the same formula with pairwise sums is far
+    from both - no order-independent value exists to hold a GPU kernel to.  At |mean| <= 3 standard deviations the two
+    orders agree well inside the parity gate."""
+    f = np.float32
+    ones, zeros = np.ones(1024, f), np.zeros(1024, f)
+
+    def pairwise(x):
+        s, ss = np.sum(x, axis=1, dtype=f), np.sum(x * x, axis=1, dtype=f)
+        mean = s * f(1 / 1024)
+        var = ss * f(1 / 1024) - mean * mean
+        with np.errstate(invalid="ignore"):
+            return (x + (-mean[:, None])) * (f(1) / (np.sqrt(var) + f(1e-5)))[:, None]
+
+    def exact(x):
+        x64 = x.astype(np.float64)
+        return (x64 - x64.mean(axis=1, keepdims=True)) / (x64.std(axis=1, keepdims=True) + 1e-5)
+
+    far = (RNG.standard_normal((16, 1024)) + 1000).astype(f)
+    with np.errstate(invalid="ignore"):
+        got = orc.layernorm(far, ones, zeros)
+    assert np.nanmax(np.abs(got - exact(far))) > 0.1                    # a two-pass variance would be exact to 1e-6
+    assert np.nanmax(np.abs(got - pairwise(far))) > 0.1
+    near = (RNG.standard_normal((16, 1024)) + 3).astype(f)
+    got = orc.layernorm(near, ones, zeros)
+    assert np.abs(got - exact(near)).max() < 5e-5 and np.abs(got - pairwise(near)).max() < 5e-5
 
 
 def test_gelu_is_sigmoid_approximation(orc):
