@@ -14,6 +14,12 @@
 //                          (S^T, dP^T in the accumulator layout lane = query; dQ^T += K^T . dS^T)
 //   sdpa_bwd_dkv_f32_d64   a wavefront owns 32 keys and walks the queries (S, dP with lane = key;
 //                          dV^T += dO^T . P, dK^T += Q^T . dS)
+// Large launches form the scores and dP once: the dK/dV kernel also stores its dS tiles to a scratch tensor
+// [batch*head][key][query] (a lane of its accumulator layout holds four consecutive queries of one key: 128-bit stores)
+// and sdpa_bwd_dq_from_ds_f32_d64 only contracts them with K (a lane of ITS accumulator layout is one query and 16 keys:
+// 16 coalesced 32-bit loads) - five products issued for five, and the scratch tensor is written once and read once.
+// The two-kernel form above, which forms the scores and dP in both kernels (seven products for five), stays as the route
+// for launches whose scratch tensor would be too large to allocate.
 // All five products of each run on v_mfma_f32_32x32x2_f32 with the operand layouts of the forward kernel.  Small launches
 // run the _split_ forms of the two (one 32-row block per workgroup, its tiles split over the four wavefronts); head dims
 // above 64 up to 128 run the 128-wide forms in sdpa_backward_d128.h; head dims the MFMA kernels do not take run the
@@ -21,9 +27,23 @@
 #include "sdpa_common.h"
 #include "sdpa_backward_d128.h"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr float LN2 = 0.69314718055994530942f;
+// Upper bound of the dS scratch tensor of the large-launch route (B * H * Lk * Lq floats): beyond it the self-contained
+// kernels run.  B8 H16 L2048 needs 2 GiB.
+constexpr long long DS_SCRATCH_MAX_BYTES = 24ll << 30;
+// The environment variable DL4S_HIP_BWD_SCRATCH_MAX_BYTES lowers (or raises) the bound for a process, e.g. to keep the
+// gradient call's footprint small; 0 always takes the self-contained kernels.
+inline long long ds_scratch_max_bytes() {
+    const char *e = getenv("DL4S_HIP_BWD_SCRATCH_MAX_BYTES");
+    if (!e || !*e) return DS_SCRATCH_MAX_BYTES;
+    char *end = nullptr;
+    const long long v = strtoll(e, &end, 10);
+    return (end && *end == 0 && v >= 0) ? v : DS_SCRATCH_MAX_BYTES;
+}
 
 // D[b,h,i] = sum_d dout[i][d] * out[i][d]; 16 lanes per row, four rows per wavefront
 __global__ __launch_bounds__(256) void sdpa_bwd_rowdot(const float *__restrict__ out, const float *__restrict__ dout,
@@ -212,13 +232,16 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_f32_d64(const float *__res
 }
 
 // ------------------------------------------------------------------------------------------------ dK, dV
-template <int KIND>
+// WRITE_DS: every visited 32 x 32 tile of dS is also stored to ds [batch*head][Lkp][Lqp] (Lkp, Lqp = the key and query
+// counts rounded up to 32), for sdpa_bwd_dq_from_ds_f32_d64.  Rows of keys at or beyond Lk are stored as zeros.
+template <int KIND, bool WRITE_DS = false>
 __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
                                                                 const float *__restrict__ v, const float *__restrict__ dout,
                                                                 const float *__restrict__ stats, const float *__restrict__ D,
                                                                 float *__restrict__ dk, float *__restrict__ dv, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict, int nkb,
-                                                                int total_blocks, int lpt, int token_major, int hd) {
+                                                                int total_blocks, int lpt, int token_major, int hd,
+                                                                float *__restrict__ ds = nullptr) {
     extern __shared__ __align__(16) float lds[];
     float *Qs = lds;                       // [2][BN][LSTR]  q * rT * log2(e)
     float *Gs = lds + 2 * TILE_FLOATS;     // [2][BN][LSTR]  dout
@@ -323,6 +346,14 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
+    // dS slab of this (batch, head) pair: row = key, column = query; the lane stores four consecutive queries of its key
+    const int Lqp = (Lq + 31) & ~31, Lkp = (Lk + 31) & ~31;
+    __amdgpu_buffer_rsrc_t dsrsrc;
+    unsigned ds_voff = 0;
+    if (WRITE_DS) {
+        dsrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lkp * Lqp * 4), 0x00020000);
+        ds_voff = ((unsigned)key * (unsigned)Lqp + 4u * half) * 4u;
+    }
 
     for (int t = t_begin; t < nqt; ++t) {
         const int buf = (t - t_begin) & 1;
@@ -377,6 +408,17 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
                 p[4 * g + 2] = p[4 * g + 2] * (dp[4 * g + 2] - d4.z);
                 p[4 * g + 3] = p[4 * g + 3] * (dp[4 * g + 3] - d4.w);
             }
+            if (WRITE_DS) {
+                if (kw0 + 32 > Lk && key >= Lk) {       // a key that does not exist: its row of dS is zero
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[r] = 0.f;
+                }
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 o = {p[4 * g + 0], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 2);
+                }
+            }
             tile_accumulate_t(Qs + buf * TILE_FLOATS + col_lds, p, k0a, k1a);                   // dK^T += Q~^T . dS
         }
         if (more) store_tile(buf ^ 1);
@@ -386,6 +428,109 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
         store_row_t(dv + kv_base + (long long)key * rs + 8 * half, v0a, v1a, 1.0f, hd - 8 * half);
         store_row_t(dk + kv_base + (long long)key * rs + 8 * half, k0a, k1a, LN2, hd - 8 * half);   // Q~ carries log2(e): dK = Q~^T dS ln 2
     }
+}
+
+// ------------------------------------------------------------------------------------------------ dQ from stored dS
+// dQ = (dS . K) * rT with dS read from the scratch tensor sdpa_bwd_dkv_f32_d64<KIND, true> wrote: a wavefront owns 32
+// queries and walks the key tiles the forward pass visits (the dK/dV kernel visits - and writes - exactly those: both
+// follow the forward pass's rule, tile by tile).  Per tile and wavefront: 16 coalesced 32-bit loads (lane = query, the
+// 16 keys of the accumulator layout) and 32 MFMAs against the K tile in LDS; no scores, no exponentials, no mask values.
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d64(const float *__restrict__ k, const float *__restrict__ ds,
+                                                                       float *__restrict__ dq, int H, int Lq, int Lk, float rT,
+                                                                       MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
+                                                                       int token_major, int hd) {
+    extern __shared__ __align__(16) float lds[];
+    float *Ks = lds;                     // [2][BN][LSTR]
+    int bh, unit;
+    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int qb = nqb - 1 - unit;   // longest rows first
+    const int q0 = qb * BM + wave * 32;
+    const int qi = q0 + ln;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
+
+    int kend = Lk, wkend = Lk;
+    bool skip_ones = false;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
+        if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
+        if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    const int ld_row = tid >> 4, ld_col = (tid & 15) * 4;
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
+    const unsigned ld_off1 = ld_off0 + 16u * rs * 4u;
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[2];
+    auto load_tile = [&](int t) {
+        kst[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, (int)(ld_off0 + t * tile_bytes), 0, 0));
+        kst[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, (int)(ld_off1 + t * tile_bytes), 0, 0));
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<f32x4 *>(Ks + buf * TILE_FLOATS + (i * 16 + ld_row) * LSTR + ld_col) = kst[i];
+    };
+
+    // dS slab of the pair, [key][query]: register r of the lane is key k0 + 8(r/4) + 4*half + r%4, query qi
+    const int Lqp = (Lq + 31) & ~31, Lkp = (Lk + 31) & ~31;
+    const __amdgpu_buffer_rsrc_t dsrsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lkp * Lqp * 4), 0x00020000);
+    const unsigned ds_voff = ((unsigned)(4 * half) * (unsigned)Lqp + (unsigned)qi) * 4u;
+    const unsigned ds_row = (unsigned)Lqp * 4u;
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
+    auto visited = [&](int t) {
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        return t * BN < wkend && !(DENSE && skip_ones && cls == 1);
+    };
+    f32x16 dsn;
+    auto load_ds = [&](int t) {
+        const unsigned base = (unsigned)(t * BN) * ds_row;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            dsn[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dsrsrc, (int)ds_voff, (int)(base + (unsigned)(8 * (r >> 2) + (r & 3)) * ds_row), 2));
+    };
+
+    f32x16 a0, a1;   // dQ^T rows d = 2m + {0,1}
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { a0[i] = 0.f; a1[i] = 0.f; dsn[i] = 0.f; }
+
+    if (ntiles > 0) {
+        load_tile(0);
+        store_tile(0);
+        if (visited(0)) load_ds(0);
+    }
+    __syncthreads();
+    const int col_lds = (4 * half) * LSTR + 2 * ln;
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        const bool more = (t + 1 < ntiles);
+        const bool now = visited(t);
+        const f32x16 p = dsn;
+        if (more) {
+            load_tile(t + 1);
+            if (visited(t + 1)) load_ds(t + 1);
+        }
+        if (now) tile_accumulate_t(Ks + buf * TILE_FLOATS + col_lds, p, a0, a1);               // dQ^T += K^T . dS^T
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+    if (qi < Lq) store_row_t(dq + q_base + (long long)qi * rs + 8 * half, a0, a1, rT, hd - 8 * half);
 }
 
 // ------------------------------------------------------------------------------------------------ small launches
@@ -849,6 +994,8 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq));
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d64<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d64<KIND, true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_split_f32_d64<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq_split));
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_split_f32_d64<KIND>),
@@ -856,9 +1003,40 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         dl4s::lds_limit_done(ctx, dl4s::LDS_BWD, KIND);
     }
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
+    const bool dq_small = !no_split && (long long)B * H * ((Lq + 31) / 32) < 8ll * ctx->cu_count && Lk >= 2 * BN;
+    const bool dkv_small = !no_split && (long long)B * H * ((Lk + 31) / 32) < 8ll * ctx->cu_count && Lq >= 2 * BN;
+    // Large launches: the dK/dV kernel stores dS, the dQ kernel only contracts it with K (five products for five).  The
+    // scratch tensor [B*H][Lk][Lq] comes from the pool; when it cannot be had (too large, pool miss while a graph is being
+    // recorded, out of memory) the two self-contained kernels below run instead.
+    if (!dq_small && !dkv_small) {
+        const long long Lqp = (Lq + 31) & ~31ll, Lkp = (Lk + 31) & ~31ll;
+        const long long slab = Lqp * Lkp * 4;
+        const int nqb = (Lq + BM - 1) / BM, nkb = (Lk + BM - 1) / BM;
+        const long long total_q = (long long)nqb * B * H, total_k = (long long)nkb * B * H;
+        void *dsv = nullptr;
+        if (slab < (1ll << 31) && (long long)B * H * slab <= ds_scratch_max_bytes() && total_q < (1ll << 30) && total_k < (1ll << 30) &&
+            dl4s_hip_alloc(ctx, (size_t)((long long)B * H * slab), &dsv) == DL4S_HIP_OK) {
+            float *ds = static_cast<float *>(dsv);
+            int lpt = (uneven && nkb >= 2) ? 1 : 0;
+            if (lpt && total_k <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+            hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d64<KIND, true>), dim3((unsigned)((total_k + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
+                               k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total_k, lpt, token_major, hd, ds);
+            int rc = dl4s::launch_status("sdpa_bwd_dkv_f32_d64");
+            if (rc == DL4S_HIP_OK) {
+                lpt = (uneven && nqb >= 2) ? 1 : 0;
+                if (lpt && total_q <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+                hipLaunchKernelGGL(sdpa_bwd_dq_from_ds_f32_d64<KIND>, dim3((unsigned)((total_q + 7) / 8 * 8)), dim3(256),
+                                   2 * TILE_FLOATS * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q,
+                                   lpt, token_major, hd);
+                rc = dl4s::launch_status("sdpa_bwd_dq_from_ds_f32_d64");
+            }
+            const int rcf = dl4s_hip_free(ctx, dsv);   // stream-ordered
+            return rc != DL4S_HIP_OK ? rc : rcf;
+        }
+    }
     // Small launches (the forward pass's rule, from the extents only): one 32-row block per workgroup, the tiles along the
     // other axis split over its four wavefronts.
-    if (!no_split && (long long)B * H * ((Lq + 31) / 32) < 8ll * ctx->cu_count && Lk >= 2 * BN) {
+    if (dq_small) {
         const int nqb32 = (Lq + 31) / 32;
         const long long total = (long long)nqb32 * B * H;
         int order = (uneven && nqb32 >= 2) ? 1 : 0;
@@ -880,7 +1058,7 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d64");
         if (rc != DL4S_HIP_OK) return rc;
     }
-    if (!no_split && (long long)B * H * ((Lk + 31) / 32) < 8ll * ctx->cu_count && Lq >= 2 * BN) {
+    if (dkv_small) {
         const int nkb32 = (Lk + 31) / 32;
         const long long total = (long long)nkb32 * B * H;
         int order = (uneven && nkb32 >= 2) ? 1 : 0;
@@ -987,11 +1165,11 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
         rc = dl4s::launch_status("sdpa_bwd_rowdot128");
         if (rc == DL4S_HIP_OK) {
             switch (m.kind) {
-                case DL4S_MASK_NONE: rc = launch_bwd128<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-                case DL4S_MASK_DENSE_F32: rc = launch_bwd128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-                case DL4S_MASK_CAUSAL: rc = launch_bwd128<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-                case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
-                default: rc = launch_bwd128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d); break;
+                case DL4S_MASK_NONE: rc = launch_bwd128<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
+                case DL4S_MASK_DENSE_F32: rc = launch_bwd128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
+                case DL4S_MASK_CAUSAL: rc = launch_bwd128<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
+                case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
+                default: rc = launch_bwd128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
             }
         }
         const int rcf = dl4s_hip_free(ctx, Dv);

@@ -199,13 +199,16 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
 }
 
 // ------------------------------------------------------------------------------------------------ dK, dV
-template <int KIND>
+// WRITE_DS: every visited tile of dS is also stored to ds [batch*head][Lkp][Lqp] for sdpa_bwd_dq_from_ds_f32_d128 (the
+// layout and rules of the 64-wide kernels).
+template <int KIND, bool WRITE_DS = false>
 __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
                                                                  const float *__restrict__ v, const float *__restrict__ dout,
                                                                  const float *__restrict__ stats, const float *__restrict__ D,
                                                                  float *__restrict__ dk, float *__restrict__ dv, int H, int Lq,
                                                                  int Lk, float rT, MaskArgs mask, int strict, int nkb,
-                                                                 int total_blocks, int lpt, int token_major, int hd) {
+                                                                 int total_blocks, int lpt, int token_major, int hd,
+                                                                 float *__restrict__ ds = nullptr) {
     extern __shared__ __align__(16) float lds[];
     float *Qs = lds;                        // [2][BN][LSTR2]  q * rT * log2(e)
     float *Gs = lds + 2 * TILE2_FLOATS;     // [2][BN][LSTR2]  dout
@@ -308,6 +311,13 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
+    const int Lqp = (Lq + 31) & ~31, Lkp = (Lk + 31) & ~31;
+    __amdgpu_buffer_rsrc_t dsrsrc;
+    unsigned ds_voff = 0;
+    if (WRITE_DS) {
+        dsrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lkp * Lqp * 4), 0x00020000);
+        ds_voff = ((unsigned)key * (unsigned)Lqp + 4u * half) * 4u;
+    }
 
     for (int t = t_begin; t < nqt; ++t) {
         const int buf = (t - t_begin) & 1;
@@ -362,6 +372,17 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                 p[4 * g + 2] = p[4 * g + 2] * (dp[4 * g + 2] - d4.z);
                 p[4 * g + 3] = p[4 * g + 3] * (dp[4 * g + 3] - d4.w);
             }
+            if (WRITE_DS) {
+                if (kw0 + 32 > Lk && key >= Lk) {       // a key that does not exist: its row of dS is zero
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[r] = 0.f;
+                }
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 o = {p[4 * g + 0], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 2);
+                }
+            }
             tile_accumulate_t128(Qs + buf * TILE2_FLOATS + col_lds, p, ka);                      // dK^T += Q~^T . dS
         }
         if (more) store_tile(buf ^ 1);
@@ -373,10 +394,114 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
     }
 }
 
+// ------------------------------------------------------------------------------------------------ dQ from stored dS
+// dQ = (dS . K) * rT with dS read from the scratch tensor sdpa_bwd_dkv_f32_d128<KIND, true> wrote; see
+// sdpa_bwd_dq_from_ds_f32_d64.  Four accumulators and one dS tile in flight: three wavefronts per SIMD instead of one.
+template <int KIND>
+__global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const float *__restrict__ k, const float *__restrict__ ds,
+                                                                        float *__restrict__ dq, int H, int Lq, int Lk, float rT,
+                                                                        MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
+                                                                        int token_major, int hd) {
+    extern __shared__ __align__(16) float lds[];
+    float *Ks = lds;                      // [2][BN][LSTR2]
+    int bh, unit;
+    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int qb = nqb - 1 - unit;   // longest rows first
+    const int q0 = qb * BM + wave * 32;
+    const int qi = q0 + ln;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
+
+    int kend = Lk, wkend = Lk;
+    bool skip_ones = false;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
+        if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
+        if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    const int ld_row = tid >> 5, ld_col = (tid & 31) * 4;
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
+    const unsigned row8_bytes = 8u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[4];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, (int)(ld_off0 + t * tile_bytes + i * row8_bytes), 0, 0));
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4 *>(Ks + buf * TILE2_FLOATS + (i * 8 + ld_row) * LSTR2 + ld_col) = kst[i];
+    };
+
+    const int Lqp = (Lq + 31) & ~31, Lkp = (Lk + 31) & ~31;
+    const __amdgpu_buffer_rsrc_t dsrsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lkp * Lqp * 4), 0x00020000);
+    const unsigned ds_voff = ((unsigned)(4 * half) * (unsigned)Lqp + (unsigned)qi) * 4u;
+    const unsigned ds_row = (unsigned)Lqp * 4u;
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
+    auto visited = [&](int t) {
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        return t * BN < wkend && !(DENSE && skip_ones && cls == 1);
+    };
+    f32x16 dsn;
+    auto load_ds = [&](int t) {
+        const unsigned base = (unsigned)(t * BN) * ds_row;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            dsn[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dsrsrc, (int)ds_voff, (int)(base + (unsigned)(8 * (r >> 2) + (r & 3)) * ds_row), 2));
+    };
+
+    f32x16 acc[4];   // dQ^T, accumulator c row i is d = 4*i + c
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dsn[i] = 0.f;
+
+    if (ntiles > 0) {
+        load_tile(0);
+        store_tile(0);
+        if (visited(0)) load_ds(0);
+    }
+    __syncthreads();
+    const int col_lds = (4 * half) * LSTR2 + 4 * ln;
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        const bool more = (t + 1 < ntiles);
+        const bool now = visited(t);
+        const f32x16 p = dsn;
+        if (more) {
+            load_tile(t + 1);
+            if (visited(t + 1)) load_ds(t + 1);
+        }
+        if (now) tile_accumulate_t128(Ks + buf * TILE2_FLOATS + col_lds, p, acc);               // dQ^T += K^T . dS^T
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+    if (qi < Lq) store_row_t128(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
+}
+
 template <int KIND>
 int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
                   const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
-                  int strict, int token_major, int hd) {
+                  int strict, int token_major, int hd, long long ds_max_bytes) {
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     const size_t lds_dq = 4 * TILE2_FLOATS * sizeof(float);
     const size_t lds_dkv = (4 * TILE2_FLOATS + 192) * sizeof(float);
@@ -385,9 +510,39 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq));
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND, true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
         dl4s::lds_limit_done(ctx, dl4s::LDS_BWD_D128, KIND);
     }
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
+    // The dK/dV kernel stores dS and a light dQ kernel contracts it with K (see sdpa_backward.hip) whenever the scratch
+    // tensor can be had; the two self-contained kernels otherwise.
+    {
+        const long long Lqp = (Lq + 31) & ~31ll, Lkp = (Lk + 31) & ~31ll;
+        const long long slab = Lqp * Lkp * 4;
+        const int nqb = (Lq + BM - 1) / BM, nkb = (Lk + BM - 1) / BM;
+        const long long total_q = (long long)nqb * B * H, total_k = (long long)nkb * B * H;
+        void *dsv = nullptr;
+        if (slab < (1ll << 31) && (long long)B * H * slab <= ds_max_bytes && total_q < (1ll << 30) && total_k < (1ll << 30) &&
+            dl4s_hip_alloc(ctx, (size_t)((long long)B * H * slab), &dsv) == DL4S_HIP_OK) {
+            float *ds = static_cast<float *>(dsv);
+            int lpt = (uneven && nkb >= 2) ? 1 : 0;
+            if (lpt && total_k <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+            hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d128<KIND, true>), dim3((unsigned)((total_k + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream,
+                               q, k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total_k, lpt, token_major, hd, ds);
+            int rc = dl4s::launch_status("sdpa_bwd_dkv_f32_d128");
+            if (rc == DL4S_HIP_OK) {
+                lpt = (uneven && nqb >= 2) ? 1 : 0;
+                if (lpt && total_q <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+                hipLaunchKernelGGL(sdpa_bwd_dq_from_ds_f32_d128<KIND>, dim3((unsigned)((total_q + 7) / 8 * 8)), dim3(256),
+                                   2 * TILE2_FLOATS * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q,
+                                   lpt, token_major, hd);
+                rc = dl4s::launch_status("sdpa_bwd_dq_from_ds_f32_d128");
+            }
+            const int rcf = dl4s_hip_free(ctx, dsv);   // stream-ordered
+            return rc != DL4S_HIP_OK ? rc : rcf;
+        }
+    }
     {
         const int nqb = (Lq + BM - 1) / BM;
         const long long total = (long long)nqb * B * H;

@@ -136,6 +136,52 @@ def test_zero_upstream_gradient_gives_zero_gradients(ctx):
     assert not dq.any() and not dk.any() and not dv.any()
 
 
+@pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 70), (1, 2, 257, 300), (2, 2, 96, 513), (1, 3, 40, 33)])
+@pytest.mark.parametrize("mask_kind", ["none", "dense", "lengths", "causal", "causal_lengths"])
+@pytest.mark.parametrize("d", [64, 128, 40, 96])
+def test_stored_ds_route_agrees_with_the_self_contained_kernels(ctx, orc, B, H, Lq, Lk, mask_kind, d):
+    """Large launches (here: forced by DL4S_SDPA_NO_KEY_SPLIT; head dims above 64 always) store dS from the dK/dV kernel and
+    contract it in a second kernel; with the scratch bound at 0 the two self-contained kernels run instead.  Both within the gate of the oracle,
+    dK and dV bit-identical (the same kernel with and without the store), and each route bit-identical run to run."""
+    import os
+    from dl4s_amd import lib
+    if not NO_SPLIT_DEFAULT[0]:
+        pytest.skip("only the unsplit kernels have the two routes")
+    rng = np.random.default_rng(B * 1000 + Lq + Lk)
+    q, k, v, dout = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lq, d)
+    lens = rng.integers(1, Lk + 1, size=B)
+    kw, mask = {}, None
+    if mask_kind == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.3).astype(np.float32)
+        mask[0, 0, 3, :] = 1.0
+        kw = dict(mask=mask)
+    elif mask_kind == "lengths":
+        mask, kw = lengths_mask(lens, Lk), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    elif mask_kind == "causal":
+        mask, kw = causal_mask(Lq, Lk), dict(kind=lib.MASK_CAUSAL)
+    elif mask_kind == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lk)[None, None])
+        kw = dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens)
+    results = {}
+    try:
+        for route, cap in (("stored", None), ("stored again", None), ("self-contained", "0")):
+            if cap is None:
+                os.environ.pop("DL4S_HIP_BWD_SCRATCH_MAX_BYTES", None)
+            else:
+                os.environ["DL4S_HIP_BWD_SCRATCH_MAX_BYTES"] = cap
+            results[route] = run_fwd_bwd(ctx, q, k, v, dout, **kw)[2:]
+    finally:
+        os.environ.pop("DL4S_HIP_BWD_SCRATCH_MAX_BYTES", None)
+    ref = orc.sdpa_backward(q, k, v, mask, dout)
+    for route, got in results.items():
+        for name, g, r in zip(("dq", "dk", "dv"), got, ref):
+            assert_parity(g, r, "%s, %s route" % (name, route))
+    for a, b_ in zip(results["stored"], results["stored again"]):
+        assert np.array_equal(a, b_)
+    assert np.array_equal(results["stored"][1], results["self-contained"][1])
+    assert np.array_equal(results["stored"][2], results["self-contained"][2])
+
+
 def test_config4_sized_gradients(ctx, orc):
     """B8 H16 L2048 d64 causal: two (batch, head) slices against the oracle, and on every slice the identities that hold
     whatever the inputs: sum over keys of dv = sum over queries of dout (every row's weights sum to 1), and
