@@ -23,6 +23,7 @@ constexpr float LOG2E = 1.44269504088896340736f;
 constexpr int HD2 = 128;
 constexpr int LSTR2 = HD2 + 4;   // 132 = 4 mod 32: the same bank spread as LSTR
 constexpr int TILE2_FLOATS = BN * LSTR2;
+constexpr int SPLIT_WAVES = 4;   // wavefronts that share the key tiles of a 32-query block in the kernels for small launches
 
 struct MaskArgs {
     int kind;

@@ -28,6 +28,7 @@
 
 #include "sdpa_common.h"
 #include "sdpa_prefill_d128.h"
+#include "sdpa_prefill_narrow.h"
 
 namespace {
 
@@ -263,7 +264,6 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_d64(const float *__re
 // four partial results (reference maximum, row sum, O^T) are merged through LDS and wavefront 0 stores the rows.
 // Same tile arithmetic as the kernel above; the summation order over keys differs, so results agree with it within
 // rounding, not bit for bit.  Which of the two kernels runs depends on the extents only, never on the mask.
-constexpr int SPLIT_WAVES = 4;
 template <int KIND>
 __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float *__restrict__ q, const float *__restrict__ k,
                                                                       const float *__restrict__ v, float *__restrict__ out,
@@ -496,6 +496,9 @@ __global__ __launch_bounds__(64) void sdpa_generic_f32(const float *__restrict__
 template <int KIND>
 int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq,
                int Lk, float rT, const MaskArgs &m, int strict, int token_major, int no_split, float *stats, int hd) {
+    // narrow heads: tiles of 16 or 32 columns
+    if (hd <= 16) return launch_narrow<KIND, 16>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, no_split, stats, hd);
+    if (hd <= 32) return launch_narrow<KIND, 32>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, no_split, stats, hd);
     // Too few 32-query wavefronts to give every SIMD about two: split the keys of each query block over 4 wavefronts.
     // The choice depends on the extents only, so every mask kind of one problem runs the same kernel.
     const long long waves = (long long)B * H * ((Lq + 31) / 32);

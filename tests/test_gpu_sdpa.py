@@ -73,7 +73,7 @@ def rand(rng, *shape, scale=1.0):
 
 # ------------------------------------------------------------------ small shapes, every mask kind
 SHAPES = [  # B, H, Lq, Lk, d
-    (1, 2, 5, 7, 4),        # the golden-fixture shape: MFMA kernel with 60 padding columns
+    (1, 2, 5, 7, 4),        # the golden-fixture shape: the 16-wide MFMA kernel with 12 padding columns
     (2, 3, 9, 11, 8),       # key size of Tests/DL4STests/TransformerTests.swift:31
     (2, 3, 9, 11, 6),       # not a multiple of 4: plain kernel
     (1, 2, 40, 50, 96),     # above 64: the 128-wide MFMA kernel with padding columns
@@ -82,7 +82,10 @@ SHAPES = [  # B, H, Lq, Lk, d
     (1, 2, 100, 100, 100),
     (1, 2, 40, 50, 130),    # not a multiple of 4 / above 128: plain kernel
     (1, 1, 33, 40, 200),
-    (2, 3, 130, 70, 32),    # padded MFMA tiles, ragged
+    (2, 3, 130, 70, 16),    # the 16-wide kernels, every column used
+    (1, 2, 100, 100, 12),   # the 16-wide kernels with padding columns
+    (2, 2, 200, 333, 24),   # the 32-wide kernels with padding columns
+    (2, 3, 130, 70, 32),    # the 32-wide kernels, ragged
     (2, 2, 200, 333, 40),
     (1, 2, 100, 100, 60),
     (1, 2, 5, 7, 64),       # MFMA kernel, ragged single tile
@@ -499,7 +502,7 @@ def test_decode_step_with_the_position_in_device_memory(ctx, orc, Tcap, steps):
         buf.release()
 
 
-@pytest.mark.parametrize("d", [64, 8, 36, 128, 80])
+@pytest.mark.parametrize("d", [64, 8, 16, 28, 36, 128, 80])
 @pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 70), (1, 2, 5, 7), (2, 4, 256, 256), (1, 5, 33, 161)])
 def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk, d):
     """[B,L,H,d] operands (what the projections of MultiHeadAttention produce before its permutes,
