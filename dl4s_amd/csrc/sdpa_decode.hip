@@ -1,9 +1,10 @@
 // Single-query attention over a key/value cache (one decode step), split over the keys.
 //
-// The cache is [B,H,Tcap,64] fp32.  A 16-lane group reads one 256-byte key (or value) row with one
+// The cache is [B,H,Tcap,d] fp32.  At d = 64 a 16-lane group reads one 256-byte key (or value) row with one
 // 128-bit load per lane, so every load instruction of a wavefront covers four whole rows (1 KiB,
 // contiguous), and a wavefront keeps the 8 K loads and 8 V loads of a 32-key block in flight together.
-// The dot product is reduced inside the 16-lane group with DPP adds.  With 16 wavefronts resident per CU
+// The dot product is reduced inside the 16-lane group with DPP adds.  Rows of 32 and 128 floats use groups of 8 and
+// 32 lanes in the same way (64 and 16 keys per iteration); other head dims run the next wider form with idle lanes.  With 16 wavefronts resident per CU
 // that is ample memory-level parallelism to keep HBM busy.
 //
 // Work split: grid = (nsplit, B*H).  When B*H alone fills the GPU (the decode benchmark: 256 pairs on 256
@@ -27,10 +28,10 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int HD = 64;
-constexpr int KB = 32;                        // keys per wavefront iteration
-constexpr int PSTR = 68;                      // floats per partial record: o[0..63], m, l, pad
+constexpr int MAXD = 128;                     // widest cache row the kernels take
 constexpr float LOG2E = 1.44269504088896340736f;
+// floats per partial record: o[0 .. D-1], m, l, pad (D = the row width the kernel instance covers: 32, 64 or 128)
+constexpr int pstr(int D) { return D + 4; }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -38,29 +39,41 @@ template <int CTRL>
 __device__ __forceinline__ float dpp(float x) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
 }
-// Sum over the 16 lanes of a DPP row; every lane of the row ends up with the total.
-__device__ __forceinline__ float row16_sum(float x) {
+// Sum over the LPR (8, 16 or 32) lanes that share a cache row; every one of them ends up with the total.
+template <int LPR>
+__device__ __forceinline__ float row_sum(float x) {
     x += dpp<0xB1>(x);   // quad_perm [1,0,3,2]
     x += dpp<0x4E>(x);   // quad_perm [2,3,0,1]
     x += dpp<0x141>(x);  // row_half_mirror
-    x += dpp<0x140>(x);  // row_mirror
+    if (LPR >= 16) x += dpp<0x140>(x);  // row_mirror
+    if (LPR >= 32) x += __shfl_xor(x, 16, 64);
     return x;
 }
 
-// NW wavefronts per workgroup; the wavefronts of a workgroup take 32-key blocks of the workgroup's key range
-// [split*chunk, split*chunk + chunk) round-robin.  Inside a wavefront each 16-lane group keeps its own running
-// (max, sum, 4 output columns per lane), so the loop has no cross-lane traffic beyond the 16-lane dot-product
-// reduction; groups, wavefronts and (through the scratch records) workgroups are merged once at the end.
+// LPR lanes read one cache row of up to 4 * LPR floats with one 128-bit load per lane (lanes at or beyond d / 4 hold
+// zeros), so a load instruction of a wavefront covers G = 64 / LPR whole rows; a wavefront iteration covers KB = 8 * G
+// keys with 8 K loads and 8 V loads per lane in flight (16 KiB per wavefront whatever the row width).
+// NW wavefronts per workgroup; the wavefronts of a workgroup take KB-key blocks of the workgroup's key range
+// [split*chunk, split*chunk + chunk) round-robin.  Inside a wavefront each LPR-lane group keeps its own running
+// (max, sum, 4 output columns per lane), so the loop has no cross-lane traffic beyond the dot-product reduction;
+// groups, wavefronts and (through the scratch records) workgroups are merged once at the end.
+// FULL: the rows are exactly 4 * LPR floats long (no lane is idle, no load is predicated).
 // DEVPOS: the row to append comes from device memory (*pos_dev) and T = row + 1, for callers that replay one recorded
 // step at successive positions; a value outside [0, Tcap) leaves caches and output untouched.
-template <bool APPEND, int NW, bool DEVPOS = false>
+// lengths (optional, one per batch element): keys at or beyond lengths[b] are blocked the way the reference blocks them,
+// score - 1e9 (NN/Models/Transformer/ScaledDotProductAttention.swift:55-57 with the mask of makeEncoderMasks).  With at
+// least one key left their weights are exactly zero and they are not visited at all; a length of zero or less blocks every
+// key, the penalty is applied to all of them and the row comes out uniform, as in the reference.
+template <bool APPEND, int NW, int LPR, bool FULL, bool DEVPOS = false>
 __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
                                                                    float *vcache, const float *__restrict__ k_new,
                                                                    const float *__restrict__ v_new,
                                                                    float *__restrict__ out, float *part, int T, int Tcap,
-                                                                   int pos, float rT, int nsplit, int chunk,
+                                                                   int pos, float rT, int nsplit, int chunk, int d, int H,
+                                                                   const int *__restrict__ lengths,
                                                                    const int *__restrict__ pos_dev = nullptr) {
-    __shared__ float sm_o[NW][HD];
+    constexpr int D = 4 * LPR, G = 64 / LPR, KB = 8 * G, PSTR = pstr(D);
+    __shared__ float sm_o[NW][D];
     __shared__ float sm_m[NW], sm_l[NW];
     if (DEVPOS) {
         pos = *pos_dev;
@@ -71,30 +84,41 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
     const int bh = blockIdx.y;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
-    const int g = lane >> 4, c = lane & 15;
+    const int g = lane / LPR, c = lane % LPR;
+    const bool col_ok = FULL || 4 * c < d;    // FULL: d = 4 * LPR, every lane has its piece of the row; else lanes beyond the row hold zeros
 
-    f32x4 qv = *reinterpret_cast<const f32x4 *>(q + (long long)bh * HD + 4 * c);
+    bool all_blocked = false;                 // a length of zero: every key takes the penalty
+    if (lengths) {
+        const int len = lengths[bh / H];
+        if (len <= 0) all_blocked = true;
+        else if (len < T) T = len;
+    }
+
+    f32x4 qv = {0.f, 0.f, 0.f, 0.f};
+    if (col_ok) qv = *reinterpret_cast<const f32x4 *>(q + (long long)bh * d + 4 * c);
     qv.x *= rT; qv.y *= rT; qv.z *= rT; qv.w *= rT;
 
-    const long long base = (long long)bh * Tcap * HD + 4 * c;
+    const long long base = (long long)bh * Tcap * d + 4 * c;
     const int c0 = split * chunk;
     const int c1 = min(T, c0 + chunk);
     // Row `pos` is the row being appended in this step: it is read from k_new / v_new (the cache does not
-    // hold it yet) by selecting the ADDRESS per lane, so that all loads stay unconditional; one 16-lane
-    // group of the workgroup whose range holds the row writes it into the cache from its own copy.
+    // hold it yet) by selecting the ADDRESS per lane, so that all loads stay unconditional; one group of lanes
+    // of the workgroup whose range holds the row writes it into the cache from its own copy.  (With lengths the
+    // row may lie beyond the keys that are visited: the first workgroup of the pair writes it then.)
     const float *kn_row = nullptr, *vn_row = nullptr;
     if (APPEND) {
-        kn_row = k_new + (long long)bh * HD + 4 * c;
-        vn_row = v_new + (long long)bh * HD + 4 * c;
-        if (pos >= c0 && pos < c1 && wave == 0 && g == 0) {
-            *reinterpret_cast<f32x4 *>(kcache + base + (long long)pos * HD) = *reinterpret_cast<const f32x4 *>(kn_row);
-            *reinterpret_cast<f32x4 *>(vcache + base + (long long)pos * HD) = *reinterpret_cast<const f32x4 *>(vn_row);
+        kn_row = k_new + (long long)bh * d + 4 * c;
+        vn_row = v_new + (long long)bh * d + 4 * c;
+        const bool mine = (pos >= c0 && pos < c1) || (pos >= T && split == 0);
+        if (mine && wave == 0 && g == 0 && col_ok) {
+            *reinterpret_cast<f32x4 *>(kcache + base + (long long)pos * d) = *reinterpret_cast<const f32x4 *>(kn_row);
+            *reinterpret_cast<f32x4 *>(vcache + base + (long long)pos * d) = *reinterpret_cast<const f32x4 *>(vn_row);
         }
     }
 
     float m_run = -INFINITY, l_run = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    // The wavefronts take the 32-key blocks of [c0, c1) round-robin, starting at a block that depends on the
+    // The wavefronts take the KB-key blocks of [c0, c1) round-robin, starting at a block that depends on the
     // (batch, head) pair: all workgroups run in lockstep, and without the rotation they would all be at the same
     // offset of their cache rows at the same time, which for some row strides (Tcap) lands on few HBM channels.
     const int nblk = (c1 - c0 + KB - 1) / KB;
@@ -103,40 +127,43 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         int bb = bi + rot;
         if (bb >= nblk) bb -= nblk;
         const int kb = c0 + bb * KB;
-        f32x4 kk[KB / 4], vv[KB / 4];
+        f32x4 kk[8], vv[8];
 #pragma unroll
-        for (int i = 0; i < KB / 4; ++i) {
-            const int key = kb + 4 * i + g;
+        for (int i = 0; i < 8; ++i) {
+            const int key = kb + G * i + g;
             const int kc = key < T ? key : T - 1;
-            const float *kp = kcache + base + (long long)kc * HD;
+            const float *kp = kcache + base + (long long)kc * d;
             if (APPEND) kp = (kc == pos) ? kn_row : kp;
-            kk[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(kp));
+            kk[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (col_ok) kk[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(kp));
         }
 #pragma unroll
-        for (int i = 0; i < KB / 4; ++i) {
-            const int key = kb + 4 * i + g;
+        for (int i = 0; i < 8; ++i) {
+            const int key = kb + G * i + g;
             const int kc = key < T ? key : T - 1;
-            const float *vp = vcache + base + (long long)kc * HD;
+            const float *vp = vcache + base + (long long)kc * d;
             if (APPEND) vp = (kc == pos) ? vn_row : vp;
-            vv[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(vp));
+            vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (col_ok) vv[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(vp));
         }
         if (kb + KB > c1) {     // the range's last block: lanes past its end re-read row T-1 and must add nothing, not 0 * Inf
 #pragma unroll
-            for (int i = 0; i < KB / 4; ++i)
-                if (kb + 4 * i + g >= c1) vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < 8; ++i)
+                if (kb + G * i + g >= c1) vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        float s[KB / 4];
+        float s[8];
         float bm = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < KB / 4; ++i) {
-            float d = qv.x * kk[i].x;
-            d += qv.y * kk[i].y;
-            d += qv.z * kk[i].z;
-            d += qv.w * kk[i].w;
-            d = row16_sum(d);
-            if (kb + 4 * i + g >= c1) d = -INFINITY;
-            s[i] = d;
-            bm = fmaxf(bm, d);
+        for (int i = 0; i < 8; ++i) {
+            float dot = qv.x * kk[i].x;
+            dot += qv.y * kk[i].y;
+            dot += qv.z * kk[i].z;
+            dot += qv.w * kk[i].w;
+            dot = row_sum<LPR>(dot);
+            if (all_blocked) dot = __fsub_rn(dot, 1e9f);
+            if (kb + G * i + g >= c1) dot = -INFINITY;
+            s[i] = dot;
+            bm = fmaxf(bm, dot);
         }
         const float m_new = fmaxf(m_run, bm);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -145,15 +172,16 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         l_run *= alpha;
         acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
 #pragma unroll
-        for (int i = 0; i < KB / 4; ++i) {
+        for (int i = 0; i < 8; ++i) {
             const float p = fast_exp2((s[i] - m_use) * LOG2E);
             l_run += p;
             acc.x += p * vv[i].x; acc.y += p * vv[i].y; acc.z += p * vv[i].z; acc.w += p * vv[i].w;
         }
     }
-    // merge the four 16-lane groups of the wavefront
-    float mw = fmaxf(m_run, __shfl_xor(m_run, 16, 64));
-    mw = fmaxf(mw, __shfl_xor(mw, 32, 64));
+    // merge the G groups of the wavefront
+    float mw = m_run;
+#pragma unroll
+    for (int o = LPR; o <= 32; o <<= 1) mw = fmaxf(mw, __shfl_xor(mw, o, 64));
     {
         const float mu = (mw == -INFINITY) ? 0.f : mw;
         const float f = fast_exp2((m_run - mu) * LOG2E);
@@ -161,7 +189,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         acc.x *= f; acc.y *= f; acc.z *= f; acc.w *= f;
     }
 #pragma unroll
-    for (int o = 16; o <= 32; o <<= 1) {
+    for (int o = LPR; o <= 32; o <<= 1) {
         l_run += __shfl_xor(l_run, o, 64);
         acc.x += __shfl_xor(acc.x, o, 64); acc.y += __shfl_xor(acc.y, o, 64);
         acc.z += __shfl_xor(acc.z, o, 64); acc.w += __shfl_xor(acc.w, o, 64);
@@ -170,7 +198,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
     if (lane == 0) { sm_m[wave] = mw; sm_l[wave] = l_run; }
     __syncthreads();
 
-    if (tid < HD) {
+    if (tid < D) {
         float M = sm_m[0];
 #pragma unroll
         for (int w = 1; w < NW; ++w) M = fmaxf(M, sm_m[w]);
@@ -183,30 +211,31 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
             O += sm_o[w][tid] * f;
         }
         if (nsplit == 1) {
-            out[(long long)bh * HD + tid] = O * (1.0f / L);
+            if (tid < d) out[(long long)bh * d + tid] = O * (1.0f / L);
         } else {
             float *rec = part + ((long long)bh * nsplit + split) * PSTR;
             rec[tid] = O;
-            if (tid == 0) { rec[HD] = M; rec[HD + 1] = L; }
+            if (tid == 0) { rec[D] = M; rec[D + 1] = L; }
         }
     }
 }
 
-// Merges the partial records of one (batch, head): one wavefront, lane = output column.
-__global__ __launch_bounds__(64) void sdpa_decode_merge_f32(const float *__restrict__ part, float *__restrict__ out,
-                                                             int nsplit) {
+// Merges the partial records of one (batch, head): one thread per output column.
+__global__ __launch_bounds__(MAXD) void sdpa_decode_merge_f32(const float *__restrict__ part, float *__restrict__ out,
+                                                               int nsplit, int D, int d) {
     const int bh = blockIdx.x, tid = threadIdx.x;
+    const int PSTR = pstr(D);
     const float *recs = part + (long long)bh * nsplit * PSTR;
     float M = -INFINITY;
-    for (int sidx = 0; sidx < nsplit; ++sidx) M = fmaxf(M, recs[sidx * PSTR + HD]);
+    for (int sidx = 0; sidx < nsplit; ++sidx) M = fmaxf(M, recs[sidx * PSTR + D]);
     const float Mu = (M == -INFINITY) ? 0.f : M;
     float L = 0.f, O = 0.f;
     for (int sidx = 0; sidx < nsplit; ++sidx) {
-        const float f = fast_exp2((recs[sidx * PSTR + HD] - Mu) * LOG2E);
-        L += recs[sidx * PSTR + HD + 1] * f;
-        O += recs[sidx * PSTR + tid] * f;
+        const float f = fast_exp2((recs[sidx * PSTR + D] - Mu) * LOG2E);
+        L += recs[sidx * PSTR + D + 1] * f;
+        if (tid < D) O += recs[sidx * PSTR + tid] * f;
     }
-    out[(long long)bh * HD + tid] = O * (1.0f / L);
+    if (tid < d) out[(long long)bh * d + tid] = O * (1.0f / L);
 }
 
 __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restrict__ k_new,
@@ -220,20 +249,55 @@ __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restr
     vcache[dst] = v_new[i];
 }
 
+// Row widths the kernel is instantiated for: 32, 64, 128 floats (8, 16, 32 lanes per row).
+inline int lanes_per_row(int64_t d) { return d <= 32 ? 8 : (d <= 64 ? 16 : 32); }
+
+template <bool APPEND, int NW, int LPR, bool DEVPOS>
+void decode_launch_kernel(dl4s_hip_ctx *ctx, dim3 grid, const float *q, float *kcache, float *vcache, const float *k_new,
+                          const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
+                          int d, int H, const int *lengths, const int *pos_dev) {
+    if (d == 4 * LPR)
+        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, true, DEVPOS>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
+                           k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev);
+    else
+        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, false, DEVPOS>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
+                           k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev);
+}
+
+template <bool APPEND, bool DEVPOS>
+void decode_launch_width(dl4s_hip_ctx *ctx, int nw, dim3 grid, const float *q, float *kcache, float *vcache, const float *k_new,
+                         const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
+                         int d, int H, const int *lengths, const int *pos_dev) {
+#define DL4S_DECODE_ARGS ctx, grid, q, kcache, vcache, k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev
+    switch (lanes_per_row(d)) {
+        case 8: if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS>(DL4S_DECODE_ARGS); break;
+        case 16: if (nw == 16) decode_launch_kernel<APPEND, 16, 16, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 16, DEVPOS>(DL4S_DECODE_ARGS); break;
+        default: if (nw == 16) decode_launch_kernel<APPEND, 16, 32, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 32, DEVPOS>(DL4S_DECODE_ARGS); break;
+    }
+#undef DL4S_DECODE_ARGS
+}
+
 int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcache, const float *k_new,
                   const float *v_new, float *out, int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t pos,
-                  int64_t d, float rT, bool append, bool fixed_scratch = false) {
+                  int64_t d, float rT, bool append, const int32_t *lengths = nullptr, bool fixed_scratch = false) {
     const int64_t BH = B * H;
     if (BH == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(q && kcache && vcache && out, DL4S_HIP_EINVALID_ARG, "sdpa_decode: NULL tensor pointer");
-    DL4S_REQUIRE(d == HD, DL4S_HIP_EUNSUPPORTED, "sdpa_decode: head dim %lld (only 64 is implemented)", (long long)d);
+    DL4S_REQUIRE(d >= 4 && d <= MAXD && d % 4 == 0, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa_decode: head dim %lld (multiples of 4 up to %d are implemented)", (long long)d, MAXD);
+    DL4S_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kcache) | reinterpret_cast<uintptr_t>(vcache) |
+                   reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) == 0, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa_decode: q, the caches and the new rows must be 16-byte aligned");
     DL4S_REQUIRE(T >= 1 && T <= Tcap, DL4S_HIP_ESHAPE, "sdpa_decode: T=%lld must be in [1, Tcap=%lld]", (long long)T,
                  (long long)Tcap);
     DL4S_REQUIRE(BH <= 65535 && Tcap < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa_decode: B*H=%lld above 65535", (long long)BH);
+    const int KB = 8 * (64 / lanes_per_row(d));   // keys per wavefront iteration
+    const int PSTR = pstr(4 * lanes_per_row(d));
     // Aim at 16 resident wavefronts on every CU.  Long caches use 16-wavefront workgroups; the key range is split
     // over several workgroups only when batch*heads alone does not fill the GPU.  Up to 512 rows one workgroup per pair
     // does it all (16 wavefronts above 128 rows): a second launch for the merge costs more than the split saves
-    // (B1 H8: 256 rows 6.4 -> 4.5 us, 512 rows 6.5 -> 4.8 us).
+    // (B1 H8: 256 rows 6.4 -> 4.5 us, 512 rows 6.5 -> 4.8 us).  The split follows T alone; with key lengths a workgroup
+    // whose share lies beyond its batch element's length leaves an empty record.
     const bool short_cache = T <= 512;
     const int nw = short_cache ? (T > 128 ? 16 : 4) : (T >= 2048 ? 16 : 4);
     const long long want_wg = ((long long)ctx->cu_count * 16 + nw - 1) / nw;
@@ -263,15 +327,15 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
         }
     }
     dim3 grid(nsplit, (unsigned)BH);
-#define DL4S_DECODE_LAUNCH(AP, NW_)                                                                                    \
-    hipLaunchKernelGGL((sdpa_decode_splitk_f32<AP, NW_>), grid, dim3(NW_ * 64), 0, ctx->stream, q, kcache, vcache, k_new,  \
-                       v_new, out, part, (int)T, (int)Tcap, (int)(AP ? pos : -1), rT, nsplit, chunk)
-    if (append) { if (nw == 16) DL4S_DECODE_LAUNCH(true, 16); else DL4S_DECODE_LAUNCH(true, 4); }
-    else { if (nw == 16) DL4S_DECODE_LAUNCH(false, 16); else DL4S_DECODE_LAUNCH(false, 4); }
-#undef DL4S_DECODE_LAUNCH
+    if (append)
+        decode_launch_width<true, false>(ctx, nw, grid, q, kcache, vcache, k_new, v_new, out, part, (int)T, (int)Tcap, (int)pos, rT, nsplit,
+                                         chunk, (int)d, (int)H, lengths, nullptr);
+    else
+        decode_launch_width<false, false>(ctx, nw, grid, q, kcache, vcache, k_new, v_new, out, part, (int)T, (int)Tcap, -1, rT, nsplit, chunk,
+                                          (int)d, (int)H, lengths, nullptr);
     int st = dl4s::launch_status("sdpa_decode_splitk_f32");
     if (st || nsplit == 1) return st;
-    hipLaunchKernelGGL(sdpa_decode_merge_f32, dim3((unsigned)BH), dim3(64), 0, ctx->stream, part, out, nsplit);
+    hipLaunchKernelGGL(sdpa_decode_merge_f32, dim3((unsigned)BH), dim3(MAXD), 0, ctx->stream, part, out, nsplit, 4 * lanes_per_row(d), (int)d);
     return dl4s::launch_status("sdpa_decode_merge_f32");
 }
 
@@ -300,12 +364,21 @@ int dl4s_hip_sdpa_decode_f32(dl4s_hip_ctx *ctx, const float *q, const float *kca
                          Tcap, -1, d, inv_temperature, false);
 }
 
+int dl4s_hip_sdpa_decode_lengths_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache, float *out,
+                                     int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d, float inv_temperature,
+                                     const int32_t *lengths) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(B >= 0 && H >= 0, DL4S_HIP_EINVALID_ARG, "sdpa_decode_lengths: negative extent");
+    return decode_launch(ctx, q, const_cast<float *>(kcache), const_cast<float *>(vcache), nullptr, nullptr, out, B, H, T,
+                         Tcap, -1, d, inv_temperature, false, lengths);
+}
+
 int dl4s_hip_sdpa_decode_noalloc_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache, float *out,
                                      int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d, float inv_temperature) {
     DL4S_CHECK_CTX(ctx);
     DL4S_REQUIRE(B >= 0 && H >= 0, DL4S_HIP_EINVALID_ARG, "sdpa_decode_noalloc: negative extent");
     return decode_launch(ctx, q, const_cast<float *>(kcache), const_cast<float *>(vcache), nullptr, nullptr, out, B, H, T,
-                         Tcap, -1, d, inv_temperature, false, true);
+                         Tcap, -1, d, inv_temperature, false, nullptr, true);
 }
 
 int dl4s_hip_kv_append_f32(dl4s_hip_ctx *ctx, float *kcache, float *vcache, const float *k_new, const float *v_new,
@@ -341,18 +414,19 @@ int dl4s_hip_sdpa_decode_step_at_f32(dl4s_hip_ctx *ctx, const float *q, float *k
     const int64_t BH = B * H;
     if (BH == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(q && kcache && vcache && out && k_new && v_new && pos_dev, DL4S_HIP_EINVALID_ARG, "sdpa_decode_step_at: NULL pointer");
-    DL4S_REQUIRE(d == HD, DL4S_HIP_EUNSUPPORTED, "sdpa_decode_step_at: head dim %lld (only 64 is implemented)", (long long)d);
+    DL4S_REQUIRE(d >= 4 && d <= MAXD && d % 4 == 0, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa_decode_step_at: head dim %lld (multiples of 4 up to %d are implemented)", (long long)d, MAXD);
+    DL4S_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kcache) | reinterpret_cast<uintptr_t>(vcache) |
+                   reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) == 0, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa_decode_step_at: q, the caches and the new rows must be 16-byte aligned");
     DL4S_REQUIRE(Tcap >= 1 && Tcap < (1ll << 30) && BH <= 65535, DL4S_HIP_EUNSUPPORTED,
                  "sdpa_decode_step_at: capacity %lld or B*H=%lld out of range", (long long)Tcap, (long long)BH);
     // the row count is not known on the host: one workgroup per pair walks whatever rows there are (16 wavefronts, 4 for a
-    // cache of up to 128 rows, where one 32-row block per wavefront covers it)
+    // cache of up to 128 rows, where one block per wavefront covers it)
+    const int KB = 8 * (64 / lanes_per_row(d));
     const int chunk = (int)((Tcap + KB - 1) / KB * KB);
-    if (Tcap > 128)
-        hipLaunchKernelGGL((sdpa_decode_splitk_f32<true, 16, true>), dim3(1, (unsigned)BH), dim3(16 * 64), 0, ctx->stream, q, kcache,
-                           vcache, k_new, v_new, out, (float *)nullptr, 0, (int)Tcap, 0, inv_temperature, 1, chunk, pos_dev);
-    else
-        hipLaunchKernelGGL((sdpa_decode_splitk_f32<true, 4, true>), dim3(1, (unsigned)BH), dim3(4 * 64), 0, ctx->stream, q, kcache,
-                           vcache, k_new, v_new, out, (float *)nullptr, 0, (int)Tcap, 0, inv_temperature, 1, chunk, pos_dev);
+    decode_launch_width<true, true>(ctx, Tcap > 128 ? 16 : 4, dim3(1, (unsigned)BH), q, kcache, vcache, k_new, v_new, out, nullptr, 0,
+                                    (int)Tcap, 0, inv_temperature, 1, chunk, (int)d, (int)H, nullptr, pos_dev);
     return dl4s::launch_status("sdpa_decode_splitk_f32");
 }
 

@@ -943,9 +943,9 @@ struct MultiHeadAttention {
         Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
         return normalized(out_drop, &q);
     }
-    // ---- one new position against cached keys and values (no counterpart in the reference; fused mode, head dim 64,
-    // dropout inactive).  x [B,1,hidden].  With a single position the joint normalisation and the per-token one coincide.
-    bool canDecodeIncrementally() const { return canCacheProjections() && keyDim == 64 && !dropout.isActive; }
+    // ---- one new position against cached keys and values (no counterpart in the reference; fused mode, head dims
+    // that are multiples of 4 up to 128, dropout inactive).  x [B,1,hidden].  With a single position the joint normalisation and the per-token one coincide.
+    bool canDecodeIncrementally() const { return canCacheProjections() && !dropout.isActive; }
     Tensor finishStep(const Tensor &x, const Tensor &attended) const {
         const int64_t B = x.shape[0];
         Tensor sum(Device::Memory::allocateBuffer(Shape{B, 1, hiddenDim}));
@@ -953,7 +953,7 @@ struct MultiHeadAttention {
         Device::Engine::denseFused(attended.view({B, heads * valueDim}).values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, sum.values());
         return norm.normalize(sum, nullptr);
     }
-    // self-attention: projects x, writes its key / value row into row `position` of the caches [B,H,capacity,64], attends
+    // self-attention: projects x, writes its key / value row into row `position` of the caches [B,H,capacity,d], attends
     // to rows 0 ... position
     // (positionOnDevice != nullptr: the row index is read from device memory instead, see Transformer::greedyCached)
     Tensor stepAppending(const Tensor &x, const Tensor &keyCache, const Tensor &valueCache, int64_t position,
@@ -976,7 +976,7 @@ struct MultiHeadAttention {
                                                      a.values(), attn.temperature);
         return finishStep(x, a);
     }
-    // attention to `rows` cached rows that do not change (the projected encoder states, head-major [B,H,rows,64])
+    // attention to `rows` cached rows that do not change (the projected encoder states, head-major [B,H,rows,d])
     Tensor stepAttending(const Tensor &x, const Tensor &keys, const Tensor &values) const {
         precondition(canDecodeIncrementally() && x.dim() == 3 && x.shape[1] == 1 && x.shape[2] == hiddenDim && keys.dim() == 4 &&
                          keys.shape == values.shape && keys.shape[0] == x.shape[0] && keys.shape[1] == heads && keys.shape[2] >= 1,
@@ -1076,7 +1076,7 @@ struct TransformerDecoderBlock {
         Tensor encAttn = encoderAttention.attendProjected(decAttn, encKeys, encValues, &encoderMask);
         return pointwiseFeedForward(encAttn);
     }
-    // one new position: decoderInput [B,1,hidden], self-attention caches [B,H,capacity,64], encoder keys / values [B,H,n,64]
+    // one new position: decoderInput [B,1,hidden], self-attention caches [B,H,capacity,d], encoder keys / values [B,H,n,d]
     Tensor step(const Tensor &decoderInput, const Tensor &keyCache, const Tensor &valueCache, int64_t position, const Tensor &encKeys,
                 const Tensor &encValues, const int32_t *positionOnDevice = nullptr) const {
         Tensor decAttn = selfAttention.stepAppending(decoderInput, keyCache, valueCache, position, positionOnDevice);
@@ -1289,15 +1289,15 @@ struct Transformer {
 
     // Greedy decoding with key / value caches: no counterpart in the reference, which re-runs the whole prefix at every
     // step (greedy() below).  A step runs the decoder on the one new position: every layer appends the position's
-    // self-attention key / value row to its cache [1,H,maxLength,64] and attends to the rows so far, then to the encoder
-    // states' keys / values, projected once and stored head-major [1,H,n,64].  Only a model whose attention layers
+    // self-attention key / value row to its cache [1,H,maxLength,d] and attends to the rows so far, then to the encoder
+    // states' keys / values, projected once and stored head-major [1,H,n,d].  Only a model whose attention layers
     // normalise per token computes the same function this way (the prefix re-run of such a model gives the same tokens and
     // the same logits up to summation order): with the reference's joint normalisation every earlier position's output
     // changes as the prefix grows, and the precondition refuses the model.
     std::vector<int32_t> greedyCached(const std::vector<int32_t> &inputSequence, int32_t startToken, int32_t endToken, int64_t maxLength,
                                       std::vector<float> *lastLogits = nullptr, bool recorded = true) const {
         precondition(canDecodeIncrementally(),
-                     "cached decoding needs fused mode, inactive dropout, head dim 64 and attention layers that normalise per token");
+                     "cached decoding needs fused mode, inactive dropout, equal key and value dims that are a multiple of 4 up to 128, and attention layers that normalise per token");
         const int64_t n = (int64_t)inputSequence.size(), D = embedding.outputSize(), vocab = embedding.embeddingMatrix.shape[0];
         precondition(startToken >= 0 && startToken < vocab, "index out of bounds");
         std::vector<int32_t> tokens;
@@ -1306,9 +1306,9 @@ struct Transformer {
         struct LayerState { Tensor encKeys, encValues, keyCache, valueCache; };
         std::vector<LayerState> state;
         for (auto &l : decoder.decoderLayers) {
-            auto kv = l.encoderAttention.projectKeysValues(encoded, encoded);                       // [1,n,H,64]
+            auto kv = l.encoderAttention.projectKeysValues(encoded, encoded);                       // [1,n,H,d]
             const Shape cache{1, l.selfAttention.heads, maxLength, l.selfAttention.keyDim};
-            state.push_back({kv.first.permuted({0, 2, 1, 3}), kv.second.permuted({0, 2, 1, 3}),    // [1,H,n,64]
+            state.push_back({kv.first.permuted({0, 2, 1, 3}), kv.second.permuted({0, 2, 1, 3}),    // [1,H,n,d]
                              Tensor(Device::Memory::allocateBuffer(cache)), Tensor(Device::Memory::allocateBuffer(cache))});
         }
         const Tensor positions = positionalEncoding(maxLength);

@@ -202,6 +202,13 @@ class Context:
         _check(self.lib.dl4s_hip_sdpa_decode_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(kcache)), _vp(_ptr(vcache)), _vp(_ptr(out)),
                                                  _i64(B), _i64(H), _i64(T), _i64(Tcap), _i64(d), C.c_float(inv_temperature)))
 
+    def sdpa_decode_lengths(self, q, kcache, vcache, out, B, H, T, Tcap, d, inv_temperature, lengths):
+        """sdpa_decode with a valid key count per batch element (device int32 [B], or None)."""
+        _check(self.lib.dl4s_hip_sdpa_decode_lengths_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(kcache)), _vp(_ptr(vcache)),
+                                                         _vp(_ptr(out)), _i64(B), _i64(H), _i64(T), _i64(Tcap), _i64(d),
+                                                         C.c_float(inv_temperature),
+                                                         _vp(_ptr(lengths)) if lengths is not None else None))
+
     def sdpa_decode_noalloc(self, q, kcache, vcache, out, B, H, T, Tcap, d, inv_temperature):
         """sdpa_decode with its partial records in the library's fixed device block (no allocation)."""
         _check(self.lib.dl4s_hip_sdpa_decode_noalloc_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(kcache)), _vp(_ptr(vcache)),

@@ -186,12 +186,22 @@ int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
                           int64_t Lq, int64_t Lk, int64_t d, float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
 
 /* One decode step: the same attention with Lq = 1 over the first T rows of a key/value cache laid
- * out [B,H,Tcap,d] (d = 64).  q, out [B,H,1,d].  The reference has no cache (greedy decoding re-runs
+ * out [B,H,Tcap,d] (d a multiple of 4 up to 128; the kernel is instantiated for rows of 32, 64 and 128 floats and other
+ * head dims run the next wider one with idle lanes; q, the caches and the new rows 16-byte aligned).  q, out [B,H,1,d].  The reference has no cache (greedy decoding re-runs
  * the prefix, NN/Models/Transformer/Transformer.swift:118-137); the result equals its
  * ScaledDotProductAttention on the gathered [B,H,T,d] tensors, no mask. */
 int dl4s_hip_sdpa_decode_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache,
                              float *out, int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d,
                              float inv_temperature);
+/* The same with a valid key count per batch element (device int32 lengths[B]): what ScaledDotProductAttention gives on the
+ * gathered [B,H,T,d] tensors under the mask of makeEncoderMasks, m[b,0,0,j] = (j >= lengths[b])
+ * (NN/Models/Transformer/TransformerUtil.swift:29-36).  With 1 <= lengths[b] the blocked keys have weight exactly zero in
+ * the reference and are not visited here (exact while K and V are finite there, as for the prefill kernels without
+ * DL4S_SDPA_STRICT); lengths[b] <= 0 blocks every key and the row comes out uniform over all T keys, as in the
+ * reference; lengths[b] >= T blocks nothing.  lengths == NULL is dl4s_hip_sdpa_decode_f32. */
+int dl4s_hip_sdpa_decode_lengths_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache,
+                                     float *out, int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d,
+                                     float inv_temperature, const int32_t *lengths);
 /* dl4s_hip_sdpa_decode_f32 for callers that cannot allocate device memory: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels, same bits;
  * the partial records of a decode that is split over the keys live in a fixed 2 MiB block of the library's own device

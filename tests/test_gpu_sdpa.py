@@ -366,10 +366,15 @@ def test_config3_shape_padding_mask_sampled(ctx, orc):
 
 
 # ------------------------------------------------------------------ decode
-def run_decode(ctx, q, kc, vc, T):
+def run_decode(ctx, q, kc, vc, T, lens=None):
     B, H, Tcap, d = kc.shape
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
     bufs = [ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc), ctx.empty((B, H, 1, d))]
-    ctx.sdpa_decode(bufs[0], bufs[1], bufs[2], bufs[3], B, H, T, Tcap, d, 0.125)
+    if lens is None:
+        ctx.sdpa_decode(bufs[0], bufs[1], bufs[2], bufs[3], B, H, T, Tcap, d, rT)
+    else:
+        bufs.append(ctx.to_device(np.asarray(lens, np.int32), dtype=np.int32))
+        ctx.sdpa_decode_lengths(bufs[0], bufs[1], bufs[2], bufs[3], B, H, T, Tcap, d, rT, bufs[4])
     out = bufs[3].numpy()
     for b in bufs:
         b.release()
@@ -390,6 +395,47 @@ def test_decode_matches_oracle(ctx, orc, B, H, T, Tcap):
     # and it is the same function as the prefill kernel with one query
     pre = run_sdpa(ctx, q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T]))
     assert_parity(got, pre, "decode vs prefill")
+
+
+@pytest.mark.parametrize("d", [32, 128, 8, 4, 40, 96, 100])
+@pytest.mark.parametrize("B,H,T,Tcap", [(1, 1, 1, 1), (2, 3, 9, 12), (2, 2, 129, 140), (1, 4, 257, 300), (1, 8, 513, 600),
+                                        (3, 2, 1000, 1024), (2, 2, 4097, 4160)])
+def test_decode_other_head_dims(ctx, orc, B, H, T, Tcap, d):
+    """Cache rows of 32 and 128 floats (8 and 32 lanes per row) and head dims that leave lanes idle."""
+    rng = np.random.default_rng(T * 1000 + d)
+    q, kc, vc = rand(rng, B, H, 1, d), rand(rng, B, H, Tcap, d), rand(rng, B, H, Tcap, d)
+    kc[:, :, T:] = np.nan
+    vc[:, :, T:] = np.nan
+    ref = orc.sdpa_decode(q, kc, vc, T)
+    got = run_decode(ctx, q, kc, vc, T)
+    assert_parity(got, ref, "decode T=%d d=%d" % (T, d))
+    assert_parity(got, run_sdpa(ctx, q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T])), "decode vs prefill")
+
+
+@pytest.mark.parametrize("d", [64, 32, 128, 24])
+@pytest.mark.parametrize("B,H,T,Tcap", [(4, 2, 9, 12), (5, 2, 300, 320), (6, 3, 1000, 1024), (4, 2, 4097, 4160)])
+def test_decode_with_key_lengths(ctx, orc, B, H, T, Tcap, d):
+    """dl4s_hip_sdpa_decode_lengths_f32 against the oracle's attention on the gathered tensors under the padding mask
+    m[b,0,0,j] = (j >= lengths[b]): a length inside the cache, the whole cache, beyond it, one key, and zero (every key
+    blocked: the row is uniform over all T keys, never NaN)."""
+    rng = np.random.default_rng(T * 100 + d)
+    q, kc, vc = rand(rng, B, H, 1, d), rand(rng, B, H, Tcap, d), rand(rng, B, H, Tcap, d)
+    kc[:, :, T:] = np.nan
+    vc[:, :, T:] = np.nan
+    lens = rng.integers(1, T + 1, size=B)
+    lens[0], lens[1], lens[2], lens[3] = T, 0, 1, T + 50
+    mask = lengths_mask(lens, T)
+    ref = orc.sdpa(q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T]), mask)
+    got = run_decode(ctx, q, kc, vc, T, lens=lens)
+    assert_parity(got, ref, "decode with lengths T=%d d=%d" % (T, d))
+    assert np.allclose(got[1], vc[1, :, :T].mean(axis=1, keepdims=True), atol=1e-5)      # length zero: uniform
+    assert np.array_equal(got[2], vc[2, :, :1])                                           # one key
+    assert np.array_equal(got[0], run_decode(ctx, q, kc, vc, T)[0])                        # nothing blocked: the plain entry's bits
+    # and it is what the prefill kernel gives for one query under the key-length descriptor
+    from dl4s_amd import lib
+    pre = run_sdpa(ctx, q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T]), kind=lib.MASK_KEY_LENGTHS,
+                   lens=np.minimum(lens, T))
+    assert_parity(got, pre, "decode with lengths vs prefill")
 
 
 def test_decode_nan_inf(ctx, orc):

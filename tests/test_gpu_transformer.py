@@ -271,13 +271,26 @@ def test_cached_greedy_decoding(ctx):
     model.close()
 
 
-def test_cached_decoding_needs_head_dim_64(ctx):
+def test_cached_decoding_with_the_reference_test_models_key_size(ctx):
+    """Key / value dim 8 (Tests/DL4STests/TransformerTests.swift:31): the decode kernels take every multiple of 4 up to
+    128, so the per-token variant of that model decodes with caches too - same tokens as the oracle's prefix re-run,
+    logits inside the gate, replayed and issued call by call the same bits."""
     from dl4s_amd import host_lib
-    params, rng = _model(48, *CONFIGS["transformer_tests_hyperparameters"])
+    from oracle import transformer as T
+    name = "transformer_tests_hyperparameters"
+    params, rng = _model(48, *CONFIGS[name])
+    src = [int(t) for t in rng.integers(0, CONFIGS[name][0], 6)]
+    steps = 18
+    ref_tokens, ref_logits = T.greedy_decode(params, src, 1, -5, steps, return_logits=True, norm_per_token=True)
+    top2 = np.sort(np.stack(ref_logits), axis=1)[:, -2:]
+    assert (top2[:, 1] - top2[:, 0]).min() > 1e-3, "the fixture must not sit on an argmax tie"
     model = host_lib.Transformer(ctx, params)
     model.set_norm_per_token(True)
-    with pytest.raises(host_lib.HostError, match="head dim 64"):
-        model.greedy([3, 4, 5], 1, 2, 4, cached=True)
+    toks, logits = model.greedy(src, 1, -5, steps, cached=True, return_logits=True)
+    assert toks == ref_tokens
+    assert_parity(logits, np.stack(ref_logits), "cached greedy logits, key size 8")
+    toks_s, logits_s = model.greedy(src, 1, -5, steps, cached="stepwise", return_logits=True)
+    assert toks_s == toks and np.array_equal(logits_s, logits)
     model.close()
 
 
