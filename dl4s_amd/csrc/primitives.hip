@@ -180,6 +180,41 @@ __global__ void permute_f32(const float *__restrict__ x, float *__restrict__ y, 
     }
 }
 
+// Copy between a box of a row-major tensor and a contiguous buffer (the slice forms of get / set(slice:)).  The box is
+// described after merging axes: `run` contiguous floats per piece, and the pieces' offsets in the tensor from up to
+// DL4S_HIP_MAX_DIM outer axes (count, stride in floats).  READ: tensor -> buffer; else buffer -> tensor.
+struct SliceBox {
+    int dim;                                 // outer axes
+    long long count[DL4S_HIP_MAX_DIM];
+    long long stride[DL4S_HIP_MAX_DIM];
+    long long run;                           // contiguous floats per piece
+    long long base;                          // offset of the box's first element in the tensor
+};
+typedef float slice_f32x4 __attribute__((ext_vector_type(4)));
+template <bool READ, int VEC>
+__global__ void slice_copy_f32(const float *__restrict__ src, float *__restrict__ dst, SliceBox bx, long long n) {
+    // n counts units of VEC floats; run is a multiple of VEC
+    const long long run_units = bx.run / VEC;
+    for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (long long)gridDim.x * blockDim.x) {
+        long long piece = e / run_units;
+        const long long within = (e - piece * run_units) * VEC;
+        long long off = bx.base + within;
+#pragma unroll 1
+        for (int i = bx.dim - 1; i >= 0; --i) {
+            off += (piece % bx.count[i]) * bx.stride[i];
+            piece /= bx.count[i];
+        }
+        const long long lin = e * VEC;
+        if (VEC == 4) {
+            if (READ) *reinterpret_cast<slice_f32x4 *>(dst + lin) = *reinterpret_cast<const slice_f32x4 *>(src + off);
+            else *reinterpret_cast<slice_f32x4 *>(dst + off) = *reinterpret_cast<const slice_f32x4 *>(src + lin);
+        } else {
+            if (READ) dst[lin] = src[off];
+            else dst[off] = src[lin];
+        }
+    }
+}
+
 __global__ void band_f32(const float *__restrict__ x, float *__restrict__ y, long long rows, long long cols, long long below,
                          long long above) {
     const long long n = rows * cols;
@@ -544,6 +579,49 @@ __global__ __launch_bounds__(256) void log_softmax_f32(const float *__restrict__
     for (long long i = threadIdx.x; i < n; i += 256) yr[i] = __fsub_rn(__fadd_rn(xr[i], -mx), lse);
 }
 
+// Validates the box and merges axes: trailing axes taken whole join the contiguous run, the rest become outer axes.
+int make_slice_box(const int64_t *shape, int dim, const int64_t *start, const int64_t *extent, SliceBox &bx, long long &total,
+                   const char *what) {
+    DL4S_REQUIRE(dim >= 0 && dim <= DL4S_HIP_MAX_DIM, DL4S_HIP_EINVALID_ARG, "%s: dim %d not in [0,%d]", what, dim, DL4S_HIP_MAX_DIM);
+    DL4S_REQUIRE(dim == 0 || (shape && start && extent), DL4S_HIP_EINVALID_ARG, "%s: NULL shape / start / extent", what);
+    long long strides[DL4S_HIP_MAX_DIM];
+    long long s = 1;
+    total = 1;
+    for (int i = dim - 1; i >= 0; --i) {
+        DL4S_REQUIRE(shape[i] >= 0 && start[i] >= 0 && extent[i] >= 0 && start[i] + extent[i] <= shape[i], DL4S_HIP_ESHAPE,
+                     "%s: axis %d: [%lld, %lld) is not inside [0, %lld)", what, i, (long long)start[i], (long long)(start[i] + extent[i]),
+                     (long long)shape[i]);
+        strides[i] = s;
+        s *= shape[i];
+        total *= extent[i];
+    }
+    bx = SliceBox{};
+    bx.run = 1;
+    int i = dim - 1;
+    for (; i >= 0; --i) {            // the run ends with the first axis (from the right) that is not taken whole
+        bx.run *= extent[i];
+        bx.base += start[i] * strides[i];
+        if (extent[i] != shape[i]) { --i; break; }
+    }
+    for (int a = 0; a <= i; ++a) {   // outer axes, those of extent 1 only move the base
+        bx.base += start[a] * strides[a];
+        if (extent[a] == 1) continue;
+        bx.count[bx.dim] = extent[a];
+        bx.stride[bx.dim] = strides[a];
+        ++bx.dim;
+    }
+    return DL4S_HIP_OK;
+}
+
+template <bool READ>
+int launch_slice_copy(dl4s_hip_ctx *ctx, const float *src, float *dst, const SliceBox &bx, long long total, const float *tensor,
+                      const float *buffer) {
+    bool vec = bx.run % 4 == 0 && bx.base % 4 == 0 && ((reinterpret_cast<uintptr_t>(tensor) | reinterpret_cast<uintptr_t>(buffer)) & 15) == 0;
+    for (int i = 0; i < bx.dim; ++i) vec = vec && bx.stride[i] % 4 == 0;
+    if (vec) hipLaunchKernelGGL((slice_copy_f32<READ, 4>), dim3(grid_for(total / 4, 2)), dim3(TPB), 0, ctx->stream, src, dst, bx, total / 4);
+    else hipLaunchKernelGGL((slice_copy_f32<READ, 1>), dim3(grid_for(total, 2)), dim3(TPB), 0, ctx->stream, src, dst, bx, total);
+    return dl4s::launch_status(READ ? "subscriptRead" : "subscriptWrite");
+}
 }  // namespace
 
 extern "C" {
@@ -773,6 +851,28 @@ int dl4s_hip_permute_axes_f32(dl4s_hip_ctx *ctx, const float *values, const int6
     for (int i = 0; i < dim; ++i) p.dstride[i] = dstr[arrangement[i]];
     hipLaunchKernelGGL(permute_f32, dim3(grid_for(n, 2)), dim3(TPB), 0, ctx->stream, values, result, p, n);
     return dl4s::launch_status("permuteAxes");
+}
+
+int dl4s_hip_subscript_read_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim, const int64_t *start,
+                                const int64_t *extent, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    SliceBox bx;
+    long long total = 0;
+    const int rc = make_slice_box(shape, dim, start, extent, bx, total, "subscriptRead");
+    if (rc != DL4S_HIP_OK || total == 0) return rc;
+    DL4S_REQUIRE(values && result, DL4S_HIP_EINVALID_ARG, "subscriptRead: NULL pointer");
+    return launch_slice_copy<true>(ctx, values, result, bx, total, values, result);
+}
+
+int dl4s_hip_subscript_write_f32(dl4s_hip_ctx *ctx, const float *values, float *result, const int64_t *shape, int dim,
+                                 const int64_t *start, const int64_t *extent) {
+    DL4S_CHECK_CTX(ctx);
+    SliceBox bx;
+    long long total = 0;
+    const int rc = make_slice_box(shape, dim, start, extent, bx, total, "subscriptWrite");
+    if (rc != DL4S_HIP_OK || total == 0) return rc;
+    DL4S_REQUIRE(values && result, DL4S_HIP_EINVALID_ARG, "subscriptWrite: NULL pointer");
+    return launch_slice_copy<false>(ctx, values, result, bx, total, result, values);
 }
 
 int dl4s_hip_band_f32(dl4s_hip_ctx *ctx, const float *buffer, float *result, int64_t rows, int64_t cols, int has_below,

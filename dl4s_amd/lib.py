@@ -325,6 +325,16 @@ class Context:
         arr = (C.c_int32 * max(1, len(arrangement)))(*arrangement)
         _check(self.lib.dl4s_hip_permute_axes_f32(self.handle, _vp(_ptr(x)), _shape_arr(shape), len(shape), arr, _vp(_ptr(y))))
 
+    def subscript_read(self, x, shape, start, extent, y):
+        """y (contiguous, shape `extent`) = x[start : start + extent] along every axis."""
+        _check(self.lib.dl4s_hip_subscript_read_f32(self.handle, _vp(_ptr(x)), _shape_arr(shape), len(shape), _shape_arr(start),
+                                                    _shape_arr(extent), _vp(_ptr(y))))
+
+    def subscript_write(self, x, y, shape, start, extent):
+        """y[start : start + extent] = x (contiguous, shape `extent`); y has shape `shape`."""
+        _check(self.lib.dl4s_hip_subscript_write_f32(self.handle, _vp(_ptr(x)), _vp(_ptr(y)), _shape_arr(shape), len(shape),
+                                                     _shape_arr(start), _shape_arr(extent)))
+
     def stack(self, buffers, count, y):
         arr = (_vp * max(1, len(buffers)))(*[_ptr(b) for b in buffers])
         _check(self.lib.dl4s_hip_stack_f32(self.handle, arr, _i64(len(buffers)), _i64(count), _vp(_ptr(y))))

@@ -304,6 +304,16 @@ int dl4s_hip_argmax_f32(dl4s_hip_ctx *ctx, const float *values, int64_t count, i
  * (Engine/CPU/CPUEngine.swift:897-935). */
 int dl4s_hip_permute_axes_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim,
                               const int32_t *arrangement, float *result);
+/* :493 subscriptRead / :500 subscriptWrite, and the slice forms of MemoryOperatorsType.get(slice:) / set(slice:) (:100-126;
+ * semantics Engine/CPU/CPU.swift:137-218): one launch copies the box [start[i], start[i] + extent[i]) of a row-major tensor
+ * of shape `shape[dim]` to (read) or from (write) a contiguous buffer of shape `extent`.  An index entry Int i is
+ * start = i, extent = 1 (the reference then drops the axis from the result's shape; the layout is the same), nil is
+ * start = 0, extent = shape, a range is its lower bound and count.  A pure prefix index needs no copy: it is the offset view
+ * of CPU.swift:146-157, plain pointer arithmetic on this side too.  A box that leaves the tensor is DL4S_HIP_ESHAPE. */
+int dl4s_hip_subscript_read_f32(dl4s_hip_ctx *ctx, const float *values, const int64_t *shape, int dim, const int64_t *start,
+                                const int64_t *extent, float *result);
+int dl4s_hip_subscript_write_f32(dl4s_hip_ctx *ctx, const float *values, float *result, const int64_t *shape, int dim,
+                                 const int64_t *start, const int64_t *extent);
 /* :536 stack along axis 0 of `n` equally shaped buffers of `count` elements each
  * (Tensor/Operators/Stack.swift:79-98 as used by broadcastMatrixMultiplied). */
 int dl4s_hip_stack_f32(dl4s_hip_ctx *ctx, const float *const *buffers, int64_t n, int64_t count, float *result);

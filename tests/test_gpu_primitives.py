@@ -336,6 +336,60 @@ def test_layernorm(ctx, orc, B, rows, D):
         t.release()
 
 
+SLICES = [   # shape, index as numpy would write it (int, slice or None = whole axis)
+    ((5, 7), (2, None)),                      # a prefix index (the reference returns a view; the copy must agree)
+    ((5, 7), (None, 3)),                      # a column: runs of one float
+    ((4, 6, 8), (None, 2, None)),
+    ((4, 6, 8), (1, None, 5)),
+    ((4, 6, 8), (slice(1, 3), slice(0, 6), slice(4, 8))),     # ranges; 128-bit pieces
+    ((4, 6, 8), (slice(1, 3), slice(2, 5), slice(1, 7))),
+    ((3, 4, 5, 6), (None, slice(1, 2), None, slice(0, 6))),
+    ((2, 3, 4, 5, 6), (1, None, slice(1, 4), 2, None)),
+    ((64, 1024), (slice(3, 60), slice(128, 896))),
+    ((7,), (slice(2, 2),)),                   # empty
+    ((6, 5), ()),                             # everything
+]
+
+
+@pytest.mark.parametrize("shape,index", SLICES)
+def test_subscript_read_and_write_match_numpy_slicing(ctx, shape, index):
+    """Engine/Engine.swift:493-500 and MemoryOperatorsType.get / set(slice:) (semantics Engine/CPU/CPU.swift:137-218): one
+    launch per slice, bit-exact against numpy's slicing of the same tensor."""
+    x = rnd(*shape)
+    idx = tuple(index) + (None,) * (len(shape) - len(index))
+    start = [i if isinstance(i, int) else (i.start if isinstance(i, slice) else 0) for i in idx]
+    extent = [1 if isinstance(i, int) else ((i.stop - i.start) if isinstance(i, slice) else n) for i, n in zip(idx, shape)]
+    box = tuple(slice(s, s + e) for s, e in zip(start, extent))
+    want = x[box]                                   # the axes an integer index would drop are kept with extent 1
+    dx, dy = ctx.to_device(x), ctx.empty(tuple(extent))
+    ctx.fill(float("nan"), dy, int(np.prod(extent)))
+    ctx.subscript_read(dx, shape, start, extent, dy)
+    assert np.array_equal(dy.numpy(), want)
+    # write: the box takes new values, every other element keeps its own
+    new = rnd(*extent)
+    dn = ctx.to_device(new)
+    ctx.subscript_write(dn, dx, shape, start, extent)
+    expect = x.copy()
+    expect[box] = new
+    assert np.array_equal(dx.numpy(), expect)
+    for t in (dx, dy, dn):
+        t.release()
+
+
+def test_subscript_box_outside_the_tensor_is_refused(ctx):
+    from dl4s_amd import lib
+    dx, dy = ctx.empty((4, 6)), ctx.empty((4, 6))
+    for start, extent in (([0, 3], [4, 4]), ([-1, 0], [2, 2]), ([4, 0], [1, 6])):
+        with pytest.raises(lib.Dl4sHipError) as e:
+            ctx.subscript_read(dx, (4, 6), start, extent, dy)
+        assert e.value.code == -2
+        with pytest.raises(lib.Dl4sHipError) as e:
+            ctx.subscript_write(dy, dx, (4, 6), start, extent)
+        assert e.value.code == -2
+    dx.release()
+    dy.release()
+
+
 def _ln(ctx, x, scale, shift):
     B, rows, D = x.shape
     dx, ds, dh, dy = ctx.to_device(x), ctx.to_device(scale), ctx.to_device(shift), ctx.empty((B, rows, D))
