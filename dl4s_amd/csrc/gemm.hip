@@ -147,30 +147,33 @@ __global__ __launch_bounds__(256, 2) void gemm_f32_mfma(GemmArgs g) {
 
 // Fast kernels: 128-bit buffer loads, K and the unit-stride extents multiples of 4, 16-byte aligned operands.  Same
 // 2x2 wavefront layout as above.  An operand is staged in one of two ways, chosen by how it lies in memory:
-//   rows x K, K contiguous (A, or B when transposeSecond)   kept [row][k] in LDS on a 20-float row stride, so that
+//   rows x K, K contiguous (A, or B when transposeSecond)   kept [row][k] in LDS on a row stride of KT + 4 floats, so that
 //                                                           128-bit operand reads of 8 rows fall on distinct banks
 //                                                           and one LDS read feeds four MFMA steps
 //   K x rows, rows contiguous (B, or A when transposeFirst) kept [k][row] in LDS, read one word per MFMA step
 // Both go through buffer loads with the whole byte offset in the (range-checked) vector operand: rows past the extent,
 // K rows past K and -- through an offset beyond any descriptor -- columns past the extent read as zeros, so a K step
-// costs one add per load and no predication.  MFMA step s of a K tile takes k = 8*half + s from both operands (any
-// bijection of k works as long as A and B agree).
-constexpr int ALS = GBK + 4;   // LDS row stride of a [row][k] tile (floats)
+// costs one add per load and no predication.  MFMA step s of a 16-deep half of a K tile takes k = 8*half + s from both
+// operands (any bijection of k works as long as A and B agree).
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr unsigned OUTSIDE = 0x80000000u;   // an offset beyond every descriptor (the host keeps them below 2^31 bytes)
 
 // One operand of the fast kernels.  XI = MFMA tiles per wavefront along this operand's extent (tile extent T = 64*XI);
-// KROWS = true for the K x rows memory layout.
-template <int XI, bool KROWS>
+// KROWS = true for the K x rows memory layout; KT = depth of a K tile (16 or 32).  A K tile of 32 is contracted as two
+// halves of 16 one after the other, so that an output element sees its products in the same order whatever KT is.
+template <int XI, bool KROWS, int KT>
 struct FastOperand {
     static constexpr int T = 64 * XI;
-    static constexpr int LDS_FLOATS = KROWS ? 2 * GBK * (T + 4) : 2 * T * ALS;
-    static constexpr int Q = T / 4, PASS_ROWS = 256 / Q;   // K x rows: float4 per K row, K rows covered per pass
+    static constexpr int LS = KT + 4;            // row stride of a [row][k] tile (floats): 128-bit reads of 8 rows on distinct banks
+    static constexpr int LDS_FLOATS = KROWS ? 2 * KT * (T + 4) : 2 * T * LS;
+    static constexpr int NV = XI * KT / 16;      // 128-bit pieces per thread and K tile
+    static constexpr int Q = T / 4, PASS_ROWS = 256 / Q;      // K x rows: pieces per K row, K rows covered per pass
+    static constexpr int QK = KT / 4, RP = 256 / QK;          // rows x K: pieces per row, rows covered per pass
     float *lds;
     __amdgpu_buffer_rsrc_t rsrc;
-    unsigned off[XI];
+    unsigned off[NV];
     unsigned step;          // byte step of one K tile
-    f32x4 st[XI];
+    f32x4 st[NV];
     int kq;                 // rows x K: the thread's k quad
     bool ragged_k;
     int K;
@@ -179,58 +182,62 @@ struct FastOperand {
     __device__ __forceinline__ void init(float *lds_, const float *base, int extent, long long rs, int r0, int K_, int tid) {
         lds = lds_;
         K = K_;
-        ragged_k = (K % GBK) != 0;
+        ragged_k = (K % KT) != 0;
         if (KROWS) {
             const int krow = tid / Q, rq = (tid % Q) * 4;
             rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(base + r0), 0, (int)((((long long)K - 1) * rs + (extent - r0)) * 4), 0x00020000);
 #pragma unroll
-            for (int i = 0; i < XI; ++i) off[i] = (r0 + rq < extent) ? (unsigned)((krow + PASS_ROWS * i) * (int)rs + rq) * 4u : OUTSIDE;
-            step = (unsigned)GBK * (unsigned)rs * 4u;
+            for (int i = 0; i < NV; ++i) off[i] = (r0 + rq < extent) ? (unsigned)((krow + PASS_ROWS * i) * (int)rs + rq) * 4u : OUTSIDE;
+            step = (unsigned)KT * (unsigned)rs * 4u;
             kq = 0;
         } else {
-            const int row = tid >> 2;
-            kq = (tid & 3) * 4;
+            const int row = tid / QK;
+            kq = (tid % QK) * 4;
             const long long rem = ((long long)(extent - r0 - 1) * rs + K) * 4;
             rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(base + (long long)r0 * rs), 0, (int)(rem < 0x7fffffffll ? rem : 0x7fffffffll), 0x00020000);
 #pragma unroll
-            for (int i = 0; i < XI; ++i) off[i] = (r0 + row + 64 * i < extent) ? (unsigned)((row + 64 * i) * (int)rs + kq) * 4u : OUTSIDE;
-            step = (unsigned)GBK * 4u;
+            for (int i = 0; i < NV; ++i) off[i] = (r0 + row + RP * i < extent) ? (unsigned)((row + RP * i) * (int)rs + kq) * 4u : OUTSIDE;
+            step = (unsigned)KT * 4u;
         }
     }
     __device__ __forceinline__ void load(int kt) {
         // rows x K on the last K step of a ragged K: quads at or past K lie inside the next row, so they are sent outside
-        const bool past = !KROWS && ragged_k && (kt * GBK + kq >= K);
+        const bool past = !KROWS && ragged_k && (kt * KT + kq >= K);
 #pragma unroll
-        for (int i = 0; i < XI; ++i)
+        for (int i = 0; i < NV; ++i)
             st[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(past ? OUTSIDE : off[i] + kt * step), 0, 0));
     }
     __device__ __forceinline__ void store(int buf, int tid) {
         if (KROWS) {
             const int krow = tid / Q, rq = (tid % Q) * 4;
 #pragma unroll
-            for (int i = 0; i < XI; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * GBK + krow + PASS_ROWS * i) * (T + 4) + rq) = st[i];
+            for (int i = 0; i < NV; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * KT + krow + PASS_ROWS * i) * (T + 4) + rq) = st[i];
         } else {
-            const int row = tid >> 2;
+            const int row = tid / QK;
 #pragma unroll
-            for (int i = 0; i < XI; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * T + row + 64 * i) * ALS + kq) = st[i];
+            for (int i = 0; i < NV; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * T + row + RP * i) * LS + kq) = st[i];
         }
     }
-    // rows x K: the lane's fragment of tile x for the whole K tile (k = 8*half .. 8*half + 7)
-    __device__ __forceinline__ void fragment(int buf, int row, int half, f32x4 (&f)[2]) const {
-        f[0] = *reinterpret_cast<const f32x4 *>(lds + (buf * T + row) * ALS + 8 * half);
-        f[1] = *reinterpret_cast<const f32x4 *>(lds + (buf * T + row) * ALS + 8 * half + 4);
+    // rows x K: the lane's fragment of tile x for half h2 of the K tile (k = 16*h2 + 8*half .. + 7)
+    __device__ __forceinline__ void fragment(int buf, int row, int half, int h2, f32x4 (&f)[2]) const {
+        f[0] = *reinterpret_cast<const f32x4 *>(lds + (buf * T + row) * LS + 16 * h2 + 8 * half);
+        f[1] = *reinterpret_cast<const f32x4 *>(lds + (buf * T + row) * LS + 16 * h2 + 8 * half + 4);
     }
-    // K x rows: the lane's value for MFMA step s8
-    __device__ __forceinline__ float word(int buf, int row, int half, int s8) const { return lds[(buf * GBK + 8 * half + s8) * (T + 4) + row]; }
+    // K x rows: the lane's value for MFMA step s8 of half h2
+    __device__ __forceinline__ float word(int buf, int row, int half, int h2, int s8) const {
+        return lds[(buf * KT + 16 * h2 + 8 * half + s8) * (T + 4) + row];
+    }
 };
 
 // MI x NI = MFMA tiles per wavefront (2x2: 128x128 workgroup tile for large products, 1x1: 64x64 so that small
 // products still put a workgroup on every CU).  TA / TB: the operand is stored transposed (transposeFirst / Second).
-template <int MI, int NI, bool EPI, bool TA, bool TB>
+// KT: K tile depth.  The 64x64 form runs one to three wavefronts per SIMD, where a K tile of 16 (8 MFMAs = 512 cycles
+// between barriers) does not cover the latency of the next tile's loads; it takes K tiles of 32.
+template <int MI, int NI, bool EPI, bool TA, bool TB, int KT>
 __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
     constexpr int TM = 64 * MI, TN = 64 * NI;       // workgroup tile
-    using OpA = FastOperand<MI, TA>;                 // A is M x K in memory unless transposed
-    using OpB = FastOperand<NI, !TB>;                // B is K x N in memory unless transposed
+    using OpA = FastOperand<MI, TA, KT>;             // A is M x K in memory unless transposed
+    using OpB = FastOperand<NI, !TB, KT>;            // B is K x N in memory unless transposed
     __shared__ __align__(16) float As[OpA::LDS_FLOATS];
     __shared__ __align__(16) float Bs[OpB::LDS_FLOATS];
     const int tid = threadIdx.x;
@@ -255,7 +262,7 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int ktiles = (g.K + GBK - 1) / GBK;
+    const int ktiles = (g.K + KT - 1) / KT;
     opa.load(0);
     opb.load(0);
     opa.store(0, tid);
@@ -267,29 +274,32 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
         constexpr int buf = decltype(buf_c)::value;
         const bool more = kt + 1 < ktiles;
         if (more) { opa.load(kt + 1); opb.load(kt + 1); }
-        f32x4 af[MI][2], bf[NI][2];
-        if (!TA) {
 #pragma unroll
-            for (int i = 0; i < MI; ++i) opa.fragment(buf, wm * 32 * MI + i * 32 + ln, half, af[i]);
-        }
-        if (TB) {
+        for (int h2 = 0; h2 < KT / 16; ++h2) {
+            f32x4 af[MI][2], bf[NI][2];
+            if (!TA) {
 #pragma unroll
-            for (int j = 0; j < NI; ++j) opb.fragment(buf, wn * 32 * NI + j * 32 + ln, half, bf[j]);
-        }
+                for (int i = 0; i < MI; ++i) opa.fragment(buf, wm * 32 * MI + i * 32 + ln, half, h2, af[i]);
+            }
+            if (TB) {
 #pragma unroll
-        for (int s8 = 0; s8 < 8; ++s8) {
-            float av[MI], bv[NI];
+                for (int j = 0; j < NI; ++j) opb.fragment(buf, wn * 32 * NI + j * 32 + ln, half, h2, bf[j]);
+            }
 #pragma unroll
-            for (int i = 0; i < MI; ++i) av[i] = TA ? opa.word(buf, wm * 32 * MI + i * 32 + ln, half, s8) : af[i][s8 >> 2][s8 & 3];
+            for (int s8 = 0; s8 < 8; ++s8) {
+                float av[MI], bv[NI];
 #pragma unroll
-            for (int j = 0; j < NI; ++j) bv[j] = TB ? bf[j][s8 >> 2][s8 & 3] : opb.word(buf, wn * 32 * NI + j * 32 + ln, half, s8);
+                for (int i = 0; i < MI; ++i) av[i] = TA ? opa.word(buf, wm * 32 * MI + i * 32 + ln, half, h2, s8) : af[i][s8 >> 2][s8 & 3];
 #pragma unroll
-            for (int i = 0; i < MI; ++i)
+                for (int j = 0; j < NI; ++j) bv[j] = TB ? bf[j][s8 >> 2][s8 & 3] : opb.word(buf, wn * 32 * NI + j * 32 + ln, half, h2, s8);
 #pragma unroll
-                for (int j = 0; j < NI; ++j)
-                    // operands swapped: the accumulator is the TRANSPOSED tile (lane = row m, registers = columns n), so
-                    // that a lane holds four consecutive columns and the epilogue moves 128 bits per access
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        // operands swapped: the accumulator is the TRANSPOSED tile (lane = row m, registers = columns n), so
+                        // that a lane holds four consecutive columns and the epilogue moves 128 bits per access
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
+            }
         }
         if (more) { opa.store(buf ^ 1, tid); opb.store(buf ^ 1, tid); }
         __syncthreads();
@@ -669,7 +679,7 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.tiles_n = (int)tn;
     DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
     const dim3 grid((unsigned)(tm * tn), 1, (unsigned)batch);
-#define DL4S_GEMM_FAST(MI_, EPI_, TA_, TB_) hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_>), grid, dim3(256), 0, ctx->stream, g)
+#define DL4S_GEMM_FAST(MI_, EPI_, TA_, TB_) hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, (MI_ == 1 ? 32 : 16)>), grid, dim3(256), 0, ctx->stream, g)
     if (fast) {
         const int variant = (small ? 0 : 8) + (epi ? 4 : 0) + (ta ? 2 : 0) + (tb ? 1 : 0);
         switch (variant) {
