@@ -26,6 +26,7 @@
 // plain kernels at the end of the file.
 #include "sdpa_common.h"
 #include "sdpa_backward_d128.h"
+#include "sdpa_backward_narrow.h"
 
 #include <cstdlib>
 
@@ -355,15 +356,26 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
         ds_voff = ((unsigned)key * (unsigned)Lqp + 4u * half) * 4u;
     }
 
-    for (int t = t_begin; t < nqt; ++t) {
+    // Tiles before the wavefront's first one (causal masks), and every tile of a wavefront without a valid key, are only
+    // staged.  The loop over the tiles the wavefront computes on is kept free of that test: with the dS stores on every
+    // path through its body the compiler can tell that they follow the next tile's loads, and the wait before the LDS
+    // writes covers the loads alone instead of the stores' round trip to memory.
+    int t = t_begin;
+    const int wt_first = __builtin_amdgcn_readfirstlane(wave_active ? max(wt_begin, t_begin) : nqt);   // the same in every lane
+    for (; t < wt_first && t < nqt; ++t) {
+        const int buf = (t - t_begin) & 1;
+        if (t + 1 < nqt) { load_tile(t + 1); store_tile(buf ^ 1); }
+        __syncthreads();
+    }
+    wait_vector_memory();   // the loads of the lane's key and value rows: nothing from before the loop is left in flight
+    for (; t < nqt; ++t) {
         const int buf = (t - t_begin) & 1;
         const bool more = (t + 1 < nqt);
         if (more) load_tile(t + 1);
         const int qt0 = t * 32;
         int cls = 2;
         if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq] & 3;
-        if (wave_active && t >= wt_begin &&
-            !(DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5))) {
+        if (!(DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5))) {
             // S[query, key] in the base-2 domain: rows = the tile's queries 8(r/4) + 4*half + r%4, column = the lane's key
             f32x16 p = tile_product(Qs + buf * TILE_FLOATS + row_lds, kr);
             if (DENSE) {
@@ -416,7 +428,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const f32x4 o = {p[4 * g + 0], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]};
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 2);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 0);
                 }
             }
             tile_accumulate_t(Qs + buf * TILE_FLOATS + col_lds, p, k0a, k1a);                   // dK^T += Q~^T . dS
@@ -985,6 +997,13 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
                int strict, int token_major, int hd, int no_split) {
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    if (hd <= 32) {     // narrow heads: tiles of 16 or 32 columns on the stored-dS route, when the launch can take it
+        const int rn = hd <= 16 ? launch_bwd_narrow<KIND, 16>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, rT, m, strict, token_major,
+                                                              hd, no_split, ds_scratch_max_bytes())
+                                : launch_bwd_narrow<KIND, 32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, rT, m, strict, token_major,
+                                                              hd, no_split, ds_scratch_max_bytes());
+        if (rn != 0) return rn < 0 ? rn : DL4S_HIP_OK;
+    }
     const size_t lds_dq = 4 * TILE_FLOATS * sizeof(float);
     const size_t lds_dkv = (4 * TILE_FLOATS + 192) * sizeof(float);
     const size_t lds_dq_split = 8 * TILE_FLOATS * sizeof(float);

@@ -319,15 +319,23 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         ds_voff = ((unsigned)key * (unsigned)Lqp + 4u * half) * 4u;
     }
 
-    for (int t = t_begin; t < nqt; ++t) {
+    // tiles the wavefront only stages first, then a loop whose every path stores dS (see sdpa_bwd_dkv_f32_d64)
+    int t = t_begin;
+    const int wt_first = __builtin_amdgcn_readfirstlane(wave_active ? max(wt_begin, t_begin) : nqt);   // the same in every lane
+    for (; t < wt_first && t < nqt; ++t) {
+        const int buf = (t - t_begin) & 1;
+        if (t + 1 < nqt) { load_tile(t + 1); store_tile(buf ^ 1); }
+        __syncthreads();
+    }
+    wait_vector_memory();   // the loads of the lane's key and value rows: nothing from before the loop is left in flight
+    for (; t < nqt; ++t) {
         const int buf = (t - t_begin) & 1;
         const bool more = (t + 1 < nqt);
         if (more) load_tile(t + 1);
         const int qt0 = t * 32;
         int cls = 2;
         if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq] & 3;
-        if (wave_active && t >= wt_begin &&
-            !(DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5))) {
+        if (!(DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5))) {
             // S[query, key] in the base-2 domain: rows = the tile's queries 8(r/4) + 4*half + r%4, column = the lane's key
             f32x16 p = tile_product128(Qs + buf * TILE2_FLOATS + row_lds, kr);
             if (DENSE) {
@@ -380,7 +388,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const f32x4 o = {p[4 * g + 0], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]};
-                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 2);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 0);
                 }
             }
             tile_accumulate_t128(Qs + buf * TILE2_FLOATS + col_lds, p, ka);                      // dK^T += Q~^T . dS

@@ -166,6 +166,11 @@ __device__ __forceinline__ const unsigned char *dense_query_bounds(const MaskArg
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// s_waitcnt vmcnt(0): every vector memory operation the wavefront has issued is complete.  Placed in front of a loop it
+// also tells the compiler so: a load left pending on some path into the loop would otherwise make it wait, inside the
+// loop, for everything issued up to the first use of that load's result - the loop's own prefetches included.
+__device__ __forceinline__ void wait_vector_memory() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
 
 // Work item of this workgroup (see work_order.h).  Returns false for padding workgroups.

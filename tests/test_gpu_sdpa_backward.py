@@ -138,7 +138,7 @@ def test_zero_upstream_gradient_gives_zero_gradients(ctx):
 
 @pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 70), (1, 2, 257, 300), (2, 2, 96, 513), (1, 3, 40, 33)])
 @pytest.mark.parametrize("mask_kind", ["none", "dense", "lengths", "causal", "causal_lengths"])
-@pytest.mark.parametrize("d", [64, 128, 40, 96])
+@pytest.mark.parametrize("d", [64, 128, 40, 96, 32, 24, 16, 8])
 def test_stored_ds_route_agrees_with_the_self_contained_kernels(ctx, orc, B, H, Lq, Lk, mask_kind, d):
     """Large launches (here: forced by DL4S_SDPA_NO_KEY_SPLIT; head dims above 64 always) store dS from the dK/dV kernel and
     contract it in a second kernel; with the scratch bound at 0 the two self-contained kernels run instead.  Both within the gate of the oracle,
@@ -178,8 +178,9 @@ def test_stored_ds_route_agrees_with_the_self_contained_kernels(ctx, orc, B, H, 
             assert_parity(g, r, "%s, %s route" % (name, route))
     for a, b_ in zip(results["stored"], results["stored again"]):
         assert np.array_equal(a, b_)
-    assert np.array_equal(results["stored"][1], results["self-contained"][1])
-    assert np.array_equal(results["stored"][2], results["self-contained"][2])
+    if d > 32:      # narrow heads: the stored route has kernels of its own (16- and 32-column tiles), the other one pads to 64
+        assert np.array_equal(results["stored"][1], results["self-contained"][1])
+        assert np.array_equal(results["stored"][2], results["self-contained"][2])
 
 
 def test_config4_sized_gradients(ctx, orc):
