@@ -28,6 +28,7 @@
 
 #include "sdpa_common.h"
 #include "sdpa_prefill_d128.h"
+#include "sdpa_prefill_w96.h"
 #include "sdpa_prefill_narrow.h"
 
 namespace {
@@ -621,6 +622,12 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
     const int no_split = (flags & DL4S_SDPA_NO_KEY_SPLIT) ? 1 : 0;
+    // head dims above 64 up to 96 on launches that fill the GPU without a key split: the 96-wide kernel, which also takes
+    // even head dims that are not a multiple of 4 as they are (rows on the 8-byte grid)
+    const bool aligned8 = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+                            reinterpret_cast<uintptr_t>(out)) & 7) == 0;
+    const bool w96_path = dk == dv && dk > HD && dk <= W96 && ((Lq + BM - 1) / BM) * B * H >= 2ll * ctx->cu_count &&
+                          ((dk % 4 == 0 && aligned) || (dk % 2 == 0 && aligned8 && !token_major));
     // The 128-wide kernel on a launch that leaves CUs without their two workgroups: the key tiles of every block are dealt
     // to several workgroups, whose partial results a second kernel adds up (B4 H8 L512 d128: 73 us unsplit).  The count
     // depends on the extents only.
@@ -638,7 +645,7 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     MaskArgs m{};
     void *part128 = nullptr;
     {
-        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path, m, part_bytes, &part128);
+        const int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path || w96_path, m, part_bytes, &part128);
         if (rc != DL4S_HIP_OK) return rc;
     }
     DL4S_REQUIRE((flags & ~(uint32_t)(DL4S_SDPA_STRICT | DL4S_SDPA_TOKEN_MAJOR | DL4S_SDPA_NO_KEY_SPLIT)) == 0, DL4S_HIP_EINVALID_ARG,
@@ -655,6 +662,12 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
             case DL4S_MASK_KEY_LENGTHS: return launch_d64<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
             default: return launch_d64<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, no_split, stats, (int)dk);
         }
+    }
+    if (w96_path) {
+        DL4S_REQUIRE(Lk * (token_major ? H : 1) * dk * 4 < (1ll << 30), DL4S_HIP_EUNSUPPORTED,
+                     "sdpa: the K/V rows of one (batch, head) pair span more than 1 GiB");
+        if (dk % 4 == 0) return launch_w96<4>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+        return launch_w96<2>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
     }
     if (mfma128_path) {
         DL4S_REQUIRE(Lk * (token_major ? H : 1) * dk * 4 < (dk == HD2 ? (1ll << 31) : (1ll << 30)), DL4S_HIP_EUNSUPPORTED,

@@ -1,0 +1,244 @@
+// Fused attention forward for head dims above 64 and up to 96 on large launches: the scheme of sdpa_prefill_f32_d128
+// (sdpa_prefill_d128.h) on tiles that are 96 columns wide, and with a second staging form for head dims that are even
+// but not a multiple of 4 (rows on an 8-byte grid: 64-bit loads and stores), which the other MFMA kernels only take
+// through zero-padded copies of the operands.  Included by sdpa_prefill.hip only.
+//
+//   S^T[key, query] = K[key, :] . Q[query, :]        48 MFMA steps: step s contracts d = 48*half + s
+//   O^T[d,   query] = V[key, d]^T . P^T[key, query]   three accumulators: accumulator c row i is d = 32*c + i; V is read
+//                                                    a float at a time (consecutive lanes, consecutive columns), and
+//                                                    register r of accumulator c is d = 32c + 8(r/4) + 4*half + r%4:
+//                                                    four consecutive outputs per 128-bit (or two 64-bit) stores
+//
+// 96 MFMAs per 32 x 32 tile of (query, key) pairs against the 128-wide kernel's 128: a head dim of 96 costs three
+// quarters, and one of 70 runs without the four streaming copies.  One workgroup = 4 wavefronts = 128 queries of one
+// (batch, head) pair, K/V in double-buffered LDS tiles of 32 keys on a 100-float row stride (2 x 2 x 32 x 100 floats =
+// 50 KiB).  Mask kinds, tile skipping, the work order, the token-major layout (head dims that are multiples of 4) and
+// the row statistics are those of the other forward kernels.  No key split over workgroups: small launches stay with
+// the 128-wide kernel.
+#pragma once
+#include "sdpa_common.h"
+
+namespace {
+
+constexpr int W96 = 96;
+constexpr int LSTR96 = W96 + 4;            // 100 = 4 mod 32: the bank spread of the other tile widths
+constexpr int TILE96_FLOATS = BN * LSTR96;
+
+// VEC: floats per staging access, 4 (head dim a multiple of 4, tensors on the 16-byte grid) or 2 (head dim even, 8-byte grid)
+template <int KIND, int VEC>
+__global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__restrict__ q, const float *__restrict__ k,
+                                                                const float *__restrict__ v, float *__restrict__ out, int H, int Lq,
+                                                                int Lk, float rT, MaskArgs mask, int strict, int nqb, int total_blocks,
+                                                                int lpt, int token_major, float *__restrict__ stats, int hd) {
+    extern __shared__ __align__(16) float lds[];
+    float *Ks = lds;                       // [2][BN][LSTR96]
+    float *Vs = lds + 2 * TILE96_FLOATS;   // [2][BN][LSTR96]
+    int bh, unit;
+    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    const int b = bh / H, hh = bh % H;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, half = lane >> 5, ln = lane & 31;
+
+    constexpr bool CAUSAL = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool LENS = (KIND == DL4S_MASK_KEY_LENGTHS || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    constexpr bool DENSE = (KIND == DL4S_MASK_DENSE_F32);
+
+    const int qb = nqb - 1 - unit;   // longest rows first
+    const int q0 = qb * BM + wave * 32;
+    const int qi = q0 + ln;
+    const int qic = qi < Lq ? qi : Lq - 1;
+    int len = Lk;
+    if (LENS) len = mask.lengths[b];
+    const int rs = token_major ? H * hd : hd;
+    const long long q_base = token_major ? ((long long)b * Lq * H + hh) * hd : (long long)bh * Lq * hd;
+    const long long kv_base = token_major ? ((long long)b * Lk * H + hh) * hd : (long long)bh * Lk * hd;
+
+    // keys this workgroup / wavefront has to visit (see sdpa_prefill_f32_d64)
+    int kend = Lk, wkend = Lk;
+    bool skip_ones = false;
+    if (!strict && !(LENS && len <= 0)) {
+        if (CAUSAL) { kend = min(kend, qb * BM + BM); wkend = min(wkend, q0 + 32); }
+        if (LENS) { kend = min(kend, len); wkend = min(wkend, len); }
+        if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
+    }
+    const int ntiles = (kend + BN - 1) / BN;
+
+    // Q fragment: Q[qi][48*half + s] * rT (one rounding, like the reference's q / temperature) * log2(e); zeros beyond hd
+    float qr[W96 / 2];
+    {
+        const float *qp = q + q_base + (long long)qic * rs + half * (W96 / 2);
+#pragma unroll
+        for (int j = 0; j < W96 / 8; ++j) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            const int c0 = half * (W96 / 2) + 4 * j;
+            if (VEC == 4) {
+                if (c0 < hd) t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
+            } else {
+                if (c0 < hd) { const f32x2 a = *reinterpret_cast<const f32x2 *>(qp + 4 * j); t.x = a.x; t.y = a.y; }
+                if (c0 + 2 < hd) { const f32x2 a = *reinterpret_cast<const f32x2 *>(qp + 4 * j + 2); t.z = a.x; t.w = a.y; }
+            }
+            qr[4 * j + 0] = (t.x * rT) * LOG2E;
+            qr[4 * j + 1] = (t.y * rT) * LOG2E;
+            qr[4 * j + 2] = (t.z * rT) * LOG2E;
+            qr[4 * j + 3] = (t.w * rT) * LOG2E;
+        }
+    }
+
+    // global -> LDS staging: a tile is 32 rows of 96 / VEC pieces; thread tid moves the pieces tid, tid + 256, ...
+    // (3 of 128 bits or 6 of 64 bits for K and as many for V).  Buffer loads with the whole byte offset in the
+    // range-checked vector operand: rows past Lk and columns past hd read as zeros.
+    constexpr int PPR = W96 / VEC;            // pieces per tile row
+    constexpr int NP = BN * PPR / 256;        // pieces per thread
+    const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
+    const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
+    unsigned ld_off[NP];
+    int lds_off[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int p = tid + 256 * i, row = p / PPR, col = (p % PPR) * VEC;
+        ld_off[i] = col < hd ? (unsigned)(row * rs + col) * 4u : 0x80000000u;
+        lds_off[i] = row * LSTR96 + col;
+    }
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    using piece_t = typename std::conditional<VEC == 4, f32x4, f32x2>::type;
+    piece_t kst[NP], vst[NP];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int o = (int)(ld_off[i] + t * tile_bytes);
+            if constexpr (VEC == 4) {
+                kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o, 0, 0));
+                vst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o, 0, 0));
+            } else {
+                kst[i] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(krsrc, o, 0, 0));
+                vst[i] = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(vrsrc, o, 0, 0));
+            }
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            *reinterpret_cast<piece_t *>(Ks + buf * TILE96_FLOATS + lds_off[i]) = kst[i];
+            *reinterpret_cast<piece_t *>(Vs + buf * TILE96_FLOATS + lds_off[i]) = vst[i];
+        }
+    };
+
+    f32x16 o[3];
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[c][i] = 0.f;
+    float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
+
+    if (ntiles > 0) { load_tile(0); store_tile(0); }
+    __syncthreads();
+
+    const int k_lds = ln * LSTR96 + half * (W96 / 2);   // K fragment base: row ln, columns 48*half ..
+    const int v_lds = (4 * half) * LSTR96 + ln;          // V operand base: row 4*half (+ const), column ln (+ 32c)
+    const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
+    const unsigned char *cls_row = nullptr;
+    if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
+
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        const bool more = (t + 1 < ntiles);
+        if (more) load_tile(t + 1);
+        const int k0 = t * BN;
+        int cls = 2;
+        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
+            f32x16 s0 = masked_scores<KIND, W96 / 8>(Ks + buf * TILE96_FLOATS + k_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+            // online softmax with a lazily moved reference maximum (see attend_tile in sdpa_prefill.hip)
+            float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
+#pragma unroll
+            for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
+            tmax = fmaxf(tmax, s0[15]);
+            tmax = fmaxf(tmax, xor32(tmax));
+            const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+            if (__any(upd)) {
+                const float m_new = fmaxf(m_run, tmax);
+                const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
+                m_run = m_new;
+                m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int c = 0; c < 3; ++c)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o[c][i] *= alpha;
+            }
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                s0[r] = fast_exp2(s0[r] - m_use);
+                psum += s0[r];
+            }
+            l_run += psum;
+            const float *Vb = Vs + buf * TILE96_FLOATS + v_lds;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float *vr = Vb + (8 * (r >> 2) + (r & 3)) * LSTR96;
+                o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[0], s0[r], o[0], 0, 0, 0);
+                o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[32], s0[r], o[1], 0, 0, 0);
+                o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[64], s0[r], o[2], 0, 0, 0);
+            }
+        }
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and store
+    const float l_tot = l_run + xor32(l_run);
+    const float inv = 1.0f / l_tot;
+    if (stats && half == 0 && qi < Lq) {
+        stats[2 * ((long long)bh * Lq + qi)] = m_use;
+        stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
+    }
+    if (qi < Lq) {
+        float *op = out + q_base + (long long)qi * rs;
+#pragma unroll
+        for (int c = 0; c < 3; ++c)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d0 = 32 * c + 8 * g + 4 * half;
+                const f32x4 a = {o[c][4 * g + 0] * inv, o[c][4 * g + 1] * inv, o[c][4 * g + 2] * inv, o[c][4 * g + 3] * inv};
+                if (VEC == 4) {
+                    if (d0 < hd) *reinterpret_cast<f32x4 *>(op + d0) = a;
+                } else {
+                    const f32x2 lo = {a.x, a.y}, hi = {a.z, a.w};
+                    if (d0 < hd) *reinterpret_cast<f32x2 *>(op + d0) = lo;
+                    if (d0 + 2 < hd) *reinterpret_cast<f32x2 *>(op + d0 + 2) = hi;
+                }
+            }
+    }
+}
+
+template <int KIND, int VEC>
+int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
+                    float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+    const int nqb = (Lq + BM - 1) / BM;
+    const long long total = (long long)nqb * B * H;
+    DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
+    constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
+    if (lpt && total <= 3ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+    const size_t lds_bytes = 4 * TILE96_FLOATS * sizeof(float);   // 50 KiB: within the default limit
+    hipLaunchKernelGGL((sdpa_prefill_f32_w96<KIND, VEC>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_bytes, ctx->stream, q, k,
+                       v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd);
+    return dl4s::launch_status("sdpa_prefill_f32_w96");
+}
+
+template <int VEC>
+int launch_w96(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk, float rT,
+               const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+    switch (m.kind) {
+        case DL4S_MASK_NONE: return launch_w96_kind<DL4S_MASK_NONE, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_DENSE_F32: return launch_w96_kind<DL4S_MASK_DENSE_F32, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_CAUSAL: return launch_w96_kind<DL4S_MASK_CAUSAL, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_KEY_LENGTHS: return launch_w96_kind<DL4S_MASK_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        default: return launch_w96_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+    }
+}
+
+}  // namespace

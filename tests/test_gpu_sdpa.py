@@ -567,6 +567,45 @@ def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk, d):
         assert np.array_equal(a, b), kw.keys()
 
 
+@pytest.mark.parametrize("d", [96, 80, 68, 70, 66, 94])
+@pytest.mark.parametrize("mk", ["none", "dense", "causal", "lens", "causal_lens"])
+def test_head_dims_up_to_96_on_launches_that_fill_the_gpu(ctx, orc, d, mk):
+    """Head dims above 64 up to 96 with at least two 128-query blocks per CU run the 96-wide kernel: multiples of 4 with
+    128-bit staging, other even head dims as they are with 64-bit staging (no padded copies).  B16 H16, ragged
+    extents, checked against the oracle on whole (batch, head) slices."""
+    from dl4s_amd import lib
+    B, H, Lq, Lk = 16, 16, 300, 300
+    rng = np.random.default_rng(zlib.crc32(repr(("w96", d, mk)).encode()))
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    lens = rng.integers(0, Lk + 1, size=B)
+    lens[0], lens[1] = Lk // 2, 0        # batch item 1: no valid key, uniform rows
+    kind, mask, lens_arg = None, None, None
+    if mk == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.4).astype(np.float32)
+        mask[:, :, 64:160, 96:224] = 1.0          # whole tiles of ones and of zeros
+        mask[:, :, 160:224, 0:96] = 0.0
+    elif mk == "causal":
+        kind, mask = lib.MASK_CAUSAL, causal_mask(Lq, Lk)
+    elif mk == "lens":
+        kind, mask, lens_arg = lib.MASK_KEY_LENGTHS, lengths_mask(lens, Lk), lens
+    elif mk == "causal_lens":
+        kind, lens_arg = lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lk)[None, None])
+    got = run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg)
+    for (b, h) in [(0, 0), (1, 5), (15, 15)]:
+        mb = None if mask is None else (mask if mask.ndim == 2 else mask[b:b + 1])
+        ref = orc.sdpa(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mb)
+        assert_parity(got[b:b + 1, h:h + 1], ref, "96-wide d=%d %s (b=%d,h=%d)" % (d, mk, b, h))
+    if kind is not None:    # descriptor == the dense mask it stands for, bit for bit, when both visit every tile
+        dense = run_sdpa(ctx, q, k, v, mask, strict=True)
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=True), dense)
+        assert_parity(got, dense, "skip vs dense")
+    if mask is not None:
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask), run_sdpa(ctx, q, k, v, mask, strict=True))
+    if d % 4 == 0:
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, token_major=True), got)
+
+
 def test_token_major_rejected_for_other_head_dims_and_unknown_flags(ctx):
     from dl4s_amd import lib
     q = ctx.empty((1, 2, 4, 256))

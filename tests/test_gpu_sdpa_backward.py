@@ -271,6 +271,34 @@ def test_gradients_on_padded_copies(ctx, orc, d, mask_kind):
     assert np.isfinite(dq).all() and np.isfinite(dk).all() and np.isfinite(dv).all()
 
 
+@pytest.mark.parametrize("d", [70, 80])
+@pytest.mark.parametrize("mask_kind", ["none", "lengths", "causal"])
+def test_gradients_after_the_96_wide_forward_kernel(ctx, orc, d, mask_kind):
+    """A launch that fills the GPU with a head dim up to 96: the forward pass with statistics runs the 96-wide kernel
+    (d = 70 as it is, no padded copies), the gradients the 128-wide kernels (d = 70 on padded copies); the statistics
+    have one form on every MFMA kernel."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(960 + d)
+    B, H, L = 16, 16, 260
+    q, k, v, dout = rand(rng, B, H, L, d), rand(rng, B, H, L, d), rand(rng, B, H, L, d), rand(rng, B, H, L, d)
+    lens = rng.integers(1, L + 1, size=B)
+    mask, kind = None, None
+    if mask_kind == "lengths":
+        mask, kind = lengths_mask(lens, L), lib.MASK_KEY_LENGTHS
+    elif mask_kind == "causal":
+        mask, kind = causal_mask(L, L), lib.MASK_CAUSAL
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, kind=kind, lens=lens)
+    for b in (0, 15):
+        sl = (slice(b, b + 1), slice(3, 5))
+        msample = mask if mask is None or mask.ndim == 2 else mask[b:b + 1]
+        assert_parity(out[sl], orc.sdpa(q[sl], k[sl], v[sl], msample), "forward d=%d" % d)
+        rq, rk, rv = orc.sdpa_backward(q[sl], k[sl], v[sl], msample, dout[sl])
+        assert_parity(dq[sl], rq, "dq d=%d" % d)
+        assert_parity(dk[sl], rk, "dk d=%d" % d)
+        assert_parity(dv[sl], rv, "dv d=%d" % d)
+    assert np.isfinite(dq).all() and np.isfinite(dk).all() and np.isfinite(dv).all()
+
+
 def test_backward_argument_errors(ctx):
     from dl4s_amd import lib
     a = ctx.empty((1, 1, 4, 300))
