@@ -64,6 +64,10 @@ int set_error(int code, const char *fmt, ...);
 int hip_error(hipError_t e, const char *what);
 // Grows ctx->scratch to at least `bytes`; returns 0 or a status.
 int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes);
+// The normalising pass of the LayerNorm kernels on partial sums some other kernel left (nblk <= 256 pairs per item, laid
+// out [item][nblk][2]); x and y may be the same tensor.  The caller holds the scratch mutex when `part` lies there.
+int layernorm_apply(dl4s_hip_ctx *ctx, const float *x, const float *scale, const float *shift, float *y, const float *part,
+                    long long items, long long n, long long D, int nblk);
 // Looks up the device address of the decode kernels' fixed scratch block (sdpa_decode.hip) for the current GPU.
 int decode_static_scratch_init(dl4s_hip_ctx *ctx);
 

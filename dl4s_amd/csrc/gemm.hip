@@ -37,6 +37,12 @@ struct GemmArgs {
     // epilogue of the fused Dense forms: C = act(alpha * A.B + bias[n]) + residual[m][n]
     const float *bias, *residual;
     int act;   // 0 none, 1 gaussianErrorLinear
+    // LayerNorm statistics from the epilogue (the fused Dense forms on the tiled kernels): when ln_part is set, every
+    // workgroup also leaves the sum and the sum of squares of the values it stored.  The rows of one normalised item
+    // span ln_tiles_m row tiles; item i's pairs are ln_part[(i * ln_tiles_m * tiles_n + (tile_m % ln_tiles_m) * tiles_n +
+    // tile_n) * 2 ..], the layout ln_apply_f32 sums in a fixed order.
+    float *ln_part;
+    int ln_tiles_m;
 };
 
 // x * (0.5 * tanh(0.5 * (1.702 * x)) + 0.5), every operation rounded, as Tensor/Operators/Unary.swift:184-186, :245-247
@@ -310,6 +316,7 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
     }
 
     // accumulator register r of a transposed 32x32 tile: row m = lane % 32, column n = 8*(r/4) + 4*half + r%4
+    float ln_s = 0.f, ln_ss = 0.f;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
         const int gm = m0 + wm * 32 * MI + i * 32 + ln;
@@ -344,9 +351,30 @@ __global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
                         val.x = __fadd_rn(val.x, rq.x); val.y = __fadd_rn(val.y, rq.y);
                         val.z = __fadd_rn(val.z, rq.z); val.w = __fadd_rn(val.w, rq.w);
                     }
+                    if (g.ln_part) {
+                        ln_s += (val.x + val.y) + (val.z + val.w);
+                        ln_ss += (__fmul_rn(val.x, val.x) + __fmul_rn(val.y, val.y)) + (__fmul_rn(val.z, val.z) + __fmul_rn(val.w, val.w));
+                    }
                 }
                 *reinterpret_cast<f32x4 *>(cp) = val;
             }
+    }
+    if (EPI) {
+        if (g.ln_part) {   // the workgroup's pair: lanes of a wavefront by butterfly, the four wavefronts in order
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                ln_s += __shfl_xor(ln_s, off, 64);
+                ln_ss += __shfl_xor(ln_ss, off, 64);
+            }
+            if (lane == 0) { As[2 * wave] = ln_s; As[2 * wave + 1] = ln_ss; }   // the K loop ended on a barrier: As is free
+            __syncthreads();
+            if (tid == 0) {
+                const int item = tile_m / g.ln_tiles_m;
+                const long long at = ((long long)item * g.ln_tiles_m + tile_m % g.ln_tiles_m) * g.tiles_n + tile_n;
+                g.ln_part[2 * at] = ((As[0] + As[2]) + As[4]) + As[6];
+                g.ln_part[2 * at + 1] = ((As[1] + As[3]) + As[5]) + As[7];
+            }
+        }
     }
 }
 
@@ -576,11 +604,18 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_finish(GemmArgs g, const 
     *cp = val;
 }
 
+constexpr int GEMM_LN_NOT_FUSED = 1;   // gemm_launch with ln_part: nothing was launched, the caller takes the two-call route
+constexpr int LN_MAX_PAIRS = 256;      // partial pairs per item that dl4s::layernorm_apply sums (one per thread)
+
 int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int64_t lbs, const float *rhs, int64_t rr,
                 int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb,
                 const float *bias = nullptr, const float *residual = nullptr, int act = 0, const float *const *group_lhs = nullptr,
-                const float *const *group_rhs = nullptr, float *const *group_result = nullptr) {
+                const float *const *group_rhs = nullptr, float *const *group_result = nullptr, float *ln_part = nullptr,
+                int64_t ln_item_rows = 0, int *ln_nblk = nullptr) {
     // group_*: `batch` (at most 4) products of one shape with unrelated operand addresses, in one launch
+    // ln_part: also leave LayerNorm partial sums over items of ln_item_rows rows (see GemmArgs); *ln_nblk receives the
+    // number of pairs per item.  A product that does not run on the tiled kernels with whole tiles per item, or would
+    // leave more pairs than ln_apply_f32 sums, is not launched at all: GEMM_LN_NOT_FUSED.
     DL4S_REQUIRE(lr >= 0 && lc >= 0 && rr >= 0 && rc >= 0 && batch >= 0, DL4S_HIP_EINVALID_ARG, "gemm: negative extent");
     const int64_t M = ta ? lc : lr, K = ta ? lr : lc;
     const int64_t K2 = tb ? rc : rr, N = tb ? rr : rc;
@@ -630,6 +665,7 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     const bool skinny = !ta && K >= 64 && (few_rows || few_blocks) && rows_by_k_any(lc) &&
                         (tb ? rows_by_k_any(rc) : true) && aligned16(lhs) && (!tb || aligned16(rhs)) && lbs % 4 == 0 &&
                         (!tb || rbs % 4 == 0) && group_aligned && M * N * batch < (1ll << 31) && K * (tb ? 1 : rc) < (1ll << 31);
+    if (ln_part && (skinny || !fast)) return GEMM_LN_NOT_FUSED;
     if (skinny) {
         // 16 x 16 output blocks (gemm_f32_skinny16) for up to 16 rows, and beyond for an unsliced K while that grid stays
         // within two workgroups per CU ([32,512].[512,512] 5.7 -> 3.7 us, [128,512].[512,512] 5.8 -> 4.0 us,
@@ -677,6 +713,14 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;
     if (small) { tm = (M + 63) / 64; tn = (N + 63) / 64; }
     g.tiles_n = (int)tn;
+    if (ln_part) {
+        const int64_t TM = small ? 64 : GBM;
+        if (ln_item_rows <= 0 || ln_item_rows % TM != 0 || M % ln_item_rows != 0 || batch != 1 || (ln_item_rows / TM) * tn > LN_MAX_PAIRS)
+            return GEMM_LN_NOT_FUSED;
+        g.ln_part = ln_part;
+        g.ln_tiles_m = (int)(ln_item_rows / TM);
+        *ln_nblk = (int)((ln_item_rows / TM) * tn);
+    }
     DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
     const dim3 grid((unsigned)(tm * tn), 1, (unsigned)batch);
 #define DL4S_GEMM_FAST(MI_, EPI_, TA_, TB_) hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, (MI_ == 1 ? 32 : 16)>), grid, dim3(256), 0, ctx->stream, g)
@@ -742,6 +786,37 @@ int dl4s_hip_dense_fused_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, in
                  "dense: unknown activation %d", activation);
     return gemm_launch(ctx, x, rows, in_features, 0, weights, in_features, out_features, 0, result, 0, 1, 1.0f, 0.0f, 0, 0, bias,
                        residual, activation);
+}
+
+// LayerNorm(act(x . weights + bias) + residual) over items of item_rows rows (NN/Layer/LayerNorm.swift:62-77 applied to
+// the sum MultiHeadAttention.swift:120-124 forms): the product's epilogue leaves the per-tile sums, so the
+// normalisation is one more pass instead of two.
+int dl4s_hip_dense_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t in_features, const float *weights,
+                                 int64_t out_features, const float *bias, int activation, const float *residual,
+                                 int64_t item_rows, const float *scale, const float *shift, float *result) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(activation == DL4S_ACT_NONE || activation == DL4S_ACT_GELU, DL4S_HIP_EINVALID_ARG,
+                 "dense: unknown activation %d", activation);
+    DL4S_REQUIRE(rows >= 0 && item_rows > 0 && rows % item_rows == 0, DL4S_HIP_ESHAPE,
+                 "dense + layernorm: %lld rows are not whole items of %lld rows", (long long)rows, (long long)item_rows);
+    DL4S_REQUIRE(scale && shift, DL4S_HIP_EINVALID_ARG, "dense + layernorm: NULL pointer");
+    const int64_t items = rows / item_rows;
+    const auto a16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (rows * out_features > 0 && items <= 65535 && out_features % 4 == 0 && a16(scale) && a16(shift) && a16(result)) {
+        std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
+        int rc = dl4s::ensure_scratch(ctx, (size_t)items * LN_MAX_PAIRS * 2 * sizeof(float));
+        if (rc != DL4S_HIP_OK) return rc;
+        int nblk = 0;
+        float *part = static_cast<float *>(ctx->scratch);
+        rc = gemm_launch(ctx, x, rows, in_features, 0, weights, in_features, out_features, 0, result, 0, 1, 1.0f, 0.0f, 0, 0, bias, residual,
+                         activation, nullptr, nullptr, nullptr, part, item_rows, &nblk);
+        if (rc == DL4S_HIP_OK) return dl4s::layernorm_apply(ctx, result, scale, shift, result, part, items, item_rows * out_features, out_features, nblk);
+        if (rc != GEMM_LN_NOT_FUSED) return rc;
+    }
+    const int rc = gemm_launch(ctx, x, rows, in_features, 0, weights, in_features, out_features, 0, result, 0, 1, 1.0f, 0.0f, 0, 0, bias,
+                               residual, activation);
+    if (rc != DL4S_HIP_OK) return rc;
+    return dl4s_hip_layernorm_f32(ctx, result, nullptr, scale, shift, result, items, item_rows, out_features);
 }
 
 }  // extern "C"

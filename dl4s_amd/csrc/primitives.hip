@@ -624,6 +624,19 @@ int launch_slice_copy(dl4s_hip_ctx *ctx, const float *src, float *dst, const Sli
 }
 }  // namespace
 
+namespace dl4s {
+int layernorm_apply(dl4s_hip_ctx *ctx, const float *x, const float *scale, const float *shift, float *y, const float *part,
+                    long long items, long long n, long long D, int nblk) {
+    DL4S_REQUIRE(nblk >= 1 && nblk <= TPB && items >= 1 && items <= 65535 && n % 4 == 0 && D % 4 == 0, DL4S_HIP_EINVALID_ARG,
+                 "layernorm: bad partial-sum layout");
+    const long long want = n / (TPB * 8);
+    const unsigned gx = (unsigned)(want < 1 ? 1 : (want > 256 ? 256 : want));
+    hipLaunchKernelGGL(ln_apply_f32<true>, dim3(gx, (unsigned)items), dim3(TPB), 0, ctx->stream, x, static_cast<const float *>(nullptr), scale,
+                       shift, y, part, n, D, nblk);
+    return launch_status("layernorm");
+}
+}  // namespace dl4s
+
 extern "C" {
 
 int dl4s_hip_fill_f32(dl4s_hip_ctx *ctx, float value, float *result, int64_t count) {

@@ -269,6 +269,16 @@ struct HIP {
                                            weights.values.memory, weights.shape[1], bias ? bias->values.memory : nullptr, activation,
                                            residual ? residual->values.memory : nullptr, result.values.memory));
         }
+        // result = LayerNorm(act(x . weights + bias) + residual), statistics over items of itemRows rows
+        static void denseFusedLayerNorm(const ShapedBuffer &x, const ShapedBuffer &weights, const ShapedBuffer *bias, int activation,
+                                        const ShapedBuffer *residual, int64_t itemRows, const ShapedBuffer &scale, const ShapedBuffer &shift,
+                                        const ShapedBuffer &result) {
+            precondition(x.count() % weights.shape[0] == 0, "Matmul operands must have matching shapes");
+            check(dl4s_hip_dense_layernorm_f32(context(), x.values.memory, x.count() / weights.shape[0], weights.shape[0],
+                                               weights.values.memory, weights.shape[1], bias ? bias->values.memory : nullptr, activation,
+                                               residual ? residual->values.memory : nullptr, itemRows, scale.values.memory,
+                                               shift.values.memory, result.values.memory));
+        }
         static void gemmBatched(const ShapedBuffer &lhs, int64_t lstride, const ShapedBuffer &rhs, int64_t rstride,
                                 const ShapedBuffer &result, int64_t batch, bool tA, bool tB) {
             const int ld = lhs.dim(), rd = rhs.dim(), od = result.dim();
@@ -935,10 +945,13 @@ struct MultiHeadAttention {
             Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true);
         Tensor a2 = a.view({batchSize * queryCount, heads * valueDim});
         if (!dropout.isActive) {
+            // the fc product, `+ res` and the normalisation (MultiHeadAttention.swift:119-124) as one call: the product's
+            // epilogue leaves the sums the LayerNorm needs
             Tensor sum(Device::Memory::allocateBuffer(Shape{batchSize, queryCount, hiddenDim}));
             const ShapedBuffer rb = q.values();
-            Device::Engine::denseFused(a2.values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, sum.values());
-            return normalized(sum, nullptr);
+            Device::Engine::denseFusedLayerNorm(a2.values(), fc.values(), nullptr, DL4S_ACT_NONE, &rb, normalizesPerToken ? 1 : queryCount,
+                                                norm.scale.values(), norm.shift.values(), sum.values());
+            return sum;
         }
         Tensor out_drop = dropout(a2.matrixMultiplied(fc).view({batchSize, queryCount, hiddenDim}));
         return normalized(out_drop, &q);

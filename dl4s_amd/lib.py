@@ -348,6 +348,12 @@ class Context:
                                                  _i64(out_features), _vp(_ptr(bias)) if bias is not None else None, int(activation),
                                                  _vp(_ptr(residual)) if residual is not None else None, _vp(_ptr(y))))
 
+    def dense_layernorm(self, x, rows, in_features, weights, out_features, bias, activation, residual, item_rows, scale, shift, y):
+        _check(self.lib.dl4s_hip_dense_layernorm_f32(self.handle, _vp(_ptr(x)), _i64(rows), _i64(in_features), _vp(_ptr(weights)),
+                                                     _i64(out_features), _vp(_ptr(bias)) if bias is not None else None, int(activation),
+                                                     _vp(_ptr(residual)) if residual is not None else None, _i64(item_rows),
+                                                     _vp(_ptr(scale)), _vp(_ptr(shift)), _vp(_ptr(y))))
+
     def bias_gelu(self, x, bias, y, rows, D):
         _check(self.lib.dl4s_hip_bias_gelu_f32(self.handle, _vp(_ptr(x)), _vp(_ptr(bias)) if bias is not None else None,
                                                _vp(_ptr(y)), _i64(rows), _i64(D)))

@@ -356,6 +356,18 @@ int dl4s_hip_log_softmax_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, in
 #define DL4S_ACT_GELU 1
 int dl4s_hip_dense_fused_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t in_features, const float *weights,
                              int64_t out_features, const float *bias, int activation, const float *residual, float *result);
+/* The tail of MultiHeadAttention in one call (NN/Models/Transformer/MultiHeadAttention.swift:119-124: the fc product,
+ * `+ res`, then norm):
+ *   result = LayerNorm(act(x . weights + bias) + residual)
+ * with the normalisation of dl4s_hip_layernorm_f32 (NN/Layer/LayerNorm.swift:62-77) over items of item_rows rows
+ * (rows % item_rows == 0; item_rows = the sequence length for the reference's joint (L, D) statistics, 1 for per-row
+ * ones); scale, shift [out].  When the product runs on the tiled kernels with whole tiles per item, the product's
+ * epilogue leaves per-tile sums and sums of squares and one more pass normalises; otherwise the call is
+ * dl4s_hip_dense_fused_f32 followed by dl4s_hip_layernorm_f32.  The two routes add the statistics up in different
+ * orders and agree to rounding; every element's arithmetic is the same.  result may alias residual. */
+int dl4s_hip_dense_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, int64_t rows, int64_t in_features, const float *weights,
+                                 int64_t out_features, const float *bias, int activation, const float *residual,
+                                 int64_t item_rows, const float *scale, const float *shift, float *result);
 
 #ifdef __cplusplus
 }

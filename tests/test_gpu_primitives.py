@@ -1,5 +1,7 @@
 """Parity of the engine primitives (C ABI) against the CPU oracle: element-wise results bit-exact where the
 arithmetic is a single IEEE operation, 1e-4 tolerance where summation order or libm differ."""
+import zlib
+
 import numpy as np
 import pytest
 
@@ -489,6 +491,53 @@ def test_dense_fused_equals_separate_engine_calls(ctx, orc, M, K, N, act, with_b
         ctx.dense_fused(dx, M, K, dW, N, db if with_bias else None, act, dr, dr)
         assert np.array_equal(dr.numpy(), fused.numpy())
     for t in (dx, dW, db, dr, fused, sep):
+        t.release()
+
+
+@pytest.mark.parametrize("items,item_rows,K,N", [
+    (4, 512, 512, 512),      # 64 x 64 tiles, 64 pairs per item: the tail of a config-2 attention layer
+    (8, 1024, 64, 1024),     # 128 x 128 tiles, 64 pairs per item
+    (2, 128, 64, 2048),      # 32 pairs per item
+    (3, 64, 128, 260),       # a last column tile that is partly outside
+    (2, 100, 128, 256),      # items that are not whole tiles: two calls
+    (600, 1, 128, 128),      # per-row statistics: two calls
+    (2, 30, 512, 512),       # a skinny product: two calls
+    (1, 8192, 64, 512),      # more pairs than the normalising pass sums: two calls
+])
+@pytest.mark.parametrize("with_bias,act,with_res", [(False, 0, True), (True, 1, False), (True, 0, True)])
+def test_dense_layernorm_in_one_call(ctx, orc, items, item_rows, K, N, with_bias, act, with_res):
+    """LayerNorm(act(x.W + b) + r) with the statistics taken from the product's epilogue: within the gate of the oracle's
+    Dense / gaussianErrorLinear / residual / LayerNorm sequence, and within rounding of the two separate calls (same
+    arithmetic per element, the sums added in another order)."""
+    rng = np.random.default_rng(zlib.crc32(repr(("dln", items, item_rows, K, N, with_bias, act, with_res)).encode()))
+    M = items * item_rows
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = (rng.standard_normal((K, N)) * 0.2).astype(np.float32)
+    b, r = rng.standard_normal(N).astype(np.float32), rng.standard_normal((M, N)).astype(np.float32)
+    scale, shift = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32), (0.1 * rng.standard_normal(N)).astype(np.float32)
+    dx, dW, db, dr, dsc, dsh = (ctx.to_device(a) for a in (x, W, b, r, scale, shift))
+    one, two = ctx.empty((M, N)), ctx.empty((M, N))
+    ctx.dense_layernorm(dx, M, K, dW, N, db if with_bias else None, act, dr if with_res else None, item_rows, dsc, dsh, one)
+    ctx.dense_fused(dx, M, K, dW, N, db if with_bias else None, act, dr if with_res else None, two)
+    ctx.layernorm(two, None, dsc, dsh, two, items, item_rows, N)
+    got, sep = one.numpy(), two.numpy()
+    assert np.allclose(got, sep, rtol=2e-5, atol=2e-5)
+    sample = list(range(items)) if M * N * K <= (1 << 26) else [0, items - 1]
+    for i in sample:
+        rows = slice(i * item_rows, (i + 1) * item_rows)
+        ref = orc.gemm(x[rows], W, False, False)
+        if with_bias:
+            ref = ref + b
+        if act:
+            ref = orc.gelu(ref)
+        if with_res:
+            ref = ref + r[rows]
+        ref = orc.layernorm(ref.reshape(1, item_rows, N), scale, shift).reshape(item_rows, N)
+        assert_parity(got[rows], ref, "dense + layernorm item %d" % i)
+    if with_res:    # the result may alias the residual
+        ctx.dense_layernorm(dx, M, K, dW, N, db if with_bias else None, act, dr, item_rows, dsc, dsh, dr)
+        assert np.array_equal(dr.numpy(), got)
+    for t in (dx, dW, db, dr, dsc, dsh, one, two):
         t.release()
 
 
