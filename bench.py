@@ -68,8 +68,9 @@ def prefill(ctx, lib, steps, warmup):
             "shape": {"B": B, "H": H, "L": L, "d": d}, "inputs": (q, k, v), "output": o}
 
 
-def decode(ctx, lib, repeats):
-    B, H, d, T0, steps = 16, 16, 64, 4096, 64
+def decode(ctx, lib, repeats, d=64):
+    B, H, T0, steps = 16, 16, 4096, 64
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
     Tcap = T0 + steps
     rng = np.random.Generator(np.random.PCG64(1005))
     kc = ctx.to_device(rng.standard_normal((B, H, Tcap, d), dtype=np.float32))
@@ -83,7 +84,7 @@ def decode(ctx, lib, repeats):
     def run():
         for t in range(steps):
             ctx.sdpa_decode_step(qs.offset(t * sb), kc, vc, kn.offset(t * sb), vn.offset(t * sb), out.offset(t * sb),
-                                 B, H, T0 + t, Tcap, d, 0.125)
+                                 B, H, T0 + t, Tcap, d, rT)
     t_end = time.perf_counter() + PREHEAT_S
     while time.perf_counter() < t_end:      # clocks back up after the idle time spent filling the cache
         run()
@@ -98,7 +99,7 @@ def decode(ctx, lib, repeats):
     for t in range(steps):
         ctx.timer_begin()
         ctx.sdpa_decode_step(qs.offset(t * sb), kc, vc, kn.offset(t * sb), vn.offset(t * sb), out.offset(t * sb),
-                             B, H, T0 + t, Tcap, d, 0.125)
+                             B, H, T0 + t, Tcap, d, rT)
         single_us.append(ctx.timer_end() * 1e3)
     o = out.numpy()
     if not np.isfinite(o).all():
@@ -185,7 +186,7 @@ def other_configs(ctx, lib, cpu, only=None):
         i, j = np.indices((L, L))
         mask = (j > i).astype(np.float32)
         fl = 4.0 * 64 * B * H * (L * (L + 1) // 2) + 4 * 2.0 * B * L * D * D
-        # config 2's fused layer (projections in one launch, attention, output product + residual, layer norm) on
+        # config 2's fused layer (projections in one launch, attention, output product + residual + layer norm) on
         # fixed buffers through the C ABI: issued one by one, and recorded once into a graph and replayed
         r = lambda *sh: ctx.to_device(rng.standard_normal(sh, dtype=np.float32) * np.float32(0.05))
         dx, dmask, w4 = ctx.to_device(x.reshape(B * L, D)), ctx.to_device(mask), [r(D, D) for _ in range(4)]
@@ -196,8 +197,7 @@ def other_configs(ctx, lib, cpu, only=None):
         def layer_calls():
             ctx.gemm_grouped([dx, dx, dx], (B * L, D), w4[:3], (D, D), t[:3])
             ctx.sdpa_fwd(t[0], t[1], t[2], t[3], B, H, L, L, dk_, dk_, 0.125, mask=md, flags=lib.SDPA_TOKEN_MAJOR)
-            ctx.dense_fused(t[3], B * L, D, w4[3], D, None, lib.ACT_NONE, dx, t[4])
-            ctx.layernorm(t[4], None, dscale, dshift, t[5], B, L, D)
+            ctx.dense_layernorm(t[3], B * L, D, w4[3], D, None, lib.ACT_NONE, dx, L, dscale, dshift, t[5])
 
         def timed(fn, n):
             for _ in range(n * 10):
@@ -268,48 +268,55 @@ def other_configs(ctx, lib, cpu, only=None):
                 "tflops": fl1 / dt / 1e12, "cores": 1, "kind": "port",
                 "sample": "one batch item cut to 256 tokens (%.1f s); extrapolated whole call %.0f s" % (dt, dt * fl / fl1)}
     if want("backward"):
-        # gradients of the headline workload (config 4 shapes): forward with row statistics, then dq, dk, dv
+        # gradients of the headline workload (config 4 shapes): forward with row statistics, then dq, dk, dv; head dim 64
+        # (the 64-wide kernels), 128 and 32 (the 128- and 32-wide ones)
         B, H, L = 8, 16, 2048
         rng = np.random.Generator(np.random.PCG64(1004))
-        bufs = [ctx.to_device(rng.standard_normal((B, H, L, 64), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
-        outs = [ctx.empty((B, H, L, 64)) for _ in range(4)]
-        st = ctx.empty((B, H, L, 2))
-        desc = ctx.mask_desc(lib.MASK_CAUSAL)
-        ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], outs[0], st, B, H, L, L, 64, 0.125, desc, 0)
-        bwd = lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, 64, 0.125, desc, 0)
-        for _ in range(20):
-            bwd()
-        ctx.sync()
-        ctx.timer_begin()
-        for _ in range(20):
-            bwd()
-        ms = ctx.timer_end() / 20
-        fl = 10.0 * 64 * B * H * (L * (L + 1) // 2)          # five products: dv, dp, dq, dk and the recomputed scores
-        res["config4_attention_backward_B8_H16_L2048_causal"] = {
-            "us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
-            "note": "algorithmic flops = 5 products; the two deterministic kernels issue 7 (scores and dp are formed in both)"}
-        if cpu:
-            from oracle import binding as orc
-            hq, hk, hv, hg = (b_.numpy()[:1, :2] for b_ in bufs)
-            i, j = np.indices((L, L))
-            t0 = time.perf_counter()
-            orc.sdpa_backward(hq, hk, hv, (j > i).astype(np.float32), hg)
-            dt = time.perf_counter() - t0
-            res["config4_attention_backward_B8_H16_L2048_causal"]["cpu_baseline"] = {
-                "tflops": fl * 2 / (B * H) / dt / 1e12, "cores": 1, "kind": "port",
-                "sample": "2 of 128 (batch, head) slices, dense causal mask (%.1f s)" % dt}
-        for b_ in bufs + outs + [st]:
-            b_.release()
+        for d in (64, 128, 32):
+            bufs = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
+            outs = [ctx.empty((B, H, L, d)) for _ in range(4)]
+            st = ctx.empty((B, H, L, 2))
+            desc = ctx.mask_desc(lib.MASK_CAUSAL)
+            rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+            ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], outs[0], st, B, H, L, L, d, rT, desc, 0)
+            bwd = lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, d, rT, desc, 0)
+            for _ in range(20):
+                bwd()
+            ctx.sync()
+            ctx.timer_begin()
+            for _ in range(20):
+                bwd()
+            ms = ctx.timer_end() / 20
+            fl = 10.0 * d * B * H * (L * (L + 1) // 2)          # five products: the recomputed scores, dp, dv, dk, dq
+            name = "config4_attention_backward_B8_H16_L2048_causal" + ("" if d == 64 else "_head_dim_%d" % d)
+            res[name] = {
+                "us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
+                "note": "algorithmic flops = the 5 products, which is what the two deterministic kernels issue: the dK/dV kernel "
+                        "stores its dS tiles (2 GiB scratch from the pool at this shape) and the dQ kernel contracts them with K"}
+            if cpu and d == 64:
+                from oracle import binding as orc
+                hq, hk, hv, hg = (b_.numpy()[:1, :2] for b_ in bufs)
+                i, j = np.indices((L, L))
+                t0 = time.perf_counter()
+                orc.sdpa_backward(hq, hk, hv, (j > i).astype(np.float32), hg)
+                dt = time.perf_counter() - t0
+                res[name]["cpu_baseline"] = {
+                    "tflops": fl * 2 / (B * H) / dt / 1e12, "cores": 1, "kind": "port",
+                    "sample": "2 of 128 (batch, head) slices, dense causal mask (%.1f s)" % dt}
+            for b_ in bufs + outs + [st]:
+                b_.release()
     if want("masks_and_head_dim"):
         # the headline shape with the mask as an unmodified DL4S passes it (a dense [L,L] tensor): all-ones tiles skipped
-        # (default) and every tile visited (DL4S_SDPA_STRICT); the same shape with head dim 128 (causal descriptor); and with
-        # head dim 70, which the MFMA kernels take through zero-padded copies of the operands
+        # (default) and every tile visited (DL4S_SDPA_STRICT); the same shape with the causal descriptor at other head dims:
+        # 128 (128-wide tiles), 96 and 70 (96-wide tiles; 70 is staged with 64-bit accesses, no padded copies), 32 and 16
+        # (32- and 16-wide tiles).  TFLOP/s on each shape's own flops.
         B, H, L = 8, 16, 2048
         rng = np.random.Generator(np.random.PCG64(1008))
         i, j = np.indices((L, L))
         dmask = ctx.to_device((j > i).astype(np.float32))
         for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal"),
-                        (70, "config4_shape_head_dim_70_causal_on_padded_copies")):
+                        (96, "config4_shape_head_dim_96_causal"), (70, "config4_shape_head_dim_70_causal"),
+                        (32, "config4_shape_head_dim_32_causal"), (16, "config4_shape_head_dim_16_causal")):
             qkv = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(3)]
             o = ctx.empty((B, H, L, d))
             rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
@@ -330,6 +337,12 @@ def other_configs(ctx, lib, cpu, only=None):
             for b_ in qkv + [o]:
                 b_.release()
         dmask.release()
+    if want("decode_head_dims"):
+        # config 5's decode (B16 H16, 4096 cached rows + 64 steps) with cache rows of 128 and of 32 floats
+        for d in (128, 32):
+            dec = decode(ctx, lib, 3, d)
+            res["config5_shape_decode_head_dim_%d" % d] = {"us_per_step": dec["us_per_step"], "gbs": dec["gbs"], "frac_hbm_peak": dec["gbs"] / HBM_PEAK_GBS,
+                                                            "bytes_per_step": dec["bytes_per_step"]}
     if want("greedy") or want("greedy_fused") or want("greedy_primitive") or want("greedy_cached") or want("greedy_cached_only"):
         # the caller of the blocks: Transformer greedy decoding (batch 1; every step re-runs the decoder on the prefix, as the
         # reference does).  6 + 6 layers, hidden 512, 8 heads of 64, ffn 2048, vocabulary 8000, 64 source tokens, 32 generated.
@@ -513,7 +526,7 @@ def main():
                          "profiler counter runs")
     ap.add_argument("--only", default="", metavar="NAMES",
                     help="instead of the benchmark, run only these of the workloads reported beside the headline (comma "
-                         "separated: config1, config2, recorded, config3, backward, masks_and_head_dim, greedy, greedy_fused, greedy_primitive, greedy_cached, greedy_cached_only) and print their entries: "
+                         "separated: config1, config2, recorded, config3, backward, masks_and_head_dim, decode_head_dims, greedy, greedy_fused, greedy_primitive, greedy_cached, greedy_cached_only) and print their entries: "
                          "short commands for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:
