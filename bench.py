@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # streaming kernel (--copy-calibration: x2.00 and x1.00).  The runs and their figures are summarised in
 # profiles/bench_prefill_config4_decode_config5.md; they are constants here because a counter run cannot be part of
 # the timed process.
-PREFILL_TRAFFIC_BYTES = (397295 * 2.00 + 65536 * 1.00) * 1024      # L2 fills (K/V re-reads included) + writes
-DECODE_TRAFFIC_BYTES = (264295 * 2.00 + 192 * 1.00) * 1024
+PREFILL_TRAFFIC_BYTES = (395661 * 2.00 + 65536 * 1.00) * 1024      # L2 fills (K/V re-reads included) + writes
+DECODE_TRAFFIC_BYTES = (264304 * 2.00 + 192 * 1.00) * 1024
 PREHEAT_S = 0.25
 
 
@@ -483,6 +483,7 @@ def kernel_sample(ctx, lib, iters):
     timed("ffn_up_gelu_8192x1024x4096", lambda: ctx.dense_fused(x, M, D, w1, F, b1, lib.ACT_GELU, None, h))
     timed("ffn_down_residual_8192x4096x1024", lambda: ctx.dense_fused(h, M, F, w2, D, b2, lib.ACT_NONE, x, y))
     timed("fc_residual_8192x1024x1024", lambda: ctx.dense_fused(x, M, D, wq, D, None, lib.ACT_NONE, x, y))
+    timed("fc_residual_layernorm_8192x1024x1024", lambda: ctx.dense_layernorm(x, M, D, wq, D, None, lib.ACT_NONE, x, 1024, b2, b2, y))
     for b_ in (x, h, w1, w2, wq, b1, b2, y):
         b_.release()
     B, H, L = 8, 16, 1024
