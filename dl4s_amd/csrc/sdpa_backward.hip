@@ -1184,11 +1184,11 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
         rc = dl4s::launch_status("sdpa_bwd_rowdot128");
         if (rc == DL4S_HIP_OK) {
             switch (m.kind) {
-                case DL4S_MASK_NONE: rc = launch_bwd128<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
-                case DL4S_MASK_DENSE_F32: rc = launch_bwd128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
-                case DL4S_MASK_CAUSAL: rc = launch_bwd128<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
-                case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
-                default: rc = launch_bwd128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes()); break;
+                case DL4S_MASK_NONE: rc = launch_bwd128<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
+                case DL4S_MASK_DENSE_F32: rc = launch_bwd128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
+                case DL4S_MASK_CAUSAL: rc = launch_bwd128<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
+                case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
+                default: rc = launch_bwd128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
             }
         }
         const int rcf = dl4s_hip_free(ctx, Dv);

@@ -201,6 +201,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
 // ------------------------------------------------------------------------------------------------ dK, dV
 // WRITE_DS: every visited tile of dS is also stored to ds [batch*head][Lkp][Lqp] for sdpa_bwd_dq_from_ds_f32_d128 (the
 // layout and rules of the 64-wide kernels).
+// nsplit > 1 (small launches: the kernel runs one workgroup per CU): workgroup blockIdx.y of nsplit takes the query tiles
+// y, y + nsplit, ... of its key block - an assignment by tile index, whatever the mask lets the block skip - and leaves its
+// unscaled sums in part [share][dk | dv][batch*head*Lk][128]; sdpa_bwd_merge_d128 adds the shares up in order.
 template <int KIND, bool WRITE_DS = false>
 __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
                                                                  const float *__restrict__ v, const float *__restrict__ dout,
@@ -208,7 +211,8 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                                                                  float *__restrict__ dk, float *__restrict__ dv, int H, int Lq,
                                                                  int Lk, float rT, MaskArgs mask, int strict, int nkb,
                                                                  int total_blocks, int lpt, int token_major, int hd,
-                                                                 float *__restrict__ ds = nullptr) {
+                                                                 float *__restrict__ ds = nullptr, int nsplit = 1,
+                                                                 float *__restrict__ part = nullptr) {
     extern __shared__ __align__(16) float lds[];
     float *Qs = lds;                        // [2][BN][LSTR2]  q * rT * log2(e)
     float *Gs = lds + 2 * TILE2_FLOATS;     // [2][BN][LSTR2]  dout
@@ -302,7 +306,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
 #pragma unroll
         for (int i = 0; i < 16; ++i) { ka[c][i] = 0.f; va[c][i] = 0.f; }
 
-    if (t_begin < nqt) { load_tile(t_begin); store_tile(0); }
+    const int sp = blockIdx.y;
+    int t = t_begin + (((sp - t_begin) % nsplit) + nsplit) % nsplit;   // the share's first tile at or after t_begin
+    if (t < nqt) { load_tile(t); store_tile(0); }
     __syncthreads();
 
     const int row_lds = ln * LSTR2 + half * 64;
@@ -320,18 +326,16 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
     }
 
     // tiles the wavefront only stages first, then a loop whose every path stores dS (see sdpa_bwd_dkv_f32_d64)
-    int t = t_begin;
+    int buf = 0;
     const int wt_first = __builtin_amdgcn_readfirstlane(wave_active ? max(wt_begin, t_begin) : nqt);   // the same in every lane
-    for (; t < wt_first && t < nqt; ++t) {
-        const int buf = (t - t_begin) & 1;
-        if (t + 1 < nqt) { load_tile(t + 1); store_tile(buf ^ 1); }
+    for (; t < wt_first && t < nqt; t += nsplit, buf ^= 1) {
+        if (t + nsplit < nqt) { load_tile(t + nsplit); store_tile(buf ^ 1); }
         __syncthreads();
     }
     wait_vector_memory();   // the loads of the lane's key and value rows: nothing from before the loop is left in flight
-    for (; t < nqt; ++t) {
-        const int buf = (t - t_begin) & 1;
-        const bool more = (t + 1 < nqt);
-        if (more) load_tile(t + 1);
+    for (; t < nqt; t += nsplit, buf ^= 1) {
+        const bool more = (t + nsplit < nqt);
+        if (more) load_tile(t + nsplit);
         const int qt0 = t * 32;
         int cls = 2;
         if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq] & 3;
@@ -396,10 +400,38 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
+    if (part) {
+        if (key < Lk) {
+            const long long rows = (long long)(total_blocks / nkb) * Lk;
+            float *pp = part + (((long long)sp * 2) * rows + (long long)bh * Lk + key) * HD2;
+            store_row_t128(pp, ka, 1.0f, half, HD2);
+            store_row_t128(pp + rows * HD2, va, 1.0f, half, HD2);
+        }
+        return;
+    }
     if (key < Lk) {
         store_row_t128(dv + kv_base + (long long)key * rs, va, 1.0f, half, hd);
         store_row_t128(dk + kv_base + (long long)key * rs, ka, 0.69314718055994530942f, half, hd);   // Q~ carries log2(e)
     }
+}
+
+// out[row][0 .. hd-1] = scale * (share 0 + share 1 + ...) of unscaled partial sums part[share][rows][128] (shares
+// share_stride floats apart); 32 lanes per row, four columns each
+__global__ __launch_bounds__(256) void sdpa_bwd_merge_d128(const float *__restrict__ part, float *__restrict__ out, int nsplit,
+                                                           long long share_stride, long long rows, int H, int L, int hd,
+                                                           int token_major, float scale) {
+    const long long row = (long long)blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int c = threadIdx.x & 31;
+    if (row >= rows || 4 * c >= hd) return;
+    f32x4 acc = *reinterpret_cast<const f32x4 *>(part + row * HD2 + 4 * c);
+    for (int s = 1; s < nsplit; ++s) {
+        const f32x4 x = *reinterpret_cast<const f32x4 *>(part + (long long)s * share_stride + row * HD2 + 4 * c);
+        acc.x += x.x; acc.y += x.y; acc.z += x.z; acc.w += x.w;
+    }
+    acc.x *= scale; acc.y *= scale; acc.z *= scale; acc.w *= scale;
+    const long long bh = row / L, i = row % L, b = bh / H, hh = bh % H;
+    const long long at = token_major ? (((b * L + i) * H + hh) * hd) : (row * hd);
+    *reinterpret_cast<f32x4 *>(out + at + 4 * c) = acc;
 }
 
 // ------------------------------------------------------------------------------------------------ dQ from stored dS
@@ -409,7 +441,10 @@ template <int KIND>
 __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const float *__restrict__ k, const float *__restrict__ ds,
                                                                         float *__restrict__ dq, int H, int Lq, int Lk, float rT,
                                                                         MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
-                                                                        int token_major, int hd) {
+                                                                        int token_major, int hd, int nsplit = 1,
+                                                                        float *__restrict__ part = nullptr) {
+    // nsplit > 1: workgroup blockIdx.y takes the key tiles y, y + nsplit, ... and leaves its unscaled sums in
+    // part [share][batch*head*Lq][128] for sdpa_bwd_merge_d128
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                      // [2][BN][LSTR2]
     int bh, unit;
@@ -483,25 +518,29 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
 #pragma unroll
     for (int i = 0; i < 16; ++i) dsn[i] = 0.f;
 
-    if (ntiles > 0) {
-        load_tile(0);
+    const int sp = blockIdx.y;
+    if (sp < ntiles) {
+        load_tile(sp);
         store_tile(0);
-        if (visited(0)) load_ds(0);
+        if (visited(sp)) load_ds(sp);
     }
     __syncthreads();
     const int col_lds = (4 * half) * LSTR2 + 4 * ln;
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        const bool more = (t + 1 < ntiles);
+    for (int t = sp, buf = 0; t < ntiles; t += nsplit, buf ^= 1) {
+        const bool more = (t + nsplit < ntiles);
         const bool now = visited(t);
         const f32x16 p = dsn;
         if (more) {
-            load_tile(t + 1);
-            if (visited(t + 1)) load_ds(t + 1);
+            load_tile(t + nsplit);
+            if (visited(t + nsplit)) load_ds(t + nsplit);
         }
         if (now) tile_accumulate_t128(Ks + buf * TILE2_FLOATS + col_lds, p, acc);               // dQ^T += K^T . dS^T
         if (more) store_tile(buf ^ 1);
         __syncthreads();
+    }
+    if (part) {
+        if (qi < Lq) store_row_t128(part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * HD2, acc, 1.0f, half, HD2);
+        return;
     }
     if (qi < Lq) store_row_t128(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
 }
@@ -509,7 +548,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
 template <int KIND>
 int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
                   const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
-                  int strict, int token_major, int hd, long long ds_max_bytes) {
+                  int strict, int token_major, int hd, long long ds_max_bytes, int no_split = 0) {
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     const size_t lds_dq = 4 * TILE2_FLOATS * sizeof(float);
     const size_t lds_dkv = (4 * TILE2_FLOATS + 192) * sizeof(float);
@@ -534,20 +573,50 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
         if (slab < (1ll << 31) && (long long)B * H * slab <= ds_max_bytes && total_q < (1ll << 30) && total_k < (1ll << 30) &&
             dl4s_hip_alloc(ctx, (size_t)((long long)B * H * slab), &dsv) == DL4S_HIP_OK) {
             float *ds = static_cast<float *>(dsv);
+            // Launches that leave CUs without a workgroup (dK/dV: one per CU; dQ: two) are split over the walked tiles
+            // across workgroups; the counts depend on the extents only.  B4 H8 L512 causal: 186 us unsplit.
+            const long long nqt = (Lq + 31) / 32, nkt = (Lk + 31) / 32;
+            long long sk = 1, sq = 1;
+            // (blocks of different length: two shares also where every CU just has its workgroup, B2 H8 L2048 causal 679 -> 497 us)
+            if (!no_split && total_k < (uneven ? 2ll : 1ll) * ctx->cu_count && nqt >= 4)
+                sk = std::min(std::min(8ll, nqt / 2), std::max(2ll, (ctx->cu_count + total_k - 1) / total_k));
+            if (!no_split && total_q < (uneven ? 4ll : 2ll) * ctx->cu_count && nkt >= 4)
+                sq = std::min(std::min(8ll, nkt / 2), std::max(2ll, (2ll * ctx->cu_count + total_q - 1) / total_q));
+            const long long krows = (long long)B * H * Lk, qrows = (long long)B * H * Lq;
+            const long long part_k = sk > 1 ? sk * 2 * krows * HD2 : 0, part_q = sq > 1 ? sq * qrows * HD2 : 0;
+            void *pv = nullptr;
+            if (part_k + part_q > 0 && dl4s_hip_alloc(ctx, (size_t)(part_k + part_q) * sizeof(float), &pv) != DL4S_HIP_OK) { sk = sq = 1; pv = nullptr; }
+            float *pk = sk > 1 ? static_cast<float *>(pv) : nullptr;
+            float *pq = sq > 1 ? static_cast<float *>(pv) + (sk > 1 ? part_k : 0) : nullptr;
             int lpt = (uneven && nkb >= 2) ? 1 : 0;
             if (lpt && total_k <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
-            hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d128<KIND, true>), dim3((unsigned)((total_k + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream,
-                               q, k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total_k, lpt, token_major, hd, ds);
+            hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d128<KIND, true>), dim3((unsigned)((total_k + 7) / 8 * 8), (unsigned)sk), dim3(256), lds_dkv,
+                               ctx->stream, q, k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total_k, lpt, token_major, hd,
+                               ds, (int)sk, pk);
             int rc = dl4s::launch_status("sdpa_bwd_dkv_f32_d128");
+            if (rc == DL4S_HIP_OK && pk) {
+                const dim3 mg((unsigned)((krows + 7) / 8));
+                hipLaunchKernelGGL(sdpa_bwd_merge_d128, mg, dim3(256), 0, ctx->stream, pk, dk, (int)sk, 2 * krows * HD2, krows, H, Lk, hd,
+                                   token_major, 0.69314718055994530942f);   // Q~ carries log2(e)
+                hipLaunchKernelGGL(sdpa_bwd_merge_d128, mg, dim3(256), 0, ctx->stream, pk + krows * HD2, dv, (int)sk, 2 * krows * HD2, krows, H,
+                                   Lk, hd, token_major, 1.0f);
+                rc = dl4s::launch_status("sdpa_bwd_merge_d128");
+            }
             if (rc == DL4S_HIP_OK) {
                 lpt = (uneven && nqb >= 2) ? 1 : 0;
                 if (lpt && total_q <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
-                hipLaunchKernelGGL(sdpa_bwd_dq_from_ds_f32_d128<KIND>, dim3((unsigned)((total_q + 7) / 8 * 8)), dim3(256),
+                hipLaunchKernelGGL(sdpa_bwd_dq_from_ds_f32_d128<KIND>, dim3((unsigned)((total_q + 7) / 8 * 8), (unsigned)sq), dim3(256),
                                    2 * TILE2_FLOATS * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q,
-                                   lpt, token_major, hd);
+                                   lpt, token_major, hd, (int)sq, pq);
                 rc = dl4s::launch_status("sdpa_bwd_dq_from_ds_f32_d128");
+                if (rc == DL4S_HIP_OK && pq) {
+                    hipLaunchKernelGGL(sdpa_bwd_merge_d128, dim3((unsigned)((qrows + 7) / 8)), dim3(256), 0, ctx->stream, pq, dq, (int)sq,
+                                       qrows * HD2, qrows, H, Lq, hd, token_major, rT);
+                    rc = dl4s::launch_status("sdpa_bwd_merge_d128");
+                }
             }
-            const int rcf = dl4s_hip_free(ctx, dsv);   // stream-ordered
+            int rcf = dl4s_hip_free(ctx, dsv);   // stream-ordered
+            if (pv) { const int rcp = dl4s_hip_free(ctx, pv); if (rcf == DL4S_HIP_OK) rcf = rcp; }
             return rc != DL4S_HIP_OK ? rc : rcf;
         }
     }
