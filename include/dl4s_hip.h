@@ -152,11 +152,13 @@ typedef struct dl4s_mask_desc {
  * v [B,H,Lk,dv], out [B,H,Lq,dv], all row-major contiguous device fp32.  inv_temperature is the
  * fp32 reciprocal the reference forms once (Engine/CPU/CPUEngine.swift:635).  mask may be NULL
  * (= DL4S_MASK_NONE).  dk = dv, a multiple of 4 and at most 128, with 16-byte aligned tensors runs
- * a fused MFMA kernel (one written for 64, one for 128; smaller head dims are padded with zero
- * columns on the fly and cost as much as the width they are padded to).  Other head dims up to 128
- * (dk != dv, not a multiple of 4, unaligned tensors) run the same kernels on zero-padded copies of the
- * operands, which the call allocates from the context's pool, when the problem is large enough to pay
- * for the copies; small problems and head dims up to 256 run a plain fused kernel. */
+ * a fused MFMA kernel written for tiles of 16, 32, 64, 96 (launches that fill the GPU) or 128 columns;
+ * a head dim between two widths is padded with zero columns on the fly and costs what the wider tile
+ * costs.  Even head dims from 66 to 94 that are not a multiple of 4 run the 96-wide kernel as they are
+ * (8-byte aligned tensors, launches that fill the GPU).  Other head dims up to 128 (dk != dv, odd,
+ * unaligned tensors) run the same kernels on zero-padded copies of the operands, which the call
+ * allocates from the context's pool, when the problem is large enough to pay for the copies; small
+ * problems and head dims up to 256 run a plain fused kernel. */
 int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
                           int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
@@ -177,6 +179,10 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
  * kernels otherwise) because the two kinds of kernels keep the statistics in different forms: pass both calls the same
  * tensors and extents.  On the direct MFMA route dout, dq, dk, dv must be 16-byte aligned too (DL4S_HIP_EUNSUPPORTED
  * otherwise).
+ * Large launches form the scores once: the dK/dV kernel stores its dS tiles in a scratch tensor of B*H*Lk*Lq floats
+ * from the context's pool and a second kernel contracts them with K.  The scratch is bounded by 24 GiB or by the
+ * environment variable DL4S_HIP_BWD_SCRATCH_MAX_BYTES (0 = never); beyond the bound, or when the pool cannot supply it,
+ * two self-contained kernels run that form the scores twice.
  * Deterministic: no atomics, the same bits on every run. */
 int dl4s_hip_sdpa_fwd_stats_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, float *stats,
                                 int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t d, float inv_temperature,
