@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256, 3) void sdpa_bwd_dkv_f32_narrow(const float *_
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
     const int Lqp = (Lq + 31) & ~31, Lkp = (Lk + 31) & ~31;
     const __amdgpu_buffer_rsrc_t dsrsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lkp * Lqp * 4), 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lk * Lqp * 4), 0x00020000);
     const unsigned ds_voff = ((unsigned)key * (unsigned)Lqp + 4u * half) * 4u;
 
     // tiles the wavefront only stages first, then a loop whose every path stores dS (see sdpa_bwd_dkv_f32_d64)
@@ -231,10 +231,8 @@ __global__ __launch_bounds__(256, 3) void sdpa_bwd_dkv_f32_narrow(const float *_
                 p[4 * g + 2] = p[4 * g + 2] * (dp[4 * g + 2] - d4.z);
                 p[4 * g + 3] = p[4 * g + 3] * (dp[4 * g + 3] - d4.w);
             }
-            if (kw0 + 32 > Lk && key >= Lk) {       // a key that does not exist: its row of dS is zero
-#pragma unroll
-                for (int r = 0; r < 16; ++r) p[r] = 0.f;
-            }
+            // (rows of dS for keys that do not exist lie outside the descriptor: their stores are dropped, and the dQ
+            // kernel, whose descriptor ends at the same row, reads them as zeros)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const f32x4 o = {p[4 * g + 0], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]};
@@ -302,7 +300,7 @@ __global__ __launch_bounds__(256, 4) void sdpa_bwd_dq_from_ds_f32_narrow(const f
 
     const int Lqp = (Lq + 31) & ~31, Lkp = (Lk + 31) & ~31;
     const __amdgpu_buffer_rsrc_t dsrsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lkp * Lqp * 4), 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc((void *)(ds + (long long)bh * Lkp * Lqp), 0, (int)((long long)Lk * Lqp * 4), 0x00020000);
     const unsigned ds_voff = ((unsigned)(4 * half) * (unsigned)Lqp + (unsigned)qi) * 4u;
     const unsigned ds_row = (unsigned)Lqp * 4u;
     const unsigned char *cls_row = nullptr;
