@@ -239,13 +239,14 @@ struct FastOperand {
 // products still put a workgroup on every CU).  TA / TB: the operand is stored transposed (transposeFirst / Second).
 // KT: K tile depth.  The 64x64 form runs one to three wavefronts per SIMD, where a K tile of 16 (8 MFMAs = 512 cycles
 // between barriers) does not cover the latency of the next tile's loads; it takes K tiles of 32.
+// (128 x 128 tiles with 32-deep K tiles hold 70 KiB of LDS: two workgroups per CU, which is all their launches have)
 template <int MI, int NI, bool EPI, bool TA, bool TB, int KT>
-__global__ __launch_bounds__(256, 3) void gemm_f32_mfma_fast(GemmArgs g) {
+__global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_mfma_fast(GemmArgs g) {
     constexpr int TM = 64 * MI, TN = 64 * NI;       // workgroup tile
     using OpA = FastOperand<MI, TA, KT>;             // A is M x K in memory unless transposed
     using OpB = FastOperand<NI, !TB, KT>;            // B is K x N in memory unless transposed
-    __shared__ __align__(16) float As[OpA::LDS_FLOATS];
-    __shared__ __align__(16) float Bs[OpB::LDS_FLOATS];
+    extern __shared__ __align__(16) float gemm_lds[];
+    float *As = gemm_lds, *Bs = gemm_lds + OpA::LDS_FLOATS;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int half = lane >> 5, ln = lane & 31;
@@ -723,7 +724,27 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     }
     DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
     const dim3 grid((unsigned)(tm * tn), 1, (unsigned)batch);
-#define DL4S_GEMM_FAST(MI_, EPI_, TA_, TB_) hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, (MI_ == 1 ? 32 : 16)>), grid, dim3(256), 0, ctx->stream, g)
+    // 128 x 128 tiles on a launch of at most two workgroups per CU: K tiles of 32 (half the barriers; contracted as two
+    // halves of 16, so the bits do not depend on the depth)
+    const bool deep = fast && !small && tm * tn * batch <= 2ll * ctx->cu_count;
+#define DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, KT_)                                                                                   \
+    do {                                                                                                                              \
+        constexpr size_t lds_bytes = (FastOperand<MI_, TA_, KT_>::LDS_FLOATS + FastOperand<MI_, !TB_, KT_>::LDS_FLOATS) * sizeof(float); \
+        if (lds_bytes > 65536) {                                                                                                      \
+            constexpr int which = (EPI_ ? 4 : 0) + (TA_ ? 2 : 0) + (TB_ ? 1 : 0);                                                     \
+            if (dl4s::lds_limit_pending(ctx, dl4s::LDS_GEMM_DEEP, which)) {                                                           \
+                DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, KT_>),  \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));                        \
+                dl4s::lds_limit_done(ctx, dl4s::LDS_GEMM_DEEP, which);                                                                \
+            }                                                                                                                         \
+        }                                                                                                                             \
+        hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, KT_>), grid, dim3(256), lds_bytes, ctx->stream, g);          \
+    } while (0)
+#define DL4S_GEMM_FAST(MI_, EPI_, TA_, TB_)                                                   \
+    do {                                                                                      \
+        if (MI_ == 1 || deep) DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, 32);                     \
+        else DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, 16);                                      \
+    } while (0)
     if (fast) {
         const int variant = (small ? 0 : 8) + (epi ? 4 : 0) + (ta ? 2 : 0) + (tb ? 1 : 0);
         switch (variant) {
@@ -740,6 +761,7 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
         }
     }
 #undef DL4S_GEMM_FAST
+#undef DL4S_GEMM_FAST_KT
     else hipLaunchKernelGGL(gemm_f32_mfma, grid, dim3(256), 0, ctx->stream, g);
     return dl4s::launch_status("gemm_f32_mfma");
 }
