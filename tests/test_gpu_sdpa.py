@@ -567,6 +567,29 @@ def test_token_major_layout_is_bit_identical(ctx, B, H, Lq, Lk, d):
         assert np.array_equal(a, b), kw.keys()
 
 
+@pytest.mark.parametrize("d", [96, 70])
+@pytest.mark.parametrize("B,H,Lq,Lk", [(64, 16, 130, 5), (32, 16, 129, 33), (128, 8, 1, 64), (64, 8, 128, 31)])
+@pytest.mark.parametrize("mk", ["none", "causal_lens"])
+def test_96_wide_kernel_on_short_and_ragged_extents(ctx, orc, B, H, Lq, Lk, d, mk):
+    """Many (batch, head) pairs with few queries and keys: single tiles, a single query row, extents one past or one short
+    of a tile edge, with 128-bit (d = 96) and 64-bit (d = 70) staging."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(zlib.crc32(repr(("w96 short", B, H, Lq, Lk, d, mk)).encode()))
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    lens = rng.integers(0, Lk + 1, size=B)
+    lens[0] = max(1, Lk // 2)
+    kind, mask, lens_arg = None, None, None
+    if mk == "causal_lens":
+        kind, lens_arg = lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lk)[None, None])
+    got = run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg)
+    for b in (0, 1, B - 1):
+        mb = None if mask is None else mask[b:b + 1]
+        assert_parity(got[b:b + 1], orc.sdpa(q[b:b + 1], k[b:b + 1], v[b:b + 1], mb), "96-wide short d=%d b=%d" % (d, b))
+    if mask is not None:
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=True), run_sdpa(ctx, q, k, v, mask, strict=True))
+
+
 @pytest.mark.parametrize("d", [96, 80, 68, 70, 66, 94])
 @pytest.mark.parametrize("mk", ["none", "dense", "causal", "lens", "causal_lens"])
 def test_head_dims_up_to_96_on_launches_that_fill_the_gpu(ctx, orc, d, mk):

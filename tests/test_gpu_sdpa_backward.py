@@ -1,5 +1,7 @@
 """Gradients of the fused attention (dl4s_hip_sdpa_fwd_stats_f32 + dl4s_hip_sdpa_bwd_f32) against the CPU oracle's
 restatement of the reference's reverse-mode closures.  Gate: |gpu - oracle| <= 1e-4 + 1e-4 |oracle|."""
+import zlib
+
 import numpy as np
 import pytest
 
@@ -240,6 +242,34 @@ def test_gradients_for_other_head_dims(ctx, orc, d, mask_kind):
     assert_parity(dv.numpy(), rv, "dv d=%d" % d)
     for b in bufs + [out, dq, dk, dv, st] + keep:
         b.release()
+
+
+@pytest.mark.parametrize("d", [4, 8, 16, 20, 32])
+@pytest.mark.parametrize("B,H,Lq,Lk", [(1, 2, 5, 7), (2, 3, 33, 1), (1, 1, 1, 1), (1, 2, 40, 100), (3, 1, 31, 32), (2, 2, 1, 65)])
+@pytest.mark.parametrize("mask_kind", ["none", "dense", "causal_lengths"])
+def test_narrow_head_gradients_on_tiny_and_ragged_extents(ctx, orc, B, H, Lq, Lk, d, mask_kind):
+    """The 16- and 32-wide gradient kernels on single tiles, single rows and extents that end one past or one short of a
+    tile edge (key counts below 64 always take the stored-dS route, whatever the batch)."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(zlib.crc32(repr(("narrow", B, H, Lq, Lk, d, mask_kind)).encode()))
+    q, k, v, dout = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lq, d)
+    lens = rng.integers(0, Lk + 1, size=B)
+    lens[0] = max(1, Lk // 2)
+    kw, mask = {}, None
+    if mask_kind == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.4).astype(np.float32)
+        kw = dict(mask=mask)
+    elif mask_kind == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lk)[None, None])
+        kw = dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens)
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, **kw)
+    assert_parity(out, orc.sdpa(q, k, v, mask), "forward")
+    rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+    assert_parity(dq, rq, "dq")
+    assert_parity(dk, rk, "dk")
+    assert_parity(dv, rv, "dv")
+    for a, b_ in zip(run_fwd_bwd(ctx, q, k, v, dout, token_major=True, **kw), (out, stats, dq, dk, dv)):
+        assert np.array_equal(a, b_)
 
 
 @pytest.mark.parametrize("d", [70, 6, 99])
