@@ -343,7 +343,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
 
     const int row_lds = ln * LSTR + half * 32;
     const int col_lds = (4 * half) * LSTR + 2 * ln;
-    const float PEN = __fmul_rn(1e9f, LOG2E);
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
@@ -381,13 +380,13 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
             if (DENSE) {
                 if (cls == 1) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) p[r] = __fsub_rn(p[r], PEN);
+                    for (int r = 0; r < 16; ++r) p[r] = blocked_score2(p[r]);
                 } else if (cls == 2) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
                         const int qc = qg < Lq ? qg : Lq - 1;
-                        p[r] = __fsub_rn(p[r], dense_penalty2(mcol[qc * mask.sq]));
+                        p[r] = dense_masked2(p[r], mcol[qc * mask.sq]);
                     }
                 }
             } else if ((CAUSAL && (kw0 + 31 > qt0)) || (LENS && (kw0 + 32 > len))) {
@@ -397,7 +396,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_f32_d64(const float *__re
                     bool blocked = false;
                     if (CAUSAL) blocked = blocked || (key > qg);
                     if (LENS) blocked = blocked || (key >= len);
-                    if (blocked) p[r] = __fsub_rn(p[r], PEN);
+                    if (blocked) p[r] = blocked_score2(p[r]);
                 }
             }
             const float *st = Ss + buf * 32 + 4 * half;
@@ -788,7 +787,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_split_f32_d64(const float
     for (int i = 0; i < 16; ++i) { k0a[i] = 0.f; k1a[i] = 0.f; v0a[i] = 0.f; v1a[i] = 0.f; }
     const int row_lds = ln * LSTR + half * 32;
     const int col_lds = (4 * half) * LSTR + 2 * ln;
-    const float PEN = __fmul_rn(1e9f, LOG2E);
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
@@ -808,13 +806,13 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_split_f32_d64(const float
         if (DENSE) {
             if (cls == 1) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) p[r] = __fsub_rn(p[r], PEN);
+                for (int r = 0; r < 16; ++r) p[r] = blocked_score2(p[r]);
             } else if (cls == 2) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
                     const int qc = qg < Lq ? qg : Lq - 1;
-                    p[r] = __fsub_rn(p[r], dense_penalty2(mcol[qc * mask.sq]));
+                    p[r] = dense_masked2(p[r], mcol[qc * mask.sq]);
                 }
             }
         } else if ((CAUSAL && (kw0 + 31 > qt0)) || (LENS && (kw0 + 32 > len))) {
@@ -824,7 +822,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_split_f32_d64(const float
                 bool blocked = false;
                 if (CAUSAL) blocked = blocked || (key > qg);
                 if (LENS) blocked = blocked || (key >= len);
-                if (blocked) p[r] = __fsub_rn(p[r], PEN);
+                if (blocked) p[r] = blocked_score2(p[r]);
             }
         }
         const float *st = Ss + 4 * half;

@@ -313,7 +313,6 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
 
     const int row_lds = ln * LSTR2 + half * 64;
     const int col_lds = (4 * half) * LSTR2 + 4 * ln;
-    const float PEN = __fmul_rn(1e9f, LOG2E);
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
@@ -345,13 +344,13 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
             if (DENSE) {
                 if (cls == 1) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) p[r] = __fsub_rn(p[r], PEN);
+                    for (int r = 0; r < 16; ++r) p[r] = blocked_score2(p[r]);
                 } else if (cls == 2) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int qg = qt0 + 8 * (r >> 2) + 4 * half + (r & 3);
                         const int qc = qg < Lq ? qg : Lq - 1;
-                        p[r] = __fsub_rn(p[r], dense_penalty2(mcol[qc * mask.sq]));
+                        p[r] = dense_masked2(p[r], mcol[qc * mask.sq]);
                     }
                 }
             } else if ((CAUSAL && (kw0 + 31 > qt0)) || (LENS && (kw0 + 32 > len))) {
@@ -361,7 +360,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                     bool blocked = false;
                     if (CAUSAL) blocked = blocked || (key > qg);
                     if (LENS) blocked = blocked || (key >= len);
-                    if (blocked) p[r] = __fsub_rn(p[r], PEN);
+                    if (blocked) p[r] = blocked_score2(p[r]);
                 }
             }
             const float *st = Ss + buf * 32 + 4 * half;

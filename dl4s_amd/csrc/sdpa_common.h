@@ -190,6 +190,26 @@ __device__ __forceinline__ float dense_penalty2(const float mval) {
     return (__builtin_isinf(pen2) && !__builtin_isinf(pen)) ? __builtin_copysignf(3.402823466e38f, pen) : pen2;
 }
 
+// A score blocked by a mask value of exactly 1 (every structured kind, and the masks TransformerUtil.swift:29-50 builds).
+// The reference forms fl(s - 1e9) in the natural domain; floats next to 1e9 are 64 apart, so that is -1e9 + 64 n with
+// n = s / 64 rounded to nearest-even: the score survives only as its bucket on a grid of 64.  Next to an unblocked key
+// that is a weight of exactly zero whatever n is, but in a row with every key blocked the buckets decide: the keys of the
+// highest bucket share the row (the next bucket weighs e^-64 of that, nothing in fp32); scores within (-32, 32) fall
+// into one bucket and the row is uniform.  Subtracting 1e9 log2(e) from the base-2 score would sort the keys into other
+// buckets (floats there are 128 apart, 88.7 in the natural domain), so the reference's bucket is formed from the score
+// itself and carried on the base-2 grid: -PEN2 + 128 n, exact in fp32, with 2^-128 between buckets.  s2 is the score
+// times log2(e); its last bits differ from the reference's, which matters only for a score within rounding of a bucket
+// edge.  NaN and infinities pass through as they do through the subtraction.
+constexpr float PEN2 = 1442695040.0f;   // fl(1e9 * log2(e)), a multiple of 128
+__device__ __forceinline__ float blocked_score2(const float s2) {
+    const float n = __builtin_rintf(__fmul_rn(s2, 0.69314718055994530942f / 64.0f));
+    return __builtin_fmaf(n, 128.0f, -PEN2);
+}
+// s2 under a dense mask value: the bucket form for a value of exactly 1, the scaled penalty for any other
+__device__ __forceinline__ float dense_masked2(const float s2, const float mval) {
+    return mval == 1.0f ? blocked_score2(s2) : __fsub_rn(s2, dense_penalty2(mval));
+}
+
 // S^T = K . Q^T for one 32-key tile of one wavefront (lane = query qi = q0 + lane % 32, 16 of the 32 keys per lane:
 // accumulator register r is key k0 + 8(r/4) + 4*half + r%4), then the mask, in registers.  Kb is the lane's K fragment
 // base in LDS; qr the lane's Q fragment, already scaled by (1/T) log2(e): the scores are in the base-2 exponent domain.
@@ -222,13 +242,13 @@ __device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&q
     if (DENSE) {
         if (cls == 1) {           // every element of the tile is 1: the penalty is a constant
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+            for (int r = 0; r < 16; ++r) s0[r] = blocked_score2(s0[r]);
         } else if (cls == 2) {    // mixed tile: read the mask values (class 0 = all zeros needs nothing)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int kg = k0 + 8 * (r >> 2) + 4 * half + (r & 3);
                 const int kc = kg < Lk ? kg : Lk - 1;
-                s0[r] = __fsub_rn(s0[r], dense_penalty2(mrow[kc * msk]));
+                s0[r] = dense_masked2(s0[r], mrow[kc * msk]);
             }
         }
     } else if ((CAUSAL && (k0 + BN - 1 > q0)) || (LENS && (k0 + BN > len))) {
@@ -238,7 +258,7 @@ __device__ __forceinline__ f32x16 masked_scores(const float *Kb, const float (&q
             bool blocked = false;
             if (CAUSAL) blocked = blocked || (kg > qi);
             if (LENS) blocked = blocked || (kg >= len);
-            if (blocked) s0[r] = __fsub_rn(s0[r], __fmul_rn(1e9f, LOG2E));
+            if (blocked) s0[r] = blocked_score2(s0[r]);
         }
     }
     if (k0 + BN > Lk) {           // keys past the end of the tensor take no part

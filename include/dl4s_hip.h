@@ -135,7 +135,9 @@ typedef struct dl4s_mask_desc {
                                of a dense mask in query blocks whose every row keeps an unblocked key (a zero) - which
                                is exact as long as K and V hold finite values at blocked positions (the reference
                                computes 0 * v there, so a NaN/Inf in V or K at a blocked key reaches the output only
-                               in strict mode).  Fully blocked rows are never skipped: they come out uniform. */
+                               in strict mode).  Fully blocked rows are never skipped: they come out as the reference computes
+                               them - uniform while their scores stay within +-32, shared by the keys of the highest
+                               bucket of fl(s - 1e9) on the grid of 64 that floats have next to 1e9 beyond that. */
 #define DL4S_SDPA_TOKEN_MAJOR 2u /* q, out are [B,Lq,H,d] and k, v are [B,Lk,H,d] (the layout the projections of
                                     MultiHeadAttention produce, NN/Models/Transformer/MultiHeadAttention.swift:105-107
                                     before its permutes :109-111, and the layout its output permute :117 produces), so a
@@ -203,7 +205,7 @@ int dl4s_hip_sdpa_decode_f32(dl4s_hip_ctx *ctx, const float *q, const float *kca
  * gathered [B,H,T,d] tensors under the mask of makeEncoderMasks, m[b,0,0,j] = (j >= lengths[b])
  * (NN/Models/Transformer/TransformerUtil.swift:29-36).  With 1 <= lengths[b] the blocked keys have weight exactly zero in
  * the reference and are not visited here (exact while K and V are finite there, as for the prefill kernels without
- * DL4S_SDPA_STRICT); lengths[b] <= 0 blocks every key and the row comes out uniform over all T keys, as in the
+ * DL4S_SDPA_STRICT); lengths[b] <= 0 blocks every key and the row comes out over all T keys (uniform for scores within +-32), as in the
  * reference; lengths[b] >= T blocks nothing.  lengths == NULL is dl4s_hip_sdpa_decode_f32. */
 int dl4s_hip_sdpa_decode_lengths_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache,
                                      float *out, int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d,

@@ -209,6 +209,56 @@ def test_blocked_keys_have_exactly_zero_weight_and_blocked_rows_are_uniform(ctx,
     assert not np.isnan(base).any()
 
 
+@pytest.mark.parametrize("d", [64, 8, 32, 128, 10])
+@pytest.mark.parametrize("mk", ["dense", "dense_ones_tiles", "lens", "causal_lens"])
+def test_fully_blocked_rows_with_large_scores_follow_the_reference_rounding(ctx, orc, d, mk):
+    """A row whose every key is blocked: the reference's fl(s - 1e9) keeps a score only as its bucket on the grid of 64
+    that floats have next to 1e9, so with scores beyond +-32 the row is not uniform - the keys of the highest bucket
+    share it (ScaledDotProductAttention.swift:55-59).  Scores here reach +-150; the oracle does that arithmetic, the
+    kernels have to land in the same buckets (MFMA kernels: d = 64, 8, 32, 128; plain kernel: d = 10)."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(zlib.crc32(repr(("blocked large", d, mk)).encode()))
+    B, H, Lq, Lk = 2, 2, 70, 100
+    if mk == "causal_lens":
+        Lk = Lq
+    q, k, v = rand(rng, B, H, Lq, d, scale=5.0), rand(rng, B, H, Lk, d, scale=5.0), rand(rng, B, H, Lk, d)
+    kind, lens_arg, lens = None, None, np.array([0, Lk // 2])
+    if mk == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.5).astype(np.float32)
+        mask[:, :, 5, :] = 1.0
+        mask[:, :, 40:44, :] = 1.0
+    elif mk == "dense_ones_tiles":
+        mask = np.zeros((B, 1, Lq, Lk), np.float32)
+        mask[:, :, 32:64, :] = 1.0           # a whole 32-row block blocked: tiles of ones only
+    elif mk == "lens":
+        kind, lens_arg, mask = lib.MASK_KEY_LENGTHS, lens, lengths_mask(lens, Lk)         # batch item 0 has no valid key
+    else:
+        kind, lens_arg = lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lk)[None, None])
+    blocked = np.broadcast_to(mask, (B, H, Lq, Lk)).min(axis=3) >= 1.0
+    assert blocked.any()
+    # In the blocked rows keep every score 0.05 away from a bucket edge (32 + 64 n), where the last bits of the kernel's
+    # score - summed in another order than the oracle's - would decide the bucket: nudge the query rows until none is left.
+    T = float(np.float32(np.sqrt(np.float32(d))))
+    for _ in range(50):
+        s = np.einsum("bhid,bhjd->bhij", q.astype(np.float64) / T, k.astype(np.float64))
+        edge = np.abs(np.abs(s) - 32.0) % 64.0
+        near = (np.minimum(edge, 64.0 - edge) < 0.05) & blocked[..., None]
+        if not near.any():
+            break
+        for b, h, i in np.argwhere(near.any(axis=3)):
+            q[b, h, i] *= np.float32(1.003)
+    assert not near.any()
+    ref = orc.sdpa(q, k, v, mask)
+    b0, h0, i0 = np.argwhere(blocked)[0]
+    assert not np.allclose(ref[b0, h0, i0], v[b0, h0].mean(axis=0), atol=1e-3)      # the reference's rows are not uniform here
+    for strict in (False, True):
+        got = run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=strict)
+        assert_parity(got, ref, "fully blocked rows, large scores, d=%d %s strict=%s" % (d, mk, strict))
+    if kind is not None:
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=True), run_sdpa(ctx, q, k, v, mask, strict=True))
+
+
 @pytest.mark.parametrize("d", [8, 10, 64, 128, 88])
 def test_nan_inf_placement_matches_oracle(ctx, orc, d):
     rng = np.random.default_rng(9)

@@ -329,6 +329,43 @@ def test_gradients_after_the_96_wide_forward_kernel(ctx, orc, d, mask_kind):
     assert np.isfinite(dq).all() and np.isfinite(dk).all() and np.isfinite(dv).all()
 
 
+@pytest.mark.parametrize("d", [64, 32, 128, 6])
+@pytest.mark.parametrize("mask_kind", ["dense", "lengths"])
+def test_gradients_of_fully_blocked_rows_with_large_scores(ctx, orc, d, mask_kind):
+    """Rows with every key blocked and scores beyond +-32: the reference's weights there are set by the rounding of
+    s - 1e9 on the grid of 64 (the keys of the highest bucket share the row), and its gradients follow those weights."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(zlib.crc32(repr(("blocked large bwd", d, mask_kind)).encode()))
+    B, H, Lq, Lk = 2, 2, 70, 100
+    q, k, v, dout = rand(rng, B, H, Lq, d, scale=5.0), rand(rng, B, H, Lk, d, scale=5.0), rand(rng, B, H, Lk, d), rand(rng, B, H, Lq, d)
+    lens = np.array([0, Lk // 2])
+    if mask_kind == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.5).astype(np.float32)
+        mask[:, :, 5, :] = 1.0
+        mask[:, :, 32:64, :] = 1.0
+        kw = dict(mask=mask)
+    else:
+        mask, kw = lengths_mask(lens, Lk), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    blocked = np.broadcast_to(mask, (B, H, Lq, Lk)).min(axis=3) >= 1.0
+    T = float(np.float32(np.sqrt(np.float32(d))))
+    for _ in range(50):     # no score of a blocked row within 0.05 of a bucket edge (32 + 64 n)
+        s = np.einsum("bhid,bhjd->bhij", q.astype(np.float64) / T, k.astype(np.float64))
+        edge = np.abs(np.abs(s) - 32.0) % 64.0
+        near = (np.minimum(edge, 64.0 - edge) < 0.05) & blocked[..., None]
+        if not near.any():
+            break
+        for b, h, i in np.argwhere(near.any(axis=3)):
+            q[b, h, i] *= np.float32(1.003)
+    assert blocked.any() and not near.any()
+    for strict in (False, True):
+        out, _, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, strict=strict, **kw)
+        assert_parity(out, orc.sdpa(q, k, v, mask), "forward")
+        rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+        assert_parity(dq, rq, "dq d=%d %s" % (d, mask_kind))
+        assert_parity(dk, rk, "dk d=%d %s" % (d, mask_kind))
+        assert_parity(dv, rv, "dv d=%d %s" % (d, mask_kind))
+
+
 def test_backward_argument_errors(ctx):
     from dl4s_amd import lib
     a = ctx.empty((1, 1, 4, 300))
