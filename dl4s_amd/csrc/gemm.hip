@@ -644,7 +644,7 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     g.lda = lc; g.ldb = rc;
     g.alpha = alpha; g.beta = beta;
     g.bias = bias; g.residual = residual; g.act = act;
-    const bool epi = bias || residual || act;
+    const bool epi = bias || residual || act || ln_part;   // the LayerNorm sums are part of the epilogue kernels
     const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     // The fast kernels: every unit-stride extent a multiple of 4 (128-bit accesses), 16-byte aligned operands, and 32-bit
     // byte offsets below 2^31 (an operand stored rows x K is addressed within a tile's 128 rows, one stored K x rows as a whole).

@@ -499,12 +499,13 @@ def test_dense_fused_equals_separate_engine_calls(ctx, orc, M, K, N, act, with_b
     (8, 1024, 64, 1024),     # 128 x 128 tiles, 64 pairs per item
     (2, 128, 64, 2048),      # 32 pairs per item
     (3, 64, 128, 260),       # a last column tile that is partly outside
+    (5, 128, 4, 512),        # a contraction of one MFMA step
     (2, 100, 128, 256),      # items that are not whole tiles: two calls
     (600, 1, 128, 128),      # per-row statistics: two calls
     (2, 30, 512, 512),       # a skinny product: two calls
     (1, 8192, 64, 512),      # more pairs than the normalising pass sums: two calls
 ])
-@pytest.mark.parametrize("with_bias,act,with_res", [(False, 0, True), (True, 1, False), (True, 0, True)])
+@pytest.mark.parametrize("with_bias,act,with_res", [(False, 0, True), (True, 1, False), (True, 0, True), (False, 0, False)])
 def test_dense_layernorm_in_one_call(ctx, orc, items, item_rows, K, N, with_bias, act, with_res):
     """LayerNorm(act(x.W + b) + r) with the statistics taken from the product's epilogue: within the gate of the oracle's
     Dense / gaussianErrorLinear / residual / LayerNorm sequence, and within rounding of the two separate calls (same
