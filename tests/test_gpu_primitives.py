@@ -542,6 +542,35 @@ def test_dense_layernorm_in_one_call(ctx, orc, items, item_rows, K, N, with_bias
         t.release()
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_dense_layernorm_random_shapes(ctx, orc, seed):
+    """Seeded random item counts, item lengths, widths and epilogue terms (none of them included): whichever route the call
+    takes - sums from the epilogue, or the two separate calls - the result is within the gate of the oracle's sequence."""
+    rng = np.random.default_rng(90000 + seed)
+    items, item_rows = int(rng.integers(1, 6)), int(rng.choice([1, 3, 32, 64, 100, 128, 256]))
+    K, N = int(rng.choice([4, 64, 100, 256])), int(rng.choice([4, 8, 64, 132, 256, 512]))
+    M = items * item_rows
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    W = (rng.standard_normal((K, N)) * 0.2).astype(np.float32)
+    bias, res = rng.standard_normal(N).astype(np.float32), rng.standard_normal((M, N)).astype(np.float32)
+    scale, shift = (1 + 0.1 * rng.standard_normal(N)).astype(np.float32), (0.1 * rng.standard_normal(N)).astype(np.float32)
+    act, with_bias, with_res = int(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    dev = [ctx.to_device(a) for a in (x, W, bias, res, scale, shift)]
+    y = ctx.empty((M, N))
+    ctx.dense_layernorm(dev[0], M, K, dev[1], N, dev[2] if with_bias else None, act, dev[3] if with_res else None, item_rows, dev[4], dev[5], y)
+    ref = orc.gemm(x, W, False, False)
+    if with_bias:
+        ref = ref + bias
+    if act:
+        ref = orc.gelu(ref)
+    if with_res:
+        ref = ref + res
+    ref = orc.layernorm(ref.reshape(items, item_rows, N), scale, shift).reshape(M, N)
+    assert_parity(y.numpy(), ref, "seed %d: items %d x %d rows, K %d, N %d, act %d bias %s residual %s" % (seed, items, item_rows, K, N, act, with_bias, with_res))
+    for t in dev + [y]:
+        t.release()
+
+
 def test_dense_fused_errors(ctx):
     from dl4s_amd import lib
     a = ctx.empty((4, 4))

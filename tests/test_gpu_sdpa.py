@@ -281,6 +281,52 @@ def test_nan_inf_placement_matches_oracle(ctx, orc, d):
     assert_parity(got, ref, "nan/inf d=%d" % d)
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_random_non_finite_values_visiting_every_tile(ctx, orc, seed):
+    """Seeded random extents, head dims, mask kinds (non-binary values among them) and layouts with NaN and infinities at
+    random places of q, k, v and the mask, every tile visited (DL4S_SDPA_STRICT, the reference's behaviour): NaN and
+    Inf at exactly the oracle's positions, everything else within the gate."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(70000 + seed)
+    B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    Lq, Lk = int(rng.integers(1, 200)), int(rng.integers(1, 200))
+    kind_name = ["none", "dense", "dense_bcast", "lengths", "causal", "causal_lengths", "scaled"][int(rng.integers(0, 7))]
+    if kind_name.startswith("causal"):
+        Lk = Lq
+    d = int(rng.choice([4, 8, 16, 24, 32, 40, 64, 64, 72, 96, 128, 10, 130]))
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    lens = rng.integers(0, Lk + 1, size=B)
+    kw, mask = {}, None
+    if kind_name == "dense":
+        mask = (rng.random((B, H, Lq, Lk)) < rng.choice([0.1, 0.5, 0.9])).astype(np.float32)
+        kw = dict(mask=mask)
+    elif kind_name == "scaled":
+        mask = ((rng.random((Lq, Lk)) < 0.5) * rng.choice([0.5, 2.0, -1.0, 1e-9])).astype(np.float32)
+        kw = dict(mask=mask)
+    elif kind_name == "dense_bcast":
+        mask = (rng.random((B, 1, 1, Lk)) < 0.5).astype(np.float32)
+        kw = dict(mask=mask)
+    elif kind_name == "lengths":
+        mask, kw = lengths_mask(lens, Lk), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    elif kind_name == "causal":
+        mask, kw = causal_mask(Lq, Lq), dict(kind=lib.MASK_CAUSAL)
+    elif kind_name == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lq)[None, None])
+        kw = dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens)
+    specials = [np.nan, np.inf, -np.inf]
+    for arr in (q, k, v):
+        if rng.random() < 0.5:
+            for _ in range(int(rng.integers(1, 4))):
+                arr[tuple(int(rng.integers(0, n)) for n in arr.shape)] = specials[int(rng.integers(0, 3))]
+    if kind_name in ("dense", "scaled") and rng.random() < 0.3:
+        mask[tuple(int(rng.integers(0, n)) for n in mask.shape)] = specials[int(rng.integers(0, 3))]
+    tm = bool(rng.integers(0, 2)) and d % 4 == 0 and d <= 128
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa(q, k, v, mask)
+    got = run_sdpa(ctx, q, k, v, strict=True, token_major=tm, **kw)
+    assert_parity(got, ref, "seed %d: B%d H%d Lq%d Lk%d d%d %s token_major=%s" % (seed, B, H, Lq, Lk, d, kind_name, tm))
+
+
 @pytest.mark.parametrize("d", [8, 10, 64, 128])
 def test_mask_penalties_at_the_top_of_the_float_range(ctx, orc, d):
     """mask * 1e9 is finite up to a mask value of 3.4e29 (the reference then subtracts about 3e38 and the row, if every key
