@@ -334,7 +334,12 @@ int dl4s_hip_stack_axis_f32(dl4s_hip_ctx *ctx, const float *const *buffers, cons
 /* ------------------------------------------------ fused layer tails (next to the path) */
 /* NN/Layer/LayerNorm.swift:62-77 on x [B, rows, D] -> result, statistics over rows*D jointly per b:
  * mean = sum/N, var = sum(x^2)/N - mean^2, y = (x - mean) * (1 / (sqrt(var) + 1e-5)) * scale + shift.
- * If residual != NULL the input is x + residual (MultiHeadAttention.swift:123-124). */
+ * If residual != NULL the input is x + residual (MultiHeadAttention.swift:123-124).
+ * The two sums are added in a tree, the reference's reduceSum adds them one after the other
+ * (Tensor/Operators/Reduce.swift:106-110).  The one-pass variance cancels when |mean| is large against the standard
+ * deviation, and there the order shows: at mean / std = 10 the two differ by 3e-4 relative, and an input whose
+ * sequential sums give a negative variance (NaN from the root) may give a small positive one here, or the other way
+ * round.  For mean / std up to about 1 - residual sums of normalised activations - the difference is below 1e-6. */
 int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *residual, const float *scale,
                            const float *shift, float *result, int64_t B, int64_t rows, int64_t D);
 /* Tensor/Operators/Unary.swift:245-247: x * (0.5 * tanh(0.5 * (1.702 * x)) + 0.5), optional bias[D] added first
