@@ -353,6 +353,32 @@ SLICES = [   # shape, index as numpy would write it (int, slice or None = whole 
 ]
 
 
+def test_subscript_known_answers_of_the_reference(ctx):
+    """The reference's own slice tests, value for value (Tests/DL4STests/EngineV2Tests.swift:235-287, testSubscriptSlice
+    and testSubscriptSliceWrite; the values 0 ... 8 are exact in fp32)."""
+    a = np.arange(9, dtype=np.float32).reshape(3, 3)
+    da = ctx.to_device(a)
+    reads = [((0, 0), (3, 2), [[0, 1], [3, 4], [6, 7]]),          # a[nil, 0 ..< 2]
+             ((0, 1), (3, 2), [[1, 2], [4, 5], [7, 8]]),          # a[nil, 1 ..< 3]
+             ((0, 0), (2, 3), [[0, 1, 2], [3, 4, 5]]),            # a[0 ..< 2]
+             ((1, 0), (2, 3), [[3, 4, 5], [6, 7, 8]])]            # a[1 ..< 3]
+    for start, extent, expected in reads:
+        dy = ctx.empty(extent)
+        ctx.subscript_read(da, (3, 3), start, extent, dy)
+        assert np.array_equal(dy.numpy(), np.array(expected, np.float32))
+        dy.release()
+    src = ctx.to_device(np.array([[0, 1], [3, 4], [6, 7]], np.float32))
+    writes = [((0, 0), [[0, 1, 0], [3, 4, 0], [6, 7, 0]]),        # result[nil, 0 ..< 2] = src1
+              ((0, 1), [[0, 0, 1], [0, 3, 4], [0, 6, 7]])]        # result[nil, 1 ..< 3] = src1
+    for start, expected in writes:
+        dr = ctx.to_device(np.zeros((3, 3), np.float32))
+        ctx.subscript_write(src, dr, (3, 3), start, (3, 2))
+        assert np.array_equal(dr.numpy(), np.array(expected, np.float32))
+        dr.release()
+    da.release()
+    src.release()
+
+
 @pytest.mark.parametrize("shape,index", SLICES)
 def test_subscript_read_and_write_match_numpy_slicing(ctx, shape, index):
     """Engine/Engine.swift:493-500 and MemoryOperatorsType.get / set(slice:) (semantics Engine/CPU/CPU.swift:137-218): one
