@@ -353,6 +353,29 @@ SLICES = [   # shape, index as numpy would write it (int, slice or None = whole 
 ]
 
 
+def test_log_of_exp_and_sigmoid_as_the_reference_tests_them(ctx):
+    """Tests/DL4STests/VecTests.swift:158-168 (testLog: log(exp(x)) = x to 1e-4 on a 10 x 10 tensor uniform in [-5, 5]) and
+    :242-258 (testSigmoid: 1 / (1 + exp(-a)) against the scalar formula to 1e-4), issued as the engine calls those
+    tensor expressions make: exp, log; negate, exp, scalar + tensor, scalar / tensor."""
+    from dl4s_amd import lib
+    rng = np.random.default_rng(158)
+    x = rng.uniform(-5, 5, (10, 10)).astype(np.float32)
+    dx, dy = ctx.to_device(x), ctx.empty((10, 10))
+    ctx.exp(dx, dy, 100)
+    ctx.log(dy, dy, 100)
+    assert np.abs(dy.numpy() - x).max() <= 1e-4
+    a = rng.standard_normal(10).astype(np.float32)
+    da, dt, one = ctx.to_device(a), ctx.empty((10,)), ctx.to_device(np.ones((), np.float32))
+    ctx.vneg(da, dt, 10)
+    ctx.exp(dt, dt, 10)
+    ctx.broadcast(lib.OP_ADD, one, (), dt, (10,), dt)
+    ctx.broadcast(lib.OP_DIV, one, (), dt, (10,), dt)
+    ref = 1.0 / (1.0 + np.exp(-a.astype(np.float64)))
+    assert np.abs(dt.numpy() - ref).max() <= 1e-4
+    for t in (dx, dy, da, dt, one):
+        t.release()
+
+
 def test_subscript_known_answers_of_the_reference(ctx):
     """The reference's own slice tests, value for value (Tests/DL4STests/EngineV2Tests.swift:235-287, testSubscriptSlice
     and testSubscriptSliceWrite; the values 0 ... 8 are exact in fp32)."""
