@@ -627,7 +627,8 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     const bool aligned8 = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                             reinterpret_cast<uintptr_t>(out)) & 7) == 0;
     const bool w96_path = dk == dv && dk > HD && dk <= W96 && ((Lq + BM - 1) / BM) * B * H >= 2ll * ctx->cu_count &&
-                          ((dk % 4 == 0 && aligned) || (dk % 2 == 0 && aligned8 && !token_major));
+                          ((dk % 4 == 0 && aligned) || (dk % 2 == 0 && aligned8 && !token_major)) &&
+                          Lk * (token_major ? H : 1) * dk * 4 < (1ll << 30);   // its 32-bit K/V offsets; beyond: the routes below
     // The 128-wide kernel on a launch that leaves CUs without their two workgroups: the key tiles of every block are dealt
     // to several workgroups, whose partial results a second kernel adds up (B4 H8 L512 d128: 73 us unsplit).  The count
     // depends on the extents only.
@@ -664,8 +665,6 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
         }
     }
     if (w96_path) {
-        DL4S_REQUIRE(Lk * (token_major ? H : 1) * dk * 4 < (1ll << 30), DL4S_HIP_EUNSUPPORTED,
-                     "sdpa: the K/V rows of one (batch, head) pair span more than 1 GiB");
         if (dk % 4 == 0) return launch_w96<4>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
         return launch_w96<2>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
     }
