@@ -210,6 +210,12 @@ def other_configs(ctx, lib, cpu, only=None):
 
         ms_calls = timed(layer_calls, 100)
         y_calls = t[5].numpy()
+        # the same calls with the mask handed over as a causal descriptor (what the host layer's model-level API does)
+        # instead of the [L, L] tensor: no tile classification launch, no mask reads
+        md_dense, md = md, ctx.mask_desc(lib.MASK_CAUSAL)
+        ms_desc = timed(layer_calls, 100)
+        same_desc = bool(np.array_equal(t[5].numpy(), y_calls))
+        md = md_dense
         ctx.graph_begin()
         layer_calls()
         graph = ctx.graph_end()
@@ -218,7 +224,8 @@ def other_configs(ctx, lib, cpu, only=None):
         same = bool(np.array_equal(t[5].numpy(), y_calls))
         res["config2_mha_B4_L512_D512_H8_causal_c_abi_calls_recorded"] = {
             "us_per_call_issued_one_by_one": ms_calls * 1e3, "us_per_call_replayed": ms_graph * 1e3, "graph_nodes": graph.nodes,
-            "replay_equals_calls_bitwise": same, "tflops": fl / ms_graph / 1e9,
+            "replay_equals_calls_bitwise": same, "us_per_call_with_causal_descriptor": ms_desc * 1e3,
+            "causal_descriptor_equals_mask_tensor_bitwise": same_desc, "tflops": fl / ms_graph / 1e9,
             "frac_mfma_peak": fl / ms_graph / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
         graph.destroy()
         for b_ in [dx, dmask, dscale, dshift] + w4 + t:
