@@ -276,10 +276,10 @@ def other_configs(ctx, lib, cpu, only=None):
                 "sample": "one batch item cut to 256 tokens (%.1f s); extrapolated whole call %.0f s" % (dt, dt * fl / fl1)}
     if want("backward"):
         # gradients of the headline workload (config 4 shapes): forward with row statistics, then dq, dk, dv; head dim 64
-        # (the 64-wide kernels), 128 and 32 (the 128- and 32-wide ones)
+        # (the 64-wide kernels), 128, 96 and 32 (the 128-, 96- and 32-wide ones)
         B, H, L = 8, 16, 2048
         rng = np.random.Generator(np.random.PCG64(1004))
-        for d in (64, 128, 32):
+        for d in (64, 128, 96, 32):
             bufs = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
             outs = [ctx.empty((B, H, L, d)) for _ in range(4)]
             st = ctx.empty((B, H, L, 2))

@@ -1179,13 +1179,18 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                            rows, token_major, (int)d);
         rc = dl4s::launch_status("sdpa_bwd_rowdot128");
         if (rc == DL4S_HIP_OK) {
+            // head dims up to 96 on 96-wide tiles (three quarters of the MFMAs), the others on 128-wide ones
+#define DL4S_BWD_WIDE(KIND_) \
+    rc = d <= 96 ? launch_bwd128<KIND_, 96>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split) \
+                 : launch_bwd128<KIND_, 128>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split)
             switch (m.kind) {
-                case DL4S_MASK_NONE: rc = launch_bwd128<DL4S_MASK_NONE>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
-                case DL4S_MASK_DENSE_F32: rc = launch_bwd128<DL4S_MASK_DENSE_F32>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
-                case DL4S_MASK_CAUSAL: rc = launch_bwd128<DL4S_MASK_CAUSAL>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
-                case DL4S_MASK_KEY_LENGTHS: rc = launch_bwd128<DL4S_MASK_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
-                default: rc = launch_bwd128<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split); break;
+                case DL4S_MASK_NONE: DL4S_BWD_WIDE(DL4S_MASK_NONE); break;
+                case DL4S_MASK_DENSE_F32: DL4S_BWD_WIDE(DL4S_MASK_DENSE_F32); break;
+                case DL4S_MASK_CAUSAL: DL4S_BWD_WIDE(DL4S_MASK_CAUSAL); break;
+                case DL4S_MASK_KEY_LENGTHS: DL4S_BWD_WIDE(DL4S_MASK_KEY_LENGTHS); break;
+                default: DL4S_BWD_WIDE(DL4S_MASK_CAUSAL_OR_KEY_LENGTHS); break;
             }
+#undef DL4S_BWD_WIDE
         }
         const int rcf = dl4s_hip_free(ctx, Dv);
         return rc != DL4S_HIP_OK ? rc : rcf;

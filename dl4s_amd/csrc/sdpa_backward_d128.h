@@ -1,12 +1,14 @@
-// Gradients of the fused attention for head dims above 64 and up to 128 (multiples of 4): the two deterministic kernels
-// of sdpa_backward.hip on 128-wide tiles.  Included by sdpa_backward.hip only.
+// Gradients of the fused attention for head dims above 64 and up to 128 (multiples of 4): the deterministic kernels of
+// sdpa_backward.hip on tiles that are W = 128 columns wide, or W = 96 for head dims up to 96.  Included by
+// sdpa_backward.hip only.
 //
-// The operand layouts follow the 128-wide forward kernel: a score product contracts d = 64*half + j over 64 MFMA steps;
-// a transposed accumulation (dQ^T, dK^T, dV^T) uses four accumulators whose rows interleave (accumulator c row i is
-// d = 4*i + c), fed by one 128-bit LDS read per key (query) and stored 128 bits at a time.  The row fragments of two
-// operands (2 x 64 registers) and up to eight accumulators leave room for one wavefront per SIMD only, so these kernels
-// run at a lower MFMA rate than the 64-wide ones; they are there so that training with such head dims stays on the
-// matrix cores at all (the plain kernels are some 40 times slower).
+// The operand layouts follow the forward kernels of the same width.  A score product contracts d = (W/2)*half + j over
+// W/2 MFMA steps.  A transposed accumulation (dQ^T, dK^T, dV^T) uses W/32 accumulators.  W = 128: their rows interleave
+// (accumulator c row i is d = 4*i + c), fed by one 128-bit LDS read per key (query) and stored 128 bits at a time.
+// W = 96: accumulator c row i is d = 32*c + i, the operand read a float at a time (sdpa_prefill_w96.h).  The row
+// fragments of two operands (2 x W/2 registers) and up to 2 x W/32 accumulators leave room for one wavefront per SIMD
+// only, so these kernels run at a lower MFMA rate than the 64-wide ones; a head dim of 96 issues three quarters of the
+// MFMAs it would on 128-wide tiles.
 #pragma once
 #include "sdpa_common.h"
 
@@ -33,12 +35,13 @@ __global__ __launch_bounds__(256) void sdpa_bwd_rowdot128(const float *__restric
     if (r < rows && (threadIdx.x & 31) == 0) D[r] = acc;
 }
 
-// 32 x 32 product tile over a 128-wide contraction: A rows from LDS (row lane % 32, columns 64*half + 4j), B from the
-// lane's 64 registers
-__device__ __forceinline__ f32x16 tile_product128(const float *Ab, const float (&br)[64]) {
+// 32 x 32 product tile over a contraction of 8 NJ columns: A rows from LDS (row lane % 32, columns (W/2)*half + 4j), B
+// from the lane's 4 NJ registers
+template <int NJ>
+__device__ __forceinline__ f32x16 tile_product_w(const float *Ab, const float (&br)[4 * NJ]) {
     f32x16 acc;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < NJ; ++j) {
         const f32x4 a0 = *reinterpret_cast<const f32x4 *>(Ab + 4 * j);
         if (j == 0) {
             const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -53,42 +56,70 @@ __device__ __forceinline__ f32x16 tile_product128(const float *Ab, const float (
     return acc;
 }
 
-// acc[c] (row i is d = 4*i + c; column = the lane's query or key) += A^T . B where A is a [32][128] LDS tile read through
-// 128-bit loads (row 8(r/4) + r%4 + 4*half, columns 4*(lane%32) ..: At already points there) and B the accumulator-layout
-// tile b
-__device__ __forceinline__ void tile_accumulate_t128(const float *At, const f32x16 &b, f32x16 (&acc)[4]) {
+// What depends on the tile width W
+template <int W> struct WideTile {
+    static constexpr int LS = W + 4;              // LDS row stride (floats): 4 mod 32
+    static constexpr int TF = BN * LS;            // floats per tile
+    static constexpr int HALF = W / 2;            // columns a half of the wavefront contracts in a score product
+    static constexpr int NJ = W / 8;              // 128-bit reads per row fragment
+    static constexpr int NC = W / 32;             // accumulators of a transposed product
+    static constexpr int PPR = W / 4;             // 128-bit pieces per tile row
+    static constexpr int NP = BN * PPR / 256;     // pieces per thread and tile: thread tid moves the pieces tid, tid + 256, ...
+    // transposed-operand base of a lane inside a [32][LS] tile (row 4*half + const)
+    static __device__ __forceinline__ int col_base(const int half, const int ln) { return (4 * half) * LS + (W == 128 ? 4 * ln : ln); }
+    // acc[c] (column = the lane's query or key) += A^T . B where A is a [32][LS] LDS tile (At points at the lane's base)
+    // and B the accumulator-layout tile b
+    static __device__ __forceinline__ void accumulate(const float *At, const f32x16 &b, f32x16 (&acc)[NC]) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const f32x4 a = *reinterpret_cast<const f32x4 *>(At + (8 * (r >> 2) + (r & 3)) * LSTR2);
-        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[r], acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[r], acc[1], 0, 0, 0);
-        acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b[r], acc[2], 0, 0, 0);
-        acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b[r], acc[3], 0, 0, 0);
-    }
-}
-
-// stores the lane's row of four interleaved transposed accumulators to p[row][0 .. hd-1], scaled
-__device__ __forceinline__ void store_row_t128(float *p, const f32x16 (&acc)[4], const float scale, const int half, const int hd) {
+        for (int r = 0; r < 16; ++r) {
+            const float *ar = At + (8 * (r >> 2) + (r & 3)) * LS;
+            if constexpr (W == 128) {
+                const f32x4 a = *reinterpret_cast<const f32x4 *>(ar);
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[r], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[r], acc[1], 0, 0, 0);
+                acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b[r], acc[2], 0, 0, 0);
+                acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b[r], acc[3], 0, 0, 0);
+            } else {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int d0 = 4 * (8 * (r >> 2) + 4 * half + (r & 3));
-        f32x4 a;
-        a.x = acc[0][r] * scale; a.y = acc[1][r] * scale; a.z = acc[2][r] * scale; a.w = acc[3][r] * scale;
-        if (d0 < hd) *reinterpret_cast<f32x4 *>(p + d0) = a;
+                for (int c = 0; c < NC; ++c) acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[32 * c], b[r], acc[c], 0, 0, 0);
+            }
+        }
     }
-}
+    // stores the lane's row of the transposed accumulators to p[0 .. hd-1], scaled
+    static __device__ __forceinline__ void store_row(float *p, const f32x16 (&acc)[NC], const float scale, const int half, const int hd) {
+        if constexpr (W == 128) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int d0 = 4 * (8 * (r >> 2) + 4 * half + (r & 3));
+                f32x4 a;
+                a.x = acc[0][r] * scale; a.y = acc[1][r] * scale; a.z = acc[2][r] * scale; a.w = acc[3][r] * scale;
+                if (d0 < hd) *reinterpret_cast<f32x4 *>(p + d0) = a;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int d0 = 32 * c + 8 * g + 4 * half;
+                    const f32x4 a = {acc[c][4 * g + 0] * scale, acc[c][4 * g + 1] * scale, acc[c][4 * g + 2] * scale, acc[c][4 * g + 3] * scale};
+                    if (d0 < hd) *reinterpret_cast<f32x4 *>(p + d0) = a;
+                }
+        }
+    }
+};
 
 // ------------------------------------------------------------------------------------------------ dQ
-template <int KIND>
+template <int KIND, int W = 128>
 __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
                                                                 const float *__restrict__ v, const float *__restrict__ dout,
                                                                 const float *__restrict__ stats, const float *__restrict__ D,
                                                                 float *__restrict__ dq, int H, int Lq, int Lk, float rT,
                                                                 MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
                                                                 int token_major, int hd) {
+    using WT = WideTile<W>;
     extern __shared__ __align__(16) float lds[];
-    float *Ks = lds;                      // [2][BN][LSTR2]
-    float *Vs = lds + 2 * TILE2_FLOATS;   // [2][BN][LSTR2]
+    float *Ks = lds;                      // [2][BN][WT::LS]
+    float *Vs = lds + 2 * WT::TF;   // [2][BN][WT::LS]
     int bh, unit;
     if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
@@ -117,14 +148,14 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
     }
     const int ntiles = (kend + BN - 1) / BN;
 
-    float qr[64], gr[64];   // the lane's Q fragment (scaled as in the forward pass) and dout fragment, columns 64*half ..
+    float qr[WT::HALF], gr[WT::HALF];   // the lane's Q fragment (scaled as in the forward pass) and dout fragment, columns (W/2)*half ..
     {
-        const float *qp = q + q_base + (long long)qic * rs + half * 64;
-        const float *gp = dout + q_base + (long long)qic * rs + half * 64;
+        const float *qp = q + q_base + (long long)qic * rs + half * WT::HALF;
+        const float *gp = dout + q_base + (long long)qic * rs + half * WT::HALF;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
+        for (int j = 0; j < WT::NJ; ++j) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f}, g = {0.f, 0.f, 0.f, 0.f};
-            if (half * 64 + 4 * j < hd) {
+            if (half * WT::HALF + 4 * j < hd) {
                 t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
                 g = *reinterpret_cast<const f32x4 *>(gp + 4 * j);
             }
@@ -137,41 +168,47 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
     const float rl_i = stats[2 * ((long long)bh * Lq + qic) + 1];
     const float D_i = D[(long long)bh * Lq + qic];
 
-    const int ld_row = tid >> 5, ld_col = (tid & 31) * 4;
+    // staging: thread tid moves the 128-bit pieces tid, tid + 256, ... of a tile (row piece / PPR, column 4 * (piece % PPR))
     const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
-    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
-    const unsigned row8_bytes = 8u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
-    f32x4 kst[4], vst[4];
+    unsigned ld_off[WT::NP];
+    int lds_off[WT::NP];
+#pragma unroll
+    for (int i = 0; i < WT::NP; ++i) {
+        const int pc = tid + 256 * i, row = pc / WT::PPR, col = (pc % WT::PPR) * 4;
+        ld_off[i] = col < hd ? (unsigned)(row * rs + col) * 4u : 0x80000000u;
+        lds_off[i] = row * WT::LS + col;
+    }
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[WT::NP], vst[WT::NP];
     auto load_tile = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int o = (int)(ld_off0 + t * tile_bytes + i * row8_bytes);
+        for (int i = 0; i < WT::NP; ++i) {
+            const int o = (int)(ld_off[i] + t * tile_bytes);
             kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o, 0, 0));
             vst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o, 0, 0));
         }
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int off = buf * TILE2_FLOATS + (i * 8 + ld_row) * LSTR2 + ld_col;
-            *reinterpret_cast<f32x4 *>(Ks + off) = kst[i];
-            *reinterpret_cast<f32x4 *>(Vs + off) = vst[i];
+        for (int i = 0; i < WT::NP; ++i) {
+            *reinterpret_cast<f32x4 *>(Ks + buf * WT::TF + lds_off[i]) = kst[i];
+            *reinterpret_cast<f32x4 *>(Vs + buf * WT::TF + lds_off[i]) = vst[i];
         }
     };
 
-    f32x16 acc[4];   // dQ^T, accumulator c row i is d = 4*i + c
+    f32x16 acc[WT::NC];   // dQ^T
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int c = 0; c < WT::NC; ++c)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
 
     if (ntiles > 0) { load_tile(0); store_tile(0); }
     __syncthreads();
 
-    const int row_lds = ln * LSTR2 + half * 64;        // row-fragment base (S^T and dP^T products)
-    const int col_lds = (4 * half) * LSTR2 + 4 * ln;   // transposed-fragment base (dQ^T product)
+    const int row_lds = ln * WT::LS + half * WT::HALF;  // row-fragment base (S^T and dP^T products)
+    const int col_lds = WT::col_base(half, ln);   // transposed-fragment base (dQ^T product)
     const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
@@ -184,18 +221,18 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
         int cls = 2;
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
         if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
-            f32x16 p = masked_scores<KIND, 16>(Ks + buf * TILE2_FLOATS + row_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+            f32x16 p = masked_scores<KIND, WT::NJ>(Ks + buf * WT::TF + row_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
 #pragma unroll
             for (int r = 0; r < 16; ++r) p[r] = fast_exp2(p[r] - m_i) * rl_i;                    // the forward pass's weights
-            const f32x16 dp = tile_product128(Vs + buf * TILE2_FLOATS + row_lds, gr);            // dP^T = V . dout^T
+            const f32x16 dp = tile_product_w<WT::NJ>(Vs + buf * WT::TF + row_lds, gr);            // dP^T = V . dout^T
 #pragma unroll
             for (int r = 0; r < 16; ++r) p[r] = p[r] * (dp[r] - D_i);                            // dS^T
-            tile_accumulate_t128(Ks + buf * TILE2_FLOATS + col_lds, p, acc);                     // dQ^T += K^T . dS^T
+            WT::accumulate(Ks + buf * WT::TF + col_lds, p, acc);                     // dQ^T += K^T . dS^T
         }
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
-    if (qi < Lq) store_row_t128(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
+    if (qi < Lq) WT::store_row(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
 }
 
 // ------------------------------------------------------------------------------------------------ dK, dV
@@ -204,7 +241,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
 // nsplit > 1 (small launches: the kernel runs one workgroup per CU): workgroup blockIdx.y of nsplit takes the query tiles
 // y, y + nsplit, ... of its key block - an assignment by tile index, whatever the mask lets the block skip - and leaves its
 // unscaled sums in part [share][dk | dv][batch*head*Lk][128]; sdpa_bwd_merge_d128 adds the shares up in order.
-template <int KIND, bool WRITE_DS = false>
+template <int KIND, bool WRITE_DS = false, int W = 128>
 __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__restrict__ q, const float *__restrict__ k,
                                                                  const float *__restrict__ v, const float *__restrict__ dout,
                                                                  const float *__restrict__ stats, const float *__restrict__ D,
@@ -213,10 +250,11 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                                                                  int total_blocks, int lpt, int token_major, int hd,
                                                                  float *__restrict__ ds = nullptr, int nsplit = 1,
                                                                  float *__restrict__ part = nullptr) {
+    using WT = WideTile<W>;
     extern __shared__ __align__(16) float lds[];
-    float *Qs = lds;                        // [2][BN][LSTR2]  q * rT * log2(e)
-    float *Gs = lds + 2 * TILE2_FLOATS;     // [2][BN][LSTR2]  dout
-    float *Ss = lds + 4 * TILE2_FLOATS;     // per query tile: [2][32] reference maxima, [2][32] 1 / row sums, [2][32] D
+    float *Qs = lds;                        // [2][BN][WT::LS]  q * rT * log2(e)
+    float *Gs = lds + 2 * WT::TF;     // [2][BN][WT::LS]  dout
+    float *Ss = lds + 4 * WT::TF;     // per query tile: [2][32] reference maxima, [2][32] 1 / row sums, [2][32] D
     int bh, unit;
     if (!work_item(nkb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
@@ -249,14 +287,14 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         if (DENSE && mask.cls) skip_cls0 = dense_query_bounds(mask, b, hh, kb * BM, wave, nqt, Lk, t_begin, wt_begin);
     }
 
-    float kr[64], vr[64];   // the lane's key and value rows (columns 64*half ..)
+    float kr[WT::HALF], vr[WT::HALF];   // the lane's key and value rows (columns (W/2)*half ..)
     {
-        const float *kp = k + kv_base + (long long)keyc * rs + half * 64;
-        const float *vp = v + kv_base + (long long)keyc * rs + half * 64;
+        const float *kp = k + kv_base + (long long)keyc * rs + half * WT::HALF;
+        const float *vp = v + kv_base + (long long)keyc * rs + half * WT::HALF;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
+        for (int j = 0; j < WT::NJ; ++j) {
             f32x4 a = {0.f, 0.f, 0.f, 0.f}, c = {0.f, 0.f, 0.f, 0.f};
-            if (half * 64 + 4 * j < hd) {
+            if (half * WT::HALF + 4 * j < hd) {
                 a = *reinterpret_cast<const f32x4 *>(kp + 4 * j);
                 c = *reinterpret_cast<const f32x4 *>(vp + 4 * j);
             }
@@ -265,18 +303,24 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         }
     }
 
-    const int ld_row = tid >> 5, ld_col = (tid & 31) * 4;
     const int q_bytes = (int)(((long long)(Lq - 1) * rs + hd) * 4);
     const __amdgpu_buffer_rsrc_t qrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(q + q_base), 0, q_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t grsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(dout + q_base), 0, q_bytes, 0x00020000);
-    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
-    const unsigned row8_bytes = 8u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
-    f32x4 qst[4], gst[4];
+    unsigned ld_off[WT::NP];   // staging pieces as in sdpa_bwd_dq_f32_d128
+    int lds_off[WT::NP];
+#pragma unroll
+    for (int i = 0; i < WT::NP; ++i) {
+        const int pc = tid + 256 * i, row = pc / WT::PPR, col = (pc % WT::PPR) * 4;
+        ld_off[i] = col < hd ? (unsigned)(row * rs + col) * 4u : 0x80000000u;
+        lds_off[i] = row * WT::LS + col;
+    }
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 qst[WT::NP], gst[WT::NP];
     float sst = 0.f;
     auto load_tile = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int o = (int)(ld_off0 + t * tile_bytes + i * row8_bytes);
+        for (int i = 0; i < WT::NP; ++i) {
+            const int o = (int)(ld_off[i] + t * tile_bytes);
             qst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(qrsrc, o, 0, 0));
             gst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(grsrc, o, 0, 0));
         }
@@ -289,8 +333,8 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int off = buf * TILE2_FLOATS + (i * 8 + ld_row) * LSTR2 + ld_col;
+        for (int i = 0; i < WT::NP; ++i) {
+            const int off = buf * WT::TF + lds_off[i];
             f32x4 s;
             s.x = (qst[i].x * rT) * LOG2E; s.y = (qst[i].y * rT) * LOG2E;
             s.z = (qst[i].z * rT) * LOG2E; s.w = (qst[i].w * rT) * LOG2E;
@@ -300,9 +344,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         if (tid < 96) Ss[(tid >> 5) * 64 + buf * 32 + (tid & 31)] = sst;
     };
 
-    f32x16 ka[4], va[4];   // dK^T and dV^T, accumulator c row i is d = 4*i + c
+    f32x16 ka[WT::NC], va[WT::NC];   // dK^T and dV^T
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int c = 0; c < WT::NC; ++c)
 #pragma unroll
         for (int i = 0; i < 16; ++i) { ka[c][i] = 0.f; va[c][i] = 0.f; }
 
@@ -311,8 +355,8 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
     if (t < nqt) { load_tile(t); store_tile(0); }
     __syncthreads();
 
-    const int row_lds = ln * LSTR2 + half * 64;
-    const int col_lds = (4 * half) * LSTR2 + 4 * ln;
+    const int row_lds = ln * WT::LS + half * WT::HALF;
+    const int col_lds = WT::col_base(half, ln);
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
@@ -340,7 +384,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         if (DENSE && cls_col) cls = cls_col[(long long)t * mask.cls_sq] & 3;
         if (!(DENSE && cls == 1 && skip_cls0 && dense_block_open(skip_cls0 + (long long)t * mask.cls_sq, mask.cls_sk, t, (Lk + 31) >> 5))) {
             // S[query, key] in the base-2 domain: rows = the tile's queries 8(r/4) + 4*half + r%4, column = the lane's key
-            f32x16 p = tile_product128(Qs + buf * TILE2_FLOATS + row_lds, kr);
+            f32x16 p = tile_product_w<WT::NJ>(Qs + buf * WT::TF + row_lds, kr);
             if (DENSE) {
                 if (cls == 1) {
 #pragma unroll
@@ -373,8 +417,8 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                 p[4 * g + 2] = fast_exp2(p[4 * g + 2] - m4.z) * r4.z;
                 p[4 * g + 3] = fast_exp2(p[4 * g + 3] - m4.w) * r4.w;
             }
-            tile_accumulate_t128(Gs + buf * TILE2_FLOATS + col_lds, p, va);                      // dV^T += dout^T . P
-            const f32x16 dp = tile_product128(Gs + buf * TILE2_FLOATS + row_lds, vr);            // dP = dout . V^T
+            WT::accumulate(Gs + buf * WT::TF + col_lds, p, va);                      // dV^T += dout^T . P
+            const f32x16 dp = tile_product_w<WT::NJ>(Gs + buf * WT::TF + row_lds, vr);            // dP = dout . V^T
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const f32x4 d4 = *reinterpret_cast<const f32x4 *>(st + 128 + 8 * g);
@@ -392,7 +436,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 0);
                 }
             }
-            tile_accumulate_t128(Qs + buf * TILE2_FLOATS + col_lds, p, ka);                      // dK^T += Q~^T . dS
+            WT::accumulate(Qs + buf * WT::TF + col_lds, p, ka);                      // dK^T += Q~^T . dS
         }
         if (more) store_tile(buf ^ 1);
         __syncthreads();
@@ -401,14 +445,14 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         if (key < Lk) {
             const long long rows = (long long)(total_blocks / nkb) * Lk;
             float *pp = part + (((long long)sp * 2) * rows + (long long)bh * Lk + key) * HD2;
-            store_row_t128(pp, ka, 1.0f, half, HD2);
-            store_row_t128(pp + rows * HD2, va, 1.0f, half, HD2);
+            WT::store_row(pp, ka, 1.0f, half, W);
+            WT::store_row(pp + rows * HD2, va, 1.0f, half, W);
         }
         return;
     }
     if (key < Lk) {
-        store_row_t128(dv + kv_base + (long long)key * rs, va, 1.0f, half, hd);
-        store_row_t128(dk + kv_base + (long long)key * rs, ka, 0.69314718055994530942f, half, hd);   // Q~ carries log2(e)
+        WT::store_row(dv + kv_base + (long long)key * rs, va, 1.0f, half, hd);
+        WT::store_row(dk + kv_base + (long long)key * rs, ka, 0.69314718055994530942f, half, hd);   // Q~ carries log2(e)
     }
 }
 
@@ -434,7 +478,7 @@ __global__ __launch_bounds__(256) void sdpa_bwd_merge_d128(const float *__restri
 // ------------------------------------------------------------------------------------------------ dQ from stored dS
 // dQ = (dS . K) * rT with dS read from the scratch tensor sdpa_bwd_dkv_f32_d128<KIND, true> wrote; see
 // sdpa_bwd_dq_from_ds_f32_d64.  Four accumulators and one dS tile in flight: three wavefronts per SIMD instead of one.
-template <int KIND>
+template <int KIND, int W = 128>
 __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const float *__restrict__ k, const float *__restrict__ ds,
                                                                         float *__restrict__ dq, int H, int Lq, int Lk, float rT,
                                                                         MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
@@ -442,8 +486,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
                                                                         float *__restrict__ part = nullptr) {
     // nsplit > 1: workgroup blockIdx.y takes the key tiles y, y + nsplit, ... and leaves its unscaled sums in
     // part [share][batch*head*Lq][128] for sdpa_bwd_merge_d128
+    using WT = WideTile<W>;
     extern __shared__ __align__(16) float lds[];
-    float *Ks = lds;                      // [2][BN][LSTR2]
+    float *Ks = lds;                      // [2][BN][WT::LS]
     int bh, unit;
     if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
@@ -471,20 +516,26 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
     }
     const int ntiles = (kend + BN - 1) / BN;
 
-    const int ld_row = tid >> 5, ld_col = (tid & 31) * 4;
     const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
-    const unsigned ld_off0 = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
-    const unsigned row8_bytes = 8u * rs * 4u, tile_bytes = (unsigned)BN * rs * 4u;
-    f32x4 kst[4];
+    unsigned ld_off[WT::NP];   // staging pieces as in sdpa_bwd_dq_f32_d128
+    int lds_off[WT::NP];
+#pragma unroll
+    for (int i = 0; i < WT::NP; ++i) {
+        const int pc = tid + 256 * i, row = pc / WT::PPR, col = (pc % WT::PPR) * 4;
+        ld_off[i] = col < hd ? (unsigned)(row * rs + col) * 4u : 0x80000000u;
+        lds_off[i] = row * WT::LS + col;
+    }
+    const unsigned tile_bytes = (unsigned)BN * rs * 4u;
+    f32x4 kst[WT::NP];
     auto load_tile = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, (int)(ld_off0 + t * tile_bytes + i * row8_bytes), 0, 0));
+        for (int i = 0; i < WT::NP; ++i)
+            kst[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, (int)(ld_off[i] + t * tile_bytes), 0, 0));
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4 *>(Ks + buf * TILE2_FLOATS + (i * 8 + ld_row) * LSTR2 + ld_col) = kst[i];
+        for (int i = 0; i < WT::NP; ++i) *reinterpret_cast<f32x4 *>(Ks + buf * WT::TF + lds_off[i]) = kst[i];
     };
 
     const int Lqp = (Lq + 31) & ~31, Lkp = (Lk + 31) & ~31;
@@ -507,9 +558,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
             dsn[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dsrsrc, (int)ds_voff, (int)(base + (unsigned)(8 * (r >> 2) + (r & 3)) * ds_row), 2));
     };
 
-    f32x16 acc[4];   // dQ^T, accumulator c row i is d = 4*i + c
+    f32x16 acc[WT::NC];   // dQ^T
 #pragma unroll
-    for (int c = 0; c < 4; ++c)
+    for (int c = 0; c < WT::NC; ++c)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
 #pragma unroll
@@ -522,7 +573,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
         if (visited(sp)) load_ds(sp);
     }
     __syncthreads();
-    const int col_lds = (4 * half) * LSTR2 + 4 * ln;
+    const int col_lds = WT::col_base(half, ln);
     for (int t = sp, buf = 0; t < ntiles; t += nsplit, buf ^= 1) {
         const bool more = (t + nsplit < ntiles);
         const bool now = visited(t);
@@ -531,30 +582,32 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
             load_tile(t + nsplit);
             if (visited(t + nsplit)) load_ds(t + nsplit);
         }
-        if (now) tile_accumulate_t128(Ks + buf * TILE2_FLOATS + col_lds, p, acc);               // dQ^T += K^T . dS^T
+        if (now) WT::accumulate(Ks + buf * WT::TF + col_lds, p, acc);               // dQ^T += K^T . dS^T
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
     if (part) {
-        if (qi < Lq) store_row_t128(part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * HD2, acc, 1.0f, half, HD2);
+        if (qi < Lq) WT::store_row(part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * HD2, acc, 1.0f, half, W);
         return;
     }
-    if (qi < Lq) store_row_t128(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
+    if (qi < Lq) WT::store_row(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
 }
 
-template <int KIND>
+template <int KIND, int W = 128>
 int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *dout, const float *stats,
                   const float *D, float *dq, float *dk, float *dv, int B, int H, int Lq, int Lk, float rT, const MaskArgs &m,
                   int strict, int token_major, int hd, long long ds_max_bytes, int no_split = 0) {
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
-    const size_t lds_dq = 4 * TILE2_FLOATS * sizeof(float);
-    const size_t lds_dkv = (4 * TILE2_FLOATS + 192) * sizeof(float);
-    if (dl4s::lds_limit_pending(ctx, dl4s::LDS_BWD_D128, KIND)) {
-        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_f32_d128<KIND>),
+    using WT = WideTile<W>;
+    const size_t lds_dq = 4 * WT::TF * sizeof(float);
+    const size_t lds_dkv = (4 * WT::TF + 192) * sizeof(float);
+    // (the 96-wide tiles stay within the default 64 KiB of dynamic LDS)
+    if (lds_dkv > 65536 && dl4s::lds_limit_pending(ctx, dl4s::LDS_BWD_D128, KIND)) {
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dq_f32_d128<KIND, W>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dq));
-        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND>),
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND, false, W>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
-        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND, true>),
+        DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_bwd_dkv_f32_d128<KIND, true, W>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv));
         dl4s::lds_limit_done(ctx, dl4s::LDS_BWD_D128, KIND);
     }
@@ -587,7 +640,7 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
             float *pq = sq > 1 ? static_cast<float *>(pv) + (sk > 1 ? part_k : 0) : nullptr;
             int lpt = (uneven && nkb >= 2) ? 1 : 0;
             if (lpt && total_k <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
-            hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d128<KIND, true>), dim3((unsigned)((total_k + 7) / 8 * 8), (unsigned)sk), dim3(256), lds_dkv,
+            hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d128<KIND, true, W>), dim3((unsigned)((total_k + 7) / 8 * 8), (unsigned)sk), dim3(256), lds_dkv,
                                ctx->stream, q, k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total_k, lpt, token_major, hd,
                                ds, (int)sk, pk);
             int rc = dl4s::launch_status("sdpa_bwd_dkv_f32_d128");
@@ -602,8 +655,8 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
             if (rc == DL4S_HIP_OK) {
                 lpt = (uneven && nqb >= 2) ? 1 : 0;
                 if (lpt && total_q <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
-                hipLaunchKernelGGL(sdpa_bwd_dq_from_ds_f32_d128<KIND>, dim3((unsigned)((total_q + 7) / 8 * 8), (unsigned)sq), dim3(256),
-                                   2 * TILE2_FLOATS * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q,
+                hipLaunchKernelGGL((sdpa_bwd_dq_from_ds_f32_d128<KIND, W>), dim3((unsigned)((total_q + 7) / 8 * 8), (unsigned)sq), dim3(256),
+                                   2 * WT::TF * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q,
                                    lpt, token_major, hd, (int)sq, pq);
                 rc = dl4s::launch_status("sdpa_bwd_dq_from_ds_f32_d128");
                 if (rc == DL4S_HIP_OK && pq) {
@@ -623,7 +676,7 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
         int lpt = (uneven && nqb >= 2) ? 1 : 0;
         if (lpt && total <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
-        hipLaunchKernelGGL(sdpa_bwd_dq_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq, ctx->stream, q, k,
+        hipLaunchKernelGGL((sdpa_bwd_dq_f32_d128<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dq, ctx->stream, q, k,
                            v, dout, stats, D, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, hd);
         const int rc = dl4s::launch_status("sdpa_bwd_dq_f32_d128");
         if (rc != DL4S_HIP_OK) return rc;
@@ -634,7 +687,7 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
         DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa backward: %lld workgroups exceed the grid limit", total);
         int lpt = (uneven && nkb >= 2) ? 1 : 0;
         if (lpt && total <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
-        hipLaunchKernelGGL(sdpa_bwd_dkv_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
+        hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d128<KIND, false, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
                            k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total, lpt, token_major, hd);
         return dl4s::launch_status("sdpa_bwd_dkv_f32_d128");
     }
