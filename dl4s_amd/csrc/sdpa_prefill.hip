@@ -622,19 +622,20 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     const int strict = (flags & DL4S_SDPA_STRICT) ? 1 : 0;
     const int token_major = (flags & DL4S_SDPA_TOKEN_MAJOR) ? 1 : 0;
     const int no_split = (flags & DL4S_SDPA_NO_KEY_SPLIT) ? 1 : 0;
-    // head dims above 64 up to 96 on launches that fill the GPU without a key split: the 96-wide kernel, which also takes
+    // head dims above 64 up to 96: the 96-wide kernel, which on launches that fill the GPU without a key split also takes
     // even head dims that are not a multiple of 4 as they are (rows on the 8-byte grid)
     const bool aligned8 = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
                             reinterpret_cast<uintptr_t>(out)) & 7) == 0;
-    const bool w96_path = dk == dv && dk > HD && dk <= W96 && ((Lq + BM - 1) / BM) * B * H >= 2ll * ctx->cu_count &&
-                          ((dk % 4 == 0 && aligned) || (dk % 2 == 0 && aligned8 && !token_major)) &&
+    const bool w96_path = dk == dv && dk > HD && dk <= W96 &&
+                          ((dk % 4 == 0 && aligned) ||
+                           (dk % 2 == 0 && aligned8 && !token_major && ((Lq + BM - 1) / BM) * B * H >= 2ll * ctx->cu_count)) &&
                           Lk * (token_major ? H : 1) * dk * 4 < (1ll << 30);   // its 32-bit K/V offsets; beyond: the routes below
     // The 128-wide kernel on a launch that leaves CUs without their two workgroups: the key tiles of every block are dealt
     // to several workgroups, whose partial results a second kernel adds up (B4 H8 L512 d128: 73 us unsplit).  The count
     // depends on the extents only.
     int nsplit128 = 1;
     size_t part_bytes = 0;
-    if (mfma128_path && !no_split) {
+    if ((mfma128_path || (w96_path && dk % 4 == 0)) && !no_split) {
         const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
         if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
             long long want = (2ll * ctx->cu_count + blocks - 1) / blocks;
@@ -665,7 +666,9 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
         }
     }
     if (w96_path) {
-        if (dk % 4 == 0) return launch_w96<4>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+        if (dk % 4 == 0)
+            return launch_w96<4>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128,
+                                 static_cast<float *>(part128));
         return launch_w96<2>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
     }
     if (mfma128_path) {

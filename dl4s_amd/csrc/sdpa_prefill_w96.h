@@ -1,4 +1,4 @@
-// Fused attention forward for head dims above 64 and up to 96 on large launches: the scheme of sdpa_prefill_f32_d128
+// Fused attention forward for head dims above 64 and up to 96: the scheme of sdpa_prefill_f32_d128
 // (sdpa_prefill_d128.h) on tiles that are 96 columns wide, and with a second staging form for head dims that are even
 // but not a multiple of 4 (rows on an 8-byte grid: 64-bit loads and stores), which the other MFMA kernels only take
 // through zero-padded copies of the operands.  Included by sdpa_prefill.hip only.
@@ -13,8 +13,9 @@
 // quarters, and one of 70 runs without the four streaming copies.  One workgroup = 4 wavefronts = 128 queries of one
 // (batch, head) pair, K/V in double-buffered LDS tiles of 32 keys on a 100-float row stride (2 x 2 x 32 x 100 floats =
 // 50 KiB).  Mask kinds, tile skipping, the work order, the token-major layout (head dims that are multiples of 4) and
-// the row statistics are those of the other forward kernels.  No key split over workgroups: small launches stay with
-// the 128-wide kernel.
+// the row statistics are those of the other forward kernels.  Small launches (head dims that are multiples of 4) are
+// split over the keys across workgroups like the 128-wide kernel: share y of n takes the key tiles y, y + n, ... and
+// sdpa_prefill_merge_d128 adds the shares up.
 #pragma once
 #include "sdpa_common.h"
 
@@ -29,12 +30,15 @@ template <int KIND, int VEC>
 __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__restrict__ q, const float *__restrict__ k,
                                                                 const float *__restrict__ v, float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict, int nqb, int total_blocks,
-                                                                int lpt, int token_major, float *__restrict__ stats, int hd) {
+                                                                int lpt, int token_major, float *__restrict__ stats, int hd,
+                                                                int nsplit, float *__restrict__ part) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                       // [2][BN][LSTR96]
     float *Vs = lds + 2 * TILE96_FLOATS;   // [2][BN][LSTR96]
     int bh, unit;
-    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    // key split with blocks of different length: odd shares walk the block order backwards (see sdpa_prefill_f32_d128)
+    const int blk = ((lpt & 1) && (blockIdx.y & 1)) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    if (!dl4s_work_order::work_item_at(blk, nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -132,7 +136,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
         for (int i = 0; i < 16; ++i) o[c][i] = 0.f;
     float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
 
-    if (ntiles > 0) { load_tile(0); store_tile(0); }
+    const int sp = blockIdx.y;     // this workgroup's share of the key tiles: sp, sp + nsplit, ...
+    if (sp < ntiles) { load_tile(sp); store_tile(0); }
     __syncthreads();
 
     const int k_lds = ln * LSTR96 + half * (W96 / 2);   // K fragment base: row ln, columns 48*half ..
@@ -141,10 +146,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
 
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        const bool more = (t + 1 < ntiles);
-        if (more) load_tile(t + 1);
+    for (int t = sp, buf = 0; t < ntiles; t += nsplit, buf ^= 1) {
+        const bool more = (t + nsplit < ntiles);
+        if (more) load_tile(t + nsplit);
         const int k0 = t * BN;
         int cls = 2;
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
@@ -190,6 +194,20 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
 
     // ---- normalise and store
     const float l_tot = l_run + xor32(l_run);
+    if (part) {   // this share's weighted sums as they are, with their reference maximum and row sum
+        if (qi < Lq) {
+            float *pp = part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * PART2_STRIDE;
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 a = {o[c][4 * g + 0], o[c][4 * g + 1], o[c][4 * g + 2], o[c][4 * g + 3]};
+                    *reinterpret_cast<f32x4 *>(pp + 32 * c + 8 * g + 4 * half) = a;
+                }
+            if (half == 0) { pp[HD2] = m_run; pp[HD2 + 1] = l_tot; }
+        }
+        return;
+    }
     const float inv = 1.0f / l_tot;
     if (stats && half == 0 && qi < Lq) {
         stats[2 * ((long long)bh * Lq + qi)] = m_use;
@@ -216,7 +234,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
 
 template <int KIND, int VEC>
 int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
-                    float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+                    float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit, float *part) {
     const int nqb = (Lq + BM - 1) / BM;
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
@@ -224,20 +242,26 @@ int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const flo
     int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
     if (lpt && total <= 3ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
     const size_t lds_bytes = 4 * TILE96_FLOATS * sizeof(float);   // 50 KiB: within the default limit
-    hipLaunchKernelGGL((sdpa_prefill_f32_w96<KIND, VEC>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_bytes, ctx->stream, q, k,
-                       v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd);
-    return dl4s::launch_status("sdpa_prefill_f32_w96");
+    if (nsplit <= 1 || !part || VEC != 4) { nsplit = 1; part = nullptr; }
+    hipLaunchKernelGGL((sdpa_prefill_f32_w96<KIND, VEC>), dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
+                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part);
+    const int st = dl4s::launch_status("sdpa_prefill_f32_w96");
+    if (st != DL4S_HIP_OK || nsplit == 1) return st;
+    const long long rows = (long long)B * H * Lq;
+    hipLaunchKernelGGL(sdpa_prefill_merge_d128, dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, ctx->stream, part, out, stats, nsplit, rows,
+                       H, Lq, hd, token_major);
+    return dl4s::launch_status("sdpa_prefill_merge_d128");
 }
 
 template <int VEC>
 int launch_w96(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk, float rT,
-               const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+               const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit = 1, float *part = nullptr) {
     switch (m.kind) {
-        case DL4S_MASK_NONE: return launch_w96_kind<DL4S_MASK_NONE, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        case DL4S_MASK_DENSE_F32: return launch_w96_kind<DL4S_MASK_DENSE_F32, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        case DL4S_MASK_CAUSAL: return launch_w96_kind<DL4S_MASK_CAUSAL, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        case DL4S_MASK_KEY_LENGTHS: return launch_w96_kind<DL4S_MASK_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        default: return launch_w96_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_NONE: return launch_w96_kind<DL4S_MASK_NONE, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_DENSE_F32: return launch_w96_kind<DL4S_MASK_DENSE_F32, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_CAUSAL: return launch_w96_kind<DL4S_MASK_CAUSAL, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_KEY_LENGTHS: return launch_w96_kind<DL4S_MASK_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        default: return launch_w96_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
     }
 }
 
