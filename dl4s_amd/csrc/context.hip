@@ -1,6 +1,9 @@
 // Context, pooled allocator, copies and the stream timer of libdl4s_hip.so.
 #include "common.h"
 
+#include <algorithm>
+#include <functional>
+
 #include <cstdlib>
 #include <cstring>
 
@@ -346,6 +349,27 @@ int dl4s_hip_get_size(dl4s_hip_ctx *ctx, const void *ptr, size_t *out_bytes) {
     --it;
     DL4S_REQUIRE(a < it->first + it->second, DL4S_HIP_EINVALID_ARG, "dl4s_hip_get_size: %p is not inside a live allocation", ptr);
     *out_bytes = it->first + it->second - a;
+    return DL4S_HIP_OK;
+}
+
+int dl4s_hip_pool_trim(dl4s_hip_ctx *ctx, size_t keep_bytes) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_NOT_WHILE_CAPTURING(ctx);
+    DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    std::lock_guard<std::mutex> g(ctx->mu);
+    // the pool is keyed by block size: walk the sizes from the largest down
+    std::vector<size_t> sizes;
+    for (const auto &kv : ctx->pool)
+        if (!kv.second.empty()) sizes.push_back(kv.first);
+    std::sort(sizes.begin(), sizes.end(), std::greater<size_t>());
+    for (size_t sz : sizes) {
+        std::vector<void *> &blocks = ctx->pool[sz];
+        while (!blocks.empty() && ctx->bytes_pooled > keep_bytes) {
+            DL4S_HIP_TRY(hipFree(blocks.back()));
+            blocks.pop_back();
+            ctx->bytes_pooled -= sz;
+        }
+    }
     return DL4S_HIP_OK;
 }
 

@@ -168,6 +168,9 @@ class Context:
         _check(self.lib.dl4s_hip_mem_stats(self.handle, C.byref(a), C.byref(b)))
         return a.value, b.value
 
+    def pool_trim(self, keep_bytes=0):
+        _check(self.lib.dl4s_hip_pool_trim(self.handle, C.c_size_t(keep_bytes)))
+
     # ---- fused attention
     def mask_desc(self, kind=MASK_NONE, dense=None, lengths=None):
         """dense: DeviceBuffer with .shape of rank <= 4; lengths: DeviceBuffer of int32 [B]."""

@@ -107,6 +107,12 @@ int dl4s_hip_set_pointee_f32(dl4s_hip_ctx *ctx, float *dst_dev, float value);
 int dl4s_hip_get_size(dl4s_hip_ctx *ctx, const void *ptr, size_t *out_bytes);
 /* Bytes currently handed out / held by the pool (leak checks; Engine/CPU/CPU.swift:38-44 traces the same). */
 int dl4s_hip_mem_stats(dl4s_hip_ctx *ctx, size_t *out_bytes_in_use, size_t *out_bytes_pooled);
+/* Returns pooled blocks to the driver, largest first, until at most keep_bytes stay pooled (0: all of them).  The pool
+ * keeps every freed block for the next allocation of its size and otherwise lets go only when an allocation fails; a
+ * caller that is done with a phase of large temporaries (the attention gradients take B*H*Lq*Lk floats) gives the
+ * memory back with this.  Waits for the stream (a pooled block may still be in use by work in flight); refused while
+ * a call sequence is being recorded.  No counterpart in the reference, whose buffers go back to malloc one by one. */
+int dl4s_hip_pool_trim(dl4s_hip_ctx *ctx, size_t keep_bytes);
 
 /* ------------------------------------------------------------ fused attention entry */
 /* Mask descriptor.  The reference takes a dense float tensor (1 = blocked, 0 = keep, any value is

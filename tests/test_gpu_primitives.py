@@ -25,6 +25,24 @@ def rnd(*shape):
     return RNG.standard_normal(shape).astype(np.float32)
 
 
+def test_pool_trim_returns_pooled_blocks_largest_first(ctx):
+    a, b, c = ctx.empty((1 << 20,)), ctx.empty((1 << 16,)), ctx.empty((1 << 10,))
+    ctx.fill(1.0, a, 1 << 20)
+    for t in (a, b, c):
+        t.release()
+    _, pooled0 = ctx.mem_stats()
+    assert pooled0 >= (4 << 20) + (4 << 16) + (4 << 10)
+    ctx.pool_trim(pooled0 - (4 << 20))            # the 4 MiB block goes first
+    used, pooled1 = ctx.mem_stats()
+    assert pooled1 <= pooled0 - (4 << 20)
+    ctx.pool_trim(0)
+    assert ctx.mem_stats() == (used, 0)
+    d = ctx.empty((1 << 20,))                     # the pool is empty: a fresh block, and everything still works
+    ctx.fill(2.0, d, 1 << 20)
+    assert d.numpy()[-1] == 2.0
+    d.release()
+
+
 def test_memory_roundtrip_views_and_stats(ctx):
     from dl4s_amd import lib
     import ctypes as C
