@@ -542,3 +542,44 @@ def test_gradients_on_the_128_wide_kernels(ctx, orc, d, mask_kind):
             assert np.array_equal(a, b_)
     for a, b_ in zip(run_fwd_bwd(ctx, q, k, v, dout, token_major=True, **kw), (out, stats, dq, dk, dv)):
         assert np.array_equal(a, b_)
+
+
+@pytest.mark.parametrize("L,d,token_major", [(16384, 64, False), (32768, 64, False), (16384, 32, False), (16384, 128, False),
+                                             (16384, 96, False), (8192, 64, True)])
+def test_long_sequences_on_sampled_rows_and_columns(ctx, L, d, token_major):
+    """Causal attention and its gradients at sequence lengths the oracle cannot finish: out and dq on sampled query rows,
+    dk and dv on sampled key columns, against an fp64 model written from the definition (softmax(q.k^T/sqrt(d)).v and the
+    chain rule), the statistics of every row recomputed in fp64 in chunks.  L = 32768 is past the size at which the
+    gradients keep their dS tiles (one (batch, head) slab would reach 4 GiB) and runs the self-contained kernels."""
+    rng = np.random.default_rng(L + d)
+    B, H = 1, 2
+    q, k, v, dout = [rand(rng, B, H, L, d, scale=0.5) for _ in range(4)]
+    from dl4s_amd import lib
+    out, _, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, kind=lib.MASK_CAUSAL, token_major=token_major)
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+    for h in (0, H - 1):
+        Q, K, V, DO, O = [x[0, h].astype(np.float64) for x in (q, k, v, dout, out)]
+        rows = sorted(set([0, 1, 31, 32, 127, 128, L // 2 - 1, L // 2, L - 129, L - 2, L - 1] + [int(i) for i in rng.integers(0, L, 6)]))
+        for i in rows:
+            s = (K[:i + 1] @ Q[i]) * rT
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            o_i = p @ V[:i + 1]
+            ds = p * (V[:i + 1] @ DO[i] - DO[i] @ o_i)
+            np.testing.assert_allclose(out[0, h, i], o_i, rtol=1e-4, atol=2e-5, err_msg="out row %d" % i)
+            np.testing.assert_allclose(dq[0, h, i], (ds @ K[:i + 1]) * rT, rtol=1e-4, atol=2e-5, err_msg="dq row %d" % i)
+        cols = np.array(sorted(set([0, 31, 32, L // 2, L - 33, L - 1] + [int(j) for j in rng.integers(0, L, 3)])))
+        dk_c, dv_c = np.zeros((len(cols), d)), np.zeros((len(cols), d))
+        row_dot = (DO * O).sum(1)
+        for r0 in range(0, L, 2048):
+            r1 = min(L, r0 + 2048)
+            ii = np.arange(r0, r1)[:, None]
+            S = np.where(np.arange(r1)[None, :] <= ii, (Q[r0:r1] @ K[:r1].T) * rT, -np.inf)
+            m = S.max(1, keepdims=True)
+            l = np.exp(S - m).sum(1, keepdims=True)
+            P = np.where(cols[None, :] <= ii, np.exp((Q[r0:r1] @ K[cols].T) * rT - m) / l, 0.0)
+            dS = P * (DO[r0:r1] @ V[cols].T - row_dot[r0:r1, None])
+            dv_c += P.T @ DO[r0:r1]
+            dk_c += dS.T @ Q[r0:r1] * rT
+        np.testing.assert_allclose(dk[0, h][cols], dk_c, rtol=1e-4, atol=1e-4)
+        np.testing.assert_allclose(dv[0, h][cols], dv_c, rtol=1e-4, atol=1e-4)
