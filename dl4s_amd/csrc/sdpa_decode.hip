@@ -4,7 +4,8 @@
 // 128-bit load per lane, so every load instruction of a wavefront covers four whole rows (1 KiB,
 // contiguous), and a wavefront keeps the 8 K loads and 8 V loads of a 32-key block in flight together.
 // The dot product is reduced inside the 16-lane group with DPP adds.  Rows of 32 and 128 floats use groups of 8 and
-// 32 lanes in the same way (64 and 16 keys per iteration); other head dims run the next wider form with idle lanes.  With 16 wavefronts resident per CU
+// 32 lanes in the same way (64 and 16 keys per iteration); other head dims run the next wider form with idle lanes, and a
+// head dim that is no multiple of 4 (rows off the 16-byte grid) reads 64 or 32 bits per load.  With 16 wavefronts resident per CU
 // that is ample memory-level parallelism to keep HBM busy.
 //
 // Work split: grid = (nsplit, B*H).  When B*H alone fills the GPU (the decode benchmark: 256 pairs on 256
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
                                                                    float *__restrict__ out, float *part, int T, int Tcap,
                                                                    int pos, float rT, int nsplit, int chunk, int d, int H,
                                                                    const int *__restrict__ lengths,
-                                                                   const int *__restrict__ pos_dev = nullptr) {
+                                                                   const int *__restrict__ pos_dev = nullptr, int vec = 4) {
     constexpr int D = 4 * LPR, G = 64 / LPR, KB = 8 * G, PSTR = pstr(D);
     __shared__ float sm_o[NW][D];
     __shared__ float sm_m[NW], sm_l[NW];
@@ -86,6 +87,41 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
     const int wave = tid >> 6, lane = tid & 63;
     const int g = lane / LPR, c = lane % LPR;
     const bool col_ok = FULL || 4 * c < d;    // FULL: d = 4 * LPR, every lane has its piece of the row; else lanes beyond the row hold zeros
+    // vec < 4: rows that are no whole number of 16-byte pieces, or operands that are not 16-byte aligned - a lane reads its
+    // (up to) four columns as two 64-bit halves (even row length, 8-byte aligned operands) or one float at a time; the
+    // wavefront's loads still cover whole contiguous rows.
+    const bool vec4 = FULL || vec == 4;
+    const int ncol = FULL ? 4 : d - 4 * c;
+    auto load4 = [&](const float *p) -> f32x4 {
+        f32x4 r = {0.f, 0.f, 0.f, 0.f};
+        if (vec4) {
+            if (col_ok) r = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+        } else if (vec == 2) {      // even row length: ncol is 2 or at least 4 wherever it is positive
+            typedef float f32x2 __attribute__((ext_vector_type(2)));
+            if (ncol > 0) { const f32x2 t = __builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(p)); r.x = t.x; r.y = t.y; }
+            if (ncol > 2) { const f32x2 t = __builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(p + 2)); r.z = t.x; r.w = t.y; }
+        } else {
+            if (ncol > 0) r.x = __builtin_nontemporal_load(p);
+            if (ncol > 1) r.y = __builtin_nontemporal_load(p + 1);
+            if (ncol > 2) r.z = __builtin_nontemporal_load(p + 2);
+            if (ncol > 3) r.w = __builtin_nontemporal_load(p + 3);
+        }
+        return r;
+    };
+    auto store4 = [&](float *p, const f32x4 r) {
+        if (vec4) {
+            if (col_ok) *reinterpret_cast<f32x4 *>(p) = r;
+        } else if (vec == 2) {
+            typedef float f32x2 __attribute__((ext_vector_type(2)));
+            if (ncol > 0) *reinterpret_cast<f32x2 *>(p) = f32x2{r.x, r.y};
+            if (ncol > 2) *reinterpret_cast<f32x2 *>(p + 2) = f32x2{r.z, r.w};
+        } else {
+            if (ncol > 0) p[0] = r.x;
+            if (ncol > 1) p[1] = r.y;
+            if (ncol > 2) p[2] = r.z;
+            if (ncol > 3) p[3] = r.w;
+        }
+    };
 
     bool all_blocked = false;                 // a length of zero: every key takes the penalty
     if (lengths) {
@@ -94,8 +130,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         else if (len < T) T = len;
     }
 
-    f32x4 qv = {0.f, 0.f, 0.f, 0.f};
-    if (col_ok) qv = *reinterpret_cast<const f32x4 *>(q + (long long)bh * d + 4 * c);
+    f32x4 qv = load4(q + (long long)bh * d + 4 * c);
     qv.x *= rT; qv.y *= rT; qv.z *= rT; qv.w *= rT;
 
     const long long base = (long long)bh * Tcap * d + 4 * c;
@@ -110,9 +145,9 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         kn_row = k_new + (long long)bh * d + 4 * c;
         vn_row = v_new + (long long)bh * d + 4 * c;
         const bool mine = (pos >= c0 && pos < c1) || (pos >= T && split == 0);
-        if (mine && wave == 0 && g == 0 && col_ok) {
-            *reinterpret_cast<f32x4 *>(kcache + base + (long long)pos * d) = *reinterpret_cast<const f32x4 *>(kn_row);
-            *reinterpret_cast<f32x4 *>(vcache + base + (long long)pos * d) = *reinterpret_cast<const f32x4 *>(vn_row);
+        if (mine && wave == 0 && g == 0) {
+            store4(kcache + base + (long long)pos * d, load4(kn_row));
+            store4(vcache + base + (long long)pos * d, load4(vn_row));
         }
     }
 
@@ -134,8 +169,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
             const int kc = key < T ? key : T - 1;
             const float *kp = kcache + base + (long long)kc * d;
             if (APPEND) kp = (kc == pos) ? kn_row : kp;
-            kk[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (col_ok) kk[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(kp));
+            kk[i] = load4(kp);
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -143,8 +177,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
             const int kc = key < T ? key : T - 1;
             const float *vp = vcache + base + (long long)kc * d;
             if (APPEND) vp = (kc == pos) ? vn_row : vp;
-            vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (col_ok) vv[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(vp));
+            vv[i] = load4(vp);
         }
         if (kb + KB > c1) {     // the range's last block: lanes past its end re-read row T-1 and must add nothing, not 0 * Inf
 #pragma unroll
@@ -252,23 +285,32 @@ __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restr
 // Row widths the kernel is instantiated for: 32, 64, 128 floats (8, 16, 32 lanes per row).
 inline int lanes_per_row(int64_t d) { return d <= 32 ? 8 : (d <= 64 ? 16 : 32); }
 
+// 4 when every cache row starts on a 16-byte boundary (the row length a multiple of 4 floats, every operand aligned): a lane
+// reads its piece of a row with one 128-bit load.  2 for an even row length and 8-byte aligned operands (two 64-bit loads),
+// 1 otherwise (one float at a time).
+inline int row_vector_width(int64_t d, const void *q, const void *kcache, const void *vcache, const void *k_new, const void *v_new) {
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kcache) | reinterpret_cast<uintptr_t>(vcache) |
+                           reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new);
+    return (d % 4 == 0 && (bits & 15) == 0) ? 4 : ((d % 2 == 0 && (bits & 7) == 0) ? 2 : 1);
+}
+
 template <bool APPEND, int NW, int LPR, bool DEVPOS>
 void decode_launch_kernel(dl4s_hip_ctx *ctx, dim3 grid, const float *q, float *kcache, float *vcache, const float *k_new,
                           const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
-                          int d, int H, const int *lengths, const int *pos_dev) {
-    if (d == 4 * LPR)
+                          int d, int H, const int *lengths, const int *pos_dev, int vec) {
+    if (d == 4 * LPR && vec == 4)
         hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, true, DEVPOS>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
-                           k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev);
+                           k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, 4);
     else
         hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, false, DEVPOS>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
-                           k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev);
+                           k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, vec);
 }
 
 template <bool APPEND, bool DEVPOS>
 void decode_launch_width(dl4s_hip_ctx *ctx, int nw, dim3 grid, const float *q, float *kcache, float *vcache, const float *k_new,
                          const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
-                         int d, int H, const int *lengths, const int *pos_dev) {
-#define DL4S_DECODE_ARGS ctx, grid, q, kcache, vcache, k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev
+                         int d, int H, const int *lengths, const int *pos_dev, int vec) {
+#define DL4S_DECODE_ARGS ctx, grid, q, kcache, vcache, k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, vec
     switch (lanes_per_row(d)) {
         case 8: if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS>(DL4S_DECODE_ARGS); break;
         case 16: if (nw == 16) decode_launch_kernel<APPEND, 16, 16, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 16, DEVPOS>(DL4S_DECODE_ARGS); break;
@@ -283,11 +325,8 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     const int64_t BH = B * H;
     if (BH == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(q && kcache && vcache && out, DL4S_HIP_EINVALID_ARG, "sdpa_decode: NULL tensor pointer");
-    DL4S_REQUIRE(d >= 4 && d <= MAXD && d % 4 == 0, DL4S_HIP_EUNSUPPORTED,
-                 "sdpa_decode: head dim %lld (multiples of 4 up to %d are implemented)", (long long)d, MAXD);
-    DL4S_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kcache) | reinterpret_cast<uintptr_t>(vcache) |
-                   reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) == 0, DL4S_HIP_EUNSUPPORTED,
-                 "sdpa_decode: q, the caches and the new rows must be 16-byte aligned");
+    DL4S_REQUIRE(d >= 1 && d <= MAXD, DL4S_HIP_EUNSUPPORTED, "sdpa_decode: head dim %lld (1 to %d are implemented)", (long long)d, MAXD);
+    const int vec = row_vector_width(d, q, kcache, vcache, k_new, v_new);
     DL4S_REQUIRE(T >= 1 && T <= Tcap, DL4S_HIP_ESHAPE, "sdpa_decode: T=%lld must be in [1, Tcap=%lld]", (long long)T,
                  (long long)Tcap);
     DL4S_REQUIRE(BH <= 65535 && Tcap < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa_decode: B*H=%lld above 65535", (long long)BH);
@@ -329,10 +368,10 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     dim3 grid(nsplit, (unsigned)BH);
     if (append)
         decode_launch_width<true, false>(ctx, nw, grid, q, kcache, vcache, k_new, v_new, out, part, (int)T, (int)Tcap, (int)pos, rT, nsplit,
-                                         chunk, (int)d, (int)H, lengths, nullptr);
+                                         chunk, (int)d, (int)H, lengths, nullptr, vec);
     else
         decode_launch_width<false, false>(ctx, nw, grid, q, kcache, vcache, k_new, v_new, out, part, (int)T, (int)Tcap, -1, rT, nsplit, chunk,
-                                          (int)d, (int)H, lengths, nullptr);
+                                          (int)d, (int)H, lengths, nullptr, vec);
     int st = dl4s::launch_status("sdpa_decode_splitk_f32");
     if (st || nsplit == 1) return st;
     hipLaunchKernelGGL(sdpa_decode_merge_f32, dim3((unsigned)BH), dim3(MAXD), 0, ctx->stream, part, out, nsplit, 4 * lanes_per_row(d), (int)d);
@@ -414,11 +453,9 @@ int dl4s_hip_sdpa_decode_step_at_f32(dl4s_hip_ctx *ctx, const float *q, float *k
     const int64_t BH = B * H;
     if (BH == 0) return DL4S_HIP_OK;
     DL4S_REQUIRE(q && kcache && vcache && out && k_new && v_new && pos_dev, DL4S_HIP_EINVALID_ARG, "sdpa_decode_step_at: NULL pointer");
-    DL4S_REQUIRE(d >= 4 && d <= MAXD && d % 4 == 0, DL4S_HIP_EUNSUPPORTED,
-                 "sdpa_decode_step_at: head dim %lld (multiples of 4 up to %d are implemented)", (long long)d, MAXD);
-    DL4S_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kcache) | reinterpret_cast<uintptr_t>(vcache) |
-                   reinterpret_cast<uintptr_t>(k_new) | reinterpret_cast<uintptr_t>(v_new)) & 15) == 0, DL4S_HIP_EUNSUPPORTED,
-                 "sdpa_decode_step_at: q, the caches and the new rows must be 16-byte aligned");
+    DL4S_REQUIRE(d >= 1 && d <= MAXD, DL4S_HIP_EUNSUPPORTED,
+                 "sdpa_decode_step_at: head dim %lld (1 to %d are implemented)", (long long)d, MAXD);
+    const int vec = row_vector_width(d, q, kcache, vcache, k_new, v_new);
     DL4S_REQUIRE(Tcap >= 1 && Tcap < (1ll << 30) && BH <= 65535, DL4S_HIP_EUNSUPPORTED,
                  "sdpa_decode_step_at: capacity %lld or B*H=%lld out of range", (long long)Tcap, (long long)BH);
     // the row count is not known on the host: one workgroup per pair walks whatever rows there are (16 wavefronts, 4 for a
@@ -426,7 +463,7 @@ int dl4s_hip_sdpa_decode_step_at_f32(dl4s_hip_ctx *ctx, const float *q, float *k
     const int KB = 8 * (64 / lanes_per_row(d));
     const int chunk = (int)((Tcap + KB - 1) / KB * KB);
     decode_launch_width<true, true>(ctx, Tcap > 128 ? 16 : 4, dim3(1, (unsigned)BH), q, kcache, vcache, k_new, v_new, out, nullptr, 0,
-                                    (int)Tcap, 0, inv_temperature, 1, chunk, (int)d, (int)H, nullptr, pos_dev);
+                                    (int)Tcap, 0, inv_temperature, 1, chunk, (int)d, (int)H, nullptr, pos_dev, vec);
     return dl4s::launch_status("sdpa_decode_splitk_f32");
 }
 

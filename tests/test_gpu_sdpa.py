@@ -493,11 +493,12 @@ def test_decode_matches_oracle(ctx, orc, B, H, T, Tcap):
     assert_parity(got, pre, "decode vs prefill")
 
 
-@pytest.mark.parametrize("d", [32, 128, 8, 4, 40, 96, 100])
+@pytest.mark.parametrize("d", [32, 128, 8, 4, 40, 96, 100, 70, 1, 3, 6, 33, 127])
 @pytest.mark.parametrize("B,H,T,Tcap", [(1, 1, 1, 1), (2, 3, 9, 12), (2, 2, 129, 140), (1, 4, 257, 300), (1, 8, 513, 600),
                                         (3, 2, 1000, 1024), (2, 2, 4097, 4160)])
 def test_decode_other_head_dims(ctx, orc, B, H, T, Tcap, d):
-    """Cache rows of 32 and 128 floats (8 and 32 lanes per row) and head dims that leave lanes idle."""
+    """Cache rows of 32 and 128 floats (8 and 32 lanes per row), head dims that leave lanes idle, and head dims that are no
+    multiple of 4 (rows off the 16-byte grid: one float per load)."""
     rng = np.random.default_rng(T * 1000 + d)
     q, kc, vc = rand(rng, B, H, 1, d), rand(rng, B, H, Tcap, d), rand(rng, B, H, Tcap, d)
     kc[:, :, T:] = np.nan
@@ -508,7 +509,7 @@ def test_decode_other_head_dims(ctx, orc, B, H, T, Tcap, d):
     assert_parity(got, run_sdpa(ctx, q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T])), "decode vs prefill")
 
 
-@pytest.mark.parametrize("d", [64, 32, 128, 24])
+@pytest.mark.parametrize("d", [64, 32, 128, 24, 70, 5])
 @pytest.mark.parametrize("B,H,T,Tcap", [(4, 2, 9, 12), (5, 2, 300, 320), (6, 3, 1000, 1024), (4, 2, 4097, 4160)])
 def test_decode_with_key_lengths(ctx, orc, B, H, T, Tcap, d):
     """dl4s_hip_sdpa_decode_lengths_f32 against the oracle's attention on the gathered tensors under the padding mask
@@ -532,6 +533,38 @@ def test_decode_with_key_lengths(ctx, orc, B, H, T, Tcap, d):
     pre = run_sdpa(ctx, q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T]), kind=lib.MASK_KEY_LENGTHS,
                    lens=np.minimum(lens, T))
     assert_parity(got, pre, "decode with lengths vs prefill")
+
+
+@pytest.mark.parametrize("shift", [1, 2])
+@pytest.mark.parametrize("d", [64, 128, 20])
+@pytest.mark.parametrize("T,Tcap", [(9, 12), (700, 701), (4100, 4100)])
+def test_decode_on_operands_off_the_16_byte_grid(ctx, orc, T, Tcap, d, shift):
+    """Every operand 4 or 8 bytes past a 16-byte boundary (a view into a larger buffer): the kernel reads 32 or 64 bits per
+    load and gives the bits of the aligned call; decode_step appends through the same path."""
+    rng = np.random.default_rng(T + d)
+    B, H = 2, 3
+    q, kc, vc = rand(rng, B, H, 1, d), rand(rng, B, H, Tcap, d), rand(rng, B, H, Tcap, d)
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+    aligned = run_decode(ctx, q, kc, vc, T)
+    pad = lambda x: np.concatenate([np.zeros(shift, np.float32), x.ravel()])
+    dq, dk_, dv_ = ctx.to_device(pad(q)), ctx.to_device(pad(kc)), ctx.to_device(pad(vc))
+    dout = ctx.empty((B * H * d + shift,))
+    off = 4 * shift
+    ctx.sdpa_decode(dq.offset(off), dk_.offset(off), dv_.offset(off), dout.offset(off), B, H, T, Tcap, d, rT)
+    got = dout.numpy()[shift:].reshape(B, H, 1, d)
+    assert np.array_equal(got, aligned)
+    assert_parity(got, orc.sdpa_decode(q, kc, vc, T), "decode, unaligned operands")
+    if T < Tcap:
+        kn, vn = rand(rng, B, H, 1, d), rand(rng, B, H, 1, d)
+        dkn, dvn = ctx.to_device(pad(kn)), ctx.to_device(pad(vn))
+        ctx.sdpa_decode_step(dq.offset(off), dk_.offset(off), dv_.offset(off), dkn.offset(off), dvn.offset(off), dout.offset(off), B, H, T, Tcap, d, rT)
+        kc2, vc2 = kc.copy(), vc.copy()
+        kc2[:, :, T], vc2[:, :, T] = kn[:, :, 0], vn[:, :, 0]
+        assert np.array_equal(dk_.numpy()[shift:].reshape(kc.shape), kc2) and np.array_equal(dv_.numpy()[shift:].reshape(vc.shape), vc2)
+        assert_parity(dout.numpy()[shift:].reshape(B, H, 1, d), orc.sdpa_decode(q, kc2, vc2, T + 1), "decode step, unaligned operands")
+        dkn.release(); dvn.release()
+    for b_ in (dq, dk_, dv_, dout):
+        b_.release()
 
 
 def test_decode_nan_inf(ctx, orc):
@@ -606,12 +639,14 @@ def test_config5_incremental_decode_append_then_attend(ctx, orc):
         buf.release()
 
 
+@pytest.mark.parametrize("d", [64, 30, 7])
 @pytest.mark.parametrize("Tcap,steps", [(300, 260), (100, 90)])      # workgroups of 16 and of 4 wavefronts
-def test_decode_step_with_the_position_in_device_memory(ctx, orc, Tcap, steps):
+def test_decode_step_with_the_position_in_device_memory(ctx, orc, Tcap, steps, d):
     """dl4s_hip_sdpa_decode_step_at_f32 reads the row to append from device memory: a sequence of steps driven by a
     device counter (advanced by dl4s_hip_argmax_to_f32, as cached decoding does) fills the cache and attends like the
     by-value entry point; a position outside the cache leaves cache and output alone."""
-    B, H, d = 2, 3, 64
+    B, H = 2, 3
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))      # 0.125 at d = 64
     rng = np.random.default_rng(5150)
     qs, kn, vn = (rng.standard_normal((steps, B, H, 1, d)).astype(np.float32) for _ in range(3))
     dq, dkn, dvn = ctx.to_device(qs), ctx.to_device(kn), ctx.to_device(vn)
@@ -624,7 +659,7 @@ def test_decode_step_with_the_position_in_device_memory(ctx, orc, Tcap, steps):
     step_bytes = B * H * d * 4
     for t in range(steps):
         ctx.sdpa_decode_step_at(dq.offset(t * step_bytes), dk_, dv_, dkn.offset(t * step_bytes), dvn.offset(t * step_bytes),
-                                dout.offset(t * step_bytes), B, H, cursor.offset(4), Tcap, d, 0.125)
+                                dout.offset(t * step_bytes), B, H, cursor.offset(4), Tcap, d, rT)
         ctx.argmax_to(scores, 7, cursor, cursor.offset(4))               # position += 1
     assert list(cursor.numpy()) == [6, steps]
     out, kfin, vfin = dout.numpy(), dk_.numpy(), dv_.numpy()
@@ -637,7 +672,7 @@ def test_decode_step_with_the_position_in_device_memory(ctx, orc, Tcap, steps):
     before = dout.numpy().copy()
     for bad in (-1, Tcap, 1 << 20):
         cur = ctx.to_device(np.array([0, bad], np.int32), dtype=np.int32)
-        ctx.sdpa_decode_step_at(dq, dk_, dv_, dkn, dvn, dout, B, H, cur.offset(4), Tcap, d, 0.125)
+        ctx.sdpa_decode_step_at(dq, dk_, dv_, dkn, dvn, dout, B, H, cur.offset(4), Tcap, d, rT)
         assert np.array_equal(dout.numpy(), before, equal_nan=True) and np.array_equal(dk_.numpy(), kfin, equal_nan=True)
         cur.release()
     for buf in (dq, dkn, dvn, dk_, dv_, dout, cursor, scores):
