@@ -567,6 +567,27 @@ def test_decode_on_operands_off_the_16_byte_grid(ctx, orc, T, Tcap, d, shift):
         b_.release()
 
 
+@pytest.mark.parametrize("B,H,T,Tcap,d", [(2, 4, 131072, 131072, 64), (1, 2, 1000001, 1000001, 32), (1, 3, 200000, 262144, 128), (2, 2, 70001, 70001, 70)])
+def test_decode_over_very_long_caches(ctx, B, H, T, Tcap, d):
+    """Caches far longer than the oracle finishes: the decode (plain and with key lengths) against an fp64 model written
+    from the definition."""
+    rng = np.random.default_rng(T + d)
+    q, kc, vc = rand(rng, B, H, 1, d), rand(rng, B, H, Tcap, d), rand(rng, B, H, Tcap, d)
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+    s = np.einsum("bhtd,bhd->bht", kc[:, :, :T].astype(np.float64), q[:, :, 0].astype(np.float64)) * rT
+
+    def model(n_of_batch):
+        ref = np.empty((B, H, 1, d))
+        for b, n in enumerate(n_of_batch):
+            p = np.exp(s[b, :, :n] - s[b, :, :n].max(-1, keepdims=True))
+            p /= p.sum(-1, keepdims=True)
+            ref[b, :, 0] = np.einsum("ht,htd->hd", p, vc[b, :, :n].astype(np.float64))
+        return ref
+    np.testing.assert_allclose(run_decode(ctx, q, kc, vc, T), model([T] * B), rtol=1e-4, atol=2e-6)
+    lens = [T - 7] + [T // 3] * (B - 1)
+    np.testing.assert_allclose(run_decode(ctx, q, kc, vc, T, lens=np.array(lens)), model(lens), rtol=1e-4, atol=2e-6)
+
+
 def test_decode_nan_inf(ctx, orc):
     rng = np.random.default_rng(77)
     B, H, T = 2, 2, 600
