@@ -82,7 +82,11 @@ int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx) {
     c->device = device_ordinal;
     c->cu_count = prop.multiProcessorCount;
     c->clock_khz = prop.clockRate;
-    snprintf(c->name, sizeof(c->name), "%s (%s)", prop.name, prop.gcnArchName);
+    // some driver stacks leave the marketing name of the properties empty: ask the other query, then say so
+    char queried[128] = "";
+    if (!prop.name[0] && hipDeviceGetName(queried, (int)sizeof(queried), device_ordinal) != hipSuccess) queried[0] = 0;
+    (void)hipGetLastError();
+    snprintf(c->name, sizeof(c->name), "%s (%s)", prop.name[0] ? prop.name : (queried[0] ? queried : "unnamed GPU"), prop.gcnArchName);
     hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_begin);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_end);
