@@ -4,7 +4,8 @@
 // 128-bit load per lane, so every load instruction of a wavefront covers four whole rows (1 KiB,
 // contiguous), and a wavefront keeps the 8 K loads and 8 V loads of a 32-key block in flight together.
 // The dot product is reduced inside the 16-lane group with DPP adds.  Rows of 32 and 128 floats use groups of 8 and
-// 32 lanes in the same way (64 and 16 keys per iteration); other head dims run the next wider form with idle lanes, and a
+// 32 lanes in the same way (64 and 16 keys per iteration), rows of 96 floats groups of 8 lanes that read three pieces each
+// (32 keys per iteration); other head dims run the next wider form with idle lanes, and a
 // head dim that is no multiple of 4 (rows off the 16-byte grid) reads 64 or 32 bits per load.  With 16 wavefronts resident per CU
 // that is ample memory-level parallelism to keep HBM busy.
 //
@@ -65,7 +66,10 @@ __device__ __forceinline__ float row_sum(float x) {
 // score - 1e9 (NN/Models/Transformer/ScaledDotProductAttention.swift:55-57 with the mask of makeEncoderMasks).  With at
 // least one key left their weights are exactly zero and they are not visited at all; a length of zero or less blocks every
 // key, the penalty is applied to all of them and the row comes out uniform, as in the reference.
-template <bool APPEND, int NW, int LPR, bool FULL, bool DEVPOS = false>
+// SEG: the row is read as SEG consecutive segments of 4 * LPR floats by the same LPR lanes (SEG loads per row and lane, NK =
+// 4 keys per lane and iteration instead of 8).  SEG = 3 with LPR = 8 serves rows of 96 floats with every lane busy, where the
+// 32-lane form would leave a quarter of the lanes idle.
+template <bool APPEND, int NW, int LPR, bool FULL, bool DEVPOS = false, int SEG = 1>
 __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
                                                                    float *vcache, const float *__restrict__ k_new,
                                                                    const float *__restrict__ v_new,
@@ -73,7 +77,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
                                                                    int pos, float rT, int nsplit, int chunk, int d, int H,
                                                                    const int *__restrict__ lengths,
                                                                    const int *__restrict__ pos_dev = nullptr, int vec = 4) {
-    constexpr int D = 4 * LPR, G = 64 / LPR, KB = 8 * G, PSTR = pstr(D);
+    constexpr int SW = 4 * LPR, D = SW * SEG, G = 64 / LPR, NK = SEG == 1 ? 8 : 4, KB = NK * G, PSTR = pstr(D);
     __shared__ float sm_o[NW][D];
     __shared__ float sm_m[NW], sm_l[NW];
     if (DEVPOS) {
@@ -86,16 +90,17 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int g = lane / LPR, c = lane % LPR;
-    const bool col_ok = FULL || 4 * c < d;    // FULL: d = 4 * LPR, every lane has its piece of the row; else lanes beyond the row hold zeros
+    // FULL: d = D, every lane has its pieces of the row; else pieces beyond the row hold zeros
     // vec < 4: rows that are no whole number of 16-byte pieces, or operands that are not 16-byte aligned - a lane reads its
     // (up to) four columns as two 64-bit halves (even row length, 8-byte aligned operands) or one float at a time; the
     // wavefront's loads still cover whole contiguous rows.
     const bool vec4 = FULL || vec == 4;
-    const int ncol = FULL ? 4 : d - 4 * c;
-    auto load4 = [&](const float *p) -> f32x4 {
+    // p: the lane's piece of segment sg of a row (row base + SW * sg + 4 * c)
+    auto load4 = [&](const float *p, const int sg) -> f32x4 {
+        const int ncol = FULL ? 4 : d - SW * sg - 4 * c;
         f32x4 r = {0.f, 0.f, 0.f, 0.f};
         if (vec4) {
-            if (col_ok) r = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+            if (ncol > 0) r = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
         } else if (vec == 2) {      // even row length: ncol is 2 or at least 4 wherever it is positive
             typedef float f32x2 __attribute__((ext_vector_type(2)));
             if (ncol > 0) { const f32x2 t = __builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(p)); r.x = t.x; r.y = t.y; }
@@ -108,9 +113,10 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         }
         return r;
     };
-    auto store4 = [&](float *p, const f32x4 r) {
+    auto store4 = [&](float *p, const f32x4 r, const int sg) {
+        const int ncol = FULL ? 4 : d - SW * sg - 4 * c;
         if (vec4) {
-            if (col_ok) *reinterpret_cast<f32x4 *>(p) = r;
+            if (ncol > 0) *reinterpret_cast<f32x4 *>(p) = r;
         } else if (vec == 2) {
             typedef float f32x2 __attribute__((ext_vector_type(2)));
             if (ncol > 0) *reinterpret_cast<f32x2 *>(p) = f32x2{r.x, r.y};
@@ -130,8 +136,12 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         else if (len < T) T = len;
     }
 
-    f32x4 qv = load4(q + (long long)bh * d + 4 * c);
-    qv.x *= rT; qv.y *= rT; qv.z *= rT; qv.w *= rT;
+    f32x4 qv[SEG];
+#pragma unroll
+    for (int sg = 0; sg < SEG; ++sg) {
+        qv[sg] = load4(q + (long long)bh * d + SW * sg + 4 * c, sg);
+        qv[sg].x *= rT; qv[sg].y *= rT; qv[sg].z *= rT; qv[sg].w *= rT;
+    }
 
     const long long base = (long long)bh * Tcap * d + 4 * c;
     const int c0 = split * chunk;
@@ -146,13 +156,18 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         vn_row = v_new + (long long)bh * d + 4 * c;
         const bool mine = (pos >= c0 && pos < c1) || (pos >= T && split == 0);
         if (mine && wave == 0 && g == 0) {
-            store4(kcache + base + (long long)pos * d, load4(kn_row));
-            store4(vcache + base + (long long)pos * d, load4(vn_row));
+#pragma unroll
+            for (int sg = 0; sg < SEG; ++sg) {
+                store4(kcache + base + (long long)pos * d + SW * sg, load4(kn_row + SW * sg, sg), sg);
+                store4(vcache + base + (long long)pos * d + SW * sg, load4(vn_row + SW * sg, sg), sg);
+            }
         }
     }
 
     float m_run = -INFINITY, l_run = 0.f;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[SEG];
+#pragma unroll
+    for (int sg = 0; sg < SEG; ++sg) acc[sg] = f32x4{0.f, 0.f, 0.f, 0.f};
     // The wavefronts take the KB-key blocks of [c0, c1) round-robin, starting at a block that depends on the
     // (batch, head) pair: all workgroups run in lockstep, and without the rotation they would all be at the same
     // offset of their cache rows at the same time, which for some row strides (Tcap) lands on few HBM channels.
@@ -162,36 +177,48 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         int bb = bi + rot;
         if (bb >= nblk) bb -= nblk;
         const int kb = c0 + bb * KB;
-        f32x4 kk[8], vv[8];
+        f32x4 kk[NK][SEG], vv[NK][SEG];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < NK; ++i) {
             const int key = kb + G * i + g;
             const int kc = key < T ? key : T - 1;
             const float *kp = kcache + base + (long long)kc * d;
             if (APPEND) kp = (kc == pos) ? kn_row : kp;
-            kk[i] = load4(kp);
+#pragma unroll
+            for (int sg = 0; sg < SEG; ++sg) kk[i][sg] = load4(kp + SW * sg, sg);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < NK; ++i) {
             const int key = kb + G * i + g;
             const int kc = key < T ? key : T - 1;
             const float *vp = vcache + base + (long long)kc * d;
             if (APPEND) vp = (kc == pos) ? vn_row : vp;
-            vv[i] = load4(vp);
+#pragma unroll
+            for (int sg = 0; sg < SEG; ++sg) vv[i][sg] = load4(vp + SW * sg, sg);
         }
         if (kb + KB > c1) {     // the range's last block: lanes past its end re-read row T-1 and must add nothing, not 0 * Inf
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (kb + G * i + g >= c1) vv[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < NK; ++i)
+                if (kb + G * i + g >= c1) {
+#pragma unroll
+                    for (int sg = 0; sg < SEG; ++sg) vv[i][sg] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
         }
-        float s[8];
+        float s[NK];
         float bm = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float dot = qv.x * kk[i].x;
-            dot += qv.y * kk[i].y;
-            dot += qv.z * kk[i].z;
-            dot += qv.w * kk[i].w;
+        for (int i = 0; i < NK; ++i) {
+            float dot = qv[0].x * kk[i][0].x;
+            dot += qv[0].y * kk[i][0].y;
+            dot += qv[0].z * kk[i][0].z;
+            dot += qv[0].w * kk[i][0].w;
+#pragma unroll
+            for (int sg = 1; sg < SEG; ++sg) {
+                dot += qv[sg].x * kk[i][sg].x;
+                dot += qv[sg].y * kk[i][sg].y;
+                dot += qv[sg].z * kk[i][sg].z;
+                dot += qv[sg].w * kk[i][sg].w;
+            }
             dot = row_sum<LPR>(dot);
             if (all_blocked) dot = __fsub_rn(dot, 1e9f);
             if (kb + G * i + g >= c1) dot = -INFINITY;
@@ -203,12 +230,16 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         const float alpha = fast_exp2((m_run - m_use) * LOG2E);
         m_run = m_new;
         l_run *= alpha;
-        acc.x *= alpha; acc.y *= alpha; acc.z *= alpha; acc.w *= alpha;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int sg = 0; sg < SEG; ++sg) { acc[sg].x *= alpha; acc[sg].y *= alpha; acc[sg].z *= alpha; acc[sg].w *= alpha; }
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
             const float p = fast_exp2((s[i] - m_use) * LOG2E);
             l_run += p;
-            acc.x += p * vv[i].x; acc.y += p * vv[i].y; acc.z += p * vv[i].z; acc.w += p * vv[i].w;
+#pragma unroll
+            for (int sg = 0; sg < SEG; ++sg) {
+                acc[sg].x += p * vv[i][sg].x; acc[sg].y += p * vv[i][sg].y; acc[sg].z += p * vv[i][sg].z; acc[sg].w += p * vv[i][sg].w;
+            }
         }
     }
     // merge the G groups of the wavefront
@@ -219,15 +250,22 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
         const float mu = (mw == -INFINITY) ? 0.f : mw;
         const float f = fast_exp2((m_run - mu) * LOG2E);
         l_run *= f;
-        acc.x *= f; acc.y *= f; acc.z *= f; acc.w *= f;
+#pragma unroll
+        for (int sg = 0; sg < SEG; ++sg) { acc[sg].x *= f; acc[sg].y *= f; acc[sg].z *= f; acc[sg].w *= f; }
     }
 #pragma unroll
     for (int o = LPR; o <= 32; o <<= 1) {
         l_run += __shfl_xor(l_run, o, 64);
-        acc.x += __shfl_xor(acc.x, o, 64); acc.y += __shfl_xor(acc.y, o, 64);
-        acc.z += __shfl_xor(acc.z, o, 64); acc.w += __shfl_xor(acc.w, o, 64);
+#pragma unroll
+        for (int sg = 0; sg < SEG; ++sg) {
+            acc[sg].x += __shfl_xor(acc[sg].x, o, 64); acc[sg].y += __shfl_xor(acc[sg].y, o, 64);
+            acc[sg].z += __shfl_xor(acc[sg].z, o, 64); acc[sg].w += __shfl_xor(acc[sg].w, o, 64);
+        }
     }
-    if (g == 0) *reinterpret_cast<f32x4 *>(&sm_o[wave][4 * c]) = acc;
+    if (g == 0) {
+#pragma unroll
+        for (int sg = 0; sg < SEG; ++sg) *reinterpret_cast<f32x4 *>(&sm_o[wave][SW * sg + 4 * c]) = acc[sg];
+    }
     if (lane == 0) { sm_m[wave] = mw; sm_l[wave] = l_run; }
     __syncthreads();
 
@@ -282,8 +320,14 @@ __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restr
     vcache[dst] = v_new[i];
 }
 
-// Row widths the kernel is instantiated for: 32, 64, 128 floats (8, 16, 32 lanes per row).
-inline int lanes_per_row(int64_t d) { return d <= 32 ? 8 : (d <= 64 ? 16 : 32); }
+// Row widths the kernel is instantiated for: 32, 64, 128 floats (8, 16, 32 lanes per row, one 128-bit piece per lane) and 96
+// floats (8 lanes per row, three pieces per lane).
+// (the 96-float form for exactly 96 floats and 128-bit pieces: with part-filled or narrower pieces its three loads per lane
+// cost more than the idle lanes of the 128-float form - B16 H16 over 4096 rows: d = 96 163 -> 137 us, d = 80 160 -> 175 us)
+inline int row_segments(int64_t d, int vec) { return d == 96 && vec == 4 ? 3 : 1; }
+inline int lanes_per_row(int64_t d, int vec) { return d <= 32 ? 8 : (d <= 64 ? 16 : (row_segments(d, vec) == 3 ? 8 : 32)); }
+inline int row_width(int64_t d, int vec) { return 4 * lanes_per_row(d, vec) * row_segments(d, vec); }
+inline int keys_per_iteration(int64_t d, int vec) { return (row_segments(d, vec) == 1 ? 8 : 4) * (64 / lanes_per_row(d, vec)); }
 
 // 4 when every cache row starts on a 16-byte boundary (the row length a multiple of 4 floats, every operand aligned): a lane
 // reads its piece of a row with one 128-bit load.  2 for an even row length and 8-byte aligned operands (two 64-bit loads),
@@ -294,15 +338,15 @@ inline int row_vector_width(int64_t d, const void *q, const void *kcache, const 
     return (d % 4 == 0 && (bits & 15) == 0) ? 4 : ((d % 2 == 0 && (bits & 7) == 0) ? 2 : 1);
 }
 
-template <bool APPEND, int NW, int LPR, bool DEVPOS>
+template <bool APPEND, int NW, int LPR, bool DEVPOS, int SEG = 1>
 void decode_launch_kernel(dl4s_hip_ctx *ctx, dim3 grid, const float *q, float *kcache, float *vcache, const float *k_new,
                           const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
                           int d, int H, const int *lengths, const int *pos_dev, int vec) {
-    if (d == 4 * LPR && vec == 4)
-        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, true, DEVPOS>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
+    if (SEG > 1 || (d == 4 * LPR && vec == 4))      // the segmented form is only chosen for full rows
+        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, true, DEVPOS, SEG>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
                            k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, 4);
-    else
-        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, false, DEVPOS>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
+    else if constexpr (SEG == 1)
+        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, false, DEVPOS, 1>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
                            k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, vec);
 }
 
@@ -311,7 +355,9 @@ void decode_launch_width(dl4s_hip_ctx *ctx, int nw, dim3 grid, const float *q, f
                          const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
                          int d, int H, const int *lengths, const int *pos_dev, int vec) {
 #define DL4S_DECODE_ARGS ctx, grid, q, kcache, vcache, k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, vec
-    switch (lanes_per_row(d)) {
+    if (row_segments(d, vec) == 3) {
+        if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS, 3>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS, 3>(DL4S_DECODE_ARGS);
+    } else switch (lanes_per_row(d, vec)) {
         case 8: if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS>(DL4S_DECODE_ARGS); break;
         case 16: if (nw == 16) decode_launch_kernel<APPEND, 16, 16, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 16, DEVPOS>(DL4S_DECODE_ARGS); break;
         default: if (nw == 16) decode_launch_kernel<APPEND, 16, 32, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 32, DEVPOS>(DL4S_DECODE_ARGS); break;
@@ -330,8 +376,8 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     DL4S_REQUIRE(T >= 1 && T <= Tcap, DL4S_HIP_ESHAPE, "sdpa_decode: T=%lld must be in [1, Tcap=%lld]", (long long)T,
                  (long long)Tcap);
     DL4S_REQUIRE(BH <= 65535 && Tcap < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa_decode: B*H=%lld above 65535", (long long)BH);
-    const int KB = 8 * (64 / lanes_per_row(d));   // keys per wavefront iteration
-    const int PSTR = pstr(4 * lanes_per_row(d));
+    const int KB = keys_per_iteration(d, vec);   // keys per wavefront iteration
+    const int PSTR = pstr(row_width(d, vec));
     // Aim at 16 resident wavefronts on every CU.  Long caches use 16-wavefront workgroups; the key range is split
     // over several workgroups only when batch*heads alone does not fill the GPU.  Up to 512 rows one workgroup per pair
     // does it all (16 wavefronts above 128 rows): a second launch for the merge costs more than the split saves
@@ -374,7 +420,7 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
                                           (int)d, (int)H, lengths, nullptr, vec);
     int st = dl4s::launch_status("sdpa_decode_splitk_f32");
     if (st || nsplit == 1) return st;
-    hipLaunchKernelGGL(sdpa_decode_merge_f32, dim3((unsigned)BH), dim3(MAXD), 0, ctx->stream, part, out, nsplit, 4 * lanes_per_row(d), (int)d);
+    hipLaunchKernelGGL(sdpa_decode_merge_f32, dim3((unsigned)BH), dim3(MAXD), 0, ctx->stream, part, out, nsplit, row_width(d, vec), (int)d);
     return dl4s::launch_status("sdpa_decode_merge_f32");
 }
 
@@ -460,7 +506,7 @@ int dl4s_hip_sdpa_decode_step_at_f32(dl4s_hip_ctx *ctx, const float *q, float *k
                  "sdpa_decode_step_at: capacity %lld or B*H=%lld out of range", (long long)Tcap, (long long)BH);
     // the row count is not known on the host: one workgroup per pair walks whatever rows there are (16 wavefronts, 4 for a
     // cache of up to 128 rows, where one block per wavefront covers it)
-    const int KB = 8 * (64 / lanes_per_row(d));
+    const int KB = keys_per_iteration(d, vec);
     const int chunk = (int)((Tcap + KB - 1) / KB * KB);
     decode_launch_width<true, true>(ctx, Tcap > 128 ? 16 : 4, dim3(1, (unsigned)BH), q, kcache, vcache, k_new, v_new, out, nullptr, 0,
                                     (int)Tcap, 0, inv_temperature, 1, chunk, (int)d, (int)H, nullptr, pos_dev, vec);
