@@ -345,8 +345,8 @@ def other_configs(ctx, lib, cpu, only=None):
                 b_.release()
         dmask.release()
     if want("decode_head_dims"):
-        # config 5's decode (B16 H16, 4096 cached rows + 64 steps) with cache rows of 128 and of 32 floats
-        for d in (128, 32):
+        # config 5's decode (B16 H16, 4096 cached rows + 64 steps) with cache rows of 128, 96 and 32 floats
+        for d in (128, 96, 32):
             dec = decode(ctx, lib, 3, d)
             res["config5_shape_decode_head_dim_%d" % d] = {"us_per_step": dec["us_per_step"], "gbs": dec["gbs"], "frac_hbm_peak": dec["gbs"] / HBM_PEAK_GBS,
                                                             "bytes_per_step": dec["bytes_per_step"]}
