@@ -99,7 +99,8 @@ int decode_static_scratch_init(dl4s_hip_ctx *ctx);
     } while (0)
 
 // Kernel families of dl4s_hip_ctx::lds_limit_raised.
-enum { LDS_PREFILL_SPLIT = 0, LDS_PREFILL = 1, LDS_PREFILL_D128 = 2, LDS_BWD = 3, LDS_BWD_D128 = 4, LDS_GEMM_DEEP = 5 };
+enum { LDS_PREFILL_SPLIT = 0, LDS_PREFILL = 1, LDS_PREFILL_D128 = 2, LDS_BWD = 3, LDS_BWD_D128 = 4, LDS_GEMM_DEEP = 5, LDS_PREFILL_W192 = 6,
+       LDS_PREFILL_W256 = 7 };
 inline bool lds_limit_pending(const dl4s_hip_ctx *ctx, int family, int kind) {
     return !(ctx->lds_limit_raised.load(std::memory_order_acquire) & (1ull << (family * 8 + kind)));
 }

@@ -163,10 +163,11 @@ typedef struct dl4s_mask_desc {
  * a fused MFMA kernel written for tiles of 16, 32, 64, 96 or 128 columns; a head dim between two
  * widths is padded with zero columns on the fly and costs what the wider tile costs.  Even head dims
  * from 66 to 94 that are not a multiple of 4 run the 96-wide kernel as they are (8-byte aligned
- * tensors, launches that fill the GPU).  Other head dims up to 128 (dk != dv, odd,
+ * tensors, launches that fill the GPU).  dk = dv above 128 up to 256 (a multiple of 4, aligned) runs
+ * the same scheme on tiles of 192 or 256 columns.  Other head dims up to 256 (dk != dv, odd,
  * unaligned tensors) run the same kernels on zero-padded copies of the operands, which the call
  * allocates from the context's pool, when the problem is large enough to pay for the copies; small
- * problems and head dims up to 256 run a plain fused kernel. */
+ * problems of such head dims run a plain fused kernel.  Head dims above 256 are refused. */
 int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out,
                           int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);

@@ -782,10 +782,84 @@ def test_head_dims_up_to_96_on_launches_that_fill_the_gpu(ctx, orc, d, mk):
         assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, token_major=True), got)
 
 
+@pytest.mark.parametrize("d", [192, 256, 132, 160, 200, 252])
+@pytest.mark.parametrize("mk", ["none", "dense", "causal", "lens", "causal_lens"])
+def test_head_dims_above_128_on_the_wide_kernels(ctx, orc, d, mk):
+    """Head dims above 128 up to 256 (multiples of 4) run the 192- and 256-wide MFMA kernels in the forward call: ragged
+    extents, every mask kind, checked against the oracle on whole (batch, head) slices; descriptors against the dense masks
+    they stand for; the token-major layout bit for bit."""
+    from dl4s_amd import lib
+    B, H, Lq, Lk = 3, 4, 300, 333
+    if mk in ("causal", "causal_lens"):
+        Lk = Lq
+    rng = np.random.default_rng(zlib.crc32(repr(("wide", d, mk)).encode()))
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    lens = rng.integers(0, Lk + 1, size=B)
+    lens[0], lens[1] = Lk // 2, 0        # batch item 1: no valid key, uniform rows
+    kind, mask, lens_arg = None, None, None
+    if mk == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.4).astype(np.float32)
+        mask[:, :, 64:160, 96:224] = 1.0          # whole tiles of ones and of zeros
+        mask[:, :, 160:224, 0:96] = 0.0
+    elif mk == "causal":
+        kind, mask = lib.MASK_CAUSAL, causal_mask(Lq, Lk)
+    elif mk == "lens":
+        kind, mask, lens_arg = lib.MASK_KEY_LENGTHS, lengths_mask(lens, Lk), lens
+    elif mk == "causal_lens":
+        kind, lens_arg = lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lk)[None, None])
+    got = run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg)
+    for (b, h) in [(0, 0), (1, 2), (2, 3)]:
+        mb = None if mask is None else (mask if mask.ndim == 2 else mask[b:b + 1])
+        ref = orc.sdpa(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mb)
+        assert_parity(got[b:b + 1, h:h + 1], ref, "wide d=%d %s (b=%d,h=%d)" % (d, mk, b, h))
+    if kind is not None:    # descriptor == the dense mask it stands for, bit for bit, when both visit every tile
+        dense = run_sdpa(ctx, q, k, v, mask, strict=True)
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=True), dense)
+        assert_parity(got, dense, "skip vs dense")
+    if mask is not None:
+        assert np.array_equal(run_sdpa(ctx, q, k, v, mask), run_sdpa(ctx, q, k, v, mask, strict=True))
+    assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, token_major=True), got)
+
+
+@pytest.mark.parametrize("d", [192, 256, 140])
+@pytest.mark.parametrize("B,H,Lq,Lk", [(2, 3, 130, 5), (1, 2, 129, 33), (4, 2, 1, 64), (2, 2, 128, 31), (1, 1, 1, 1), (1, 1, 700, 900)])
+def test_wide_kernels_on_short_and_ragged_extents(ctx, orc, B, H, Lq, Lk, d):
+    rng = np.random.default_rng(zlib.crc32(repr(("wide short", B, H, Lq, Lk, d)).encode()))
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    lens = rng.integers(0, Lk + 1, size=B)
+    lens[0] = max(1, Lk // 2)
+    from dl4s_amd import lib
+    assert_parity(run_sdpa(ctx, q, k, v), orc.sdpa(q, k, v, None), "wide short d=%d" % d)
+    mask = lengths_mask(lens, Lk)
+    assert_parity(run_sdpa(ctx, q, k, v, mask, kind=lib.MASK_KEY_LENGTHS, lens=lens), orc.sdpa(q, k, v, mask), "wide short lens d=%d" % d)
+    # non-finite values: a NaN key row, an Inf value
+    k2, v2 = k.copy(), v.copy()
+    k2[0, 0, Lk // 2] = np.nan
+    v2[-1, -1, 0, d - 1] = np.inf
+    with np.errstate(all="ignore"):
+        ref = orc.sdpa(q, k2, v2, None)
+    assert_parity(run_sdpa(ctx, q, k2, v2), ref, "wide short non-finite d=%d" % d)
+
+
+@pytest.mark.parametrize("dk,dv", [(200, 130), (130, 256), (150, 150), (255, 255), (64, 192)])
+@pytest.mark.parametrize("mk", ["none", "causal"])
+def test_head_dims_up_to_256_served_by_padded_copies(ctx, orc, dk, dv, mk):
+    """Unequal or odd head dims above 128: the forward call runs the wide kernels on zero-padded copies."""
+    from dl4s_amd import lib
+    B, H, Lq, Lk = 2, 3, 260, 260
+    rng = np.random.default_rng(zlib.crc32(repr(("wide padded", dk, dv, mk)).encode()))
+    q, k, v = rand(rng, B, H, Lq, dk), rand(rng, B, H, Lk, dk), rand(rng, B, H, Lk, dv)
+    kind, mask = (lib.MASK_CAUSAL, causal_mask(Lq, Lk)) if mk == "causal" else (None, None)
+    got = run_sdpa(ctx, q, k, v, mask, kind=kind)
+    assert_parity(got[1:2, 2:3], orc.sdpa(q[1:2, 2:3], k[1:2, 2:3], v[1:2, 2:3], mask), "padded wide dk=%d dv=%d" % (dk, dv))
+    assert_parity(got[0:1, 0:1], orc.sdpa(q[0:1, 0:1], k[0:1, 0:1], v[0:1, 0:1], mask), "padded wide dk=%d dv=%d" % (dk, dv))
+
+
 def test_token_major_rejected_for_other_head_dims_and_unknown_flags(ctx):
     from dl4s_amd import lib
-    q = ctx.empty((1, 2, 4, 256))
-    for d in (6, 130, 200):     # not a multiple of 4 up to 128
+    q = ctx.empty((1, 2, 4, 260))
+    for d in (6, 130, 202, 260):     # not a multiple of 4 up to 256
         with pytest.raises(lib.Dl4sHipError):
             ctx.sdpa_fwd(q, q, q, q, 1, 2, 4, 4, d, d, 0.5, None, lib.SDPA_TOKEN_MAJOR)
     with pytest.raises(lib.Dl4sHipError):       # different key and value dims
