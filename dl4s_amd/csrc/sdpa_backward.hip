@@ -1096,6 +1096,9 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
 
 }  // namespace
 
+#include "sdpa_backward_wide.h"
+
+
 extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *out,
                                      const float *stats, const float *dout, float *dq, float *dk, float *dv, int64_t B,
                                      int64_t H, int64_t Lq, int64_t Lk, int64_t d, float inv_temperature,
@@ -1129,8 +1132,11 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                                  reinterpret_cast<uintptr_t>(dv)) & 15) == 0;
     const bool mfma_path = d > 0 && d <= HD && d % 4 == 0 && fwd_aligned;
     const bool mfma128_path = d > HD && d <= HD2 && d % 4 == 0 && fwd_aligned;
+    // head dims above 128: the forward call ran the 192- / 256-wide kernels
+    const bool wide_as_is = d > HD2 && d <= 256 && d % 4 == 0 && fwd_aligned;    // no copies, whichever kernel it was
+    const bool wide_path = wide_as_is && sdpa_wide_route(H, Lk, d, token_major);
     // the forward pass ran on zero-padded copies (sdpa_padded_route): so does this call, gradients included
-    if (!token_major && sdpa_padded_route(mfma_path || mfma128_path, B, H, Lq, Lk, d, d)) {
+    if (!token_major && sdpa_padded_route(mfma_path || mfma128_path || wide_as_is, B, H, Lq, Lk, d, d)) {
         const int64_t dp = (d + 3) / 4 * 4, qrows = B * H * Lq, krows = B * H * Lk;
         const int64_t rows_of[8] = {qrows, krows, krows, qrows, qrows, qrows, krows, krows};   // q k v out dout dq dk dv
         void *bufs[8] = {nullptr};
@@ -1154,7 +1160,7 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
         for (int i = 0; i < 8; ++i) (void)dl4s_hip_free(ctx, bufs[i]);
         return rc;
     }
-    DL4S_REQUIRE(!(mfma_path || mfma128_path) || grads_aligned, DL4S_HIP_EUNSUPPORTED,
+    DL4S_REQUIRE(!(mfma_path || mfma128_path || wide_path) || grads_aligned, DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: dout, dq, dk and dv must be 16-byte aligned when q, k, v and out are (the forward pass ran on "
                  "the MFMA kernels and left its row statistics in their form)");
     DL4S_REQUIRE(!mfma128_path || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * d * 4 < (d == HD2 ? (1ll << 31) : (1ll << 30)),
@@ -1163,6 +1169,10 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
     DL4S_REQUIRE(!mfma_path || (Lk > Lq ? Lk : Lq) * (token_major ? H : 1) * d * 4 < (d == HD ? (1ll << 31) : (1ll << 30)),
                  DL4S_HIP_EUNSUPPORTED,
                  "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB (1 GiB for head dims below 64)");
+    if (wide_path) {
+        DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa backward: the token-major layout needs a head dim of at most 128");
+        return sdpa_backward_wide(ctx, q, k, v, out, stats, dout, dq, dk, dv, B, H, Lq, Lk, d, inv_temperature, mask, ds_scratch_max_bytes());
+    }
     std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     MaskArgs m{};
     int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, mfma_path || mfma128_path, m);

@@ -1,0 +1,108 @@
+// Gradients of the fused attention for head dims above 128 and up to 256 (multiples of 4, head-major tensors): the row
+// fragments and accumulators of a fused kernel of that width do not fit a wavefront's registers, so the five products run
+// as batched GEMMs around one elementwise pass, on score tensors held in the context's pool.  Included by
+// sdpa_backward.hip only.
+//
+//   S2 = ((q * rT) * log2(e)) . k^T        the forward kernel's scores (base-2 exponent domain), [pairs, Lq, Lk]
+//   dP = dout . v^T                        [pairs, Lq, Lk]
+//   P  = 2^(mask(S2) - m) * inv            in place of S2; (m, inv) are the forward call's row statistics
+//   dS = P * (dP - D)                      in place of dP; D_i = dout_i . out_i
+//   dv = P^T . dout,  dk = rT * dS^T . q,  dq = rT * dS . k
+//
+// (Tensor/Operators/Matrix.swift:139-174, Binary.swift:235-300, Unary.swift:33-55, Reduce.swift:35-62 give the same
+// gradients closure by closure.)  The (batch, head) pairs are taken in chunks whose two score tensors stay inside the
+// gradient scratch bound.  Every key is visited, blocked or not (the behaviour of DL4S_SDPA_STRICT).  Deterministic: no
+// atomics, every sum in a fixed order.
+#pragma once
+#include "sdpa_common.h"
+
+namespace {
+
+// qs = (q * rT) * log2(e): the two roundings of the forward kernels' Q fragment
+__global__ __launch_bounds__(256) void sdpa_bwd_wide_scale_q(const float *__restrict__ q, float *__restrict__ qs, long long n4, float rT) {
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n4; i += (long long)gridDim.x * 256) {
+        const f32x4 t = reinterpret_cast<const f32x4 *>(q)[i];
+        const f32x4 r = {(t.x * rT) * LOG2E, (t.y * rT) * LOG2E, (t.z * rT) * LOG2E, (t.w * rT) * LOG2E};
+        reinterpret_cast<f32x4 *>(qs)[i] = r;
+    }
+}
+
+// One workgroup per query row of a chunk: S2 -> P and dP -> dS in place.  pair0: the chunk's first (batch, head) pair.
+__global__ __launch_bounds__(256) void sdpa_bwd_wide_weights(float *__restrict__ S, float *__restrict__ dP, const float *__restrict__ stats,
+                                                             const float *__restrict__ D, MaskArgs mask, long long pair0, int H, int Lq,
+                                                             int Lk) {
+    const long long row = blockIdx.x;                 // over the chunk's pairs x Lq
+    const long long bh = pair0 + row / Lq;
+    const int qi = (int)(row % Lq);
+    const int b = (int)(bh / H), hh = (int)(bh % H);
+    const long long grow = bh * Lq + qi;              // row of the whole problem: statistics and D
+    const float m = stats[2 * grow], inv = stats[2 * grow + 1], Di = D[grow];
+    const bool causal = mask.kind == DL4S_MASK_CAUSAL || mask.kind == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS;
+    const bool lens = mask.kind == DL4S_MASK_KEY_LENGTHS || mask.kind == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS;
+    const int len = lens ? mask.lengths[b] : Lk;
+    const float *mrow = mask.kind == DL4S_MASK_DENSE_F32 ? mask.dense + b * mask.sb + hh * mask.sh + qi * mask.sq : nullptr;
+    float *srow = S + row * Lk, *drow = dP + row * Lk;
+    for (int j = threadIdx.x; j < Lk; j += 256) {
+        float s = srow[j];
+        if (mrow) s = dense_masked2(s, mrow[j * mask.sk]);
+        else if ((causal && j > qi) || (lens && j >= len)) s = blocked_score2(s);
+        const float p = fast_exp2(s - m) * inv;
+        srow[j] = p;
+        drow[j] = p * (drow[j] - Di);
+    }
+}
+
+int sdpa_backward_wide(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *out, const float *stats,
+                       const float *dout, float *dq, float *dk, float *dv, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t d,
+                       float rT, const dl4s_mask_desc *mask, long long scratch_max_bytes) {
+    MaskArgs m{};
+    int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, false, m);
+    if (rc != DL4S_HIP_OK) return rc;
+    const int64_t pairs = B * H;
+    DL4S_REQUIRE(pairs * Lq < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "sdpa backward: too many query rows");
+    // (batch, head) pairs per chunk: two [Lq, Lk] tensors per pair inside the bound, at least one pair
+    const long long per_pair = 2ll * Lq * Lk * (long long)sizeof(float);
+    int64_t chunk = scratch_max_bytes / per_pair;
+    if (chunk < 1) chunk = 1;
+    if (chunk > pairs) chunk = pairs;
+    void *bufs[4] = {nullptr, nullptr, nullptr, nullptr};     // S2 / P, dP / dS, scaled q, D
+    const size_t sizes[4] = {(size_t)(chunk * Lq * Lk) * sizeof(float), (size_t)(chunk * Lq * Lk) * sizeof(float),
+                             (size_t)(chunk * Lq * d) * sizeof(float), (size_t)(pairs * Lq) * sizeof(float)};
+    for (int i = 0; i < 4; ++i)
+        if (dl4s_hip_alloc(ctx, sizes[i], &bufs[i]) != DL4S_HIP_OK) {
+            for (int j = 0; j < i; ++j) (void)dl4s_hip_free(ctx, bufs[j]);
+            return DL4S_HIP_EOOM;
+        }
+    float *S = static_cast<float *>(bufs[0]), *dP = static_cast<float *>(bufs[1]), *qs = static_cast<float *>(bufs[2]),
+          *D = static_cast<float *>(bufs[3]);
+    hipLaunchKernelGGL(sdpa_bwd_rowdot_plain, dim3((unsigned)(pairs * Lq)), dim3(64), 0, ctx->stream, out, dout, D, (int)d);
+    rc = dl4s::launch_status("sdpa_bwd_rowdot_plain");
+    for (int64_t p0 = 0; p0 < pairs && rc == DL4S_HIP_OK; p0 += chunk) {
+        const int64_t n = std::min(chunk, pairs - p0);
+        const float *qc = q + p0 * Lq * d, *kc = k + p0 * Lk * d, *vc = v + p0 * Lk * d, *gc = dout + p0 * Lq * d;
+        const long long n4 = n * Lq * d / 4;
+        hipLaunchKernelGGL(sdpa_bwd_wide_scale_q, dim3((unsigned)std::min<long long>((n4 + 255) / 256, 65536)), dim3(256), 0, ctx->stream, qc,
+                           qs, n4, rT);
+        rc = dl4s::launch_status("sdpa_bwd_wide_scale_q");
+        if (rc == DL4S_HIP_OK)      // S2 = qs . k^T
+            rc = dl4s_hip_gemm_batched_f32(ctx, qs, Lq, d, Lq * d, kc, Lk, d, Lk * d, S, Lq * Lk, n, 1.0f, 0.0f, 0, 1);
+        if (rc == DL4S_HIP_OK)      // dP = dout . v^T
+            rc = dl4s_hip_gemm_batched_f32(ctx, gc, Lq, d, Lq * d, vc, Lk, d, Lk * d, dP, Lq * Lk, n, 1.0f, 0.0f, 0, 1);
+        if (rc == DL4S_HIP_OK) {
+            hipLaunchKernelGGL(sdpa_bwd_wide_weights, dim3((unsigned)(n * Lq)), dim3(256), 0, ctx->stream, S, dP, stats, D, m, (long long)p0,
+                               (int)H, (int)Lq, (int)Lk);
+            rc = dl4s::launch_status("sdpa_bwd_wide_weights");
+        }
+        if (rc == DL4S_HIP_OK)      // dv = P^T . dout
+            rc = dl4s_hip_gemm_batched_f32(ctx, S, Lq, Lk, Lq * Lk, gc, Lq, d, Lq * d, dv + p0 * Lk * d, Lk * d, n, 1.0f, 0.0f, 1, 0);
+        if (rc == DL4S_HIP_OK)      // dk = rT * dS^T . q
+            rc = dl4s_hip_gemm_batched_f32(ctx, dP, Lq, Lk, Lq * Lk, qc, Lq, d, Lq * d, dk + p0 * Lk * d, Lk * d, n, rT, 0.0f, 1, 0);
+        if (rc == DL4S_HIP_OK)      // dq = rT * dS . k
+            rc = dl4s_hip_gemm_batched_f32(ctx, dP, Lq, Lk, Lq * Lk, kc, Lk, d, Lk * d, dq + p0 * Lq * d, Lq * d, n, rT, 0.0f, 0, 0);
+    }
+    // the pool hands a block out again only to work enqueued later on the same stream
+    for (int i = 0; i < 4; ++i) (void)dl4s_hip_free(ctx, bufs[i]);
+    return rc;
+}
+
+}  // namespace

@@ -299,15 +299,18 @@ __device__ __forceinline__ float plain_score(const float *qs, const float *krow,
 // Validates a mask descriptor against [B,H,Lq,Lk], fills the kernels' view of it and, for dense masks on the MFMA
 // kernels, launches the tile classifier (its result lives in the context's scratch block until the next call that uses it).
 // Head dims the MFMA kernels do not take as they are (not a multiple of 4, key dim != value dim, q / k / v / out off the
-// 16-byte grid), up to 128 (256 in the forward call without row statistics), on a problem large enough to pay for streaming
-// copies: the kernels run on zero-padded copies.
+// 16-byte grid), up to 256, on a problem large enough to pay for streaming copies: the kernels run on zero-padded copies.
 // The forward call that leaves row statistics and the gradient call evaluate this on the same arguments, so both land
 // on the same kind of kernel.
-// widest: the widest head dim the MFMA kernels of the call take (128 where row statistics are involved, 256 for the
-// forward call without them)
-inline bool sdpa_padded_route(bool mfma_as_is, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv, int64_t widest = HD2) {
+// Head dims above 128 up to 256 that the 192- and 256-wide forward kernels take as they are (the tensors 16-byte aligned
+// besides): a multiple of 4 whose K/V rows of one (batch, head) pair stay inside the kernels' 32-bit byte offsets.
+inline bool sdpa_wide_route(int64_t H, int64_t Lk, int64_t d, int token_major) {
+    return d > HD2 && d <= 256 && d % 4 == 0 && Lk * (token_major ? H : 1) * d * 4 < ((d == 192 || d == 256) ? (1ll << 31) : (1ll << 30));
+}
+
+inline bool sdpa_padded_route(bool mfma_as_is, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv) {
     const int64_t dmax = dk > dv ? dk : dv;
-    return !mfma_as_is && dk > 0 && dv > 0 && dmax <= widest && (double)B * H * Lq * Lk * (double)dmax >= (double)(1ll << 24);
+    return !mfma_as_is && dk > 0 && dv > 0 && dmax <= 256 && (double)B * H * Lq * Lk * (double)dmax >= (double)(1ll << 24);
 }
 
 // rows x d_src -> rows x d_dst: the common columns copied, the rest of a wider destination zeroed

@@ -557,7 +557,7 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
                         uint32_t flags);
 
 // Head dims the MFMA kernels do not take as they are (key dim != value dim, not a multiple of 4, tensors off the 16-byte
-// grid), up to 128 (256 without row statistics): the operands are copied into tensors of one padded head dim - zero columns change neither scores nor
+// grid), up to 256: the operands are copied into tensors of one padded head dim - zero columns change neither scores nor
 // outputs - the MFMA kernels run on the copies and the output's own columns are copied back.  Four streaming passes for
 // a kernel that is 30 - 40 times faster than the one-wavefront-per-row fallback (B8 H16 L2048 d72: 42 ms there).
 // Returns DL4S_HIP_EOOM without side effects when the copies cannot be allocated (the caller falls back).
@@ -631,10 +631,10 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
                           ((dk % 4 == 0 && aligned) ||
                            (dk % 2 == 0 && aligned8 && !token_major && ((Lq + BM - 1) / BM) * B * H >= 2ll * ctx->cu_count)) &&
                           Lk * (token_major ? H : 1) * dk * 4 < (1ll << 30);   // its 32-bit K/V offsets; beyond: the routes below
-    // head dims above 128 up to 256, forward only (no row statistics: the gradient kernels of these head dims read the plain
-    // kernel's): the 192- and 256-wide kernels
-    const bool wide_path = dk == dv && dk > HD2 && dk <= 256 && dk % 4 == 0 && aligned && !stats &&
-                           Lk * (token_major ? H : 1) * dk * 4 < ((dk == 192 || dk == 256) ? (1ll << 31) : (1ll << 30));
+    // head dims above 128 up to 256: the 192- and 256-wide kernels (the gradient call evaluates sdpa_wide_route on the same
+    // arguments)
+    const bool wide_as_is = dk == dv && aligned && dk > HD2 && dk <= 256 && dk % 4 == 0;   // never copied, whichever kernel it runs
+    const bool wide_path = wide_as_is && sdpa_wide_route(H, Lk, dk, token_major);
     // The 128-wide kernel on a launch that leaves CUs without their two workgroups: the key tiles of every block are dealt
     // to several workgroups, whose partial results a second kernel adds up (B4 H8 L512 d128: 73 us unsplit).  The count
     // depends on the extents only.
@@ -688,14 +688,14 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
         }
     }
     if (wide_path) {
-        if (dk <= 192) return launch_wide<192>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)dk);
-        return launch_wide<256>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)dk);
+        if (dk <= 192) return launch_wide<192>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+        return launch_wide<256>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
     }
     DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 128, and 16-byte aligned tensors");
     // Large enough to pay for four copies: the MFMA kernels on padded copies of the operands.  When row statistics are
     // asked for there is no falling back to the plain kernel: the gradient call decides by the same rule and reads the
     // statistics in the MFMA kernels' form.
-    if (sdpa_padded_route(false, B, H, Lq, Lk, dk, dv, stats ? HD2 : 256)) {
+    if (sdpa_padded_route(wide_as_is, B, H, Lq, Lk, dk, dv)) {
         const int rc = sdpa_forward_padded(ctx, q, k, v, out, stats, B, H, Lq, Lk, dk, dv, inv_temperature, mask, flags);
         if (stats || (rc != DL4S_HIP_EOOM && rc != DL4S_HIP_EUNSUPPORTED)) return rc;   // else: the plain kernel below
     }

@@ -13,8 +13,7 @@
 // SIMD; K/V in double-buffered LDS tiles of 32 keys on a (W + 4)-float row stride (4 x 32 x (W + 4) floats: 98 or 130 KiB,
 // one workgroup per CU).  With 2 x W/2 MFMAs per key tile against the same softmax work as the narrower kernels the matrix
 // pipe stays busy nonetheless.  Mask kinds, tile skipping, the token-major layout and the work order are those of the
-// 64-wide kernel; there is no key split over workgroups and no row statistics (the gradient kernels of these head dims read
-// the plain kernel's).
+// 64-wide kernel, the row statistics have the form every MFMA kernel leaves; there is no key split over workgroups.
 #pragma once
 #include "sdpa_common.h"
 
@@ -34,7 +33,8 @@ template <int KIND, int W>
 __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__restrict__ q, const float *__restrict__ k,
                                                                  const float *__restrict__ v, float *__restrict__ out, int H,
                                                                  int Lq, int Lk, float rT, MaskArgs mask, int strict, int nqb,
-                                                                 int total_blocks, int lpt, int token_major, int hd) {
+                                                                 int total_blocks, int lpt, int token_major,
+                                                                 float *__restrict__ stats, int hd) {
     using WT = WideFwdTile<W>;
     constexpr int LS = WT::LS, TF = WT::TF, NC = WT::NC, NC2 = WT::NC2, NP = WT::NP, PPR = WT::PPR;
     extern __shared__ __align__(16) float lds[];
@@ -208,6 +208,10 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
     // d = 128 + NC2*(8(r/4) + 4*half + r%4) + c.
     const float l_tot = l_run + xor32(l_run);
     const float inv = 1.0f / l_tot;
+    if (stats && half == 0 && qi < Lq) {      // for the gradient call: a weight is 2^(s - m_use) * inv
+        stats[2 * ((long long)bh * Lq + qi)] = m_use;
+        stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
+    }
     if (qi < Lq) {
         float *op = out + q_base + (long long)qi * rs;
 #pragma unroll
@@ -229,7 +233,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
 
 template <int KIND, int W>
 int launch_wide_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
-                     float rT, const MaskArgs &m, int strict, int token_major, int hd) {
+                     float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
     const int nqb = (Lq + BM - 1) / BM;
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
@@ -244,19 +248,19 @@ int launch_wide_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const fl
         dl4s::lds_limit_done(ctx, family, KIND);
     }
     hipLaunchKernelGGL((sdpa_prefill_f32_wide<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_bytes, ctx->stream, q, k, v,
-                       out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, hd);
+                       out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_wide");
 }
 
 template <int W>
 int launch_wide(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk, float rT,
-                const MaskArgs &m, int strict, int token_major, int hd) {
+                const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
     switch (m.kind) {
-        case DL4S_MASK_NONE: return launch_wide_kind<DL4S_MASK_NONE, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, hd);
-        case DL4S_MASK_DENSE_F32: return launch_wide_kind<DL4S_MASK_DENSE_F32, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, hd);
-        case DL4S_MASK_CAUSAL: return launch_wide_kind<DL4S_MASK_CAUSAL, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, hd);
-        case DL4S_MASK_KEY_LENGTHS: return launch_wide_kind<DL4S_MASK_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, hd);
-        default: return launch_wide_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, hd);
+        case DL4S_MASK_NONE: return launch_wide_kind<DL4S_MASK_NONE, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_DENSE_F32: return launch_wide_kind<DL4S_MASK_DENSE_F32, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_CAUSAL: return launch_wide_kind<DL4S_MASK_CAUSAL, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_KEY_LENGTHS: return launch_wide_kind<DL4S_MASK_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        default: return launch_wide_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
     }
 }
 

@@ -172,7 +172,9 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
                           int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv,
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
 
-/* Training form of the fused attention (key dim = value dim = d; MFMA kernels for d a multiple of 4 up to 128 and 16-byte aligned tensors, plain kernels up to 256).  The reference differentiates ScaledDotProductAttention through
+/* Training form of the fused attention (key dim = value dim = d; MFMA kernels for d a multiple of 4 up to 256 and 16-byte
+ * aligned tensors - above 128 the gradients are batched MFMA products around one elementwise pass, head-major layout only -
+ * plain kernels for what those do not take, up to 256).  The reference differentiates ScaledDotProductAttention through
  * the backward closures of its primitive operators (Tensor/Operators/Matrix.swift:139-174 for the products through the
  * subscript views and the stack of broadcastMatrixMultiplied :79-117, Binary.swift:235-300 for e / sum,
  * Reduce.swift:35-62, Unary.swift:33-55 for exp, Binary.swift:161-224 for the subtractions); a backend that fuses the
@@ -183,8 +185,8 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
  *   dl4s_hip_sdpa_bwd_f32        dq, dk, dv for the upstream gradient dout of out, from q, k, v, out, stats and the
  *                                same mask and flags as the forward call (the mask takes no gradient)
  * Layouts follow the forward call ([B,H,L,d], or [B,L,H,d] with DL4S_SDPA_TOKEN_MAJOR; stats is always [B,H,Lq,2]).
- * The gradient call takes the route the forward call took (MFMA kernels for d a multiple of 4 up to 128 with 16-byte
- * aligned q, k, v, out; the same kernels on zero-padded copies for other d up to 128 on large problems; the plain
+ * The gradient call takes the route the forward call took (MFMA kernels for d a multiple of 4 up to 256 with 16-byte
+ * aligned q, k, v, out; the same kernels on zero-padded copies for other d up to 256 on large problems; the plain
  * kernels otherwise) because the two kinds of kernels keep the statistics in different forms: pass both calls the same
  * tensors and extents.  On the direct MFMA route dout, dq, dk, dv must be 16-byte aligned too (DL4S_HIP_EUNSUPPORTED
  * otherwise).

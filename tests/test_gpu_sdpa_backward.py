@@ -583,3 +583,54 @@ def test_long_sequences_on_sampled_rows_and_columns(ctx, L, d, token_major):
             dk_c += dS.T @ Q[r0:r1] * rT
         np.testing.assert_allclose(dk[0, h][cols], dk_c, rtol=1e-4, atol=1e-4)
         np.testing.assert_allclose(dv[0, h][cols], dv_c, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("d", [256, 192, 132, 200])
+@pytest.mark.parametrize("B,H,Lq,Lk", [(2, 2, 200, 200), (1, 3, 70, 133), (2, 1, 1, 40), (1, 2, 129, 5)])
+@pytest.mark.parametrize("mask_kind", ["none", "dense", "lengths", "causal", "causal_lengths"])
+def test_gradients_for_head_dims_above_128(ctx, orc, monkeypatch, B, H, Lq, Lk, d, mask_kind):
+    """Head dims above 128 up to 256: the forward call leaves its statistics from the 192- / 256-wide kernels, the gradient
+    call composes batched products around one elementwise pass.  Parity with the oracle for every mask kind, including a
+    fully blocked row, and the same bits when the (batch, head) pairs are taken one per chunk."""
+    from dl4s_amd import lib
+    if mask_kind.startswith("causal") and Lq != Lk:
+        pytest.skip("causal masks are square here")
+    rng = np.random.default_rng(zlib.crc32(repr(("wide bwd", B, H, Lq, Lk, d, mask_kind)).encode()))
+    q, k, v, dout = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lq, d)
+    lens = rng.integers(1, Lk + 1, size=B)
+    kw, mask = {}, None
+    if mask_kind == "dense":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.3).astype(np.float32)
+        mask[0, 0, Lq // 2, :] = 1.0          # one fully blocked row: uniform weights
+        kw = dict(mask=mask)
+    elif mask_kind == "lengths":
+        mask, kw = lengths_mask(lens, Lk), dict(kind=lib.MASK_KEY_LENGTHS, lens=lens)
+    elif mask_kind == "causal":
+        mask, kw = causal_mask(Lq, Lq), dict(kind=lib.MASK_CAUSAL)
+    elif mask_kind == "causal_lengths":
+        mask = np.maximum(lengths_mask(lens, Lk), causal_mask(Lq, Lq)[None, None])
+        kw = dict(kind=lib.MASK_CAUSAL_OR_KEY_LENGTHS, lens=lens)
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, **kw)
+    assert_parity(out, orc.sdpa(q, k, v, mask), "forward with stats d=%d" % d)
+    rq, rk, rv = orc.sdpa_backward(q, k, v, mask, dout)
+    assert_parity(dq, rq, "dq d=%d %s" % (d, mask_kind))
+    assert_parity(dk, rk, "dk d=%d %s" % (d, mask_kind))
+    assert_parity(dv, rv, "dv d=%d %s" % (d, mask_kind))
+    monkeypatch.setenv("DL4S_HIP_BWD_SCRATCH_MAX_BYTES", "1")      # one pair per chunk
+    for a, b_ in zip(run_fwd_bwd(ctx, q, k, v, dout, **kw), (out, stats, dq, dk, dv)):
+        assert np.array_equal(a, b_)
+
+
+@pytest.mark.parametrize("d", [150, 255])
+def test_gradients_for_odd_head_dims_above_128_on_padded_copies(ctx, orc, d):
+    from dl4s_amd import lib
+    B, H, L = 2, 2, 260
+    rng = np.random.default_rng(d)
+    q, k, v, dout = (rand(rng, B, H, L, d) for _ in range(4))
+    mask = causal_mask(L, L)
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, kind=lib.MASK_CAUSAL)
+    assert_parity(out[:1, :1], orc.sdpa(q[:1, :1], k[:1, :1], v[:1, :1], mask), "forward d=%d" % d)
+    rq, rk, rv = orc.sdpa_backward(q[:1, :1], k[:1, :1], v[:1, :1], mask, dout[:1, :1])
+    assert_parity(dq[:1, :1], rq, "dq d=%d" % d)
+    assert_parity(dk[:1, :1], rk, "dk d=%d" % d)
+    assert_parity(dv[:1, :1], rv, "dv d=%d" % d)
