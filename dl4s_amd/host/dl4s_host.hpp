@@ -908,10 +908,10 @@ struct MultiHeadAttention {
           qDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})), kDense(Tensor::repeating(0.f, {hiddenDim_, keyDim_ * heads_})),
           vDense(Tensor::repeating(0.f, {hiddenDim_, valueDim_ * heads_})), fc(Tensor::repeating(0.f, {valueDim_ * heads_, hiddenDim_})),
           norm(Shape{hiddenDim_}), dropout(dropoutRate) {}
-    // fused mode, equal head dims that are a multiple of 4 up to 128 (what the token-major attention kernels take): the
+    // fused mode, equal head dims that are a multiple of 4 up to 256 (what the token-major attention kernels take): the
     // key / value projections alone, [B,L,H,d], for callers that attend to the same keys and values repeatedly (the
     // encoder states during greedy decoding)
-    bool canCacheProjections() const { return Device::fused() && keyDim == valueDim && keyDim <= 128 && keyDim % 4 == 0; }
+    bool canCacheProjections() const { return Device::fused() && keyDim == valueDim && keyDim <= 256 && keyDim % 4 == 0; }
     // The projections are separate products in the reference (MultiHeadAttention.swift:105-107); the key and value ones
     // (and the query one, when all three inputs have one length) go out as one grouped launch.
     std::pair<Tensor, Tensor> projectKeysValues(const Tensor &k, const Tensor &v, const Tensor *q = nullptr, Tensor *qp = nullptr) const {
@@ -958,7 +958,7 @@ struct MultiHeadAttention {
     }
     // ---- one new position against cached keys and values (no counterpart in the reference; fused mode, head dims
     // that are multiples of 4 up to 128, dropout inactive).  x [B,1,hidden].  With a single position the joint normalisation and the per-token one coincide.
-    bool canDecodeIncrementally() const { return canCacheProjections() && !dropout.isActive; }
+    bool canDecodeIncrementally() const { return canCacheProjections() && keyDim <= 128 && !dropout.isActive; }    // the decode kernel's rows
     Tensor finishStep(const Tensor &x, const Tensor &attended) const {
         const int64_t B = x.shape[0];
         Tensor sum(Device::Memory::allocateBuffer(Shape{B, 1, hiddenDim}));

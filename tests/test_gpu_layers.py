@@ -103,10 +103,10 @@ def test_tiny_transformer_layers(ctx, host, orc, fused):
 
 
 @pytest.mark.parametrize("fused", MODES)
-@pytest.mark.parametrize("dk", [96, 128, 12])
+@pytest.mark.parametrize("dk", [96, 128, 12, 192, 256, 140])
 def test_mha_with_other_head_dims(ctx, host, orc, fused, dk):
-    """Head dims other than 64: in fused mode the token-major attention kernels take every multiple of 4 up to 128 (the
-    64-wide and 128-wide MFMA kernels with padding columns)."""
+    """Head dims other than 64: in fused mode the token-major attention kernels take every multiple of 4 up to 256 (the
+    MFMA kernels of the next tile width with padding columns)."""
     B, L, Le, D, H = 2, 40, 50, 32, 2
     rng = np.random.default_rng(dk)
     attn, _ = m64.make_params(rng, D, H, dk, dk, 8)
