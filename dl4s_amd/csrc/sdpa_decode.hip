@@ -30,7 +30,7 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int MAXD = 128;                     // widest cache row the kernels take
+constexpr int MAXD = 256;                     // widest cache row the kernels take
 constexpr float LOG2E = 1.44269504088896340736f;
 // floats per partial record: o[0 .. D-1], m, l, pad (D = the row width the kernel instance covers: 32, 64 or 128)
 constexpr int pstr(int D) { return D + 4; }
@@ -67,8 +67,8 @@ __device__ __forceinline__ float row_sum(float x) {
 // least one key left their weights are exactly zero and they are not visited at all; a length of zero or less blocks every
 // key, the penalty is applied to all of them and the row comes out uniform, as in the reference.
 // SEG: the row is read as SEG consecutive segments of 4 * LPR floats by the same LPR lanes (SEG loads per row and lane, NK =
-// 4 keys per lane and iteration instead of 8).  SEG = 3 with LPR = 8 serves rows of 96 floats with every lane busy, where the
-// 32-lane form would leave a quarter of the lanes idle.
+// 4 keys per lane and iteration instead of 8).  SEG = 3 with LPR = 8 (16) serves rows of 96 (192) floats with every lane busy,
+// where the one-piece form would leave a quarter of the lanes idle; SEG = 2 with LPR = 32 serves rows of 129 to 256 floats.
 template <bool APPEND, int NW, int LPR, bool FULL, bool DEVPOS = false, int SEG = 1>
 __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
                                                                    float *vcache, const float *__restrict__ k_new,
@@ -320,12 +320,12 @@ __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restr
     vcache[dst] = v_new[i];
 }
 
-// Row widths the kernel is instantiated for: 32, 64, 128 floats (8, 16, 32 lanes per row, one 128-bit piece per lane) and 96
-// floats (8 lanes per row, three pieces per lane).
-// (the 96-float form for exactly 96 floats and 128-bit pieces: with part-filled or narrower pieces its three loads per lane
+// Row widths the kernel is instantiated for: 32, 64, 128 floats (8, 16, 32 lanes per row, one 128-bit piece per lane), 96 and
+// 192 floats (8 and 16 lanes per row, three pieces per lane) and 256 floats (32 lanes per row, two pieces per lane).
+// (the three-piece forms for exactly 96 or 192 floats and 128-bit pieces: with part-filled or narrower pieces its three loads per lane
 // cost more than the idle lanes of the 128-float form - B16 H16 over 4096 rows: d = 96 163 -> 137 us, d = 80 160 -> 175 us)
-inline int row_segments(int64_t d, int vec) { return d == 96 && vec == 4 ? 3 : 1; }
-inline int lanes_per_row(int64_t d, int vec) { return d <= 32 ? 8 : (d <= 64 ? 16 : (row_segments(d, vec) == 3 ? 8 : 32)); }
+inline int row_segments(int64_t d, int vec) { return (d == 96 || d == 192) && vec == 4 ? 3 : (d > 128 ? 2 : 1); }
+inline int lanes_per_row(int64_t d, int vec) { return row_segments(d, vec) == 3 ? (int)d / 12 : (d <= 32 ? 8 : (d <= 64 ? 16 : 32)); }
 inline int row_width(int64_t d, int vec) { return 4 * lanes_per_row(d, vec) * row_segments(d, vec); }
 inline int keys_per_iteration(int64_t d, int vec) { return (row_segments(d, vec) == 1 ? 8 : 4) * (64 / lanes_per_row(d, vec)); }
 
@@ -342,11 +342,11 @@ template <bool APPEND, int NW, int LPR, bool DEVPOS, int SEG = 1>
 void decode_launch_kernel(dl4s_hip_ctx *ctx, dim3 grid, const float *q, float *kcache, float *vcache, const float *k_new,
                           const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
                           int d, int H, const int *lengths, const int *pos_dev, int vec) {
-    if (SEG > 1 || (d == 4 * LPR && vec == 4))      // the segmented form is only chosen for full rows
+    if (SEG == 3 || (d == 4 * LPR * SEG && vec == 4))      // the 96-float form is only chosen for full rows
         hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, true, DEVPOS, SEG>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
                            k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, 4);
-    else if constexpr (SEG == 1)
-        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, false, DEVPOS, 1>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
+    else if constexpr (SEG != 3)
+        hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, false, DEVPOS, SEG>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
                            k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, vec);
 }
 
@@ -355,8 +355,12 @@ void decode_launch_width(dl4s_hip_ctx *ctx, int nw, dim3 grid, const float *q, f
                          const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
                          int d, int H, const int *lengths, const int *pos_dev, int vec) {
 #define DL4S_DECODE_ARGS ctx, grid, q, kcache, vcache, k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, vec
-    if (row_segments(d, vec) == 3) {
+    if (row_segments(d, vec) == 3 && d == 96) {
         if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS, 3>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS, 3>(DL4S_DECODE_ARGS);
+    } else if (row_segments(d, vec) == 3) {
+        if (nw == 16) decode_launch_kernel<APPEND, 16, 16, DEVPOS, 3>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 16, DEVPOS, 3>(DL4S_DECODE_ARGS);
+    } else if (row_segments(d, vec) == 2) {
+        if (nw == 16) decode_launch_kernel<APPEND, 16, 32, DEVPOS, 2>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 32, DEVPOS, 2>(DL4S_DECODE_ARGS);
     } else switch (lanes_per_row(d, vec)) {
         case 8: if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS>(DL4S_DECODE_ARGS); break;
         case 16: if (nw == 16) decode_launch_kernel<APPEND, 16, 16, DEVPOS>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 16, DEVPOS>(DL4S_DECODE_ARGS); break;

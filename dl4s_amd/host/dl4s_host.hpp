@@ -957,8 +957,8 @@ struct MultiHeadAttention {
         return normalized(out_drop, &q);
     }
     // ---- one new position against cached keys and values (no counterpart in the reference; fused mode, head dims
-    // that are multiples of 4 up to 128, dropout inactive).  x [B,1,hidden].  With a single position the joint normalisation and the per-token one coincide.
-    bool canDecodeIncrementally() const { return canCacheProjections() && keyDim <= 128 && !dropout.isActive; }    // the decode kernel's rows
+    // that are multiples of 4 up to 256, dropout inactive).  x [B,1,hidden].  With a single position the joint normalisation and the per-token one coincide.
+    bool canDecodeIncrementally() const { return canCacheProjections() && !dropout.isActive; }
     Tensor finishStep(const Tensor &x, const Tensor &attended) const {
         const int64_t B = x.shape[0];
         Tensor sum(Device::Memory::allocateBuffer(Shape{B, 1, hiddenDim}));
@@ -1310,7 +1310,7 @@ struct Transformer {
     std::vector<int32_t> greedyCached(const std::vector<int32_t> &inputSequence, int32_t startToken, int32_t endToken, int64_t maxLength,
                                       std::vector<float> *lastLogits = nullptr, bool recorded = true) const {
         precondition(canDecodeIncrementally(),
-                     "cached decoding needs fused mode, inactive dropout, equal key and value dims that are a multiple of 4 up to 128, and attention layers that normalise per token");
+                     "cached decoding needs fused mode, inactive dropout, equal key and value dims that are a multiple of 4 up to 256, and attention layers that normalise per token");
         const int64_t n = (int64_t)inputSequence.size(), D = embedding.outputSize(), vocab = embedding.embeddingMatrix.shape[0];
         precondition(startToken >= 0 && startToken < vocab, "index out of bounds");
         std::vector<int32_t> tokens;

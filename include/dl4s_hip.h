@@ -203,7 +203,7 @@ int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
                           int64_t Lq, int64_t Lk, int64_t d, float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
 
 /* One decode step: the same attention with Lq = 1 over the first T rows of a key/value cache laid
- * out [B,H,Tcap,d] (d from 1 to 128; the kernel is instantiated for rows of 32, 64, 96 and 128 floats and other
+ * out [B,H,Tcap,d] (d from 1 to 256; the kernel is instantiated for rows of 32, 64, 96, 128 and 256 floats and other
  * head dims run the next wider one with idle lanes; with d a multiple of 4 and q, the caches and the new rows 16-byte
  * aligned a lane reads its piece of a row with one 128-bit load, otherwise with 64-bit loads (d even, 8-byte aligned) or one
  * float at a time).  q, out [B,H,1,d].  The reference has no cache (greedy decoding re-runs
