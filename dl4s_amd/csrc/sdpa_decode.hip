@@ -21,7 +21,7 @@
 // Partial records of dl4s_hip_sdpa_decode_noalloc_f32: a fixed block in the code object's own device memory (one copy per
 // GPU, held until the process ends), so that entry point never asks the driver for memory.  Host code must not pass this
 // name to a kernel: it uses the device address hipGetSymbolAddress returns (dl4s::decode_static_scratch_init).
-constexpr size_t NOALLOC_SCRATCH_FLOATS = size_t(1) << 19;   // 2 MiB
+constexpr size_t NOALLOC_SCRATCH_FLOATS = size_t(1) << 20;   // 4 MiB
 static __device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
 // Serialises the two launches of a split decode on the fixed block between host threads (whatever their context).
 static std::mutex g_static_scratch_mu;

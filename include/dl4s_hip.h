@@ -223,11 +223,11 @@ int dl4s_hip_sdpa_decode_lengths_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                                      float inv_temperature, const int32_t *lengths);
 /* dl4s_hip_sdpa_decode_f32 for callers that cannot allocate device memory: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels, same bits;
- * the partial records of a decode that is split over the keys live in a fixed 2 MiB block of the library's own device
+ * the partial records of a decode that is split over the keys live in a fixed 4 MiB block of the library's own device
  * memory (one per GPU, held until the process ends) instead of the context's growable scratch block, and the call
  * makes no allocating or freeing runtime call.  A problem whose records do not fit - B*H pairs times the number of key
- * splits times (d + 4) floats above 2 MiB - is refused with DL4S_HIP_EUNSUPPORTED; the split rule aims at 16 wavefronts
- * per compute unit, so on a 256-CU GPU it asks for about 2048 records (1 MiB at d = 128) at most and the limit guards
+ * splits times (the row width the kernel runs at + 4) floats above 4 MiB - is refused with DL4S_HIP_EUNSUPPORTED; the split rule aims at 16 wavefronts
+ * per compute unit, so on a 256-CU GPU it asks for about 2048 records (2.1 MiB at d = 256) at most and the limit guards
  * larger GPUs.  Every call on a GPU shares that GPU's block: calls on one context are ordered by its stream; calls on
  * different contexts of the same GPU that overlap in time race.  Nothing in the block has to start at zero (every
  * record a call reads was written by that call). */

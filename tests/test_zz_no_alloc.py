@@ -18,21 +18,22 @@ def ctx():
     c.close()
 
 
-def _case(ctx, orc, seed, B, H, T, Tcap):
+def _case(ctx, orc, seed, B, H, T, Tcap, d=64):
     rng = np.random.default_rng(seed)
-    q = rng.standard_normal((B, H, 1, 64)).astype(np.float32)
-    kc = rng.standard_normal((B, H, Tcap, 64)).astype(np.float32)
-    vc = rng.standard_normal((B, H, Tcap, 64)).astype(np.float32)
+    q = rng.standard_normal((B, H, 1, d)).astype(np.float32)
+    kc = rng.standard_normal((B, H, Tcap, d)).astype(np.float32)
+    vc = rng.standard_normal((B, H, Tcap, d)).astype(np.float32)
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))     # 0.125 at d = 64
     kc[:, :, T:] = np.nan     # rows beyond T are never read
     vc[:, :, T:] = np.nan
     dq, dk, dv = ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc)
-    out_a, out_b = ctx.empty((B, H, 1, 64)), ctx.empty((B, H, 1, 64))
-    ctx.fill(float("nan"), out_a, B * H * 64)
-    ctx.fill(float("nan"), out_b, B * H * 64)
+    out_a, out_b = ctx.empty((B, H, 1, d)), ctx.empty((B, H, 1, d))
+    ctx.fill(float("nan"), out_a, B * H * d)
+    ctx.fill(float("nan"), out_b, B * H * d)
     in_use, pooled = ctx.mem_stats()
-    ctx.sdpa_decode_noalloc(dq, dk, dv, out_a, B, H, T, Tcap, 64, 0.125)
+    ctx.sdpa_decode_noalloc(dq, dk, dv, out_a, B, H, T, Tcap, d, rT)
     assert ctx.mem_stats() == (in_use, pooled)       # the pool was not touched
-    ctx.sdpa_decode(dq, dk, dv, out_b, B, H, T, Tcap, 64, 0.125)
+    ctx.sdpa_decode(dq, dk, dv, out_b, B, H, T, Tcap, d, rT)
     a, b = out_a.numpy(), out_b.numpy()
     for buf in (dq, dk, dv, out_a, out_b):
         buf.release()
@@ -44,6 +45,8 @@ def test_no_alloc_decode_two_calls_the_second_smaller(ctx, orc):
     _case(ctx, orc, 1, 2, 4, 3000, 3072)     # 8 pairs: split over many workgroups, records in the fixed block
     _case(ctx, orc, 2, 1, 2, 700, 700)       # fewer pairs, fewer splits: most of the block keeps the first call's records
     _case(ctx, orc, 3, 2, 2, 300, 320)       # a short cache: one workgroup per pair, the block is not used at all
+    _case(ctx, orc, 4, 2, 4, 3000, 3072, d=256)     # the widest rows: the largest records
+    _case(ctx, orc, 5, 1, 3, 900, 900, d=96)
 
 
 def test_no_alloc_decode_error_paths(ctx):
