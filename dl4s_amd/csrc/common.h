@@ -68,6 +68,11 @@ int ensure_scratch(dl4s_hip_ctx *ctx, size_t bytes);
 // out [item][nblk][2]); x and y may be the same tensor.  The caller holds the scratch mutex when `part` lies there.
 int layernorm_apply(dl4s_hip_ctx *ctx, const float *x, const float *scale, const float *shift, float *y, const float *part,
                     long long items, long long n, long long D, int nblk);
+// dl4s_hip_gemm_batched_f32 for callers inside the library whose batch fills the GPU by itself: always the tiled kernels,
+// never the skinny form that a single product of the shape would take (so not the bits of the public entry for such shapes).
+int gemm_batched_tiled(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols, int64_t lhs_stride, const float *rhs,
+                       int64_t rhs_rows, int64_t rhs_cols, int64_t rhs_stride, float *result, int64_t result_stride, int64_t batch,
+                       float alpha, float beta, int transpose_first, int transpose_second);
 // Looks up the device address of the decode kernels' fixed scratch block (sdpa_decode.hip) for the current GPU.
 int decode_static_scratch_init(dl4s_hip_ctx *ctx);
 

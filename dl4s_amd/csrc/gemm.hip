@@ -612,7 +612,7 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
                 int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb,
                 const float *bias = nullptr, const float *residual = nullptr, int act = 0, const float *const *group_lhs = nullptr,
                 const float *const *group_rhs = nullptr, float *const *group_result = nullptr, float *ln_part = nullptr,
-                int64_t ln_item_rows = 0, int *ln_nblk = nullptr) {
+                int64_t ln_item_rows = 0, int *ln_nblk = nullptr, bool tiled_only = false) {
     // group_*: `batch` (at most 4) products of one shape with unrelated operand addresses, in one launch
     // ln_part: also leave LayerNorm partial sums over items of ln_item_rows rows (see GemmArgs); *ln_nblk receives the
     // number of pairs per item.  A product that does not run on the tiled kernels with whole tiles per item, or would
@@ -663,7 +663,9 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     const auto rows_by_k_any = [&](int64_t ld) { return K % 4 == 0 && ld % 4 == 0; };
     const bool few_rows = M <= 128 && ((M + 63) / 64) * ((N + 63) / 64) < ctx->cu_count;
     const bool few_blocks = ((M + 31) / 32) * ((N + 31) / 32) <= 2 * ctx->cu_count;
-    const bool skinny = !ta && K >= 64 && (few_rows || few_blocks) && rows_by_k_any(lc) &&
+    // tiled_only: a caller inside the library with a batch that fills the GPU by itself (the skinny rule looks at one
+    // product's shape, which says nothing about such a launch)
+    const bool skinny = !tiled_only && !ta && K >= 64 && (few_rows || few_blocks) && rows_by_k_any(lc) &&
                         (tb ? rows_by_k_any(rc) : true) && aligned16(lhs) && (!tb || aligned16(rhs)) && lbs % 4 == 0 &&
                         (!tb || rbs % 4 == 0) && group_aligned && M * N * batch < (1ll << 31) && K * (tb ? 1 : rc) < (1ll << 31);
     if (ln_part && (skinny || !fast)) return GEMM_LN_NOT_FUSED;
@@ -767,6 +769,17 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
 }
 
 }  // namespace
+
+namespace dl4s {
+
+int gemm_batched_tiled(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols, int64_t lhs_stride, const float *rhs,
+                       int64_t rhs_rows, int64_t rhs_cols, int64_t rhs_stride, float *result, int64_t result_stride, int64_t batch,
+                       float alpha, float beta, int transpose_first, int transpose_second) {
+    return gemm_launch(ctx, lhs, lhs_rows, lhs_cols, lhs_stride, rhs, rhs_rows, rhs_cols, rhs_stride, result, result_stride, batch, alpha,
+                       beta, transpose_first, transpose_second, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0, nullptr, true);
+}
+
+}  // namespace dl4s
 
 extern "C" {
 

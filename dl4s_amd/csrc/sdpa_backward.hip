@@ -1171,7 +1171,8 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                  "sdpa backward: the rows of one (batch, head) pair span more than 2 GiB (1 GiB for head dims below 64)");
     if (wide_path) {
         DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa backward: the token-major layout needs a head dim of at most 128");
-        return sdpa_backward_wide(ctx, q, k, v, out, stats, dout, dq, dk, dv, B, H, Lq, Lk, d, inv_temperature, mask, ds_scratch_max_bytes());
+        return sdpa_backward_wide(ctx, q, k, v, out, stats, dout, dq, dk, dv, B, H, Lq, Lk, d, inv_temperature, mask,
+                                  (flags & DL4S_SDPA_STRICT) ? 1 : 0, ds_scratch_max_bytes());
     }
     std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
     MaskArgs m{};

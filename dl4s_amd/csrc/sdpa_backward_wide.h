@@ -11,8 +11,10 @@
 //
 // (Tensor/Operators/Matrix.swift:139-174, Binary.swift:235-300, Unary.swift:33-55, Reduce.swift:35-62 give the same
 // gradients closure by closure.)  The (batch, head) pairs are taken in chunks whose two score tensors stay inside the
-// gradient scratch bound.  Every key is visited, blocked or not (the behaviour of DL4S_SDPA_STRICT).  Deterministic: no
-// atomics, every sum in a fixed order.
+// gradient scratch bound.  Under the plain causal mask (without DL4S_SDPA_STRICT) the queries go in blocks of 512 rows
+// that contract only the keys up to their last row - the weights beyond are exactly zero - and add their dk / dv
+// contributions block after block; every other mask kind visits every key.  Deterministic: no atomics, every sum in a fixed
+// order.
 #pragma once
 #include "sdpa_common.h"
 
@@ -27,13 +29,15 @@ __global__ __launch_bounds__(256) void sdpa_bwd_wide_scale_q(const float *__rest
     }
 }
 
-// One workgroup per query row of a chunk: S2 -> P and dP -> dS in place.  pair0: the chunk's first (batch, head) pair.
+// One workgroup per query row of a block of a chunk: S2 -> P and dP -> dS in place.  pair0: the chunk's first (batch, head)
+// pair; the block holds the query rows i0 .. i0 + nq - 1 of every pair against the keys 0 .. Lk - 1 (Lk: the block's key
+// count, the row length of S and dP).
 __global__ __launch_bounds__(256) void sdpa_bwd_wide_weights(float *__restrict__ S, float *__restrict__ dP, const float *__restrict__ stats,
                                                              const float *__restrict__ D, MaskArgs mask, long long pair0, int H, int Lq,
-                                                             int Lk) {
-    const long long row = blockIdx.x;                 // over the chunk's pairs x Lq
-    const long long bh = pair0 + row / Lq;
-    const int qi = (int)(row % Lq);
+                                                             int i0, int nq, int Lk) {
+    const long long row = blockIdx.x;                 // over the chunk's pairs x nq
+    const long long bh = pair0 + row / nq;
+    const int qi = i0 + (int)(row % nq);
     const int b = (int)(bh / H), hh = (int)(bh % H);
     const long long grow = bh * Lq + qi;              // row of the whole problem: statistics and D
     const float m = stats[2 * grow], inv = stats[2 * grow + 1], Di = D[grow];
@@ -54,7 +58,7 @@ __global__ __launch_bounds__(256) void sdpa_bwd_wide_weights(float *__restrict__
 
 int sdpa_backward_wide(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, const float *out, const float *stats,
                        const float *dout, float *dq, float *dk, float *dv, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t d,
-                       float rT, const dl4s_mask_desc *mask, long long scratch_max_bytes) {
+                       float rT, const dl4s_mask_desc *mask, int strict, long long scratch_max_bytes) {
     MaskArgs m{};
     int rc = build_mask_args(ctx, mask, B, H, Lq, Lk, false, m);
     if (rc != DL4S_HIP_OK) return rc;
@@ -77,28 +81,49 @@ int sdpa_backward_wide(dl4s_hip_ctx *ctx, const float *q, const float *k, const 
           *D = static_cast<float *>(bufs[3]);
     hipLaunchKernelGGL(sdpa_bwd_rowdot_plain, dim3((unsigned)(pairs * Lq)), dim3(64), 0, ctx->stream, out, dout, D, (int)d);
     rc = dl4s::launch_status("sdpa_bwd_rowdot_plain");
+    // A product whose own shape would send it to the skinny kernels (few output blocks) comes here with a batch of pairs: when
+    // the batch as a whole has more blocks than that rule's bound, the tiled kernels take it.
+    const auto gemm = [&](dl4s_hip_ctx *c, const float *a, int64_t ar, int64_t ac, int64_t as, const float *b, int64_t br, int64_t bc,
+                          int64_t bs, float *r, int64_t rs, int64_t n, float alpha, float beta, int ta, int tb) {
+        const int64_t M = ta ? ac : ar, N = tb ? br : bc;
+        if (n * ((M + 31) / 32) * ((N + 31) / 32) > 2ll * c->cu_count)
+            return dl4s::gemm_batched_tiled(c, a, ar, ac, as, b, br, bc, bs, r, rs, n, alpha, beta, ta, tb);
+        return dl4s_hip_gemm_batched_f32(c, a, ar, ac, as, b, br, bc, bs, r, rs, n, alpha, beta, ta, tb);
+    };
+    // the plain causal mask: blocks of query rows against the keys up to the block's last row (with key lengths a sequence
+    // of length zero spreads its weights over every key, so that kind visits them all)
+    const bool blocks = m.kind == DL4S_MASK_CAUSAL && !strict && Lq > 512;
+    const int64_t QB = blocks ? 512 : Lq;
     for (int64_t p0 = 0; p0 < pairs && rc == DL4S_HIP_OK; p0 += chunk) {
         const int64_t n = std::min(chunk, pairs - p0);
         const float *qc = q + p0 * Lq * d, *kc = k + p0 * Lk * d, *vc = v + p0 * Lk * d, *gc = dout + p0 * Lq * d;
+        float *dqc = dq + p0 * Lq * d, *dkc = dk + p0 * Lk * d, *dvc = dv + p0 * Lk * d;
         const long long n4 = n * Lq * d / 4;
         hipLaunchKernelGGL(sdpa_bwd_wide_scale_q, dim3((unsigned)std::min<long long>((n4 + 255) / 256, 65536)), dim3(256), 0, ctx->stream, qc,
                            qs, n4, rT);
         rc = dl4s::launch_status("sdpa_bwd_wide_scale_q");
-        if (rc == DL4S_HIP_OK)      // S2 = qs . k^T
-            rc = dl4s_hip_gemm_batched_f32(ctx, qs, Lq, d, Lq * d, kc, Lk, d, Lk * d, S, Lq * Lk, n, 1.0f, 0.0f, 0, 1);
-        if (rc == DL4S_HIP_OK)      // dP = dout . v^T
-            rc = dl4s_hip_gemm_batched_f32(ctx, gc, Lq, d, Lq * d, vc, Lk, d, Lk * d, dP, Lq * Lk, n, 1.0f, 0.0f, 0, 1);
-        if (rc == DL4S_HIP_OK) {
-            hipLaunchKernelGGL(sdpa_bwd_wide_weights, dim3((unsigned)(n * Lq)), dim3(256), 0, ctx->stream, S, dP, stats, D, m, (long long)p0,
-                               (int)H, (int)Lq, (int)Lk);
-            rc = dl4s::launch_status("sdpa_bwd_wide_weights");
+        if (blocks && rc == DL4S_HIP_OK) rc = dl4s_hip_fill_f32(ctx, 0.f, dkc, n * Lk * d);     // the blocks add into dk and dv
+        if (blocks && rc == DL4S_HIP_OK) rc = dl4s_hip_fill_f32(ctx, 0.f, dvc, n * Lk * d);
+        for (int64_t i0 = 0; i0 < Lq && rc == DL4S_HIP_OK; i0 += QB) {
+            const int64_t nq = std::min(QB, Lq - i0);
+            const int64_t nk = blocks ? std::min(Lk, i0 + nq) : Lk;      // keys beyond the block's last row are blocked for all of it
+            const float beta = blocks ? 1.0f : 0.0f;
+            // S2 = qs . k^T
+            rc = gemm(ctx, qs + i0 * d, nq, d, Lq * d, kc, nk, d, Lk * d, S, nq * nk, n, 1.0f, 0.0f, 0, 1);
+            if (rc == DL4S_HIP_OK)      // dP = dout . v^T
+                rc = gemm(ctx, gc + i0 * d, nq, d, Lq * d, vc, nk, d, Lk * d, dP, nq * nk, n, 1.0f, 0.0f, 0, 1);
+            if (rc == DL4S_HIP_OK) {
+                hipLaunchKernelGGL(sdpa_bwd_wide_weights, dim3((unsigned)(n * nq)), dim3(256), 0, ctx->stream, S, dP, stats, D, m, (long long)p0,
+                                   (int)H, (int)Lq, (int)i0, (int)nq, (int)nk);
+                rc = dl4s::launch_status("sdpa_bwd_wide_weights");
+            }
+            if (rc == DL4S_HIP_OK)      // dv (+)= P^T . dout
+                rc = gemm(ctx, S, nq, nk, nq * nk, gc + i0 * d, nq, d, Lq * d, dvc, Lk * d, n, 1.0f, beta, 1, 0);
+            if (rc == DL4S_HIP_OK)      // dk (+)= rT * dS^T . q
+                rc = gemm(ctx, dP, nq, nk, nq * nk, qc + i0 * d, nq, d, Lq * d, dkc, Lk * d, n, rT, beta, 1, 0);
+            if (rc == DL4S_HIP_OK)      // dq = rT * dS . k
+                rc = gemm(ctx, dP, nq, nk, nq * nk, kc, nk, d, Lk * d, dqc + i0 * d, Lq * d, n, rT, 0.0f, 0, 0);
         }
-        if (rc == DL4S_HIP_OK)      // dv = P^T . dout
-            rc = dl4s_hip_gemm_batched_f32(ctx, S, Lq, Lk, Lq * Lk, gc, Lq, d, Lq * d, dv + p0 * Lk * d, Lk * d, n, 1.0f, 0.0f, 1, 0);
-        if (rc == DL4S_HIP_OK)      // dk = rT * dS^T . q
-            rc = dl4s_hip_gemm_batched_f32(ctx, dP, Lq, Lk, Lq * Lk, qc, Lq, d, Lq * d, dk + p0 * Lk * d, Lk * d, n, rT, 0.0f, 1, 0);
-        if (rc == DL4S_HIP_OK)      // dq = rT * dS . k
-            rc = dl4s_hip_gemm_batched_f32(ctx, dP, Lq, Lk, Lq * Lk, kc, Lk, d, Lk * d, dq + p0 * Lq * d, Lq * d, n, rT, 0.0f, 0, 0);
     }
     // the pool hands a block out again only to work enqueued later on the same stream
     for (int i = 0; i < 4; ++i) (void)dl4s_hip_free(ctx, bufs[i]);

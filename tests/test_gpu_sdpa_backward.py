@@ -634,3 +634,21 @@ def test_gradients_for_odd_head_dims_above_128_on_padded_copies(ctx, orc, d):
     assert_parity(dq[:1, :1], rq, "dq d=%d" % d)
     assert_parity(dk[:1, :1], rk, "dk d=%d" % d)
     assert_parity(dv[:1, :1], rv, "dv d=%d" % d)
+
+
+@pytest.mark.parametrize("d,Lq,Lk", [(256, 1100, 1100), (192, 1300, 700), (160, 600, 1000)])
+def test_causal_gradients_above_head_dim_128_in_query_blocks(ctx, orc, d, Lq, Lk):
+    """Long causal problems at head dims above 128 take the queries in blocks of 512 rows that skip the keys beyond their
+    last row: against the oracle on one (batch, head) pair, and against the same call visiting every key."""
+    from dl4s_amd import lib
+    B, H = 1, 2
+    rng = np.random.default_rng(d + Lq)
+    q, k, v, dout = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lq, d)
+    mask = causal_mask(Lq, Lk)
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, kind=lib.MASK_CAUSAL)
+    rq, rk, rv = orc.sdpa_backward(q[:, 1:], k[:, 1:], v[:, 1:], mask, dout[:, 1:])
+    assert_parity(dq[:, 1:], rq, "dq d=%d" % d)
+    assert_parity(dk[:, 1:], rk, "dk d=%d" % d)
+    assert_parity(dv[:, 1:], rv, "dv d=%d" % d)
+    for a, b_ in zip(run_fwd_bwd(ctx, q, k, v, dout, kind=lib.MASK_CAUSAL, strict=True)[2:], (dq, dk, dv)):
+        assert_parity(b_, a, "blocks vs every key")
