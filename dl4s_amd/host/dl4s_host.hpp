@@ -18,6 +18,9 @@
 //   true   the layers take the backend's fused entry points where it has them: one fused attention launch in
 //          ScaledDotProductAttention, one strided-batched gemm per broadcastMatrixMultiplied, fused
 //          residual + LayerNorm, fused bias + GELU.
+// HIP::attentionHook() with fused() == false is the reference with nothing but the fused-attention hook patched into
+// ScaledDotProductAttention.callAsFunction: that layer makes its one fused call on the [B,H,L,d] tensors it is handed,
+// every other operator issues the reference's engine calls.
 #pragma once
 
 #include <algorithm>
@@ -84,6 +87,10 @@ struct HIP {
     }
     static bool &fused() {
         static bool f = true;
+        return f;
+    }
+    static bool &attentionHook() {
+        static bool f = false;
         return f;
     }
     // Fused attention only.  false: key tiles that the mask blocks entirely are skipped (their weights are exactly zero;
@@ -867,7 +874,7 @@ struct ScaledDotProductAttention {
     explicit ScaledDotProductAttention(float t) : temperature(t) {}
     Tensor operator()(const Tensor &q, const Tensor &k, const Tensor &v, const Tensor *mask) const {
         precondition(k.dim() == 4, "k must have 4 dimensions");
-        if (Device::fused()) {
+        if (Device::fused() || Device::attentionHook()) {
             precondition(q.dim() == 4 && v.dim() == 4 && q.shape[0] == k.shape[0] && q.shape[1] == k.shape[1] &&
                              v.shape[0] == k.shape[0] && v.shape[1] == k.shape[1] && q.shape[3] == k.shape[3] && k.shape[2] == v.shape[2],
                          "Matmul operands must have matching shapes");

@@ -20,8 +20,9 @@ int guarded(dl4s_hip_ctx *ctx, int fused, const std::function<void()> &body) {
         return -1;
     }
     HIP::context() = ctx;
-    HIP::fused() = fused != 0;
-    HIP::strictMasks() = fused == 2;
+    HIP::fused() = fused == 1 || fused == 2;
+    HIP::strictMasks() = fused == 2 || fused == 4;
+    HIP::attentionHook() = fused == 3 || fused == 4;
     try {
         body();
         return 0;

@@ -8,7 +8,9 @@
  * `fused` selects the execution mode of the host layer: 0 issues exactly the engine primitive calls the
  * reference's tensor operators issue; 1 lets the layers use the backend's fused entry points; 2 is 1 with
  * DL4S_SDPA_STRICT on every attention call (no tile skipping: NaN / Inf in keys or values at blocked
- * positions then reach the output as in the reference).
+ * positions then reach the output as in the reference); 3 is 0 with the fused attention call in
+ * ScaledDotProductAttention only - what a DL4S checkout gets from the engine conformance plus the hook in
+ * ScaledDotProductAttention.callAsFunction, every other layer untouched - and 4 is 3 with DL4S_SDPA_STRICT.
  * A mask pointer may be NULL (no mask); mshape/mdim describe the mask tensor handed to the layer
  * (float, 1 = blocked), which must be broadcastable to [B,H,Lq,Lk].
  */

@@ -30,7 +30,8 @@ def host():
     return host_lib
 
 
-MODES = [pytest.param(False, id="primitive"), pytest.param(True, id="fused"), pytest.param(2, id="fused_strict")]
+MODES = [pytest.param(False, id="primitive"), pytest.param(True, id="fused"), pytest.param(2, id="fused_strict"),
+         pytest.param(3, id="attention_hook_only"), pytest.param(4, id="attention_hook_only_strict")]
 
 
 def test_mask_builders_match_oracle_exactly(ctx, host, orc):
