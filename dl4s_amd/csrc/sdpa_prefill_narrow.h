@@ -6,7 +6,7 @@
 //   S^T   the two halves of the wavefront contract d = s and d = W/2 + s in step s: W/2 MFMAs (16 or 8 instead of 32)
 //   O^T   one 32 x 32 accumulator (row = d, column = query) instead of two: 16 MFMAs instead of 32; V is read a float at a
 //         time (row = key, column = the lane's d); rows at or beyond the head dim are computed on whatever follows in LDS
-//         and never stored
+//         and never stored.  The main 16-wide kernel uses two 16 x 16 accumulators instead (attend_tile_16).
 // Everything else - the transposed products that keep the weights in the registers they were computed in, the mask in
 // registers, the online softmax with a lazy reference maximum, tile skipping, the work order, the token-major layout, the
 // row statistics for the gradient kernels - is the 64-wide kernels'.  The summation order over d differs from theirs, so
@@ -61,6 +61,54 @@ __device__ __forceinline__ void attend_tile_narrow(const float *Kb, const float 
     // O^T += V^T . P^T: A operand = V[key 8(r/4) + 4*half + r%4][d = ln]
 #pragma unroll
     for (int r = 0; r < 16; ++r) o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(Vb[(8 * (r >> 2) + (r & 3)) * LS], s0[r], o0, 0, 0, 0);
+}
+
+// The 16-wide tile in the main kernel: O^T on 16 x 16 x 4 MFMAs, so that no accumulator row is idle (a 32 x 32 accumulator
+// of a 16-wide head is half empty: 16 MFMAs of 64 cycles against 16 of 32 cycles here).  og[0] holds the queries q0 .. q0+15,
+// og[1] q0+16 .. q0+31; lane: column = lane % 16, rows d = 4 * (lane / 16) + i.  The weights leave the score product with
+// lane = query (lane % 32) and 16 keys in registers; v_permlane16_swap of a register pair (2p, 2p+1) puts, for both groups
+// at once, the weight of key 8(p/2) + 2(p%2) + (s&1) + 4(s>>1) of query lane % 16 (+16) into lane 16 s + lane % 16 - the B
+// operand of one MFMA step per group, with V read at that key's row as the A operand of both.
+// Vt: the lane's V base, row (s&1) + 4(s>>1), column lane % 16 (s = lane / 16).
+template <int KIND>
+__device__ __forceinline__ void attend_tile_16(const float *Kb, const float *Vt, const float (&qr)[8], f32x4 (&og)[2], float &m_run,
+                                               float &m_use, float &l_run, const int k0, const int q0, const int qi, const int half,
+                                               const int ln, const int Lk, const int len, const float *mrow, const long long msk,
+                                               const int cls) {
+    constexpr int LS = NarrowTile<16>::LS;
+    f32x16 s0 = masked_scores<KIND, 2>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
+    float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
+#pragma unroll
+    for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
+    tmax = fmaxf(tmax, s0[15]);
+    tmax = fmaxf(tmax, xor32(tmax));
+    const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+    if (__any(upd)) {
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
+        m_run = m_new;
+        m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        l_run *= alpha;
+        // the lane's own factor belongs to the group its query is in; the other group's comes from the lane 16 away
+        const float other = __shfl_xor(alpha, 16, 64);
+        const float a0 = ln < 16 ? alpha : other, a1 = ln < 16 ? other : alpha;
+        og[0].x *= a0; og[0].y *= a0; og[0].z *= a0; og[0].w *= a0;
+        og[1].x *= a1; og[1].y *= a1; og[1].z *= a1; og[1].w *= a1;
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        s0[r] = fast_exp2(s0[r] - m_use);
+        psum += s0[r];
+    }
+    l_run += psum;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(s0[2 * p]), __float_as_uint(s0[2 * p + 1]), false, false);
+        const float va = Vt[(8 * (p >> 1) + 2 * (p & 1)) * LS];
+        og[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[0]), og[0], 0, 0, 0);
+        og[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[1]), og[1], 0, 0, 0);
+    }
 }
 
 // Stores the lane's query row: register r of o0 is d = 8(r/4) + 4*half + r%4.
@@ -162,6 +210,7 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
     f32x16 o0;   // O^T, row d = 8(r/4) + 4*half + r%4
 #pragma unroll
     for (int i = 0; i < 16; ++i) o0[i] = 0.f;
+    f32x4 og[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};   // W = 16: O^T on two 16 x 16 accumulators (attend_tile_16)
     float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
 
     if (ntiles > 0) {
@@ -172,6 +221,8 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
 
     const int k_lds = ln * LS + half * (W / 2);
     const int v_lds = (4 * half) * LS + ln;
+    const int slot = lane >> 4;
+    const int v_lds16 = ((slot & 1) + 4 * (slot >> 1)) * LS + (lane & 15);
     const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
@@ -183,9 +234,14 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
         const int k0 = t * BN;
         int cls = 2;
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
-        if (k0 < wkend && !(DENSE && skip_ones && cls == 1))
-            attend_tile_narrow<KIND, W>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds, qr, o0, m_run, m_use, l_run, k0, q0, qi, half, Lk,
-                                        len, mrow, mask.sk, cls);
+        if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
+            if constexpr (W == 16)
+                attend_tile_16<KIND>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds16, qr, og, m_run, m_use, l_run, k0, q0, qi, half, ln, Lk,
+                                     len, mrow, mask.sk, cls);
+            else
+                attend_tile_narrow<KIND, W>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds, qr, o0, m_run, m_use, l_run, k0, q0, qi, half, Lk,
+                                            len, mrow, mask.sk, cls);
+        }
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     };
@@ -200,7 +256,20 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
         stats[2 * ((long long)bh * Lq + qi)] = m_use;
         stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
     }
-    if (qi < Lq) store_row_narrow(out + q_base + (long long)qi * rs, o0, inv, half, hd);
+    if constexpr (W == 16) {
+        // group g of the lane: query q0 + 16 g + lane % 16, columns 4 * slot ..; the reciprocal sum of that query is the lane's own
+        // when the lane's query lies in the group, else the one of the lane 16 away
+        const float other = __shfl_xor(inv, 16, 64);
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const int qg = q0 + 16 * g + (lane & 15);
+            const float f = ((ln < 16) == (g == 0)) ? inv : other;
+            const f32x4 a = {og[g].x * f, og[g].y * f, og[g].z * f, og[g].w * f};
+            if (qg < Lq && 4 * slot < hd) *reinterpret_cast<f32x4 *>(out + q_base + (long long)qg * rs + 4 * slot) = a;
+        }
+    } else {
+        if (qi < Lq) store_row_narrow(out + q_base + (long long)qi * rs, o0, inv, half, hd);
+    }
 }
 
 // Small launches: one workgroup = 32 queries, its key tiles dealt round-robin to the 4 wavefronts through
