@@ -281,7 +281,7 @@ def other_configs(ctx, lib, cpu, only=None):
         # (the 64-wide kernels), 128, 96 and 32 (the 128-, 96- and 32-wide ones)
         B, H, L = 8, 16, 2048
         rng = np.random.Generator(np.random.PCG64(1004))
-        for d in (64, 128, 96, 32):
+        for d in (64, 128, 96, 32, 256):
             bufs = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
             outs = [ctx.empty((B, H, L, d)) for _ in range(4)]
             st = ctx.empty((B, H, L, 2))
@@ -289,19 +289,23 @@ def other_configs(ctx, lib, cpu, only=None):
             rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
             ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], outs[0], st, B, H, L, L, d, rT, desc, 0)
             bwd = lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, d, rT, desc, 0)
-            for _ in range(20):
+            reps = 20 if d <= 128 else 5
+            for _ in range(reps):
                 bwd()
             ctx.sync()
             ctx.timer_begin()
-            for _ in range(20):
+            for _ in range(reps):
                 bwd()
-            ms = ctx.timer_end() / 20
+            ms = ctx.timer_end() / reps
             fl = 10.0 * d * B * H * (L * (L + 1) // 2)          # five products: the recomputed scores, dp, dv, dk, dq
             name = "config4_attention_backward_B8_H16_L2048_causal" + ("" if d == 64 else "_head_dim_%d" % d)
             res[name] = {
                 "us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
-                "note": "algorithmic flops = the 5 products, which is what the two deterministic kernels issue: the dK/dV kernel "
-                        "stores its dS tiles (2 GiB scratch from the pool at this shape) and the dQ kernel contracts them with K"}
+                "note": ("algorithmic flops = the 5 products, which is what the two deterministic kernels issue: the dK/dV kernel "
+                         "stores its dS tiles (2 GiB scratch from the pool at this shape) and the dQ kernel contracts them with K")
+                        if d <= 128 else
+                        "head dims above 128: the five products as batched GEMMs around one elementwise pass, query blocks of "
+                        "512 rows under the causal mask; TFLOP/s on the algorithmic flops"}
             if cpu and d == 64:
                 from oracle import binding as orc
                 hq, hk, hv, hg = (b_.numpy()[:1, :2] for b_ in bufs)
