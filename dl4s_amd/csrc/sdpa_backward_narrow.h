@@ -41,6 +41,22 @@ __device__ __forceinline__ void tile_accumulate_1(const float *At, const f32x16 
     for (int r = 0; r < 16; ++r) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(At[(8 * (r >> 2) + (r & 3)) * LS], b[r], acc, 0, 0, 0);
 }
 
+// The 16-wide form of tile_accumulate_1 on 16 x 16 x 4 MFMAs (a 32 x 32 accumulator of a 16-wide head is half empty):
+// og[0] holds the columns (keys) 0 .. 15 of the wavefront, og[1] 16 .. 31; lane: column = lane % 16, rows d = 4 * (lane / 16) + i.
+// v_permlane16_swap of a register pair (2p, 2p+1) of b puts, for both accumulators at once, the value of row
+// 8(p/2) + 2(p%2) + (s&1) + 4(s>>1) into lane 16 s + lane % 16 (see attend_tile_16 in sdpa_prefill_narrow.h).
+// At16: the lane's base in the [32][LS] tile, row (s&1) + 4(s>>1), column lane % 16 (s = lane / 16).
+template <int LS>
+__device__ __forceinline__ void tile_accumulate_16(const float *At16, const f32x16 &b, f32x4 (&og)[2]) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(b[2 * p]), __float_as_uint(b[2 * p + 1]), false, false);
+        const float a = At16[(8 * (p >> 1) + 2 * (p & 1)) * LS];
+        og[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, __uint_as_float(sw[0]), og[0], 0, 0, 0);
+        og[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, __uint_as_float(sw[1]), og[1], 0, 0, 0);
+    }
+}
+
 // stores the lane's row: register r of acc is d = 8(r/4) + 4*half + r%4
 __device__ __forceinline__ void store_row_1(float *p, const f32x16 &acc, const float scale, const int half, const int hd) {
 #pragma unroll
@@ -156,12 +172,15 @@ __global__ __launch_bounds__(256, 3) void sdpa_bwd_dkv_f32_narrow(const float *_
     f32x16 ka, va;   // dK^T and dV^T, row d = 8(r/4) + 4*half + r%4
 #pragma unroll
     for (int i = 0; i < 16; ++i) { ka[i] = 0.f; va[i] = 0.f; }
+    f32x4 kg[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, vg[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};   // W = 16 (tile_accumulate_16)
 
     if (t_begin < nqt) { load_tile(t_begin); store_tile(0); }
     __syncthreads();
 
     const int row_lds = ln * LS + half * (W / 2);
     const int col_lds = (4 * half) * LS + ln;
+    const int slot = lane >> 4;
+    const int col_lds16 = ((slot & 1) + 4 * (slot >> 1)) * LS + (lane & 15);
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
@@ -220,7 +239,8 @@ __global__ __launch_bounds__(256, 3) void sdpa_bwd_dkv_f32_narrow(const float *_
                 p[4 * g + 2] = fast_exp2(p[4 * g + 2] - m4.z) * r4.z;
                 p[4 * g + 3] = fast_exp2(p[4 * g + 3] - m4.w) * r4.w;
             }
-            tile_accumulate_1<LS>(Gs + buf * TF + col_lds, p, va);                           // dV^T += dout^T . P
+            if constexpr (W == 16) tile_accumulate_16<LS>(Gs + buf * TF + col_lds16, p, vg);
+            else tile_accumulate_1<LS>(Gs + buf * TF + col_lds, p, va);                      // dV^T += dout^T . P
             const f32x16 dp = tile_product_n<NJ>(Gs + buf * TF + row_lds, vr);               // dP = dout . V^T
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
@@ -237,12 +257,24 @@ __global__ __launch_bounds__(256, 3) void sdpa_bwd_dkv_f32_narrow(const float *_
                 const f32x4 o = {p[4 * g + 0], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]};
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 0);
             }
-            tile_accumulate_1<LS>(Qs + buf * TF + col_lds, p, ka);                           // dK^T += Q~^T . dS
+            if constexpr (W == 16) tile_accumulate_16<LS>(Qs + buf * TF + col_lds16, p, kg);
+            else tile_accumulate_1<LS>(Qs + buf * TF + col_lds, p, ka);                      // dK^T += Q~^T . dS
         }
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
-    if (key < Lk) {
+    if constexpr (W == 16) {
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {      // accumulator g: key kw0 + 16 g + lane % 16, columns 4 * slot ..
+            const int kg_ = kw0 + 16 * g + (lane & 15);
+            if (kg_ < Lk && 4 * slot < hd) {
+                constexpr float LN2 = 0.69314718055994530942f;    // Q~ carries log2(e)
+                const f32x4 a = {kg[g].x * LN2, kg[g].y * LN2, kg[g].z * LN2, kg[g].w * LN2};
+                *reinterpret_cast<f32x4 *>(dv + kv_base + (long long)kg_ * rs + 4 * slot) = vg[g];
+                *reinterpret_cast<f32x4 *>(dk + kv_base + (long long)kg_ * rs + 4 * slot) = a;
+            }
+        }
+    } else if (key < Lk) {
         store_row_1(dv + kv_base + (long long)key * rs, va, 1.0f, half, hd);
         store_row_1(dk + kv_base + (long long)key * rs, ka, 0.69314718055994530942f, half, hd);   // Q~ carries log2(e)
     }
