@@ -321,14 +321,14 @@ def other_configs(ctx, lib, cpu, only=None):
     if want("masks_and_head_dim"):
         # the headline shape with the mask as an unmodified DL4S passes it (a dense [L,L] tensor): all-ones tiles skipped
         # (default) and every tile visited (DL4S_SDPA_STRICT); the same shape with the causal descriptor at other head dims:
-        # 128 (128-wide tiles), 96 and 70 (96-wide tiles; 70 is staged with 64-bit accesses, no padded copies), 32 and 16
+        # 128 (128-wide tiles), 96, 80 and 70 (96-wide tiles, their 80-column form for the latter two; 70 is staged with 64-bit accesses, no padded copies), 32 and 16
         # (32- and 16-wide tiles), 192 and 256 (192- and 256-wide tiles).  TFLOP/s on each shape's own flops.
         B, H, L = 8, 16, 2048
         rng = np.random.Generator(np.random.PCG64(1008))
         i, j = np.indices((L, L))
         dmask = ctx.to_device((j > i).astype(np.float32))
         for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal"),
-                        (96, "config4_shape_head_dim_96_causal"), (70, "config4_shape_head_dim_70_causal"),
+                        (96, "config4_shape_head_dim_96_causal"), (80, "config4_shape_head_dim_80_causal"), (70, "config4_shape_head_dim_70_causal"),
                         (32, "config4_shape_head_dim_32_causal"), (16, "config4_shape_head_dim_16_causal"),
                         (192, "config4_shape_head_dim_192_causal"), (256, "config4_shape_head_dim_256_causal")):
             qkv = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(3)]

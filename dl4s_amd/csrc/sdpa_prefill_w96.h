@@ -10,7 +10,7 @@
 //                                                    four consecutive outputs per 128-bit (or two 64-bit) stores
 //
 // 96 MFMAs per 32 x 32 tile of (query, key) pairs against the 128-wide kernel's 128: a head dim of 96 costs three
-// quarters, and one of 70 runs without the four streaming copies.  One workgroup = 4 wavefronts = 128 queries of one
+// quarters, and one of 70 runs without the four streaming copies.  Head dims up to 80 run the W = 80 form (below).  One workgroup = 4 wavefronts = 128 queries of one
 // (batch, head) pair, K/V in double-buffered LDS tiles of 32 keys on a 100-float row stride (2 x 2 x 32 x 100 floats =
 // 50 KiB).  Mask kinds, tile skipping, the work order, the token-major layout (head dims that are multiples of 4) and
 // the row statistics are those of the other forward kernels.  Small launches (head dims that are multiples of 4) are
@@ -26,7 +26,12 @@ constexpr int LSTR96 = W96 + 4;            // 100 = 4 mod 32: the bank spread of
 constexpr int TILE96_FLOATS = BN * LSTR96;
 
 // VEC: floats per staging access, 4 (head dim a multiple of 4, tensors on the 16-byte grid) or 2 (head dim even, 8-byte grid)
-template <int KIND, int VEC>
+// W: 96, or 80 for head dims up to 80: the same tiles in LDS (columns from the head dim up are zeros either way), but the
+// score product contracts 40 steps per half (d = 40*half + s) and the columns 64 .. 79 of O^T live in two 16 x 16
+// accumulators on v_mfma_f32_16x16x4_f32 (queries 0-15 and 16-31 of the wavefront; lane: column = lane % 16, rows
+// d = 64 + 4 * (lane / 16) + i), fed through v_permlane16_swap like attend_tile_16 (sdpa_prefill_narrow.h): 80 MFMA units
+// per tile instead of 96.
+template <int KIND, int VEC, int W = 96>
 __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__restrict__ q, const float *__restrict__ k,
                                                                 const float *__restrict__ v, float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict, int nqb, int total_blocks,
@@ -68,14 +73,14 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
     }
     const int ntiles = (kend + BN - 1) / BN;
 
-    // Q fragment: Q[qi][48*half + s] * rT (one rounding, like the reference's q / temperature) * log2(e); zeros beyond hd
-    float qr[W96 / 2];
+    // Q fragment: Q[qi][(W/2)*half + s] * rT (one rounding, like the reference's q / temperature) * log2(e); zeros beyond hd
+    float qr[W / 2];
     {
-        const float *qp = q + q_base + (long long)qic * rs + half * (W96 / 2);
+        const float *qp = q + q_base + (long long)qic * rs + half * (W / 2);
 #pragma unroll
-        for (int j = 0; j < W96 / 8; ++j) {
+        for (int j = 0; j < W / 8; ++j) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
-            const int c0 = half * (W96 / 2) + 4 * j;
+            const int c0 = half * (W / 2) + 4 * j;
             if (VEC == 4) {
                 if (c0 < hd) t = *reinterpret_cast<const f32x4 *>(qp + 4 * j);
             } else {
@@ -129,19 +134,23 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
         }
     };
 
+    constexpr int NC = W == 96 ? 3 : 2;    // 32 x 32 accumulators
     f32x16 o[3];
 #pragma unroll
     for (int c = 0; c < 3; ++c)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[c][i] = 0.f;
+    f32x4 og[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};   // W = 80: the columns 64 .. 79
     float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
 
     const int sp = blockIdx.y;     // this workgroup's share of the key tiles: sp, sp + nsplit, ...
     if (sp < ntiles) { load_tile(sp); store_tile(0); }
     __syncthreads();
 
-    const int k_lds = ln * LSTR96 + half * (W96 / 2);   // K fragment base: row ln, columns 48*half ..
+    const int k_lds = ln * LSTR96 + half * (W / 2);     // K fragment base: row ln, columns (W/2)*half ..
     const int v_lds = (4 * half) * LSTR96 + ln;          // V operand base: row 4*half (+ const), column ln (+ 32c)
+    const int slot = lane >> 4;
+    const int v_lds16 = ((slot & 1) + 4 * (slot >> 1)) * LSTR96 + 64 + (lane & 15);   // W = 80: row of the lane's MFMA slot, column 64 + lane % 16
     const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
@@ -153,7 +162,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
         int cls = 2;
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
         if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
-            f32x16 s0 = masked_scores<KIND, W96 / 8>(Ks + buf * TILE96_FLOATS + k_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
+            f32x16 s0 = masked_scores<KIND, W / 8>(Ks + buf * TILE96_FLOATS + k_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
             // online softmax with a lazily moved reference maximum (see attend_tile in sdpa_prefill.hip)
             float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
 #pragma unroll
@@ -168,9 +177,15 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
                 m_use = (m_new == -INFINITY) ? 0.f : m_new;
                 l_run *= alpha;
 #pragma unroll
-                for (int c = 0; c < 3; ++c)
+                for (int c = 0; c < NC; ++c)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) o[c][i] *= alpha;
+                if constexpr (W == 80) {    // the other group's factor comes from the lane 16 away
+                    const float other = __shfl_xor(alpha, 16, 64);
+                    const float a0 = ln < 16 ? alpha : other, a1 = ln < 16 ? other : alpha;
+                    og[0].x *= a0; og[0].y *= a0; og[0].z *= a0; og[0].w *= a0;
+                    og[1].x *= a1; og[1].y *= a1; og[1].z *= a1; og[1].w *= a1;
+                }
             }
             float psum = 0.f;
 #pragma unroll
@@ -185,7 +200,17 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
                 const float *vr = Vb + (8 * (r >> 2) + (r & 3)) * LSTR96;
                 o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[0], s0[r], o[0], 0, 0, 0);
                 o[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[32], s0[r], o[1], 0, 0, 0);
-                o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[64], s0[r], o[2], 0, 0, 0);
+                if constexpr (W == 96) o[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[64], s0[r], o[2], 0, 0, 0);
+            }
+            if constexpr (W == 80) {
+                const float *Vt = Vs + buf * TILE96_FLOATS + v_lds16;
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(s0[2 * p]), __float_as_uint(s0[2 * p + 1]), false, false);
+                    const float va = Vt[(8 * (p >> 1) + 2 * (p & 1)) * LSTR96];
+                    og[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[0]), og[0], 0, 0, 0);
+                    og[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[1]), og[1], 0, 0, 0);
+                }
             }
         }
         if (more) store_tile(buf ^ 1);
@@ -198,13 +223,21 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
         if (qi < Lq) {
             float *pp = part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * PART2_STRIDE;
 #pragma unroll
-            for (int c = 0; c < 3; ++c)
+            for (int c = 0; c < NC; ++c)
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const f32x4 a = {o[c][4 * g + 0], o[c][4 * g + 1], o[c][4 * g + 2], o[c][4 * g + 3]};
                     *reinterpret_cast<f32x4 *>(pp + 32 * c + 8 * g + 4 * half) = a;
                 }
             if (half == 0) { pp[HD2] = m_run; pp[HD2 + 1] = l_tot; }
+        }
+        if constexpr (W == 80) {     // the 16 x 16 accumulators: query q0 + 16 g + lane % 16, columns 64 + 4 * slot ..
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                const int qg = q0 + 16 * g + (lane & 15);
+                if (qg < Lq)
+                    *reinterpret_cast<f32x4 *>(part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qg) * PART2_STRIDE + 64 + 4 * slot) = og[g];
+            }
         }
         return;
     }
@@ -216,7 +249,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
     if (qi < Lq) {
         float *op = out + q_base + (long long)qi * rs;
 #pragma unroll
-        for (int c = 0; c < 3; ++c)
+        for (int c = 0; c < NC; ++c)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int d0 = 32 * c + 8 * g + 4 * half;
@@ -230,9 +263,29 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__re
                 }
             }
     }
+    if constexpr (W == 80) {
+        // the reciprocal sum of a group's query is the lane's own when its query lies in the group, else the lane's 16 away
+        const float other = __shfl_xor(inv, 16, 64);
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            const int qg = q0 + 16 * g + (lane & 15), d0 = 64 + 4 * slot;
+            const float f = ((ln < 16) == (g == 0)) ? inv : other;
+            const f32x4 a = {og[g].x * f, og[g].y * f, og[g].z * f, og[g].w * f};
+            if (qg < Lq) {
+                float *op = out + q_base + (long long)qg * rs;
+                if (VEC == 4) {
+                    if (d0 < hd) *reinterpret_cast<f32x4 *>(op + d0) = a;
+                } else {
+                    const f32x2 lo = {a.x, a.y}, hi = {a.z, a.w};
+                    if (d0 < hd) *reinterpret_cast<f32x2 *>(op + d0) = lo;
+                    if (d0 + 2 < hd) *reinterpret_cast<f32x2 *>(op + d0 + 2) = hi;
+                }
+            }
+        }
+    }
 }
 
-template <int KIND, int VEC>
+template <int KIND, int VEC, int W>
 int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
                     float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit, float *part) {
     const int nqb = (Lq + BM - 1) / BM;
@@ -243,7 +296,7 @@ int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const flo
     if (lpt && total <= 3ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
     const size_t lds_bytes = 4 * TILE96_FLOATS * sizeof(float);   // 50 KiB: within the default limit
     if (nsplit <= 1 || !part || VEC != 4) { nsplit = 1; part = nullptr; }
-    hipLaunchKernelGGL((sdpa_prefill_f32_w96<KIND, VEC>), dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
+    hipLaunchKernelGGL((sdpa_prefill_f32_w96<KIND, VEC, W>), dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part);
     const int st = dl4s::launch_status("sdpa_prefill_f32_w96");
     if (st != DL4S_HIP_OK || nsplit == 1) return st;
@@ -253,16 +306,24 @@ int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const flo
     return dl4s::launch_status("sdpa_prefill_merge_d128");
 }
 
+template <int VEC, int W>
+int launch_w96_width(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk, float rT,
+                     const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit, float *part) {
+    switch (m.kind) {
+        case DL4S_MASK_NONE: return launch_w96_kind<DL4S_MASK_NONE, VEC, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_DENSE_F32: return launch_w96_kind<DL4S_MASK_DENSE_F32, VEC, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_CAUSAL: return launch_w96_kind<DL4S_MASK_CAUSAL, VEC, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_KEY_LENGTHS: return launch_w96_kind<DL4S_MASK_KEY_LENGTHS, VEC, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        default: return launch_w96_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, VEC, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+    }
+}
+
+// head dims up to 80 on the 80-column form, the others on all 96
 template <int VEC>
 int launch_w96(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk, float rT,
                const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit = 1, float *part = nullptr) {
-    switch (m.kind) {
-        case DL4S_MASK_NONE: return launch_w96_kind<DL4S_MASK_NONE, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
-        case DL4S_MASK_DENSE_F32: return launch_w96_kind<DL4S_MASK_DENSE_F32, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
-        case DL4S_MASK_CAUSAL: return launch_w96_kind<DL4S_MASK_CAUSAL, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
-        case DL4S_MASK_KEY_LENGTHS: return launch_w96_kind<DL4S_MASK_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
-        default: return launch_w96_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, VEC>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
-    }
+    if (hd <= 80) return launch_w96_width<VEC, 80>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+    return launch_w96_width<VEC, 96>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
 }
 
 }  // namespace
