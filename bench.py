@@ -329,7 +329,7 @@ def other_configs(ctx, lib, cpu, only=None):
         dmask = ctx.to_device((j > i).astype(np.float32))
         for d, name in ((64, "config4_shape_dense_causal_mask_tensor"), (128, "config4_shape_head_dim_128_causal"),
                         (96, "config4_shape_head_dim_96_causal"), (80, "config4_shape_head_dim_80_causal"), (70, "config4_shape_head_dim_70_causal"),
-                        (32, "config4_shape_head_dim_32_causal"), (16, "config4_shape_head_dim_16_causal"),
+                        (48, "config4_shape_head_dim_48_causal"), (32, "config4_shape_head_dim_32_causal"), (16, "config4_shape_head_dim_16_causal"),
                         (192, "config4_shape_head_dim_192_causal"), (256, "config4_shape_head_dim_256_causal")):
             qkv = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(3)]
             o = ctx.empty((B, H, L, d))

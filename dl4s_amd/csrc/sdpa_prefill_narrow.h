@@ -1,5 +1,6 @@
 // Fused attention forward for narrow heads (head dims up to 32): the kernels of sdpa_prefill.hip on tiles that are W = 32
-// or W = 16 columns wide instead of 64.  Included by sdpa_prefill.hip only.
+// or W = 16 columns wide instead of 64, and a W = 48 form of the main kernel for head dims 36 .. 48 (attend_tile_48).
+// Included by sdpa_prefill.hip only.
 //
 // A 64-wide tile spends 32 MFMA steps on S^T = K . Q^T and 32 on O^T += V^T . P^T whatever the head dim; a model with key
 // size 8 (the reference's own test model, Tests/DL4STests/TransformerTests.swift:31) needs a fraction of that:
@@ -19,7 +20,7 @@
 namespace {
 
 template <int W> struct NarrowTile {
-    static constexpr int LS = W + 4;          // LDS row stride: keeps 128-bit reads of consecutive rows on distinct banks
+    static constexpr int LS = W + 4;          // LDS row stride (36, 20, 52): keeps 128-bit reads of consecutive rows on distinct banks
     static constexpr int TF = BN * LS;        // floats per tile
     static constexpr int NJ = W / 8;          // 128-bit reads per K row fragment
 };
@@ -111,6 +112,54 @@ __device__ __forceinline__ void attend_tile_16(const float *Kb, const float *Vt,
     }
 }
 
+// The 48-wide tile of the main kernel (head dims 36 .. 48): S^T takes 24 MFMAs, the columns 0 .. 31 of O^T one 32 x 32
+// accumulator like the 32-wide tile (Vb: row 4 * half, column lane % 32), the columns 32 .. 47 two 16 x 16 accumulators like
+// attend_tile_16 (Vt: row of the lane's MFMA slot, column 32 + lane % 16): 48 MFMA units per tile against the 64 of the
+// 64-wide kernel these head dims ran on.
+template <int KIND>
+__device__ __forceinline__ void attend_tile_48(const float *Kb, const float *Vb, const float *Vt, const float (&qr)[24], f32x16 &o0,
+                                               f32x4 (&og)[2], float &m_run, float &m_use, float &l_run, const int k0, const int q0,
+                                               const int qi, const int half, const int ln, const int Lk, const int len,
+                                               const float *mrow, const long long msk, const int cls) {
+    constexpr int LS = NarrowTile<48>::LS;
+    f32x16 s0 = masked_scores<KIND, 6>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
+    float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
+#pragma unroll
+    for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
+    tmax = fmaxf(tmax, s0[15]);
+    tmax = fmaxf(tmax, xor32(tmax));
+    const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+    if (__any(upd)) {
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
+        m_run = m_new;
+        m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o0[i] *= alpha;
+        const float other = __shfl_xor(alpha, 16, 64);
+        const float a0 = ln < 16 ? alpha : other, a1 = ln < 16 ? other : alpha;
+        og[0].x *= a0; og[0].y *= a0; og[0].z *= a0; og[0].w *= a0;
+        og[1].x *= a1; og[1].y *= a1; og[1].z *= a1; og[1].w *= a1;
+    }
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        s0[r] = fast_exp2(s0[r] - m_use);
+        psum += s0[r];
+    }
+    l_run += psum;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(Vb[(8 * (r >> 2) + (r & 3)) * LS], s0[r], o0, 0, 0, 0);
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(s0[2 * p]), __float_as_uint(s0[2 * p + 1]), false, false);
+        const float va = Vt[(8 * (p >> 1) + 2 * (p & 1)) * LS];
+        og[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[0]), og[0], 0, 0, 0);
+        og[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[1]), og[1], 0, 0, 0);
+    }
+}
+
 // Stores the lane's query row: register r of o0 is d = 8(r/4) + 4*half + r%4.
 __device__ __forceinline__ void store_row_narrow(float *op, const f32x16 &o0, const float inv, const int half, const int hd) {
 #pragma unroll
@@ -176,9 +225,10 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
 
     // global -> LDS staging.  W = 32: every thread moves one 128-bit piece of the K tile and one of the V tile (row tid/8,
     // column 4 * (tid%8)).  W = 16: wavefronts 0, 1 move the K tile and wavefronts 2, 3 the V tile (row t/4, column
-    // 4 * (t%4) with t = tid % 128).  Rows at or beyond Lk and columns at or beyond hd lie outside the descriptor: zeros.
+    // 4 * (t%4) with t = tid % 128).  W = 48: 384 pieces per tile - every thread piece tid of both tiles, the threads of
+    // wavefronts 0, 1 also piece tid + 256.  Rows at or beyond Lk and columns at or beyond hd lie outside the descriptor: zeros.
     constexpr int CPR = W / 4;                       // 128-bit pieces per tile row
-    const int st = (W == 32) ? tid : (tid & 127);
+    const int st = (W == 16) ? (tid & 127) : tid;
     const int ld_row = st / CPR, ld_col = (st % CPR) * 4;
     const int kv_bytes = (int)(((long long)(Lk - 1) * rs + hd) * 4);
     const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(k + kv_base), 0, kv_bytes, 0x00020000);
@@ -186,12 +236,20 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
     const unsigned ld_off = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
     const unsigned tile_bytes = (unsigned)BN * rs * 4u;
     const int lds_off = ld_row * LS + ld_col;
-    f32x4 kst, vst;
+    const int ld_row2 = (tid + 256) / CPR, ld_col2 = ((tid + 256) % CPR) * 4;      // W = 48, wavefronts 0, 1
+    const unsigned ld_off2 = ld_col2 < hd ? (unsigned)(ld_row2 * rs + ld_col2) * 4u : 0x80000000u;
+    const int lds_off2 = ld_row2 * LS + ld_col2;
+    f32x4 kst, vst, kst2, vst2;
     auto load_tile = [&](int t) {
         const int o = (int)(ld_off + t * tile_bytes);
-        if (W == 32) {
+        if (W != 16) {
             kst = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o, 0, 0));
             vst = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o, 0, 0));
+            if (W == 48 && wave < 2) {
+                const int o2 = (int)(ld_off2 + t * tile_bytes);
+                kst2 = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o2, 0, 0));
+                vst2 = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(vrsrc, o2, 0, 0));
+            }
         } else if (wave < 2) {
             kst = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(krsrc, o, 0, 0));
         } else {
@@ -199,9 +257,13 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
         }
     };
     auto store_tile = [&](int buf) {
-        if (W == 32) {
+        if (W != 16) {
             *reinterpret_cast<f32x4 *>(Ks + buf * TF + lds_off) = kst;
             *reinterpret_cast<f32x4 *>(Vs + buf * TF + lds_off) = vst;
+            if (W == 48 && wave < 2) {
+                *reinterpret_cast<f32x4 *>(Ks + buf * TF + lds_off2) = kst2;
+                *reinterpret_cast<f32x4 *>(Vs + buf * TF + lds_off2) = vst2;
+            }
         } else {
             *reinterpret_cast<f32x4 *>((wave < 2 ? Ks : Vs) + buf * TF + lds_off) = kst;
         }
@@ -210,7 +272,7 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
     f32x16 o0;   // O^T, row d = 8(r/4) + 4*half + r%4
 #pragma unroll
     for (int i = 0; i < 16; ++i) o0[i] = 0.f;
-    f32x4 og[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};   // W = 16: O^T on two 16 x 16 accumulators (attend_tile_16)
+    f32x4 og[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};   // W = 16: O^T on two 16 x 16 accumulators (attend_tile_16); W = 48: its columns 32 .. 47
     float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
 
     if (ntiles > 0) {
@@ -222,7 +284,7 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
     const int k_lds = ln * LS + half * (W / 2);
     const int v_lds = (4 * half) * LS + ln;
     const int slot = lane >> 4;
-    const int v_lds16 = ((slot & 1) + 4 * (slot >> 1)) * LS + (lane & 15);
+    const int v_lds16 = ((slot & 1) + 4 * (slot >> 1)) * LS + (W == 48 ? 32 : 0) + (lane & 15);
     const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
@@ -238,6 +300,9 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
             if constexpr (W == 16)
                 attend_tile_16<KIND>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds16, qr, og, m_run, m_use, l_run, k0, q0, qi, half, ln, Lk,
                                      len, mrow, mask.sk, cls);
+            else if constexpr (W == 48)
+                attend_tile_48<KIND>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds, Vs + buf * TF + v_lds16, qr, o0, og, m_run, m_use, l_run,
+                                     k0, q0, qi, half, ln, Lk, len, mrow, mask.sk, cls);
             else
                 attend_tile_narrow<KIND, W>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds, qr, o0, m_run, m_use, l_run, k0, q0, qi, half, Lk,
                                             len, mrow, mask.sk, cls);
@@ -256,19 +321,21 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
         stats[2 * ((long long)bh * Lq + qi)] = m_use;
         stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
     }
-    if constexpr (W == 16) {
-        // group g of the lane: query q0 + 16 g + lane % 16, columns 4 * slot ..; the reciprocal sum of that query is the lane's own
-        // when the lane's query lies in the group, else the one of the lane 16 away
+    if constexpr (W != 16) {
+        if (qi < Lq) store_row_narrow(out + q_base + (long long)qi * rs, o0, inv, half, hd);
+    }
+    if constexpr (W != 32) {
+        // group g of the lane: query q0 + 16 g + lane % 16, columns (32 +) 4 * slot ..; the reciprocal sum of that query is the
+        // lane's own when the lane's query lies in the group, else the one of the lane 16 away
         const float other = __shfl_xor(inv, 16, 64);
+        const int d0 = (W == 48 ? 32 : 0) + 4 * slot;
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             const int qg = q0 + 16 * g + (lane & 15);
             const float f = ((ln < 16) == (g == 0)) ? inv : other;
             const f32x4 a = {og[g].x * f, og[g].y * f, og[g].z * f, og[g].w * f};
-            if (qg < Lq && 4 * slot < hd) *reinterpret_cast<f32x4 *>(out + q_base + (long long)qg * rs + 4 * slot) = a;
+            if (qg < Lq && d0 < hd) *reinterpret_cast<f32x4 *>(out + q_base + (long long)qg * rs + d0) = a;
         }
-    } else {
-        if (qi < Lq) store_row_narrow(out + q_base + (long long)qi * rs, o0, inv, half, hd);
     }
 }
 
@@ -450,6 +517,24 @@ int launch_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
     const int lpt = (uneven && nqb >= 2) ? 1 : 0;
     const int lpt_arg = lpt | ((lpt && total <= 3ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
     hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
+                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
+    return dl4s::launch_status("sdpa_prefill_f32_narrow");
+}
+
+// The 48-column form of the main kernel for head dims 36 .. 48 on launches large enough for it (small ones run the 64-wide
+// key-split kernel)
+template <int KIND>
+int launch_narrow48_main(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
+                         float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+    constexpr int TF = NarrowTile<48>::TF;
+    constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
+    const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
+    const int nqb = (Lq + BM - 1) / BM;
+    const long long total = (long long)nqb * B * H;
+    DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
+    const int lpt = (uneven && nqb >= 2) ? 1 : 0;
+    const int lpt_arg = lpt | ((lpt && total <= 3ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
+    hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, 48>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_narrow");
 }

@@ -160,7 +160,7 @@ typedef struct dl4s_mask_desc {
  * v [B,H,Lk,dv], out [B,H,Lq,dv], all row-major contiguous device fp32.  inv_temperature is the
  * fp32 reciprocal the reference forms once (Engine/CPU/CPUEngine.swift:635).  mask may be NULL
  * (= DL4S_MASK_NONE).  dk = dv, a multiple of 4 and at most 128, with 16-byte aligned tensors runs
- * a fused MFMA kernel written for tiles of 16, 32, 64, 80, 96 or 128 columns; a head dim between two
+ * a fused MFMA kernel written for tiles of 16, 32, 48, 64, 80, 96 or 128 columns; a head dim between two
  * widths is padded with zero columns on the fly and costs what the wider tile costs.  Even head dims
  * from 66 to 94 that are not a multiple of 4 run the 96-wide kernel as they are (8-byte aligned
  * tensors, launches that fill the GPU).  dk = dv above 128 up to 256 (a multiple of 4, aligned) runs

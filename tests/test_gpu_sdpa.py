@@ -744,12 +744,13 @@ def test_96_wide_kernel_on_short_and_ragged_extents(ctx, orc, B, H, Lq, Lk, d, m
         assert np.array_equal(run_sdpa(ctx, q, k, v, mask, kind=kind, lens=lens_arg, strict=True), run_sdpa(ctx, q, k, v, mask, strict=True))
 
 
-@pytest.mark.parametrize("d", [96, 80, 68, 70, 66, 94])
+@pytest.mark.parametrize("d", [96, 80, 68, 70, 66, 94, 48, 40, 36, 44])
 @pytest.mark.parametrize("mk", ["none", "dense", "causal", "lens", "causal_lens"])
 def test_head_dims_up_to_96_on_launches_that_fill_the_gpu(ctx, orc, d, mk):
-    """Head dims above 64 up to 96 with at least two 128-query blocks per CU run the 96-wide kernel: multiples of 4 with
-    128-bit staging, other even head dims as they are with 64-bit staging (no padded copies).  B16 H16, ragged
-    extents, checked against the oracle on whole (batch, head) slices."""
+    """Head dims above 64 up to 96 with at least two 128-query blocks per CU run the 96-wide kernel (its 80-column form up
+    to 80): multiples of 4 with 128-bit staging, other even head dims as they are with 64-bit staging (no padded copies).
+    Head dims 36 .. 48 run the 48-column form of the narrow kernel.  B16 H16, ragged extents, checked against the oracle on
+    whole (batch, head) slices."""
     from dl4s_amd import lib
     B, H, Lq, Lk = 16, 16, 300, 300
     rng = np.random.default_rng(zlib.crc32(repr(("w96", d, mk)).encode()))
