@@ -46,7 +46,7 @@ struct dl4s_hip_ctx {
     // One bit per (kernel family, mask kind): the dynamic-LDS limit of those kernels has been raised on this context's
     // device (hipFuncSetAttribute is per device; two host threads that both find a bit clear both set the attribute, which
     // is harmless, and then the bit).
-    std::atomic<unsigned long long> lds_limit_raised{0};
+    std::atomic<unsigned long long> lds_limit_raised[2] = {{0}, {0}};   // bit family * 8 + kind
 };
 
 struct dl4s_hip_graph {
@@ -105,12 +105,14 @@ int decode_static_scratch_init(dl4s_hip_ctx *ctx);
 
 // Kernel families of dl4s_hip_ctx::lds_limit_raised.
 enum { LDS_PREFILL_SPLIT = 0, LDS_PREFILL = 1, LDS_PREFILL_D128 = 2, LDS_BWD = 3, LDS_BWD_D128 = 4, LDS_GEMM_DEEP = 5, LDS_PREFILL_W192 = 6,
-       LDS_PREFILL_W256 = 7 };
+       LDS_PREFILL_W256 = 7, LDS_PREFILL_W160 = 8 };
 inline bool lds_limit_pending(const dl4s_hip_ctx *ctx, int family, int kind) {
-    return !(ctx->lds_limit_raised.load(std::memory_order_acquire) & (1ull << (family * 8 + kind)));
+    const int bit = family * 8 + kind;
+    return !(ctx->lds_limit_raised[bit >> 6].load(std::memory_order_acquire) & (1ull << (bit & 63)));
 }
 inline void lds_limit_done(dl4s_hip_ctx *ctx, int family, int kind) {
-    ctx->lds_limit_raised.fetch_or(1ull << (family * 8 + kind), std::memory_order_release);
+    const int bit = family * 8 + kind;
+    ctx->lds_limit_raised[bit >> 6].fetch_or(1ull << (bit & 63), std::memory_order_release);
 }
 
 inline int launch_status(const char *kernel) {

@@ -305,7 +305,7 @@ __device__ __forceinline__ float plain_score(const float *qs, const float *krow,
 // Head dims above 128 up to 256 that the 192- and 256-wide forward kernels take as they are (the tensors 16-byte aligned
 // besides): a multiple of 4 whose K/V rows of one (batch, head) pair stay inside the kernels' 32-bit byte offsets.
 inline bool sdpa_wide_route(int64_t H, int64_t Lk, int64_t d, int token_major) {
-    return d > HD2 && d <= 256 && d % 4 == 0 && Lk * (token_major ? H : 1) * d * 4 < ((d == 192 || d == 256) ? (1ll << 31) : (1ll << 30));
+    return d > HD2 && d <= 256 && d % 4 == 0 && Lk * (token_major ? H : 1) * d * 4 < ((d == 160 || d == 192 || d == 256) ? (1ll << 31) : (1ll << 30));
 }
 
 inline bool sdpa_padded_route(bool mfma_as_is, int64_t B, int64_t H, int64_t Lq, int64_t Lk, int64_t dk, int64_t dv) {

@@ -690,6 +690,7 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
         }
     }
     if (wide_path) {
+        if (dk <= 160) return launch_wide<160>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
         if (dk <= 192) return launch_wide<192>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
         return launch_wide<256>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
     }

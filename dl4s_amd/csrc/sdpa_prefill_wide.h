@@ -1,13 +1,13 @@
 // Fused attention forward for head dims above 128 and up to 256 (key dim = value dim, a multiple of 4): the transposed
-// two-contraction scheme of sdpa_prefill_f32_d128 on tiles that are W = 192 or W = 256 columns wide.  Included by
+// two-contraction scheme of sdpa_prefill_f32_d128 on tiles that are W = 160, 192 or 256 columns wide.  Included by
 // sdpa_prefill.hip only.
 //
 //   S^T[key, query] = K[key, :] . Q[query, :]       W/2 MFMA steps: step j contracts d = (W/2)*half + j
 //   O^T[d,   query] = V[key, d]^T . P^T[key, query]  W/32 accumulators in groups of columns: the first 128 columns on four
 //                                                   accumulators whose rows interleave (accumulator c row i is d = 4*i + c,
 //                                                   one 128-bit LDS read per key); the columns from 128 up the same way on
-//                                                   four more (W = 256: d = 128 + 4*i + c) or on two (W = 192:
-//                                                   d = 128 + 2*i + c, one 64-bit read)
+//                                                   four more (W = 256: d = 128 + 4*i + c), on two (W = 192:
+//                                                   d = 128 + 2*i + c, one 64-bit read) or on one (W = 160: d = 128 + i)
 //
 // The Q fragment (W/2 registers), the accumulators (W/2 registers) and the staged K/V pieces leave room for one wavefront per
 // SIMD; K/V in double-buffered LDS tiles of 32 keys on a (W + 4)-float row stride (4 x 32 x (W + 4) floats: 98 or 130 KiB,
@@ -20,11 +20,11 @@
 namespace {
 
 template <int W> struct WideFwdTile {
-    static_assert(W == 192 || W == 256, "tile widths above 128");
+    static_assert(W == 160 || W == 192 || W == 256, "tile widths above 128");
     static constexpr int LS = W + 4;              // LDS row stride (floats): 4 mod 32
     static constexpr int TF = BN * LS;            // floats per tile
     static constexpr int NC = W / 32;             // accumulators
-    static constexpr int NC2 = NC - 4;            // accumulators of the columns from 128 up: 2 or 4
+    static constexpr int NC2 = NC - 4;            // accumulators of the columns from 128 up: 1, 2 or 4
     static constexpr int PPR = W / 4;             // 128-bit pieces per tile row
     static constexpr int NP = BN * PPR / 256;     // pieces per thread and tile: thread tid moves the pieces tid, tid + 256, ...
 };
@@ -193,10 +193,12 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
                     o[5] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb.y, s0[r], o[5], 0, 0, 0);
                     o[6] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb.z, s0[r], o[6], 0, 0, 0);
                     o[7] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb.w, s0[r], o[7], 0, 0, 0);
-                } else {
+                } else if constexpr (NC2 == 2) {
                     const f32x2 vb = *reinterpret_cast<const f32x2 *>(Vb + v_lds2 + row_off);
                     o[4] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb.x, s0[r], o[4], 0, 0, 0);
                     o[5] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb.y, s0[r], o[5], 0, 0, 0);
+                } else {
+                    o[4] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vb[v_lds2 + row_off], s0[r], o[4], 0, 0, 0);
                 }
             }
         }
@@ -223,9 +225,17 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
             if constexpr (NC2 == 4) {
                 const f32x4 c4 = {o[4][r] * inv, o[5][r] * inv, o[6][r] * inv, o[7][r] * inv};
                 if (d2 < hd) *reinterpret_cast<f32x4 *>(op + d2) = c4;
-            } else {     // head dims are multiples of 4 and d2 is even: a pair is inside or outside as a whole
+            } else if constexpr (NC2 == 2) {     // head dims are multiples of 4 and d2 is even: a pair is inside or outside as a whole
                 const f32x2 c2 = {o[4][r] * inv, o[5][r] * inv};
                 if (d2 < hd) *reinterpret_cast<f32x2 *>(op + d2) = c2;
+            }
+        }
+        if constexpr (NC2 == 1) {     // registers 4g .. 4g+3 of the fifth accumulator are four consecutive columns
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d2 = 128 + 8 * g + 4 * half;
+                const f32x4 c4 = {o[4][4 * g + 0] * inv, o[4][4 * g + 1] * inv, o[4][4 * g + 2] * inv, o[4][4 * g + 3] * inv};
+                if (d2 < hd) *reinterpret_cast<f32x4 *>(op + d2) = c4;
             }
         }
     }
@@ -241,7 +251,7 @@ int launch_wide_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const fl
     int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
     if (lpt && total <= 1ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
     const size_t lds_bytes = 4 * WideFwdTile<W>::TF * sizeof(float);
-    constexpr int family = W == 192 ? dl4s::LDS_PREFILL_W192 : dl4s::LDS_PREFILL_W256;
+    constexpr int family = W == 160 ? dl4s::LDS_PREFILL_W160 : (W == 192 ? dl4s::LDS_PREFILL_W192 : dl4s::LDS_PREFILL_W256);
     if (dl4s::lds_limit_pending(ctx, family, KIND)) {
         DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&sdpa_prefill_f32_wide<KIND, W>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));

@@ -164,7 +164,7 @@ typedef struct dl4s_mask_desc {
  * widths is padded with zero columns on the fly and costs what the wider tile costs.  Even head dims
  * from 66 to 94 that are not a multiple of 4 run the 96-wide kernel as they are (8-byte aligned
  * tensors, launches that fill the GPU).  dk = dv above 128 up to 256 (a multiple of 4, aligned) runs
- * the same scheme on tiles of 192 or 256 columns.  Other head dims up to 256 (dk != dv, odd,
+ * the same scheme on tiles of 160, 192 or 256 columns.  Other head dims up to 256 (dk != dv, odd,
  * unaligned tensors) run the same kernels on zero-padded copies of the operands, which the call
  * allocates from the context's pool, when the problem is large enough to pay for the copies; small
  * problems of such head dims run a plain fused kernel.  Head dims above 256 are refused. */
