@@ -173,7 +173,8 @@ int dl4s_hip_sdpa_fwd_f32(dl4s_hip_ctx *ctx, const float *q, const float *k, con
                           float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags);
 
 /* Training form of the fused attention (key dim = value dim = d; MFMA kernels for d a multiple of 4 up to 256 and 16-byte
- * aligned tensors - above 128 the gradients are batched MFMA products around one elementwise pass, head-major layout only -
+ * aligned tensors - above 128 the gradients are batched MFMA products around one elementwise pass that forms its own row
+ * statistics (stats is not read there), head-major layout only -
  * plain kernels for what those do not take, up to 256).  The reference differentiates ScaledDotProductAttention through
  * the backward closures of its primitive operators (Tensor/Operators/Matrix.swift:139-174 for the products through the
  * subscript views and the stack of broadcastMatrixMultiplied :79-117, Binary.swift:235-300 for e / sum,
