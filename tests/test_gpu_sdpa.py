@@ -209,7 +209,7 @@ def test_blocked_keys_have_exactly_zero_weight_and_blocked_rows_are_uniform(ctx,
     assert not np.isnan(base).any()
 
 
-@pytest.mark.parametrize("d", [64, 8, 32, 128, 10])
+@pytest.mark.parametrize("d", [64, 8, 32, 128, 10, 16, 48, 80, 96, 160, 256])
 @pytest.mark.parametrize("mk", ["dense", "dense_ones_tiles", "lens", "causal_lens"])
 def test_fully_blocked_rows_with_large_scores_follow_the_reference_rounding(ctx, orc, d, mk):
     """A row whose every key is blocked: the reference's fl(s - 1e9) keeps a score only as its bucket on the grid of 64

@@ -329,7 +329,7 @@ def test_gradients_after_the_96_wide_forward_kernel(ctx, orc, d, mask_kind):
     assert np.isfinite(dq).all() and np.isfinite(dk).all() and np.isfinite(dv).all()
 
 
-@pytest.mark.parametrize("d", [64, 32, 128, 6])
+@pytest.mark.parametrize("d", [64, 32, 128, 6, 256, 160, 48, 80, 16])
 @pytest.mark.parametrize("mask_kind", ["dense", "lengths"])
 def test_gradients_of_fully_blocked_rows_with_large_scores(ctx, orc, d, mask_kind):
     """Rows with every key blocked and scores beyond +-32: the reference's weights there are set by the rounding of
