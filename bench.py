@@ -476,7 +476,7 @@ def cpu_blas_proxy_prefill(q, k, v, pairs):
 def kernel_sample(ctx, lib, iters):
     """A short fixed sequence of the kernels behind configs 3 and 4 that the headline run does not time one by one (the
     fused Dense products, the dense-mask attention of config 3, the attention gradients, forward and gradients at head dims
-    128, 96 and 32), `iters` launches each, for
+    128, 96, 32, 256, 80, 48 and 16), `iters` launches each, for
     counter runs of a profiler: no pre-heat loops, a few dozen launches in all.  Returns the mean event time of each."""
     rng = np.random.Generator(np.random.PCG64(1007))
     res = {}
@@ -521,8 +521,8 @@ def kernel_sample(ctx, lib, iters):
           lambda: ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], outs[0], st, bufs[3], outs[1], outs[2], outs[3], B, H, L, L, 64, 0.125, desc, 0))
     for b_ in bufs + outs + [st]:
         b_.release()
-    # the same shape at other head dims: forward and gradients on the 128-, 96- and 32-wide tiles
-    for d in (128, 96, 32):
+    # the same shape at other head dims: forward and gradients on the other tile widths
+    for d in (128, 96, 32, 256, 80, 48, 16):
         bufs = [ctx.to_device(rng.standard_normal((B, H, L, d), dtype=np.float32) * np.float32(0.5)) for _ in range(4)]
         outs = [ctx.empty((B, H, L, d)) for _ in range(4)]
         st = ctx.empty((B, H, L, 2))
