@@ -41,12 +41,12 @@ template <int CTRL>
 __device__ __forceinline__ float dpp(float x) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
 }
-// Sum over the LPR (8, 16 or 32) lanes that share a cache row; every one of them ends up with the total.
+// Sum over the LPR (4, 8, 16 or 32) lanes that share a cache row; every one of them ends up with the total.
 template <int LPR>
 __device__ __forceinline__ float row_sum(float x) {
     x += dpp<0xB1>(x);   // quad_perm [1,0,3,2]
     x += dpp<0x4E>(x);   // quad_perm [2,3,0,1]
-    x += dpp<0x141>(x);  // row_half_mirror
+    if (LPR >= 8) x += dpp<0x141>(x);  // row_half_mirror
     if (LPR >= 16) x += dpp<0x140>(x);  // row_mirror
     if (LPR >= 32) x += __shfl_xor(x, 16, 64);
     return x;
@@ -68,7 +68,8 @@ __device__ __forceinline__ float row_sum(float x) {
 // key, the penalty is applied to all of them and the row comes out uniform, as in the reference.
 // SEG: the row is read as SEG consecutive segments of 4 * LPR floats by the same LPR lanes (SEG loads per row and lane, NK =
 // 4 keys per lane and iteration instead of 8).  SEG = 3 with LPR = 8 (16) serves rows of 96 (192) floats with every lane busy,
-// where the one-piece form would leave a quarter of the lanes idle; SEG = 2 with LPR = 32 serves rows of 129 to 256 floats.
+// where the one-piece form would leave a quarter of the lanes idle; SEG = 5 with LPR = 4 (8) rows of 80 (160) floats, 2 keys per
+// lane and iteration; SEG = 2 with LPR = 32 serves rows of 129 to 256 floats.
 template <bool APPEND, int NW, int LPR, bool FULL, bool DEVPOS = false, int SEG = 1>
 __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
                                                                    float *vcache, const float *__restrict__ k_new,
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
                                                                    int pos, float rT, int nsplit, int chunk, int d, int H,
                                                                    const int *__restrict__ lengths,
                                                                    const int *__restrict__ pos_dev = nullptr, int vec = 4) {
-    constexpr int SW = 4 * LPR, D = SW * SEG, G = 64 / LPR, NK = SEG == 1 ? 8 : 4, KB = NK * G, PSTR = pstr(D);
+    constexpr int SW = 4 * LPR, D = SW * SEG, G = 64 / LPR, NK = SEG == 1 ? 8 : (SEG <= 3 ? 4 : 2), KB = NK * G, PSTR = pstr(D);
     __shared__ float sm_o[NW][D];
     __shared__ float sm_m[NW], sm_l[NW];
     if (DEVPOS) {
@@ -321,13 +322,24 @@ __global__ void kv_append_f32(float *kcache, float *vcache, const float *__restr
 }
 
 // Row widths the kernel is instantiated for: 32, 64, 128 floats (8, 16, 32 lanes per row, one 128-bit piece per lane), 96 and
-// 192 floats (8 and 16 lanes per row, three pieces per lane) and 256 floats (32 lanes per row, two pieces per lane).
-// (the three-piece forms for exactly 96 or 192 floats and 128-bit pieces: with part-filled or narrower pieces its three loads per lane
+// 192 floats (8 and 16 lanes per row, three pieces per lane), 80 and 160 floats (4 and 8 lanes per row, five pieces per lane)
+// and 256 floats (32 lanes per row, two pieces per lane).
+// (the three- and five-piece forms for exactly 96 / 192 and 80 / 160 floats and 128-bit pieces: with part-filled or narrower pieces its three loads per lane
 // cost more than the idle lanes of the 128-float form - B16 H16 over 4096 rows: d = 96 163 -> 137 us, d = 80 160 -> 175 us)
-inline int row_segments(int64_t d, int vec) { return (d == 96 || d == 192) && vec == 4 ? 3 : (d > 128 ? 2 : 1); }
-inline int lanes_per_row(int64_t d, int vec) { return row_segments(d, vec) == 3 ? (int)d / 12 : (d <= 32 ? 8 : (d <= 64 ? 16 : 32)); }
+inline int row_segments(int64_t d, int vec) {
+    if (vec == 4 && (d == 96 || d == 192)) return 3;
+    if (vec == 4 && (d == 80 || d == 160)) return 5;
+    return d > 128 ? 2 : 1;
+}
+inline int lanes_per_row(int64_t d, int vec) {
+    const int seg = row_segments(d, vec);
+    return seg == 3 ? (int)d / 12 : (seg == 5 ? (int)d / 20 : (d <= 32 ? 8 : (d <= 64 ? 16 : 32)));
+}
 inline int row_width(int64_t d, int vec) { return 4 * lanes_per_row(d, vec) * row_segments(d, vec); }
-inline int keys_per_iteration(int64_t d, int vec) { return (row_segments(d, vec) == 1 ? 8 : 4) * (64 / lanes_per_row(d, vec)); }
+inline int keys_per_iteration(int64_t d, int vec) {
+    const int seg = row_segments(d, vec);
+    return (seg == 1 ? 8 : (seg <= 3 ? 4 : 2)) * (64 / lanes_per_row(d, vec));
+}
 
 // 4 when every cache row starts on a 16-byte boundary (the row length a multiple of 4 floats, every operand aligned): a lane
 // reads its piece of a row with one 128-bit load.  2 for an even row length and 8-byte aligned operands (two 64-bit loads),
@@ -342,10 +354,10 @@ template <bool APPEND, int NW, int LPR, bool DEVPOS, int SEG = 1>
 void decode_launch_kernel(dl4s_hip_ctx *ctx, dim3 grid, const float *q, float *kcache, float *vcache, const float *k_new,
                           const float *v_new, float *out, float *part, int T, int Tcap, int pos, float rT, int nsplit, int chunk,
                           int d, int H, const int *lengths, const int *pos_dev, int vec) {
-    if (SEG == 3 || (d == 4 * LPR * SEG && vec == 4))      // the 96-float form is only chosen for full rows
+    if (SEG == 3 || SEG == 5 || (d == 4 * LPR * SEG && vec == 4))      // the three- and five-piece forms are only chosen for full rows
         hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, true, DEVPOS, SEG>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
                            k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, 4);
-    else if constexpr (SEG != 3)
+    else if constexpr (SEG != 3 && SEG != 5)
         hipLaunchKernelGGL((sdpa_decode_splitk_f32<APPEND, NW, LPR, false, DEVPOS, SEG>), grid, dim3(NW * 64), 0, ctx->stream, q, kcache, vcache,
                            k_new, v_new, out, part, T, Tcap, pos, rT, nsplit, chunk, d, H, lengths, pos_dev, vec);
 }
@@ -359,6 +371,10 @@ void decode_launch_width(dl4s_hip_ctx *ctx, int nw, dim3 grid, const float *q, f
         if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS, 3>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS, 3>(DL4S_DECODE_ARGS);
     } else if (row_segments(d, vec) == 3) {
         if (nw == 16) decode_launch_kernel<APPEND, 16, 16, DEVPOS, 3>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 16, DEVPOS, 3>(DL4S_DECODE_ARGS);
+    } else if (row_segments(d, vec) == 5 && d == 80) {
+        if (nw == 16) decode_launch_kernel<APPEND, 16, 4, DEVPOS, 5>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 4, DEVPOS, 5>(DL4S_DECODE_ARGS);
+    } else if (row_segments(d, vec) == 5) {
+        if (nw == 16) decode_launch_kernel<APPEND, 16, 8, DEVPOS, 5>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 8, DEVPOS, 5>(DL4S_DECODE_ARGS);
     } else if (row_segments(d, vec) == 2) {
         if (nw == 16) decode_launch_kernel<APPEND, 16, 32, DEVPOS, 2>(DL4S_DECODE_ARGS); else decode_launch_kernel<APPEND, 4, 32, DEVPOS, 2>(DL4S_DECODE_ARGS);
     } else switch (lanes_per_row(d, vec)) {

@@ -493,7 +493,7 @@ def test_decode_matches_oracle(ctx, orc, B, H, T, Tcap):
     assert_parity(got, pre, "decode vs prefill")
 
 
-@pytest.mark.parametrize("d", [32, 128, 8, 4, 40, 96, 100, 70, 1, 3, 6, 33, 127, 256, 192, 130, 255])
+@pytest.mark.parametrize("d", [32, 128, 8, 4, 40, 96, 100, 70, 1, 3, 6, 33, 127, 256, 192, 130, 255, 80, 160])
 @pytest.mark.parametrize("B,H,T,Tcap", [(1, 1, 1, 1), (2, 3, 9, 12), (2, 2, 129, 140), (1, 4, 257, 300), (1, 8, 513, 600),
                                         (3, 2, 1000, 1024), (2, 2, 4097, 4160)])
 def test_decode_other_head_dims(ctx, orc, B, H, T, Tcap, d):
@@ -509,7 +509,7 @@ def test_decode_other_head_dims(ctx, orc, B, H, T, Tcap, d):
     assert_parity(got, run_sdpa(ctx, q, np.ascontiguousarray(kc[:, :, :T]), np.ascontiguousarray(vc[:, :, :T])), "decode vs prefill")
 
 
-@pytest.mark.parametrize("d", [64, 32, 128, 24, 70, 5, 96, 256, 200, 192])
+@pytest.mark.parametrize("d", [64, 32, 128, 24, 70, 5, 96, 256, 200, 192, 80, 160])
 @pytest.mark.parametrize("B,H,T,Tcap", [(4, 2, 9, 12), (5, 2, 300, 320), (6, 3, 1000, 1024), (4, 2, 4097, 4160)])
 def test_decode_with_key_lengths(ctx, orc, B, H, T, Tcap, d):
     """dl4s_hip_sdpa_decode_lengths_f32 against the oracle's attention on the gathered tensors under the padding mask
@@ -536,7 +536,7 @@ def test_decode_with_key_lengths(ctx, orc, B, H, T, Tcap, d):
 
 
 @pytest.mark.parametrize("shift", [1, 2])
-@pytest.mark.parametrize("d", [64, 128, 20, 96, 256, 192])
+@pytest.mark.parametrize("d", [64, 128, 20, 96, 256, 192, 80])
 @pytest.mark.parametrize("T,Tcap", [(9, 12), (700, 701), (4100, 4100)])
 def test_decode_on_operands_off_the_16_byte_grid(ctx, orc, T, Tcap, d, shift):
     """Every operand 4 or 8 bytes past a 16-byte boundary (a view into a larger buffer): the kernel reads 32 or 64 bits per
@@ -552,7 +552,7 @@ def test_decode_on_operands_off_the_16_byte_grid(ctx, orc, T, Tcap, d, shift):
     off = 4 * shift
     ctx.sdpa_decode(dq.offset(off), dk_.offset(off), dv_.offset(off), dout.offset(off), B, H, T, Tcap, d, rT)
     got = dout.numpy()[shift:].reshape(B, H, 1, d)
-    if d not in (96, 192):     # aligned rows of exactly 96 or 192 floats run a form of their own (three pieces per lane): another summation order
+    if d not in (96, 192, 80, 160):     # aligned rows of exactly 96, 192, 80 or 160 floats run forms of their own (three pieces per lane): another summation order
         assert np.array_equal(got, aligned)
     assert_parity(got, orc.sdpa_decode(q, kc, vc, T), "decode, unaligned operands")
     if T < Tcap:
@@ -662,7 +662,7 @@ def test_config5_incremental_decode_append_then_attend(ctx, orc):
         buf.release()
 
 
-@pytest.mark.parametrize("d", [64, 30, 7, 96, 256, 132, 192])
+@pytest.mark.parametrize("d", [64, 30, 7, 96, 256, 132, 192, 80, 160])
 @pytest.mark.parametrize("Tcap,steps", [(300, 260), (100, 90)])      # workgroups of 16 and of 4 wavefronts
 def test_decode_step_with_the_position_in_device_memory(ctx, orc, Tcap, steps, d):
     """dl4s_hip_sdpa_decode_step_at_f32 reads the row to append from device memory: a sequence of steps driven by a
