@@ -525,8 +525,10 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                            ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb32, (int)total32, token_major, stats, hd, split_order);
         return dl4s::launch_status("sdpa_prefill_split_f32_d64");
     }
-    // head dims 36 .. 48: the 48-column form of the narrow kernel (48 MFMA units per tile instead of 64)
-    if (hd <= 48) return launch_narrow48_main<KIND>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+    // head dims 36 .. 48: the 48-column form of the narrow kernel (48 MFMA units per tile instead of 64) - unless the call
+    // leaves row statistics: the gradient kernels form the scores again in the 64-column order, and the statistics must
+    // belong to those scores to the last bit
+    if (hd <= 48 && !stats) return launch_narrow48_main<KIND>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
     const int nqb = (Lq + BM - 1) / BM;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     // longest-first order for causal masks.  Measured on B8 H16 L2048 causal with the order applied to groups of
