@@ -1190,9 +1190,11 @@ extern "C" int dl4s_hip_sdpa_bwd_f32(dl4s_hip_ctx *ctx, const float *q, const fl
                            rows, token_major, (int)d);
         rc = dl4s::launch_status("sdpa_bwd_rowdot128");
         if (rc == DL4S_HIP_OK) {
-            // head dims up to 96 on 96-wide tiles (three quarters of the MFMAs), the others on 128-wide ones
+            // head dims up to 96 on 96-wide tiles (three quarters of the MFMAs; up to 80 on their 80-column form, like the
+            // forward call that left the statistics), the others on 128-wide ones
 #define DL4S_BWD_WIDE(KIND_) \
-    rc = d <= 96 ? launch_bwd128<KIND_, 96>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split) \
+    rc = d <= 80 ? launch_bwd128<KIND_, 80>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split) \
+       : d <= 96 ? launch_bwd128<KIND_, 96>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split) \
                  : launch_bwd128<KIND_, 128>(ctx, q, k, v, dout, stats, D, dq, dk, dv, B, H, Lq, Lk, inv_temperature, m, strict, token_major, (int)d, ds_scratch_max_bytes(), no_split)
             switch (m.kind) {
                 case DL4S_MASK_NONE: DL4S_BWD_WIDE(DL4S_MASK_NONE); break;

@@ -1,6 +1,6 @@
 // Gradients of the fused attention for head dims above 64 and up to 128 (multiples of 4): the deterministic kernels of
-// sdpa_backward.hip on tiles that are W = 128 columns wide, or W = 96 for head dims up to 96.  Included by
-// sdpa_backward.hip only.
+// sdpa_backward.hip on tiles that are W = 128 columns wide, W = 96 for head dims up to 96, or the 80-column form of the
+// latter for head dims up to 80.  Included by sdpa_backward.hip only.
 //
 // The operand layouts follow the forward kernels of the same width.  A score product contracts d = (W/2)*half + j over
 // W/2 MFMA steps.  A transposed accumulation (dQ^T, dK^T, dV^T) uses W/32 accumulators.  W = 128: their rows interleave
@@ -56,54 +56,97 @@ __device__ __forceinline__ f32x16 tile_product_w(const float *Ab, const float (&
     return acc;
 }
 
-// What depends on the tile width W
+// What depends on the tile width W.  W = 80 (head dims up to 80): the LDS tiles of W = 96 (columns from the head dim up are
+// zeros either way), score products that contract 40 steps per half, and transposed accumulations whose columns 64 .. 79
+// live in two 16 x 16 accumulators on v_mfma_f32_16x16x4_f32 (the wavefront's columns 0-15 and 16-31; lane: column =
+// lane % 16, rows d = 64 + 4 * (lane / 16) + i) fed through v_permlane16_swap - see attend_tile_16 in sdpa_prefill_narrow.h.
 template <int W> struct WideTile {
-    static constexpr int LS = W + 4;              // LDS row stride (floats): 4 mod 32
+    static constexpr int SW = W == 80 ? 96 : W;   // columns of a tile in LDS
+    static constexpr int LS = SW + 4;             // LDS row stride (floats): 4 mod 32
     static constexpr int TF = BN * LS;            // floats per tile
     static constexpr int HALF = W / 2;            // columns a half of the wavefront contracts in a score product
     static constexpr int NJ = W / 8;              // 128-bit reads per row fragment
-    static constexpr int NC = W / 32;             // accumulators of a transposed product
-    static constexpr int PPR = W / 4;             // 128-bit pieces per tile row
+    static constexpr int NC = W == 80 ? 2 : W / 32;   // 32 x 32 accumulators of a transposed product
+    static constexpr int PPR = SW / 4;            // 128-bit pieces per tile row
     static constexpr int NP = BN * PPR / 256;     // pieces per thread and tile: thread tid moves the pieces tid, tid + 256, ...
-    // transposed-operand base of a lane inside a [32][LS] tile (row 4*half + const)
-    static __device__ __forceinline__ int col_base(const int half, const int ln) { return (4 * half) * LS + (W == 128 ? 4 * ln : ln); }
-    // acc[c] (column = the lane's query or key) += A^T . B where A is a [32][LS] LDS tile (At points at the lane's base)
-    // and B the accumulator-layout tile b
-    static __device__ __forceinline__ void accumulate(const float *At, const f32x16 &b, f32x16 (&acc)[NC]) {
+    // the accumulators of one transposed product (column = the lane's query or key); g: W = 80 only
+    struct Acc {
+        f32x16 a[NC];
+        f32x4 g[2];
+    };
+    static __device__ __forceinline__ void zero(Acc &x) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) x.a[c][i] = 0.f;
+        x.g[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+        x.g[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    // acc += A^T . B where A is a [32][LS] LDS tile and B the accumulator-layout tile b
+    static __device__ __forceinline__ void accumulate(const float *tile, const int half, const int ln, const int lane, const f32x16 &b,
+                                                      Acc &acc) {
+        const float *At = tile + (4 * half) * LS + (W == 128 ? 4 * ln : ln);   // the lane's base: row 4*half + const
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const float *ar = At + (8 * (r >> 2) + (r & 3)) * LS;
             if constexpr (W == 128) {
                 const f32x4 a = *reinterpret_cast<const f32x4 *>(ar);
-                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[r], acc[0], 0, 0, 0);
-                acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[r], acc[1], 0, 0, 0);
-                acc[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b[r], acc[2], 0, 0, 0);
-                acc[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b[r], acc[3], 0, 0, 0);
+                acc.a[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[r], acc.a[0], 0, 0, 0);
+                acc.a[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[r], acc.a[1], 0, 0, 0);
+                acc.a[2] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b[r], acc.a[2], 0, 0, 0);
+                acc.a[3] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b[r], acc.a[3], 0, 0, 0);
             } else {
 #pragma unroll
-                for (int c = 0; c < NC; ++c) acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[32 * c], b[r], acc[c], 0, 0, 0);
+                for (int c = 0; c < NC; ++c) acc.a[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(ar[32 * c], b[r], acc.a[c], 0, 0, 0);
+            }
+        }
+        if constexpr (W == 80) {
+            const int slot = lane >> 4;
+            const float *At16 = tile + ((slot & 1) + 4 * (slot >> 1)) * LS + 64 + (lane & 15);
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(b[2 * p]), __float_as_uint(b[2 * p + 1]), false, false);
+                const float a = At16[(8 * (p >> 1) + 2 * (p & 1)) * LS];
+                acc.g[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, __uint_as_float(sw[0]), acc.g[0], 0, 0, 0);
+                acc.g[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, __uint_as_float(sw[1]), acc.g[1], 0, 0, 0);
             }
         }
     }
-    // stores the lane's row of the transposed accumulators to p[0 .. hd-1], scaled
-    static __device__ __forceinline__ void store_row(float *p, const f32x16 (&acc)[NC], const float scale, const int half, const int hd) {
-        if constexpr (W == 128) {
+    // Stores the wavefront's 32 rows row0 .. row0 + 31 (those below nrows) of the transposed accumulators, scaled, to
+    // base[row * stride + 0 .. ncols - 1]: the lane's own row row0 + ln from the 32 x 32 accumulators, the rows
+    // row0 + 16 g + lane % 16 from the 16 x 16 ones.
+    static __device__ __forceinline__ void store_rows(float *base, const long long stride, const int row0, const int nrows, const Acc &acc,
+                                                      const float scale, const int half, const int ln, const int lane, const int ncols) {
+        if (row0 + ln < nrows) {
+            float *p = base + (long long)(row0 + ln) * stride;
+            if constexpr (W == 128) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int d0 = 4 * (8 * (r >> 2) + 4 * half + (r & 3));
-                f32x4 a;
-                a.x = acc[0][r] * scale; a.y = acc[1][r] * scale; a.z = acc[2][r] * scale; a.w = acc[3][r] * scale;
-                if (d0 < hd) *reinterpret_cast<f32x4 *>(p + d0) = a;
-            }
-        } else {
-#pragma unroll
-            for (int c = 0; c < NC; ++c)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int d0 = 32 * c + 8 * g + 4 * half;
-                    const f32x4 a = {acc[c][4 * g + 0] * scale, acc[c][4 * g + 1] * scale, acc[c][4 * g + 2] * scale, acc[c][4 * g + 3] * scale};
-                    if (d0 < hd) *reinterpret_cast<f32x4 *>(p + d0) = a;
+                for (int r = 0; r < 16; ++r) {
+                    const int d0 = 4 * (8 * (r >> 2) + 4 * half + (r & 3));
+                    f32x4 a;
+                    a.x = acc.a[0][r] * scale; a.y = acc.a[1][r] * scale; a.z = acc.a[2][r] * scale; a.w = acc.a[3][r] * scale;
+                    if (d0 < ncols) *reinterpret_cast<f32x4 *>(p + d0) = a;
                 }
+            } else {
+#pragma unroll
+                for (int c = 0; c < NC; ++c)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int d0 = 32 * c + 8 * g + 4 * half;
+                        const f32x4 a = {acc.a[c][4 * g + 0] * scale, acc.a[c][4 * g + 1] * scale, acc.a[c][4 * g + 2] * scale,
+                                         acc.a[c][4 * g + 3] * scale};
+                        if (d0 < ncols) *reinterpret_cast<f32x4 *>(p + d0) = a;
+                    }
+            }
+        }
+        if constexpr (W == 80) {
+            const int d0 = 64 + 4 * (lane >> 4);
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                const int row = row0 + 16 * g + (lane & 15);
+                const f32x4 a = {acc.g[g].x * scale, acc.g[g].y * scale, acc.g[g].z * scale, acc.g[g].w * scale};
+                if (row < nrows && d0 < ncols) *reinterpret_cast<f32x4 *>(base + (long long)row * stride + d0) = a;
+            }
         }
     }
 };
@@ -198,17 +241,13 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
         }
     };
 
-    f32x16 acc[WT::NC];   // dQ^T
-#pragma unroll
-    for (int c = 0; c < WT::NC; ++c)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
+    typename WT::Acc acc;   // dQ^T
+    WT::zero(acc);
 
     if (ntiles > 0) { load_tile(0); store_tile(0); }
     __syncthreads();
 
     const int row_lds = ln * WT::LS + half * WT::HALF;  // row-fragment base (S^T and dP^T products)
-    const int col_lds = WT::col_base(half, ln);   // transposed-fragment base (dQ^T product)
     const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
@@ -227,12 +266,12 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dq_f32_d128(const float *__re
             const f32x16 dp = tile_product_w<WT::NJ>(Vs + buf * WT::TF + row_lds, gr);            // dP^T = V . dout^T
 #pragma unroll
             for (int r = 0; r < 16; ++r) p[r] = p[r] * (dp[r] - D_i);                            // dS^T
-            WT::accumulate(Ks + buf * WT::TF + col_lds, p, acc);                     // dQ^T += K^T . dS^T
+            WT::accumulate(Ks + buf * WT::TF, half, ln, lane, p, acc);               // dQ^T += K^T . dS^T
         }
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
-    if (qi < Lq) WT::store_row(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
+    WT::store_rows(dq + q_base, rs, q0, Lq, acc, rT, half, ln, lane, hd);
 }
 
 // ------------------------------------------------------------------------------------------------ dK, dV
@@ -344,11 +383,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
         if (tid < 96) Ss[(tid >> 5) * 64 + buf * 32 + (tid & 31)] = sst;
     };
 
-    f32x16 ka[WT::NC], va[WT::NC];   // dK^T and dV^T
-#pragma unroll
-    for (int c = 0; c < WT::NC; ++c)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) { ka[c][i] = 0.f; va[c][i] = 0.f; }
+    typename WT::Acc ka, va;   // dK^T and dV^T
+    WT::zero(ka);
+    WT::zero(va);
 
     const int sp = blockIdx.y;
     int t = t_begin + (((sp - t_begin) % nsplit) + nsplit) % nsplit;   // the share's first tile at or after t_begin
@@ -356,7 +393,6 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
     __syncthreads();
 
     const int row_lds = ln * WT::LS + half * WT::HALF;
-    const int col_lds = WT::col_base(half, ln);
     const unsigned char *cls_col = nullptr;
     if (DENSE && mask.cls) cls_col = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(kw0, Lk - 1) >> 5) * mask.cls_sk;
     const float *mcol = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + keyc * mask.sk : nullptr;
@@ -417,7 +453,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                 p[4 * g + 2] = fast_exp2(p[4 * g + 2] - m4.z) * r4.z;
                 p[4 * g + 3] = fast_exp2(p[4 * g + 3] - m4.w) * r4.w;
             }
-            WT::accumulate(Gs + buf * WT::TF + col_lds, p, va);                      // dV^T += dout^T . P
+            WT::accumulate(Gs + buf * WT::TF, half, ln, lane, p, va);                // dV^T += dout^T . P
             const f32x16 dp = tile_product_w<WT::NJ>(Gs + buf * WT::TF + row_lds, vr);            // dP = dout . V^T
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
@@ -436,24 +472,20 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o), dsrsrc, (int)ds_voff, (qt0 + 8 * g) * 4, 0);
                 }
             }
-            WT::accumulate(Qs + buf * WT::TF + col_lds, p, ka);                      // dK^T += Q~^T . dS
+            WT::accumulate(Qs + buf * WT::TF, half, ln, lane, p, ka);                // dK^T += Q~^T . dS
         }
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
     if (part) {
-        if (key < Lk) {
-            const long long rows = (long long)(total_blocks / nkb) * Lk;
-            float *pp = part + (((long long)sp * 2) * rows + (long long)bh * Lk + key) * HD2;
-            WT::store_row(pp, ka, 1.0f, half, W);
-            WT::store_row(pp + rows * HD2, va, 1.0f, half, W);
-        }
+        const long long rows = (long long)(total_blocks / nkb) * Lk;
+        float *pp = part + (((long long)sp * 2) * rows + (long long)bh * Lk) * HD2;
+        WT::store_rows(pp, HD2, kw0, Lk, ka, 1.0f, half, ln, lane, W);
+        WT::store_rows(pp + rows * HD2, HD2, kw0, Lk, va, 1.0f, half, ln, lane, W);
         return;
     }
-    if (key < Lk) {
-        WT::store_row(dv + kv_base + (long long)key * rs, va, 1.0f, half, hd);
-        WT::store_row(dk + kv_base + (long long)key * rs, ka, 0.69314718055994530942f, half, hd);   // Q~ carries log2(e)
-    }
+    WT::store_rows(dv + kv_base, rs, kw0, Lk, va, 1.0f, half, ln, lane, hd);
+    WT::store_rows(dk + kv_base, rs, kw0, Lk, ka, 0.69314718055994530942f, half, ln, lane, hd);   // Q~ carries log2(e)
 }
 
 // out[row][0 .. hd-1] = scale * (share 0 + share 1 + ...) of unscaled partial sums part[share][rows][128] (shares
@@ -558,11 +590,8 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
             dsn[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dsrsrc, (int)ds_voff, (int)(base + (unsigned)(8 * (r >> 2) + (r & 3)) * ds_row), 2));
     };
 
-    f32x16 acc[WT::NC];   // dQ^T
-#pragma unroll
-    for (int c = 0; c < WT::NC; ++c)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[c][i] = 0.f;
+    typename WT::Acc acc;   // dQ^T
+    WT::zero(acc);
 #pragma unroll
     for (int i = 0; i < 16; ++i) dsn[i] = 0.f;
 
@@ -573,7 +602,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
         if (visited(sp)) load_ds(sp);
     }
     __syncthreads();
-    const int col_lds = WT::col_base(half, ln);
     for (int t = sp, buf = 0; t < ntiles; t += nsplit, buf ^= 1) {
         const bool more = (t + nsplit < ntiles);
         const bool now = visited(t);
@@ -582,15 +610,15 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
             load_tile(t + nsplit);
             if (visited(t + nsplit)) load_ds(t + nsplit);
         }
-        if (now) WT::accumulate(Ks + buf * WT::TF + col_lds, p, acc);               // dQ^T += K^T . dS^T
+        if (now) WT::accumulate(Ks + buf * WT::TF, half, ln, lane, p, acc);         // dQ^T += K^T . dS^T
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
     if (part) {
-        if (qi < Lq) WT::store_row(part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * HD2, acc, 1.0f, half, W);
+        WT::store_rows(part + (((long long)sp * (total_blocks / nqb) + bh) * Lq) * HD2, HD2, q0, Lq, acc, 1.0f, half, ln, lane, W);
         return;
     }
-    if (qi < Lq) WT::store_row(dq + q_base + (long long)qi * rs, acc, rT, half, hd);
+    WT::store_rows(dq + q_base, rs, q0, Lq, acc, rT, half, ln, lane, hd);
 }
 
 template <int KIND, int W = 128>

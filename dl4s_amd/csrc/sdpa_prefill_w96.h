@@ -318,13 +318,12 @@ int launch_w96_width(dl4s_hip_ctx *ctx, const float *q, const float *k, const fl
     }
 }
 
-// head dims up to 80 on the 80-column form, the others on all 96.  A call that leaves row statistics for the gradient kernels
-// runs all 96: those kernels form the scores again in the 96-column order, and statistics from another summation order would
-// not belong to their scores to the last bit (which a score on the edge of a blocked row's rounding bucket needs).
+// head dims up to 80 on the 80-column form, the others on all 96 (the gradient kernels choose by the same rule, so that they
+// form the scores in the summation order of the call that left the row statistics)
 template <int VEC>
 int launch_w96(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk, float rT,
                const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit = 1, float *part = nullptr) {
-    if (hd <= 80 && !stats) return launch_w96_width<VEC, 80>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+    if (hd <= 80) return launch_w96_width<VEC, 80>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
     return launch_w96_width<VEC, 96>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
 }
 
