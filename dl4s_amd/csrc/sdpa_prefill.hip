@@ -646,10 +646,26 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     size_t part_bytes = 0;
     if ((mfma128_path || (w96_path && dk % 4 == 0)) && !no_split) {
         const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
+        // enough shares to give every CU its workgroup; two where every CU just has one (blocks of different length then pair up
+        // long with short, the odd shares walking the block order backwards: B2 H8 L2048 d256 causal 570 -> 510 us; without a
+        // mask 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
         if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
-            long long want = (2ll * ctx->cu_count + blocks - 1) / blocks;
+            long long want = std::max(2ll, ((long long)ctx->cu_count + blocks - 1) / blocks);
             want = std::min(want, std::min(8ll, nkt / 2));
             const size_t bytes = (size_t)want * B * H * Lq * PART2_STRIDE * sizeof(float);
+            if (want > 1 && bytes <= (size_t(256) << 20)) { nsplit128 = (int)want; part_bytes = bytes; }
+        }
+    }
+    // the wide kernels run one workgroup per CU: the same split on launches that leave CUs without one
+    if (wide_path && !no_split) {
+        const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
+        // enough shares to give every CU its workgroup; two where every CU just has one (blocks of different length then pair up
+        // long with short, the odd shares walking the block order backwards: B2 H8 L2048 d256 causal 570 -> 510 us; without a
+        // mask 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
+        if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
+            long long want = std::max(2ll, ((long long)ctx->cu_count + blocks - 1) / blocks);
+            want = std::min(want, std::min(8ll, nkt / 2));
+            const size_t bytes = (size_t)want * B * H * Lq * PARTW_STRIDE * sizeof(float);
             if (want > 1 && bytes <= (size_t(256) << 20)) { nsplit128 = (int)want; part_bytes = bytes; }
         }
     }
@@ -692,9 +708,10 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
         }
     }
     if (wide_path) {
-        if (dk <= 160) return launch_wide<160>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
-        if (dk <= 192) return launch_wide<192>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
-        return launch_wide<256>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk);
+        float *partw = static_cast<float *>(part128);
+        if (dk <= 160) return launch_wide<160>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, partw);
+        if (dk <= 192) return launch_wide<192>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, partw);
+        return launch_wide<256>(ctx, q, k, v, out, B, H, Lq, Lk, inv_temperature, m, strict, token_major, stats, (int)dk, nsplit128, partw);
     }
     DL4S_REQUIRE(!token_major, DL4S_HIP_EUNSUPPORTED, "sdpa: the token-major layout needs equal head dims that are a multiple of 4, at most 128, and 16-byte aligned tensors");
     // Large enough to pay for four copies: the MFMA kernels on padded copies of the operands.  When row statistics are

@@ -13,7 +13,10 @@
 // SIMD; K/V in double-buffered LDS tiles of 32 keys on a (W + 4)-float row stride (4 x 32 x (W + 4) floats: 98 or 130 KiB,
 // one workgroup per CU).  With 2 x W/2 MFMAs per key tile against the same softmax work as the narrower kernels the matrix
 // pipe stays busy nonetheless.  Mask kinds, tile skipping, the token-major layout and the work order are those of the
-// 64-wide kernel, the row statistics have the form every MFMA kernel leaves; there is no key split over workgroups.
+// 64-wide kernel, the row statistics have the form every MFMA kernel leaves.  Launches that leave CUs without a workgroup
+// are split over the keys across workgroups like the 128-wide kernel's: share y of n takes the key tiles y, y + n, ..., leaves
+// its weighted sums with their reference maximum and row sum in a scratch record, and sdpa_prefill_merge_wide adds the
+// shares up.
 #pragma once
 #include "sdpa_common.h"
 
@@ -29,19 +32,57 @@ template <int W> struct WideFwdTile {
     static constexpr int NP = BN * PPR / 256;     // pieces per thread and tile: thread tid moves the pieces tid, tid + 256, ...
 };
 
+constexpr int PARTW_STRIDE = 256 + 4;   // floats per partial row: up to 256 weighted sums, reference maximum, row sum, padding
+
+// Adds up the nsplit partial results of every query row (64 lanes per row, four columns each), normalises and stores; see
+// sdpa_prefill_merge_d128.
+__global__ __launch_bounds__(256) void sdpa_prefill_merge_wide(const float *__restrict__ part, float *__restrict__ out,
+                                                               float *__restrict__ stats, int nsplit, long long rows, int H, int Lq,
+                                                               int hd, int token_major) {
+    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int c = threadIdx.x & 63;
+    if (row >= rows) return;
+    float m_all = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) m_all = fmaxf(m_all, part[((long long)s * rows + row) * PARTW_STRIDE + 256]);
+    const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
+    float l_tot = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < nsplit; ++s) {
+        const float *p = part + ((long long)s * rows + row) * PARTW_STRIDE;
+        const float ms = p[256];
+        const float f = (ms == -INFINITY) ? 1.0f : fast_exp2(ms - m_ref);
+        l_tot += p[257] * f;
+        if (4 * c < hd) {
+            const f32x4 x = *reinterpret_cast<const f32x4 *>(p + 4 * c);
+            acc.x += x.x * f; acc.y += x.y * f; acc.z += x.z * f; acc.w += x.w * f;
+        }
+    }
+    const float inv = 1.0f / l_tot;
+    if (stats && c == 0) { stats[2 * row] = m_ref; stats[2 * row + 1] = inv; }
+    if (4 * c < hd) {
+        const long long bh = row / Lq, qi = row % Lq, b = bh / H, hh = bh % H;
+        const long long at = token_major ? (((b * Lq + qi) * H + hh) * hd) : (row * hd);
+        acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+        *reinterpret_cast<f32x4 *>(out + at + 4 * c) = acc;
+    }
+}
+
 template <int KIND, int W>
 __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__restrict__ q, const float *__restrict__ k,
                                                                  const float *__restrict__ v, float *__restrict__ out, int H,
                                                                  int Lq, int Lk, float rT, MaskArgs mask, int strict, int nqb,
                                                                  int total_blocks, int lpt, int token_major,
-                                                                 float *__restrict__ stats, int hd) {
+                                                                 float *__restrict__ stats, int hd, int nsplit,
+                                                                 float *__restrict__ part) {
     using WT = WideFwdTile<W>;
     constexpr int LS = WT::LS, TF = WT::TF, NC = WT::NC, NC2 = WT::NC2, NP = WT::NP, PPR = WT::PPR;
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;              // [2][BN][LS]
     float *Vs = lds + 2 * TF;     // [2][BN][LS]
     int bh, unit;
-    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    // key split with blocks of different length: odd shares walk the block order backwards (see sdpa_prefill_f32_d128)
+    const int blk = ((lpt & 1) && (blockIdx.y & 1)) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    if (!dl4s_work_order::work_item_at(blk, nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -70,6 +111,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
         if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
     }
     const int ntiles = (kend + BN - 1) / BN;
+    const int sp = blockIdx.y;       // this workgroup's share of the key tiles: sp, sp + nsplit, ...
 
     // Q fragment: Q[qi][(W/2)*half + s] * rT (one rounding, like the reference's q / temperature) * log2(e)
     float qr[W / 2];
@@ -121,10 +163,10 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
         for (int i = 0; i < 16; ++i) o[c][i] = 0.f;
     float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
 
-    if (ntiles > 0) {
-        load_pieces(krsrc, 0);
+    if (sp < ntiles) {
+        load_pieces(krsrc, sp);
         store_pieces(Ks);
-        load_pieces(vrsrc, 0);
+        load_pieces(vrsrc, sp);
         store_pieces(Vs);
     }
     __syncthreads();
@@ -136,10 +178,9 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
 
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        const bool more = (t + 1 < ntiles);
-        if (more) load_pieces(krsrc, t + 1);
+    for (int t = sp, buf = 0; t < ntiles; t += nsplit, buf ^= 1) {
+        const bool more = (t + nsplit < ntiles);
+        if (more) load_pieces(krsrc, t + nsplit);
         const int k0 = t * BN;
         int cls = 2;
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
@@ -175,7 +216,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
         }
         if (more) {
             store_pieces(Ks + (buf ^ 1) * TF);
-            load_pieces(vrsrc, t + 1);
+            load_pieces(vrsrc, t + nsplit);
         }
         if (visit) {
             const float *Vb = Vs + buf * TF;
@@ -209,6 +250,28 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
     // ---- normalise and store.  Register r of accumulator c < 4 is d = 4*(8(r/4) + 4*half + r%4) + c; of accumulator 4 + c,
     // d = 128 + NC2*(8(r/4) + 4*half + r%4) + c.
     const float l_tot = l_run + xor32(l_run);
+    if (part) {   // this share's weighted sums as they are, with their reference maximum and row sum
+        if (qi < Lq) {
+            float *pp = part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * PARTW_STRIDE;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = 8 * (r >> 2) + 4 * half + (r & 3);
+                const f32x4 a = {o[0][r], o[1][r], o[2][r], o[3][r]};
+                *reinterpret_cast<f32x4 *>(pp + 4 * i) = a;
+                if constexpr (NC2 == 4) {
+                    const f32x4 c4 = {o[4][r], o[5][r], o[6][r], o[7][r]};
+                    *reinterpret_cast<f32x4 *>(pp + 128 + 4 * i) = c4;
+                } else if constexpr (NC2 == 2) {
+                    const f32x2 c2 = {o[4][r], o[5][r]};
+                    *reinterpret_cast<f32x2 *>(pp + 128 + 2 * i) = c2;
+                } else {
+                    pp[128 + i] = o[4][r];
+                }
+            }
+            if (half == 0) { pp[256] = m_run; pp[257] = l_tot; }
+        }
+        return;
+    }
     const float inv = 1.0f / l_tot;
     if (stats && half == 0 && qi < Lq) {      // for the gradient call: a weight is 2^(s - m_use) * inv
         stats[2 * ((long long)bh * Lq + qi)] = m_use;
@@ -243,7 +306,7 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
 
 template <int KIND, int W>
 int launch_wide_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
-                     float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+                     float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit, float *part) {
     const int nqb = (Lq + BM - 1) / BM;
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
@@ -257,20 +320,26 @@ int launch_wide_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const fl
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
         dl4s::lds_limit_done(ctx, family, KIND);
     }
-    hipLaunchKernelGGL((sdpa_prefill_f32_wide<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), lds_bytes, ctx->stream, q, k, v,
-                       out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd);
-    return dl4s::launch_status("sdpa_prefill_f32_wide");
+    if (nsplit <= 1 || !part) { nsplit = 1; part = nullptr; }
+    hipLaunchKernelGGL((sdpa_prefill_f32_wide<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
+                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part);
+    const int st = dl4s::launch_status("sdpa_prefill_f32_wide");
+    if (st != DL4S_HIP_OK || nsplit == 1) return st;
+    const long long rows = (long long)B * H * Lq;
+    hipLaunchKernelGGL(sdpa_prefill_merge_wide, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, ctx->stream, part, out, stats, nsplit, rows,
+                       H, Lq, hd, token_major);
+    return dl4s::launch_status("sdpa_prefill_merge_wide");
 }
 
 template <int W>
 int launch_wide(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk, float rT,
-                const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
+                const MaskArgs &m, int strict, int token_major, float *stats, int hd, int nsplit = 1, float *part = nullptr) {
     switch (m.kind) {
-        case DL4S_MASK_NONE: return launch_wide_kind<DL4S_MASK_NONE, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        case DL4S_MASK_DENSE_F32: return launch_wide_kind<DL4S_MASK_DENSE_F32, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        case DL4S_MASK_CAUSAL: return launch_wide_kind<DL4S_MASK_CAUSAL, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        case DL4S_MASK_KEY_LENGTHS: return launch_wide_kind<DL4S_MASK_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
-        default: return launch_wide_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd);
+        case DL4S_MASK_NONE: return launch_wide_kind<DL4S_MASK_NONE, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_DENSE_F32: return launch_wide_kind<DL4S_MASK_DENSE_F32, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_CAUSAL: return launch_wide_kind<DL4S_MASK_CAUSAL, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        case DL4S_MASK_KEY_LENGTHS: return launch_wide_kind<DL4S_MASK_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
+        default: return launch_wide_kind<DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, W>(ctx, q, k, v, out, B, H, Lq, Lk, rT, m, strict, token_major, stats, hd, nsplit, part);
     }
 }
 
