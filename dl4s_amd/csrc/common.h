@@ -72,7 +72,12 @@ int layernorm_apply(dl4s_hip_ctx *ctx, const float *x, const float *scale, const
 // never the skinny form that a single product of the shape would take (so not the bits of the public entry for such shapes).
 int gemm_batched_tiled(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols, int64_t lhs_stride, const float *rhs,
                        int64_t rhs_rows, int64_t rhs_cols, int64_t rhs_stride, float *result, int64_t result_stride, int64_t batch,
-                       float alpha, float beta, int transpose_first, int transpose_second);
+                       float alpha, float beta, int transpose_first, int transpose_second, int triangle = 0);
+// (triangle: 0, or a product with a causal triangle - 1: only output tiles that reach column <= row are computed, the
+// rest of the result is left untouched; 2: lhs^T is zero before the diagonal, the contraction starts at the output tile's
+// first row; 3: lhs is zero beyond the diagonal, the contraction ends with the output tile's last row.  Tiles are at most
+// 128 wide and start at multiples of their width.  Operands the fast tiled kernels do not take - extents that are not
+// multiples of 4, operands off the 16-byte grid - fail with DL4S_HIP_EUNSUPPORTED before anything is launched.)
 // Looks up the device address of the decode kernels' fixed scratch block (sdpa_decode.hip) for the current GPU.
 int decode_static_scratch_init(dl4s_hip_ctx *ctx);
 

@@ -43,6 +43,11 @@ struct GemmArgs {
     // tile_n) * 2 ..], the layout ln_apply_f32 sums in a fixed order.
     float *ln_part;
     int ln_tiles_m;
+    // Products with a causal triangle (the tiled fast kernels, callers inside the library; rows and columns count from the
+    // same origin): 1 = only the output tiles that hold an element with column <= row are computed, the others are
+    // left untouched; 2 = the contraction index starts at the output tile's first row (everything before it is known to be
+    // zero in A); 3 = the contraction index ends with the output tile's last row (everything after it is zero in A).
+    int tri;
 };
 
 // x * (0.5 * tanh(0.5 * (1.702 * x)) + 0.5), every operation rounded, as Tensor/Operators/Unary.swift:184-186, :245-247
@@ -251,15 +256,41 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
     const int wave = tid >> 6, lane = tid & 63;
     const int half = lane >> 5, ln = lane & 31;
     const int wm = wave >> 1, wn = wave & 1;
-    const int tile_m = blockIdx.x / g.tiles_n, tile_n = blockIdx.x % g.tiles_n;
+    int tile_m = blockIdx.x / g.tiles_n, tile_n = blockIdx.x % g.tiles_n, zb = blockIdx.z;
+    if (g.tri == 1) {
+        // The grid holds only the tiles that reach the diagonal (column tile <= row tile; TM == TN), row after row: rows
+        // 0 .. t0 - 1 have 1, 2, .. t0 tiles (t0 = the smaller tile count), the rows after them all tiles_n.
+        const int tiles_m = (g.M + TM - 1) / TM, t0 = min(tiles_m, g.tiles_n), tri_count = t0 * (t0 + 1) / 2;
+        const int idx = blockIdx.x;
+        if (idx < tri_count) {
+            int m = (int)((__fsqrt_rn(8.0f * (float)idx + 1.0f) - 1.0f) * 0.5f);
+            while (m * (m + 1) / 2 > idx) --m;
+            while ((m + 1) * (m + 2) / 2 <= idx) ++m;
+            tile_m = m;
+            tile_n = idx - m * (m + 1) / 2;
+        } else {
+            tile_m = t0 + (idx - tri_count) / g.tiles_n;
+            tile_n = (idx - tri_count) % g.tiles_n;
+        }
+    } else if (g.tri >= 2) {
+        // The contraction length depends on the row tile.  Workgroups start in the order of their linear index (and go to
+        // the chip's eight dies by that index modulo 8): column tile fastest, then the batch, the row tiles slowest and
+        // from the longest contraction to the shortest - the dies get equal shares and the launch ends on its lightest work.
+        const long long lin = (long long)blockIdx.z * gridDim.x + blockIdx.x;
+        const int tiles_m = (g.M + TM - 1) / TM;
+        tile_n = (int)(lin % g.tiles_n);
+        zb = (int)((lin / g.tiles_n) % gridDim.z);
+        const int rank = (int)(lin / ((long long)g.tiles_n * gridDim.z));
+        tile_m = g.tri == 3 ? tiles_m - 1 - rank : rank;
+    }
     const int m0 = tile_m * TM, n0 = tile_n * TN;
-    const long long c_at = g.groups ? g.c_off[blockIdx.z] : (long long)blockIdx.z * g.c_bs;
+    const long long c_at = g.groups ? g.c_off[zb] : (long long)zb * g.c_bs;
     float *C = g.C + c_at;
 
     OpA opa;
     OpB opb;
-    opa.init(As, g.A + (g.groups ? g.a_off[blockIdx.z] : (long long)blockIdx.z * g.a_bs), g.M, g.lda, m0, g.K, tid);
-    opb.init(Bs, g.B + (g.groups ? g.b_off[blockIdx.z] : (long long)blockIdx.z * g.b_bs), g.N, g.ldb, n0, g.K, tid);
+    opa.init(As, g.A + (g.groups ? g.a_off[zb] : (long long)zb * g.a_bs), g.M, g.lda, m0, g.K, tid);
+    opb.init(Bs, g.B + (g.groups ? g.b_off[zb] : (long long)zb * g.b_bs), g.N, g.ldb, n0, g.K, tid);
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -269,9 +300,11 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int ktiles = (g.K + KT - 1) / KT;
-    opa.load(0);
-    opb.load(0);
+    const int ktiles_all = (g.K + KT - 1) / KT;
+    const int kt_first = g.tri == 2 ? min(m0 / KT, ktiles_all) : 0;      // (a tile past the end reads as zeros)
+    const int ktiles = g.tri == 3 ? min(ktiles_all, (m0 + TM + KT - 1) / KT) : ktiles_all;
+    opa.load(kt_first);
+    opb.load(kt_first);
     opa.store(0, tid);
     opb.store(0, tid);
     __syncthreads();
@@ -311,7 +344,7 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
         if (more) { opa.store(buf ^ 1, tid); opb.store(buf ^ 1, tid); }
         __syncthreads();
     };
-    for (int kt = 0; kt < ktiles; kt += 2) {
+    for (int kt = kt_first; kt < ktiles; kt += 2) {
         k_step(kt, std::integral_constant<int, 0>{});
         if (kt + 1 < ktiles) k_step(kt + 1, std::integral_constant<int, 1>{});
     }
@@ -612,7 +645,7 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
                 int64_t rc, int64_t rbs, float *result, int64_t cbs, int64_t batch, float alpha, float beta, int ta, int tb,
                 const float *bias = nullptr, const float *residual = nullptr, int act = 0, const float *const *group_lhs = nullptr,
                 const float *const *group_rhs = nullptr, float *const *group_result = nullptr, float *ln_part = nullptr,
-                int64_t ln_item_rows = 0, int *ln_nblk = nullptr, bool tiled_only = false) {
+                int64_t ln_item_rows = 0, int *ln_nblk = nullptr, bool tiled_only = false, int tri = 0) {
     // group_*: `batch` (at most 4) products of one shape with unrelated operand addresses, in one launch
     // ln_part: also leave LayerNorm partial sums over items of ln_item_rows rows (see GemmArgs); *ln_nblk receives the
     // number of pairs per item.  A product that does not run on the tiled kernels with whole tiles per item, or would
@@ -669,6 +702,9 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
                         (tb ? rows_by_k_any(rc) : true) && aligned16(lhs) && (!tb || aligned16(rhs)) && lbs % 4 == 0 &&
                         (!tb || rbs % 4 == 0) && group_aligned && M * N * batch < (1ll << 31) && K * (tb ? 1 : rc) < (1ll << 31);
     if (ln_part && (skinny || !fast)) return GEMM_LN_NOT_FUSED;
+    // (callers check their operands first; nothing has been launched when this fails)
+    DL4S_REQUIRE(!tri || (fast && !skinny), DL4S_HIP_EUNSUPPORTED, "gemm: a triangular product on operands the tiled fast kernels do not take");
+    g.tri = tri;
     if (skinny) {
         // 16 x 16 output blocks (gemm_f32_skinny16) for up to 16 rows, and beyond for an unsliced K while that grid stays
         // within two workgroups per CU ([32,512].[512,512] 5.7 -> 3.7 us, [128,512].[512,512] 5.8 -> 4.0 us,
@@ -725,7 +761,9 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
         *ln_nblk = (int)((ln_item_rows / TM) * tn);
     }
     DL4S_REQUIRE(tm * tn < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "gemm: too many tiles");
-    const dim3 grid((unsigned)(tm * tn), 1, (unsigned)batch);
+    // (tri == 1: only the tiles that reach the diagonal, see the kernel)
+    const long long t0 = std::min(tm, tn);
+    const dim3 grid((unsigned)(tri == 1 ? t0 * (t0 + 1) / 2 + (tm - t0) * tn : tm * tn), 1, (unsigned)batch);
     // 128 x 128 tiles on a launch of at most two workgroups per CU: K tiles of 32 (half the barriers; contracted as two
     // halves of 16, so the bits do not depend on the depth)
     const bool deep = fast && !small && tm * tn * batch <= 2ll * ctx->cu_count;
@@ -774,9 +812,10 @@ namespace dl4s {
 
 int gemm_batched_tiled(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, int64_t lhs_cols, int64_t lhs_stride, const float *rhs,
                        int64_t rhs_rows, int64_t rhs_cols, int64_t rhs_stride, float *result, int64_t result_stride, int64_t batch,
-                       float alpha, float beta, int transpose_first, int transpose_second) {
+                       float alpha, float beta, int transpose_first, int transpose_second, int triangle) {
     return gemm_launch(ctx, lhs, lhs_rows, lhs_cols, lhs_stride, rhs, rhs_rows, rhs_cols, rhs_stride, result, result_stride, batch, alpha,
-                       beta, transpose_first, transpose_second, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0, nullptr, true);
+                       beta, transpose_first, transpose_second, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0, nullptr, true,
+                       triangle);
 }
 
 }  // namespace dl4s
