@@ -545,9 +545,12 @@ int launch_d64(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
         dl4s::lds_limit_done(ctx, dl4s::LDS_PREFILL, KIND);
     }
-    // a launch that fits the chip at once (three workgroups per CU): every second round of the CUs reversed as well
-    // (B2 H16 L2048 causal: 203 -> 161 us, B4 H16 L1024: 106 -> 88 us)
-    const int lpt_arg = lpt | ((lpt && total <= 3ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
+    // a launch that fits the chip at once (four workgroups per CU), or nearly: little or nothing is left for the
+    // dispatcher to balance, so every second round of the CUs is reversed as well (B2 H16 L2048 causal: 203 -> 161 us,
+    // B4 H16 L1024: 106 -> 88 us; with exactly four per CU B4 H16 L2048 319 -> 277 us, B1 H16 L8192 1251 -> 1038 us,
+    // B8 H16 L1024 165 -> 151 us; five per CU B5 H16 L2048 379 -> 362 us; from six per CU on it loses: B8 H16 L2048
+    // 540 -> 555 us, B2 H16 L8192 2.03 -> 2.13 ms)
+    const int lpt_arg = lpt | ((lpt && total <= 5ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
     hipLaunchKernelGGL(sdpa_prefill_f32_d64<KIND>, dim3(chunk * 8), dim3(256), lds_bytes, ctx->stream, q, k, v, out, H,
                        Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_d64");

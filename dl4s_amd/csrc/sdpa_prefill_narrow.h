@@ -515,7 +515,7 @@ int launch_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int lpt = (uneven && nqb >= 2) ? 1 : 0;
-    const int lpt_arg = lpt | ((lpt && total <= 3ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
+    const int lpt_arg = lpt | ((lpt && total <= 4ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
     hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_narrow");
@@ -533,7 +533,7 @@ int launch_narrow48_main(dl4s_hip_ctx *ctx, const float *q, const float *k, cons
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int lpt = (uneven && nqb >= 2) ? 1 : 0;
-    const int lpt_arg = lpt | ((lpt && total <= 3ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
+    const int lpt_arg = lpt | ((lpt && total <= 4ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
     hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, 48>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_narrow");
