@@ -304,8 +304,8 @@ def other_configs(ctx, lib, cpu, only=None):
                 "note": ("algorithmic flops = the 5 products, which is what the two deterministic kernels issue: the dK/dV kernel "
                          "stores its dS tiles (2 GiB scratch from the pool at this shape) and the dQ kernel contracts them with K")
                         if d <= 128 else
-                        "head dims above 128: the five products as batched GEMMs around one elementwise pass, query blocks of "
-                        "512 rows under the causal mask; TFLOP/s on the algorithmic flops"}
+                        "head dims above 128: the five products as batched GEMMs around one elementwise pass, the tiles "
+                        "beyond the diagonal left out under the causal mask; TFLOP/s on the algorithmic flops"}
             if cpu and d == 64:
                 from oracle import binding as orc
                 hq, hk, hv, hg = (b_.numpy()[:1, :2] for b_ in bufs)
