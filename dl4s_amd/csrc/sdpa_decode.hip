@@ -52,6 +52,12 @@ __device__ __forceinline__ float row_sum(float x) {
     return x;
 }
 
+// Keys per lane and loop iteration of the decode kernel for rows read in `seg` pieces: as many as keep the two batches of
+// loads (K, then V) of an iteration in registers at 128 per lane, the budget of 16 wavefronts per CU.  Three- and five-piece
+// rows had 4 and 2 and spilled 18 and 15 registers inside the loop: with 3 and 1, B16 H16 T4096 went from 136 to 117 us at
+// head dim 96 (5.9 -> 6.9 TB/s), 256 -> 232 us at 192, 145 -> 120 us at 80 and 217 -> 196 us at 160.
+__host__ __device__ constexpr int keys_per_lane(int seg) { return seg == 1 ? 8 : seg == 2 ? 4 : seg == 3 ? 3 : 1; }
+
 // LPR lanes read one cache row of up to 4 * LPR floats with one 128-bit load per lane (lanes at or beyond d / 4 hold
 // zeros), so a load instruction of a wavefront covers G = 64 / LPR whole rows; a wavefront iteration covers KB = 8 * G
 // keys with 8 K loads and 8 V loads per lane in flight (16 KiB per wavefront whatever the row width).
@@ -66,10 +72,10 @@ __device__ __forceinline__ float row_sum(float x) {
 // score - 1e9 (NN/Models/Transformer/ScaledDotProductAttention.swift:55-57 with the mask of makeEncoderMasks).  With at
 // least one key left their weights are exactly zero and they are not visited at all; a length of zero or less blocks every
 // key, the penalty is applied to all of them and the row comes out uniform, as in the reference.
-// SEG: the row is read as SEG consecutive segments of 4 * LPR floats by the same LPR lanes (SEG loads per row and lane, NK =
-// 4 keys per lane and iteration instead of 8).  SEG = 3 with LPR = 8 (16) serves rows of 96 (192) floats with every lane busy,
-// where the one-piece form would leave a quarter of the lanes idle; SEG = 5 with LPR = 4 (8) rows of 80 (160) floats, 2 keys per
-// lane and iteration; SEG = 2 with LPR = 32 serves rows of 129 to 256 floats.
+// SEG: the row is read as SEG consecutive segments of 4 * LPR floats by the same LPR lanes (SEG loads per row and lane, fewer
+// keys per lane and iteration, see keys_per_lane).  SEG = 3 with LPR = 8 (16) serves rows of 96 (192) floats with every lane
+// busy, where the one-piece form would leave a quarter of the lanes idle; SEG = 5 with LPR = 4 (8) rows of 80 (160) floats;
+// SEG = 2 with LPR = 32 serves rows of 129 to 256 floats.
 template <bool APPEND, int NW, int LPR, bool FULL, bool DEVPOS = false, int SEG = 1>
 __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *__restrict__ q, float *kcache,
                                                                    float *vcache, const float *__restrict__ k_new,
@@ -78,7 +84,7 @@ __global__ __launch_bounds__(NW * 64) void sdpa_decode_splitk_f32(const float *_
                                                                    int pos, float rT, int nsplit, int chunk, int d, int H,
                                                                    const int *__restrict__ lengths,
                                                                    const int *__restrict__ pos_dev = nullptr, int vec = 4) {
-    constexpr int SW = 4 * LPR, D = SW * SEG, G = 64 / LPR, NK = SEG == 1 ? 8 : (SEG <= 3 ? 4 : 2), KB = NK * G, PSTR = pstr(D);
+    constexpr int SW = 4 * LPR, D = SW * SEG, G = 64 / LPR, NK = keys_per_lane(SEG), KB = NK * G, PSTR = pstr(D);
     __shared__ float sm_o[NW][D];
     __shared__ float sm_m[NW], sm_l[NW];
     if (DEVPOS) {
@@ -336,10 +342,7 @@ inline int lanes_per_row(int64_t d, int vec) {
     return seg == 3 ? (int)d / 12 : (seg == 5 ? (int)d / 20 : (d <= 32 ? 8 : (d <= 64 ? 16 : 32)));
 }
 inline int row_width(int64_t d, int vec) { return 4 * lanes_per_row(d, vec) * row_segments(d, vec); }
-inline int keys_per_iteration(int64_t d, int vec) {
-    const int seg = row_segments(d, vec);
-    return (seg == 1 ? 8 : (seg <= 3 ? 4 : 2)) * (64 / lanes_per_row(d, vec));
-}
+inline int keys_per_iteration(int64_t d, int vec) { return keys_per_lane(row_segments(d, vec)) * (64 / lanes_per_row(d, vec)); }
 
 // 4 when every cache row starts on a 16-byte boundary (the row length a multiple of 4 floats, every operand aligned): a lane
 // reads its piece of a row with one 128-bit load.  2 for an even row length and 8-byte aligned operands (two 64-bit loads),
