@@ -1033,13 +1033,15 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
             dl4s_hip_alloc(ctx, (size_t)((long long)B * H * slab), &dsv) == DL4S_HIP_OK) {
             float *ds = static_cast<float *>(dsv);
             int lpt = (uneven && nkb >= 2) ? 1 : 0;
-            if (lpt && total_k <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+            // (reversed rounds as well up to five workgroups per CU, two and a half times what is resident at once: B4 H16 L2048
+            // 792 -> 764 us, B8 H16 L1024 438 -> 415 us, B1 H16 L8192 3.00 -> 2.85 ms; at eight per CU it loses 1.5 %)
+            if (lpt && total_k <= 5ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
             hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d64<KIND, true>), dim3((unsigned)((total_k + 7) / 8 * 8)), dim3(256), lds_dkv, ctx->stream, q,
                                k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total_k, lpt, token_major, hd, ds);
             int rc = dl4s::launch_status("sdpa_bwd_dkv_f32_d64");
             if (rc == DL4S_HIP_OK) {
                 lpt = (uneven && nqb >= 2) ? 1 : 0;
-                if (lpt && total_q <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+                if (lpt && total_q <= 5ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
                 hipLaunchKernelGGL(sdpa_bwd_dq_from_ds_f32_d64<KIND>, dim3((unsigned)((total_q + 7) / 8 * 8)), dim3(256),
                                    2 * TILE_FLOATS * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q,
                                    lpt, token_major, hd);

@@ -397,7 +397,7 @@ int launch_bwd_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const f
     if (dl4s_hip_alloc(ctx, (size_t)((long long)B * H * slab), &dsv) != DL4S_HIP_OK) return 0;
     float *ds = static_cast<float *>(dsv);
     int lpt = (uneven && nkb >= 2) ? 1 : 0;
-    if (lpt && total_k <= 3ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+    if (lpt && total_k <= 5ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
     // 32 floats of LDS beyond the tiles: at W = 16 the lanes that stand for rows d >= 16 read past the last tile
     hipLaunchKernelGGL((sdpa_bwd_dkv_f32_narrow<KIND, W>), dim3((unsigned)((total_k + 7) / 8 * 8)), dim3(256),
                        (size_t)(4 * TF + 192 + 32) * sizeof(float), ctx->stream, q, k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb,
@@ -405,7 +405,7 @@ int launch_bwd_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const f
     int rc = dl4s::launch_status("sdpa_bwd_dkv_f32_narrow");
     if (rc == DL4S_HIP_OK) {
         lpt = (uneven && nqb >= 2) ? 1 : 0;
-        if (lpt && total_q <= 4ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+        if (lpt && total_q <= 7ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
         hipLaunchKernelGGL((sdpa_bwd_dq_from_ds_f32_narrow<KIND, W>), dim3((unsigned)((total_q + 7) / 8 * 8)), dim3(256),
                            (size_t)(2 * TF + 32) * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q, lpt,
                            token_major, hd);

@@ -515,7 +515,10 @@ int launch_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int lpt = (uneven && nqb >= 2) ? 1 : 0;
-    const int lpt_arg = lpt | ((lpt && total <= 4ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
+    // every second round of the CUs reversed as well, on launches of any size: these short workgroups (16 or 32 columns)
+    // gain from it well beyond the four per CU that are resident at once (B5 H16 L2048 d32 causal 216 -> 191 us, B6
+    // 248 -> 222 us, B8 299 -> 295 us; d16 133 -> 119, 154 -> 138, 188 -> 180 us), where the 64-wide kernel starts to lose
+    const int lpt_arg = lpt | (lpt ? (ctx->cu_count / 8) << 1 : 0);
     hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_narrow");
@@ -533,7 +536,8 @@ int launch_narrow48_main(dl4s_hip_ctx *ctx, const float *q, const float *k, cons
     const long long total = (long long)nqb * B * H;
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     const int lpt = (uneven && nqb >= 2) ? 1 : 0;
-    const int lpt_arg = lpt | ((lpt && total <= 4ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
+    // (reversed rounds up to five workgroups per CU, like the 64-wide kernel: B5 H16 L2048 d48 296 -> 289 us, beyond it loses)
+    const int lpt_arg = lpt | ((lpt && total <= 5ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
     hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, 48>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_narrow");

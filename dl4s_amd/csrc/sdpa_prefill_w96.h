@@ -293,7 +293,7 @@ int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const flo
     DL4S_REQUIRE(total < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total);
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     int lpt = ((causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict && nqb >= 2) ? 1 : 0;
-    if (lpt && total <= 3ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
+    if (lpt && total <= 5ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
     const size_t lds_bytes = 4 * TILE96_FLOATS * sizeof(float);   // 50 KiB: within the default limit
     if (nsplit <= 1 || !part || VEC != 4) { nsplit = 1; part = nullptr; }
     hipLaunchKernelGGL((sdpa_prefill_f32_w96<KIND, VEC, W>), dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
