@@ -31,8 +31,11 @@ constexpr int TILE96_FLOATS = BN * LSTR96;
 // accumulators on v_mfma_f32_16x16x4_f32 (queries 0-15 and 16-31 of the wavefront; lane: column = lane % 16, rows
 // d = 64 + 4 * (lane / 16) + i), fed through v_permlane16_swap like attend_tile_16 (sdpa_prefill_narrow.h): 80 MFMA units
 // per tile instead of 96.
+// Three workgroups per CU with 128-bit staging (168 registers; the kinds that need a few more spill 4 to 21 outside the MFMA
+// chains and still gain: B8 H16 L2048 d96 causal 846 -> 827 us, key lengths 1109 -> 1081 us, dense causal 922 -> 891 us), two
+// with 64-bit staging, whose address arithmetic does not fit (d90 causal 880 us against 905 us at three).
 template <int KIND, int VEC, int W = 96>
-__global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_w96(const float *__restrict__ q, const float *__restrict__ k,
+__global__ __launch_bounds__(256, VEC == 4 ? 3 : 2) void sdpa_prefill_f32_w96(const float *__restrict__ q, const float *__restrict__ k,
                                                                 const float *__restrict__ v, float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict, int nqb, int total_blocks,
                                                                 int lpt, int token_major, float *__restrict__ stats, int hd,
