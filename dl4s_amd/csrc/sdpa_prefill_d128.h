@@ -57,15 +57,18 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__r
                                                                  int Lq, int Lk, float rT, MaskArgs mask, int strict, int nqb,
                                                                  int total_blocks, int lpt, int token_major,
                                                                  float *__restrict__ stats, int hd, int nsplit,
-                                                                 float *__restrict__ part) {
+                                                                 float *__restrict__ part, int shares_adjacent) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                      // [2][BN][LSTR2]
     float *Vs = lds + 2 * TILE2_FLOATS;   // [2][BN][LSTR2]
     int bh, unit;
-    // Key split with blocks of different length: the workgroups of an odd share walk the block order backwards, so that the
-    // CU that got the longest block's first share gets the shortest block's second (the dispatcher deals both rounds out
-    // in the same order).
-    const int blk = ((lpt & 1) && (blockIdx.y & 1)) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    // Key split with blocks of different length.  A launch that is resident at once: the workgroups of an odd share walk the
+    // block order backwards, so that the CU that got the longest block's first share gets the shortest block's second (the
+    // dispatcher deals both rounds out in the same order).  A larger launch: the shares of a block next to each other in the
+    // longest-first order, so that the dispatcher hands the short blocks to whichever CU is free first.
+    int blk = ((lpt & 1) && (blockIdx.y & 1) && !shares_adjacent) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    int sp = blockIdx.y;
+    if ((lpt & 1) && shares_adjacent) dl4s_work_order::split_item_at(blockIdx.x, blockIdx.y, gridDim.x, nsplit, blk, sp);
     if (!dl4s_work_order::work_item_at(blk, nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x;
@@ -146,7 +149,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_f32_d128(const float *__r
 
     // Key split over workgroups (small launches): workgroup blockIdx.y of nsplit takes the key tiles y, y + nsplit, ... -
     // an assignment that does not depend on how many tiles the mask lets the block skip, so skipping keeps the bits.
-    const int sp = blockIdx.y;
     if (sp < ntiles) { load_tile(sp); store_tile(0); }
     __syncthreads();
 
@@ -254,7 +256,10 @@ int launch_d128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *
     }
     if (nsplit <= 1 || !part) { nsplit = 1; part = nullptr; }
     hipLaunchKernelGGL(sdpa_prefill_f32_d128<KIND>, dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
-                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part);
+                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part,
+                       // (two workgroups per CU are resident: B1 H24 L2048 d128 causal 348 -> 274 us; B1 H16 L2048, which fits, 166 us
+                       // against 205 us with the shares adjacent)
+                       ((total + 7) / 8 * 8 * nsplit > 2ll * ctx->cu_count) ? 1 : 0);
     int st = dl4s::launch_status("sdpa_prefill_f32_d128");
     if (st != DL4S_HIP_OK || nsplit == 1) return st;
     const long long rows = (long long)B * H * Lq;

@@ -39,13 +39,15 @@ __global__ __launch_bounds__(256, VEC == 4 ? 3 : 2) void sdpa_prefill_f32_w96(co
                                                                 const float *__restrict__ v, float *__restrict__ out, int H, int Lq,
                                                                 int Lk, float rT, MaskArgs mask, int strict, int nqb, int total_blocks,
                                                                 int lpt, int token_major, float *__restrict__ stats, int hd,
-                                                                int nsplit, float *__restrict__ part) {
+                                                                int nsplit, float *__restrict__ part, int shares_adjacent) {
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                       // [2][BN][LSTR96]
     float *Vs = lds + 2 * TILE96_FLOATS;   // [2][BN][LSTR96]
     int bh, unit;
-    // key split with blocks of different length: odd shares walk the block order backwards (see sdpa_prefill_f32_d128)
-    const int blk = ((lpt & 1) && (blockIdx.y & 1)) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    // key split with blocks of different length: see sdpa_prefill_f32_d128
+    int blk = ((lpt & 1) && (blockIdx.y & 1) && !shares_adjacent) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    int sp = blockIdx.y;     // this workgroup's share of the key tiles: sp, sp + nsplit, ...
+    if ((lpt & 1) && shares_adjacent) dl4s_work_order::split_item_at(blockIdx.x, blockIdx.y, gridDim.x, nsplit, blk, sp);
     if (!dl4s_work_order::work_item_at(blk, nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x;
@@ -146,7 +148,6 @@ __global__ __launch_bounds__(256, VEC == 4 ? 3 : 2) void sdpa_prefill_f32_w96(co
     f32x4 og[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};   // W = 80: the columns 64 .. 79
     float m_run = -INFINITY, m_use = 0.f, l_run = 0.f;
 
-    const int sp = blockIdx.y;     // this workgroup's share of the key tiles: sp, sp + nsplit, ...
     if (sp < ntiles) { load_tile(sp); store_tile(0); }
     __syncthreads();
 
@@ -300,7 +301,8 @@ int launch_w96_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const flo
     const size_t lds_bytes = 4 * TILE96_FLOATS * sizeof(float);   // 50 KiB: within the default limit
     if (nsplit <= 1 || !part || VEC != 4) { nsplit = 1; part = nullptr; }
     hipLaunchKernelGGL((sdpa_prefill_f32_w96<KIND, VEC, W>), dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
-                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part);
+                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part,
+                       ((total + 7) / 8 * 8 * nsplit > (VEC == 4 ? 3ll : 2ll) * ctx->cu_count) ? 1 : 0);   // (beyond what is resident at once)
     const int st = dl4s::launch_status("sdpa_prefill_f32_w96");
     if (st != DL4S_HIP_OK || nsplit == 1) return st;
     const long long rows = (long long)B * H * Lq;

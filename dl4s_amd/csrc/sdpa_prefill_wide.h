@@ -73,15 +73,17 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
                                                                  int Lq, int Lk, float rT, MaskArgs mask, int strict, int nqb,
                                                                  int total_blocks, int lpt, int token_major,
                                                                  float *__restrict__ stats, int hd, int nsplit,
-                                                                 float *__restrict__ part) {
+                                                                 float *__restrict__ part, int shares_adjacent) {
     using WT = WideFwdTile<W>;
     constexpr int LS = WT::LS, TF = WT::TF, NC = WT::NC, NC2 = WT::NC2, NP = WT::NP, PPR = WT::PPR;
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;              // [2][BN][LS]
     float *Vs = lds + 2 * TF;     // [2][BN][LS]
     int bh, unit;
-    // key split with blocks of different length: odd shares walk the block order backwards (see sdpa_prefill_f32_d128)
-    const int blk = ((lpt & 1) && (blockIdx.y & 1)) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    // key split with blocks of different length: see sdpa_prefill_f32_d128
+    int blk = ((lpt & 1) && (blockIdx.y & 1) && !shares_adjacent) ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+    int sp = blockIdx.y;       // this workgroup's share of the key tiles: sp, sp + nsplit, ...
+    if ((lpt & 1) && shares_adjacent) dl4s_work_order::split_item_at(blockIdx.x, blockIdx.y, gridDim.x, nsplit, blk, sp);
     if (!dl4s_work_order::work_item_at(blk, nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x;
@@ -111,7 +113,6 @@ __global__ __launch_bounds__(256, 1) void sdpa_prefill_f32_wide(const float *__r
         if (DENSE && mask.cls) dense_key_bounds(mask, b, hh, qb * BM, wave, Lq, Lk, kend, wkend, skip_ones);
     }
     const int ntiles = (kend + BN - 1) / BN;
-    const int sp = blockIdx.y;       // this workgroup's share of the key tiles: sp, sp + nsplit, ...
 
     // Q fragment: Q[qi][(W/2)*half + s] * rT (one rounding, like the reference's q / temperature) * log2(e)
     float qr[W / 2];
@@ -322,7 +323,9 @@ int launch_wide_kind(dl4s_hip_ctx *ctx, const float *q, const float *k, const fl
     }
     if (nsplit <= 1 || !part) { nsplit = 1; part = nullptr; }
     hipLaunchKernelGGL((sdpa_prefill_f32_wide<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8), (unsigned)nsplit), dim3(256), lds_bytes,
-                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part);
+                       ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt, token_major, stats, hd, nsplit, part,
+                       // (one workgroup per CU is resident: B1 H16 L2048 d256 causal 514 -> 353 us, B1 H8 L4096 967 -> 644 us)
+                       ((total + 7) / 8 * 8 * nsplit > (long long)ctx->cu_count) ? 1 : 0);
     const int st = dl4s::launch_status("sdpa_prefill_f32_wide");
     if (st != DL4S_HIP_OK || nsplit == 1) return st;
     const long long rows = (long long)B * H * Lq;

@@ -87,4 +87,16 @@ DL4S_WORK_ORDER_FN bool work_item_at(const int block, const int nunits, const in
     return true;
 }
 
+// A launch whose items are each cut into `nsplit` shares: grid x = the items (padded to a multiple of 8), grid y = the shares.
+// Workgroups start in the order of bx + gx * by and go to XCD (bx + gx * by) % 8 = bx % 8.  Returns the item index `blk` (to be
+// passed to work_item_at) and the share `sp` such that an XCD's sequence runs over its items in their order with the shares of
+// an item next to each other - with the longest-first order every share of a long item starts before any share of a
+// shorter one, which a share-major walk (all first shares, then all second shares) does not give.
+DL4S_WORK_ORDER_FN void split_item_at(const int bx, const int by, const int gx, const int nsplit, int &blk, int &sp) {
+    const long long lin = (long long)by * gx + bx;
+    const long long wl = lin >> 3;
+    sp = (int)(wl % nsplit);
+    blk = (int)(wl / nsplit) * 8 + (int)(lin & 7);
+}
+
 }  // namespace dl4s_work_order

@@ -91,3 +91,23 @@ def test_round_reversal_pairs_long_with_short(shim):
         local = {block // 8: u for block, _, u in got if block % 8 == x}
         sums = {local[c] + local[32 + c] for c in range(32)}
         assert sums == {nunits - 1}
+
+
+@pytest.mark.parametrize("nsplit", [1, 2, 3, 5, 8])
+def test_adjacent_shares_hand_out_every_item_and_share_once(shim, nsplit):
+    """split_item_at: over the grid (x = items padded to a multiple of 8, y = shares) every (item, share) exactly once, an item
+    on the XCD of its index, and in an XCD's dispatch sequence the shares of an item next to each other, items ascending."""
+    shim.split_item_at.argtypes = [C.c_int] * 4 + [C.POINTER(C.c_int)] * 2
+    shim.split_item_at.restype = None
+    blk, sp = C.c_int(), C.c_int()
+    for gx in (8, 16, 64, 256, 520):
+        got = []
+        for by in range(nsplit):
+            for bx in range(gx):
+                shim.split_item_at(bx, by, gx, nsplit, C.byref(blk), C.byref(sp))
+                got.append((by * gx + bx, blk.value, sp.value))
+        assert sorted((b, s) for _, b, s in got) == [(b, s) for b in range(gx) for s in range(nsplit)], gx
+        assert all(lin % 8 == b % 8 for lin, b, _ in got)
+        for x in range(8):
+            seq = [(b, s) for lin, b, s in got if lin % 8 == x]      # dispatch order on that XCD
+            assert seq == sorted(seq), (gx, x)
