@@ -288,14 +288,18 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
                                                                  int Lk, float rT, MaskArgs mask, int strict, int nkb,
                                                                  int total_blocks, int lpt, int token_major, int hd,
                                                                  float *__restrict__ ds = nullptr, int nsplit = 1,
-                                                                 float *__restrict__ part = nullptr) {
+                                                                 float *__restrict__ part = nullptr, int shares_adjacent = 0) {
     using WT = WideTile<W>;
     extern __shared__ __align__(16) float lds[];
     float *Qs = lds;                        // [2][BN][WT::LS]  q * rT * log2(e)
     float *Gs = lds + 2 * WT::TF;     // [2][BN][WT::LS]  dout
     float *Ss = lds + 4 * WT::TF;     // per query tile: [2][32] reference maxima, [2][32] 1 / row sums, [2][32] D
     int bh, unit;
-    if (!work_item(nkb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    // (the shares of a split launch beyond what is resident at once: next to each other in the longest-first order, see
+    // sdpa_prefill_f32_d128)
+    int blk = blockIdx.x, sp = blockIdx.y;
+    if ((lpt & 1) && shares_adjacent) dl4s_work_order::split_item_at(blockIdx.x, blockIdx.y, gridDim.x, nsplit, blk, sp);
+    if (!dl4s_work_order::work_item_at(blk, nkb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
 
@@ -387,7 +391,6 @@ __global__ __launch_bounds__(256, 1) void sdpa_bwd_dkv_f32_d128(const float *__r
     WT::zero(ka);
     WT::zero(va);
 
-    const int sp = blockIdx.y;
     int t = t_begin + (((sp - t_begin) % nsplit) + nsplit) % nsplit;   // the share's first tile at or after t_begin
     if (t < nqt) { load_tile(t); store_tile(0); }
     __syncthreads();
@@ -515,14 +518,16 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
                                                                         float *__restrict__ dq, int H, int Lq, int Lk, float rT,
                                                                         MaskArgs mask, int strict, int nqb, int total_blocks, int lpt,
                                                                         int token_major, int hd, int nsplit = 1,
-                                                                        float *__restrict__ part = nullptr) {
+                                                                        float *__restrict__ part = nullptr, int shares_adjacent = 0) {
     // nsplit > 1: workgroup blockIdx.y takes the key tiles y, y + nsplit, ... and leaves its unscaled sums in
     // part [share][batch*head*Lq][128] for sdpa_bwd_merge_d128
     using WT = WideTile<W>;
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;                      // [2][BN][WT::LS]
     int bh, unit;
-    if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
+    int blk = blockIdx.x, sp = blockIdx.y;
+    if ((lpt & 1) && shares_adjacent) dl4s_work_order::split_item_at(blockIdx.x, blockIdx.y, gridDim.x, nsplit, blk, sp);
+    if (!dl4s_work_order::work_item_at(blk, nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
     const int b = bh / H, hh = bh % H;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
 
@@ -595,7 +600,6 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
 #pragma unroll
     for (int i = 0; i < 16; ++i) dsn[i] = 0.f;
 
-    const int sp = blockIdx.y;
     if (sp < ntiles) {
         load_tile(sp);
         store_tile(0);
@@ -670,7 +674,7 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
             if (lpt && total_k <= (long long)ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
             hipLaunchKernelGGL((sdpa_bwd_dkv_f32_d128<KIND, true, W>), dim3((unsigned)((total_k + 7) / 8 * 8), (unsigned)sk), dim3(256), lds_dkv,
                                ctx->stream, q, k, v, dout, stats, D, dk, dv, H, Lq, Lk, rT, m, strict, nkb, (int)total_k, lpt, token_major, hd,
-                               ds, (int)sk, pk);
+                               ds, (int)sk, pk, ((total_k + 7) / 8 * 8 * sk > (long long)ctx->cu_count) ? 1 : 0);   // (B1 H12 L2048 causal 444 -> 414 us, B1 H8 L4096 913 -> 881 us)
             int rc = dl4s::launch_status("sdpa_bwd_dkv_f32_d128");
             if (rc == DL4S_HIP_OK && pk) {
                 const dim3 mg((unsigned)((krows + 7) / 8));
@@ -685,7 +689,7 @@ int launch_bwd128(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
                 if (lpt && total_q <= 2ll * ctx->cu_count) lpt |= (ctx->cu_count / 8) << 1;
                 hipLaunchKernelGGL((sdpa_bwd_dq_from_ds_f32_d128<KIND, W>), dim3((unsigned)((total_q + 7) / 8 * 8), (unsigned)sq), dim3(256),
                                    2 * WT::TF * sizeof(float), ctx->stream, k, ds, dq, H, Lq, Lk, rT, m, strict, nqb, (int)total_q,
-                                   lpt, token_major, hd, (int)sq, pq);
+                                   lpt, token_major, hd, (int)sq, pq, ((total_q + 7) / 8 * 8 * sq > 2ll * ctx->cu_count) ? 1 : 0);
                 rc = dl4s::launch_status("sdpa_bwd_dq_from_ds_f32_d128");
                 if (rc == DL4S_HIP_OK && pq) {
                     hipLaunchKernelGGL(sdpa_bwd_merge_d128, dim3((unsigned)((qrows + 7) / 8)), dim3(256), 0, ctx->stream, pq, dq, (int)sq,
