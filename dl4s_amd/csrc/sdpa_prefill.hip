@@ -650,8 +650,8 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     if ((mfma128_path || (w96_path && dk % 4 == 0)) && !no_split) {
         const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
         // enough shares to give every CU its workgroup; two where every CU just has one (blocks of different length then pair up
-        // long with short, the odd shares walking the block order backwards: B2 H8 L2048 d256 causal 570 -> 510 us; without a
-        // mask 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
+        // long with short through the order of their workgroups: B2 H8 L2048 d256 causal 570 -> 353 us; without a mask
+        // 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
         if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
             long long want = std::max(2ll, ((long long)ctx->cu_count + blocks - 1) / blocks);
             want = std::min(want, std::min(8ll, nkt / 2));
@@ -663,8 +663,8 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     if (wide_path && !no_split) {
         const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
         // enough shares to give every CU its workgroup; two where every CU just has one (blocks of different length then pair up
-        // long with short, the odd shares walking the block order backwards: B2 H8 L2048 d256 causal 570 -> 510 us; without a
-        // mask 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
+        // long with short through the order of their workgroups: B2 H8 L2048 d256 causal 570 -> 353 us; without a mask
+        // 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
         if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
             long long want = std::max(2ll, ((long long)ctx->cu_count + blocks - 1) / blocks);
             want = std::min(want, std::min(8ll, nkt / 2));
