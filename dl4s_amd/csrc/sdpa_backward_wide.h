@@ -217,11 +217,12 @@ int sdpa_backward_wide(dl4s_hip_ctx *ctx, const float *q, const float *k, const 
         }
     float *S = static_cast<float *>(bufs[0]), *dP = static_cast<float *>(bufs[1]), *qs = static_cast<float *>(bufs[2]);
     // A product whose own shape would send it to the skinny kernels (few output blocks) comes here with a batch of pairs: when
-    // the batch as a whole has more blocks than that rule's bound, the tiled kernels take it.
+    // the call's pairs as a whole have more blocks than that rule's bound, the tiled kernels take it (all the pairs, not the
+    // chunk's: a call gets the same kernels, and with them the same bits, whatever the scratch bound makes of its chunks).
     const auto gemm = [&](dl4s_hip_ctx *c, const float *a, int64_t ar, int64_t ac, int64_t as, const float *b, int64_t br, int64_t bc,
                           int64_t bs, float *r, int64_t rs, int64_t n, float alpha, float beta, int ta, int tb, int triangle) {
         const int64_t M = ta ? ac : ar, N = tb ? br : bc;
-        if (triangle || n * ((M + 31) / 32) * ((N + 31) / 32) > 2ll * c->cu_count)
+        if (triangle || pairs * ((M + 31) / 32) * ((N + 31) / 32) > 2ll * c->cu_count)
             return dl4s::gemm_batched_tiled(c, a, ar, ac, as, b, br, bc, bs, r, rs, n, alpha, beta, ta, tb, triangle);
         return dl4s_hip_gemm_batched_f32(c, a, ar, ac, as, b, br, bc, bs, r, rs, n, alpha, beta, ta, tb);
     };
