@@ -22,6 +22,12 @@ namespace {
 template <int W> struct NarrowTile {
     static constexpr int LS = W + 4;          // LDS row stride (36, 20, 52): keeps 128-bit reads of consecutive rows on distinct banks
     static constexpr int TF = BN * LS;        // floats per tile
+    // Row stride of the V tile in the main kernel.  Its 16 x 16 x 4 MFMA operand reads (W = 16, and the columns 32 .. 47 of
+    // W = 48) put the lanes 16 s .. 16 s + 15 on 16 consecutive floats of row r + (s & 1) + 4 (s >> 1): with rows of exactly
+    // W floats (16, 48: an odd multiple of 16) the two rows that a half of the wavefront reads land on the two halves of the
+    // 32 banks; on the K tile's stride they overlapped in four (W + 4 = 20, 52) and the read took twice as long.
+    static constexpr int LSV = (W == 32) ? LS : W;
+    static constexpr int TFV = BN * LSV;
     static constexpr int NJ = W / 8;          // 128-bit reads per K row fragment
 };
 
@@ -76,7 +82,7 @@ __device__ __forceinline__ void attend_tile_16(const float *Kb, const float *Vt,
                                                float &m_use, float &l_run, const int k0, const int q0, const int qi, const int half,
                                                const int ln, const int Lk, const int len, const float *mrow, const long long msk,
                                                const int cls) {
-    constexpr int LS = NarrowTile<16>::LS;
+    constexpr int LSV = NarrowTile<16>::LSV;
     f32x16 s0 = masked_scores<KIND, 2>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
     float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
 #pragma unroll
@@ -106,7 +112,7 @@ __device__ __forceinline__ void attend_tile_16(const float *Kb, const float *Vt,
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
         const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(s0[2 * p]), __float_as_uint(s0[2 * p + 1]), false, false);
-        const float va = Vt[(8 * (p >> 1) + 2 * (p & 1)) * LS];
+        const float va = Vt[(8 * (p >> 1) + 2 * (p & 1)) * LSV];
         og[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[0]), og[0], 0, 0, 0);
         og[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[1]), og[1], 0, 0, 0);
     }
@@ -121,7 +127,7 @@ __device__ __forceinline__ void attend_tile_48(const float *Kb, const float *Vb,
                                                f32x4 (&og)[2], float &m_run, float &m_use, float &l_run, const int k0, const int q0,
                                                const int qi, const int half, const int ln, const int Lk, const int len,
                                                const float *mrow, const long long msk, const int cls) {
-    constexpr int LS = NarrowTile<48>::LS;
+    constexpr int LSV = NarrowTile<48>::LSV;
     f32x16 s0 = masked_scores<KIND, 6>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
     float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
 #pragma unroll
@@ -150,11 +156,11 @@ __device__ __forceinline__ void attend_tile_48(const float *Kb, const float *Vb,
     }
     l_run += psum;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(Vb[(8 * (r >> 2) + (r & 3)) * LS], s0[r], o0, 0, 0, 0);
+    for (int r = 0; r < 16; ++r) o0 = __builtin_amdgcn_mfma_f32_32x32x2f32(Vb[(8 * (r >> 2) + (r & 3)) * LSV], s0[r], o0, 0, 0, 0);
 #pragma unroll
     for (int p = 0; p < 8; ++p) {
         const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(s0[2 * p]), __float_as_uint(s0[2 * p + 1]), false, false);
-        const float va = Vt[(8 * (p >> 1) + 2 * (p & 1)) * LS];
+        const float va = Vt[(8 * (p >> 1) + 2 * (p & 1)) * LSV];
         og[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[0]), og[0], 0, 0, 0);
         og[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(va, __uint_as_float(sw[1]), og[1], 0, 0, 0);
     }
@@ -176,10 +182,10 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
                                                                    int Lq, int Lk, float rT, MaskArgs mask, int strict, int nqb,
                                                                    int total_blocks, int lpt, int token_major,
                                                                    float *__restrict__ stats, int hd) {
-    constexpr int LS = NarrowTile<W>::LS, TF = NarrowTile<W>::TF;
+    constexpr int LS = NarrowTile<W>::LS, TF = NarrowTile<W>::TF, LSV = NarrowTile<W>::LSV, TFV = NarrowTile<W>::TFV;
     extern __shared__ __align__(16) float lds[];
     float *Ks = lds;              // [2][BN][LS]
-    float *Vs = lds + 2 * TF;     // [2][BN][LS]
+    float *Vs = lds + 2 * TF;     // [2][BN][LSV]
 
     int bh, unit;
     if (!work_item(nqb, total_blocks, lpt & 1, bh, unit, lpt >> 1)) return;
@@ -235,10 +241,10 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
     const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(v + kv_base), 0, kv_bytes, 0x00020000);
     const unsigned ld_off = ld_col < hd ? (unsigned)(ld_row * rs + ld_col) * 4u : 0x80000000u;
     const unsigned tile_bytes = (unsigned)BN * rs * 4u;
-    const int lds_off = ld_row * LS + ld_col;
+    const int lds_off = ld_row * LS + ld_col, lds_off_v = ld_row * LSV + ld_col;
     const int ld_row2 = (tid + 256) / CPR, ld_col2 = ((tid + 256) % CPR) * 4;      // W = 48, wavefronts 0, 1
     const unsigned ld_off2 = ld_col2 < hd ? (unsigned)(ld_row2 * rs + ld_col2) * 4u : 0x80000000u;
-    const int lds_off2 = ld_row2 * LS + ld_col2;
+    const int lds_off2 = ld_row2 * LS + ld_col2, lds_off2_v = ld_row2 * LSV + ld_col2;
     f32x4 kst, vst, kst2, vst2;
     auto load_tile = [&](int t) {
         const int o = (int)(ld_off + t * tile_bytes);
@@ -259,13 +265,14 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
     auto store_tile = [&](int buf) {
         if (W != 16) {
             *reinterpret_cast<f32x4 *>(Ks + buf * TF + lds_off) = kst;
-            *reinterpret_cast<f32x4 *>(Vs + buf * TF + lds_off) = vst;
+            *reinterpret_cast<f32x4 *>(Vs + buf * TFV + lds_off_v) = vst;
             if (W == 48 && wave < 2) {
                 *reinterpret_cast<f32x4 *>(Ks + buf * TF + lds_off2) = kst2;
-                *reinterpret_cast<f32x4 *>(Vs + buf * TF + lds_off2) = vst2;
+                *reinterpret_cast<f32x4 *>(Vs + buf * TFV + lds_off2_v) = vst2;
             }
         } else {
-            *reinterpret_cast<f32x4 *>((wave < 2 ? Ks : Vs) + buf * TF + lds_off) = kst;
+            if (wave < 2) *reinterpret_cast<f32x4 *>(Ks + buf * TF + lds_off) = kst;
+            else *reinterpret_cast<f32x4 *>(Vs + buf * TFV + lds_off_v) = kst;
         }
     };
 
@@ -282,9 +289,9 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
     __syncthreads();
 
     const int k_lds = ln * LS + half * (W / 2);
-    const int v_lds = (4 * half) * LS + ln;
+    const int v_lds = (4 * half) * LSV + ln;
     const int slot = lane >> 4;
-    const int v_lds16 = ((slot & 1) + 4 * (slot >> 1)) * LS + (W == 48 ? 32 : 0) + (lane & 15);
+    const int v_lds16 = ((slot & 1) + 4 * (slot >> 1)) * LSV + (W == 48 ? 32 : 0) + (lane & 15);
     const float *mrow = DENSE ? mask.dense + b * mask.sb + hh * mask.sh + qic * mask.sq : nullptr;
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;
@@ -298,13 +305,13 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
         if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
         if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
             if constexpr (W == 16)
-                attend_tile_16<KIND>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds16, qr, og, m_run, m_use, l_run, k0, q0, qi, half, ln, Lk,
+                attend_tile_16<KIND>(Ks + buf * TF + k_lds, Vs + buf * TFV + v_lds16, qr, og, m_run, m_use, l_run, k0, q0, qi, half, ln, Lk,
                                      len, mrow, mask.sk, cls);
             else if constexpr (W == 48)
-                attend_tile_48<KIND>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds, Vs + buf * TF + v_lds16, qr, o0, og, m_run, m_use, l_run,
+                attend_tile_48<KIND>(Ks + buf * TF + k_lds, Vs + buf * TFV + v_lds, Vs + buf * TFV + v_lds16, qr, o0, og, m_run, m_use, l_run,
                                      k0, q0, qi, half, ln, Lk, len, mrow, mask.sk, cls);
             else
-                attend_tile_narrow<KIND, W>(Ks + buf * TF + k_lds, Vs + buf * TF + v_lds, qr, o0, m_run, m_use, l_run, k0, q0, qi, half, Lk,
+                attend_tile_narrow<KIND, W>(Ks + buf * TF + k_lds, Vs + buf * TFV + v_lds, qr, o0, m_run, m_use, l_run, k0, q0, qi, half, Lk,
                                             len, mrow, mask.sk, cls);
         }
         if (more) store_tile(buf ^ 1);
@@ -496,7 +503,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_narrow(const fl
 template <int KIND, int W>
 int launch_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
                   float rT, const MaskArgs &m, int strict, int token_major, int no_split, float *stats, int hd) {
-    constexpr int TF = NarrowTile<W>::TF;
+    constexpr int TF = NarrowTile<W>::TF, TFV = NarrowTile<W>::TFV;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
     const long long waves = (long long)B * H * ((Lq + 31) / 32);
@@ -519,7 +526,7 @@ int launch_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
     // gain from it well beyond the four per CU that are resident at once (B5 H16 L2048 d32 causal 216 -> 191 us, B6
     // 248 -> 222 us, B8 299 -> 295 us; d16 133 -> 119, 154 -> 138, 188 -> 180 us), where the 64-wide kernel starts to lose
     const int lpt_arg = lpt | (lpt ? (ctx->cu_count / 8) << 1 : 0);
-    hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
+    hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, W>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(2 * TF + 2 * TFV + 32) * sizeof(float),
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_narrow");
 }
@@ -529,7 +536,7 @@ int launch_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
 template <int KIND>
 int launch_narrow48_main(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v, float *out, int B, int H, int Lq, int Lk,
                          float rT, const MaskArgs &m, int strict, int token_major, float *stats, int hd) {
-    constexpr int TF = NarrowTile<48>::TF;
+    constexpr int TF = NarrowTile<48>::TF, TFV = NarrowTile<48>::TFV;
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
     const int nqb = (Lq + BM - 1) / BM;
@@ -538,7 +545,7 @@ int launch_narrow48_main(dl4s_hip_ctx *ctx, const float *q, const float *k, cons
     const int lpt = (uneven && nqb >= 2) ? 1 : 0;
     // (reversed rounds up to five workgroups per CU, like the 64-wide kernel: B5 H16 L2048 d48 296 -> 289 us, beyond it loses)
     const int lpt_arg = lpt | ((lpt && total <= 5ll * ctx->cu_count) ? (ctx->cu_count / 8) << 1 : 0);
-    hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, 48>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(4 * TF + 32) * sizeof(float),
+    hipLaunchKernelGGL((sdpa_prefill_f32_narrow<KIND, 48>), dim3((unsigned)((total + 7) / 8 * 8)), dim3(256), (size_t)(2 * TF + 2 * TFV + 32) * sizeof(float),
                        ctx->stream, q, k, v, out, H, Lq, Lk, rT, m, strict, nqb, (int)total, lpt_arg, token_major, stats, hd);
     return dl4s::launch_status("sdpa_prefill_f32_narrow");
 }
