@@ -401,13 +401,15 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     DL4S_REQUIRE(BH <= 65535 && Tcap < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa_decode: B*H=%lld above 65535", (long long)BH);
     const int KB = keys_per_iteration(d, vec);   // keys per wavefront iteration
     const int PSTR = pstr(row_width(d, vec));
-    // Aim at 16 resident wavefronts on every CU.  Long caches use 16-wavefront workgroups; the key range is split
-    // over several workgroups only when batch*heads alone does not fill the GPU.  Up to 512 rows one workgroup per pair
-    // does it all (16 wavefronts above 128 rows): a second launch for the merge costs more than the split saves
-    // (B1 H8: 256 rows 6.4 -> 4.5 us, 512 rows 6.5 -> 4.8 us).  The split follows T alone; with key lengths a workgroup
-    // whose share lies beyond its batch element's length leaves an empty record.
+    // Aim at 16 resident wavefronts on every CU.  Caches above 128 rows use 16-wavefront workgroups (between 512 and 2048
+    // rows they had four: B16 H16 d64 over 600 rows 17.1 -> 13.0 us, 1536 rows 35.2 -> 30.2 us, B4 H16 d128 over 1536 rows
+    // 27.2 -> 20.2 us - fewer, larger workgroups, and with 256 pairs no split and no merge launch at all); the key range is
+    // split over several workgroups only when batch*heads alone does not fill the GPU.  Up to 512 rows one workgroup per
+    // pair does it all: a second launch for the merge costs more than the split saves (B1 H8: 256 rows 6.4 -> 4.5 us,
+    // 512 rows 6.5 -> 4.8 us).  The split follows T alone; with key lengths a workgroup whose share lies beyond its batch
+    // element's length leaves an empty record.
     const bool short_cache = T <= 512;
-    const int nw = short_cache ? (T > 128 ? 16 : 4) : (T >= 2048 ? 16 : 4);
+    const int nw = T > 128 ? 16 : 4;
     const long long want_wg = ((long long)ctx->cu_count * 16 + nw - 1) / nw;
     long long max_split = short_cache ? 1 : (T + (long long)nw * KB - 1) / ((long long)nw * KB);
     long long ns = (want_wg + BH - 1) / BH;
