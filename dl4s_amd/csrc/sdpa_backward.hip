@@ -1018,8 +1018,8 @@ int launch_bwd(dl4s_hip_ctx *ctx, const float *q, const float *k, const float *v
         dl4s::lds_limit_done(ctx, dl4s::LDS_BWD, KIND);
     }
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
-    const bool dq_small = !no_split && (long long)B * H * ((Lq + 31) / 32) < 8ll * ctx->cu_count && Lk >= 2 * BN;
-    const bool dkv_small = !no_split && (long long)B * H * ((Lk + 31) / 32) < 8ll * ctx->cu_count && Lq >= 2 * BN;
+    const bool dq_small = !no_split && sdpa_bwd_small_launch(ctx, B, H, Lq, uneven, false) && Lk >= 2 * BN;
+    const bool dkv_small = !no_split && sdpa_bwd_small_launch(ctx, B, H, Lk, uneven, false) && Lq >= 2 * BN;
     // Large launches: the dK/dV kernel stores dS, the dQ kernel only contracts it with K (five products for five).  The
     // scratch tensor [B*H][Lk][Lq] comes from the pool; when it cannot be had (too large, pool miss while a graph is being
     // recorded, out of memory) the two self-contained kernels below run instead.

@@ -385,8 +385,8 @@ int launch_bwd_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const f
     constexpr int TF = BN * (W + 4);
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
-    const bool dq_small = !no_split && (long long)B * H * ((Lq + 31) / 32) < 8ll * ctx->cu_count && Lk >= 2 * BN;
-    const bool dkv_small = !no_split && (long long)B * H * ((Lk + 31) / 32) < 8ll * ctx->cu_count && Lq >= 2 * BN;
+    const bool dq_small = !no_split && sdpa_bwd_small_launch(ctx, B, H, Lq, uneven, true) && Lk >= 2 * BN;
+    const bool dkv_small = !no_split && sdpa_bwd_small_launch(ctx, B, H, Lk, uneven, true) && Lq >= 2 * BN;
     if (dq_small || dkv_small) return 0;
     const long long Lqp = (Lq + 31) & ~31ll, Lkp = (Lk + 31) & ~31ll;
     const long long slab = Lqp * Lkp * 4;

@@ -304,6 +304,22 @@ __device__ __forceinline__ float plain_score(const float *qs, const float *krow,
 // on the same kind of kernel.
 // Head dims above 128 up to 256 that the 192- and 256-wide forward kernels take as they are (the tensors 16-byte aligned
 // besides): a multiple of 4 whose K/V rows of one (batch, head) pair stay inside the kernels' 32-bit byte offsets.
+// Gradient launches of the 64-wide and narrower classes that count as small (one 32-row block per workgroup, the tiles along
+// the other axis split over its wavefronts; the narrow classes run these on 64-wide padded tiles) for L rows along the axis
+// the workgroups own.  64-wide: fewer 32-row blocks than four per CU.  (The bound was eight per CU: between four and eight
+// the 128-row kernels are faster - B1 H16 L2048 d64 without a mask 490 -> 370 us, B8 H16 L256 99 -> 66 us, B3 H16 L1024 causal
+// 263 -> 223 us.)  One case keeps the 32-row kernels up to eight per CU: blocks of different length, at most one 128-row
+// workgroup per CU and 2048 rows or more - there the longest block sets the time of the 128-row launch (B1 H16 L2048
+// causal 328 us against 369 us, B1 H8 L4096 584 against 717 us).  Narrow classes, whose own 128-row kernels do not pay for
+// padding: fewer than two per CU, four with blocks of different length from 512 rows on (B3 H16 L1024 d32 causal 244 -> 130
+// us, B1 H16 L1024 d32 without a mask 138 -> 115 us, B8 H16 L128 d16 27 -> 20 us; B1 H8 L2048 d32 causal stays at 161 us
+// against 213 us on the 128-row kernels).
+inline bool sdpa_bwd_small_launch(const dl4s_hip_ctx *ctx, int64_t B, int64_t H, int64_t L, bool uneven, bool narrow) {
+    const long long blocks32 = (long long)B * H * ((L + 31) / 32), blocks128 = (long long)B * H * ((L + 127) / 128);
+    if (narrow) return blocks32 < 2ll * ctx->cu_count || (uneven && L >= 512 && blocks32 < 4ll * ctx->cu_count);
+    return blocks32 < 4ll * ctx->cu_count || (uneven && L >= 2048 && blocks128 <= ctx->cu_count && blocks32 < 8ll * ctx->cu_count);
+}
+
 inline bool sdpa_wide_route(int64_t H, int64_t Lk, int64_t d, int token_major) {
     return d > HD2 && d <= 256 && d % 4 == 0 && Lk * (token_major ? H : 1) * d * 4 < ((d == 160 || d == 192 || d == 256) ? (1ll << 31) : (1ll << 30));
 }

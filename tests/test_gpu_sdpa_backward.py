@@ -636,6 +636,25 @@ def test_gradients_for_odd_head_dims_above_128_on_padded_copies(ctx, orc, d):
     assert_parity(dv[:1, :1], rv, "dv d=%d" % d)
 
 
+@pytest.mark.parametrize("d", [64, 32, 16])
+@pytest.mark.parametrize("mask_kind", ["causal", "none"])
+def test_mid_size_launches_between_the_small_and_the_large_forms(ctx, orc, d, mask_kind):
+    """Launches of four to eight 32-row blocks per CU (here 6: 48 pairs of 1024 rows on 256 CUs) run the 128-row kernels of
+    their class; checked against the oracle on the first and the last (batch, head) pair."""
+    from dl4s_amd import lib
+    B, H, L = 3, 16, 1024
+    rng = np.random.default_rng(1000 + d)
+    q, k, v, dout = (rand(rng, B, H, L, d) for _ in range(4))
+    mask = causal_mask(L, L) if mask_kind == "causal" else None
+    kw = dict(kind=lib.MASK_CAUSAL) if mask_kind == "causal" else {}
+    out, stats, dq, dk, dv = run_fwd_bwd(ctx, q, k, v, dout, **kw)
+    for sl in (np.s_[:1, :1], np.s_[-1:, -1:]):
+        rq, rk, rv = orc.sdpa_backward(q[sl], k[sl], v[sl], mask, dout[sl])
+        assert_parity(dq[sl], rq, "dq d=%d %s" % (d, mask_kind))
+        assert_parity(dk[sl], rk, "dk d=%d %s" % (d, mask_kind))
+        assert_parity(dv[sl], rv, "dv d=%d %s" % (d, mask_kind))
+
+
 @pytest.mark.parametrize("d,Lq,Lk,B,H", [(256, 1100, 1100, 1, 2), (192, 1300, 700, 1, 2), (160, 600, 1000, 1, 2), (256, 1100, 1100, 4, 8),
                                          (160, 700, 4200, 1, 1), (160, 600, 1001, 1, 2), (192, 1030, 1030, 1, 2),
                                          (132, 513, 4, 1, 1), (132, 513, 2048, 1, 2)])
