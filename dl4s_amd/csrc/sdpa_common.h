@@ -320,6 +320,23 @@ inline bool sdpa_bwd_small_launch(const dl4s_hip_ctx *ctx, int64_t B, int64_t H,
     return blocks32 < 4ll * ctx->cu_count || (uneven && L >= 2048 && blocks128 <= ctx->cu_count && blocks32 < 8ll * ctx->cu_count);
 }
 
+// Shares of the key tiles per query block on a forward launch with fewer blocks than two per CU (the 96-wide and wider
+// kernels): the even count w up to 8 with the least ceil(blocks * w / CUs) / w * (1 + per_share * w) - rounds of the CUs per
+// share, times what a share costs in partial records and in the merge (measured: 2 % per share on the 96- and 128-wide
+// kernels, 4 to 5 % on the 160- to 256-wide ones) - taking a larger count only for 5 % less.  256 blocks on 256 CUs: 2; 192: 4
+// (three rounds of quarter shares against two rounds of halves: B1 H12 L2048 d128 without a mask 267 -> 219 us, causal
+// 218 -> 160 us); 160: 8 / 4 (B1 H10 L2048 d128 266 -> 203 us, d256 593 -> 487 us); 128: 2; 96: 8; 64 and 48: 4.  Odd counts lose
+// on every shape measured.  From the extents only: every mask kind of a problem adds in one order.
+inline long long sdpa_key_shares(long long blocks, long long nkt, int cu, double per_share) {
+    long long best = 2;
+    double best_cost = 1e30;
+    for (long long w = 2; w <= 8 && w <= nkt / 2; w += 2) {
+        const double cost = (double)((blocks * w + cu - 1) / cu) / (double)w * (1.0 + per_share * (double)w);
+        if (cost < 0.95 * best_cost) { best_cost = cost; best = w; }
+    }
+    return best;
+}
+
 inline bool sdpa_wide_route(int64_t H, int64_t Lk, int64_t d, int token_major) {
     return d > HD2 && d <= 256 && d % 4 == 0 && Lk * (token_major ? H : 1) * d * 4 < ((d == 160 || d == 192 || d == 256) ? (1ll << 31) : (1ll << 30));
 }

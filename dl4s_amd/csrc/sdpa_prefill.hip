@@ -649,12 +649,12 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     size_t part_bytes = 0;
     if ((mfma128_path || (w96_path && dk % 4 == 0)) && !no_split) {
         const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
-        // enough shares to give every CU its workgroup; two where every CU just has one (blocks of different length then pair up
-        // long with short through the order of their workgroups: B2 H8 L2048 d256 causal 570 -> 353 us; without a mask
-        // 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
+        // the count that leaves the fewest rounds of the CUs per share (sdpa_key_shares); two where every CU just has one block
+        // (blocks of different length then pair up long with short through the order of their workgroups: B2 H8 L2048 d256
+        // causal 570 -> 353 us; without a mask 569 -> 609 us - the count depends on the extents only, so that every mask kind of
+        // a problem adds in one order)
         if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
-            long long want = std::max(2ll, ((long long)ctx->cu_count + blocks - 1) / blocks);
-            want = std::min(want, std::min(8ll, nkt / 2));
+            const long long want = sdpa_key_shares(blocks, nkt, ctx->cu_count, 0.02);
             const size_t bytes = (size_t)want * B * H * Lq * PART2_STRIDE * sizeof(float);
             if (want > 1 && bytes <= (size_t(256) << 20)) { nsplit128 = (int)want; part_bytes = bytes; }
         }
@@ -662,12 +662,12 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
     // the wide kernels run one workgroup per CU: the same split on launches that leave CUs without one
     if (wide_path && !no_split) {
         const long long blocks = ((Lq + BM - 1) / BM) * B * H, nkt = (Lk + BN - 1) / BN;
-        // enough shares to give every CU its workgroup; two where every CU just has one (blocks of different length then pair up
-        // long with short through the order of their workgroups: B2 H8 L2048 d256 causal 570 -> 353 us; without a mask
-        // 569 -> 609 us - the count depends on the extents only, so that every mask kind of a problem adds in one order)
+        // the count that leaves the fewest rounds of the CUs per share (sdpa_key_shares); two where every CU just has one block
+        // (blocks of different length then pair up long with short through the order of their workgroups: B2 H8 L2048 d256
+        // causal 570 -> 353 us; without a mask 569 -> 609 us - the count depends on the extents only, so that every mask kind of
+        // a problem adds in one order)
         if (blocks < 2ll * ctx->cu_count && nkt >= 4) {
-            long long want = std::max(2ll, ((long long)ctx->cu_count + blocks - 1) / blocks);
-            want = std::min(want, std::min(8ll, nkt / 2));
+            const long long want = sdpa_key_shares(blocks, nkt, ctx->cu_count, 0.045);
             const size_t bytes = (size_t)want * B * H * Lq * PARTW_STRIDE * sizeof(float);
             if (want > 1 && bytes <= (size_t(256) << 20)) { nsplit128 = (int)want; part_bytes = bytes; }
         }
