@@ -507,7 +507,10 @@ int launch_narrow(dl4s_hip_ctx *ctx, const float *q, const float *k, const float
     constexpr bool causal_kind = (KIND == DL4S_MASK_CAUSAL || KIND == DL4S_MASK_CAUSAL_OR_KEY_LENGTHS);
     const bool uneven = (causal_kind || (KIND == DL4S_MASK_DENSE_F32 && m.cls && m.sq)) && !strict;
     const long long waves = (long long)B * H * ((Lq + 31) / 32);
-    if (!no_split && waves < 8ll * ctx->cu_count && Lk >= 2 * BN) {
+    // (from 1024 keys on up to sixteen wavefronts per CU: B1 H8 L8192 d32 causal 382 -> 292 us, B1 H16 L4096 203 -> 161 us,
+    // B3 H16 L2048 145 -> 129 us, without a mask 3 - 7 %; with short rows the 128-query kernel wins from eight on: B16 H16 L256
+    // 20 us against 24 us)
+    if (!no_split && (waves < 8ll * ctx->cu_count || (Lk >= 1024 && waves < 16ll * ctx->cu_count)) && Lk >= 2 * BN) {
         const int nqb32 = (Lq + 31) / 32;
         const long long total32 = (long long)nqb32 * B * H;
         DL4S_REQUIRE(total32 < (1ll << 30), DL4S_HIP_EUNSUPPORTED, "sdpa: %lld workgroups exceed the grid limit", total32);
