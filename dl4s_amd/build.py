@@ -11,7 +11,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdl4s_hip.so")
 HOST_LIB = os.path.join(HERE, "libdl4s_host.so")
-MICROBENCH = os.path.join(HERE, "mfma_issue")      # stand-alone program, see csrc/microbench/mfma_issue.hip
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -20,8 +19,6 @@ FLAGS = [
     # keep the compiler from forming packed fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
-# extra compiler flags for experiments, e.g. DL4S_HIP_EXTRA_FLAGS=-DDL4S_LPT_GROUP=4 (see csrc/work_order.h)
-FLAGS += os.environ.get("DL4S_HIP_EXTRA_FLAGS", "").split()
 
 
 def build(verbose=False):
@@ -51,21 +48,7 @@ def build(verbose=False):
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(cmd)
     build_host(verbose)
-    build_microbench(verbose)
     return LIB
-
-
-def build_microbench(verbose=False):
-    """The MFMA / VALU issue microbenchmark quoted for the prefill kernel's ceiling (a program of its own, not in the library)."""
-    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-o", MICROBENCH, os.path.join(CSRC, "microbench", "mfma_issue.hip")]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if p.returncode != 0:
-        sys.stderr.write(p.stdout)
-        raise RuntimeError("hipcc failed on the microbenchmark")
-    return MICROBENCH
 
 
 def build_host(verbose=False):

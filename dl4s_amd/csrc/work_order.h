@@ -42,18 +42,8 @@ DL4S_WORK_ORDER_FN bool work_item_at(const int block, const int nunits, const in
         const int x = bid & 7, wl = bid >> 3, cnt = npairs >> 3;
         if (wl >= cnt * nunits) return false;
         if (lpt) {
-#ifdef DL4S_LPT_GROUP
-            // Experiment (compile with -DDL4S_LPT_GROUP=G): longest first over groups of G of the XCD's pairs instead of all
-            // of them - fewer pairs' K and V in the L2 at a time, less balance at the end of the launch.  Measured on
-            // B8 H16 L2048 causal: G = 2 / 4 / 8 / all 16 give 105 / 116 / 101 / 127 TFLOP/s, so the default stays.
-            const int per = DL4S_LPT_GROUP * nunits, grp = wl / per, r = wl - grp * per;
-            const int size = imin(DL4S_LPT_GROUP, cnt - grp * DL4S_LPT_GROUP);     // the last group may be smaller
-            unit = r / size;
-            bh = x + 8 * (grp * DL4S_LPT_GROUP + r % size);
-#else
             unit = wl / cnt;
             bh = x + 8 * (wl % cnt);
-#endif
         }
         else { bh = x + 8 * (wl / nunits); unit = wl % nunits; }
         return true;

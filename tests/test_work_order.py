@@ -23,22 +23,6 @@ def shim():
     return lib
 
 
-@pytest.mark.parametrize("group", [1, 2, 4, 5])
-def test_longest_first_over_groups_of_pairs_hands_out_every_item_once(group):
-    """The -DDL4S_LPT_GROUP=G build of the order (an experiment that is kept compilable): still every item exactly once, a
-    pair still on one XCD."""
-    out = os.path.join(tempfile.mkdtemp(prefix="dl4s_work_order_g_"), "libwork_order.so")
-    subprocess.check_call(["g++", "-O1", "-shared", "-fPIC", "-std=c++17", "-DDL4S_LPT_GROUP=%d" % group, "-o", out,
-                           os.path.join(HERE, "work_order_shim.cpp")])
-    lib = C.CDLL(out)
-    lib.work_item_at.argtypes = [C.c_int] * 5 + [C.POINTER(C.c_int)] * 2
-    lib.work_item_at.restype = C.c_int
-    for npairs, nunits in [(8, 16), (128, 16), (24, 5), (40, 3), (16, 1), (72, 7)]:
-        total, got = items(lib, npairs, nunits, 1, 0)
-        assert sorted((b, u) for _, b, u in got) == [(b, u) for b in range(npairs) for u in range(nunits)], (npairs, nunits)
-        assert all(block % 8 == b % 8 for block, b, _ in got)
-
-
 def items(lib, npairs, nunits, lpt, snake):
     total = npairs * nunits
     grid = (total + 7) // 8 * 8
