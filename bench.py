@@ -60,11 +60,24 @@ def prefill(ctx, lib, steps, warmup):
     ctx.sync()
     wall = time.perf_counter() - t0
     o = out.numpy()
+    # The same call with DL4S_SDPA_STRICT: every key tile visited, so that NaN / Inf in K or V at blocked keys reach the
+    # output as in the reference (0 x NaN).  Same bits as the default on finite inputs; reported beside the headline.
+    strict_out = ctx.empty((B, H, L, d))
+    nstrict = max(3, steps // 4)
+    for _ in range(3):
+        ctx.sdpa_fwd(dq, dk, dv, strict_out, B, H, L, L, d, d, 0.125, desc, lib.SDPA_STRICT)
+    ctx.timer_begin()
+    for _ in range(nstrict):
+        ctx.sdpa_fwd(dq, dk, dv, strict_out, B, H, L, L, d, d, 0.125, desc, lib.SDPA_STRICT)
+    strict_ms = ctx.timer_end() / nstrict
+    strict_same = bool(np.array_equal(strict_out.numpy(), o))
+    strict_out.release()
     if not (np.isfinite(o).all() and np.allclose(o[:, :, 0], v[:, :, 0], atol=1e-6)):
         raise RuntimeError("prefill output failed its sanity check")
     for b in (dq, dk, dv, out):
         b.release()
-    return {"flops": flops, "wall_s": wall, "event_ms_per_launch": ev_ms / steps,
+    return {"flops": flops, "wall_s": wall, "event_ms_per_launch": ev_ms / steps, "strict_ms_per_launch": strict_ms,
+            "strict_bit_identical": strict_same,
             "shape": {"B": B, "H": H, "L": L, "d": d}, "inputs": (q, k, v), "output": o}
 
 
@@ -588,7 +601,10 @@ def main():
 
     tflops = pre["flops"] * args.steps / pre["wall_s"] / 1e12
     ach = pre["flops"] / (pre["event_ms_per_launch"] * 1e-3) / 1e12
-    line = {
+    line = {}
+    if others is not None:
+        line["other_configs"] = others      # first, so that the headline objects end the line
+    line.update({
         "metric": "attention fwd TFLOP/s (fp32)",
         "value": tflops,
         "unit": "TFLOP/s",
@@ -607,7 +623,22 @@ def main():
                      "frac": ach / MFMA_FP32_PEAK_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
                      "traffic_unit": "bytes per launch (L2 fills + writes, rocprofv3 --pmc)", "kernel": "sdpa_prefill_f32_d64",
                      "ms_per_launch": pre["event_ms_per_launch"]},
-    }
+    })
+    sh = pre["shape"]
+    dense_flops = 4.0 * sh["d"] * sh["B"] * sh["H"] * sh["L"] * sh["L"]
+    # strict mode issues the dense problem's MFMAs for the causal problem's algorithmic flops
+    line["roofline"]["strict_mode"] = {
+        "what": "same launch with DL4S_SDPA_STRICT (every key tile visited: the reference's NaN/Inf behaviour at blocked keys)",
+        "ms_per_launch": pre["strict_ms_per_launch"],
+        "achieved": pre["flops"] / (pre["strict_ms_per_launch"] * 1e-3) / 1e12,
+        "frac": pre["flops"] / (pre["strict_ms_per_launch"] * 1e-3) / 1e12 / MFMA_FP32_PEAK_TFLOPS,
+        "issued_tflops": dense_flops / (pre["strict_ms_per_launch"] * 1e-3) / 1e12,
+        "bit_identical_to_default_on_these_inputs": pre["strict_bit_identical"]}
+    if dec:
+        line["roofline"]["decode"] = {"bound": "hbm", "kernel": "sdpa_decode_splitk_f32", "us_per_step": dec["us_per_step"],
+                                      "achieved": dec["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dec["gbs"] / HBM_PEAK_GBS,
+                                      "tokens_per_s": dec["tokens_per_s"], "traffic": DECODE_TRAFFIC_BYTES,
+                                      "bytes_per_step": dec["bytes_per_step"]}
     if dec:
         line["decode"] = {"workload": "incremental decode B=16 H=16 d=64, KV cache 4096 rows + 64 append+attend steps "
                                       "(benchmark config 5)",
@@ -622,8 +653,6 @@ def main():
         line["cpu_blas_proxy"] = cpu_blas_proxy_prefill(q, k, v, min(32, q.shape[0] * q.shape[1]))
         if dec:
             line["decode"]["cpu_baseline"] = cpu_baseline_decode()
-    if others is not None:
-        line["other_configs"] = others
     print(json.dumps(line))
 
 

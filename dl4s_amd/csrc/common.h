@@ -33,6 +33,8 @@ struct dl4s_hip_ctx {
     std::mutex scratch_mu;
     // Device address, on this context's GPU, of the fixed block dl4s_hip_sdpa_decode_noalloc_f32 keeps its partial records in.
     float *static_scratch = nullptr;
+    // Recorded behind every use of that block by this context; a call on another context of the same GPU waits for it.
+    hipEvent_t static_scratch_done = nullptr;
     // Stream capture (dl4s_hip_graph_begin .. dl4s_hip_graph_end): entry points that would wait for the stream, copy to or
     // from host memory or change device allocations refuse to run while it is set.  scratch_generation counts the
     // regrowths of the scratch block; a captured graph holds the block's address and is refused once it has moved.
@@ -80,6 +82,7 @@ int gemm_batched_tiled(dl4s_hip_ctx *ctx, const float *lhs, int64_t lhs_rows, in
 // multiples of 4, operands off the 16-byte grid - fail with DL4S_HIP_EUNSUPPORTED before anything is launched.)
 // Looks up the device address of the decode kernels' fixed scratch block (sdpa_decode.hip) for the current GPU.
 int decode_static_scratch_init(dl4s_hip_ctx *ctx);
+void decode_static_scratch_release(dl4s_hip_ctx *ctx);
 
 #define DL4S_CHECK_CTX(ctx)                                                        \
     do {                                                                           \

@@ -86,7 +86,11 @@ int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx) {
     char queried[128] = "";
     if (!prop.name[0] && hipDeviceGetName(queried, (int)sizeof(queried), device_ordinal) != hipSuccess) queried[0] = 0;
     (void)hipGetLastError();
-    snprintf(c->name, sizeof(c->name), "%s (%s)", prop.name[0] ? prop.name : (queried[0] ? queried : "unnamed GPU"), prop.gcnArchName);
+    if (prop.name[0] || queried[0])
+        snprintf(c->name, sizeof(c->name), "%s (%s)", prop.name[0] ? prop.name : queried, prop.gcnArchName);
+    else   // name the GPU by what the properties do hold
+        snprintf(c->name, sizeof(c->name), "AMD GPU %s, %d CUs, %.2f GHz, %.0f GiB", prop.gcnArchName, prop.multiProcessorCount,
+                 prop.clockRate * 1e-6, (double)prop.totalGlobalMem / (double)(1ull << 30));
     hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_begin);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_end);
@@ -100,6 +104,7 @@ int dl4s_hip_create(int device_ordinal, dl4s_hip_ctx **out_ctx) {
     {
         const int rc = decode_static_scratch_init(c);
         if (rc) {
+            decode_static_scratch_release(c);
             (void)hipEventDestroy(c->ev_end);
             (void)hipEventDestroy(c->ev_begin);
             (void)hipStreamDestroy(c->stream);
@@ -120,6 +125,7 @@ int dl4s_hip_destroy(dl4s_hip_ctx *ctx) {
         ctx->capturing = false;
     }
     (void)hipStreamSynchronize(ctx->stream);
+    decode_static_scratch_release(ctx);
     for (auto &b : ctx->held_by_recording) (void)hipFree(b.first);
     for (auto &kv : ctx->pool)
         for (void *p : kv.second) (void)hipFree(p);

@@ -328,6 +328,85 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     }
 }
 
+// ---- LayerNorm whose two sums are added in the reference's order (Engine/CPU/CPUEngine.swift:306-378 with the generic
+// Float.sum, Engine/CPU/Numeric/CPUFloat.swift:239-261): every row of D elements is added left to right starting from
+// zero, then the rows of an item are added to zero one after the other.  Such a sum has one rounding per element in a
+// fixed sequence, so it cannot be spread over lanes: a lane owns a row.  A wavefront takes 64 rows and walks them in
+// tiles of 64 columns, staged through LDS so that global memory is read 256 contiguous bytes per row (lane = column)
+// while the additions run with lane = row (a row stride of 65 floats keeps the 64 lanes on 64 banks).
+constexpr int LN_SEQ_ROWS = 64, LN_SEQ_COLS = 64, LN_SEQ_STRIDE = LN_SEQ_COLS + 1;
+
+__global__ __launch_bounds__(64) void ln_row_sums_seq_f32(const float *__restrict__ x, const float *__restrict__ res,
+                                                            float *__restrict__ part, long long R, long long D) {
+    __shared__ float tile[LN_SEQ_ROWS * LN_SEQ_STRIDE];
+    const int lane = threadIdx.x;
+    const long long r0 = (long long)blockIdx.x * LN_SEQ_ROWS;
+    const int nr = (int)(R - r0 < LN_SEQ_ROWS ? R - r0 : LN_SEQ_ROWS);
+    float st[LN_SEQ_ROWS];
+    auto load = [&](long long c0) {
+        const long long c = c0 + lane;
+#pragma unroll
+        for (int i = 0; i < LN_SEQ_ROWS; ++i) {
+            float v = 0.f;
+            if (i < nr && c < D) {
+                v = x[(r0 + i) * D + c];
+                if (res) v = __fadd_rn(v, res[(r0 + i) * D + c]);
+            }
+            st[i] = v;
+        }
+    };
+    float s = 0.f, ss = 0.f;
+    load(0);
+    for (long long c0 = 0; c0 < D; c0 += LN_SEQ_COLS) {
+        __syncthreads();                  // the lanes are done with the tile before
+#pragma unroll
+        for (int i = 0; i < LN_SEQ_ROWS; ++i) tile[i * LN_SEQ_STRIDE + lane] = st[i];
+        __syncthreads();
+        if (c0 + LN_SEQ_COLS < D) load(c0 + LN_SEQ_COLS);       // in flight during the additions
+        const float *row = tile + lane * LN_SEQ_STRIDE;
+        if (D - c0 >= LN_SEQ_COLS) {
+#pragma unroll
+            for (int c = 0; c < LN_SEQ_COLS; ++c) {
+                const float e = row[c];
+                s = __fadd_rn(s, e);
+                ss = __fadd_rn(ss, __fmul_rn(e, e));
+            }
+        } else {
+            const int nc = (int)(D - c0);
+            for (int c = 0; c < nc; ++c) {
+                const float e = row[c];
+                s = __fadd_rn(s, e);
+                ss = __fadd_rn(ss, __fmul_rn(e, e));
+            }
+        }
+    }
+    if (lane < nr) { part[(r0 + lane) * 2] = s; part[(r0 + lane) * 2 + 1] = ss; }
+}
+
+// The rows of an item, one after the other: rowpart [items][rows][2] -> itempart [items][2].  One wavefront per item
+// stages 512 rows' pairs at a time in LDS; lane 0 adds.
+__global__ __launch_bounds__(64) void ln_item_sums_seq_f32(const float *__restrict__ rowpart, float *__restrict__ itempart, long long rows) {
+    constexpr int CH = 512;
+    __shared__ float sm[2 * CH];
+    const int lane = threadIdx.x;
+    const float *p = rowpart + (long long)blockIdx.x * rows * 2;
+    float s = 0.f, ss = 0.f;
+    for (long long r0 = 0; r0 < rows; r0 += CH) {
+        const int cnt = (int)(rows - r0 < CH ? rows - r0 : CH);
+        __syncthreads();
+        for (int i = lane; i < 2 * cnt; i += 64) sm[i] = p[r0 * 2 + i];
+        __syncthreads();
+        if (lane == 0) {
+#pragma unroll 8
+            for (int i = 0; i < cnt; ++i) {
+                s = __fadd_rn(s, sm[2 * i]);
+                ss = __fadd_rn(ss, sm[2 * i + 1]);
+            }
+        }
+    }
+    if (lane == 0) { itempart[(long long)blockIdx.x * 2] = s; itempart[(long long)blockIdx.x * 2 + 1] = ss; }
+}
+
 // one workgroup (of NT threads: 256, or 1024 when a row is longer than 4096) per batch item, for short rows (per-token LayerNorm of the feed-forward block)
 template <bool VEC, int NT>
 __global__ __launch_bounds__(NT) void ln_small_f32(const float *__restrict__ x, const float *__restrict__ res,
@@ -1056,6 +1135,41 @@ int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *resid
                            n, (long long)D, nblk);
     }
     return dl4s::launch_status("layernorm");
+}
+
+int dl4s_hip_layernorm_reference_order_f32(dl4s_hip_ctx *ctx, const float *x, const float *residual, const float *scale,
+                                           const float *shift, float *result, int64_t B, int64_t rows, int64_t D) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(B >= 0 && rows >= 0 && D >= 0, DL4S_HIP_EINVALID_ARG, "layernorm: negative extent");
+    const long long n = rows * D, R = B * rows;
+    if (B * n == 0) return DL4S_HIP_OK;
+    DL4S_REQUIRE(x && scale && shift && result, DL4S_HIP_EINVALID_ARG, "layernorm: NULL pointer");
+    DL4S_REQUIRE(R < (1ll << 36) && B < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "layernorm: too many rows");
+    const auto a16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool vec = n % 4 == 0 && D % 4 == 0 && a16(x) && a16(residual) && a16(scale) && a16(shift) && a16(result);
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
+    // per-row pairs, then (items of more than one row) per-item pairs behind them
+    const size_t row_floats = (size_t)R * 2, item_floats = rows > 1 ? (size_t)B * 2 : 0;
+    int rc = dl4s::ensure_scratch(ctx, (row_floats + item_floats) * sizeof(float));
+    if (rc) return rc;
+    float *rowpart = reinterpret_cast<float *>(ctx->scratch), *itempart = rows > 1 ? rowpart + row_floats : rowpart;
+    hipLaunchKernelGGL(ln_row_sums_seq_f32, dim3((unsigned)((R + LN_SEQ_ROWS - 1) / LN_SEQ_ROWS)), dim3(64), 0, ctx->stream, x, residual,
+                       rowpart, R, (long long)D);
+    if (rows > 1) hipLaunchKernelGGL(ln_item_sums_seq_f32, dim3((unsigned)B), dim3(64), 0, ctx->stream, rowpart, itempart, (long long)rows);
+    // the normalising pass of the tree-sum kernels on one pair per item (0 + the pair: exact)
+    const long long want = n / (TPB * 8);
+    const unsigned gx = (unsigned)(want < 1 ? 1 : (want > 256 ? 256 : want));
+    for (long long b0 = 0; b0 < B; b0 += 65535) {
+        const unsigned nb = (unsigned)(B - b0 < 65535 ? B - b0 : 65535);
+        const float *xp = x + b0 * n, *rp = residual ? residual + b0 * n : nullptr;
+        if (vec)
+            hipLaunchKernelGGL(ln_apply_f32<true>, dim3(gx, nb), dim3(TPB), 0, ctx->stream, xp, rp, scale, shift, result + b0 * n,
+                               itempart + b0 * 2, n, (long long)D, 1);
+        else
+            hipLaunchKernelGGL(ln_apply_f32<false>, dim3(gx, nb), dim3(TPB), 0, ctx->stream, xp, rp, scale, shift, result + b0 * n,
+                               itempart + b0 * 2, n, (long long)D, 1);
+    }
+    return dl4s::launch_status("layernorm_reference_order");
 }
 
 int dl4s_hip_bias_gelu_f32(dl4s_hip_ctx *ctx, const float *x, const float *bias, float *result, int64_t rows, int64_t D) {

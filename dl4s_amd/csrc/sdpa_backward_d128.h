@@ -609,7 +609,15 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_from_ds_f32_d128(const flo
     for (int t = sp, buf = 0; t < ntiles; t += nsplit, buf ^= 1) {
         const bool more = (t + nsplit < ntiles);
         const bool now = visited(t);
-        const f32x16 p = dsn;
+        f32x16 p = dsn;
+        // The slab's rows of the keys Lk ... (padded to 32) are never written, and the row term of the load sits in the
+        // scalar offset, which the descriptor's range check does not cover: clear them (their K rows are zeros, but
+        // 0 x a stale NaN would not be).
+        if (t * BN + BN > Lk) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (t * BN + 8 * (r >> 2) + 4 * half + (r & 3) >= Lk) p[r] = 0.f;
+        }
         if (more) {
             load_tile(t + nsplit);
             if (visited(t + nsplit)) load_ds(t + nsplit);

@@ -23,8 +23,14 @@
 // name to a kernel: it uses the device address hipGetSymbolAddress returns (dl4s::decode_static_scratch_init).
 constexpr size_t NOALLOC_SCRATCH_FLOATS = size_t(1) << 20;   // 4 MiB
 static __device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
-// Serialises the two launches of a split decode on the fixed block between host threads (whatever their context).
+// Held while the two launches of a split decode on the fixed block are enqueued, so that host threads cannot interleave
+// them.  That orders calls of ONE context (one stream).  Calls of different contexts on one GPU run on different
+// streams: g_static_scratch_user remembers the context that used the GPU's block last, and a call on another context
+// makes its stream wait for that context's event first (events are created with the context: no allocation here).
+// Replays of a recorded graph are outside this bookkeeping: their owner keeps them apart from other contexts' calls.
 static std::mutex g_static_scratch_mu;
+constexpr int MAX_DEVICES = 64;
+static dl4s_hip_ctx *g_static_scratch_user[MAX_DEVICES];
 
 namespace {
 
@@ -430,6 +436,8 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
                          "holds %zu: use dl4s_hip_sdpa_decode_f32", (long long)BH, nsplit, need * sizeof(float),
                          NOALLOC_SCRATCH_FLOATS * sizeof(float));
             part = ctx->static_scratch;
+            dl4s_hip_ctx *last = ctx->device < MAX_DEVICES ? g_static_scratch_user[ctx->device] : nullptr;
+            if (last && last != ctx && !ctx->capturing) DL4S_HIP_TRY(hipStreamWaitEvent(ctx->stream, last->static_scratch_done, 0));
         } else {
             int rc = dl4s::ensure_scratch(ctx, need * sizeof(float));
             if (rc) return rc;
@@ -446,7 +454,12 @@ int decode_launch(dl4s_hip_ctx *ctx, const float *q, float *kcache, float *vcach
     int st = dl4s::launch_status("sdpa_decode_splitk_f32");
     if (st || nsplit == 1) return st;
     hipLaunchKernelGGL(sdpa_decode_merge_f32, dim3((unsigned)BH), dim3(MAXD), 0, ctx->stream, part, out, nsplit, row_width(d, vec), (int)d);
-    return dl4s::launch_status("sdpa_decode_merge_f32");
+    st = dl4s::launch_status("sdpa_decode_merge_f32");
+    if (st == DL4S_HIP_OK && fixed_scratch && !ctx->capturing && ctx->device < MAX_DEVICES) {
+        DL4S_HIP_TRY(hipEventRecord(ctx->static_scratch_done, ctx->stream));
+        g_static_scratch_user[ctx->device] = ctx;
+    }
+    return st;
 }
 
 }  // namespace
@@ -459,7 +472,16 @@ int decode_static_scratch_init(dl4s_hip_ctx *ctx) {
     void *p = nullptr;
     DL4S_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     ctx->static_scratch = reinterpret_cast<float *>(p);
+    DL4S_HIP_TRY(hipEventCreateWithFlags(&ctx->static_scratch_done, hipEventDisableTiming));
     return DL4S_HIP_OK;
+}
+
+// Called by dl4s_hip_destroy after the context's stream has drained.
+void decode_static_scratch_release(dl4s_hip_ctx *ctx) {
+    std::lock_guard<std::mutex> lock(g_static_scratch_mu);
+    if (ctx->device < MAX_DEVICES && g_static_scratch_user[ctx->device] == ctx) g_static_scratch_user[ctx->device] = nullptr;
+    if (ctx->static_scratch_done) (void)hipEventDestroy(ctx->static_scratch_done);
+    ctx->static_scratch_done = nullptr;
 }
 
 }  // namespace dl4s

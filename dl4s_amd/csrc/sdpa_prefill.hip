@@ -636,7 +636,10 @@ int sdpa_forward_locked(dl4s_hip_ctx *ctx, const float *q, const float *k, const
                             reinterpret_cast<uintptr_t>(out)) & 7) == 0;
     const bool w96_path = dk == dv && dk > HD && dk <= W96 &&
                           ((dk % 4 == 0 && aligned) ||
-                           (dk % 2 == 0 && aligned8 && !token_major && ((Lq + BM - 1) / BM) * B * H >= 2ll * ctx->cu_count)) &&
+                           (dk % 2 == 0 && aligned8 && !token_major && ((Lq + BM - 1) / BM) * B * H >= 2ll * ctx->cu_count &&
+                            // with row statistics only where the gradient call's rule lands on the MFMA kernels as well (it
+                            // pads such head dims, sdpa_padded_route): the statistics have the MFMA kernels' base-2 form
+                            (!stats || sdpa_padded_route(false, B, H, Lq, Lk, dk, dv)))) &&
                           Lk * (token_major ? H : 1) * dk * 4 < (1ll << 30);   // its 32-bit K/V offsets; beyond: the routes below
     // head dims above 128 up to 256: the 192- and 256-wide kernels (the gradient call evaluates sdpa_wide_route on the same
     // arguments)

@@ -93,8 +93,10 @@ struct HIP {
         static bool f = false;
         return f;
     }
-    // Fused attention only.  false: key tiles that the mask blocks entirely are skipped (their weights are exactly zero;
-    // the reference's 0 * v at such keys only differs when k or v hold NaN / Inf there).  true: every tile is visited.
+    // Fused layers only.  false: key tiles that the mask blocks entirely are skipped (their weights are exactly zero;
+    // the reference's 0 * v at such keys only differs when k or v hold NaN / Inf there) and the LayerNorm sums are
+    // added in a tree.  true: every tile is visited and the LayerNorm sums are added in the reference's sequential
+    // order, so that NaN / Inf come out where the reference has them whatever the values.
     static bool &strictMasks() {
         static bool f = false;
         return f;
@@ -281,6 +283,13 @@ struct HIP {
                                         const ShapedBuffer *residual, int64_t itemRows, const ShapedBuffer &scale, const ShapedBuffer &shift,
                                         const ShapedBuffer &result) {
             precondition(x.count() % weights.shape[0] == 0, "Matmul operands must have matching shapes");
+            if (strictMasks()) {      // the product with its epilogue, then the statistics in the reference's order
+                denseFused(x, weights, bias, activation, residual, result);
+                const int64_t rows = x.count() / weights.shape[0], D = weights.shape[1];
+                check(dl4s_hip_layernorm_reference_order_f32(context(), result.values.memory, nullptr, scale.values.memory,
+                                                             shift.values.memory, result.values.memory, rows / itemRows, itemRows, D));
+                return;
+            }
             check(dl4s_hip_dense_layernorm_f32(context(), x.values.memory, x.count() / weights.shape[0], weights.shape[0],
                                                weights.values.memory, weights.shape[1], bias ? bias->values.memory : nullptr, activation,
                                                residual ? residual->values.memory : nullptr, itemRows, scale.values.memory,
@@ -311,7 +320,7 @@ struct HIP {
         static void layerNorm(const ShapedBuffer &x, const ShapedBuffer *residual, const ShapedBuffer &scale,
                               const ShapedBuffer &shift, const ShapedBuffer &result) {
             const int64_t B = x.shape[0], D = scale.count();
-            check(dl4s_hip_layernorm_f32(context(), x.values.memory, residual ? residual->values.memory : nullptr, scale.values.memory,
+            check((strictMasks() ? dl4s_hip_layernorm_reference_order_f32 : dl4s_hip_layernorm_f32)(context(), x.values.memory, residual ? residual->values.memory : nullptr, scale.values.memory,
                                          shift.values.memory, result.values.memory, B, x.count() / (B * D), D));
         }
         // rows of `table` for device int32 tokens [batch, L], optionally * scale + positions[l]

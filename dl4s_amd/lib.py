@@ -346,6 +346,11 @@ class Context:
         _check(self.lib.dl4s_hip_layernorm_f32(self.handle, _vp(_ptr(x)), _vp(_ptr(residual)) if residual is not None else None,
                                                _vp(_ptr(scale)), _vp(_ptr(shift)), _vp(_ptr(y)), _i64(B), _i64(rows), _i64(D)))
 
+    def layernorm_reference_order(self, x, residual, scale, shift, y, B, rows, D):
+        _check(self.lib.dl4s_hip_layernorm_reference_order_f32(
+            self.handle, _vp(_ptr(x)), _vp(_ptr(residual)) if residual is not None else None, _vp(_ptr(scale)), _vp(_ptr(shift)),
+            _vp(_ptr(y)), _i64(B), _i64(rows), _i64(D)))
+
     def dense_fused(self, x, rows, in_features, weights, out_features, bias, activation, residual, y):
         _check(self.lib.dl4s_hip_dense_fused_f32(self.handle, _vp(_ptr(x)), _i64(rows), _i64(in_features), _vp(_ptr(weights)),
                                                  _i64(out_features), _vp(_ptr(bias)) if bias is not None else None, int(activation),

@@ -229,9 +229,11 @@ int dl4s_hip_sdpa_decode_lengths_f32(dl4s_hip_ctx *ctx, const float *q, const fl
  * makes no allocating or freeing runtime call.  A problem whose records do not fit - B*H pairs times the number of key
  * splits times (the row width the kernel runs at + 4) floats above 4 MiB - is refused with DL4S_HIP_EUNSUPPORTED; the split rule aims at 16 wavefronts
  * per compute unit, so on a 256-CU GPU it asks for about 2048 records (2.1 MiB at d = 256) at most and the limit guards
- * larger GPUs.  Every call on a GPU shares that GPU's block: calls on one context are ordered by its stream; calls on
- * different contexts of the same GPU that overlap in time race.  Nothing in the block has to start at zero (every
- * record a call reads was written by that call). */
+ * larger GPUs.  Every call on a GPU shares that GPU's block: calls on one context are ordered by its stream, and a call
+ * on another context of the same GPU first makes its stream wait for the last user's (an event created with the
+ * context).  What stays the caller's job: replays of a recorded graph that holds this call are outside that
+ * bookkeeping and race with calls on other contexts that overlap them in time.  Nothing in the block has to start at
+ * zero (every record a call reads was written by that call). */
 int dl4s_hip_sdpa_decode_noalloc_f32(dl4s_hip_ctx *ctx, const float *q, const float *kcache, const float *vcache,
                                      float *out, int64_t B, int64_t H, int64_t T, int64_t Tcap, int64_t d,
                                      float inv_temperature);
@@ -354,6 +356,18 @@ int dl4s_hip_stack_axis_f32(dl4s_hip_ctx *ctx, const float *const *buffers, cons
  * round.  For mean / std up to about 1 - residual sums of normalised activations - the difference is below 1e-6. */
 int dl4s_hip_layernorm_f32(dl4s_hip_ctx *ctx, const float *x, const float *residual, const float *scale,
                            const float *shift, float *result, int64_t B, int64_t rows, int64_t D);
+/* dl4s_hip_layernorm_f32 with the two sums added in the order the reference's generic CPU engine adds them
+ * (Tensor/Operators/Reduce.swift:35-46 -> Engine/CPU/CPUEngine.swift:306-378: reduced = 0, then for every row
+ * reduced = reduced + Float.sum(row), Engine/CPU/Numeric/CPUFloat.swift:256-259: dst = 0; dst += src[i] left to right;
+ * x * x is rounded before it is added, Reduce.swift:106-110).  Mean, variance and with them every output element are then
+ * the reference's to the last bit whatever the input's mean - including the rows where its one-pass variance comes out
+ * negative and the root is NaN (NN/Layer/LayerNorm.swift:62-77).  A serial sum cannot be spread over lanes: a lane
+ * adds a whole row of D elements, one lane the rows of an item, so the call costs three small launches and a chain of
+ * D + rows dependent additions (about 12 us at rows = D = 1024) where dl4s_hip_layernorm_f32 needs two passes.  Same
+ * arguments.  The reference built against MKL or Accelerate adds in those libraries' own order, which this does not
+ * restate. */
+int dl4s_hip_layernorm_reference_order_f32(dl4s_hip_ctx *ctx, const float *x, const float *residual, const float *scale,
+                                           const float *shift, float *result, int64_t B, int64_t rows, int64_t D);
 /* Tensor/Operators/Unary.swift:245-247: x * (0.5 * tanh(0.5 * (1.702 * x)) + 0.5), optional bias[D] added first
  * (Dense bias, NN/Layer/Dense.swift:64-68). */
 int dl4s_hip_bias_gelu_f32(dl4s_hip_ctx *ctx, const float *x, const float *bias, float *result, int64_t rows,

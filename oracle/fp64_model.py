@@ -19,6 +19,23 @@ def sdpa64(q, k, v, mask=None, temperature=None):
     return np.matmul(scipy.special.softmax(s, axis=-1), v)
 
 
+def sdpa_backward64(q, k, v, mask, dout, temperature=None):
+    """Gradients of sdpa64 with respect to q, k, v for an upstream gradient `dout`, in closed form:
+    dv = p^T.dout, dp = dout.v^T, ds = p.(dp - rowsum(dp.p)), dq = ds.k / T, dk = ds^T.q / T.  The mask enters as the
+    additive -1e9 penalty; a row with an unblocked key gives its blocked keys a weight of exactly 0 in fp64 as in fp32
+    (rows with every key blocked are a rounding artefact of fp32 and are not modelled here)."""
+    q, k, v, dout = f64(q), f64(k), f64(v), f64(dout)
+    T = np.sqrt(q.shape[-1]) if temperature is None else temperature
+    s = np.matmul(q, np.swapaxes(k, -1, -2)) / T
+    if mask is not None:
+        s = s - f64(mask) * 1e9
+    p = scipy.special.softmax(s, axis=-1)
+    dv = np.matmul(np.swapaxes(p, -1, -2), dout)
+    dp = np.matmul(dout, np.swapaxes(v, -1, -2))
+    ds = p * (dp - (dp * p).sum(axis=-1, keepdims=True))
+    return np.matmul(ds, k) / T, np.matmul(np.swapaxes(ds, -1, -2), q) / T, dv
+
+
 def layernorm64(x, scale, shift):
     """NN/Layer/LayerNorm.swift:62-77: statistics over all non-batch axes, eps outside the square root."""
     x = f64(x)

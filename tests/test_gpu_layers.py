@@ -120,6 +120,19 @@ def test_mha_with_other_head_dims(ctx, host, orc, fused, dk):
     assert_parity(host.mha(ctx, x, x, x, cm, attn, H, dk, dk, fused=fused), orc.mha(x, x, x, cm, attn, H, dk, dk), "MHA self dk=%d" % dk)
 
 
+def test_mha_with_a_query_far_from_zero_mean_in_strict_mode(ctx, host, orc):
+    """The residual of MultiHeadAttention is its query input; ten standard deviations from zero the one-pass variance of
+    the joint LayerNorm depends on the order of its sums beyond the parity gate.  The strict fused mode adds them in the
+    reference's order and stays inside the gate."""
+    B, L, D, H, dk = 2, 64, 64, 2, 32
+    rng = np.random.default_rng(97)
+    attn, _ = m64.make_params(rng, D, H, dk, dk, 8)
+    x = rng.standard_normal((B, L, D)).astype(np.float32)
+    q = (x + np.float32(10)).astype(np.float32)
+    ref = orc.mha(q, x, x, None, attn, H, dk, dk)
+    assert_parity(host.mha(ctx, q, x, x, None, attn, H, dk, dk, fused=2), ref, "MHA, query mean = 10 std, strict")
+
+
 def _config2():
     B, L, D, H, dk = 4, 512, 512, 8, 64
     rng = np.random.Generator(np.random.PCG64(1002))

@@ -513,6 +513,61 @@ def test_layernorm_off_centre_input(ctx, orc, rows, D):
     assert np.array_equal(nan_rows, np.isnan(got).all(axis=(1, 2)))
 
 
+def _ln_ref_order(ctx, x, scale, shift, res=None):
+    B, rows, D = x.shape
+    dx, ds, dh, dy = ctx.to_device(x), ctx.to_device(scale), ctx.to_device(shift), ctx.empty((B, rows, D))
+    dr = ctx.to_device(res) if res is not None else None
+    ctx.layernorm_reference_order(dx, dr, ds, dh, dy, B, rows, D)
+    y = dy.numpy()
+    for t in (dx, ds, dh, dy) + ((dr,) if dr is not None else ()):
+        t.release()
+    return y
+
+
+def _same_bits(a, b):
+    return np.array_equal(a.view(np.uint32), b.view(np.uint32)) or np.array_equal(a, b, equal_nan=True)
+
+
+@pytest.mark.parametrize("B,rows,D", [(3, 5, 64), (15, 1, 64), (2, 300, 68), (4, 1, 1024), (2, 1, 33), (1, 130, 1), (70, 1, 7),
+                                      (2, 64, 128), (3, 65, 63), (2, 512, 512), (1, 1024, 1024)])
+def test_layernorm_in_the_reference_order_is_the_oracle_bit_for_bit(ctx, orc, B, rows, D):
+    """The sums of dl4s_hip_layernorm_reference_order_f32 are the reference's sequential ones, every other step one
+    correctly rounded operation: the result is the oracle's to the last bit, with and without the residual."""
+    x, res = rnd(B, rows, D) * 2 + np.float32(0.3), rnd(B, rows, D)
+    scale, shift = rnd(D), rnd(D)
+    assert _same_bits(_ln_ref_order(ctx, x, scale, shift), orc.layernorm(x, scale, shift))
+    assert _same_bits(_ln_ref_order(ctx, x, scale, shift, res), orc.layernorm(x + res, scale, shift))
+
+
+@pytest.mark.parametrize("rows,D", [(1, 1024), (64, 512), (16, 256)])
+@pytest.mark.parametrize("offset", [3.0, 10.0, 1000.0])
+def test_layernorm_off_centre_input_in_the_reference_order(ctx, orc, rows, D, offset):
+    """Far from a zero mean the one-pass variance is rounding noise of the summation order; in the reference's order the
+    kernel gives the reference's numbers, NaN rows (a negative variance under the root) included."""
+    scale, shift = rnd(D), rnd(D)
+    x = rnd(8, rows, D) + np.float32(offset)
+    with np.errstate(invalid="ignore"):
+        ref = orc.layernorm(x, scale, shift)
+    assert _same_bits(_ln_ref_order(ctx, x, scale, shift), ref)
+
+
+@pytest.mark.parametrize("rows,D", [(1, 1024), (1, 512), (32, 256)])
+def test_layernorm_negative_variance_at_full_row_length_in_the_reference_order(ctx, orc, rows, D):
+    """Items whose elements sit within a few ulp of one value: the variance is zero up to the rounding of the two sums, so
+    its sign - a finite item or a NaN item - is decided by the order of every single addition.  The tree-sum kernel cannot
+    be held to the oracle here; this one must give NaN for exactly the oracle's items."""
+    rng = np.random.default_rng(rows * 7919 + D)
+    B = 64
+    base = rng.uniform(1, 2, (B, 1, 1)).astype(np.float32)
+    x = (base + rng.integers(-3, 4, (B, rows, D)).astype(np.float32) * np.spacing(base)).astype(np.float32)
+    scale, shift = np.ones(D, np.float32), np.zeros(D, np.float32)
+    with np.errstate(invalid="ignore"):
+        ref = orc.layernorm(x, scale, shift)
+    nan_items = np.isnan(ref).all(axis=(1, 2))
+    assert 4 <= nan_items.sum() <= B - 4, "the input must mix NaN items and finite ones (%d of %d)" % (nan_items.sum(), B)
+    assert _same_bits(_ln_ref_order(ctx, x, scale, shift), ref)
+
+
 def test_bias_gelu(ctx, orc):
     rows, D = 50, 129
     x, bias = rnd(rows, D) * 3, rnd(D)

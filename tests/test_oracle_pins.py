@@ -605,6 +605,23 @@ def test_sdpa_backward_against_finite_differences():
         assert abs(fd - float((grad * direction).sum())) < 1e-4
 
 
+def test_fp64_gradient_model_against_torch_autograd():
+    """fp64_model.sdpa_backward64 (the referee where the fp32 oracle's own sums run out of precision) is the closed form
+    of the gradients: torch autograd in fp64 on the same expression gives the same numbers to rounding."""
+    import torch
+    from oracle import fp64_model as m64
+    rng = np.random.default_rng(14)
+    q, dout = rng.standard_normal((2, 3, 9, 8)), rng.standard_normal((2, 3, 9, 8))
+    k, v = rng.standard_normal((2, 3, 11, 8)), rng.standard_normal((2, 3, 11, 8))
+    mask = (rng.random((9, 11)) < 0.3).astype(np.float64)
+    mask[:, 0] = 0                                  # every row keeps a key
+    tq, tk, tv = (torch.tensor(x, requires_grad=True) for x in (q, k, v))
+    o = torch.softmax(tq @ tk.transpose(-1, -2) / np.sqrt(8) - torch.tensor(mask) * 1e9, -1) @ tv
+    o.backward(torch.tensor(dout))
+    for got, ref, name in zip(m64.sdpa_backward64(q, k, v, mask, dout), (tq, tk, tv), ("dq", "dk", "dv")):
+        assert np.abs(got - ref.grad.numpy()).max() < 1e-13, name
+
+
 def test_per_token_attention_variant_of_the_transformer_oracle(orc):
     """oracle.transformer.mha_per_token is not the reference's layer; it is pinned by two properties.  With a single
     position the joint normalisation and the per-token one are the same computation (bit for bit against the pinned

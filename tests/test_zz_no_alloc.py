@@ -62,3 +62,32 @@ def test_no_alloc_decode_error_paths(ctx):
     assert e.value.code == -5
     for buf in (q, kc, out):
         buf.release()
+
+
+def test_no_alloc_decode_from_two_contexts_of_one_gpu(ctx):
+    """Two contexts (two streams) share the GPU's one fixed block: calls on them, issued back to back without a wait in
+    between, must not see each other's partial records."""
+    from dl4s_amd import lib
+    other = lib.Context(0)
+    try:
+        rng = np.random.default_rng(77)
+        cases = []
+        for c, (B, H, T) in zip((ctx, other, ctx, other), ((2, 4, 3000), (1, 6, 2500), (1, 3, 1800), (2, 4, 2900))):
+            q = rng.standard_normal((B, H, 1, 64)).astype(np.float32)
+            kc = rng.standard_normal((B, H, T, 64)).astype(np.float32)
+            vc = rng.standard_normal((B, H, T, 64)).astype(np.float32)
+            cases.append((c, q, kc, vc, c.to_device(q), c.to_device(kc), c.to_device(vc), c.empty((B, H, 1, 64)), c.empty((B, H, 1, 64))))
+        ctx.sync()
+        other.sync()
+        for _ in range(3):
+            for c, q, kc, vc, dq, dk, dv, out, _ in cases:       # alternating contexts, nothing waits
+                B, H, T = kc.shape[:3]
+                c.sdpa_decode_noalloc(dq, dk, dv, out, B, H, T, T, 64, 0.125)
+        for c, q, kc, vc, dq, dk, dv, out, ref in cases:
+            B, H, T = kc.shape[:3]
+            c.sdpa_decode(dq, dk, dv, ref, B, H, T, T, 64, 0.125)
+            assert np.array_equal(out.numpy(), ref.numpy()), "B%d H%d T%d" % (B, H, T)
+            for buf in (dq, dk, dv, out, ref):
+                buf.release()
+    finally:
+        other.close()
