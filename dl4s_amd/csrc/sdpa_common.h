@@ -398,15 +398,19 @@ inline int build_mask_args(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_
         const int64_t nqt = m.sq ? (Lq + 31) / 32 : 1, nkt = m.sk ? (Lk + 31) / 32 : 1;
         const long long total = MB * MH * nqt * nkt;
         if (total < (1ll << 31)) {
-            const size_t cls_bytes = ((size_t)total + 255) / 256 * 256;
-            const int rc = dl4s::ensure_scratch(ctx, cls_bytes + extra_bytes);
-            if (rc != DL4S_HIP_OK) return rc;
-            unsigned char *cls = static_cast<unsigned char *>(ctx->scratch);
-            if (extra && extra_bytes) { *extra = cls + cls_bytes; extra_bytes = 0; }
-            hipLaunchKernelGGL(sdpa_mask_classify, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, ctx->stream, m, (int)MB,
-                               (int)MH, (int)nqt, (int)nkt, (int)Lq, (int)Lk, total, cls);
-            const int st = dl4s::launch_status("sdpa_mask_classify");
-            if (st != DL4S_HIP_OK) return st;
+            const unsigned char *cls = mask->classes;   // prepared by dl4s_hip_mask_classify_f32 for this mask and these extents
+            if (!cls) {
+                const size_t cls_bytes = ((size_t)total + 255) / 256 * 256;
+                const int rc = dl4s::ensure_scratch(ctx, cls_bytes + extra_bytes);
+                if (rc != DL4S_HIP_OK) return rc;
+                unsigned char *own = static_cast<unsigned char *>(ctx->scratch);
+                if (extra && extra_bytes) { *extra = own + cls_bytes; extra_bytes = 0; }
+                hipLaunchKernelGGL(sdpa_mask_classify, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, ctx->stream, m, (int)MB,
+                                   (int)MH, (int)nqt, (int)nkt, (int)Lq, (int)Lk, total, own);
+                const int st = dl4s::launch_status("sdpa_mask_classify");
+                if (st != DL4S_HIP_OK) return st;
+                cls = own;
+            }
             m.cls = cls;
             m.cls_sk = m.sk ? 1 : 0;
             m.cls_sq = m.sq ? (int)nkt : 0;

@@ -213,6 +213,15 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_d64(const float *__re
     const unsigned char *cls_row = nullptr;
     if (DENSE && mask.cls) cls_row = mask.cls + (long long)b * mask.cls_sb + hh * mask.cls_sh + (long long)(min(q0, Lq - 1) >> 5) * mask.cls_sq;   // wavefronts past Lq store nothing
 
+    // the classes of 64 key tiles at a time, one per lane, read ahead of the loop: a class byte fetched inside a tile step
+    // would put a global load's latency on every step's critical path
+    int clsv = 2;
+    auto load_classes = [&](const int t0) {
+        const int t = t0 + lane;
+        clsv = t < ntiles ? (int)cls_row[(long long)t * mask.cls_sk] : 2;
+    };
+    if (DENSE && cls_row) load_classes(0);
+
     // one key tile; the LDS buffer index is a compile-time constant (the loop is unrolled by two), so every LDS address
     // in the step is a per-thread base plus a literal
     auto tile_step = [&](const int t, auto buf_c) {
@@ -221,7 +230,10 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_d64(const float *__re
         if (more) load_tile(t + 1);
         const int k0 = t * BN;
         int cls = 2;
-        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        if (DENSE && cls_row) {
+            if ((t & 63) == 0 && t > 0) load_classes(t);
+            cls = __builtin_amdgcn_readlane(clsv, t & 63) & 3;
+        }
 
         if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
             attend_tile<KIND>(Ks + buf * TILE_FLOATS + k_lds, Vs + buf * TILE_FLOATS + v_lds, qr, o0, o1, m_run, m_use, l_run, k0, q0,
@@ -374,11 +386,22 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
         load_tile(wave);
         store_tile();
     }
-    for (int t = wave; t < ntiles; t += SPLIT_WAVES) {
+    // the classes of this wavefront's next 64 tiles, one per lane, read ahead of the loop (a class byte fetched inside a
+    // step would put a global load's latency on every step's critical path)
+    int clsv = 2;
+    auto load_classes = [&](const int t0) {
+        const int t = t0 + SPLIT_WAVES * lane;
+        clsv = t < ntiles ? (int)cls_row[(long long)t * mask.cls_sk] : 2;
+    };
+    if (DENSE && cls_row) load_classes(wave);
+    for (int t = wave, j = 0; t < ntiles; t += SPLIT_WAVES, ++j) {
         const bool more = (t + SPLIT_WAVES < ntiles);
         if (more) load_tile(t + SPLIT_WAVES);
         int cls = 2;
-        if (DENSE && cls_row) cls = cls_row[t * mask.cls_sk] & 3;
+        if (DENSE && cls_row) {
+            if ((j & 63) == 0 && j > 0) load_classes(t);
+            cls = __builtin_amdgcn_readlane(clsv, j & 63) & 3;
+        }
         if (!(DENSE && skip_ones && cls == 1))
             attend_tile<KIND>(Ks + k_lds, Vs + v_lds, qr, o0, o1, m_run, m_use, l_run, t * BN, q0, qi, half, Lk, len, mrow, mask.sk, cls);
         if (more) store_tile();
@@ -748,4 +771,137 @@ extern "C" int dl4s_hip_sdpa_fwd_stats_f32(dl4s_hip_ctx *ctx, const float *q, co
                                            float inv_temperature, const dl4s_mask_desc *mask, uint32_t flags) {
     DL4S_REQUIRE(stats || B * H * Lq == 0, DL4S_HIP_EINVALID_ARG, "sdpa: stats pointer is NULL");
     return sdpa_forward(ctx, q, k, v, out, stats, B, H, Lq, Lk, d, d, inv_temperature, mask, flags);
+}
+
+// ---- tile classes of a dense mask, prepared once for many attention calls
+namespace {
+// number of class bytes of a dense mask broadcastable to [B,H,Lq,Lk]
+int mask_class_count(const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk, long long &total) {
+    DL4S_REQUIRE(mask && mask->kind == DL4S_MASK_DENSE_F32, DL4S_HIP_EINVALID_ARG, "mask classes: the descriptor is not a dense mask");
+    const int64_t full[4] = {B, H, Lq, Lk};
+    for (int i = 0; i < 4; ++i)
+        DL4S_REQUIRE(full[i] > 0 && (mask->shape[i] == 1 || mask->shape[i] == full[i]), DL4S_HIP_ESHAPE,
+                     "mask classes: mask axis %d has size %lld, expected 1 or %lld", i, (long long)mask->shape[i], (long long)full[i]);
+    total = (mask->shape[0] == 1 ? 1 : B) * (mask->shape[1] == 1 ? 1 : H) * (mask->shape[2] == 1 ? 1 : (Lq + 31) / 32) *
+            (mask->shape[3] == 1 ? 1 : (Lk + 31) / 32);
+    DL4S_REQUIRE(total < (1ll << 31), DL4S_HIP_EUNSUPPORTED, "mask classes: more than 2^31 tiles");
+    return DL4S_HIP_OK;
+}
+}  // namespace
+
+extern "C" int dl4s_hip_mask_classes_size(const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk, size_t *out_bytes) {
+    DL4S_REQUIRE(out_bytes, DL4S_HIP_EINVALID_ARG, "mask classes: NULL argument");
+    long long total = 0;
+    const int rc = mask_class_count(mask, B, H, Lq, Lk, total);
+    if (rc != DL4S_HIP_OK) return rc;
+    *out_bytes = (size_t)total;
+    return DL4S_HIP_OK;
+}
+
+extern "C" int dl4s_hip_mask_classify_f32(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                                          uint8_t *classes) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(classes, DL4S_HIP_EINVALID_ARG, "mask classes: NULL argument");
+    long long total = 0;
+    int rc = mask_class_count(mask, B, H, Lq, Lk, total);
+    if (rc != DL4S_HIP_OK) return rc;
+    DL4S_REQUIRE(mask->dense, DL4S_HIP_EINVALID_ARG, "mask classes: dense mask pointer is NULL");
+    MaskArgs m{};
+    dl4s_mask_desc plain = *mask;
+    plain.classes = nullptr;
+    rc = build_mask_args(ctx, &plain, B, H, Lq, Lk, false, m);
+    if (rc != DL4S_HIP_OK) return rc;
+    const int MB = m.sb ? (int)B : 1, MH = m.sh ? (int)H : 1;
+    const int nqt = m.sq ? (int)((Lq + 31) / 32) : 1, nkt = m.sk ? (int)((Lk + 31) / 32) : 1;
+    hipLaunchKernelGGL(sdpa_mask_classify, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, ctx->stream, m, MB, MH, nqt, nkt, (int)Lq,
+                       (int)Lk, total, classes);
+    return dl4s::launch_status("sdpa_mask_classify");
+}
+
+// ---- a dense mask whose values are exactly those of a structured kind
+namespace {
+// One workgroup per mask batch entry: the number of leading zeros of the entry's designated row (the only row of a mask
+// without a query axis, the last query's row otherwise), as the valid key count the structured kinds would need to
+// reproduce the mask.  Under the causal rule a count that reaches the last query blocks nothing beyond what the rule
+// blocks already: it is recorded as Lk.  ok[0] is set to 1 for the verification pass.
+__global__ __launch_bounds__(256) void sdpa_mask_structure_lengths(MaskArgs m, int Lq, int Lk, int causal, int *lengths, int *ok) {
+    __shared__ int first_one;
+    const int bm = blockIdx.x;
+    if (threadIdx.x == 0) first_one = Lk;
+    __syncthreads();
+    const float *row = m.dense + bm * m.sb + (causal ? (long long)(Lq - 1) * m.sq : 0);
+    const int jmax = causal ? min(Lk, Lq) : Lk;     // beyond the last query the causal rule blocks anyway
+    int mine = Lk;
+    for (int j = threadIdx.x; j < jmax; j += 256)
+        if (row[j * m.sk] != 0.0f) { mine = j; break; }
+    if (mine < Lk) atomicMin(&first_one, mine);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        lengths[bm] = first_one >= jmax ? Lk : first_one;
+        if (bm == 0) ok[0] = 1;
+    }
+}
+// Every element against the structured kind's rule: 1 where key j >= lengths[b] or (causal) j > query i, else 0.
+__global__ __launch_bounds__(256) void sdpa_mask_structure_verify(MaskArgs m, int MB, int nq, int Lk, int causal, const int *lengths,
+                                                                  int *ok) {
+    const long long total = (long long)MB * nq * Lk;
+    bool bad = false;
+    for (long long e = (long long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long long)gridDim.x * 256) {
+        const int j = (int)(e % Lk);
+        const int i = (int)((e / Lk) % nq);
+        const int bm = (int)(e / Lk / nq);
+        const float want = (j >= lengths[bm] || (causal && j > i)) ? 1.0f : 0.0f;
+        bad = bad || !(m.dense[bm * m.sb + i * m.sq + j * m.sk] == want);
+    }
+    if (bad) ok[0] = 0;
+}
+}  // namespace
+
+extern "C" int dl4s_hip_mask_describe_f32(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                                          int32_t *lengths, dl4s_mask_desc *out) {
+    DL4S_CHECK_CTX(ctx);
+    DL4S_REQUIRE(mask && out && lengths, DL4S_HIP_EINVALID_ARG, "mask describe: NULL argument");
+    DL4S_NOT_WHILE_CAPTURING(ctx);
+    *out = *mask;
+    if (mask->kind != DL4S_MASK_DENSE_F32) return DL4S_HIP_OK;
+    long long tiles = 0;
+    int rc = mask_class_count(mask, B, H, Lq, Lk, tiles);      // validates the shape
+    if (rc != DL4S_HIP_OK) return rc;
+    DL4S_REQUIRE(mask->dense, DL4S_HIP_EINVALID_ARG, "mask describe: dense mask pointer is NULL");
+    // the structured kinds know no head axis, and a query axis only through the causal rule
+    const bool has_b = mask->shape[0] != 1, has_h = mask->shape[1] != 1, has_q = mask->shape[2] != 1, has_k = mask->shape[3] != 1;
+    if (has_h || (!has_k && Lk > 1) || B > 65536 || Lq >= (1ll << 30) || Lk >= (1ll << 30)) return DL4S_HIP_OK;
+    const int causal = has_q ? 1 : 0;
+    const int MB = has_b ? (int)B : 1;
+    std::lock_guard<std::mutex> scratch_lock(ctx->scratch_mu);
+    rc = dl4s::ensure_scratch(ctx, 256);
+    if (rc != DL4S_HIP_OK) return rc;
+    int *ok = static_cast<int *>(ctx->scratch);
+    MaskArgs m{};
+    dl4s_mask_desc plain = *mask;
+    plain.classes = nullptr;
+    rc = build_mask_args(ctx, &plain, B, H, Lq, Lk, false, m);
+    if (rc != DL4S_HIP_OK) return rc;
+    // one workgroup per batch element (a mask without a batch axis has stride 0 there: every element reads the one entry)
+    hipLaunchKernelGGL(sdpa_mask_structure_lengths, dim3((unsigned)B), dim3(256), 0, ctx->stream, m, (int)Lq, (int)Lk, causal, lengths, ok);
+    rc = dl4s::launch_status("sdpa_mask_structure_lengths");
+    if (rc != DL4S_HIP_OK) return rc;
+    const int nq = has_q ? (int)Lq : 1;
+    const long long total = (long long)MB * nq * Lk;
+    const unsigned grid = (unsigned)std::min<long long>((total + 255) / 256, 4096);
+    hipLaunchKernelGGL(sdpa_mask_structure_verify, dim3(grid), dim3(256), 0, ctx->stream, m, MB, nq, (int)Lk, causal, lengths, ok);
+    rc = dl4s::launch_status("sdpa_mask_structure_verify");
+    if (rc != DL4S_HIP_OK) return rc;
+    std::vector<int32_t> host((size_t)MB + 1);
+    DL4S_HIP_TRY(hipMemcpyAsync(host.data(), lengths, sizeof(int32_t) * MB, hipMemcpyDeviceToHost, ctx->stream));
+    DL4S_HIP_TRY(hipMemcpyAsync(host.data() + MB, ok, sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
+    DL4S_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    if (!host[(size_t)MB]) return DL4S_HIP_OK;      // not a structured mask: *out is the dense descriptor
+    bool all_open = true;
+    for (int b = 0; b < MB; ++b) all_open = all_open && host[(size_t)b] >= Lk;
+    dl4s_mask_desc d{};
+    d.kind = all_open ? (causal ? DL4S_MASK_CAUSAL : DL4S_MASK_NONE) : (causal ? DL4S_MASK_CAUSAL_OR_KEY_LENGTHS : DL4S_MASK_KEY_LENGTHS);
+    d.lengths = all_open ? nullptr : lengths;
+    *out = d;
+    return DL4S_HIP_OK;
 }

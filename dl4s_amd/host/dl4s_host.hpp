@@ -208,20 +208,27 @@ struct HIP {
         }
         // Fused entry points of this backend (no counterpart in EngineType).
         // tokenMajor: q, result are [B,Lq,H,d] and k, v [B,Lk,H,d] (the projections before their permutes)
-        static void fusedAttention(const ShapedBuffer &q, const ShapedBuffer &k, const ShapedBuffer &v, const ShapedBuffer *mask,
-                                   const ShapedBuffer &result, float temperature, bool tokenMajor = false) {
+        // the dense mask tensor of a layer as the library's descriptor (right-aligned to [B,H,Lq,Lk])
+        static dl4s_mask_desc denseMaskDescriptor(const ShapedBuffer &mask) {
+            precondition(mask.dim() <= 4, "mask must be broadcastable to [batchSize, heads, queryCount, keyCount]");
             dl4s_mask_desc md{};
-            if (mask) {
-                precondition(mask->dim() <= 4, "mask must be broadcastable to [batchSize, heads, queryCount, keyCount]");
-                md.kind = DL4S_MASK_DENSE_F32;
-                md.dense = mask->values.memory;
-                for (int i = 0; i < 4; ++i) md.shape[i] = 1;
-                for (int i = 0; i < mask->dim(); ++i) md.shape[4 - mask->dim() + i] = mask->shape[i];
-            }
+            md.kind = DL4S_MASK_DENSE_F32;
+            md.dense = mask.values.memory;
+            for (int i = 0; i < 4; ++i) md.shape[i] = 1;
+            for (int i = 0; i < mask.dim(); ++i) md.shape[4 - mask.dim() + i] = mask.shape[i];
+            return md;
+        }
+        // prepared: the mask as Tensor::attentionMask left it (structured, or dense with its tile classes), or nullptr to
+        // hand the mask tensor over as it is
+        static void fusedAttention(const ShapedBuffer &q, const ShapedBuffer &k, const ShapedBuffer &v, const ShapedBuffer *mask,
+                                   const ShapedBuffer &result, float temperature, bool tokenMajor = false,
+                                   const dl4s_mask_desc *prepared = nullptr) {
+            dl4s_mask_desc md{};
+            if (mask) md = prepared ? *prepared : denseMaskDescriptor(*mask);
             const int h = tokenMajor ? 2 : 1, l = tokenMajor ? 1 : 2;
             check(dl4s_hip_sdpa_fwd_f32(context(), q.values.memory, k.values.memory, v.values.memory, result.values.memory,
                                         q.shape[0], q.shape[h], q.shape[l], k.shape[l], q.shape[3], v.shape[3],
-                                        1.0f / temperature, mask ? &md : nullptr,
+                                        1.0f / temperature, mask && md.kind != DL4S_MASK_NONE ? &md : nullptr,
                                         (strictMasks() ? DL4S_SDPA_STRICT : 0u) | (tokenMajor ? DL4S_SDPA_TOKEN_MAJOR : 0u)));
         }
         // the same with a structured mask descriptor (kind + device int32 lengths) instead of a dense mask tensor
@@ -383,9 +390,28 @@ class RecordedCalls {
 struct TensorHandle {
     ShapedBuffer values;
     std::shared_ptr<TensorHandle> parent;
+    // Not in the reference.  This buffer read as the attention mask of a [B,H,Lq,Lk] problem, prepared by the first fused
+    // attention call that receives the tensor as its mask: the structured descriptor when the values are exactly those of
+    // a causal and / or key-length mask (dl4s_hip_mask_describe_f32), else the dense descriptor with its tile classes
+    // (dl4s_hip_mask_classify_f32).  The layers of a model all receive the one mask tensor their model built
+    // (TransformerEncoder.swift:63, TransformerDecoder.swift:53-54), and tensors of this layer are never written after
+    // they are made.
+    struct PreparedMask {
+        dl4s_mask_desc descriptor{};
+        unsigned char *classes = nullptr;
+        int32_t *lengths = nullptr;
+        Shape shape;
+        int64_t extents[4] = {0, 0, 0, 0};
+        ~PreparedMask() {
+            if (classes) dl4s_hip_free(Device::context(), classes);
+            if (lengths) dl4s_hip_free(Device::context(), lengths);
+        }
+    };
+    std::unique_ptr<PreparedMask> preparedMask;
     TensorHandle(ShapedBuffer v, std::shared_ptr<TensorHandle> p) : values(std::move(v)), parent(std::move(p)) {}
     TensorHandle(const TensorHandle &) = delete;
     ~TensorHandle() {
+        preparedMask.reset();
         if (!parent) dl4s_hip_free(Device::context(), values.values.memory);
     }
 };
@@ -426,6 +452,35 @@ class Tensor {
         return out;
     }
     float item() const { return Device::Memory::getValue(buffer()); }
+    // Not in the reference.  This tensor as the attention mask of a [B,H,Lq,Lk] problem, prepared by the first call and
+    // kept with the handle (see TensorHandle::PreparedMask), so that the attention calls of every layer that receives the
+    // tensor neither classify its tiles nor, where it is a structured mask, read its values.  nullptr when the shape does
+    // not fit the problem (the attention call then reports it).
+    const dl4s_mask_desc *attentionMask(int64_t B, int64_t H, int64_t Lq, int64_t Lk) const {
+        auto &slot = handle->preparedMask;
+        if (slot && slot->shape == shape && slot->extents[0] == B && slot->extents[1] == H && slot->extents[2] == Lq && slot->extents[3] == Lk)
+            return &slot->descriptor;
+        if (dim() > 4 || B < 1) return nullptr;
+        const dl4s_mask_desc dense = Device::Engine::denseMaskDescriptor(values());
+        size_t bytes = 0;
+        if (dl4s_hip_mask_classes_size(&dense, B, H, Lq, Lk, &bytes) != DL4S_HIP_OK) return nullptr;
+        slot.reset(new TensorHandle::PreparedMask());
+        slot->shape = shape;
+        slot->extents[0] = B; slot->extents[1] = H; slot->extents[2] = Lq; slot->extents[3] = Lk;
+        void *p = nullptr;
+        Device::check(dl4s_hip_alloc(Device::context(), (size_t)B * sizeof(int32_t), &p));
+        slot->lengths = static_cast<int32_t *>(p);
+        // (refused while a call sequence is being recorded - it waits for the stream: the dense descriptor then)
+        if (dl4s_hip_mask_describe_f32(Device::context(), &dense, B, H, Lq, Lk, slot->lengths, &slot->descriptor) != DL4S_HIP_OK)
+            slot->descriptor = dense;
+        if (slot->descriptor.kind == DL4S_MASK_DENSE_F32) {
+            Device::check(dl4s_hip_alloc(Device::context(), bytes ? bytes : 1, &p));
+            slot->classes = static_cast<unsigned char *>(p);
+            Device::check(dl4s_hip_mask_classify_f32(Device::context(), &dense, B, H, Lq, Lk, slot->classes));
+            slot->descriptor.classes = slot->classes;
+        }
+        return &slot->descriptor;
+    }
 
     // view(as:) -- shares the handle; one extent may be -1 (Tensor/Operators/Shape.swift:40-67)
     Tensor view(Shape s) const {
@@ -890,7 +945,10 @@ struct ScaledDotProductAttention {
             Tensor out(Device::Memory::allocateBuffer(Shape{q.shape[0], q.shape[1], q.shape[2], v.shape[3]}));
             ShapedBuffer mb;
             if (mask) mb = mask->values();
-            Device::Engine::fusedAttention(q.values(), k.values(), v.values(), mask ? &mb : nullptr, out.values(), temperature);
+            // fused mode: the mask is looked at once per mask tensor; the hook alone hands the tensor over on every call
+            const dl4s_mask_desc *prepared =
+                mask && Device::fused() ? mask->attentionMask(q.shape[0], q.shape[1], q.shape[2], k.shape[2]) : nullptr;
+            Device::Engine::fusedAttention(q.values(), k.values(), v.values(), mask ? &mb : nullptr, out.values(), temperature, false, prepared);
             return out;
         }
         Tensor attn = (q / Tensor(temperature)).broadcastMatrixMultiplied(k, false, true);
@@ -958,7 +1016,8 @@ struct MultiHeadAttention {
             Device::Engine::fusedAttentionStructured(qp.values(), kp.values(), vp.values(), structured->kind, structured->lengthsPointer(),
                                                      a.values(), attn.temperature, true);
         else
-            Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true);
+            Device::Engine::fusedAttention(qp.values(), kp.values(), vp.values(), mask ? &mb : nullptr, a.values(), attn.temperature, true,
+                                           mask ? mask->attentionMask(batchSize, heads, queryCount, kp.shape[1]) : nullptr);
         Tensor a2 = a.view({batchSize * queryCount, heads * valueDim});
         if (!dropout.isActive) {
             // the fc product, `+ res` and the normalisation (MultiHeadAttention.swift:119-124) as one call: the product's

@@ -23,7 +23,7 @@ _i64 = C.c_int64
 
 
 class MaskDesc(C.Structure):
-    _fields_ = [("kind", C.c_int32), ("dense", _vp), ("shape", _i64 * 4), ("lengths", _vp)]
+    _fields_ = [("kind", C.c_int32), ("dense", _vp), ("shape", _i64 * 4), ("lengths", _vp), ("classes", _vp)]
 
 
 class Dl4sHipError(RuntimeError):
@@ -133,6 +133,12 @@ class Context:
         _check(self.lib.dl4s_hip_assign_h2d(self.handle, _vp(buf.ptr), a.ctypes.data_as(_vp), C.c_size_t(a.nbytes)))
         return buf
 
+    def assign_h2d(self, buf, arr):
+        """Overwrites a DeviceBuffer with a host array of the same byte size."""
+        a = np.ascontiguousarray(arr, dtype=buf.dtype)
+        assert a.nbytes == buf.nbytes
+        _check(self.lib.dl4s_hip_assign_h2d(self.handle, _vp(buf.ptr), a.ctypes.data_as(_vp), C.c_size_t(a.nbytes)))
+
     def sync(self):
         _check(self.lib.dl4s_hip_sync(self.handle))
 
@@ -183,6 +189,25 @@ class Context:
         if kind in (MASK_KEY_LENGTHS, MASK_CAUSAL_OR_KEY_LENGTHS):
             m.lengths = lengths.ptr
         return m
+
+    def mask_describe(self, mask, B, H, Lq, Lk):
+        """dl4s_hip_mask_describe_f32: returns (descriptor, lengths DeviceBuffer); the descriptor is structured when the
+        dense mask's values are exactly a structured kind's (keep the lengths buffer alive while it is used)."""
+        lengths = DeviceBuffer(self, 4 * max(int(B), 1), shape=(int(B),), dtype=np.int32)
+        out = MaskDesc()
+        _check(self.lib.dl4s_hip_mask_describe_f32(self.handle, C.byref(mask), _i64(B), _i64(H), _i64(Lq), _i64(Lk), _vp(lengths.ptr),
+                                                   C.byref(out)))
+        return out, lengths
+
+    def mask_classify(self, mask, B, H, Lq, Lk):
+        """Prepares the tile classes of a dense mask descriptor once; returns the DeviceBuffer that holds them and sets
+        mask.classes (keep the buffer alive as long as the descriptor is used)."""
+        n = C.c_size_t()
+        _check(self.lib.dl4s_hip_mask_classes_size(C.byref(mask), _i64(B), _i64(H), _i64(Lq), _i64(Lk), C.byref(n)))
+        buf = DeviceBuffer(self, max(int(n.value), 1), shape=(int(n.value),), dtype=np.uint8)
+        _check(self.lib.dl4s_hip_mask_classify_f32(self.handle, C.byref(mask), _i64(B), _i64(H), _i64(Lq), _i64(Lk), _vp(buf.ptr)))
+        mask.classes = buf.ptr
+        return buf
 
     def sdpa_fwd(self, q, k, v, out, B, H, Lq, Lk, dk, dv, inv_temperature, mask=None, flags=0):
         _check(self.lib.dl4s_hip_sdpa_fwd_f32(self.handle, _vp(_ptr(q)), _vp(_ptr(k)), _vp(_ptr(v)), _vp(_ptr(out)), _i64(B), _i64(H),

@@ -133,7 +133,33 @@ typedef struct dl4s_mask_desc {
     const float *dense;      /* DENSE_F32: device pointer, row-major, shape below */
     int64_t shape[4];        /* DENSE_F32: right-aligned to [B,H,Lq,Lk]; each entry is 1 or the full size */
     const int32_t *lengths;  /* KEY_LENGTHS kinds: device pointer to B valid lengths */
+    const uint8_t *classes;  /* DENSE_F32, optional: the mask's tile classes as dl4s_hip_mask_classify_f32 left them for
+                                this mask tensor and these extents; NULL = the attention call classifies the mask itself */
 } dl4s_mask_desc;
+
+/* Every layer of a model receives the same mask tensor (TransformerEncoder.swift:63, TransformerDecoder.swift:53-54 build
+ * it once per forward pass), and an attention call under a dense mask first sorts the mask's 32 x 32 tiles into all
+ * zeros / all ones / mixed (one small launch, about 5 us).  A caller can do that once per mask instead:
+ *   dl4s_hip_mask_classes_size      bytes of device memory the classes of this mask take (host arithmetic only)
+ *   dl4s_hip_mask_classify_f32      writes them to `classes` (device memory of that size, the caller's)
+ * and passes the pointer in dl4s_mask_desc.classes of every attention call (forward, forward with statistics,
+ * gradients) on the same mask tensor, B, H, Lq and Lk.  The classes describe the mask's values: classify again after
+ * writing into the mask.  Results are the bits of the call that classifies by itself.  No counterpart in the reference. */
+/* The masks the reference's builders make are structured: makeEncoderMasks blocks the keys from a sequence's length on,
+ * makeDecoderMasks adds the keys after the query (TransformerUtil.swift:29-50), and the layers receive them as dense
+ * tensors.  dl4s_hip_mask_describe_f32 looks at a dense mask once and, when its values are exactly those of
+ * DL4S_MASK_NONE (all zeros), DL4S_MASK_KEY_LENGTHS, DL4S_MASK_CAUSAL or DL4S_MASK_CAUSAL_OR_KEY_LENGTHS, writes that
+ * descriptor to *out, with the valid key counts in `lengths` (device int32 [B], the caller's; it must stay allocated
+ * while *out is used); any other mask comes back as the dense descriptor it was.  An attention call gives the same bits
+ * under either descriptor, and the structured one reads no mask values.  The call waits for the context's stream and
+ * reads B + 1 integers back, so it is meant to run once per mask tensor (not inside a recorded sequence); describe
+ * again after writing into the mask.  A mask with a head axis, or a query axis without a key axis, is not looked at.
+ * No counterpart in the reference. */
+int dl4s_hip_mask_describe_f32(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                               int32_t *lengths, dl4s_mask_desc *out);
+int dl4s_hip_mask_classes_size(const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk, size_t *out_bytes);
+int dl4s_hip_mask_classify_f32(dl4s_hip_ctx *ctx, const dl4s_mask_desc *mask, int64_t B, int64_t H, int64_t Lq, int64_t Lk,
+                               uint8_t *classes);
 
 /* flags for dl4s_hip_sdpa_fwd_f32 */
 #define DL4S_SDPA_STRICT 1u /* visit every key tile even where the mask blocks all of it.  Without it fully blocked

@@ -155,6 +155,16 @@ def test_config2_mha_layer_causal(ctx, host, orc, fused):
     assert np.array_equal(host.mha(ctx, x, x, x, dmask, attn, H, dk, dk, fused=fused), got)
 
 
+def test_repeated_layer_calls_on_one_mask_tensor(ctx, host):
+    """In fused mode the mask tensor's tile classes are formed by the first attention call that receives it and serve the
+    later ones: four calls of the layer on the same tensors give the bits of one call."""
+    B, L, D, H, dk, x, attn, mask = _config2()
+    for fused in (1, 2):
+        once = host.mha(ctx, x, x, x, mask, attn, H, dk, dk, fused=fused)
+        again, _ = host.mha(ctx, x, x, x, mask, attn, H, dk, dk, fused=fused, iters=3)
+        assert np.array_equal(once, again)
+
+
 def test_config3_encoder_block_padding_mask(ctx, host, orc):
     """TransformerEncoderBlock fp32, B8 L1024 D1024 H16 F4096, sigmoid-GELU, LayerNorm, key-length mask U[512,1024].
     The fused mode is checked against the fp64 model on the whole batch (the single-threaded oracle needs

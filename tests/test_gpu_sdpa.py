@@ -902,6 +902,132 @@ def test_dense_mask_with_uniform_and_mixed_tiles(ctx, orc, mshape):
     assert np.array_equal(got, got_tm)
 
 
+@pytest.mark.parametrize("mshape", ["full", "b1qk", "qk", "b11k", "k", "1hq1"])
+@pytest.mark.parametrize("d", [64, 32, 96, 128, 192])
+def test_prepared_mask_classes_give_the_bits_of_the_call_that_classifies(ctx, mshape, d):
+    """dl4s_hip_mask_classify_f32 once, then attention calls that take the classes from the descriptor: the same bits as
+    calls that classify the mask themselves, with and without tile skipping, on every broadcast shape; after the mask
+    changes, classifying again follows it."""
+    from dl4s_amd import lib
+    B, H, Lq, Lk = 2, 3, 150, 200
+    rng = np.random.default_rng(zlib.crc32(repr(("classes", mshape, d)).encode()))
+    q, k, v = rand(rng, B, H, Lq, d), rand(rng, B, H, Lk, d), rand(rng, B, H, Lk, d)
+    shape = {"full": (B, H, Lq, Lk), "b1qk": (B, 1, Lq, Lk), "qk": (Lq, Lk), "b11k": (B, 1, 1, Lk), "k": (Lk,), "1hq1": (1, H, Lq, 1)}[mshape]
+
+    def make_mask():
+        m = np.zeros(shape, np.float32)
+        m4 = m.reshape((1,) * (4 - m.ndim) + m.shape)
+        for qi in range(0, m4.shape[2], 32):
+            for ki in range(0, m4.shape[3], 32):
+                c = rng.integers(0, 4)
+                blk = m4[:, :, qi:qi + 32, ki:ki + 32]
+                blk[...] = {0: 0.0, 1: 1.0, 3: 0.5}.get(int(c), 0.0)
+                if c == 2:
+                    blk[...] = rng.random(blk.shape) < 0.5
+        return m
+
+    bufs = [ctx.to_device(x) for x in (q, k, v)]
+    out = ctx.empty((B, H, Lq, d))
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+    md = ctx.to_device(make_mask())
+    for round_ in range(2):
+        plain = ctx.mask_desc(lib.MASK_DENSE, dense=md)
+        prepared = ctx.mask_desc(lib.MASK_DENSE, dense=md)
+        classes = ctx.mask_classify(prepared, B, H, Lq, Lk)
+        assert prepared.classes
+        for flags in (0, lib.SDPA_STRICT):
+            ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], out, B, H, Lq, Lk, d, d, rT, plain, flags)
+            want = out.numpy()
+            for _ in range(2):      # the classes serve any number of calls
+                ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], out, B, H, Lq, Lk, d, d, rT, prepared, flags)
+                assert np.array_equal(out.numpy(), want, equal_nan=True)
+        classes.release()
+        ctx.assign_h2d(md, make_mask())     # a new mask in the same buffer: its classes are formed again
+    # descriptors that have no classes
+    import ctypes
+    n, causal = ctypes.c_size_t(), ctx.mask_desc(lib.MASK_CAUSAL)
+    i64 = ctypes.c_int64
+    assert ctx.lib.dl4s_hip_mask_classes_size(ctypes.byref(causal), i64(1), i64(1), i64(8), i64(8), ctypes.byref(n)) != 0
+    for b in bufs + [out, md]:
+        b.release()
+
+
+DESCRIBE_CASES = [  # name, B, H, Lq, Lk, expected kind
+    ("zeros_b11k", 3, 2, 40, 50, "none"), ("zeros_qk", 2, 3, 70, 90, "dense"),     # a query axis is only looked at under the causal rule
+    ("lens_b11k", 4, 2, 130, 200, "lens"), ("lens_k", 2, 2, 33, 64, "lens"), ("lens_with_empty_and_full", 3, 2, 65, 65, "lens"),
+    ("causal_qk", 2, 3, 150, 150, "causal"), ("causal_wide", 1, 2, 100, 260, "causal"), ("causal_tall", 1, 2, 260, 100, "causal"),
+    ("causal_11qk", 2, 2, 64, 64, "causal"),
+    ("decoder_b1qk", 4, 2, 130, 130, "causal_lens"), ("decoder_with_empty_sequence", 3, 2, 96, 96, "causal_lens"),
+    ("random", 2, 2, 70, 90, "dense"), ("half_causal", 1, 2, 64, 64, "dense"), ("lens_not_monotone", 2, 2, 40, 50, "dense"),
+    ("head_axis", 2, 3, 40, 50, "dense"), ("causal_shifted", 1, 2, 64, 64, "dense"), ("q_axis_only", 1, 2, 64, 64, "dense"),
+]
+
+
+@pytest.mark.parametrize("case", DESCRIBE_CASES, ids=[c[0] for c in DESCRIBE_CASES])
+def test_dense_masks_described_as_structured_kinds(ctx, case):
+    """dl4s_hip_mask_describe_f32 finds the structured kind whose values a dense mask holds exactly (the masks of
+    makeEncoderMasks / makeDecoderMasks, TransformerUtil.swift:29-50) and leaves every other mask dense; the attention call
+    gives the same bits under the descriptor it returns as under the mask tensor, with and without tile skipping."""
+    from dl4s_amd import lib
+    name, B, H, Lq, Lk, want = case
+    rng = np.random.default_rng(zlib.crc32(repr(case).encode()))
+    lens = rng.integers(1, Lk, size=B)
+    want_lens = None
+    if name.startswith("zeros"):
+        mask = np.zeros((Lq, Lk) if name == "zeros_qk" else (B, 1, 1, Lk), np.float32)
+    elif name == "lens_b11k":
+        mask, want_lens = lengths_mask(lens, Lk), lens
+    elif name == "lens_k":
+        mask, want_lens = lengths_mask(lens[:1], Lk).reshape(Lk), np.full(B, lens[0])
+    elif name == "lens_with_empty_and_full":
+        lens = np.array([0, Lk, 7])
+        mask, want_lens = lengths_mask(lens, Lk), lens
+    elif name in ("causal_qk", "causal_wide", "causal_tall"):
+        mask = causal_mask(Lq, Lk)
+    elif name == "causal_11qk":
+        mask = causal_mask(Lq, Lk).reshape(1, 1, Lq, Lk)
+    elif name == "decoder_b1qk":
+        lens[0] = Lk                                    # one full sequence: recorded as Lk
+        mask, want_lens = np.maximum(causal_mask(Lq, Lk)[None, None], lengths_mask(lens, Lk)), lens
+    elif name == "decoder_with_empty_sequence":
+        lens = np.array([0, 50, Lk])
+        mask, want_lens = np.maximum(causal_mask(Lq, Lk)[None, None], lengths_mask(lens, Lk)), lens
+    elif name == "random":
+        mask = (rng.random((B, 1, Lq, Lk)) < 0.3).astype(np.float32)
+    elif name == "half_causal":
+        mask = causal_mask(Lq, Lk) * np.float32(0.5)
+    elif name == "lens_not_monotone":
+        mask = lengths_mask(lens, Lk)
+        mask[1, 0, 0, Lk - 1] = 0.0
+    elif name == "head_axis":
+        mask = np.broadcast_to(lengths_mask(lens, Lk), (B, H, 1, Lk)).copy()
+    elif name == "causal_shifted":
+        mask = np.triu(np.ones((Lq, Lk), np.float32), k=2)
+    else:
+        mask = np.zeros((Lq, 1), np.float32)
+    md = ctx.to_device(mask)
+    dense = ctx.mask_desc(lib.MASK_DENSE, dense=md)
+    desc, lbuf = ctx.mask_describe(dense, B, H, Lq, Lk)
+    kinds = {"none": lib.MASK_NONE, "lens": lib.MASK_KEY_LENGTHS, "causal": lib.MASK_CAUSAL, "causal_lens": lib.MASK_CAUSAL_OR_KEY_LENGTHS,
+             "dense": lib.MASK_DENSE}
+    assert desc.kind == kinds[want], (desc.kind, want)
+    if want in ("lens", "causal_lens"):
+        assert desc.lengths == lbuf.ptr
+        assert np.array_equal(lbuf.numpy(), np.asarray(want_lens, np.int32))
+    if want == "dense":
+        assert desc.dense == md.ptr and tuple(desc.shape) == tuple(dense.shape)
+    q, k, v = rand(rng, B, H, Lq, 64), rand(rng, B, H, Lk, 64), rand(rng, B, H, Lk, 64)
+    bufs = [ctx.to_device(x) for x in (q, k, v)]
+    out = ctx.empty((B, H, Lq, 64))
+    for flags in (0, lib.SDPA_STRICT):
+        ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], out, B, H, Lq, Lk, 64, 64, 0.125, dense, flags)
+        ref = out.numpy()
+        ctx.sdpa_fwd(bufs[0], bufs[1], bufs[2], out, B, H, Lq, Lk, 64, 64, 0.125, None if desc.kind == lib.MASK_NONE else desc, flags)
+        assert np.array_equal(out.numpy(), ref, equal_nan=True)
+    for b in bufs + [out, md, lbuf]:
+        b.release()
+
+
 def test_tensors_beyond_2_31_elements(ctx, orc):
     """32768 (batch, head) pairs of 1024 x 64: every tensor holds 2^31 elements (8 GiB), so any 32-bit element index in
     the kernels or their launch arithmetic would wrap.  The tensors are filled on the device from one 64-pair block

@@ -408,6 +408,31 @@ def test_gradients_of_fully_blocked_rows_with_large_scores(ctx, orc, d, mask_kin
         assert_parity(dv, rv, "dv d=%d %s" % (d, mask_kind))
 
 
+@pytest.mark.parametrize("d", [64, 32, 128])
+def test_prepared_mask_classes_in_the_gradient_calls(ctx, d):
+    """The forward call with statistics and the gradient call take a dense mask's tile classes from the descriptor
+    (dl4s_hip_mask_classify_f32, once) and give the bits of the calls that classify the mask themselves."""
+    from dl4s_amd import lib
+    B, H, L = 2, 4, 260
+    rng = np.random.default_rng(zlib.crc32(repr(("bwd classes", d)).encode()))
+    q, k, v, dout = (rand(rng, B, H, L, d) for _ in range(4))
+    lens = np.array([L, 100])
+    mask = np.maximum(causal_mask(L, L)[None, None], (np.arange(L)[None, None, None, :] >= lens[:, None, None, None]).astype(np.float32))
+    bufs = [ctx.to_device(x) for x in (q, k, v, dout)]
+    md = ctx.to_device(mask)
+    outs = [[ctx.empty((B, H, L, d)) for _ in range(4)] + [ctx.empty((B, H, L, 2))] for _ in range(2)]
+    rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
+    descs = [ctx.mask_desc(lib.MASK_DENSE, dense=md), ctx.mask_desc(lib.MASK_DENSE, dense=md)]
+    classes = ctx.mask_classify(descs[1], B, H, L, L)
+    for (out, dq_, dk_, dv_, stats), desc in zip(outs, descs):
+        ctx.sdpa_fwd_stats(bufs[0], bufs[1], bufs[2], out, stats, B, H, L, L, d, rT, desc, 0)
+        ctx.sdpa_bwd(bufs[0], bufs[1], bufs[2], out, stats, bufs[3], dq_, dk_, dv_, B, H, L, L, d, rT, desc, 0)
+    for a, b in zip(outs[0], outs[1]):
+        assert np.array_equal(a.numpy(), b.numpy(), equal_nan=True)
+    for b in bufs + [md, classes] + outs[0] + outs[1]:
+        b.release()
+
+
 def test_backward_argument_errors(ctx):
     from dl4s_amd import lib
     a = ctx.empty((1, 1, 4, 300))
