@@ -58,13 +58,14 @@ void load(PointwiseFeedForward &f, const dl4s_host_ffn_params *p) {
     f.dropout.isActive = false;
 }
 
-// runs fn `iters` times between the stream timer's begin/end and returns the last result
+// runs fn `iters` times between the stream timer's begin/end and returns the last result; a timed run is preceded by as
+// many untimed calls (allocations then come from the pool, and the GPU, which needs some 20 ms of load after the idle gap
+// of the uploads to reach its clocks, is at speed when the timer starts)
 Tensor timed(dl4s_hip_ctx *ctx, int iters, float *out_ms, const std::function<Tensor()> &fn) {
     if (iters < 1) iters = 1;
     Tensor r;
     if (out_ms) {
-        r = fn();  // warm-up: allocations come from the pool afterwards
-        HIP::check(dl4s_hip_sync(ctx));
+        for (int i = 0; i < iters; ++i) r = fn();
         HIP::check(dl4s_hip_timer_begin(ctx));
     }
     for (int i = 0; i < iters; ++i) r = fn();

@@ -2,7 +2,8 @@
  * dl4s_host.h -- C entry points of libdl4s_host.so, the C++ host layer that mirrors DL4S's Tensor and
  * layer interfaces (dl4s_amd/host/dl4s_host.hpp) on top of libdl4s_hip.so.  They exist so that a test
  * or benchmark harness in any language can drive whole layers: every function uploads its host inputs,
- * runs the layer `iters` times on the GPU (timed with the context's stream timer when out_ms != NULL),
+ * runs the layer `iters` times on the GPU (when out_ms != NULL: `iters` untimed calls first, then `iters` calls timed
+ * with the context's stream timer),
  * downloads the last result and returns 0, or -1 with the text in dl4s_host_last_error().
  *
  * `fused` selects the execution mode of the host layer: 0 issues exactly the engine primitive calls the
