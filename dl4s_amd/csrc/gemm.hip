@@ -172,7 +172,9 @@ constexpr unsigned OUTSIDE = 0x80000000u;   // an offset beyond every descriptor
 // One operand of the fast kernels.  XI = MFMA tiles per wavefront along this operand's extent (tile extent T = 64*XI);
 // KROWS = true for the K x rows memory layout; KT = depth of a K tile (16 or 32).  A K tile of 32 is contracted as two
 // halves of 16 one after the other, so that an output element sees its products in the same order whatever KT is.
-template <int XI, bool KROWS, int KT>
+// SLOTS = register sets for tiles in flight: with two, the tile after the next is requested while the next one waits in
+// registers for its turn in LDS, so a load has two K steps to arrive.
+template <int XI, bool KROWS, int KT, int SLOTS = 1>
 struct FastOperand {
     static constexpr int T = 64 * XI;
     static constexpr int LS = KT + 4;            // row stride of a [row][k] tile (floats): 128-bit reads of 8 rows on distinct banks
@@ -184,7 +186,7 @@ struct FastOperand {
     __amdgpu_buffer_rsrc_t rsrc;
     unsigned off[NV];
     unsigned step;          // byte step of one K tile
-    f32x4 st[NV];
+    f32x4 st[SLOTS][NV];
     int kq;                 // rows x K: the thread's k quad
     bool ragged_k;
     int K;
@@ -211,22 +213,24 @@ struct FastOperand {
             step = (unsigned)KT * 4u;
         }
     }
+    template <int SLOT = 0>
     __device__ __forceinline__ void load(int kt) {
         // rows x K on the last K step of a ragged K: quads at or past K lie inside the next row, so they are sent outside
         const bool past = !KROWS && ragged_k && (kt * KT + kq >= K);
 #pragma unroll
         for (int i = 0; i < NV; ++i)
-            st[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(past ? OUTSIDE : off[i] + kt * step), 0, 0));
+            st[SLOT][i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(past ? OUTSIDE : off[i] + kt * step), 0, 0));
     }
+    template <int SLOT = 0>
     __device__ __forceinline__ void store(int buf, int tid) {
         if (KROWS) {
             const int krow = tid / Q, rq = (tid % Q) * 4;
 #pragma unroll
-            for (int i = 0; i < NV; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * KT + krow + PASS_ROWS * i) * (T + 4) + rq) = st[i];
+            for (int i = 0; i < NV; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * KT + krow + PASS_ROWS * i) * (T + 4) + rq) = st[SLOT][i];
         } else {
             const int row = tid / QK;
 #pragma unroll
-            for (int i = 0; i < NV; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * T + row + RP * i) * LS + kq) = st[i];
+            for (int i = 0; i < NV; ++i) *reinterpret_cast<f32x4 *>(lds + (buf * T + row + RP * i) * LS + kq) = st[SLOT][i];
         }
     }
     // rows x K: the lane's fragment of tile x for half h2 of the K tile (k = 16*h2 + 8*half .. + 7)
@@ -248,8 +252,12 @@ struct FastOperand {
 template <int MI, int NI, bool EPI, bool TA, bool TB, int KT>
 __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_mfma_fast(GemmArgs g) {
     constexpr int TM = 64 * MI, TN = 64 * NI;       // workgroup tile
-    using OpA = FastOperand<MI, TA, KT>;             // A is M x K in memory unless transposed
-    using OpB = FastOperand<NI, !TB, KT>;            // B is K x N in memory unless transposed
+    // The 64 x 64 form runs one to three wavefronts per SIMD and a K step of 16 MFMAs (0.4 us) is shorter than a load's way
+    // through L2: it keeps two tiles in flight ([2048,512]x[512,512] 15.1 -> 14.0 us, with the LayerNorm sums 21.0 -> 19.7 us,
+    // three such products in one launch 29.9 -> 29.2 us).  Same order of additions, same bits.
+    constexpr int SLOTS = (MI == 1 && NI == 1 && KT == 32) ? 2 : 1;
+    using OpA = FastOperand<MI, TA, KT, SLOTS>;      // A is M x K in memory unless transposed
+    using OpB = FastOperand<NI, !TB, KT, SLOTS>;     // B is K x N in memory unless transposed
     extern __shared__ __align__(16) float gemm_lds[];
     float *As = gemm_lds, *Bs = gemm_lds + OpA::LDS_FLOATS;
     const int tid = threadIdx.x;
@@ -303,17 +311,32 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
     const int ktiles_all = (g.K + KT - 1) / KT;
     const int kt_first = g.tri == 2 ? min(m0 / KT, ktiles_all) : 0;      // (a tile past the end reads as zeros)
     const int ktiles = g.tri == 3 ? min(ktiles_all, (m0 + TM + KT - 1) / KT) : ktiles_all;
-    opa.load(kt_first);
-    opb.load(kt_first);
-    opa.store(0, tid);
-    opb.store(0, tid);
+    opa.template load<0>(kt_first);
+    opb.template load<0>(kt_first);
+    if (SLOTS == 2) {
+        // the second tile is requested with the first and both are waited for (they arrive together): entering the loop
+        // with loads pending in another order than the loop's own made the compiler wait, at the head of every second
+        // step, for loads that step does not need yet
+        opa.template load<SLOTS - 1>(kt_first + 1);
+        opb.template load<SLOTS - 1>(kt_first + 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0)
+    }
+    opa.template store<0>(0, tid);
+    opb.template store<0>(0, tid);
+    // (with two register sets the loads and the LDS stores of a step are unconditional: a tile past the end reads as zeros
+    // or as values nobody uses, and on straight-line code the compiler's wait before the stores covers exactly the older
+    // set's loads - with the loads under a condition it waited for the newest ones too)
     __syncthreads();
     // one K step; the LDS buffer index is a compile-time constant (the loop below is unrolled by two) so that every LDS
     // address is a per-thread base plus a literal
     auto k_step = [&](const int kt, auto buf_c) {
         constexpr int buf = decltype(buf_c)::value;
         const bool more = kt + 1 < ktiles;
-        if (more) { opa.load(kt + 1); opb.load(kt + 1); }
+        if (SLOTS == 2) {      // tile kt + 1 is in the other register set already; set `buf` (tile kt, stored a step ago) is free
+            opa.template load<(SLOTS == 2 ? buf : 0)>(kt + 2);
+            opb.template load<(SLOTS == 2 ? buf : 0)>(kt + 2);
+            __builtin_amdgcn_sched_barrier(0);      // the requests go out before the step's MFMAs, not after them
+        } else if (more) { opa.template load<0>(kt + 1); opb.template load<0>(kt + 1); }
 #pragma unroll
         for (int h2 = 0; h2 < KT / 16; ++h2) {
             f32x4 af[MI][2], bf[NI][2];
@@ -341,12 +364,25 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
             }
         }
-        if (more) { opa.store(buf ^ 1, tid); opb.store(buf ^ 1, tid); }
+        if (more || SLOTS == 2) { opa.template store<(SLOTS == 2 ? (buf ^ 1) : 0)>(buf ^ 1, tid); opb.template store<(SLOTS == 2 ? (buf ^ 1) : 0)>(buf ^ 1, tid); }
         __syncthreads();
     };
-    for (int kt = kt_first; kt < ktiles; kt += 2) {
-        k_step(kt, std::integral_constant<int, 0>{});
-        if (kt + 1 < ktiles) k_step(kt + 1, std::integral_constant<int, 1>{});
+    if (SLOTS == 2) {
+        // The odd last step stands outside the loop: with an exit between the two steps of the body the compiler sees a way
+        // from the first step back to the loop's head, and makes every first step wait for the loads the second one
+        // issued - which is what the second register set is there to avoid.  (The 128 x 128 form keeps the plain loop:
+        // peeled, [8192,1024]x[1024,1024] ran 135 instead of 132 us.)
+        int kt = kt_first;
+        for (; kt + 1 < ktiles; kt += 2) {
+            k_step(kt, std::integral_constant<int, 0>{});
+            k_step(kt + 1, std::integral_constant<int, 1>{});
+        }
+        if (kt < ktiles) k_step(kt, std::integral_constant<int, 0>{});
+    } else {
+        for (int kt = kt_first; kt < ktiles; kt += 2) {
+            k_step(kt, std::integral_constant<int, 0>{});
+            if (kt + 1 < ktiles) k_step(kt + 1, std::integral_constant<int, 1>{});
+        }
     }
 
     // accumulator register r of a transposed 32x32 tile: row m = lane % 32, column n = 8*(r/4) + 4*half + r%4
