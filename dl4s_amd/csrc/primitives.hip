@@ -294,6 +294,20 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
                                                      long long D, int nblk) {
     __shared__ float sm[2 * TPB / 64];
     const long long b = blockIdx.y;
+    const float *xp = x + b * n;
+    const float *rp = res ? res + b * n : nullptr;
+    float *yp = y + b * n;
+    // the column of element i advances by a constant per iteration: no division in the loop
+    const long long step = (long long)gridDim.x * TPB * 4, dstep = step % D;
+    long long i = ((long long)blockIdx.x * TPB + threadIdx.x) * 4, d = i % D;
+    // the thread's first two pieces are requested before the statistics are formed (the launcher sizes the grid for two
+    // per thread): their way through memory overlaps the reduction instead of following it
+    f32x4 pre[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    if (VEC) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            if (i + u * step < n) pre[u] = ln_load4(xp, rp, i + u * step);
+    }
     float s = 0.f, ss = 0.f;
     if ((int)threadIdx.x < nblk) {      // nblk <= TPB: one partial pair per thread, summed in a fixed order
         s = part[(b * nblk + threadIdx.x) * 2];
@@ -304,13 +318,14 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     const float mean = __fmul_rn(s, rN);
     const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
     const float rden = __fdiv_rn(1.0f, __fadd_rn(sqrt_rn(var), 1e-5f));
-    const float *xp = x + b * n;
-    const float *rp = res ? res + b * n : nullptr;
-    float *yp = y + b * n;
     if (VEC) {
-        // the column of element i advances by a constant per iteration: no division in the loop
-        const long long step = (long long)gridDim.x * TPB * 4, dstep = step % D;
-        long long i = ((long long)blockIdx.x * TPB + threadIdx.x) * 4, d = i % D;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            if (i < n) *reinterpret_cast<f32x4 *>(yp + i) = ln_norm4(pre[u], mean, rden, scale, shift, d);
+            i += step;
+            d += dstep;
+            if (d >= D) d -= D;
+        }
         for (; i < n; i += step) {
             *reinterpret_cast<f32x4 *>(yp + i) = ln_norm4(ln_load4(xp, rp, i), mean, rden, scale, shift, d);
             d += dstep;

@@ -945,9 +945,8 @@ struct ScaledDotProductAttention {
             Tensor out(Device::Memory::allocateBuffer(Shape{q.shape[0], q.shape[1], q.shape[2], v.shape[3]}));
             ShapedBuffer mb;
             if (mask) mb = mask->values();
-            // fused mode: the mask is looked at once per mask tensor; the hook alone hands the tensor over on every call
-            const dl4s_mask_desc *prepared =
-                mask && Device::fused() ? mask->attentionMask(q.shape[0], q.shape[1], q.shape[2], k.shape[2]) : nullptr;
+            // the mask is looked at once per mask tensor (as the Swift hook does through its table of mask buffers)
+            const dl4s_mask_desc *prepared = mask ? mask->attentionMask(q.shape[0], q.shape[1], q.shape[2], k.shape[2]) : nullptr;
             Device::Engine::fusedAttention(q.values(), k.values(), v.values(), mask ? &mb : nullptr, out.values(), temperature, false, prepared);
             return out;
         }

@@ -94,7 +94,19 @@ public struct HIPMemory: MemoryOperatorsType {
     /// Stream-ordered: the block returns to the library's pool at once, later work on the stream may reuse it
     /// (TensorHandle.deinit frees right after the last use was enqueued, Tensor/Tensor.swift:38-42).
     public static func free<Element>(_ buffer: Buffer<Element, HIP>) {
+        forgetPreparedMasks(in: buffer)
         hipCheck(dl4s_hip_free(HIP.context, buffer.memory.ptr))
+    }
+
+    /// What the fused attention calls remember about mask buffers (HIPPreparedMasks) describes the buffers' values: it goes
+    /// when the allocation is freed or written through this type.
+    @inline(__always)
+    static func forgetPreparedMasks<Element>(in buffer: Buffer<Element, HIP>) {
+        if HIPPreparedMasks.entries.isEmpty { return }
+        var bytes = 0
+        if dl4s_hip_get_size(HIP.context, buffer.memory.ptr, &bytes) == 0 {
+            HIPPreparedMasks.forget(from: buffer.memory.ptr, bytes: bytes)
+        }
     }
 
     public static func free<Element>(_ buffer: ShapedBuffer<Element, HIP>) {
@@ -102,10 +114,12 @@ public struct HIPMemory: MemoryOperatorsType {
     }
 
     public static func assign<Element>(from source: UnsafeBufferPointer<Element>, to destination: Buffer<Element, HIP>, count: Int) {
+        forgetPreparedMasks(in: destination)
         hipCheck(dl4s_hip_assign_h2d(HIP.context, destination.memory.ptr, source.baseAddress, count * MemoryLayout<Element>.stride))
     }
 
     public static func assign<Element>(from source: Buffer<Element, HIP>, to destination: Buffer<Element, HIP>, count: Int) {
+        forgetPreparedMasks(in: destination)
         hipCheck(dl4s_hip_assign_d2d(HIP.context, destination.memory.ptr, source.memory.ptr, count * MemoryLayout<Element>.stride))
     }
 
@@ -158,6 +172,7 @@ public struct HIPMemory: MemoryOperatorsType {
     }
 
     public static func set<Element>(slice: [Int?], of buffer: Buffer<Element, HIP>, with dstShape: [Int], from source: Buffer<Element, HIP>, with sourceShape: [Int]) {
+        forgetPreparedMasks(in: buffer)
         let countDelta = dstShape.count - slice.filter { $0 != nil }.count
         precondition(sourceShape.count == countDelta, "Dimensionality of source must be equal to dimensionality of destination minus number of knowns in slice")
         let padded = slice + [Int?](repeating: nil, count: dstShape.count - slice.count)
@@ -167,6 +182,7 @@ public struct HIPMemory: MemoryOperatorsType {
     }
 
     public static func set<Element>(slice: [Range<Int>?], of buffer: Buffer<Element, HIP>, with dstShape: [Int], from source: Buffer<Element, HIP>, with sourceShape: [Int]) {
+        forgetPreparedMasks(in: buffer)
         precondition(sourceShape.count == dstShape.count, "Dimensionality of source must be equal to dimensionality of destination")
         let padded = slice + [Range<Int>?](repeating: nil, count: dstShape.count - slice.count)
         let start = padded.map { Int64($0?.lowerBound ?? 0) }
@@ -175,6 +191,7 @@ public struct HIPMemory: MemoryOperatorsType {
     }
 
     public static func setPointee<Element>(of buffer: Buffer<Element, HIP>, to newValue: Element) {
+        forgetPreparedMasks(in: buffer)
         var value = newValue
         withUnsafePointer(to: &value) { pointer in
             hipCheck(dl4s_hip_assign_h2d(HIP.context, buffer.memory.ptr, pointer, MemoryLayout<Element>.stride))

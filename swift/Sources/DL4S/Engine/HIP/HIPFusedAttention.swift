@@ -50,21 +50,30 @@ extension HIPEngine {
     public static var hasFusedAttention: Bool { return true }
 
     /// The layer's dense float mask as the library's descriptor: right-aligned to [batch, heads, queries, keys], size-1 axes
-    /// broadcast (Util.swift:40-45).  The library classifies the mask's 32 x 32 tiles once per call and reads mask values
-    /// only in tiles that are neither all zeros nor all ones, so the masks of TransformerUtil.swift:29-50 cost about what a
-    /// structured descriptor costs.
-    static func descriptor<N: NumericType>(for mask: ShapedBuffer<N, HIP>?) -> dl4s_mask_desc {
-        var descriptor = dl4s_mask_desc()
-        guard let mask = mask else {
-            descriptor.kind = Int32(DL4S_MASK_NONE.rawValue)
-            return descriptor
-        }
+    /// broadcast (Util.swift:40-45).
+    static func denseDescriptor<N: NumericType>(for mask: ShapedBuffer<N, HIP>) -> dl4s_mask_desc {
         precondition(mask.dim <= 4, "attention masks have at most 4 axes")
         let padded = [Int](repeating: 1, count: 4 - mask.dim) + mask.shape
+        var descriptor = dl4s_mask_desc()
         descriptor.kind = Int32(DL4S_MASK_DENSE_F32.rawValue)
         descriptor.dense = UnsafePointer(f(mask))
         descriptor.shape = (Int64(padded[0]), Int64(padded[1]), Int64(padded[2]), Int64(padded[3]))
         return descriptor
+    }
+
+    /// The descriptor an attention call passes for `mask`.  Every layer of a model receives the one mask tensor its model
+    /// built (TransformerEncoder.swift:63, TransformerDecoder.swift:53-54), so a mask buffer is looked at once
+    /// (`HIPPreparedMasks`): when its values are exactly a causal and / or key-length mask - what makeEncoderMasks and
+    /// makeDecoderMasks build, TransformerUtil.swift:29-50 - the calls get the structured descriptor and read no mask
+    /// values; any other mask keeps its dense descriptor together with its tile classes, so that later calls skip the
+    /// classification.  The results are the bits of the dense descriptor either way.
+    static func descriptor<N: NumericType>(for mask: ShapedBuffer<N, HIP>?, batchSize: Int, heads: Int, queryCount: Int, keyCount: Int) -> dl4s_mask_desc {
+        guard let mask = mask else {
+            var none = dl4s_mask_desc()
+            none.kind = Int32(DL4S_MASK_NONE.rawValue)
+            return none
+        }
+        return HIPPreparedMasks.descriptor(for: mask, batchSize: batchSize, heads: heads, queryCount: queryCount, keyCount: keyCount)
     }
 
     static var attentionFlags: UInt32 {
@@ -74,23 +83,24 @@ extension HIPEngine {
     public static func fusedAttention<N: NumericType>(q: ShapedBuffer<N, HIP>, k: ShapedBuffer<N, HIP>, v: ShapedBuffer<N, HIP>,
                                                       mask: ShapedBuffer<N, HIP>?, result: ShapedBuffer<N, HIP>, temperature: N) {
         precondition(q.dim == 4 && k.dim == 4 && v.dim == 4)
-        var descriptor = self.descriptor(for: mask)
+        var descriptor = self.descriptor(for: mask, batchSize: q.shape[0], heads: q.shape[1], queryCount: q.shape[2], keyCount: k.shape[2])
         // the reference forms the reciprocal once in Float and multiplies (Engine/CPU/CPUEngine.swift:635)
         let reciprocal = Float(1) / (temperature as! Float)
         hipCheck(dl4s_hip_sdpa_fwd_f32(HIP.context, f(q), f(k), f(v), f(result),
                                        Int64(q.shape[0]), Int64(q.shape[1]), Int64(q.shape[2]), Int64(k.shape[2]),
-                                       Int64(q.shape[3]), Int64(v.shape[3]), reciprocal, mask == nil ? nil : &descriptor, attentionFlags))
+                                       Int64(q.shape[3]), Int64(v.shape[3]), reciprocal,
+                                       descriptor.kind == Int32(DL4S_MASK_NONE.rawValue) ? nil : &descriptor, attentionFlags))
     }
 
     public static func fusedAttentionForwardStats<N: NumericType>(q: ShapedBuffer<N, HIP>, k: ShapedBuffer<N, HIP>, v: ShapedBuffer<N, HIP>,
                                                                   mask: ShapedBuffer<N, HIP>?, result: ShapedBuffer<N, HIP>,
                                                                   stats: ShapedBuffer<N, HIP>, temperature: N) {
         precondition(q.dim == 4 && k.dim == 4 && v.dim == 4 && q.shape[3] == v.shape[3], "the training form needs keyDim == valueDim")
-        var descriptor = self.descriptor(for: mask)
+        var descriptor = self.descriptor(for: mask, batchSize: q.shape[0], heads: q.shape[1], queryCount: q.shape[2], keyCount: k.shape[2])
         let reciprocal = Float(1) / (temperature as! Float)
         hipCheck(dl4s_hip_sdpa_fwd_stats_f32(HIP.context, f(q), f(k), f(v), f(result), f(stats),
                                              Int64(q.shape[0]), Int64(q.shape[1]), Int64(q.shape[2]), Int64(k.shape[2]), Int64(q.shape[3]),
-                                             reciprocal, mask == nil ? nil : &descriptor, attentionFlags))
+                                             reciprocal, descriptor.kind == Int32(DL4S_MASK_NONE.rawValue) ? nil : &descriptor, attentionFlags))
     }
 
     public static func fusedAttentionBackward<N: NumericType>(q: ShapedBuffer<N, HIP>, k: ShapedBuffer<N, HIP>, v: ShapedBuffer<N, HIP>,
@@ -98,12 +108,73 @@ extension HIPEngine {
                                                               stats: ShapedBuffer<N, HIP>, resultGradient: ShapedBuffer<N, HIP>,
                                                               qGradient: ShapedBuffer<N, HIP>, kGradient: ShapedBuffer<N, HIP>,
                                                               vGradient: ShapedBuffer<N, HIP>, temperature: N) {
-        var descriptor = self.descriptor(for: mask)
+        var descriptor = self.descriptor(for: mask, batchSize: q.shape[0], heads: q.shape[1], queryCount: q.shape[2], keyCount: k.shape[2])
         let reciprocal = Float(1) / (temperature as! Float)
         hipCheck(dl4s_hip_sdpa_bwd_f32(HIP.context, f(q), f(k), f(v), f(result), f(stats), f(resultGradient),
                                        f(qGradient), f(kGradient), f(vGradient),
                                        Int64(q.shape[0]), Int64(q.shape[1]), Int64(q.shape[2]), Int64(k.shape[2]), Int64(q.shape[3]),
-                                       reciprocal, mask == nil ? nil : &descriptor, attentionFlags))
+                                       reciprocal, descriptor.kind == Int32(DL4S_MASK_NONE.rawValue) ? nil : &descriptor, attentionFlags))
+    }
+}
+
+/// Mask buffers the fused attention calls have looked at (see `HIPEngine.descriptor(for:batchSize:heads:queryCount:keyCount:)`),
+/// keyed by the buffer's device address.  An entry owns the device memory of its valid key counts or tile classes.  It is
+/// dropped when the buffer it describes is freed (`HIPMemory.free`, which also covers offset views into the freed
+/// allocation) or written through `HIPMemory` (`assign`, `set(slice:)`, `setPointee`); the engine's operators always
+/// write to result buffers they have just allocated, so nothing else changes a mask under its entry.
+enum HIPPreparedMasks {
+    struct Entry {
+        var descriptor: dl4s_mask_desc
+        var shape: [Int]
+        var extents: [Int]
+        var lengths: UnsafeMutableRawPointer?
+        var classes: UnsafeMutableRawPointer?
+    }
+    static var entries: [UnsafeMutableRawPointer: Entry] = [:]
+    static let lock = NSLock()
+
+    static func release(_ entry: Entry) {
+        if let lengths = entry.lengths { hipCheck(dl4s_hip_free(HIP.context, lengths)) }
+        if let classes = entry.classes { hipCheck(dl4s_hip_free(HIP.context, classes)) }
+    }
+
+    static func descriptor<N: NumericType>(for mask: ShapedBuffer<N, HIP>, batchSize: Int, heads: Int, queryCount: Int, keyCount: Int) -> dl4s_mask_desc {
+        let key = mask.values.memory.ptr
+        let extents = [batchSize, heads, queryCount, keyCount]
+        lock.lock()
+        defer { lock.unlock() }
+        if let known = entries[key], known.shape == mask.shape, known.extents == extents {
+            return known.descriptor
+        }
+        if let stale = entries.removeValue(forKey: key) { release(stale) }
+        var dense = HIPEngine.denseDescriptor(for: mask)
+        var entry = Entry(descriptor: dense, shape: mask.shape, extents: extents, lengths: nil, classes: nil)
+        let (b, h, lq, lk) = (Int64(batchSize), Int64(heads), Int64(queryCount), Int64(keyCount))
+        var classBytes = 0
+        // a shape that does not fit the problem: the attention call reports it
+        guard dl4s_hip_mask_classes_size(&dense, b, h, lq, lk, &classBytes) == 0 else { return dense }
+        hipCheck(dl4s_hip_alloc(HIP.context, max(batchSize, 1) * MemoryLayout<Int32>.stride, &entry.lengths))
+        var described = dl4s_mask_desc()
+        hipCheck(dl4s_hip_mask_describe_f32(HIP.context, &dense, b, h, lq, lk, entry.lengths!.assumingMemoryBound(to: Int32.self), &described))
+        if described.kind == Int32(DL4S_MASK_DENSE_F32.rawValue) {
+            hipCheck(dl4s_hip_alloc(HIP.context, max(classBytes, 1), &entry.classes))
+            hipCheck(dl4s_hip_mask_classify_f32(HIP.context, &dense, b, h, lq, lk, entry.classes!.assumingMemoryBound(to: UInt8.self)))
+            described.classes = UnsafePointer(entry.classes!.assumingMemoryBound(to: UInt8.self))
+        }
+        entry.descriptor = described
+        entries[key] = entry
+        return described
+    }
+
+    /// Drops the entries of mask buffers inside [start, start + bytes): the allocation is being freed or written.
+    static func forget(from start: UnsafeMutableRawPointer, bytes: Int) {
+        lock.lock()
+        defer { lock.unlock() }
+        if entries.isEmpty { return }
+        let end = start + max(bytes, 1)
+        for key in entries.keys.filter({ $0 >= start && $0 < end }) {
+            release(entries.removeValue(forKey: key)!)
+        }
     }
 }
 
@@ -122,7 +193,11 @@ extension ScaledDotProductAttention {
     /// Tensor/Operators/Unary.swift:40-53.
     func fusedForward(q: Tensor<Element, Device>, k: Tensor<Element, Device>, v: Tensor<Element, Device>,
                       mask: Tensor<Element, Device>?) -> Tensor<Element, Device>? {
-        guard Device.Engine.hasFusedAttention, q.dim == 4, v.dim == 4 else {
+        // outside what the fused call takes - head dims above 256, a mask with more than four axes - and for a mask that
+        // requires a gradient (the operator sequence propagates through `mask * 1e9`, the fused call does not) the layer
+        // runs its operator sequence
+        guard Device.Engine.hasFusedAttention, q.dim == 4, v.dim == 4, q.shape[3] <= 256, v.shape[3] <= 256,
+              (mask?.dim ?? 0) <= 4, !(mask?.requiresGradient ?? false) else {
             return nil
         }
         let needsGradient = q.requiresGradient || k.requiresGradient || v.requiresGradient
