@@ -173,6 +173,35 @@ __device__ __forceinline__ void wait_vector_memory() { __builtin_amdgcn_s_waitcn
 
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
 
+// The value of lane l and the value of lane l ^ 32 in both lanes: v_permlane32_swap exchanges the upper half of its first
+// operand with the lower half of its second, so (x, x) becomes (the lower half's values twice, the upper half's twice) - one
+// instruction where a shuffle through the LDS crossbar costs an address computation, the round trip and its wait.
+__device__ __forceinline__ void both_halves(const float x, float &lower, float &upper) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lower = __uint_as_float(sw[0]);
+    upper = __uint_as_float(sw[1]);
+}
+// fmaxf(x, xor32(x)) and x + xor32(x) (the sum of two floats does not depend on their order: the same bits in both lanes)
+// (the maximum is formed as max3(-inf, a, b): a two-operand maximum of values the compiler cannot prove canonical - register
+// contents that come from an MFMA or a lane exchange - costs one quieting instruction per operand, the three-operand form none)
+__device__ __forceinline__ float max_across_halves(const float x) {
+    float a, b;
+    both_halves(x, a, b);
+    return fmaxf(fmaxf(-INFINITY, a), b);
+}
+// The largest of 16 scores, NaN ignored; -inf when all of them are NaN.
+__device__ __forceinline__ float max_of_16(const f32x16 &s) {
+    float t = fmaxf(fmaxf(-INFINITY, s[0]), s[1]);
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) t = fmaxf(fmaxf(t, s[r]), s[r + 1]);
+    return t;
+}
+__device__ __forceinline__ float sum_across_halves(const float x) {
+    float a, b;
+    both_halves(x, a, b);
+    return a + b;
+}
+
 // Work item of this workgroup (see work_order.h).  Returns false for padding workgroups.
 __device__ __forceinline__ bool work_item(const int nunits, const int total_blocks, const int lpt, int &bh, int &unit,
                                           const int snake = 0) {

@@ -50,12 +50,9 @@ __device__ __forceinline__ void attend_tile(const float *Kb, const float *Vb, co
     // The reference maximum m_run only moves -- and the accumulators are only rescaled -- when a tile's maximum
     // would give a weight above 2^8; any per-row factor 2^(max - m_run) left in the weights cancels in the
     // final division by the row sum.
-    float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
-#pragma unroll
-    for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
-    tmax = fmaxf(tmax, s0[15]);
-    tmax = fmaxf(tmax, xor32(tmax));
-    const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+    const float tmax = max_across_halves(max_of_16(s0));
+    // tmax above m_run by more than 8; with m_run = -inf the difference is +inf for any other tmax and NaN for tmax = -inf
+    const bool upd = tmax - m_run > 8.0f;
     if (__any(upd)) {
         const float m_new = fmaxf(m_run, tmax);
         // lanes whose maximum did not move keep factor 1 (also when it is still -inf: -inf - -inf would be NaN)
@@ -249,7 +246,7 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_d64(const float *__re
     }
 
     // ---- normalise and store.  Register r of o0/o1 is d = 2*(8(r/4) + 4*half + r%4) + {0,1}.
-    const float l_tot = l_run + xor32(l_run);
+    const float l_tot = sum_across_halves(l_run);
     const float inv = 1.0f / l_tot;
     // row statistics for the backward pass, [B,H,Lq,2]: the reference maximum m and 1 / sum_j 2^(s_j - m), so that a weight
     // is 2^(s - m) * that (kept apart: m can be of the order of the 1e9 mask penalty, where a float cannot also hold log2 l)
@@ -410,7 +407,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
     // ---- merge the four partial results.  Wavefront w > 0 leaves (m_run, row sum, O^T) in its own LDS region (the tiles
     // are dead by now); wavefront 0 folds them in.  A partial result with m_run = -inf has seen no finite score: its
     // sums are zeros (or NaN, which must survive), so it is added with factor 1.
-    float l_tot = l_run + xor32(l_run);
+    float l_tot = sum_across_halves(l_run);
     __syncthreads();   // every wavefront is done with its tile region
     float *mine = lds + wave * 2 * TILE_FLOATS;   // [34][64]: rows 0..31 = o0/o1 registers, row 32 = m_run, row 33 = l_tot
     if (wave > 0) {

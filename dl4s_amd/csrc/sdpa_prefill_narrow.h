@@ -42,12 +42,8 @@ __device__ __forceinline__ void attend_tile_narrow(const float *Kb, const float 
     f32x16 s0 = masked_scores<KIND, NarrowTile<W>::NJ>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
 
     // online softmax with a lazy reference maximum (see attend_tile in sdpa_prefill.hip)
-    float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
-#pragma unroll
-    for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
-    tmax = fmaxf(tmax, s0[15]);
-    tmax = fmaxf(tmax, xor32(tmax));
-    const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+    const float tmax = max_across_halves(max_of_16(s0));
+    const bool upd = tmax - m_run > 8.0f;      // also right at m_run = -inf: +inf, or NaN for tmax = -inf
     if (__any(upd)) {
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
@@ -84,12 +80,8 @@ __device__ __forceinline__ void attend_tile_16(const float *Kb, const float *Vt,
                                                const int cls) {
     constexpr int LSV = NarrowTile<16>::LSV;
     f32x16 s0 = masked_scores<KIND, 2>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
-    float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
-#pragma unroll
-    for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
-    tmax = fmaxf(tmax, s0[15]);
-    tmax = fmaxf(tmax, xor32(tmax));
-    const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+    const float tmax = max_across_halves(max_of_16(s0));
+    const bool upd = tmax - m_run > 8.0f;      // also right at m_run = -inf: +inf, or NaN for tmax = -inf
     if (__any(upd)) {
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
@@ -129,12 +121,8 @@ __device__ __forceinline__ void attend_tile_48(const float *Kb, const float *Vb,
                                                const float *mrow, const long long msk, const int cls) {
     constexpr int LSV = NarrowTile<48>::LSV;
     f32x16 s0 = masked_scores<KIND, 6>(Kb, qr, k0, q0, qi, half, Lk, len, mrow, msk, cls);
-    float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
-#pragma unroll
-    for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
-    tmax = fmaxf(tmax, s0[15]);
-    tmax = fmaxf(tmax, xor32(tmax));
-    const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+    const float tmax = max_across_halves(max_of_16(s0));
+    const bool upd = tmax - m_run > 8.0f;      // also right at m_run = -inf: +inf, or NaN for tmax = -inf
     if (__any(upd)) {
         const float m_new = fmaxf(m_run, tmax);
         const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
@@ -322,7 +310,7 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_f32_narrow(const float *_
         if (t + 1 < ntiles) tile_step(t + 1, std::integral_constant<int, 1>{});
     }
 
-    const float l_tot = l_run + xor32(l_run);
+    const float l_tot = sum_across_halves(l_run);
     const float inv = 1.0f / l_tot;
     if (stats && half == 0 && qi < Lq) {
         stats[2 * ((long long)bh * Lq + qi)] = m_use;
@@ -461,7 +449,7 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_narrow(const fl
     }
 
     // merge the four partial results (reference maximum, row sum, O^T) in wavefront order
-    float l_tot = l_run + xor32(l_run);
+    float l_tot = sum_across_halves(l_run);
     __syncthreads();
     float *mine = lds + wave * REGION;   // rows 0..15 = o0 registers, row 16 = m_run, row 17 = l_tot
     if (wave > 0) {

@@ -168,12 +168,8 @@ __global__ __launch_bounds__(256, VEC == 4 ? 3 : 2) void sdpa_prefill_f32_w96(co
         if (k0 < wkend && !(DENSE && skip_ones && cls == 1)) {
             f32x16 s0 = masked_scores<KIND, W / 8>(Ks + buf * TILE96_FLOATS + k_lds, qr, k0, q0, qi, half, Lk, len, mrow, mask.sk, cls);
             // online softmax with a lazily moved reference maximum (see attend_tile in sdpa_prefill.hip)
-            float tmax = fmaxf(fmaxf(s0[0], s0[1]), s0[2]);
-#pragma unroll
-            for (int r = 3; r < 15; r += 2) tmax = fmaxf(fmaxf(tmax, s0[r]), s0[r + 1]);
-            tmax = fmaxf(tmax, s0[15]);
-            tmax = fmaxf(tmax, xor32(tmax));
-            const bool upd = (tmax > m_run) && (m_run == -INFINITY || tmax - m_run > 8.0f);
+            const float tmax = max_across_halves(max_of_16(s0));
+            const bool upd = tmax - m_run > 8.0f;      // also right at m_run = -inf: +inf, or NaN for tmax = -inf
             if (__any(upd)) {
                 const float m_new = fmaxf(m_run, tmax);
                 const float alpha = (m_run == m_new) ? 1.0f : fast_exp2(m_run - m_new);
@@ -222,7 +218,7 @@ __global__ __launch_bounds__(256, VEC == 4 ? 3 : 2) void sdpa_prefill_f32_w96(co
     }
 
     // ---- normalise and store
-    const float l_tot = l_run + xor32(l_run);
+    const float l_tot = sum_across_halves(l_run);
     if (part) {   // this share's weighted sums as they are, with their reference maximum and row sum
         if (qi < Lq) {
             float *pp = part + (((long long)sp * (total_blocks / nqb) + bh) * Lq + qi) * PART2_STRIDE;
