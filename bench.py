@@ -136,6 +136,16 @@ def under_rocprof():
     return not lib.graph_supported()
 
 
+# What a DL4S checkout has to contain for each host mode of the layer rows (the Swift sources and patches under swift/).
+PATCH_SETS = {
+    "primitive": "HIP.swift + module map + Package.swift.patch: the reference's engine calls one by one",
+    "attention_hook_only": "primitive + Engine.swift.patch + HIPFusedAttention.swift + ScaledDotProductAttention.swift.patch",
+    "fused": "attention_hook_only + HIPFusedLayers.swift + MultiHeadAttention.swift.patch + PointwiseFeedForward.swift.patch, "
+             "HIP.fusedLayers = true (forward only)",
+    "fused_strict": "fused with HIP.strictMasks = true: every key tile visited, LayerNorm sums in the reference's order",
+}
+
+
 def other_configs(ctx, lib, cpu, only=None):
     """Configs 1-3 of the baseline: us/call, TFLOP/s on the algorithmic flops, fraction of the fp32 MFMA peak; the
     CPU oracle beside each (whole call for configs 1 and 2, one batch item of config 3), single thread."""
@@ -185,7 +195,8 @@ def other_configs(ctx, lib, cpu, only=None):
             # the harness runs as many untimed calls as timed ones first (0.04 - 0.1 s: the clocks are up when the timer starts)
             _, ms = host_lib.mha(ctx, x, x, x, mask, attn, H, dk_, dk_, fused=fused, iters=1000 if quick else (300 if fused else 60))
             res["config2_mha_B4_L512_D512_H8_causal_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
-                                                                "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
+                                                                "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
+                                                                "swift_patch_set": PATCH_SETS[mode]}
         if cpu:
             t0 = time.perf_counter()
             orc.mha(x, x, x, mask, attn, H, dk_, dk_)
@@ -267,8 +278,8 @@ def other_configs(ctx, lib, cpu, only=None):
         graph.destroy()
         a_.release()
         b_.release()
-    if want("config3"):
-        # config 3: encoder block B8 L1024 D1024 H16 F4096, key-length mask
+    if want("config3") or (only is not None and "config3_hook_only" in only):
+        # config 3: encoder block B8 L1024 D1024 H16 F4096, key-length mask ("config3_hook_only": that host mode alone)
         B, L, D, H, F = 8, 1024, 1024, 16, 4096
         rng = np.random.Generator(np.random.PCG64(1003))
         x = rng.standard_normal((B, L, D), dtype=np.float32)
@@ -277,11 +288,14 @@ def other_configs(ctx, lib, cpu, only=None):
         mask = (np.arange(L)[None, None, None, :] >= lens[:, None, None, None]).astype(np.float32)
         fl = 4.0 * 64 * H * L * float(lens.sum()) + 4 * 2.0 * B * L * D * D + 2 * 2.0 * B * L * D * F
         for mode, fused in (("fused", 1), ("fused_strict", 2), ("attention_hook_only", 3)):
+            if not want("config3") and mode != "attention_hook_only":
+                continue
             # the harness runs as many untimed calls as timed ones first (about 0.1 s: the clocks are up when the timer starts)
             _, ms = host_lib.encoder_block(ctx, x, mask, attn, ffn, H, 64, 64, fused=fused, iters=50 if fused < 3 else 30)
             res["config3_encoder_block_B8_L1024_D1024_H16_F4096_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
-                                                                             "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl}
-        if cpu:
+                                                                             "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
+                                                                             "swift_patch_set": PATCH_SETS[mode]}
+        if cpu and want("config3"):
             t0 = time.perf_counter()
             orc.encoder_block(x[:1, :256], mask[:1, :, :, :256], attn, ffn, H, 64, 64)
             dt = time.perf_counter() - t0
@@ -567,7 +581,7 @@ def main():
                          "profiler counter runs")
     ap.add_argument("--only", default="", metavar="NAMES",
                     help="instead of the benchmark, run only these of the workloads reported beside the headline (comma "
-                         "separated: config1, config2, recorded, config3, backward, masks_and_head_dim, decode_head_dims, greedy, greedy_fused, greedy_primitive, greedy_cached, greedy_cached_only) and print their entries: "
+                         "separated: config1, config2, recorded, config3, config3_hook_only, backward, masks_and_head_dim, decode_head_dims, greedy, greedy_fused, greedy_primitive, greedy_cached, greedy_cached_only) and print their entries: "
                          "short commands for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:
