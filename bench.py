@@ -363,8 +363,20 @@ def other_configs(ctx, lib, cpu, only=None):
             rT = float(np.float32(1.0) / np.float32(np.sqrt(np.float32(d))))
             fl = 4.0 * d * B * H * (L * (L + 1) // 2)
             entry = {"flops": fl}
-            variants = (("tile_skipping", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), 0), ("strict", ctx.mask_desc(lib.MASK_DENSE, dense=dmask), lib.SDPA_STRICT)) \
-                if d == 64 else (("causal_descriptor", ctx.mask_desc(lib.MASK_CAUSAL), 0),)
+            keep = []
+            if d == 64:
+                # the tensor as it is (classified on every call), with its tile classes prepared once, and looked at once
+                # by dl4s_hip_mask_describe_f32 (what the Swift hook and the host layer do per mask tensor: it is recognised
+                # as the causal kind); then every tile visited
+                plain, prepared = ctx.mask_desc(lib.MASK_DENSE, dense=dmask), ctx.mask_desc(lib.MASK_DENSE, dense=dmask)
+                keep.append(ctx.mask_classify(prepared, B, H, L, L))
+                described, lengths = ctx.mask_describe(plain, B, H, L, L)
+                keep.append(lengths)
+                entry["described_as_kind"] = int(described.kind)
+                variants = (("tile_skipping", plain, 0), ("tile_skipping_classes_prepared_once", prepared, 0),
+                            ("tile_skipping_described_once", described, 0), ("strict", plain, lib.SDPA_STRICT))
+            else:
+                variants = (("causal_descriptor", ctx.mask_desc(lib.MASK_CAUSAL), 0),)
             for vname, desc, flags in variants:
                 for _ in range(100):
                     ctx.sdpa_fwd(qkv[0], qkv[1], qkv[2], o, B, H, L, L, d, d, rT, desc, flags)
@@ -375,7 +387,7 @@ def other_configs(ctx, lib, cpu, only=None):
                 ms = ctx.timer_end() / 30
                 entry[vname] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9, "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS}
             res[name] = entry
-            for b_ in qkv + [o]:
+            for b_ in qkv + [o] + keep:
                 b_.release()
         dmask.release()
     if want("decode_head_dims"):
