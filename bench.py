@@ -29,8 +29,8 @@ HBM_PEAK_GBS = 8000.0
 # streaming kernel (--copy-calibration: x2.00 and x1.00).  The runs and their figures are summarised in
 # profiles/bench_prefill_config4_decode_config5.md; they are constants here because a counter run cannot be part of
 # the timed process.
-PREFILL_TRAFFIC_BYTES = (395661 * 2.00 + 65536 * 1.00) * 1024      # L2 fills (K/V re-reads included) + writes
-DECODE_TRAFFIC_BYTES = (264304 * 2.00 + 192 * 1.00) * 1024
+PREFILL_TRAFFIC_BYTES = (407114 * 2.00 + 65536 * 1.00) * 1024      # L2 fills (K/V re-reads included) + writes
+DECODE_TRAFFIC_BYTES = (264315 * 2.00 + 192 * 1.00) * 1024
 PREHEAT_S = 0.25
 
 
@@ -178,8 +178,9 @@ def other_configs(ctx, lib, cpu, only=None):
             orc.sdpa(q, k, v, None)
             dt = time.perf_counter() - t0
             res["config1_sdpa_B1_H8_L128_d64"]["cpu_baseline"] = {"us_per_call": dt * 1e6, "tflops": fl / dt / 1e12, "cores": 1, "kind": "port"}
-    if want("config2"):
-        # config 2: MHA layer B4 L512 D512 H8 causal (dense mask tensor, as the layer receives it)
+    if want("config2") or (only is not None and "config2_fused_only" in only):
+        # config 2: MHA layer B4 L512 D512 H8 causal (dense mask tensor, as the layer receives it; "config2_fused_only": that
+        # host mode alone)
         B, L, D, H, dk_ = 4, 512, 512, 8, 64
         rng = np.random.Generator(np.random.PCG64(1002))
         x = rng.standard_normal((B, L, D), dtype=np.float32)
@@ -191,13 +192,15 @@ def other_configs(ctx, lib, cpu, only=None):
         # the reference); primitive: the reference's engine calls one by one; attention_hook_only: the primitive layer with the
         # one fused call inside ScaledDotProductAttention (a DL4S checkout with the five-line hook and nothing else)
         for mode, fused in (("fused", 1), ("fused_strict", 2), ("primitive", 0), ("attention_hook_only", 3)):
+            if not want("config2") and mode != "fused":
+                continue
             quick = fused in (1, 2)
             # the harness runs as many untimed calls as timed ones first (0.04 - 0.1 s: the clocks are up when the timer starts)
             _, ms = host_lib.mha(ctx, x, x, x, mask, attn, H, dk_, dk_, fused=fused, iters=1000 if quick else (300 if fused else 60))
             res["config2_mha_B4_L512_D512_H8_causal_" + mode] = {"us_per_call": ms * 1e3, "tflops": fl / ms / 1e9,
                                                                 "frac_mfma_peak": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS, "flops": fl,
                                                                 "swift_patch_set": PATCH_SETS[mode]}
-        if cpu:
+        if cpu and want("config2"):
             t0 = time.perf_counter()
             orc.mha(x, x, x, mask, attn, H, dk_, dk_)
             dt = time.perf_counter() - t0
@@ -593,7 +596,7 @@ def main():
                          "profiler counter runs")
     ap.add_argument("--only", default="", metavar="NAMES",
                     help="instead of the benchmark, run only these of the workloads reported beside the headline (comma "
-                         "separated: config1, config2, recorded, config3, config3_hook_only, backward, masks_and_head_dim, decode_head_dims, greedy, greedy_fused, greedy_primitive, greedy_cached, greedy_cached_only) and print their entries: "
+                         "separated: config1, config2, config2_fused_only, recorded, config3, config3_hook_only, backward, masks_and_head_dim, decode_head_dims, greedy, greedy_fused, greedy_primitive, greedy_cached, greedy_cached_only) and print their entries: "
                          "short commands for profiler runs")
     args = ap.parse_args()
     if args.gpus != 1:
