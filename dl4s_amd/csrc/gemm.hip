@@ -313,6 +313,24 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
     const int ktiles = g.tri == 3 ? min(ktiles_all, (m0 + TM + KT - 1) / KT) : ktiles_all;
     opa.template load<0>(kt_first);
     opb.template load<0>(kt_first);
+    // The 64 x 64 form with an epilogue asks for its bias and residual values now, behind the first tile: requested in the
+    // epilogue, they would add a trip to memory (the residual is the layer's input, long out of the caches) to a launch
+    // that has nothing else left to do.  16 + 16 registers, which this form can spare.
+    constexpr bool PRE = EPI && MI == 1 && NI == 1;
+    f32x4 pre_bias[PRE ? 4 : 1], pre_res[PRE ? 4 : 1];
+    if (PRE) {
+        const int gm = m0 + wm * 32 + ln;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            const int gn = n0 + wn * 32 + 8 * q4 + 4 * half;
+            pre_bias[q4] = f32x4{0.f, 0.f, 0.f, 0.f};
+            pre_res[q4] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (gm < g.M && gn < g.N) {
+                if (g.bias) pre_bias[q4] = *reinterpret_cast<const f32x4 *>(g.bias + gn);
+                if (g.residual) pre_res[q4] = *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
+            }
+        }
+    }
     if (SLOTS == 2) {
         // the second tile is requested with the first and both are waited for (they arrive together): entering the loop
         // with loads pending in another order than the loop's own made the compiler wait, at the head of every second
@@ -408,7 +426,7 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
                 }
                 if (EPI) {
                     if (g.bias) {
-                        const f32x4 bq = *reinterpret_cast<const f32x4 *>(g.bias + gn);
+                        const f32x4 bq = PRE ? pre_bias[PRE ? q4 : 0] : *reinterpret_cast<const f32x4 *>(g.bias + gn);
                         val.x = __fadd_rn(val.x, bq.x); val.y = __fadd_rn(val.y, bq.y);
                         val.z = __fadd_rn(val.z, bq.z); val.w = __fadd_rn(val.w, bq.w);
                     }
@@ -417,7 +435,7 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
                         val.z = gelu_sigmoid(val.z); val.w = gelu_sigmoid(val.w);
                     }
                     if (g.residual) {
-                        const f32x4 rq = *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
+                        const f32x4 rq = PRE ? pre_res[PRE ? q4 : 0] : *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
                         val.x = __fadd_rn(val.x, rq.x); val.y = __fadd_rn(val.y, rq.y);
                         val.z = __fadd_rn(val.z, rq.z); val.w = __fadd_rn(val.w, rq.w);
                     }

@@ -251,14 +251,17 @@ __device__ __forceinline__ f32x4 ln_load4(const float *xp, const float *rp, long
     return v;
 }
 
-__device__ __forceinline__ f32x4 ln_norm4(f32x4 v, float mean, float rden, const float *scale, const float *shift, long long d) {
-    const f32x4 sc = *reinterpret_cast<const f32x4 *>(scale + d), sh = *reinterpret_cast<const f32x4 *>(shift + d);
+__device__ __forceinline__ f32x4 ln_norm4(f32x4 v, float mean, float rden, const f32x4 sc, const f32x4 sh) {
     f32x4 y;
     y.x = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.x, -mean), rden), sc.x), sh.x);
     y.y = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.y, -mean), rden), sc.y), sh.y);
     y.z = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.z, -mean), rden), sc.z), sh.z);
     y.w = __fadd_rn(__fmul_rn(__fmul_rn(__fadd_rn(v.w, -mean), rden), sc.w), sh.w);
     return y;
+}
+
+__device__ __forceinline__ f32x4 ln_norm4(f32x4 v, float mean, float rden, const float *scale, const float *shift, long long d) {
+    return ln_norm4(v, mean, rden, *reinterpret_cast<const f32x4 *>(scale + d), *reinterpret_cast<const f32x4 *>(shift + d));
 }
 
 template <bool VEC>
@@ -297,21 +300,41 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     const float *xp = x + b * n;
     const float *rp = res ? res + b * n : nullptr;
     float *yp = y + b * n;
-    // the column of element i advances by a constant per iteration: no division in the loop
-    const long long step = (long long)gridDim.x * TPB * 4, dstep = step % D;
-    long long i = ((long long)blockIdx.x * TPB + threadIdx.x) * 4, d = i % D;
-    // the thread's first two pieces are requested before the statistics are formed (the launcher sizes the grid for two
-    // per thread): their way through memory overlaps the reduction instead of following it
+    // Everything the block waits for is requested at once, the partial sums first: the pairs, the thread's first two
+    // pieces (the launcher sizes the grid for two per thread) and their scale / shift values travel together while the
+    // column indices are computed, instead of one trip to memory before the reduction and two behind it.
+    // (The arguments likewise: fetched where the code first needs them, they arrive in five trips, one behind the other.)
+    asm volatile("" ::"s"(x), "s"(res), "s"(scale), "s"(shift), "s"(y), "s"(part), "s"(n), "s"(D), "s"(nblk));
+    float s = 0.f, ss = 0.f;
+    if ((int)threadIdx.x < nblk) {      // nblk <= TPB: one partial pair per thread, summed in a fixed order
+        s = part[(b * nblk + threadIdx.x) * 2];
+        ss = part[(b * nblk + threadIdx.x) * 2 + 1];
+    }
+    const long long step = (long long)gridDim.x * TPB * 4;
+    long long i = ((long long)blockIdx.x * TPB + threadIdx.x) * 4;
     f32x4 pre[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     if (VEC) {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
             if (i + u * step < n) pre[u] = ln_load4(xp, rp, i + u * step);
     }
-    float s = 0.f, ss = 0.f;
-    if ((int)threadIdx.x < nblk) {      // nblk <= TPB: one partial pair per thread, summed in a fixed order
-        s = part[(b * nblk + threadIdx.x) * 2];
-        ss = part[(b * nblk + threadIdx.x) * 2 + 1];
+    // the column of element i advances by a constant per iteration: no division in the loop (and 32-bit ones before it
+    // wherever the item has fewer than 2^31 elements)
+    long long d, dstep;
+    if (n + step < (1ll << 31)) { d = (unsigned)i % (unsigned)D; dstep = (unsigned)step % (unsigned)D; }
+    else { d = i % D; dstep = step % D; }
+    f32x4 sc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}}, sh[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    if (VEC) {
+        long long du = d;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            if (i + u * step < n) {
+                sc[u] = *reinterpret_cast<const f32x4 *>(scale + du);
+                sh[u] = *reinterpret_cast<const f32x4 *>(shift + du);
+            }
+            du += dstep;
+            if (du >= D) du -= D;
+        }
     }
     block_sum2(s, ss, sm);
     const float rN = __fdiv_rn(1.0f, (float)n);
@@ -321,7 +344,7 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     if (VEC) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            if (i < n) *reinterpret_cast<f32x4 *>(yp + i) = ln_norm4(pre[u], mean, rden, scale, shift, d);
+            if (i < n) *reinterpret_cast<f32x4 *>(yp + i) = ln_norm4(pre[u], mean, rden, sc[u], sh[u]);
             i += step;
             d += dstep;
             if (d >= D) d -= D;

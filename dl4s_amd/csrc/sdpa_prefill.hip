@@ -298,6 +298,10 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
                                                                       int strict, int nqb, int total_blocks, int token_major,
                                                                       float *__restrict__ stats, int hd, int order) {
     extern __shared__ __align__(16) float lds[];
+    // every argument the block's first loads depend on is asked for at once: fetched as the code first needs them, the
+    // arguments arrive in three round trips, one behind the other, before the first row is requested
+    asm volatile("" ::"s"(q), "s"(k), "s"(v), "s"(out), "s"(H), "s"(Lq), "s"(Lk), "s"(rT), "s"(nqb), "s"(total_blocks),
+                 "s"(token_major), "s"(hd), "s"(order), "s"(strict), "s"(stats));
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: lets the per-wavefront tile conditions branch on scalars
     const int lane = tid & 63;
@@ -420,61 +424,57 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_d64(const float
         if (more) store_tile();
     }
 
-    // ---- merge the four partial results.  Wavefront w > 0 leaves (m_run, row sum, O^T) in its own LDS region (the tiles
-    // are dead by now); wavefront 0 folds them in.  A partial result with m_run = -inf has seen no finite score: its
-    // sums are zeros (or NaN, which must survive), so it is added with factor 1.
-    float l_tot = sum_across_halves(l_run);
-    __syncthreads();   // every wavefront is done with its tile region
-    float *mine = lds + wave * 2 * TILE_FLOATS;   // [34][64]: rows 0..31 = o0/o1 registers, row 32 = m_run, row 33 = l_tot
-    if (wave > 0) {
+    // ---- merge the four partial results.  Every wavefront leaves (m_run, row sum, O^T) in its own LDS region (its
+    // tiles are dead by now, and the LDS operations of one wavefront execute in order: no barrier before the writes);
+    // after the barrier wavefront w folds the four partial results of the accumulator registers 4w .. 4w + 3 (16 of the
+    // 64 output columns) in the order 0, 1, 2, 3 and stores them.  A partial result with m_run = -inf has seen no finite
+    // score: its sums are zeros (or NaN, which must survive), so it is added with factor 1.
+    {
+        const float l_part = sum_across_halves(l_run);
+        float *mine = lds + wave * 2 * TILE_FLOATS;   // [34][64]: rows 0..31 = o0/o1 registers, row 32 = m_run, row 33 = row sum
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             mine[(2 * r) * 64 + lane] = o0[r];
             mine[(2 * r + 1) * 64 + lane] = o1[r];
         }
         mine[32 * 64 + lane] = m_run;
-        mine[33 * 64 + lane] = l_tot;
+        mine[33 * 64 + lane] = l_part;
     }
     __syncthreads();
-    if (wave == 0) {
-        float m_all = m_run;
+    float m_all = lds[32 * 64 + lane];
 #pragma unroll
-        for (int x = 1; x < SPLIT_WAVES; ++x) m_all = fmaxf(m_all, lds[x * 2 * TILE_FLOATS + 32 * 64 + lane]);
-        const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
-        const float f0 = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - m_ref);
-        l_tot *= f0;
+    for (int x = 1; x < SPLIT_WAVES; ++x) m_all = fmaxf(m_all, lds[x * 2 * TILE_FLOATS + 32 * 64 + lane]);
+    const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
+    float l_tot = 0.f, acc[8];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { o0[r] *= f0; o1[r] *= f0; }
+    for (int x = 0; x < SPLIT_WAVES; ++x) {
+        const float *part = lds + x * 2 * TILE_FLOATS;
+        const float mx = part[32 * 64 + lane];
+        const float fx = (mx == -INFINITY) ? 1.0f : fast_exp2(mx - m_ref);
+        const float *rows = part + (8 * wave) * 64 + lane;   // rows 8w .. 8w + 7 = o0[4w], o1[4w], o0[4w + 1], ...
+        if (x == 0) {
+            l_tot = part[33 * 64 + lane] * fx;
 #pragma unroll
-        for (int x = 1; x < SPLIT_WAVES; ++x) {
-            const float *other = lds + x * 2 * TILE_FLOATS;
-            const float mx = other[32 * 64 + lane];
-            const float fx = (mx == -INFINITY) ? 1.0f : fast_exp2(mx - m_ref);
-            l_tot += other[33 * 64 + lane] * fx;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                o0[r] += other[(2 * r) * 64 + lane] * fx;
-                o1[r] += other[(2 * r + 1) * 64 + lane] * fx;
-            }
+            for (int r = 0; r < 8; ++r) acc[r] = rows[r * 64] * fx;
         }
-        const float inv = 1.0f / l_tot;
-        if (stats && half == 0 && qi < Lq) {
-            stats[2 * ((long long)bh * Lq + qi)] = m_ref;
-            stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
-        }
-        if (qi < Lq) {
-            float *op = out + q_base + (long long)qi * rs + 8 * half;
+        else {
+            l_tot += part[33 * 64 + lane] * fx;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                f32x4 a, c;
-                a.x = o0[4 * g + 0] * inv; a.y = o1[4 * g + 0] * inv;
-                a.z = o0[4 * g + 1] * inv; a.w = o1[4 * g + 1] * inv;
-                c.x = o0[4 * g + 2] * inv; c.y = o1[4 * g + 2] * inv;
-                c.z = o0[4 * g + 3] * inv; c.w = o1[4 * g + 3] * inv;
-                if (8 * half + 16 * g < hd) *reinterpret_cast<f32x4 *>(op + 16 * g) = a;
-                if (8 * half + 16 * g + 4 < hd) *reinterpret_cast<f32x4 *>(op + 16 * g + 4) = c;
-            }
+            for (int r = 0; r < 8; ++r) acc[r] += rows[r * 64] * fx;
         }
+    }
+    const float inv = 1.0f / l_tot;
+    if (stats && wave == 0 && half == 0 && qi < Lq) {
+        stats[2 * ((long long)bh * Lq + qi)] = m_ref;
+        stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
+    }
+    if (qi < Lq) {
+        float *op = out + q_base + (long long)qi * rs + 8 * half + 16 * wave;
+        f32x4 a, c;
+        a.x = acc[0] * inv; a.y = acc[1] * inv; a.z = acc[2] * inv; a.w = acc[3] * inv;
+        c.x = acc[4] * inv; c.y = acc[5] * inv; c.z = acc[6] * inv; c.w = acc[7] * inv;
+        if (8 * half + 16 * wave < hd) *reinterpret_cast<f32x4 *>(op) = a;
+        if (8 * half + 16 * wave + 4 < hd) *reinterpret_cast<f32x4 *>(op + 4) = c;
     }
 }
 
