@@ -113,7 +113,7 @@ void decode_static_scratch_release(dl4s_hip_ctx *ctx);
 
 // Kernel families of dl4s_hip_ctx::lds_limit_raised.
 enum { LDS_PREFILL_SPLIT = 0, LDS_PREFILL = 1, LDS_PREFILL_D128 = 2, LDS_BWD = 3, LDS_BWD_D128 = 4, LDS_GEMM_DEEP = 5, LDS_PREFILL_W192 = 6,
-       LDS_PREFILL_W256 = 7, LDS_PREFILL_W160 = 8 };
+       LDS_PREFILL_W256 = 7, LDS_PREFILL_W160 = 8, LDS_GEMM_HALVES = 9 };
 inline bool lds_limit_pending(const dl4s_hip_ctx *ctx, int family, int kind) {
     const int bit = family * 8 + kind;
     return !(ctx->lds_limit_raised[bit >> 6].load(std::memory_order_acquire) & (1ull << (bit & 63)));

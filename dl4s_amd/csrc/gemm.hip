@@ -249,8 +249,15 @@ struct FastOperand {
 // KT: K tile depth.  The 64x64 form runs one to three wavefronts per SIMD, where a K tile of 16 (8 MFMAs = 512 cycles
 // between barriers) does not cover the latency of the next tile's loads; it takes K tiles of 32.
 // (128 x 128 tiles with 32-deep K tiles hold 70 KiB of LDS: two workgroups per CU, which is all their launches have)
-template <int MI, int NI, bool EPI, bool TA, bool TB, int KT>
-__global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_mfma_fast(GemmArgs g) {
+// HV: how the contraction is summed.  0 = tile after tile from zero.  1 and 2 (products the launcher's shape rule picks:
+// few output tiles, K a whole even number of tiles) = the first and the second half of the K tiles each summed from zero
+// and the two sums added at the end - by one group of four wavefronts that sets the first sum aside when it reaches the
+// middle (1), or by two groups of four wavefronts that work on the halves side by side, each with its own LDS tiles (2:
+// a launch of one workgroup per CU or less, which would otherwise run one wavefront per SIMD).  Same additions in the same
+// order, same bits; which of the two runs depends on how many workgroups the launch has, which the result cannot see.
+template <int MI, int NI, bool EPI, bool TA, bool TB, int KT, int HV = 0>
+__global__ __launch_bounds__(HV == 2 ? 512 : 256, HV == 2 ? 1 : ((MI == 2 && KT == 32) ? 2 : 3)) void gemm_f32_mfma_fast(GemmArgs g) {
+    static_assert(HV == 0 || (MI == 1 && NI == 1), "the halved contraction exists for the 64 x 64 form");
     constexpr int TM = 64 * MI, TN = 64 * NI;       // workgroup tile
     // The 64 x 64 form runs one to three wavefronts per SIMD and a K step of 16 MFMAs (0.4 us) is shorter than a load's way
     // through L2: it keeps two tiles in flight ([2048,512]x[512,512] 15.1 -> 14.0 us, with the LayerNorm sums 21.0 -> 19.7 us,
@@ -259,7 +266,8 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
     using OpA = FastOperand<MI, TA, KT, SLOTS>;      // A is M x K in memory unless transposed
     using OpB = FastOperand<NI, !TB, KT, SLOTS>;     // B is K x N in memory unless transposed
     extern __shared__ __align__(16) float gemm_lds[];
-    float *As = gemm_lds, *Bs = gemm_lds + OpA::LDS_FLOATS;
+    const int grp = HV == 2 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) : 0;     // the wavefront's group
+    float *As = gemm_lds + grp * (OpA::LDS_FLOATS + OpB::LDS_FLOATS), *Bs = As + OpA::LDS_FLOATS;
     // Every argument on the way to the first tile's loads is asked for at once (fetched where the code first needs them,
     // they arrive in six trips, one behind the other - a microsecond of a 15 us launch); the offsets of a grouped launch
     // are picked from registers for the same reason.
@@ -267,7 +275,7 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
                  "s"(g.groups), "s"(g.lda), "s"(g.ldb), "s"(g.tiles_n), "s"(g.tri), "s"(g.a_off[0]), "s"(g.a_off[1]),
                  "s"(g.a_off[2]), "s"(g.a_off[3]), "s"(g.b_off[0]), "s"(g.b_off[1]), "s"(g.b_off[2]), "s"(g.b_off[3]),
                  "s"(g.c_off[0]), "s"(g.c_off[1]), "s"(g.c_off[2]), "s"(g.c_off[3]));
-    const int tid = threadIdx.x;
+    const int tid = HV == 2 ? (int)(threadIdx.x & 255) : (int)threadIdx.x;      // the thread within its group
     const int wave = tid >> 6, lane = tid & 63;
     const int half = lane >> 5, ln = lane & 31;
     const int wm = wave >> 1, wn = wave & 1;
@@ -317,8 +325,18 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     const int ktiles_all = (g.K + KT - 1) / KT;
-    const int kt_first = g.tri == 2 ? min(m0 / KT, ktiles_all) : 0;      // (a tile past the end reads as zeros)
-    const int ktiles = g.tri == 3 ? min(ktiles_all, (m0 + TM + KT - 1) / KT) : ktiles_all;
+    const int kh = ktiles_all / 2;      // HV != 0: where the second half of the contraction starts
+    int kt_first = g.tri == 2 ? min(m0 / KT, ktiles_all) : 0;      // (a tile past the end reads as zeros)
+    int ktiles = g.tri == 3 ? min(ktiles_all, (m0 + TM + KT - 1) / KT) : ktiles_all;
+    if (HV == 2) {      // (no triangle forms here: both groups walk kh tiles and meet at the same barriers)
+        if (grp == 0) ktiles = kh;
+        else kt_first = kh;
+    }
+    f32x16 first_half[MI][NI];      // HV == 1: the sum over the first half, set aside at the middle
+    if (HV == 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) first_half[0][0][r] = 0.f;
+    }
     opa.template load<0>(kt_first);
     opb.template load<0>(kt_first);
     // The 64 x 64 form with an epilogue asks for its bias and residual values now, behind the first tile: requested in the
@@ -333,7 +351,7 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
             const int gn = n0 + wn * 32 + 8 * q4 + 4 * half;
             pre_bias[q4] = f32x4{0.f, 0.f, 0.f, 0.f};
             pre_res[q4] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (gm < g.M && gn < g.N) {
+            if (gm < g.M && gn < g.N && grp == 0) {
                 if (g.bias) pre_bias[q4] = *reinterpret_cast<const f32x4 *>(g.bias + gn);
                 if (g.residual) pre_res[q4] = *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
             }
@@ -393,7 +411,22 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
         if (more || SLOTS == 2) { opa.template store<(SLOTS == 2 ? (buf ^ 1) : 0)>(buf ^ 1, tid); opb.template store<(SLOTS == 2 ? (buf ^ 1) : 0)>(buf ^ 1, tid); }
         __syncthreads();
     };
-    if (SLOTS == 2) {
+    if (HV == 1) {
+        // Two loops with the first sum set aside between them (the launcher's rule makes kh even and keeps the triangle
+        // forms away).  Set aside under a condition inside the step, the accumulator went through 32 selects per step,
+        // each of which waits for the matrix pipe to drain: three such products in one launch 29.2 -> 32.0 us.
+        int kt = kt_first;
+        for (; kt + 1 < kh; kt += 2) {
+            k_step(kt, std::integral_constant<int, 0>{});
+            k_step(kt + 1, std::integral_constant<int, 1>{});
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { first_half[0][0][r] = acc[0][0][r]; acc[0][0][r] = 0.f; }
+        for (; kt + 1 < ktiles; kt += 2) {
+            k_step(kt, std::integral_constant<int, 0>{});
+            k_step(kt + 1, std::integral_constant<int, 1>{});
+        }
+    } else if (SLOTS == 2) {
         // The odd last step stands outside the loop: with an exit between the two steps of the body the compiler sees a way
         // from the first step back to the loop's head, and makes every first step wait for the loads the second one
         // issued - which is what the second register set is there to avoid.  (The 128 x 128 form keeps the plain loop:
@@ -411,12 +444,28 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
         }
     }
 
+    if (HV == 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[0][0][r] = first_half[0][0][r] + acc[0][0][r];
+    }
+    if (HV == 2) {      // the K loop ended on a barrier: the tiles are dead.  Group 1 hands its sum over, group 0 finishes.
+        float *sums = gemm_lds + (wave * 16) * 64 + lane;
+        if (grp == 1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sums[r * 64] = acc[0][0][r];
+        }
+        __syncthreads();
+        if (grp == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[0][0][r] = acc[0][0][r] + sums[r * 64];
+        }
+    }
     // accumulator register r of a transposed 32x32 tile: row m = lane % 32, column n = 8*(r/4) + 4*half + r%4
     float ln_s = 0.f, ln_ss = 0.f;
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
         const int gm = m0 + wm * 32 * MI + i * 32 + ln;
-        if (gm >= g.M) continue;
+        if (gm >= g.M || grp != 0) continue;
 #pragma unroll
         for (int j = 0; j < NI; ++j)
 #pragma unroll
@@ -459,13 +508,16 @@ __global__ __launch_bounds__(256, (MI == 2 && KT == 32) ? 2 : 3) void gemm_f32_m
         if (g.ln_part) {   // the workgroup's pair: the lanes of a wavefront, then the four wavefronts in order
             ln_s = dl4s::wave_sum(ln_s);
             ln_ss = dl4s::wave_sum(ln_ss);
-            if (lane == 0) { As[2 * wave] = ln_s; As[2 * wave + 1] = ln_ss; }   // the K loop ended on a barrier: As is free
+            // the K loop ended on a barrier: the tiles are dead (HV == 2: behind the 4096 floats of group 1's sum, which a
+            // slower wavefront of group 0 may still be reading)
+            float *pairs = gemm_lds + (HV == 2 ? 4096 : 0);
+            if (lane == 0 && grp == 0) { pairs[2 * wave] = ln_s; pairs[2 * wave + 1] = ln_ss; }
             __syncthreads();
-            if (tid == 0) {
+            if (tid == 0 && grp == 0) {
                 const int item = tile_m / g.ln_tiles_m;
                 const long long at = ((long long)item * g.ln_tiles_m + tile_m % g.ln_tiles_m) * g.tiles_n + tile_n;
-                g.ln_part[2 * at] = ((As[0] + As[2]) + As[4]) + As[6];
-                g.ln_part[2 * at + 1] = ((As[1] + As[3]) + As[5]) + As[7];
+                g.ln_part[2 * at] = ((pairs[0] + pairs[2]) + pairs[4]) + pairs[6];
+                g.ln_part[2 * at + 1] = ((pairs[1] + pairs[3]) + pairs[5]) + pairs[7];
             }
         }
     }
@@ -807,8 +859,16 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
         return dl4s::launch_status("gemm_f32_skinny");
     }
     long long tm = (M + GBM - 1) / GBM, tn = (N + GBN - 1) / GBN;
+    // Products of at most one 64 x 64 tile per CU with a long contraction (K a multiple of 128 from 256 on: two halves of
+    // an even number of 32-deep tiles): alone, such a product runs one wavefront per SIMD, so its K tiles are summed in two halves that two
+    // groups of wavefronts can work on side by side ([2048,512].[512,512]: 13.7 -> 11.3 us).  The rule looks at one product's
+    // shape only and fixes the order of the additions; a batch or a group of such products that fills the GPU anyway
+    // runs the one-group form of the same order.  (Callers inside the library with their own batches keep the plain order.)
+    const long long t64 = ((M + 63) / 64) * ((N + 63) / 64);
+    const bool halves = fast && !tiled_only && !tri && t64 <= ctx->cu_count && K >= 256 && K % 128 == 0;
+    const int hv = !halves ? 0 : (t64 * batch <= ctx->cu_count ? 2 : 1);
     // small products: 64x64 tiles, so that there are at least about two workgroups per CU
-    const bool small = fast && tm * tn * batch < 2ll * ctx->cu_count;
+    const bool small = fast && (halves || tm * tn * batch < 2ll * ctx->cu_count);
     if (small) { tm = (M + 63) / 64; tn = (N + 63) / 64; }
     g.tiles_n = (int)tn;
     if (ln_part) {
@@ -826,23 +886,27 @@ int gemm_launch(dl4s_hip_ctx *ctx, const float *lhs, int64_t lr, int64_t lc, int
     // 128 x 128 tiles on a launch of at most two workgroups per CU: K tiles of 32 (half the barriers; contracted as two
     // halves of 16, so the bits do not depend on the depth)
     const bool deep = fast && !small && tm * tn * batch <= 2ll * ctx->cu_count;
-#define DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, KT_)                                                                                   \
+#define DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, KT_, HV_)                                                                              \
     do {                                                                                                                              \
-        constexpr size_t lds_bytes = (FastOperand<MI_, TA_, KT_>::LDS_FLOATS + FastOperand<MI_, !TB_, KT_>::LDS_FLOATS) * sizeof(float); \
+        constexpr size_t lds_bytes = (HV_ == 2 ? 2 : 1) * (FastOperand<MI_, TA_, KT_>::LDS_FLOATS + FastOperand<MI_, !TB_, KT_>::LDS_FLOATS) * sizeof(float); \
         if (lds_bytes > 65536) {                                                                                                      \
             constexpr int which = (EPI_ ? 4 : 0) + (TA_ ? 2 : 0) + (TB_ ? 1 : 0);                                                     \
-            if (dl4s::lds_limit_pending(ctx, dl4s::LDS_GEMM_DEEP, which)) {                                                           \
-                DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, KT_>),  \
+            constexpr int family = HV_ == 2 ? dl4s::LDS_GEMM_HALVES : dl4s::LDS_GEMM_DEEP;                                            \
+            if (dl4s::lds_limit_pending(ctx, family, which)) {                                                                        \
+                DL4S_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, KT_, HV_>), \
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));                        \
-                dl4s::lds_limit_done(ctx, dl4s::LDS_GEMM_DEEP, which);                                                                \
+                dl4s::lds_limit_done(ctx, family, which);                                                                             \
             }                                                                                                                         \
         }                                                                                                                             \
-        hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, KT_>), grid, dim3(256), lds_bytes, ctx->stream, g);          \
+        hipLaunchKernelGGL((gemm_f32_mfma_fast<MI_, MI_, EPI_, TA_, TB_, KT_, HV_>), grid, dim3(HV_ == 2 ? 512 : 256), lds_bytes,     \
+                           ctx->stream, g);                                                                                           \
     } while (0)
 #define DL4S_GEMM_FAST(MI_, EPI_, TA_, TB_)                                                   \
     do {                                                                                      \
-        if (MI_ == 1 || deep) DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, 32);                     \
-        else DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, 16);                                      \
+        if (MI_ == 1 && hv == 2) DL4S_GEMM_FAST_KT(1, EPI_, TA_, TB_, 32, 2);                 \
+        else if (MI_ == 1 && hv == 1) DL4S_GEMM_FAST_KT(1, EPI_, TA_, TB_, 32, 1);            \
+        else if (MI_ == 1 || deep) DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, 32, 0);             \
+        else DL4S_GEMM_FAST_KT(MI_, EPI_, TA_, TB_, 16, 0);                                   \
     } while (0)
     if (fast) {
         const int variant = (small ? 0 : 8) + (epi ? 4 : 0) + (ta ? 2 : 0) + (tb ? 1 : 0);

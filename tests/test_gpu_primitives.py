@@ -233,6 +233,43 @@ def test_gemm_grouped_gives_the_bits_of_single_calls(ctx, orc, M, N, K, ta, tb, 
         x.release()
 
 
+@pytest.mark.parametrize("M,N,K,ta,tb", [(2048, 512, 512, False, False), (1000, 1000, 256, False, False), (1030, 900, 384, False, True),
+                                          (1024, 1024, 1024, False, False), (512, 512, 256, True, False), (640, 320, 768, True, True)])
+def test_gemm_products_summed_in_two_halves(ctx, orc, M, N, K, ta, tb):
+    """Products of at most one 64 x 64 tile per CU whose K is a multiple of 128 (from 256 on) are summed as two halves
+    (so that a launch of one such product can put two groups of wavefronts on every tile).  The order is a property of the
+    product's shape: the call alone (two groups side by side), a batch that fills the GPU (one group, the first half set
+    aside at the middle), a group of three and the product with an epilogue give the same bits; against an fp64 product."""
+    rng = np.random.default_rng(zlib.crc32(repr(("halves", M, N, K, ta, tb)).encode()))
+    count = 6
+    As = [rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32) for _ in range(count)]
+    Bm = (rng.standard_normal((N, K) if tb else (K, N)) * 0.1).astype(np.float32)
+    dA, dB = ctx.to_device(np.stack(As)), ctx.to_device(Bm)
+    single = [ctx.empty((M, N)) for _ in range(count)]
+    for i in range(count):
+        ctx.gemm(dA.offset(i * As[0].size * 4), As[0].shape, dB, Bm.shape, single[i], 1.0, 0.0, ta, tb)
+    ref = (As[0].T if ta else As[0]).astype(np.float64) @ (Bm.T if tb else Bm).astype(np.float64)
+    bound = 2e-6 * np.sqrt(K) * (np.abs(ref).max() + 1.0) + 1e-6
+    assert np.abs(single[0].numpy() - ref).max() <= bound
+    batched = ctx.empty((count, M, N))
+    ctx.gemm_batched(dA, As[0].shape, As[0].size, dB, Bm.shape, 0, batched, M * N, count, 1.0, 0.0, ta, tb)
+    got = batched.numpy()
+    for i in range(count):
+        assert np.array_equal(got[i], single[i].numpy()), "batch item %d" % i
+    grouped = [ctx.empty((M, N)) for _ in range(3)]
+    ctx.gemm_grouped([dA.offset(i * As[0].size * 4) for i in range(3)], As[0].shape, [dB] * 3, Bm.shape, grouped, 1.0, 0.0, ta, tb)
+    for i in range(3):
+        assert np.array_equal(grouped[i].numpy(), single[i].numpy()), "group entry %d" % i
+    keep = [dA, dB, batched] + single + grouped
+    if not ta and not tb:      # the epilogue forms: + 0 leaves the bits (no sum here is -0)
+        zero, fused = ctx.to_device(np.zeros((M, N), np.float32)), ctx.empty((M, N))
+        ctx.dense_fused(dA, M, K, dB, N, None, 0, zero, fused)
+        assert np.array_equal(fused.numpy(), single[0].numpy())
+        keep += [zero, fused]
+    for x in keep:
+        x.release()
+
+
 def test_gemm_grouped_argument_errors(ctx):
     from dl4s_amd import lib
     a = ctx.empty((4, 4))
