@@ -426,11 +426,64 @@ __global__ __launch_bounds__(64) void ln_row_sums_seq_f32(const float *__restric
     if (lane < nr) { part[(r0 + lane) * 2] = s; part[(r0 + lane) * 2 + 1] = ss; }
 }
 
+// The same sums for rows that allow 128-bit accesses (D % 4 == 0, 16-byte aligned operands), with fewer rows per
+// wavefront: the sums of a row are one chain of D dependent additions whoever runs it, so what a launch can win is
+// the number of chains that run side by side - 2048 rows of 512 on wavefronts of 64 rows occupy 32 of the 1024 SIMDs
+// (28.8 us), on wavefronts of 8 rows 256 of them.  A wavefront stages RW rows x 256 columns per step (all 64 lanes load
+// and store, 16 bytes each; the next step's loads are in flight during the additions), then lanes 0 .. RW - 1 walk their
+// rows left to right, four elements per LDS read.
+template <int RW>
+__global__ __launch_bounds__(64) void ln_row_sums_seq_vec_f32(const float *__restrict__ x, const float *__restrict__ res,
+                                                                float *__restrict__ part, long long R, long long D) {
+    constexpr int CT = 256, STRIDE = CT + 4;      // (a row stride of 260 floats: the RW lanes' 128-bit reads fall on distinct banks)
+    __shared__ __align__(16) float tile[RW * STRIDE];
+    const int lane = threadIdx.x;
+    const long long r0 = (long long)blockIdx.x * RW;
+    const int nr = (int)(R - r0 < RW ? R - r0 : RW);
+    f32x4 st[RW];
+    auto load = [&](long long c0) {
+        const long long c = c0 + 4 * lane;
+#pragma unroll
+        for (int i = 0; i < RW; ++i) {
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (i < nr && c < D) v = ln_load4(x, res, (r0 + i) * D + c);
+            st[i] = v;
+        }
+    };
+    float s = 0.f, ss = 0.f;
+    load(0);
+    for (long long c0 = 0; c0 < D; c0 += CT) {
+        __syncthreads();                  // the lanes are done with the tile before
+#pragma unroll
+        for (int i = 0; i < RW; ++i) *reinterpret_cast<f32x4 *>(tile + i * STRIDE + 4 * lane) = st[i];
+        __syncthreads();
+        if (c0 + CT < D) load(c0 + CT);       // in flight during the additions
+        if (lane < RW) {
+            const float *row = tile + lane * STRIDE;
+            const int nc = (int)(D - c0 < CT ? D - c0 : CT);
+            auto add4 = [&](int c) {
+                const f32x4 e = *reinterpret_cast<const f32x4 *>(row + c);
+                s = __fadd_rn(s, e.x); ss = __fadd_rn(ss, __fmul_rn(e.x, e.x));
+                s = __fadd_rn(s, e.y); ss = __fadd_rn(ss, __fmul_rn(e.y, e.y));
+                s = __fadd_rn(s, e.z); ss = __fadd_rn(ss, __fmul_rn(e.z, e.z));
+                s = __fadd_rn(s, e.w); ss = __fadd_rn(ss, __fmul_rn(e.w, e.w));
+            };
+            if (nc == CT) {
+#pragma unroll
+                for (int c = 0; c < CT; c += 4) add4(c);
+            } else {
+                for (int c = 0; c < nc; c += 4) add4(c);
+            }
+        }
+    }
+    if (lane < nr) { part[(r0 + lane) * 2] = s; part[(r0 + lane) * 2 + 1] = ss; }
+}
+
 // The rows of an item, one after the other: rowpart [items][rows][2] -> itempart [items][2].  One wavefront per item
 // stages 512 rows' pairs at a time in LDS; lane 0 adds.
 __global__ __launch_bounds__(64) void ln_item_sums_seq_f32(const float *__restrict__ rowpart, float *__restrict__ itempart, long long rows) {
     constexpr int CH = 512;
-    __shared__ float sm[2 * CH];
+    __shared__ __align__(16) float sm[2 * CH];
     const int lane = threadIdx.x;
     const float *p = rowpart + (long long)blockIdx.x * rows * 2;
     float s = 0.f, ss = 0.f;
@@ -439,9 +492,17 @@ __global__ __launch_bounds__(64) void ln_item_sums_seq_f32(const float *__restri
         __syncthreads();
         for (int i = lane; i < 2 * cnt; i += 64) sm[i] = p[r0 * 2 + i];
         __syncthreads();
-        if (lane == 0) {
+        if (lane == 0) {      // two rows' pairs per LDS read
+            int i = 0;
 #pragma unroll 8
-            for (int i = 0; i < cnt; ++i) {
+            for (; i + 1 < cnt; i += 2) {
+                const f32x4 e = *reinterpret_cast<const f32x4 *>(sm + 2 * i);
+                s = __fadd_rn(s, e.x);
+                ss = __fadd_rn(ss, e.y);
+                s = __fadd_rn(s, e.z);
+                ss = __fadd_rn(ss, e.w);
+            }
+            if (i < cnt) {
                 s = __fadd_rn(s, sm[2 * i]);
                 ss = __fadd_rn(ss, sm[2 * i + 1]);
             }
@@ -1196,8 +1257,13 @@ int dl4s_hip_layernorm_reference_order_f32(dl4s_hip_ctx *ctx, const float *x, co
     int rc = dl4s::ensure_scratch(ctx, (row_floats + item_floats) * sizeof(float));
     if (rc) return rc;
     float *rowpart = reinterpret_cast<float *>(ctx->scratch), *itempart = rows > 1 ? rowpart + row_floats : rowpart;
-    hipLaunchKernelGGL(ln_row_sums_seq_f32, dim3((unsigned)((R + LN_SEQ_ROWS - 1) / LN_SEQ_ROWS)), dim3(64), 0, ctx->stream, x, residual,
-                       rowpart, R, (long long)D);
+    if (vec && R < 32ll * 2 * ctx->cu_count)
+        hipLaunchKernelGGL(ln_row_sums_seq_vec_f32<8>, dim3((unsigned)((R + 7) / 8)), dim3(64), 0, ctx->stream, x, residual, rowpart, R, (long long)D);
+    else if (vec)
+        hipLaunchKernelGGL(ln_row_sums_seq_vec_f32<32>, dim3((unsigned)((R + 31) / 32)), dim3(64), 0, ctx->stream, x, residual, rowpart, R, (long long)D);
+    else
+        hipLaunchKernelGGL(ln_row_sums_seq_f32, dim3((unsigned)((R + LN_SEQ_ROWS - 1) / LN_SEQ_ROWS)), dim3(64), 0, ctx->stream, x, residual,
+                           rowpart, R, (long long)D);
     if (rows > 1) hipLaunchKernelGGL(ln_item_sums_seq_f32, dim3((unsigned)B), dim3(64), 0, ctx->stream, rowpart, itempart, (long long)rows);
     // the normalising pass of the tree-sum kernels on one pair per item (0 + the pair: exact)
     const long long want = n / (TPB * 8);

@@ -566,7 +566,8 @@ def _same_bits(a, b):
 
 
 @pytest.mark.parametrize("B,rows,D", [(3, 5, 64), (15, 1, 64), (2, 300, 68), (4, 1, 1024), (2, 1, 33), (1, 130, 1), (70, 1, 7),
-                                      (2, 64, 128), (3, 65, 63), (2, 512, 512), (1, 1024, 1024)])
+                                      (2, 64, 128), (3, 65, 63), (2, 512, 512), (1, 1024, 1024),
+                                      (2, 8200, 260)])      # the last: enough rows for the 32-row form, a second column step of 4
 def test_layernorm_in_the_reference_order_is_the_oracle_bit_for_bit(ctx, orc, B, rows, D):
     """The sums of dl4s_hip_layernorm_reference_order_f32 are the reference's sequential ones, every other step one
     correctly rounded operation: the result is the oracle's to the last bit, with and without the residual."""
