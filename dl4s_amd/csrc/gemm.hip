@@ -341,21 +341,27 @@ __global__ __launch_bounds__(HV == 2 ? 512 : 256, HV == 2 ? 1 : ((MI == 2 && KT 
     opb.template load<0>(kt_first);
     // The 64 x 64 form with an epilogue asks for its bias and residual values now, behind the first tile: requested in the
     // epilogue, they would add a trip to memory (the residual is the layer's input, long out of the caches) to a launch
-    // that has nothing else left to do.  16 + 16 registers, which this form can spare.
-    constexpr bool PRE = EPI && MI == 1 && NI == 1;
-    f32x4 pre_bias[PRE ? 4 : 1], pre_res[PRE ? 4 : 1];
+    // that has nothing else left to do.  16 + 16 registers, which this form can spare.  So does the 128 x 128 form on K tiles
+    // of 32 (64 + 8 registers; it runs two workgroups per CU and may use 256): its workgroups all end together, and the
+    // residual then no longer shares the memory system with the burst of their stores.
+    constexpr bool PRE = EPI && ((MI == 1 && NI == 1) || (MI == 2 && NI == 2 && KT == 32));
+    f32x4 pre_bias[PRE ? NI : 1][4], pre_res[PRE ? MI : 1][PRE ? NI : 1][4];
     if (PRE) {
-        const int gm = m0 + wm * 32 + ln;
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            const int gn = n0 + wn * 32 + 8 * q4 + 4 * half;
-            pre_bias[q4] = f32x4{0.f, 0.f, 0.f, 0.f};
-            pre_res[q4] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (gm < g.M && gn < g.N && grp == 0) {
-                if (g.bias) pre_bias[q4] = *reinterpret_cast<const f32x4 *>(g.bias + gn);
-                if (g.residual) pre_res[q4] = *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int gn = n0 + wn * 32 * NI + j * 32 + 8 * q4 + 4 * half;
+                pre_bias[j][q4] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (gn < g.N && grp == 0 && g.bias) pre_bias[j][q4] = *reinterpret_cast<const f32x4 *>(g.bias + gn);
+#pragma unroll
+                for (int i = 0; i < MI; ++i) {
+                    const int gm = m0 + wm * 32 * MI + i * 32 + ln;
+                    pre_res[i][j][q4] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    if (gm < g.M && gn < g.N && grp == 0 && g.residual)
+                        pre_res[i][j][q4] = *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
+                }
             }
-        }
     }
     if (SLOTS == 2) {
         // the second tile is requested with the first and both are waited for (they arrive together): entering the loop
@@ -483,7 +489,7 @@ __global__ __launch_bounds__(HV == 2 ? 512 : 256, HV == 2 ? 1 : ((MI == 2 && KT 
                 }
                 if (EPI) {
                     if (g.bias) {
-                        const f32x4 bq = PRE ? pre_bias[PRE ? q4 : 0] : *reinterpret_cast<const f32x4 *>(g.bias + gn);
+                        const f32x4 bq = PRE ? pre_bias[PRE ? j : 0][q4] : *reinterpret_cast<const f32x4 *>(g.bias + gn);
                         val.x = __fadd_rn(val.x, bq.x); val.y = __fadd_rn(val.y, bq.y);
                         val.z = __fadd_rn(val.z, bq.z); val.w = __fadd_rn(val.w, bq.w);
                     }
@@ -492,7 +498,7 @@ __global__ __launch_bounds__(HV == 2 ? 512 : 256, HV == 2 ? 1 : ((MI == 2 && KT 
                         val.z = gelu_sigmoid(val.z); val.w = gelu_sigmoid(val.w);
                     }
                     if (g.residual) {
-                        const f32x4 rq = PRE ? pre_res[PRE ? q4 : 0] : *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
+                        const f32x4 rq = PRE ? pre_res[PRE ? i : 0][PRE ? j : 0][q4] : *reinterpret_cast<const f32x4 *>(g.residual + c_at + (long long)gm * g.N + gn);
                         val.x = __fadd_rn(val.x, rq.x); val.y = __fadd_rn(val.y, rq.y);
                         val.z = __fadd_rn(val.z, rq.z); val.w = __fadd_rn(val.w, rq.w);
                     }
