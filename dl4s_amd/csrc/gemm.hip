@@ -543,10 +543,16 @@ constexpr int SKW = 16;
 template <bool TB>
 __global__ __launch_bounds__(64 * SKW) void gemm_f32_skinny(GemmArgs g, float *__restrict__ part, int kslice, int nbn, int S) {
     __shared__ float red[SKW][32][32];
+    // (every argument on the way to the first loads is asked for in one trip, the offsets of a grouped launch picked from
+    // registers: see gemm_f32_mfma_fast)
+    asm volatile("" ::"s"(g.A), "s"(g.B), "s"(g.C), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.a_bs), "s"(g.b_bs), "s"(g.c_bs),
+                 "s"(g.groups), "s"(g.lda), "s"(g.ldb), "s"(g.a_off[0]), "s"(g.a_off[1]), "s"(g.a_off[2]), "s"(g.a_off[3]),
+                 "s"(g.b_off[0]), "s"(g.b_off[1]), "s"(g.b_off[2]), "s"(g.b_off[3]), "s"(part), "s"(kslice), "s"(nbn), "s"(S));
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, ln = lane & 31;
     const int cb = blockIdx.x % nbn, rb = blockIdx.x / nbn, s = blockIdx.y, z = blockIdx.z;
-    const float *A = g.A + (g.groups ? g.a_off[z] : (long long)z * g.a_bs);
-    const float *B = g.B + (g.groups ? g.b_off[z] : (long long)z * g.b_bs);
+    auto pick = [&](const long long (&off)[4]) { return z == 0 ? off[0] : z == 1 ? off[1] : z == 2 ? off[2] : off[3]; };
+    const float *A = g.A + (g.groups ? pick(g.a_off) : (long long)z * g.a_bs);
+    const float *B = g.B + (g.groups ? pick(g.b_off) : (long long)z * g.b_bs);
     const int m = rb * 32 + ln, n = cb * 32 + ln;
     const int share = kslice / SKW;   // a multiple of 8
     const int k_begin = s * kslice + wave * share;
@@ -644,10 +650,16 @@ __global__ __launch_bounds__(64 * SKW) void gemm_f32_skinny(GemmArgs g, float *_
 template <bool TB>
 __global__ __launch_bounds__(64 * SKW) void gemm_f32_skinny16(GemmArgs g, float *__restrict__ part, int kslice, int nbn, int S) {
     __shared__ float red[SKW][16][16];
+    // (every argument on the way to the first loads is asked for in one trip, the offsets of a grouped launch picked from
+    // registers: see gemm_f32_mfma_fast)
+    asm volatile("" ::"s"(g.A), "s"(g.B), "s"(g.C), "s"(g.M), "s"(g.N), "s"(g.K), "s"(g.a_bs), "s"(g.b_bs), "s"(g.c_bs),
+                 "s"(g.groups), "s"(g.lda), "s"(g.ldb), "s"(g.a_off[0]), "s"(g.a_off[1]), "s"(g.a_off[2]), "s"(g.a_off[3]),
+                 "s"(g.b_off[0]), "s"(g.b_off[1]), "s"(g.b_off[2]), "s"(g.b_off[3]), "s"(part), "s"(kslice), "s"(nbn), "s"(S));
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, q = lane >> 4, ln = lane & 15;
     const int cb = blockIdx.x % nbn, rb = blockIdx.x / nbn, s = blockIdx.y, z = blockIdx.z;
-    const float *A = g.A + (g.groups ? g.a_off[z] : (long long)z * g.a_bs);
-    const float *B = g.B + (g.groups ? g.b_off[z] : (long long)z * g.b_bs);
+    auto pick = [&](const long long (&off)[4]) { return z == 0 ? off[0] : z == 1 ? off[1] : z == 2 ? off[2] : off[3]; };
+    const float *A = g.A + (g.groups ? pick(g.a_off) : (long long)z * g.a_bs);
+    const float *B = g.B + (g.groups ? pick(g.b_off) : (long long)z * g.b_bs);
     const int m = rb * 16 + ln, n = cb * 16 + ln;
     const int share = kslice / SKW;   // a multiple of 16
     const int k_begin = s * kslice + wave * share;
