@@ -288,7 +288,7 @@ __global__ __launch_bounds__(256, 4) void sdpa_prefill_strict_f32_d64(const floa
 // Variant for launches with too few wavefronts to fill the GPU (fewer 32-query wavefronts than about two per SIMD):
 // one workgroup = 32 queries of one (batch, head), and its 4 wavefronts share the keys, wavefront w taking the 32-key
 // tiles w, w + 4, w + 8, ... through a wavefront-private LDS tile (no workgroup barrier in the loop).  At the end the
-// four partial results (reference maximum, row sum, O^T) are merged through LDS and wavefront 0 stores the rows.
+// four partial results (reference maximum, row sum, O^T) are merged through LDS, each wavefront finishing 16 of the 64 columns.
 // Same tile arithmetic as the kernel above; the summation order over keys differs, so results agree with it within
 // rounding, not bit for bit.  Which of the two kernels runs depends on the extents only, never on the mask.
 template <int KIND>
