@@ -563,6 +563,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_split_f32_d64(const float 
                                                                      MaskArgs mask, int strict, int nqb, int total_blocks, int order,
                                                                      int token_major, int hd) {
     extern __shared__ __align__(16) float lds[];
+    // (the arguments in one trip to memory instead of several, one behind the other, before the first row is requested)
+    asm volatile("" ::"s"(q), "s"(k), "s"(v), "s"(dout), "s"(stats), "s"(D), "s"(dq), "s"(H), "s"(Lq), "s"(Lk), "s"(rT), "s"(strict),
+                 "s"(nqb), "s"(total_blocks), "s"(order), "s"(token_major), "s"(hd));
     int bh, unit;
     if (!work_item(nqb, total_blocks, order & 1, bh, unit, order >> 1)) return;
     const int b = bh / H, hh = bh % H;
@@ -671,22 +674,27 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dq_split_f32_d64(const float 
         if (more) store_tile();
     }
 
-    // add the four partial dQ^T blocks in wavefront order
-    __syncthreads();
-    float *mine = lds + wave * 2 * TILE_FLOATS;   // [32][64]
-    if (wave > 0) {
+    // Add the four partial dQ^T blocks in wavefront order.  Every wavefront leaves its block in its own LDS region (its
+    // tiles are dead, and the LDS operations of one wavefront execute in order: no barrier before the writes); behind the
+    // barrier wavefront w adds the accumulator registers 4w .. 4w + 3 of the four blocks (16 of the 64 columns) and
+    // stores them.
+    float *mine = lds + wave * 2 * TILE_FLOATS;   // [32][64]: row 2r = a0[r], row 2r + 1 = a1[r]
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { mine[(2 * r) * 64 + lane] = a0[r]; mine[(2 * r + 1) * 64 + lane] = a1[r]; }
+    for (int r = 0; r < 16; ++r) { mine[(2 * r) * 64 + lane] = a0[r]; mine[(2 * r + 1) * 64 + lane] = a1[r]; }
+    __syncthreads();
+    float sum[8];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        const float *rows = lds + x * 2 * TILE_FLOATS + (8 * wave) * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum[i] = x == 0 ? rows[i * 64] : sum[i] + rows[i * 64];
     }
-    __syncthreads();
-    if (wave == 0) {
-#pragma unroll
-        for (int x = 1; x < 4; ++x) {
-            const float *other = lds + x * 2 * TILE_FLOATS;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) { a0[r] += other[(2 * r) * 64 + lane]; a1[r] += other[(2 * r + 1) * 64 + lane]; }
-        }
-        if (qi < Lq) store_row_t(dq + q_base + (long long)qi * rs + 8 * half, a0, a1, rT, hd - 8 * half);
+    if (qi < Lq) {
+        float *p = dq + q_base + (long long)qi * rs + 8 * half + 16 * wave;
+        const int ncols = hd - 8 * half - 16 * wave;
+        const f32x4 lo = {sum[0] * rT, sum[1] * rT, sum[2] * rT, sum[3] * rT}, hi = {sum[4] * rT, sum[5] * rT, sum[6] * rT, sum[7] * rT};
+        if (0 < ncols) *reinterpret_cast<f32x4 *>(p) = lo;
+        if (4 < ncols) *reinterpret_cast<f32x4 *>(p + 4) = hi;
     }
 }
 
@@ -698,6 +706,9 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_split_f32_d64(const float
                                                                       int Lk, float rT, MaskArgs mask, int strict, int nkb,
                                                                       int total_blocks, int order, int token_major, int hd) {
     extern __shared__ __align__(16) float lds[];
+    // (the arguments in one trip to memory instead of several, one behind the other, before the first row is requested)
+    asm volatile("" ::"s"(q), "s"(k), "s"(v), "s"(dout), "s"(stats), "s"(D), "s"(dk), "s"(dv), "s"(H), "s"(Lq), "s"(Lk), "s"(rT),
+                 "s"(strict), "s"(nkb), "s"(total_blocks), "s"(order), "s"(token_major), "s"(hd));
     int bh, unit;
     if (!work_item(nkb, total_blocks, order & 1, bh, unit, order >> 1)) return;
     const int b = bh / H, hh = bh % H;
@@ -856,31 +867,31 @@ __global__ __launch_bounds__(256, 2) void sdpa_bwd_dkv_split_f32_d64(const float
         tile_accumulate_t(Qs + col_lds, p, k0a, k1a);
     }
 
-    // add the four partial dK^T / dV^T blocks in wavefront order
-    __syncthreads();
-    float *mine = lds + wave * REGION;   // [64][64]
-    if (wave > 0) {
+    // Add the four partial dK^T / dV^T blocks in wavefront order: every wavefront leaves its blocks in its own LDS region
+    // (no barrier before the writes, as above), and behind the barrier wavefront w adds and stores the accumulator
+    // registers 4w .. 4w + 3 (16 of the 64 columns of dK and of dV).
+    float *mine = lds + wave * REGION;   // [64][64]: rows 4r .. 4r + 3 = k0a[r], k1a[r], v0a[r], v1a[r]
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            mine[(4 * r + 0) * 64 + lane] = k0a[r]; mine[(4 * r + 1) * 64 + lane] = k1a[r];
-            mine[(4 * r + 2) * 64 + lane] = v0a[r]; mine[(4 * r + 3) * 64 + lane] = v1a[r];
-        }
+    for (int r = 0; r < 16; ++r) {
+        mine[(4 * r + 0) * 64 + lane] = k0a[r]; mine[(4 * r + 1) * 64 + lane] = k1a[r];
+        mine[(4 * r + 2) * 64 + lane] = v0a[r]; mine[(4 * r + 3) * 64 + lane] = v1a[r];
     }
     __syncthreads();
-    if (wave == 0) {
+    float sum[16];
 #pragma unroll
-        for (int x = 1; x < 4; ++x) {
-            const float *other = lds + x * REGION;
+    for (int x = 0; x < 4; ++x) {
+        const float *rows = lds + x * REGION + (16 * wave) * 64 + lane;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                k0a[r] += other[(4 * r + 0) * 64 + lane]; k1a[r] += other[(4 * r + 1) * 64 + lane];
-                v0a[r] += other[(4 * r + 2) * 64 + lane]; v1a[r] += other[(4 * r + 3) * 64 + lane];
-            }
-        }
-        if (key < Lk) {
-            store_row_t(dv + kv_base + (long long)key * rs + 8 * half, v0a, v1a, 1.0f, hd - 8 * half);
-            store_row_t(dk + kv_base + (long long)key * rs + 8 * half, k0a, k1a, LN2, hd - 8 * half);
-        }
+        for (int i = 0; i < 16; ++i) sum[i] = x == 0 ? rows[i * 64] : sum[i] + rows[i * 64];
+    }
+    if (key < Lk) {
+        // sum[4i + {0,1,2,3}] = k0a, k1a, v0a, v1a of register 4w + i: columns 16w + 4(i/2)... in store_row_t's order
+        const int ncols = hd - 8 * half - 16 * wave;
+        float *pk = dk + kv_base + (long long)key * rs + 8 * half + 16 * wave, *pv = dv + kv_base + (long long)key * rs + 8 * half + 16 * wave;
+        const f32x4 klo = {sum[0] * LN2, sum[1] * LN2, sum[4] * LN2, sum[5] * LN2}, khi = {sum[8] * LN2, sum[9] * LN2, sum[12] * LN2, sum[13] * LN2};
+        const f32x4 vlo = {sum[2] * 1.0f, sum[3] * 1.0f, sum[6] * 1.0f, sum[7] * 1.0f}, vhi = {sum[10] * 1.0f, sum[11] * 1.0f, sum[14] * 1.0f, sum[15] * 1.0f};
+        if (0 < ncols) { *reinterpret_cast<f32x4 *>(pv) = vlo; *reinterpret_cast<f32x4 *>(pk) = klo; }
+        if (4 < ncols) { *reinterpret_cast<f32x4 *>(pv + 4) = vhi; *reinterpret_cast<f32x4 *>(pk + 4) = khi; }
     }
 }
 
