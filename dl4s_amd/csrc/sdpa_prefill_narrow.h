@@ -448,41 +448,48 @@ __global__ __launch_bounds__(256, 2) void sdpa_prefill_split_f32_narrow(const fl
         if (more) store_tile();
     }
 
-    // merge the four partial results (reference maximum, row sum, O^T) in wavefront order
-    float l_tot = sum_across_halves(l_run);
-    __syncthreads();
-    float *mine = lds + wave * REGION;   // rows 0..15 = o0 registers, row 16 = m_run, row 17 = l_tot
-    if (wave > 0) {
+    // Merge the four partial results (reference maximum, row sum, O^T) in wavefront order: every wavefront leaves its
+    // partial result in its own (dead) tile region, and behind the one barrier wavefront w folds the accumulator registers
+    // 4w .. 4w + 3 of the four (8 of the 32 columns) and stores them - see sdpa_prefill_split_f32_d64.
+    {
+        const float l_part = sum_across_halves(l_run);
+        float *mine = lds + wave * REGION;   // rows 0..15 = o0 registers, row 16 = m_run, row 17 = row sum
 #pragma unroll
         for (int r = 0; r < 16; ++r) mine[r * 64 + lane] = o0[r];
         mine[16 * 64 + lane] = m_run;
-        mine[17 * 64 + lane] = l_tot;
+        mine[17 * 64 + lane] = l_part;
     }
     __syncthreads();
-    if (wave == 0) {
-        float m_all = m_run;
+    float m_all = lds[16 * 64 + lane];
 #pragma unroll
-        for (int x = 1; x < SPLIT_WAVES; ++x) m_all = fmaxf(m_all, lds[x * REGION + 16 * 64 + lane]);
-        const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
-        const float f0 = (m_run == -INFINITY) ? 1.0f : fast_exp2(m_run - m_ref);
-        l_tot *= f0;
+    for (int x = 1; x < SPLIT_WAVES; ++x) m_all = fmaxf(m_all, lds[x * REGION + 16 * 64 + lane]);
+    const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
+    float l_tot = 0.f, acc[4];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o0[r] *= f0;
+    for (int x = 0; x < SPLIT_WAVES; ++x) {
+        const float *part = lds + x * REGION;
+        const float mx = part[16 * 64 + lane];
+        const float fx = (mx == -INFINITY) ? 1.0f : fast_exp2(mx - m_ref);
+        const float *rows = part + (4 * wave) * 64 + lane;
+        if (x == 0) {
+            l_tot = part[17 * 64 + lane] * fx;
 #pragma unroll
-        for (int x = 1; x < SPLIT_WAVES; ++x) {
-            const float *other = lds + x * REGION;
-            const float mx = other[16 * 64 + lane];
-            const float fx = (mx == -INFINITY) ? 1.0f : fast_exp2(mx - m_ref);
-            l_tot += other[17 * 64 + lane] * fx;
+            for (int r = 0; r < 4; ++r) acc[r] = rows[r * 64] * fx;
+        } else {
+            l_tot += part[17 * 64 + lane] * fx;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o0[r] += other[r * 64 + lane] * fx;
+            for (int r = 0; r < 4; ++r) acc[r] += rows[r * 64] * fx;
         }
-        const float inv = 1.0f / l_tot;
-        if (stats && half == 0 && qi < Lq) {
-            stats[2 * ((long long)bh * Lq + qi)] = m_ref;
-            stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
-        }
-        if (qi < Lq) store_row_narrow(out + q_base + (long long)qi * rs, o0, inv, half, hd);
+    }
+    const float inv = 1.0f / l_tot;
+    if (stats && wave == 0 && half == 0 && qi < Lq) {
+        stats[2 * ((long long)bh * Lq + qi)] = m_ref;
+        stats[2 * ((long long)bh * Lq + qi) + 1] = inv;
+    }
+    const int d0 = 8 * wave + 4 * half;      // store_row_narrow's group `wave`
+    if (qi < Lq && d0 < hd) {
+        const f32x4 a = {acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv};
+        *reinterpret_cast<f32x4 *>(out + q_base + (long long)qi * rs + d0) = a;
     }
 }
 
